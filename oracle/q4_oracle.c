@@ -1,0 +1,566 @@
+/*
+ * q4_oracle.c — CPU restatement of lattice's Q4 block-quantized matmul semantics.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This file is the checker the HIP path is compared
+ * against; nothing in the shipped library links, loads or calls it.  Build with
+ * `make -C oracle` (flags matter: -ffp-contract=off keeps `acc += x*w` as a
+ * separate multiply and add, exactly as the Rust reference evaluates it).
+ *
+ * Every function cites the reference span it restates (paths relative to the
+ * lattice repository root).  How each one is pinned (golden bytes, closed
+ * forms, brute force vs hardware conversions) is listed in tests/test_oracle_*.py.
+ *
+ * Parity status: every function in this file is pinned by at least one
+ * reference-held vector or a mathematical identity; none is "parity unpinned".
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define LQ4_BLOCK_BYTES 20 /* crates/inference/src/weights/q4_weights.rs:84 */
+#define LQ4_BLOCK_WEIGHTS 32 /* crates/inference/src/weights/q4_weights.rs:92 */
+
+/* ------------------------------------------------------------------------- */
+/* f16 <-> f32 bit conversion                                                 */
+/* ------------------------------------------------------------------------- */
+
+static float bits_to_f32(uint32_t b) {
+    float f;
+    memcpy(&f, &b, 4);
+    return f;
+}
+static uint32_t f32_to_bits(float f) {
+    uint32_t b;
+    memcpy(&b, &f, 4);
+    return b;
+}
+
+/* crates/inference/src/weights/half_bits.rs:24-53 — exact widening, subnormals
+ * normalised, NaN payload shifted into the f32 mantissa. */
+float lq4o_f16_to_f32(uint16_t h) {
+    uint32_t sign = (uint32_t)(h >> 15) & 1u;
+    uint32_t exp = (uint32_t)(h >> 10) & 0x1fu;
+    uint32_t frac = (uint32_t)h & 0x3ffu;
+    uint32_t out;
+    if (exp == 0 && frac == 0) {
+        out = sign << 31;
+    } else if (exp == 0) {
+        int e = -14;
+        uint32_t mant = frac;
+        while ((mant & 0x400u) == 0) {
+            mant <<= 1;
+            e -= 1;
+        }
+        mant &= 0x3ffu;
+        out = (sign << 31) | ((uint32_t)(e + 127) << 23) | (mant << 13);
+    } else if (exp == 0x1f && frac == 0) {
+        out = (sign << 31) | 0x7f800000u;
+    } else if (exp == 0x1f) {
+        out = (sign << 31) | 0x7f800000u | (frac << 13);
+    } else {
+        out = (sign << 31) | ((uint32_t)((int)exp - 15 + 127) << 23) | (frac << 13);
+    }
+    return bits_to_f32(out);
+}
+
+/* crates/inference/src/weights/f16_encode.rs:4-23 */
+static uint32_t round_shift_right_even(uint32_t value, uint32_t shift) {
+    if (shift == 0) return value;
+    if (shift >= 32) return 0;
+    uint32_t base = value >> shift;
+    uint32_t mask = (1u << shift) - 1u;
+    uint32_t rem = value & mask;
+    uint32_t half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (base & 1u) != 0)) return base + 1;
+    return base;
+}
+
+/* crates/inference/src/weights/f16_encode.rs:27-84 — round-to-nearest-even,
+ * overflow -> inf, f32 subnormal input -> signed zero, NaN quieted. */
+uint16_t lq4o_f32_to_f16(float v) {
+    uint32_t bits = f32_to_bits(v);
+    uint16_t sign = (uint16_t)((bits >> 16) & 0x8000u);
+    int exp = (int)((bits >> 23) & 0xffu);
+    uint32_t frac = bits & 0x007fffffu;
+
+    if (exp == 0xff) {
+        if (frac == 0) return sign | 0x7c00u;
+        uint16_t payload = (uint16_t)(frac >> 13);
+        if (payload == 0) payload = 1;
+        payload |= 0x0200u;
+        return sign | 0x7c00u | (payload & 0x03ffu);
+    }
+    if (exp == 0) return sign;
+
+    int exp32 = exp - 127;
+    if (exp32 > 15) return sign | 0x7c00u;
+
+    if (exp32 >= -14) {
+        uint16_t exp16 = (uint16_t)(exp32 + 15);
+        uint16_t frac16 = (uint16_t)round_shift_right_even(frac, 13);
+        if (frac16 == 0x0400u) {
+            frac16 = 0;
+            exp16 += 1;
+            if (exp16 >= 0x1f) return sign | 0x7c00u;
+        }
+        return sign | (uint16_t)(exp16 << 10) | frac16;
+    }
+
+    uint32_t mant = frac | 0x00800000u;
+    uint32_t shift = (uint32_t)(-exp32 - 1);
+    if (shift >= 32) return sign;
+    uint16_t frac16 = (uint16_t)round_shift_right_even(mant, shift);
+    if (frac16 == 0) return sign;
+    if (frac16 == 0x0400u) return sign | 0x0400u;
+    return sign | frac16;
+}
+
+/* crates/inference/src/weights/half_bits.rs:55-63 */
+float lq4o_bf16_to_f32(uint16_t b) { return bits_to_f32((uint32_t)b << 16); }
+
+/* Array forms of the two conversions (inputs/outputs are raw bit patterns). */
+void lq4o_f16_to_f32_array(const uint16_t* in, uint32_t* out_bits, size_t n) {
+    for (size_t i = 0; i < n; ++i) out_bits[i] = f32_to_bits(lq4o_f16_to_f32(in[i]));
+}
+void lq4o_f32_to_f16_array(const uint32_t* in_bits, uint16_t* out, size_t n) {
+    for (size_t i = 0; i < n; ++i) out[i] = lq4o_f32_to_f16(bits_to_f32(in_bits[i]));
+}
+
+/* ------------------------------------------------------------------------- */
+/* Block quantizer                                                            */
+/* ------------------------------------------------------------------------- */
+
+/* crates/inference/src/weights/q4_weights.rs:161-165 */
+static int scale_survives_f16(float scale) {
+    float s = lq4o_f16_to_f32(lq4o_f32_to_f16(scale));
+    return isfinite(s) && s > 0.0f;
+}
+
+/* crates/inference/src/weights/q4_weights.rs:210-216 */
+static float degenerate_safe_scale(float candidate) {
+    if (candidate < 1.0f && !scale_survives_f16(candidate)) return 1.0f;
+    return candidate;
+}
+
+/* Rust `f32::clamp(0.0, 15.0) as u8`: NaN saturates to 0 in the cast. */
+static uint8_t clamp_nibble(float v) {
+    if (v != v) return 0;
+    if (v < 0.0f) v = 0.0f;
+    if (v > 15.0f) v = 15.0f;
+    return (uint8_t)v;
+}
+
+/* Error codes shared by the quantizer entry points. */
+#define LQ4O_OK 0
+#define LQ4O_ERR_VALID_LEN 1  /* valid_len outside 1..=32 */
+#define LQ4O_ERR_NONFINITE 2  /* a source weight is NaN/inf */
+#define LQ4O_ERR_SCALE 3      /* scale not a finite, strictly positive f16 */
+#define LQ4O_ERR_BIAS 4       /* bias not a finite f16 */
+
+/* crates/inference/src/weights/q4_weights.rs:239-295 (+ metadata rule :166-181).
+ * `vals` holds 32 floats (caller zero-pads the tail); writes one 20-byte block. */
+int lq4o_quantize_block(const float* vals, int valid_len, int symmetric, uint8_t* out) {
+    if (valid_len < 1 || valid_len > 32) return LQ4O_ERR_VALID_LEN;
+    for (int i = 0; i < 32; ++i)
+        if (!isfinite(vals[i])) return LQ4O_ERR_NONFINITE;
+
+    float scale, bias, sub;
+    if (symmetric) {
+        float abs_max = 0.0f;
+        for (int i = 0; i < 32; ++i) {
+            float a = fabsf(vals[i]);
+            if (a > abs_max) abs_max = a;
+        }
+        scale = degenerate_safe_scale(abs_max / 7.0f);
+        bias = -8.0f * scale;
+        sub = 0.0f;
+    } else {
+        float mn = INFINITY, mx = -INFINITY;
+        for (int i = 0; i < valid_len; ++i) {
+            if (vals[i] < mn) mn = vals[i];
+            if (vals[i] > mx) mx = vals[i];
+        }
+        scale = degenerate_safe_scale((mx - mn) / 15.0f);
+        bias = mn;
+        sub = mn;
+    }
+    uint16_t scale_bits = lq4o_f32_to_f16(scale);
+    uint16_t bias_bits = lq4o_f32_to_f16(bias);
+    if (!scale_survives_f16(scale)) return LQ4O_ERR_SCALE;
+    if (!isfinite(lq4o_f16_to_f32(bias_bits))) return LQ4O_ERR_BIAS;
+
+    float inv_scale = 1.0f / scale;
+    out[0] = (uint8_t)(scale_bits & 0xff);
+    out[1] = (uint8_t)(scale_bits >> 8);
+    out[2] = (uint8_t)(bias_bits & 0xff);
+    out[3] = (uint8_t)(bias_bits >> 8);
+    for (int b = 0; b < 16; ++b) {
+        uint8_t q0, q1;
+        if (symmetric) {
+            q0 = clamp_nibble(roundf(vals[2 * b] * inv_scale) + 8.0f);
+            q1 = clamp_nibble(roundf(vals[2 * b + 1] * inv_scale) + 8.0f);
+        } else {
+            q0 = clamp_nibble(roundf((vals[2 * b] - sub) * inv_scale));
+            q1 = clamp_nibble(roundf((vals[2 * b + 1] - sub) * inv_scale));
+        }
+        out[4 + b] = (uint8_t)((q1 << 4) | (q0 & 0x0f));
+    }
+    return LQ4O_OK;
+}
+
+/* Flat blocking over `n` values, last block zero-padded:
+ * quantize_row_q4_0 (q4_weights.rs:312-328, asymmetric) and
+ * quantize_f32_to_q4 / quantize_f64_to_q4_mode (q4_weights.rs:470-556).
+ * `out` must hold ceil(n/32)*20 bytes. */
+int lq4o_quantize_flat(const float* src, size_t n, int symmetric, uint8_t* out) {
+    size_t nb = (n + 31) / 32;
+    for (size_t blk = 0; blk < nb; ++blk) {
+        float vals[32];
+        size_t base = blk * 32;
+        int len = (int)((n - base) < 32 ? (n - base) : 32);
+        for (int i = 0; i < 32; ++i) vals[i] = i < len ? src[base + i] : 0.0f;
+        int rc = lq4o_quantize_block(vals, len, symmetric, out + blk * LQ4_BLOCK_BYTES);
+        if (rc) return rc;
+    }
+    return LQ4O_OK;
+}
+
+/* quantize_tensor_q4_0 (q4_weights.rs:364-388): each row blocked on its own. */
+int lq4o_quantize_rows(const float* src, size_t rows, size_t cols, int symmetric, uint8_t* out) {
+    size_t bpr = (cols + 31) / 32;
+    for (size_t r = 0; r < rows; ++r) {
+        int rc = lq4o_quantize_flat(src + r * cols, cols, symmetric, out + r * bpr * LQ4_BLOCK_BYTES);
+        if (rc) return rc;
+    }
+    return LQ4O_OK;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Dequantize                                                                 */
+/* ------------------------------------------------------------------------- */
+
+/* dequantize_row_q4_0 (q4_weights.rs:340-353): complete blocks only, output
+ * truncated to n_weights; returns the number of floats written. */
+size_t lq4o_dequantize(const uint8_t* data, size_t nbytes, size_t n_weights, float* out) {
+    size_t nb = nbytes / LQ4_BLOCK_BYTES;
+    size_t w = 0;
+    for (size_t blk = 0; blk < nb && w < n_weights; ++blk) {
+        const uint8_t* c = data + blk * LQ4_BLOCK_BYTES;
+        float scale = lq4o_f16_to_f32((uint16_t)(c[0] | (c[1] << 8)));
+        float bias = lq4o_f16_to_f32((uint16_t)(c[2] | (c[3] << 8)));
+        for (int b = 0; b < 16 && w < n_weights; ++b) {
+            uint8_t byte = c[4 + b];
+            out[w++] = (float)(byte & 0x0f) * scale + bias;
+            if (w < n_weights) out[w++] = (float)(byte >> 4) * scale + bias;
+        }
+    }
+    return w;
+}
+
+/* Per-block metadata rule (weights/ingress.rs:542-559 through
+ * q4_weights.rs:876-918): scale finite and > 0, bias finite.  Returns the index
+ * of the first offending block, or -1 when every block passes.  `*why` gets
+ * 1 for a bad scale, 2 for a bad bias. */
+long lq4o_validate_blocks(const uint8_t* payload, size_t nbytes, int* why) {
+    size_t nb = nbytes / LQ4_BLOCK_BYTES;
+    for (size_t blk = 0; blk < nb; ++blk) {
+        const uint8_t* c = payload + blk * LQ4_BLOCK_BYTES;
+        float scale = lq4o_f16_to_f32((uint16_t)(c[0] | (c[1] << 8)));
+        float bias = lq4o_f16_to_f32((uint16_t)(c[2] | (c[3] << 8)));
+        if (!isfinite(scale) || scale <= 0.0f) {
+            if (why) *why = 1;
+            return (long)blk;
+        }
+        if (!isfinite(bias)) {
+            if (why) *why = 2;
+            return (long)blk;
+        }
+    }
+    if (why) *why = 0;
+    return -1;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Matmul oracle:  Y[M,N] = X[M,K] . dequant(W_q4[N,K])^T                      */
+/* ------------------------------------------------------------------------- */
+
+/* Composition the reference's own GPU tests use as ground truth:
+ * dequantize_row_q4_0 per weight row, then cpu_matmul_ref — sequential f32
+ * `acc += x*w`, k ascending (forward/metal_qwen35.rs:22850-22899).
+ * W is N rows of (K/32) blocks, row stride (K/32)*20 bytes. */
+int lq4o_gemm_f32(const float* x, const uint8_t* wq, float* y, size_t m, size_t n, size_t k) {
+    if (k == 0 || k % 32 != 0) return 1;
+    size_t row_bytes = (k / 32) * LQ4_BLOCK_BYTES;
+    float* wrow = (float*)malloc(k * sizeof(float));
+    if (!wrow) return 2;
+    for (size_t ni = 0; ni < n; ++ni) {
+        lq4o_dequantize(wq + ni * row_bytes, row_bytes, k, wrow);
+        for (size_t mi = 0; mi < m; ++mi) {
+            const float* xr = x + mi * k;
+            float acc = 0.0f;
+            for (size_t ki = 0; ki < k; ++ki) acc += xr[ki] * wrow[ki];
+            y[mi * n + ni] = acc;
+        }
+    }
+    free(wrow);
+    return 0;
+}
+
+/* Same contraction accumulated in f64 (products of two f32 are exact in f64):
+ * separates a kernel's error from the f32 oracle's own summation error.  This
+ * is the form quarot_rotated_q4_forward_matches_f64_reference uses
+ * (weights/q4_weights.rs:2487-2672). */
+int lq4o_gemm_f64(const float* x, const uint8_t* wq, double* y, size_t m, size_t n, size_t k) {
+    if (k == 0 || k % 32 != 0) return 1;
+    size_t row_bytes = (k / 32) * LQ4_BLOCK_BYTES;
+    float* wrow = (float*)malloc(k * sizeof(float));
+    if (!wrow) return 2;
+    for (size_t ni = 0; ni < n; ++ni) {
+        lq4o_dequantize(wq + ni * row_bytes, row_bytes, k, wrow);
+        for (size_t mi = 0; mi < m; ++mi) {
+            const float* xr = x + mi * k;
+            double acc = 0.0;
+            for (size_t ki = 0; ki < k; ++ki) acc += (double)xr[ki] * (double)wrow[ki];
+            y[mi * n + ni] = acc;
+        }
+    }
+    free(wrow);
+    return 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* LoRA delta:  y[row] += scale * B . (A . x[row])                             */
+/* ------------------------------------------------------------------------- */
+
+/* apply_lora (crates/tune/src/lora/apply.rs:48-98): t[r] = sum_k A[r,k]*x[k]
+ * (sequential f32), then y[n] += scale * sum_j B[n,j]*t[j].  A is [rank,d_in],
+ * B is [d_out,rank], both row-major f32.  Applied independently to each of
+ * `m` rows, as apply_lora_rows does (crates/inference/src/lora_hook.rs). */
+void lq4o_lora_apply(const float* a, const float* b, size_t rank, size_t d_in, size_t d_out,
+                     float scale, const float* x, float* y, size_t m) {
+    float* t = (float*)malloc((rank ? rank : 1) * sizeof(float));
+    for (size_t mi = 0; mi < m; ++mi) {
+        const float* xr = x + mi * d_in;
+        float* yr = y + mi * d_out;
+        for (size_t r = 0; r < rank; ++r) {
+            float acc = 0.0f;
+            for (size_t kk = 0; kk < d_in; ++kk) acc += a[r * d_in + kk] * xr[kk];
+            t[r] = acc;
+        }
+        for (size_t nn = 0; nn < d_out; ++nn) {
+            float acc = 0.0f;
+            for (size_t j = 0; j < rank; ++j) acc += b[nn * rank + j] * t[j];
+            yr[nn] += scale * acc;
+        }
+    }
+    free(t);
+}
+
+/* f64 twin of the above (A, B, x widened exactly), y accumulated in f64. */
+void lq4o_lora_apply_f64(const float* a, const float* b, size_t rank, size_t d_in, size_t d_out,
+                         float scale, const float* x, double* y, size_t m) {
+    double* t = (double*)malloc((rank ? rank : 1) * sizeof(double));
+    for (size_t mi = 0; mi < m; ++mi) {
+        const float* xr = x + mi * d_in;
+        double* yr = y + mi * d_out;
+        for (size_t r = 0; r < rank; ++r) {
+            double acc = 0.0;
+            for (size_t kk = 0; kk < d_in; ++kk) acc += (double)a[r * d_in + kk] * (double)xr[kk];
+            t[r] = acc;
+        }
+        for (size_t nn = 0; nn < d_out; ++nn) {
+            double acc = 0.0;
+            for (size_t j = 0; j < rank; ++j) acc += (double)b[nn * rank + j] * t[j];
+            yr[nn] += (double)scale * acc;
+        }
+    }
+    free(t);
+}
+
+/* ------------------------------------------------------------------------- */
+/* MoE routing and routed-expert accumulation                                 */
+/* ------------------------------------------------------------------------- */
+
+/* compute_router_probs (crates/inference/src/model/qwen35/moe.rs:39-95), from the
+ * logits row on (the router GEMV itself is not on this path): softmax over all
+ * E with the max subtracted; a non-finite max, or a denominator that is not
+ * > 0 (NaN included), zeroes the whole row. */
+void lq4o_router_softmax(const float* logits, int num_experts, float* probs) {
+    float mx = -INFINITY;
+    for (int e = 0; e < num_experts; ++e) {
+        /* Rust f32::max returns the other operand when one is NaN. */
+        if (logits[e] > mx || mx != mx) mx = logits[e];
+    }
+    if (!isfinite(mx)) {
+        for (int e = 0; e < num_experts; ++e) probs[e] = 0.0f;
+        return;
+    }
+    float denom = 0.0f;
+    for (int e = 0; e < num_experts; ++e) {
+        probs[e] = expf(logits[e] - mx);
+        denom += probs[e];
+    }
+    if (denom > 0.0f) {
+        for (int e = 0; e < num_experts; ++e) probs[e] /= denom;
+    } else {
+        for (int e = 0; e < num_experts; ++e) probs[e] = 0.0f;
+    }
+}
+
+/* select_top_k (moe.rs:97-116): insertion by strict `>` against slots seeded
+ * with -inf, so equal probabilities keep the lower expert id first and a slot
+ * nothing beats stays unfilled (id -1 here, usize::MAX there). */
+void lq4o_select_top_k(const float* probs, int num_experts, int top_k, int32_t* ids, float* vals) {
+    for (int r = 0; r < top_k; ++r) {
+        ids[r] = -1;
+        vals[r] = -INFINITY;
+    }
+    for (int e = 0; e < num_experts; ++e) {
+        float p = probs[e];
+        for (int r = 0; r < top_k; ++r) {
+            if (p > vals[r]) {
+                for (int s = top_k - 1; s > r; --s) {
+                    ids[s] = ids[s - 1];
+                    vals[s] = vals[s - 1];
+                }
+                ids[r] = e;
+                vals[r] = p;
+                break;
+            }
+        }
+    }
+}
+
+/* renormalize_selected (moe.rs:118-125): divide by the sequential f32 sum of
+ * the selected values when that sum is positive. */
+void lq4o_renormalize_selected(float* vals, int top_k) {
+    float top_sum = 0.0f;
+    for (int r = 0; r < top_k; ++r) top_sum += vals[r];
+    if (top_sum > 0.0f)
+        for (int r = 0; r < top_k; ++r) vals[r] /= top_sum;
+}
+
+/* The three steps in the order moe_ffn_step runs them (moe.rs:25-31). */
+void lq4o_moe_route(const float* logits, int num_experts, int top_k, float* probs, int32_t* ids,
+                    float* weights) {
+    lq4o_router_softmax(logits, num_experts, probs);
+    lq4o_select_top_k(probs, num_experts, top_k, ids, weights);
+    lq4o_renormalize_selected(weights, top_k);
+}
+
+/* silu_inplace_scalar (crates/inference/src/forward/cpu/elementwise.rs:140-144) */
+static float silu_f32(float v) { return v * (1.0f / (1.0f + expf(-v))); }
+
+/* accumulate_routed_experts (moe.rs:127-190) with the expert tensors held as Q4
+ * blocks instead of f32: gate_up is [E, 2I, H] (gate rows first, then up rows),
+ * down is [E, H, I]; out[t,:] = sum over the token's selected experts of
+ * w * W_down . (silu(W_gate . x) * (W_up . x)).  Slots with id outside
+ * [0, E) are skipped, as the reference does for unfilled slots.  Each GEMV is
+ * dequantize -> sequential f32 dot.  H and I must be multiples of 32. */
+int lq4o_moe_ffn_f32(const uint8_t* gate_up_q4, const uint8_t* down_q4, int num_experts, int inter,
+                     int hidden, const float* x, int tokens, const int32_t* ids,
+                     const float* weights, int top_k, float* out) {
+    if (hidden % 32 || inter % 32) return 1;
+    size_t gu_bytes = (size_t)2 * inter * (hidden / 32) * LQ4_BLOCK_BYTES;
+    size_t dn_bytes = (size_t)hidden * (inter / 32) * LQ4_BLOCK_BYTES;
+    float* gu = (float*)malloc((size_t)2 * inter * sizeof(float));
+    float* o = (float*)malloc((size_t)hidden * sizeof(float));
+    for (int t = 0; t < tokens; ++t) {
+        const float* xt = x + (size_t)t * hidden;
+        float* ot = out + (size_t)t * hidden;
+        for (int i = 0; i < hidden; ++i) ot[i] = 0.0f;
+        for (int s = 0; s < top_k; ++s) {
+            int e = ids[t * top_k + s];
+            float w = weights[t * top_k + s];
+            if (e < 0 || e >= num_experts) continue;
+            lq4o_gemm_f32(xt, gate_up_q4 + (size_t)e * gu_bytes, gu, 1, (size_t)2 * inter, hidden);
+            for (int i = 0; i < inter; ++i) gu[i] = silu_f32(gu[i]) * gu[inter + i];
+            lq4o_gemm_f32(gu, down_q4 + (size_t)e * dn_bytes, o, 1, hidden, inter);
+            for (int i = 0; i < hidden; ++i) ot[i] += w * o[i];
+        }
+    }
+    free(gu);
+    free(o);
+    return 0;
+}
+
+/* f64 twin: every dot, the SiLU and the weighted sum carried in f64. */
+int lq4o_moe_ffn_f64(const uint8_t* gate_up_q4, const uint8_t* down_q4, int num_experts, int inter,
+                     int hidden, const float* x, int tokens, const int32_t* ids,
+                     const float* weights, int top_k, double* out) {
+    if (hidden % 32 || inter % 32) return 1;
+    size_t gu_row = (size_t)(hidden / 32) * LQ4_BLOCK_BYTES;
+    size_t dn_row = (size_t)(inter / 32) * LQ4_BLOCK_BYTES;
+    size_t gu_bytes = (size_t)2 * inter * gu_row;
+    size_t dn_bytes = (size_t)hidden * dn_row;
+    float* wrow = (float*)malloc((size_t)(hidden > inter ? hidden : inter) * sizeof(float));
+    double* gu = (double*)malloc((size_t)2 * inter * sizeof(double));
+    for (int t = 0; t < tokens; ++t) {
+        const float* xt = x + (size_t)t * hidden;
+        double* ot = out + (size_t)t * hidden;
+        for (int i = 0; i < hidden; ++i) ot[i] = 0.0;
+        for (int s = 0; s < top_k; ++s) {
+            int e = ids[t * top_k + s];
+            double w = (double)weights[t * top_k + s];
+            if (e < 0 || e >= num_experts) continue;
+            const uint8_t* gw = gate_up_q4 + (size_t)e * gu_bytes;
+            for (int r = 0; r < 2 * inter; ++r) {
+                lq4o_dequantize(gw + (size_t)r * gu_row, gu_row, hidden, wrow);
+                double acc = 0.0;
+                for (int kk = 0; kk < hidden; ++kk) acc += (double)xt[kk] * (double)wrow[kk];
+                gu[r] = acc;
+            }
+            for (int i = 0; i < inter; ++i) gu[i] = gu[i] / (1.0 + exp(-gu[i])) * gu[inter + i];
+            const uint8_t* dw = down_q4 + (size_t)e * dn_bytes;
+            for (int r = 0; r < hidden; ++r) {
+                lq4o_dequantize(dw + (size_t)r * dn_row, dn_row, inter, wrow);
+                double acc = 0.0;
+                for (int kk = 0; kk < inter; ++kk) acc += gu[kk] * (double)wrow[kk];
+                ot[r] += w * acc;
+            }
+        }
+    }
+    free(wrow);
+    free(gu);
+    return 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* `.q4` file header                                                          */
+/* ------------------------------------------------------------------------- */
+
+/* read_q4_header + validate_q4_header_payload_bounds
+ * (weights/q4_weights.rs:709-812): "KHQ4", u32 version (1 = legacy, rejected;
+ * only 2 accepted), u32 ndim, u64 shape[ndim], u64 original_len, then exactly
+ * ceil(original_len/32) blocks and nothing after them.
+ * Returns 0 and fills the outputs, or: 1 short/bad magic, 2 legacy v1,
+ * 3 unsupported version, 4 header truncated / ndim beyond max_dims,
+ * 5 payload truncated, 6 trailing bytes, 7 shape product != original_len. */
+int lq4o_parse_q4_file(const uint8_t* file, size_t file_len, uint64_t* shape, int max_dims,
+                       int* ndim_out, uint64_t* original_len, uint64_t* payload_offset) {
+    if (file_len < 12 || memcmp(file, "KHQ4", 4) != 0) return 1;
+    uint32_t ver, ndim;
+    memcpy(&ver, file + 4, 4);
+    memcpy(&ndim, file + 8, 4);
+    if (ver == 1) return 2;
+    if (ver != 2) return 3;
+    if ((int)ndim > max_dims || (uint64_t)ndim * 8 + 20 > file_len) return 4;
+    uint64_t prod = 1;
+    for (uint32_t i = 0; i < ndim; ++i) {
+        memcpy(&shape[i], file + 12 + 8 * (size_t)i, 8);
+        prod *= shape[i];
+    }
+    uint64_t olen;
+    memcpy(&olen, file + 12 + 8 * (size_t)ndim, 8);
+    uint64_t off = 20 + 8 * (uint64_t)ndim;
+    uint64_t need = off + ((olen + 31) / 32) * LQ4_BLOCK_BYTES;
+    if (file_len < need) return 5;
+    if (file_len > need) return 6;
+    if (prod != olen) return 7;
+    *ndim_out = (int)ndim;
+    *original_len = olen;
+    *payload_offset = off;
+    return 0;
+}

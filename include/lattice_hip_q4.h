@@ -1,0 +1,178 @@
+/*
+ * lattice_hip_q4.h — C ABI of liblattice_hip_q4.so: lattice's Q4 block-quantized
+ * matmul path (decode GEMV, prefill GEMM, single-LoRA epilogue, grouped MoE expert
+ * GEMV) on AMD MI355X (gfx950).
+ *
+ * Conventions shared with the reference backend this replaces
+ * (crates/inference/src/forward/metal_qwen35/inner/dispatch.rs):
+ *   - row-major everywhere; a weight matrix is W[N,K] (out x in) and the op is
+ *     Y[M,N] = X[M,K] . W^T;
+ *   - weights are lattice's native 20-byte Q4 blocks, byte for byte
+ *     ([f16 scale][f16 bias][16 bytes, low nibble = even index], 32 weights per
+ *     block, row stride (K/32)*20 bytes; crates/inference/src/weights/q4_weights.rs:65-92);
+ *   - offsets are BYTES; M == 0 or N == 0 is a silent no-op; K == 0 or K % 32 != 0
+ *     is an error (the reference asserts, dispatch.rs:185-188);
+ *   - every output element of rows < N is overwritten (no accumulate) except where a
+ *     function says it accumulates.
+ * Pointers named *_dev are device addresses on the context's GPU.  `stream` is a
+ * hipStream_t passed as void* (NULL = the default stream); launches are asynchronous.
+ * Every function returns LQ4_OK (0) or a negative LQ4_E_* code and never throws or
+ * aborts; lq4_last_error() gives the message for the calling thread's last failure.
+ */
+#ifndef LATTICE_HIP_Q4_H
+#define LATTICE_HIP_Q4_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LQ4_BLOCK_BYTES 20   /* q4_weights.rs:84  Q4_BLOCK_BYTES   */
+#define LQ4_BLOCK_WEIGHTS 32 /* q4_weights.rs:92  Q4_BLOCK_WEIGHTS */
+
+enum {
+    LQ4_OK = 0,
+    LQ4_E_INVALID = -1,  /* bad argument (null pointer, K % 32 != 0, out-of-range view) */
+    LQ4_E_HIP = -2,      /* a HIP runtime call failed; message carries hipGetErrorString */
+    LQ4_E_BLOCK = -3,    /* a block's scale/bias failed the ingress rule               */
+    LQ4_E_NOMEM = -4,
+    LQ4_E_UNSUPPORTED = -5 /* e.g. LoRA rank above LQ4_MAX_LORA_RANK                   */
+};
+
+enum { LQ4_F32 = 0, LQ4_F16 = 1 }; /* element type of activations / LoRA factors */
+
+#define LQ4_MAX_LORA_RANK 64   /* the reference's kernels assume rank <= 64 (qwen35.metal:2302) */
+#define LQ4_MAX_GEMV_BATCH 16  /* lq4_gemv handles 1..16 rows; use lq4_gemm above that          */
+
+typedef struct lq4_ctx lq4_ctx;       /* one per GPU; owns small scratch buffers          */
+typedef struct lq4_weight lq4_weight; /* replaces Q4WeightBuf (forward/metal_qwen35.rs:599-636) */
+typedef struct lq4_lora lq4_lora;     /* replaces one LoraLayerData projection (metal_qwen35.rs:1701-1716) */
+
+const char* lq4_last_error(void);
+const char* lq4_version(void);
+
+/* ---- context ------------------------------------------------------------------ */
+int lq4_ctx_create(int device_ordinal, lq4_ctx** out);
+int lq4_ctx_destroy(lq4_ctx* ctx);
+/* hipStreamSynchronize(stream); the counterpart of commit()+wait_until_completed()
+ * (forward/metal_qwen35.rs:6447). */
+int lq4_sync(lq4_ctx* ctx, void* stream);
+
+/* ---- weights: upload and residency ------------------------------------------- */
+/* Host-side per-block ingress rule = validate_q4_block_metadata_scan
+ * (q4_weights.rs:907-918; rule in weights/ingress.rs:542-559): every block's scale
+ * finite and > 0, bias finite.  On failure returns LQ4_E_BLOCK and stores the first
+ * offending block index and reason (1 = scale, 2 = bias). */
+int lq4_validate_blocks(const uint8_t* host_payload, size_t nbytes, int64_t* bad_block,
+                        int* reason);
+
+/* Replaces mmap_q4_weight + new_buffer_with_bytes_no_copy (metal_qwen35.rs:660-702):
+ * copies `nbytes` of host memory VERBATIM into a resident device allocation (no
+ * repacking).  `payload_offset` is where the block payload starts inside that buffer
+ * (36 for a whole 2-D .q4 file, 0 for raw blocks), as in Q4WeightBuf.  `validate` != 0
+ * runs lq4_validate_blocks over the payload first (Q4BlockCheck::Now,
+ * q4_weights.rs:926-947) and publishes nothing to the GPU if it fails. */
+int lq4_weight_upload(lq4_ctx* ctx, const uint8_t* host_bytes, size_t nbytes,
+                      uint64_t payload_offset, int validate, lq4_weight** out);
+/* Wraps bytes that already live on the device (caller keeps ownership and must keep
+ * them alive); used for buffers assembled on the GPU, e.g. fused gate||up
+ * (metal_qwen35.rs:12137-12152). */
+int lq4_weight_wrap(lq4_ctx* ctx, const void* blocks_dev, size_t nbytes, uint64_t payload_offset,
+                    lq4_weight** out);
+int lq4_weight_free(lq4_weight* w);
+/* Device address of byte 0 of the buffer (payload_offset not applied) and its size. */
+int lq4_weight_info(const lq4_weight* w, const void** base_dev, size_t* nbytes,
+                    uint64_t* payload_offset);
+
+/* ---- LoRA --------------------------------------------------------------------- */
+/* Replaces the per-projection upload in load_lora_adapter (metal_qwen35.rs:3806-3986):
+ * A is [rank, d_in], B is [d_out, rank], row-major, host memory, f32 (as the
+ * reference stores them) or f16.  rank <= LQ4_MAX_LORA_RANK. */
+int lq4_lora_upload(lq4_ctx* ctx, const void* a_host, const void* b_host, int dtype,
+                    uint32_t rank, uint32_t d_in, uint32_t d_out, lq4_lora** out);
+int lq4_lora_free(lq4_lora* l);
+
+/* Stand-alone form of dispatch_lora_if_active (layers/mod.rs:15-51), for callers that
+ * keep the base projection and the adapter as separate steps:
+ *   y[r, 0..d_out) += lora_scale * B . (A . x[r, 0..d_in))      for r < rows.
+ * ACCUMULATES into y.  A NULL `lora` (no adapter for this layer/module) is a no-op.
+ * x_dev: f32 or f16 [rows, d_in]; y_dev: f32 [rows, d_out]. */
+int lq4_lora_apply(lq4_ctx* ctx, const lq4_lora* lora, float lora_scale, const void* x_dev,
+                   int x_dtype, uint32_t rows, float* y_dev, void* stream);
+
+/* ---- decode GEMV ---------------------------------------------------------------
+ * Replaces dispatch_matmul / dispatch_matmul_q4 (dispatch.rs:148-168, 231-245) and
+ * the m == 1 arm of dispatch_gemm_q4 (dispatch.rs:190-200), extended to small
+ * batches so the weights stream from HBM once for all rows:
+ *   y[b, 0..N) = W . x[b, 0..K)            for b < batch (1..LQ4_MAX_GEMV_BATCH)
+ * and, when `lora` is non-NULL, the delta of dispatch_lora_if_active
+ * (layers/mod.rs:15-51) fused into the same store:
+ *   y[b, n] += lora_scale * sum_j B[n, j] * (sum_k A[j, k] * x[b, k]).
+ * x_dev: f32 [batch, K]; y_dev: f32 [batch, N]; W starts at
+ * payload_offset + w_extra_offset bytes into the weight buffer (qw_extra_offset of
+ * dispatch_gemm_at, dispatch.rs:935-980). */
+int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
+             const float* x_dev, uint32_t batch, float* y_dev, const lq4_lora* lora,
+             float lora_scale, void* stream);
+
+/* ---- prefill GEMM --------------------------------------------------------------
+ * Replaces dispatch_gemm / dispatch_gemm_at -> dispatch_gemm_q4[_at]
+ * (dispatch.rs:170-229, 507-525, 935-1097): Y[M,N] = X[M,K] . W^T, X f32 or f16
+ * (the reference's tiled kernel rounds f32 X to half in-tile,
+ * shaders/gemm_q4_tiled.metal:45-48), f32 accumulate, Y f32.  m <= LQ4_MAX_GEMV_BATCH
+ * with f32 X routes to the GEMV kernel, as m == 1 does in the reference.  Optional
+ * LoRA delta as in lq4_gemv, applied per row (apply_lora_rows,
+ * crates/inference/src/lora_hook.rs). */
+int lq4_gemm(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
+             const void* x_dev, int x_dtype, uint32_t m, float* y_dev, const lq4_lora* lora,
+             float lora_scale, void* stream);
+
+/* ---- MoE ----------------------------------------------------------------------
+ * Device restatement of compute_router_probs (from the logits on) + select_top_k +
+ * renormalize_selected (crates/inference/src/model/qwen35/moe.rs:39-125; GPU twin
+ * layers/mod.rs:226-289): softmax over all E, top-k by strict '>' (ties keep the lower
+ * id), selected weights renormalised to sum 1.  logits_dev f32 [tokens, E];
+ * ids_dev i32 [tokens, top_k] (-1 = unfilled slot); weights_dev f32 [tokens, top_k]. */
+int lq4_moe_route(lq4_ctx* ctx, const float* logits_dev, uint32_t tokens, uint32_t num_experts,
+                  uint32_t top_k, int32_t* ids_dev, float* weights_dev, void* stream);
+
+/* Replaces accumulate_routed_experts (moe.rs:127-190) / the expert part of
+ * encode_moe_ffn (layers/mod.rs:542-660), reading the experts' Q4 blocks directly
+ * instead of a CPU-dequantised f16 copy:
+ *   y[t,:] = sum_s weights[t,s] * W_down[e] . ( silu(W_gate[e] . x[t]) * (W_up[e] . x[t]) ),
+ *   e = ids[t,s]; slots with e outside [0, E) are skipped.
+ * gate_up: [E, 2*inter, hidden] (gate rows then up rows per expert); down:
+ * [E, hidden, inter]; both expert-major native blocks.  Tokens routed to the same
+ * expert share one pass over that expert's weights.  x_dev f32 [tokens, hidden];
+ * y_dev f32 [tokens, hidden] (overwritten).  tokens*top_k <= 4096. */
+int lq4_moe_grouped_gemv(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_weight* down,
+                         uint32_t num_experts, uint32_t inter, uint32_t hidden,
+                         const float* x_dev, uint32_t tokens, const int32_t* ids_dev,
+                         const float* weights_dev, uint32_t top_k, float* y_dev, void* stream);
+
+/* ---- probes --------------------------------------------------------------------
+ * Writes f32(nibble)*scale + bias for every weight of W[N,K] to out_dev (f32 [N,K]):
+ * the bit-exactness probe for nibble unpack and scale/bias indexing against
+ * dequantize_row_q4_0 (q4_weights.rs:340-353). */
+int lq4_dequant(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n,
+                uint32_t k, float* out_dev, void* stream);
+
+/* Launch counters per kernel family since context creation (the role of
+ * PathProofCounters, metal_qwen35.rs:2144-2190): proves which path served a call. */
+typedef struct lq4_path_counters {
+    uint64_t gemv, gemm, lora_a, moe_route, moe_gate_up, moe_down, dequant;
+} lq4_path_counters;
+int lq4_get_path_counters(const lq4_ctx* ctx, lq4_path_counters* out);
+
+/* ---- plain device-memory helpers for callers without a HIP binding ------------ */
+int lq4_malloc(lq4_ctx* ctx, size_t nbytes, void** out_dev);
+int lq4_free(lq4_ctx* ctx, void* p_dev);
+int lq4_memcpy_h2d(lq4_ctx* ctx, void* dst_dev, const void* src_host, size_t nbytes);
+int lq4_memcpy_d2h(lq4_ctx* ctx, void* dst_host, const void* src_dev, size_t nbytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LATTICE_HIP_Q4_H */

@@ -1,0 +1,378 @@
+"""Host-side mirror of the reference's Q4 dispatch contract, over the C ABI.
+
+The reference exposes this path as inherent methods of ``MetalQwen35State``
+(crates/inference/src/forward/metal_qwen35/inner/dispatch.rs and layers/mod.rs);
+:class:`HipQ4Backend` keeps the same method names, argument order, byte-offset
+convention and error behaviour so a parity test reads like the reference's own:
+
+=====================================  ===========================================
+reference                              here
+=====================================  ===========================================
+``Q4WeightBuf`` (metal_qwen35.rs:599)  :class:`Q4WeightBuf`
+``mmap_q4_weight`` (:660)              :meth:`HipQ4Backend.mmap_q4_weight`
+``make_buffer_q4_0`` (:2362)           :meth:`HipQ4Backend.upload_q4_blocks`
+``dispatch_matmul`` (dispatch.rs:231)  :meth:`HipQ4Backend.dispatch_matmul`
+``dispatch_gemm`` (:507)               :meth:`HipQ4Backend.dispatch_gemm`
+``dispatch_gemm_at`` (:935)            :meth:`HipQ4Backend.dispatch_gemm_at`
+``load_lora_adapter`` (mq35.rs:3806)   :meth:`HipQ4Backend.load_lora_adapter`
+``dispatch_lora_if_active`` (mod.rs:15) :meth:`HipQ4Backend.dispatch_lora_if_active`
+=====================================  ===========================================
+
+Device buffers are torch CUDA tensors (torch is only the allocator and stream
+provider); every computation goes through ``liblattice_hip_q4.so``.  There is no CPU
+fallback: a missing library raises :class:`Q4LibraryMissing` at first use.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+
+from . import q4_file
+from .q4_layout import BLOCK_BYTES, BLOCK_WEIGHTS
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "liblattice_hip_q4.so")
+
+LQ4_F32, LQ4_F16 = 0, 1
+MAX_GEMV_BATCH = 16
+
+EXPORTS = [
+    "lq4_last_error", "lq4_version", "lq4_ctx_create", "lq4_ctx_destroy", "lq4_sync",
+    "lq4_validate_blocks", "lq4_weight_upload", "lq4_weight_wrap", "lq4_weight_free",
+    "lq4_weight_info", "lq4_lora_upload", "lq4_lora_free", "lq4_lora_apply", "lq4_gemv",
+    "lq4_gemm", "lq4_moe_route", "lq4_moe_grouped_gemv", "lq4_dequant",
+    "lq4_get_path_counters", "lq4_malloc", "lq4_free", "lq4_memcpy_h2d", "lq4_memcpy_d2h",
+]
+
+
+class Q4LibraryMissing(RuntimeError):
+    pass
+
+
+class Q4Error(RuntimeError):
+    """A C-ABI call returned a negative code; ``code`` is the LQ4_E_* value."""
+
+    def __init__(self, code: int, message: str):
+        super().__init__(f"[{code}] {message}")
+        self.code = code
+        self.message = message
+
+
+class PathCounters(C.Structure):
+    _fields_ = [(n, C.c_uint64) for n in ("gemv", "gemm", "lora_a", "moe_route", "moe_gate_up",
+                                         "moe_down", "dequant")]
+
+
+_lib = None
+
+
+def load_library() -> C.CDLL:
+    """Loads the in-tree shared library (after torch, so both share one HIP runtime)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise Q4LibraryMissing(
+            f"{LIB_PATH} is not built; run `python -m lattice_amd.build` (there is no CPU fallback)")
+    import torch  # noqa: F401  (loads libamdhip64 first)
+    L = C.CDLL(LIB_PATH)
+    vp, u32, u64, f32 = C.c_void_p, C.c_uint32, C.c_uint64, C.c_float
+    sig = {
+        "lq4_last_error": (C.c_char_p, []),
+        "lq4_version": (C.c_char_p, []),
+        "lq4_ctx_create": (C.c_int, [C.c_int, C.POINTER(vp)]),
+        "lq4_ctx_destroy": (C.c_int, [vp]),
+        "lq4_sync": (C.c_int, [vp, vp]),
+        "lq4_validate_blocks": (C.c_int, [vp, C.c_size_t, C.POINTER(C.c_int64), C.POINTER(C.c_int)]),
+        "lq4_weight_upload": (C.c_int, [vp, vp, C.c_size_t, u64, C.c_int, C.POINTER(vp)]),
+        "lq4_weight_wrap": (C.c_int, [vp, vp, C.c_size_t, u64, C.POINTER(vp)]),
+        "lq4_weight_free": (C.c_int, [vp]),
+        "lq4_weight_info": (C.c_int, [vp, C.POINTER(vp), C.POINTER(C.c_size_t), C.POINTER(u64)]),
+        "lq4_lora_upload": (C.c_int, [vp, vp, vp, C.c_int, u32, u32, u32, C.POINTER(vp)]),
+        "lq4_lora_free": (C.c_int, [vp]),
+        "lq4_lora_apply": (C.c_int, [vp, vp, f32, vp, C.c_int, u32, vp, vp]),
+        "lq4_gemv": (C.c_int, [vp, vp, u64, u32, u32, vp, u32, vp, vp, f32, vp]),
+        "lq4_gemm": (C.c_int, [vp, vp, u64, u32, u32, vp, C.c_int, u32, vp, vp, f32, vp]),
+        "lq4_moe_route": (C.c_int, [vp, vp, u32, u32, u32, vp, vp, vp]),
+        "lq4_moe_grouped_gemv": (C.c_int, [vp, vp, vp, u32, u32, u32, vp, u32, vp, vp, u32, vp, vp]),
+        "lq4_dequant": (C.c_int, [vp, vp, u64, u32, u32, vp, vp]),
+        "lq4_get_path_counters": (C.c_int, [vp, C.POINTER(PathCounters)]),
+        "lq4_malloc": (C.c_int, [vp, C.c_size_t, C.POINTER(vp)]),
+        "lq4_free": (C.c_int, [vp, vp]),
+        "lq4_memcpy_h2d": (C.c_int, [vp, vp, vp, C.c_size_t]),
+        "lq4_memcpy_d2h": (C.c_int, [vp, vp, vp, C.c_size_t]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(L, name)
+        fn.restype, fn.argtypes = res, args
+    _lib = L
+    return L
+
+
+def _check(rc: int):
+    if rc != 0:
+        raise Q4Error(rc, load_library().lq4_last_error().decode(errors="replace"))
+
+
+def validate_blocks(payload) -> None:
+    """Host-side ``Q4BlockCheck::Now`` (q4_weights.rs:907-947): raises :class:`Q4Error`
+    naming the first block whose scale is non-finite or non-positive or whose bias is
+    non-finite.  Needs no GPU."""
+    buf = np.ascontiguousarray(np.frombuffer(payload, dtype=np.uint8) if isinstance(
+        payload, (bytes, bytearray, memoryview)) else payload, dtype=np.uint8)
+    _check(load_library().lq4_validate_blocks(buf.ctypes.data, buf.size, None, None))
+
+
+@dataclass
+class Q4WeightBuf:
+    """Device-resident Q4 buffer plus the byte offset of its block payload
+    (``Q4WeightBuf { buffer, payload_offset, .. }``, metal_qwen35.rs:599-636)."""
+    handle: int
+    nbytes: int
+    payload_offset: int
+    _backend: "HipQ4Backend"
+    _keepalive: object = None
+
+    def free(self):
+        if self.handle:
+            _check(load_library().lq4_weight_free(self.handle))
+            self.handle = 0
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+@dataclass
+class LoraLayerData:
+    """One layer's adapter factors (metal_qwen35.rs:1701-1716): ``modules`` maps a
+    projection name ("q_proj", "v_proj", ...) to ``(A [rank, d_in], B [d_out, rank])``."""
+    layer_idx: int
+    modules: Dict[str, Tuple[np.ndarray, np.ndarray]]
+
+
+class _LoraProjection:
+    def __init__(self, handle, rank, d_in, d_out):
+        self.handle, self.rank, self.d_in, self.d_out = handle, rank, d_in, d_out
+
+
+def _dtype_code(t) -> int:
+    import torch
+    if t.dtype == torch.float32:
+        return LQ4_F32
+    if t.dtype == torch.float16:
+        return LQ4_F16
+    raise TypeError(f"activations must be float32 or float16, got {t.dtype}")
+
+
+class HipQ4Backend:
+    """One GPU's Q4 matmul backend: owns a ``lq4_ctx`` and the loaded LoRA adapter."""
+
+    def __init__(self, device: int = 0):
+        import torch
+        if not torch.cuda.is_available():
+            raise RuntimeError("HipQ4Backend needs a HIP device; there is no CPU fallback")
+        self.lib = load_library()
+        self.device = device
+        self.torch_device = torch.device("cuda", device)
+        ctx = C.c_void_p()
+        _check(self.lib.lq4_ctx_create(device, C.byref(ctx)))
+        self.ctx = ctx
+        self._lora: Dict[Tuple[int, str], _LoraProjection] = {}
+        self._lora_scale = 0.0
+
+    def close(self):
+        self.unload_lora_adapter()
+        if self.ctx:
+            self.lib.lq4_ctx_destroy(self.ctx)
+            self.ctx = None
+
+    # ------------------------------------------------------------------ helpers
+    def _stream(self):
+        import torch
+        return C.c_void_p(torch.cuda.current_stream(self.torch_device).cuda_stream)
+
+    def synchronize(self):
+        _check(self.lib.lq4_sync(self.ctx, self._stream()))
+
+    def path_counters(self) -> Dict[str, int]:
+        pc = PathCounters()
+        _check(self.lib.lq4_get_path_counters(self.ctx, C.byref(pc)))
+        return {n: int(getattr(pc, n)) for n, _ in PathCounters._fields_}
+
+    # ------------------------------------------------------- weights / residency
+    def upload_q4_blocks(self, blocks, payload_offset: int = 0, validate: bool = True) -> Q4WeightBuf:
+        """Uploads host bytes verbatim (``make_buffer_q4_0``, metal_qwen35.rs:2362-2378, for raw
+        blocks; the whole-file no-copy buffer of ``mmap_q4_weight`` when ``payload_offset`` > 0)."""
+        buf = np.ascontiguousarray(np.frombuffer(blocks, dtype=np.uint8) if isinstance(
+            blocks, (bytes, bytearray, memoryview)) else blocks, dtype=np.uint8)
+        h = C.c_void_p()
+        _check(self.lib.lq4_weight_upload(self.ctx, buf.ctypes.data, buf.size, payload_offset,
+                                          int(validate), C.byref(h)))
+        return Q4WeightBuf(h.value, buf.size, payload_offset, self)
+
+    def wrap_device_blocks(self, t, payload_offset: int = 0) -> Q4WeightBuf:
+        """Adopts a uint8 CUDA tensor that already holds native blocks (kept alive by the
+        returned buffer); e.g. a fused gate||up buffer (metal_qwen35.rs:12137-12152)."""
+        import torch
+        assert t.is_cuda and t.dtype == torch.uint8 and t.is_contiguous()
+        h = C.c_void_p()
+        _check(self.lib.lq4_weight_wrap(self.ctx, t.data_ptr(), t.numel(), payload_offset, C.byref(h)))
+        return Q4WeightBuf(h.value, t.numel(), payload_offset, self, _keepalive=t)
+
+    def mmap_q4_weight(self, path: str, label: str, expected_shape: Sequence[int]) -> Q4WeightBuf:
+        """``mmap_q4_weight(device, path, label, expected_shape)`` (metal_qwen35.rs:660-702):
+        header + exact-extent + shape preflight, per-block scale/bias scan, then the whole
+        file becomes one resident buffer with ``payload_offset`` past the header."""
+        data = np.memmap(path, dtype=np.uint8, mode="r")
+        try:
+            header = q4_file.validate_q4_file(data, path, expected_shape)
+        except q4_file.Q4FileError as e:
+            raise Q4Error(-1, f"failed to validate Q4 payload {path}: {e}") from None
+        try:
+            return self.upload_q4_blocks(data, payload_offset=header.payload_offset, validate=True)
+        except Q4Error as e:
+            raise Q4Error(e.code, f"{path}: tensor {label} (Q4): {e.message}") from None
+
+    # ---------------------------------------------------------------- dispatch
+    @staticmethod
+    def _assert_k(k: int, who: str):
+        # the reference panics here (dispatch.rs:185-188)
+        assert k > 0 and k % BLOCK_WEIGHTS == 0, \
+            f"{who} requires K to be non-zero and divisible by 32, got {k}"
+
+    def _lora_for(self, layer_idx, module, n, k):
+        if layer_idx is None or module is None:
+            return None
+        proj = self._lora.get((layer_idx, module))
+        if proj is None:
+            return None
+        assert (proj.d_in, proj.d_out) == (k, n), "LoRA projection shape does not match the GEMV"
+        return proj.handle
+
+    def dispatch_matmul(self, x, qw: Q4WeightBuf, y, m: int, n: int, k: int, *, layer_idx=None,
+                        module=None):
+        """``dispatch_matmul(enc, x, qw, y, m, n, k)`` (dispatch.rs:231-245): decode GEMV
+        ``y[0..n) = W . x[0..k)``; ``m`` is ignored as in the reference.  Passing
+        ``layer_idx``/``module`` fuses that projection's LoRA delta into the same pass."""
+        if n == 0:
+            return
+        self._assert_k(k, "dispatch_matmul_q4")
+        lora = self._lora_for(layer_idx, module, n, k)
+        _check(self.lib.lq4_gemv(self.ctx, qw.handle, 0, n, k, x.data_ptr(), 1, y.data_ptr(), lora,
+                                 self._lora_scale, self._stream()))
+
+    def dispatch_gemm(self, x, x_offset: int, qw: Q4WeightBuf, y, y_offset: int, m: int, n: int,
+                      k: int, *, layer_idx=None, module=None):
+        """``dispatch_gemm`` (dispatch.rs:507-525 -> dispatch_gemm_q4 :170-229)."""
+        self.dispatch_gemm_at(x, x_offset, qw, 0, y, y_offset, m, n, k, layer_idx=layer_idx,
+                              module=module)
+
+    def dispatch_gemm_at(self, x, x_offset: int, qw: Q4WeightBuf, qw_extra_offset: int, y,
+                         y_offset: int, m: int, n: int, k: int, *, layer_idx=None, module=None):
+        """``dispatch_gemm_at`` (dispatch.rs:935-1097): offsets are bytes into ``x``, the weight
+        buffer (on top of ``payload_offset``) and ``y``; ``m == 0 or n == 0`` is a no-op;
+        small ``m`` with f32 activations takes the GEMV kernel (m == 1 in the reference)."""
+        if m == 0 or n == 0:
+            return
+        self._assert_k(k, "dispatch_gemm_q4")
+        lora = self._lora_for(layer_idx, module, n, k)
+        _check(self.lib.lq4_gemm(self.ctx, qw.handle, qw_extra_offset, n, k, x.data_ptr() + x_offset,
+                                 _dtype_code(x), m, y.data_ptr() + y_offset, lora, self._lora_scale,
+                                 self._stream()))
+
+    def gemv_batch(self, x, qw: Q4WeightBuf, y, batch: int, n: int, k: int, qw_extra_offset: int = 0,
+                   *, layer_idx=None, module=None):
+        """Small-batch decode: ``y[b] = W . x[b]`` for ``b < batch <= 16`` in one pass over W."""
+        if batch == 0 or n == 0:
+            return
+        self._assert_k(k, "dispatch_matmul_q4")
+        lora = self._lora_for(layer_idx, module, n, k)
+        _check(self.lib.lq4_gemv(self.ctx, qw.handle, qw_extra_offset, n, k, x.data_ptr(), batch,
+                                 y.data_ptr(), lora, self._lora_scale, self._stream()))
+
+    def dequantize(self, qw: Q4WeightBuf, n: int, k: int, qw_extra_offset: int = 0):
+        """f32 [n, k] tensor of ``f32(nibble)*scale + bias`` (bit-exactness probe)."""
+        import torch
+        self._assert_k(k, "dequantize")
+        out = torch.empty((n, k), dtype=torch.float32, device=self.torch_device)
+        _check(self.lib.lq4_dequant(self.ctx, qw.handle, qw_extra_offset, n, k, out.data_ptr(),
+                                    self._stream()))
+        return out
+
+    # -------------------------------------------------------------------- LoRA
+    def load_lora_adapter(self, layers: List[LoraLayerData], scale: float,
+                          quarot_seed: Optional[int] = None):
+        """``load_lora_adapter(layers, scale, quarot_seed)`` (metal_qwen35.rs:3806-3986): uploads
+        every projection's A/B, replacing any adapter already loaded; ``scale`` (= alpha/rank,
+        crates/fann/src/lora.rs:110-117) is applied verbatim.  Rotating A/B for a QuaRot
+        checkpoint is the offline converter's job and is not part of this path."""
+        if quarot_seed is not None:
+            raise Q4Error(-5, "QuaRot rotation of LoRA factors is not supported by this backend")
+        staged: Dict[Tuple[int, str], _LoraProjection] = {}
+        try:
+            for layer in layers:
+                for module, (a, b) in layer.modules.items():
+                    a = np.ascontiguousarray(a)
+                    b = np.ascontiguousarray(b)
+                    if a.ndim != 2 or b.ndim != 2 or b.shape[1] != a.shape[0]:
+                        raise Q4Error(-1, f"layer {layer.layer_idx} {module}: A {a.shape} / B {b.shape} "
+                                          "are not [rank, d_in] / [d_out, rank]")
+                    if a.dtype != b.dtype or a.dtype not in (np.float32, np.float16):
+                        raise Q4Error(-1, f"layer {layer.layer_idx} {module}: A and B must both be "
+                                          "float32 or float16")
+                    rank, d_in = a.shape
+                    d_out = b.shape[0]
+                    h = C.c_void_p()
+                    _check(self.lib.lq4_lora_upload(self.ctx, a.ctypes.data, b.ctypes.data,
+                                                    LQ4_F16 if a.dtype == np.float16 else LQ4_F32,
+                                                    rank, d_in, d_out, C.byref(h)))
+                    staged[(layer.layer_idx, module)] = _LoraProjection(h.value, rank, d_in, d_out)
+        except Exception:
+            for p in staged.values():
+                self.lib.lq4_lora_free(p.handle)
+            raise
+        self.unload_lora_adapter()
+        self._lora, self._lora_scale = staged, float(scale)
+
+    def unload_lora_adapter(self):
+        for p in self._lora.values():
+            self.lib.lq4_lora_free(p.handle)
+        self._lora, self._lora_scale = {}, 0.0
+
+    def dispatch_lora_if_active(self, x, x_byte_offset: int, y, y_byte_offset: int, layer_idx: int,
+                                module: str, rows: int = 1):
+        """``dispatch_lora_if_active`` (layers/mod.rs:15-51): ``y += scale * B.(A.x)``; a no-op
+        when no adapter is loaded or it has no projection for ``(layer_idx, module)``."""
+        proj = self._lora.get((layer_idx, module))
+        if proj is None:
+            return
+        _check(self.lib.lq4_lora_apply(self.ctx, proj.handle, self._lora_scale,
+                                       x.data_ptr() + x_byte_offset, _dtype_code(x), rows,
+                                       y.data_ptr() + y_byte_offset, self._stream()))
+
+    # --------------------------------------------------------------------- MoE
+    def moe_route(self, logits, top_k: int):
+        """Router softmax + top-k + renormalise on the device (moe.rs:39-125); returns
+        ``(ids int32 [T, top_k], weights f32 [T, top_k])``."""
+        import torch
+        t, e = logits.shape
+        ids = torch.empty((t, top_k), dtype=torch.int32, device=self.torch_device)
+        wts = torch.empty((t, top_k), dtype=torch.float32, device=self.torch_device)
+        _check(self.lib.lq4_moe_route(self.ctx, logits.data_ptr(), t, e, top_k, ids.data_ptr(),
+                                      wts.data_ptr(), self._stream()))
+        return ids, wts
+
+    def moe_experts(self, gate_up: Q4WeightBuf, down: Q4WeightBuf, num_experts: int, inter: int,
+                    hidden: int, x, ids, weights, y):
+        """Routed-expert FFN over Q4 expert tensors (moe.rs:127-190); ``y`` is overwritten."""
+        tokens, top_k = ids.shape
+        _check(self.lib.lq4_moe_grouped_gemv(self.ctx, gate_up.handle, down.handle, num_experts, inter,
+                                             hidden, x.data_ptr(), tokens, ids.data_ptr(),
+                                             weights.data_ptr(), top_k, y.data_ptr(), self._stream()))

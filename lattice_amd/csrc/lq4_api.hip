@@ -1,0 +1,464 @@
+// C ABI of liblattice_hip_q4.so (declared in include/lattice_hip_q4.h): argument and
+// bounds checking, device residency of weights and LoRA factors, and kernel dispatch.
+// Nothing here falls back to the CPU: without a working HIP device every entry point
+// that would launch returns LQ4_E_HIP.
+#include "../../include/lattice_hip_q4.h"
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+
+#include "lq4_internal.hpp"
+
+using namespace lq4;
+
+struct lq4_ctx {
+    int device;
+    float* lora_t;        // [kLoraTRows, kMaxLoraRank] f32: A.x of the call in flight
+    uint8_t* moe_scratch; // grown on demand
+    size_t moe_scratch_bytes;
+    lq4_path_counters counters;
+};
+
+struct lq4_weight {
+    lq4_ctx* ctx;
+    uint8_t* base;  // byte 0 of the uploaded buffer
+    size_t nbytes;
+    uint64_t payload_offset;
+    bool owned;
+};
+
+struct lq4_lora {
+    lq4_ctx* ctx;
+    void* a;  // [rank, d_in]
+    void* b;  // [d_out, rank]
+    int is_f16;
+    uint32_t rank, d_in, d_out;
+};
+
+namespace {
+
+constexpr uint32_t kLoraTRows = 4096;  // most rows one LoRA-fused call may carry
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+#define LQ4_HIP(call)                                                                     \
+    do {                                                                                  \
+        hipError_t e_ = (call);                                                           \
+        if (e_ != hipSuccess) return fail(LQ4_E_HIP, "%s: %s", #call, hipGetErrorString(e_)); \
+    } while (0)
+
+struct DeviceGuard {
+    int prev = -1;
+    bool ok = true;
+    explicit DeviceGuard(int dev) {
+        if (hipGetDevice(&prev) != hipSuccess) prev = -1;
+        if (prev != dev) ok = hipSetDevice(dev) == hipSuccess;
+    }
+    ~DeviceGuard() {
+        if (prev >= 0) (void)hipSetDevice(prev);
+    }
+};
+
+float half_bits_to_float(uint16_t h) {
+    // exact widening incl. subnormals (crates/inference/src/weights/half_bits.rs:24-53)
+    const uint32_t sign = (h >> 15) & 1u, exp = (h >> 10) & 0x1fu, frac = h & 0x3ffu;
+    float mag;
+    if (exp == 0) mag = std::ldexp(static_cast<float>(frac), -24);
+    else if (exp == 0x1f) mag = frac ? NAN : INFINITY;
+    else mag = std::ldexp(static_cast<float>(frac | 0x400u), static_cast<int>(exp) - 25);
+    return sign ? -mag : mag;
+}
+
+// Checks K and that W[n,k] lies inside the buffer; yields the device address of W.
+int resolve_weight(const lq4_weight* w, uint64_t extra, uint32_t n, uint32_t k,
+                   const uint8_t** out) {
+    if (!w) return fail(LQ4_E_INVALID, "weight handle is null");
+    if (k == 0 || k % kBlockWeights != 0)
+        return fail(LQ4_E_INVALID, "Q4 matmul requires K to be non-zero and divisible by 32, got %u", k);
+    const uint64_t need = static_cast<uint64_t>(n) * (k / kBlockWeights) * kBlockBytes;
+    const uint64_t start = w->payload_offset + extra;
+    if (start > w->nbytes || need > w->nbytes - start)
+        return fail(LQ4_E_INVALID, "W[%u,%u] at byte %llu needs %llu bytes but the buffer holds %zu", n, k,
+                    static_cast<unsigned long long>(start), static_cast<unsigned long long>(need), w->nbytes);
+    if (start % 4 != 0) return fail(LQ4_E_INVALID, "weight byte offset %llu is not 4-byte aligned",
+                                    static_cast<unsigned long long>(start));
+    *out = w->base + start;
+    return LQ4_OK;
+}
+
+int resolve_lora(const lq4_ctx* ctx, const lq4_lora* l, float scale, uint32_t n, uint32_t k,
+                 uint32_t rows, LoraEpilogue* out) {
+    *out = LoraEpilogue{nullptr, nullptr, 0, 0, 0.0f};
+    if (!l) return LQ4_OK;
+    if (l->d_in != k || l->d_out != n)
+        return fail(LQ4_E_INVALID, "LoRA is [%u -> %u] but the projection is [%u -> %u]", l->d_in, l->d_out, k, n);
+    if (rows > kLoraTRows) return fail(LQ4_E_UNSUPPORTED, "LoRA-fused call limited to %u rows, got %u", kLoraTRows, rows);
+    out->b = l->b;
+    out->t = ctx->lora_t;
+    out->rank = l->rank;
+    out->b_is_f16 = l->is_f16;
+    out->scale = scale;
+    return LQ4_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* lq4_last_error(void) { return g_err; }
+const char* lq4_version(void) { return "lattice-hip-q4 0.1 (gfx950)"; }
+
+int lq4_ctx_create(int device_ordinal, lq4_ctx** out) {
+    if (!out) return fail(LQ4_E_INVALID, "out is null");
+    *out = nullptr;
+    int count = 0;
+    LQ4_HIP(hipGetDeviceCount(&count));
+    if (device_ordinal < 0 || device_ordinal >= count)
+        return fail(LQ4_E_INVALID, "device %d out of range (%d visible)", device_ordinal, count);
+    DeviceGuard g(device_ordinal);
+    if (!g.ok) return fail(LQ4_E_HIP, "hipSetDevice(%d) failed", device_ordinal);
+    lq4_ctx* c = new (std::nothrow) lq4_ctx();
+    if (!c) return fail(LQ4_E_NOMEM, "out of host memory");
+    c->device = device_ordinal;
+    hipError_t e = hipMalloc(reinterpret_cast<void**>(&c->lora_t), sizeof(float) * kLoraTRows * kMaxLoraRank);
+    if (e != hipSuccess) {
+        delete c;
+        return fail(LQ4_E_HIP, "hipMalloc(lora scratch): %s", hipGetErrorString(e));
+    }
+    *out = c;
+    return LQ4_OK;
+}
+
+int lq4_ctx_destroy(lq4_ctx* ctx) {
+    if (!ctx) return LQ4_OK;
+    DeviceGuard g(ctx->device);
+    (void)hipFree(ctx->lora_t);
+    if (ctx->moe_scratch) (void)hipFree(ctx->moe_scratch);
+    delete ctx;
+    return LQ4_OK;
+}
+
+int lq4_sync(lq4_ctx* ctx, void* stream) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    LQ4_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    return LQ4_OK;
+}
+
+int lq4_validate_blocks(const uint8_t* p, size_t nbytes, int64_t* bad_block, int* reason) {
+    if (!p && nbytes) return fail(LQ4_E_INVALID, "payload is null");
+    const size_t nb = nbytes / kBlockBytes;
+    for (size_t i = 0; i < nb; ++i) {
+        const uint8_t* c = p + i * kBlockBytes;
+        const float scale = half_bits_to_float(static_cast<uint16_t>(c[0] | (c[1] << 8)));
+        const float bias = half_bits_to_float(static_cast<uint16_t>(c[2] | (c[3] << 8)));
+        int why = 0;
+        if (!std::isfinite(scale) || scale <= 0.0f) why = 1;
+        else if (!std::isfinite(bias)) why = 2;
+        if (why) {
+            if (bad_block) *bad_block = static_cast<int64_t>(i);
+            if (reason) *reason = why;
+            return why == 1
+                       ? fail(LQ4_E_BLOCK, "Q4 block %zu has invalid scale %g; scale must be finite and strictly positive", i, scale)
+                       : fail(LQ4_E_BLOCK, "Q4 block %zu has non-finite bias %g", i, bias);
+        }
+    }
+    if (bad_block) *bad_block = -1;
+    if (reason) *reason = 0;
+    return LQ4_OK;
+}
+
+int lq4_weight_upload(lq4_ctx* ctx, const uint8_t* host_bytes, size_t nbytes, uint64_t payload_offset,
+                      int validate, lq4_weight** out) {
+    if (!ctx || !host_bytes || !out) return fail(LQ4_E_INVALID, "null argument");
+    *out = nullptr;
+    if (payload_offset > nbytes) return fail(LQ4_E_INVALID, "payload_offset %llu beyond buffer length %zu",
+                                             static_cast<unsigned long long>(payload_offset), nbytes);
+    if (payload_offset % 4) return fail(LQ4_E_INVALID, "payload_offset must be 4-byte aligned");
+    if (validate) {
+        int rc = lq4_validate_blocks(host_bytes + payload_offset, nbytes - payload_offset, nullptr, nullptr);
+        if (rc) return rc;
+    }
+    DeviceGuard g(ctx->device);
+    lq4_weight* w = new (std::nothrow) lq4_weight{ctx, nullptr, nbytes, payload_offset, true};
+    if (!w) return fail(LQ4_E_NOMEM, "out of host memory");
+    hipError_t e = hipMalloc(reinterpret_cast<void**>(&w->base), nbytes ? nbytes : 4);
+    if (e == hipSuccess && nbytes) e = hipMemcpy(w->base, host_bytes, nbytes, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        if (w->base) (void)hipFree(w->base);
+        delete w;
+        return fail(LQ4_E_HIP, "weight upload (%zu bytes): %s", nbytes, hipGetErrorString(e));
+    }
+    *out = w;
+    return LQ4_OK;
+}
+
+int lq4_weight_wrap(lq4_ctx* ctx, const void* blocks_dev, size_t nbytes, uint64_t payload_offset,
+                    lq4_weight** out) {
+    if (!ctx || !blocks_dev || !out) return fail(LQ4_E_INVALID, "null argument");
+    if (payload_offset > nbytes || payload_offset % 4) return fail(LQ4_E_INVALID, "bad payload_offset");
+    if (reinterpret_cast<uintptr_t>(blocks_dev) % 4) return fail(LQ4_E_INVALID, "device buffer must be 4-byte aligned");
+    lq4_weight* w = new (std::nothrow) lq4_weight{
+        ctx, const_cast<uint8_t*>(static_cast<const uint8_t*>(blocks_dev)), nbytes, payload_offset, false};
+    if (!w) return fail(LQ4_E_NOMEM, "out of host memory");
+    *out = w;
+    return LQ4_OK;
+}
+
+int lq4_weight_free(lq4_weight* w) {
+    if (!w) return LQ4_OK;
+    if (w->owned) {
+        DeviceGuard g(w->ctx->device);
+        (void)hipFree(w->base);
+    }
+    delete w;
+    return LQ4_OK;
+}
+
+int lq4_weight_info(const lq4_weight* w, const void** base_dev, size_t* nbytes, uint64_t* payload_offset) {
+    if (!w) return fail(LQ4_E_INVALID, "weight handle is null");
+    if (base_dev) *base_dev = w->base;
+    if (nbytes) *nbytes = w->nbytes;
+    if (payload_offset) *payload_offset = w->payload_offset;
+    return LQ4_OK;
+}
+
+int lq4_lora_upload(lq4_ctx* ctx, const void* a_host, const void* b_host, int dtype, uint32_t rank,
+                    uint32_t d_in, uint32_t d_out, lq4_lora** out) {
+    if (!ctx || !a_host || !b_host || !out) return fail(LQ4_E_INVALID, "null argument");
+    *out = nullptr;
+    if (dtype != LQ4_F32 && dtype != LQ4_F16) return fail(LQ4_E_INVALID, "dtype must be LQ4_F32 or LQ4_F16");
+    if (rank == 0 || d_in == 0 || d_out == 0) return fail(LQ4_E_INVALID, "LoRA rank/d_in/d_out must be non-zero");
+    if (rank > kMaxLoraRank) return fail(LQ4_E_UNSUPPORTED, "LoRA rank %u above the supported maximum %d", rank, kMaxLoraRank);
+    const size_t es = dtype == LQ4_F16 ? 2 : 4;
+    DeviceGuard g(ctx->device);
+    lq4_lora* l = new (std::nothrow) lq4_lora{ctx, nullptr, nullptr, dtype == LQ4_F16, rank, d_in, d_out};
+    if (!l) return fail(LQ4_E_NOMEM, "out of host memory");
+    const size_t a_bytes = es * rank * d_in, b_bytes = es * d_out * rank;
+    hipError_t e = hipMalloc(&l->a, a_bytes);
+    if (e == hipSuccess) e = hipMalloc(&l->b, b_bytes);
+    if (e == hipSuccess) e = hipMemcpy(l->a, a_host, a_bytes, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(l->b, b_host, b_bytes, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        if (l->a) (void)hipFree(l->a);
+        if (l->b) (void)hipFree(l->b);
+        delete l;
+        return fail(LQ4_E_HIP, "LoRA upload: %s", hipGetErrorString(e));
+    }
+    *out = l;
+    return LQ4_OK;
+}
+
+int lq4_lora_free(lq4_lora* l) {
+    if (!l) return LQ4_OK;
+    DeviceGuard g(l->ctx->device);
+    (void)hipFree(l->a);
+    (void)hipFree(l->b);
+    delete l;
+    return LQ4_OK;
+}
+
+int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
+             const float* x_dev, uint32_t batch, float* y_dev, const lq4_lora* lora, float lora_scale,
+             void* stream) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    if (batch == 0 || n == 0) return LQ4_OK;
+    const uint8_t* wp;
+    int rc = resolve_weight(w, w_extra_offset, n, k, &wp);
+    if (rc) return rc;
+    if (!x_dev || !y_dev) return fail(LQ4_E_INVALID, "x/y device pointer is null");
+    if (batch > kMaxGemvBatch) return fail(LQ4_E_INVALID, "lq4_gemv batch %u above %d; use lq4_gemm", batch, kMaxGemvBatch);
+    if (reinterpret_cast<uintptr_t>(x_dev) % 16) return fail(LQ4_E_INVALID, "x must be 16-byte aligned");
+    if (reinterpret_cast<uintptr_t>(y_dev) % 4) return fail(LQ4_E_INVALID, "y must be 4-byte aligned");
+    LoraEpilogue ep;
+    rc = resolve_lora(ctx, lora, lora_scale, n, k, batch, &ep);
+    if (rc) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    DeviceGuard g(ctx->device);
+    if (ep.rank) {
+        launch_lora_a(lora->a, lora->is_f16, lora->rank, k, x_dev, 0, k, batch, ctx->lora_t, s);
+        ctx->counters.lora_a++;
+    }
+    launch_gemv(wp, n, k, x_dev, k, batch, y_dev, n, ep, s);
+    ctx->counters.gemv++;
+    LQ4_HIP(hipGetLastError());
+    return LQ4_OK;
+}
+
+int lq4_lora_apply(lq4_ctx* ctx, const lq4_lora* lora, float lora_scale, const void* x_dev, int x_dtype,
+                   uint32_t rows, float* y_dev, void* stream) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    if (!lora || rows == 0) return LQ4_OK;  // no adapter for this projection: no-op
+    if (!x_dev || !y_dev) return fail(LQ4_E_INVALID, "x/y device pointer is null");
+    if (x_dtype != LQ4_F32 && x_dtype != LQ4_F16) return fail(LQ4_E_INVALID, "x_dtype must be LQ4_F32 or LQ4_F16");
+    if (rows > kLoraTRows) return fail(LQ4_E_UNSUPPORTED, "LoRA call limited to %u rows, got %u", kLoraTRows, rows);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    DeviceGuard g(ctx->device);
+    launch_lora_a(lora->a, lora->is_f16, lora->rank, lora->d_in, x_dev, x_dtype == LQ4_F16, lora->d_in, rows,
+                  ctx->lora_t, s);
+    launch_lora_b_accum(lora->b, lora->is_f16, lora->rank, lora->d_out, ctx->lora_t, lora_scale, rows, y_dev,
+                        lora->d_out, s);
+    ctx->counters.lora_a++;
+    LQ4_HIP(hipGetLastError());
+    return LQ4_OK;
+}
+
+int lq4_gemm(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
+             const void* x_dev, int x_dtype, uint32_t m, float* y_dev, const lq4_lora* lora,
+             float lora_scale, void* stream) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    if (m == 0 || n == 0) return LQ4_OK;
+    if (x_dtype != LQ4_F32 && x_dtype != LQ4_F16) return fail(LQ4_E_INVALID, "x_dtype must be LQ4_F32 or LQ4_F16");
+    if (x_dtype == LQ4_F32 && m <= kMaxGemvBatch)
+        return lq4_gemv(ctx, w, w_extra_offset, n, k, static_cast<const float*>(x_dev), m, y_dev, lora, lora_scale, stream);
+    const uint8_t* wp;
+    int rc = resolve_weight(w, w_extra_offset, n, k, &wp);
+    if (rc) return rc;
+    if (!x_dev || !y_dev) return fail(LQ4_E_INVALID, "x/y device pointer is null");
+    if (reinterpret_cast<uintptr_t>(x_dev) % 16) return fail(LQ4_E_INVALID, "x must be 16-byte aligned");
+    if (reinterpret_cast<uintptr_t>(y_dev) % 4) return fail(LQ4_E_INVALID, "y must be 4-byte aligned");
+    LoraEpilogue ep;
+    rc = resolve_lora(ctx, lora, lora_scale, n, k, m, &ep);
+    if (rc) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    DeviceGuard g(ctx->device);
+    if (ep.rank) {
+        launch_lora_a(lora->a, lora->is_f16, lora->rank, k, x_dev, x_dtype == LQ4_F16, k, m, ctx->lora_t, s);
+        ctx->counters.lora_a++;
+    }
+    launch_gemm(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, ep, s);
+    ctx->counters.gemm++;
+    LQ4_HIP(hipGetLastError());
+    return LQ4_OK;
+}
+
+int lq4_moe_route(lq4_ctx* ctx, const float* logits_dev, uint32_t tokens, uint32_t num_experts,
+                  uint32_t top_k, int32_t* ids_dev, float* weights_dev, void* stream) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    if (tokens == 0) return LQ4_OK;
+    if (!logits_dev || !ids_dev || !weights_dev) return fail(LQ4_E_INVALID, "null device pointer");
+    if (top_k == 0 || top_k > 16 || top_k > num_experts)
+        return fail(LQ4_E_INVALID, "top_k must be in 1..min(16, num_experts), got %u", top_k);
+    DeviceGuard g(ctx->device);
+    launch_moe_route(logits_dev, tokens, num_experts, top_k, ids_dev, weights_dev, static_cast<hipStream_t>(stream));
+    ctx->counters.moe_route++;
+    LQ4_HIP(hipGetLastError());
+    return LQ4_OK;
+}
+
+int lq4_moe_grouped_gemv(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_weight* down,
+                         uint32_t num_experts, uint32_t inter, uint32_t hidden, const float* x_dev,
+                         uint32_t tokens, const int32_t* ids_dev, const float* weights_dev,
+                         uint32_t top_k, float* y_dev, void* stream) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    if (tokens == 0 || hidden == 0) return LQ4_OK;
+    if (!x_dev || !ids_dev || !weights_dev || !y_dev) return fail(LQ4_E_INVALID, "null device pointer");
+    if (num_experts == 0 || num_experts > 1024) return fail(LQ4_E_INVALID, "num_experts must be in 1..1024");
+    if (top_k == 0 || static_cast<uint64_t>(tokens) * top_k > 4096)
+        return fail(LQ4_E_INVALID, "tokens*top_k must be in 1..4096");
+    if (inter == 0 || inter % kBlockWeights)
+        return fail(LQ4_E_INVALID, "expert intermediate size must be a non-zero multiple of 32, got %u", inter);
+    if (reinterpret_cast<uintptr_t>(x_dev) % 16) return fail(LQ4_E_INVALID, "x must be 16-byte aligned");
+    const uint8_t *gu, *dn;
+    const uint64_t gu_rows = static_cast<uint64_t>(num_experts) * 2 * inter;
+    const uint64_t dn_rows = static_cast<uint64_t>(num_experts) * hidden;
+    if (gu_rows > UINT32_MAX || dn_rows > UINT32_MAX) return fail(LQ4_E_INVALID, "expert tensor too large");
+    int rc = resolve_weight(gate_up, 0, static_cast<uint32_t>(gu_rows), hidden, &gu);
+    if (rc) return rc;
+    rc = resolve_weight(down, 0, static_cast<uint32_t>(dn_rows), inter, &dn);
+    if (rc) return rc;
+
+    DeviceGuard g(ctx->device);
+    const size_t pairs = static_cast<size_t>(tokens) * top_k;
+    auto up256 = [](size_t v) { return (v + 255) / 256 * 256; };
+    const size_t off_counts = 0;
+    const size_t off_offsets = off_counts + up256(sizeof(int32_t) * num_experts);
+    const size_t off_order = off_offsets + up256(sizeof(int32_t) * (num_experts + 1));
+    const size_t off_h = off_order + up256(sizeof(int32_t) * pairs);
+    const size_t off_o = off_h + up256(sizeof(float) * pairs * inter);
+    const size_t total = off_o + up256(sizeof(float) * pairs * hidden);
+    if (total > ctx->moe_scratch_bytes) {
+        // growing the scratch is a synchronising allocation; steady-state calls reuse it
+        if (ctx->moe_scratch) {
+            LQ4_HIP(hipDeviceSynchronize());
+            (void)hipFree(ctx->moe_scratch);
+            ctx->moe_scratch = nullptr;
+            ctx->moe_scratch_bytes = 0;
+        }
+        LQ4_HIP(hipMalloc(reinterpret_cast<void**>(&ctx->moe_scratch), total));
+        ctx->moe_scratch_bytes = total;
+    }
+    MoeScratch s;
+    s.counts = reinterpret_cast<int32_t*>(ctx->moe_scratch + off_counts);
+    s.offsets = reinterpret_cast<int32_t*>(ctx->moe_scratch + off_offsets);
+    s.order = reinterpret_cast<int32_t*>(ctx->moe_scratch + off_order);
+    s.h = reinterpret_cast<float*>(ctx->moe_scratch + off_h);
+    s.o = reinterpret_cast<float*>(ctx->moe_scratch + off_o);
+    launch_moe_grouped(gu, dn, num_experts, inter, hidden, x_dev, tokens, ids_dev, weights_dev, top_k, y_dev, s,
+                       static_cast<hipStream_t>(stream));
+    ctx->counters.moe_gate_up++;
+    ctx->counters.moe_down++;
+    LQ4_HIP(hipGetLastError());
+    return LQ4_OK;
+}
+
+int lq4_dequant(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
+                float* out_dev, void* stream) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    if (n == 0) return LQ4_OK;
+    const uint8_t* wp;
+    int rc = resolve_weight(w, w_extra_offset, n, k, &wp);
+    if (rc) return rc;
+    if (!out_dev || reinterpret_cast<uintptr_t>(out_dev) % 8) return fail(LQ4_E_INVALID, "out must be non-null and 8-byte aligned");
+    DeviceGuard g(ctx->device);
+    launch_dequant(wp, n, k, out_dev, static_cast<hipStream_t>(stream));
+    ctx->counters.dequant++;
+    LQ4_HIP(hipGetLastError());
+    return LQ4_OK;
+}
+
+int lq4_get_path_counters(const lq4_ctx* ctx, lq4_path_counters* out) {
+    if (!ctx || !out) return fail(LQ4_E_INVALID, "null argument");
+    *out = ctx->counters;
+    return LQ4_OK;
+}
+
+int lq4_malloc(lq4_ctx* ctx, size_t nbytes, void** out_dev) {
+    if (!ctx || !out_dev) return fail(LQ4_E_INVALID, "null argument");
+    DeviceGuard g(ctx->device);
+    LQ4_HIP(hipMalloc(out_dev, nbytes ? nbytes : 4));
+    return LQ4_OK;
+}
+
+int lq4_free(lq4_ctx* ctx, void* p_dev) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    DeviceGuard g(ctx->device);
+    LQ4_HIP(hipFree(p_dev));
+    return LQ4_OK;
+}
+
+int lq4_memcpy_h2d(lq4_ctx* ctx, void* dst_dev, const void* src_host, size_t nbytes) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    DeviceGuard g(ctx->device);
+    LQ4_HIP(hipMemcpy(dst_dev, src_host, nbytes, hipMemcpyHostToDevice));
+    return LQ4_OK;
+}
+
+int lq4_memcpy_d2h(lq4_ctx* ctx, void* dst_host, const void* src_dev, size_t nbytes) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    DeviceGuard g(ctx->device);
+    LQ4_HIP(hipMemcpy(dst_host, src_dev, nbytes, hipMemcpyDeviceToHost));
+    return LQ4_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,187 @@
+// Decode GEMV over native Q4 blocks: y[b, n] = sum_k W[n, k] * x[b, k].
+//
+// Memory-bound: every weight byte is read exactly once per call and shared by all
+// batch rows.  Bias is factored out of the inner loop the way the reference kernel
+// does it (crates/inference/src/forward/shaders/qwen35.metal:838-847):
+//   sum_k (q_k*d + b) * x_k  =  d * sum_k q_k x_k  +  b * sum_k x_k     per block.
+#include "lq4_internal.hpp"
+
+namespace lq4 {
+
+namespace {
+
+constexpr int kWavesPerBlock = 4;
+constexpr int kRowsPerWave = 2;
+constexpr int kRowsPerBlock = kWavesPerBlock * kRowsPerWave;
+
+__device__ __forceinline__ float load_b(const void* b, int is_f16, size_t idx) {
+    return is_f16 ? static_cast<float>(static_cast<const _Float16*>(b)[idx])
+                  : static_cast<const float*>(b)[idx];
+}
+
+// One wave owns kRowsPerWave weight rows.  Lane l works on packed dword (l & 3) of
+// block (l >> 2) + 16*i: 8 consecutive weights against 8 consecutive activations.
+template <int NB>
+__global__ __launch_bounds__(kWavesPerBlock * 64) void gemv_q4_rows(
+    const uint8_t* __restrict__ w, uint32_t n, uint32_t k, const float* __restrict__ x,
+    uint32_t x_stride, uint32_t batch, float* __restrict__ y, uint32_t y_stride,
+    LoraEpilogue lora) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const uint32_t row0 = blockIdx.x * kRowsPerBlock + wave * kRowsPerWave;
+    if (row0 >= n) return;
+    const uint32_t nb = k / kBlockWeights;
+    const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
+
+    float acc[kRowsPerWave][NB];
+#pragma unroll
+    for (int r = 0; r < kRowsPerWave; ++r)
+#pragma unroll
+        for (int b = 0; b < NB; ++b) acc[r][b] = 0.0f;
+
+    const uint8_t* rowp[kRowsPerWave];
+#pragma unroll
+    for (int r = 0; r < kRowsPerWave; ++r) {
+        // rows past N re-read the last valid row; their result is never stored
+        const uint32_t row = row0 + r < n ? row0 + r : n - 1;
+        rowp[r] = w + row * row_bytes;
+    }
+    const float* xrow[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+        xrow[b] = x + static_cast<size_t>(b < static_cast<int>(batch) ? b : 0) * x_stride;
+
+    q4_rows_dot<kRowsPerWave, NB>(rowp, nb, xrow, lane, acc);
+
+#pragma unroll
+    for (int r = 0; r < kRowsPerWave; ++r)
+#pragma unroll
+        for (int b = 0; b < NB; ++b) acc[r][b] = wave_sum(acc[r][b]);
+
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < kRowsPerWave; ++r) {
+            const uint32_t row = row0 + r;
+            if (row >= n) continue;
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                if (b >= static_cast<int>(batch)) continue;
+                float v = acc[r][b];
+                if (lora.rank) {
+                    float s = 0.0f;
+                    for (uint32_t j = 0; j < lora.rank; ++j)
+                        s += load_b(lora.b, lora.b_is_f16, static_cast<size_t>(row) * lora.rank + j) *
+                             lora.t[b * lora.rank + j];
+                    v += lora.scale * s;
+                }
+                y[static_cast<size_t>(b) * y_stride + row] = v;
+            }
+        }
+    }
+}
+
+// t[row, j] = A[j, :] . x[row, :]   — one workgroup per (j, row).
+template <typename TA, typename TX>
+__global__ __launch_bounds__(256) void lora_a_kernel(const TA* __restrict__ a, uint32_t rank,
+                                                     uint32_t d_in, const TX* __restrict__ x,
+                                                     uint32_t x_stride, float* __restrict__ t) {
+    const uint32_t j = blockIdx.x, row = blockIdx.y;
+    const TA* ar = a + static_cast<size_t>(j) * d_in;
+    const TX* xr = x + static_cast<size_t>(row) * x_stride;
+    float p = 0.0f;
+    for (uint32_t kk = threadIdx.x; kk < d_in; kk += 256)
+        p = fmaf(static_cast<float>(ar[kk]), static_cast<float>(xr[kk]), p);
+    p = wave_sum(p);
+    __shared__ float part[4];
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = p;
+    __syncthreads();
+    if (threadIdx.x == 0) t[row * rank + j] = (part[0] + part[1]) + (part[2] + part[3]);
+}
+
+// y[row, n] += scale * sum_j B[n, j] * t[row, j]   (sequential over j, as
+// lora_gemv_b_accum does, shaders/qwen35.metal:2300-2320)
+__global__ __launch_bounds__(256) void lora_b_accum_kernel(const void* __restrict__ b, int b_is_f16,
+                                                           uint32_t rank, uint32_t d_out,
+                                                           const float* __restrict__ t, float scale,
+                                                           float* __restrict__ y, uint32_t y_stride) {
+    const uint32_t nn = blockIdx.x * 256 + threadIdx.x, row = blockIdx.y;
+    if (nn >= d_out) return;
+    float s = 0.0f;
+    for (uint32_t j = 0; j < rank; ++j)
+        s += load_b(b, b_is_f16, static_cast<size_t>(nn) * rank + j) * t[row * rank + j];
+    y[static_cast<size_t>(row) * y_stride + nn] += scale * s;
+}
+
+__global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict__ w,
+                                                      uint64_t n_blocks, float* __restrict__ out) {
+    // one thread per packed byte: two weights, w = f32(nibble)*scale + bias with a
+    // rounded multiply followed by a rounded add (q4_weights.rs:347-349)
+    const uint64_t idx = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= n_blocks * 16) return;
+    const uint64_t blk = idx >> 4;
+    const uint32_t byte_i = idx & 15;
+    const uint8_t* p = w + blk * kBlockBytes;
+    const float d = f16_bits_to_f32(p[0] | (static_cast<uint32_t>(p[1]) << 8));
+    const float b = f16_bits_to_f32(p[2] | (static_cast<uint32_t>(p[3]) << 8));
+    const uint32_t q = p[4 + byte_i];
+    float2 r;
+    r.x = __fadd_rn(__fmul_rn(static_cast<float>(q & 0xfu), d), b);
+    r.y = __fadd_rn(__fmul_rn(static_cast<float>(q >> 4), d), b);
+    reinterpret_cast<float2*>(out)[idx] = r;
+}
+
+}  // namespace
+
+void launch_gemv(const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint32_t x_stride,
+                 uint32_t batch, float* y, uint32_t y_stride, const LoraEpilogue& lora,
+                 hipStream_t stream) {
+    const dim3 grid((n + kRowsPerBlock - 1) / kRowsPerBlock), block(kWavesPerBlock * 64);
+    // batches above 8 run as two passes over the weights
+    for (uint32_t b0 = 0; b0 < batch; b0 += 8) {
+        const uint32_t nb = batch - b0 < 8 ? batch - b0 : 8;
+        const float* xb = x + static_cast<size_t>(b0) * x_stride;
+        float* yb = y + static_cast<size_t>(b0) * y_stride;
+        LoraEpilogue l = lora;
+        if (l.rank) l.t = lora.t + static_cast<size_t>(b0) * lora.rank;
+        if (nb == 1)
+            hipLaunchKernelGGL(gemv_q4_rows<1>, grid, block, 0, stream, w, n, k, xb, x_stride, nb, yb, y_stride, l);
+        else if (nb == 2)
+            hipLaunchKernelGGL(gemv_q4_rows<2>, grid, block, 0, stream, w, n, k, xb, x_stride, nb, yb, y_stride, l);
+        else if (nb <= 4)
+            hipLaunchKernelGGL(gemv_q4_rows<4>, grid, block, 0, stream, w, n, k, xb, x_stride, nb, yb, y_stride, l);
+        else
+            hipLaunchKernelGGL(gemv_q4_rows<8>, grid, block, 0, stream, w, n, k, xb, x_stride, nb, yb, y_stride, l);
+    }
+}
+
+void launch_lora_a(const void* a, int a_is_f16, uint32_t rank, uint32_t d_in, const void* x,
+                   int x_is_f16, uint32_t x_stride, uint32_t rows, float* t, hipStream_t stream) {
+    const dim3 grid(rank, rows), block(256);
+    if (a_is_f16 && x_is_f16)
+        hipLaunchKernelGGL((lora_a_kernel<_Float16, _Float16>), grid, block, 0, stream,
+                           static_cast<const _Float16*>(a), rank, d_in, static_cast<const _Float16*>(x), x_stride, t);
+    else if (a_is_f16)
+        hipLaunchKernelGGL((lora_a_kernel<_Float16, float>), grid, block, 0, stream,
+                           static_cast<const _Float16*>(a), rank, d_in, static_cast<const float*>(x), x_stride, t);
+    else if (x_is_f16)
+        hipLaunchKernelGGL((lora_a_kernel<float, _Float16>), grid, block, 0, stream,
+                           static_cast<const float*>(a), rank, d_in, static_cast<const _Float16*>(x), x_stride, t);
+    else
+        hipLaunchKernelGGL((lora_a_kernel<float, float>), grid, block, 0, stream,
+                           static_cast<const float*>(a), rank, d_in, static_cast<const float*>(x), x_stride, t);
+}
+
+void launch_lora_b_accum(const void* b, int b_is_f16, uint32_t rank, uint32_t d_out, const float* t,
+                         float scale, uint32_t rows, float* y, uint32_t y_stride, hipStream_t stream) {
+    hipLaunchKernelGGL(lora_b_accum_kernel, dim3((d_out + 255) / 256, rows), dim3(256), 0, stream, b,
+                       b_is_f16, rank, d_out, t, scale, y, y_stride);
+}
+
+void launch_dequant(const uint8_t* w, uint32_t n, uint32_t k, float* out, hipStream_t stream) {
+    const uint64_t n_blocks = static_cast<uint64_t>(n) * (k / kBlockWeights);
+    const uint64_t threads = n_blocks * 16;
+    hipLaunchKernelGGL(dequant_kernel, dim3(static_cast<uint32_t>((threads + 255) / 256)), dim3(256), 0,
+                       stream, w, n_blocks, out);
+}
+
+}  // namespace lq4

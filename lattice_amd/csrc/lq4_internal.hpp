@@ -1,0 +1,125 @@
+// Internal declarations shared by the translation units of liblattice_hip_q4.so.
+// Kernel launchers validate nothing: the C ABI layer (lq4_api.hip) checks every
+// shape, alignment and bound before a launcher is called.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace lq4 {
+
+constexpr int kBlockBytes = 20;    // one Q4 block: u16 scale, u16 bias, 16 packed bytes
+constexpr int kBlockWeights = 32;  // weights per block
+constexpr int kMaxLoraRank = 64;
+constexpr int kMaxGemvBatch = 16;
+
+// Optional LoRA epilogue operands.  t = A.x is produced by launch_lora_a into
+// ctx scratch before the main kernel runs; the main kernel adds
+// scale * sum_j B[n,j] * t[row,j] before its single store of y.
+struct LoraEpilogue {
+    const void* b;     // [d_out, rank] row-major, f32 or f16
+    const float* t;    // [rows, rank] f32
+    uint32_t rank;     // 0 = no LoRA
+    int b_is_f16;
+    float scale;
+};
+
+// y[b, n] = W . x[b]  (+ LoRA), b < batch <= kMaxGemvBatch.  x rows are `x_stride`
+// floats apart, y rows `y_stride` floats apart.
+void launch_gemv(const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint32_t x_stride,
+                 uint32_t batch, float* y, uint32_t y_stride, const LoraEpilogue& lora,
+                 hipStream_t stream);
+
+// t[row, j] = sum_k A[j, k] * x[row, k]; x f32 or f16 with row stride x_stride elements.
+void launch_lora_a(const void* a, int a_is_f16, uint32_t rank, uint32_t d_in, const void* x,
+                   int x_is_f16, uint32_t x_stride, uint32_t rows, float* t, hipStream_t stream);
+
+// y[row, n] += scale * sum_j B[n, j] * t[row, j]  for row < rows.
+void launch_lora_b_accum(const void* b, int b_is_f16, uint32_t rank, uint32_t d_out, const float* t,
+                         float scale, uint32_t rows, float* y, uint32_t y_stride, hipStream_t stream);
+
+// Y[M,N] = X[M,K] . W^T (+ LoRA); X f32 or f16, Y f32.
+void launch_gemm(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
+                 float* y, const LoraEpilogue& lora, hipStream_t stream);
+
+void launch_dequant(const uint8_t* w, uint32_t n, uint32_t k, float* out, hipStream_t stream);
+
+void launch_moe_route(const float* logits, uint32_t tokens, uint32_t num_experts, uint32_t top_k,
+                      int32_t* ids, float* weights, hipStream_t stream);
+
+// Scratch layout for the grouped MoE path, all sized by the caller:
+//   counts  i32 [E]        pairs routed to each expert
+//   offsets i32 [E + 1]    exclusive prefix of counts
+//   order   i32 [P]        pair indices (token*top_k + slot) sorted by expert, stable
+//   h       f32 [P, inter] silu(gate)*up per pair
+//   o       f32 [P, hidden] down-projection per pair
+struct MoeScratch {
+    int32_t* counts;
+    int32_t* offsets;
+    int32_t* order;
+    float* h;
+    float* o;
+};
+void launch_moe_grouped(const uint8_t* gate_up, const uint8_t* down, uint32_t num_experts,
+                        uint32_t inter, uint32_t hidden, const float* x, uint32_t tokens,
+                        const int32_t* ids, const float* weights, uint32_t top_k, float* y,
+                        const MoeScratch& s, hipStream_t stream);
+
+// ---- device helpers ---------------------------------------------------------------
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t bits16) {
+    // v_cvt_f32_f16 widens exactly, subnormals included (f16 denormals are not flushed
+    // in the default HIP float mode).
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(bits16)));
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+// Shared inner loop of the GEMV-class kernels.  One wave accumulates R weight rows
+// (rowp[r] = first block of row r) against NB activation rows (xrow[b]), each of
+// `nb` blocks / nb*32 floats.  Lane l handles packed dword (l & 3) of blocks
+// (l >> 2), (l >> 2) + 16, ...: 8 consecutive weights against 8 consecutive
+// activations.  acc holds per-lane partial sums; the caller reduces across the wave.
+// Every xrow[b] must be 16-byte aligned.
+template <int R, int NB>
+__device__ __forceinline__ void q4_rows_dot(const uint8_t* const (&rowp)[R], uint32_t nb,
+                                            const float* const (&xrow)[NB], int lane,
+                                            float (&acc)[R][NB]) {
+    const int il = lane & 3;
+    for (uint32_t ib = lane >> 2; ib < nb; ib += 16) {
+        float xv[NB][8];
+        float xs[NB];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const float4* xp = reinterpret_cast<const float4*>(xrow[b] + ib * kBlockWeights + il * 8);
+            const float4 lo = xp[0], hi = xp[1];
+            xv[b][0] = lo.x; xv[b][1] = lo.y; xv[b][2] = lo.z; xv[b][3] = lo.w;
+            xv[b][4] = hi.x; xv[b][5] = hi.y; xv[b][6] = hi.z; xv[b][7] = hi.w;
+            xs[b] = ((lo.x + lo.y) + (lo.z + lo.w)) + ((hi.x + hi.y) + (hi.z + hi.w));
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const uint32_t* blk =
+                reinterpret_cast<const uint32_t*>(rowp[r] + static_cast<size_t>(ib) * kBlockBytes);
+            const uint32_t sb = blk[0];
+            const uint32_t q = blk[1 + il];
+            const float d = f16_bits_to_f32(sb & 0xffffu);
+            const float bias = f16_bits_to_f32(sb >> 16);
+            float qf[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) qf[i] = static_cast<float>((q >> (4 * i)) & 0xfu);
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                float s = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) s = fmaf(qf[i], xv[b][i], s);
+                acc[r][b] = fmaf(s, d, fmaf(bias, xs[b], acc[r][b]));
+            }
+        }
+    }
+}
+
+}  // namespace lq4

@@ -1,0 +1,213 @@
+// MoE routing and grouped expert GEMV over native Q4 expert tensors.
+//
+// Routing restates compute_router_probs / select_top_k / renormalize_selected
+// (crates/inference/src/model/qwen35/moe.rs:39-125).  The expert pass groups the
+// (token, slot) pairs by expert so each routed expert's blocks stream from HBM once
+// for all of its tokens, then combines per token in slot order, the order
+// accumulate_routed_experts uses (moe.rs:127-190).
+#include "lq4_internal.hpp"
+
+namespace lq4 {
+
+namespace {
+
+constexpr int kMaxTopK = 16;
+constexpr int kMaxExperts = 1024;
+
+__global__ void moe_route_kernel(const float* __restrict__ logits, uint32_t tokens,
+                                 uint32_t num_experts, uint32_t top_k, int32_t* __restrict__ ids,
+                                 float* __restrict__ weights) {
+    const uint32_t t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= tokens) return;
+    const float* lg = logits + static_cast<size_t>(t) * num_experts;
+    float mx = -INFINITY;
+    for (uint32_t e = 0; e < num_experts; ++e) {
+        const float v = lg[e];
+        if (v > mx || mx != mx) mx = v;  // f32::max semantics: a NaN operand is ignored
+    }
+    int32_t sel_id[kMaxTopK];
+    float sel_p[kMaxTopK];
+    for (uint32_t r = 0; r < top_k; ++r) {
+        sel_id[r] = -1;
+        sel_p[r] = -INFINITY;
+    }
+    float denom = 0.0f;
+    const bool finite_max = mx == mx && fabsf(mx) != INFINITY;
+    if (finite_max)
+        for (uint32_t e = 0; e < num_experts; ++e) denom += expf(lg[e] - mx);
+    const bool live = finite_max && denom > 0.0f;
+    for (uint32_t e = 0; e < num_experts; ++e) {
+        const float p = live ? expf(lg[e] - mx) / denom : 0.0f;
+        for (uint32_t r = 0; r < top_k; ++r) {
+            if (p > sel_p[r]) {
+                for (uint32_t s = top_k - 1; s > r; --s) {
+                    sel_id[s] = sel_id[s - 1];
+                    sel_p[s] = sel_p[s - 1];
+                }
+                sel_id[r] = static_cast<int32_t>(e);
+                sel_p[r] = p;
+                break;
+            }
+        }
+    }
+    float top_sum = 0.0f;
+    for (uint32_t r = 0; r < top_k; ++r) top_sum += sel_p[r];
+    for (uint32_t r = 0; r < top_k; ++r) {
+        ids[t * top_k + r] = sel_id[r];
+        weights[t * top_k + r] = top_sum > 0.0f ? sel_p[r] / top_sum : sel_p[r];
+    }
+}
+
+// Single workgroup: counts per expert, exclusive prefix, then a stable fill of `order`
+// (pairs of one expert stay in ascending pair index, so results do not depend on
+// scheduling).
+__global__ __launch_bounds__(256) void moe_group_kernel(const int32_t* __restrict__ ids,
+                                                        uint32_t pairs, uint32_t num_experts,
+                                                        int32_t* __restrict__ counts,
+                                                        int32_t* __restrict__ offsets,
+                                                        int32_t* __restrict__ order) {
+    __shared__ int32_t s_off[kMaxExperts + 1];
+    for (uint32_t e = threadIdx.x; e < num_experts; e += 256) {
+        int32_t c = 0;
+        for (uint32_t p = 0; p < pairs; ++p) c += (ids[p] == static_cast<int32_t>(e));
+        counts[e] = c;
+        s_off[e + 1] = c;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        s_off[0] = 0;
+        for (uint32_t e = 0; e < num_experts; ++e) s_off[e + 1] += s_off[e];
+    }
+    __syncthreads();
+    for (uint32_t e = threadIdx.x; e <= num_experts; e += 256) offsets[e] = s_off[e];
+    for (uint32_t e = threadIdx.x; e < num_experts; e += 256) {
+        int32_t at = s_off[e];
+        for (uint32_t p = 0; p < pairs; ++p)
+            if (ids[p] == static_cast<int32_t>(e)) order[at++] = static_cast<int32_t>(p);
+    }
+}
+
+constexpr int kMoeWaves = 4;
+constexpr int kMoeCols = 4;  // routed tokens of one expert handled per pass over its rows
+
+__device__ __forceinline__ float silu(float v) { return v * (1.0f / (1.0f + expf(-v))); }
+
+// grid (ceil(inter / kMoeWaves), E).  Each wave owns gate row i and up row inter + i of
+// expert e and produces h[pair, i] = silu(gate . x) * (up . x) for every pair routed to e.
+__global__ __launch_bounds__(kMoeWaves * 64) void moe_gate_up_kernel(
+    const uint8_t* __restrict__ gate_up, uint32_t inter, uint32_t hidden,
+    const float* __restrict__ x, uint32_t top_k, const int32_t* __restrict__ offsets,
+    const int32_t* __restrict__ order, float* __restrict__ h) {
+    const uint32_t e = blockIdx.y;
+    const int32_t beg = offsets[e], end = offsets[e + 1];
+    if (beg == end) return;
+    const int lane = threadIdx.x & 63;
+    const uint32_t i = blockIdx.x * kMoeWaves + (threadIdx.x >> 6);
+    if (i >= inter) return;
+    const uint32_t nb = hidden / kBlockWeights;
+    const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
+    const uint8_t* base = gate_up + static_cast<size_t>(e) * 2 * inter * row_bytes;
+    const uint8_t* rowp[2] = {base + static_cast<size_t>(i) * row_bytes,
+                              base + static_cast<size_t>(inter + i) * row_bytes};
+    for (int32_t c0 = beg; c0 < end; c0 += kMoeCols) {
+        const float* xrow[kMoeCols];
+        int32_t pair[kMoeCols];
+#pragma unroll
+        for (int b = 0; b < kMoeCols; ++b) {
+            pair[b] = order[c0 + b < end ? c0 + b : beg];
+            xrow[b] = x + static_cast<size_t>(pair[b] / static_cast<int32_t>(top_k)) * hidden;
+        }
+        float acc[2][kMoeCols] = {};
+        q4_rows_dot<2, kMoeCols>(rowp, nb, xrow, lane, acc);
+#pragma unroll
+        for (int b = 0; b < kMoeCols; ++b) {
+            const float g = wave_sum(acc[0][b]);
+            const float u = wave_sum(acc[1][b]);
+            if (lane == 0 && c0 + b < end) h[static_cast<size_t>(pair[b]) * inter + i] = silu(g) * u;
+        }
+    }
+}
+
+// grid (ceil(hidden / (2*kMoeWaves)), E).  o[pair, r] = W_down[e][r, :] . h[pair, :].
+__global__ __launch_bounds__(kMoeWaves * 64) void moe_down_kernel(
+    const uint8_t* __restrict__ down, uint32_t inter, uint32_t hidden,
+    const float* __restrict__ h, const int32_t* __restrict__ offsets,
+    const int32_t* __restrict__ order, float* __restrict__ o) {
+    const uint32_t e = blockIdx.y;
+    const int32_t beg = offsets[e], end = offsets[e + 1];
+    if (beg == end) return;
+    const int lane = threadIdx.x & 63;
+    const uint32_t r0 = (blockIdx.x * kMoeWaves + (threadIdx.x >> 6)) * 2;
+    if (r0 >= hidden) return;
+    const uint32_t nb = inter / kBlockWeights;
+    const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
+    const uint8_t* base = down + static_cast<size_t>(e) * hidden * row_bytes;
+    const uint32_t r1 = r0 + 1 < hidden ? r0 + 1 : r0;
+    const uint8_t* rowp[2] = {base + static_cast<size_t>(r0) * row_bytes,
+                              base + static_cast<size_t>(r1) * row_bytes};
+    for (int32_t c0 = beg; c0 < end; c0 += kMoeCols) {
+        const float* xrow[kMoeCols];
+        int32_t pair[kMoeCols];
+#pragma unroll
+        for (int b = 0; b < kMoeCols; ++b) {
+            pair[b] = order[c0 + b < end ? c0 + b : beg];
+            xrow[b] = h + static_cast<size_t>(pair[b]) * inter;
+        }
+        float acc[2][kMoeCols] = {};
+        q4_rows_dot<2, kMoeCols>(rowp, nb, xrow, lane, acc);
+#pragma unroll
+        for (int b = 0; b < kMoeCols; ++b) {
+            const float v0 = wave_sum(acc[0][b]);
+            const float v1 = wave_sum(acc[1][b]);
+            if (lane == 0 && c0 + b < end) {
+                o[static_cast<size_t>(pair[b]) * hidden + r0] = v0;
+                if (r0 + 1 < hidden) o[static_cast<size_t>(pair[b]) * hidden + r0 + 1] = v1;
+            }
+        }
+    }
+}
+
+// y[t, c] = sum over slots, in slot order, of weights[t, s] * o[t*top_k + s, c].
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ o,
+                                                          const int32_t* __restrict__ ids,
+                                                          const float* __restrict__ weights,
+                                                          uint32_t num_experts, uint32_t top_k,
+                                                          uint32_t hidden, float* __restrict__ y) {
+    const uint32_t t = blockIdx.y;
+    const uint32_t c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= hidden) return;
+    float acc = 0.0f;
+    for (uint32_t s = 0; s < top_k; ++s) {
+        const int32_t e = ids[t * top_k + s];
+        if (e < 0 || e >= static_cast<int32_t>(num_experts)) continue;
+        acc += weights[t * top_k + s] * o[static_cast<size_t>(t * top_k + s) * hidden + c];
+    }
+    y[static_cast<size_t>(t) * hidden + c] = acc;
+}
+
+}  // namespace
+
+void launch_moe_route(const float* logits, uint32_t tokens, uint32_t num_experts, uint32_t top_k,
+                      int32_t* ids, float* weights, hipStream_t stream) {
+    hipLaunchKernelGGL(moe_route_kernel, dim3((tokens + 63) / 64), dim3(64), 0, stream, logits, tokens,
+                       num_experts, top_k, ids, weights);
+}
+
+void launch_moe_grouped(const uint8_t* gate_up, const uint8_t* down, uint32_t num_experts,
+                        uint32_t inter, uint32_t hidden, const float* x, uint32_t tokens,
+                        const int32_t* ids, const float* weights, uint32_t top_k, float* y,
+                        const MoeScratch& s, hipStream_t stream) {
+    const uint32_t pairs = tokens * top_k;
+    hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(256), 0, stream, ids, pairs, num_experts,
+                       s.counts, s.offsets, s.order);
+    hipLaunchKernelGGL(moe_gate_up_kernel, dim3((inter + kMoeWaves - 1) / kMoeWaves, num_experts),
+                       dim3(kMoeWaves * 64), 0, stream, gate_up, inter, hidden, x, top_k, s.offsets,
+                       s.order, s.h);
+    hipLaunchKernelGGL(moe_down_kernel, dim3((hidden + 2 * kMoeWaves - 1) / (2 * kMoeWaves), num_experts),
+                       dim3(kMoeWaves * 64), 0, stream, down, inter, hidden, s.h, s.offsets, s.order,
+                       s.o);
+    hipLaunchKernelGGL(moe_combine_kernel, dim3((hidden + 255) / 256, tokens), dim3(256), 0, stream,
+                       s.o, ids, weights, num_experts, top_k, hidden, y);
+}
+
+}  // namespace lq4

@@ -61,6 +61,31 @@ def timed(torch, fn, iters):
     return start.elapsed_time(stop) / iters
 
 
+def graph_timed(torch, fn, iters, replays=3):
+    """Like timed(), but the `iters` calls are captured once into a HIP graph and the graph is
+    replayed: the launches reach the GPU back to back, with no per-call host overhead between
+    them.  Returns average milliseconds per call over the last replay."""
+    g = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(g):
+        for i in range(iters):
+            fn(i)
+    torch.cuda.synchronize()
+    g.replay()
+    best = None
+    for _ in range(replays):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        start.record()
+        g.replay()
+        stop.record()
+        torch.cuda.synchronize()
+        ms = start.elapsed_time(stop) / iters
+        best = ms if best is None or ms < best else best
+    del g
+    return best
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -70,6 +95,8 @@ def main():
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--skip-extras", action="store_true", help="headline workload only")
     ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--eager", action="store_true",
+                    help="launch every step from Python instead of replaying a captured HIP graph")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path is measured on one GPU only (one process, one device); "
@@ -120,13 +147,15 @@ def main():
     # ---- headline: rotating (HBM) ------------------------------------------------------
     for i in range(args.warmup):
         layer_step(i)
-    ms_step = timed(torch, layer_step, args.steps)
+    tm = timed if args.eager else graph_timed
+    ms_step = tm(torch, layer_step, args.steps)
+    eager_ms = timed(torch, layer_step, args.steps)
     value = step_bytes / (ms_step * 1e-3) / 1e9
     launches_per_step = len(LAYER)
     us_per_launch = ms_step * 1e3 / launches_per_step
 
     # same loop on one layer: weights stay in the Infinity Cache
-    hot_ms = timed(torch, lambda i: layer_step(0), max(50, args.steps // 4))
+    hot_ms = tm(torch, lambda i: layer_step(0), max(50, args.steps // 4))
 
     out = {
         "metric": "Q4 GEMV HBM GB/s @batch 1 (Qwen3.5-2B decode layer)",
@@ -152,11 +181,14 @@ def main():
         },
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
         "tokens_per_s_equivalent_24_layers": round(1.0 / (24 * ms_step * 1e-3), 1),
+        "launch_mode": "eager launches from Python" if args.eager else "captured HIP graph, replayed",
+        "eager_python_launch": {"ms_per_step": round(eager_ms, 5),
+                                "GB/s": round(step_bytes / (eager_ms * 1e-3) / 1e9, 1)},
         "hot_cache": {"ms_per_step": round(hot_ms, 5),
                       "GB/s": round(step_bytes / (hot_ms * 1e-3) / 1e9, 1)},
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_q4_rows<%d>" % (1 if B == 1 else 2 if B == 2 else 4 if B <= 4 else 8),
+            "kernel": "gemv_q4_b1<R>" if B == 1 else "gemv_q4_rows<%d>" % (2 if B == 2 else 4 if B <= 4 else 8),
             "achieved": round(value, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
@@ -170,22 +202,34 @@ def main():
 
     # ---- per-shape and secondary workloads ---------------------------------------------
     if not args.skip_extras:
+        # Per shape: the GEMV and, on the same buffers, the read-only probe kernel whose time is
+        # the ceiling for a launch of that size on this GPU.  "27b_*" are the BASELINE config 2
+        # matrices driven as batch-1 decode GEMVs: launches large enough to approach the HBM
+        # streaming rate.
         shapes = {}
-        for name, n, k in LAYER + [("cfg0", 4096, 1024)]:
-            pool = [be.wrap_device_blocks(device_q4_weight(torch, n, k, gen))
-                    for _ in range(max(2, int(1.2e9 // (n * (k // 32) * 20))))] if name == "cfg0" \
-                else [l[name] for l in layers]
+        extra_shapes = [("cfg0", 4096, 1024), ("27b_up", 17408, 5120), ("27b_down", 5120, 17408)]
+        for name, n, k in LAYER + extra_shapes:
+            wbytes = n * (k // 32) * 20
+            pool = [l[name] for l in layers] if name in dict((a, 1) for a, _, _ in LAYER) else \
+                [be.wrap_device_blocks(device_q4_weight(torch, n, k, gen))
+                 for _ in range(max(2, min(400, int(1.2e9 // wbytes))))]
             x = torch.randn((B, k), device="cuda", generator=gen)
             y = torch.empty((B, n), device="cuda")
             f = lambda i, pool=pool, x=x, y=y, n=n, k=k: be.gemv_batch(x, pool[i % len(pool)], y, B, n, k)
+            pr = lambda i, pool=pool: be.probe_read(pool[i % len(pool)]._keepalive)
             for i in range(len(pool)):
                 f(i)
-            cold = timed(torch, f, 4 * len(pool))
-            hot = timed(torch, lambda i: f(0), 200)
+            reps = max(4 * len(pool), 100) if wbytes < 3e7 else 2 * len(pool)
+            cold = tm(torch, f, reps)
+            hot = tm(torch, lambda i: f(0), 100)
+            pcold = tm(torch, pr, reps)
             by = gemv_bytes(n, k, B)
             shapes[name] = {"n": n, "k": k, "bytes": by, "cold_us": round(cold * 1e3, 3),
                             "cold_GB/s": round(by / cold / 1e6, 1), "hot_us": round(hot * 1e3, 3),
-                            "hot_GB/s": round(by / hot / 1e6, 1)}
+                            "hot_GB/s": round(by / hot / 1e6, 1),
+                            "read_probe_cold_us": round(pcold * 1e3, 3),
+                            "read_probe_cold_GB/s": round(wbytes / pcold / 1e6, 1),
+                            "gemv_vs_probe": round(pcold / cold, 3)}
             del pool
         out["gemv_shapes_batch%d" % B] = shapes
 
@@ -199,7 +243,7 @@ def main():
                     be.gemv_batch(x8[k], bufs[name], y8[n], 8, n, k)
             for i in range(len(layers)):
                 step8(i)
-            ms8 = timed(torch, step8, max(72, args.steps // 2))
+            ms8 = tm(torch, step8, max(72, args.steps // 2))
             b8 = sum(gemv_bytes(n, k, 8) for _, n, k in LAYER)
             out["decode_layer_batch8"] = {"ms_per_step": round(ms8, 5), "GB/s": round(b8 / ms8 / 1e6, 1),
                                           "pct_of_hbm_peak": round(100 * b8 / ms8 / 1e6 / HBM_PEAK_GBPS, 2)}
@@ -216,7 +260,7 @@ def main():
                 f = lambda i: be.dispatch_gemm(x, 0, qw, y, 0, m, n, k)
                 for i in range(3):
                     f(i)
-                ms = timed(torch, f, 10)
+                ms = tm(torch, f, 10)
                 tf = 2.0 * m * n * k / (ms * 1e-3) / 1e12
                 gemm["M%d_N%d_K%d" % (m, n, k)] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 1),
                                                    "pct_of_f16_mfma_peak": round(100 * tf / MFMA_F16_PEAK_TFLOPS, 2)}
@@ -239,7 +283,7 @@ def main():
         f = lambda i: be.moe_experts(sets[i % len(sets)][0], sets[i % len(sets)][1], E, I, H, xm, ids, wts, ym)
         for i in range(len(sets)):
             f(i)
-        ms = timed(torch, f, 40)
+        ms = tm(torch, f, 40)
         out["moe_grouped_gemv"] = {"distinct_experts": distinct, "algorithmic_bytes": moe_bytes,
                                    "ms_per_step": round(ms, 4), "GB/s": round(moe_bytes / ms / 1e6, 1),
                                    "pct_of_hbm_peak": round(100 * moe_bytes / ms / 1e6 / HBM_PEAK_GBPS, 2)}

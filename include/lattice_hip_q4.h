@@ -159,6 +159,12 @@ int lq4_moe_grouped_gemv(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_weig
 int lq4_dequant(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n,
                 uint32_t k, float* out_dev, void* stream);
 
+/* Calibration: one launch that only streams `nbytes` (16-byte aligned buffer) through the
+ * vector memory path.  Timing it gives the read-bandwidth ceiling of this GPU at that
+ * launch size, the figure the GEMV kernels are held against; rocprofv3 counter runs use it
+ * as the copy kernel of known size.  No counterpart in the reference. */
+int lq4_probe_read(lq4_ctx* ctx, const void* p_dev, size_t nbytes, void* stream);
+
 /* Launch counters per kernel family since context creation (the role of
  * PathProofCounters, metal_qwen35.rs:2144-2190): proves which path served a call. */
 typedef struct lq4_path_counters {

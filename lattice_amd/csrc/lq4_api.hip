@@ -427,6 +427,15 @@ int lq4_dequant(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
     return LQ4_OK;
 }
 
+int lq4_probe_read(lq4_ctx* ctx, const void* p_dev, size_t nbytes, void* stream) {
+    if (!ctx || !p_dev) return fail(LQ4_E_INVALID, "null argument");
+    if (reinterpret_cast<uintptr_t>(p_dev) % 16) return fail(LQ4_E_INVALID, "buffer must be 16-byte aligned");
+    DeviceGuard g(ctx->device);
+    launch_probe_read(p_dev, nbytes, reinterpret_cast<uint32_t*>(ctx->lora_t), static_cast<hipStream_t>(stream));
+    LQ4_HIP(hipGetLastError());
+    return LQ4_OK;
+}
+
 int lq4_get_path_counters(const lq4_ctx* ctx, lq4_path_counters* out) {
     if (!ctx || !out) return fail(LQ4_E_INVALID, "null argument");
     *out = ctx->counters;

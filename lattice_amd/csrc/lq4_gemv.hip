@@ -112,6 +112,27 @@ __global__ __launch_bounds__(256) void lora_b_accum_kernel(const void* __restric
     y[static_cast<size_t>(row) * y_stride + nn] += scale * s;
 }
 
+// Calibration kernel: streams `n16` 16-byte words through the vector memory path and does
+// nothing else (the xor keeps the loads alive; the store never fires for real data).  Its
+// duration at a given size is the ceiling any read-only kernel of that size can reach.
+__global__ __launch_bounds__(256) void probe_read_kernel(const uint4* __restrict__ p, size_t n16,
+                                                         uint32_t* __restrict__ sink) {
+    const size_t per_wg = (n16 + gridDim.x - 1) / gridDim.x;
+    const size_t beg = blockIdx.x * per_wg;
+    const size_t end = beg + per_wg < n16 ? beg + per_wg : n16;
+    uint32_t acc = 0;
+    size_t i = beg + threadIdx.x;
+    for (; i + 768 < end; i += 1024) {
+        const uint4 a = p[i], b = p[i + 256], c = p[i + 512], d = p[i + 768];
+        acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
+    }
+    for (; i < end; i += 256) {
+        const uint4 a = p[i];
+        acc ^= a.x ^ a.y ^ a.z ^ a.w;
+    }
+    if (acc == 0x9E3779B9u && sink) sink[0] = acc;
+}
+
 __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict__ w,
                                                       uint64_t n_blocks, float* __restrict__ out) {
     // one thread per packed byte: two weights, w = f32(nibble)*scale + bias with a
@@ -135,6 +156,26 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
 void launch_gemv(const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint32_t x_stride,
                  uint32_t batch, float* y, uint32_t y_stride, const LoraEpilogue& lora,
                  hipStream_t stream) {
+    // batch 1: the dot2 kernel (one wave streams whole 1280-byte row slabs); batch 2..16: the
+    // matrix-core kernel, 8 activation rows per pass.  Either needs the activations to fit in
+    // LDS; the plain row kernel below covers K too large for that.
+    if (batch == 1 && gemv_b1_lds_bytes(k) <= 128 * 1024) {
+        launch_gemv_b1(w, n, k, x, y, lora, stream);
+        return;
+    }
+    bool fits = true;
+    for (uint32_t b0 = 0; b0 < batch && fits; b0 += 8)
+        fits = gemv_mfma_lds_bytes(k, batch - b0 < 8 ? batch - b0 : 8) <= 150 * 1024;
+    if (fits) {
+        for (uint32_t b0 = 0; b0 < batch; b0 += 8) {
+            const uint32_t nb = batch - b0 < 8 ? batch - b0 : 8;
+            LoraEpilogue l = lora;
+            if (l.rank) l.t = lora.t + static_cast<size_t>(b0) * lora.rank;
+            launch_gemv_mfma(w, n, k, x + static_cast<size_t>(b0) * x_stride, x_stride, nb,
+                             y + static_cast<size_t>(b0) * y_stride, y_stride, l, stream);
+        }
+        return;
+    }
     const dim3 grid((n + kRowsPerBlock - 1) / kRowsPerBlock), block(kWavesPerBlock * 64);
     // batches above 8 run as two passes over the weights
     for (uint32_t b0 = 0; b0 < batch; b0 += 8) {
@@ -175,6 +216,13 @@ void launch_lora_b_accum(const void* b, int b_is_f16, uint32_t rank, uint32_t d_
                          float scale, uint32_t rows, float* y, uint32_t y_stride, hipStream_t stream) {
     hipLaunchKernelGGL(lora_b_accum_kernel, dim3((d_out + 255) / 256, rows), dim3(256), 0, stream, b,
                        b_is_f16, rank, d_out, t, scale, y, y_stride);
+}
+
+void launch_probe_read(const void* p, size_t nbytes, uint32_t* sink, hipStream_t stream) {
+    const size_t n16 = nbytes / 16;
+    uint32_t grid = static_cast<uint32_t>((n16 + 1023) / 1024);
+    grid = grid > 1024 ? 1024 : grid < 1 ? 1 : grid;
+    hipLaunchKernelGGL(probe_read_kernel, dim3(grid), dim3(256), 0, stream, static_cast<const uint4*>(p), n16, sink);
 }
 
 void launch_dequant(const uint8_t* w, uint32_t n, uint32_t k, float* out, hipStream_t stream) {

@@ -1,0 +1,313 @@
+// Batch-1 decode GEMV, the bandwidth-critical kernel:  y[n] = sum_k W[n,k] * x[k].
+//
+// Work layout.  A "slab" is 64 consecutive blocks of one weight row (2048 weights,
+// 1280 contiguous bytes).  Lane l of a wave owns block 64*s + l of every row the wave
+// processes, so one load-instruction pair per lane (dwordx4 + dword) covers a whole slab
+// with no byte fetched twice, and the 32 activations a lane needs are the same for every
+// row: they are staged once per workgroup in LDS and held in registers across rows.
+// Rows shorter than a slab (K = 1024 or 512) put 2 or 4 rows side by side in one wave.
+// Waves are persistent: each walks a strided list of row groups and keeps the next
+// group's blocks in flight while it works on the current one.
+//
+// Arithmetic.  A naive unpack (shift, mask, int->float, fma per nibble) would make VALU
+// issue, not HBM, the limit on this chip.  Instead a masked dword IS a pair of f16
+// subnormals:  q & 0x000F000F = (n_lo, n_hi) * 2^-24 and q & 0x00F000F0 = (n_lo, n_hi) * 2^-20
+// (gfx950's v_dot2_f32_f16 honours f16 subnormals), so one v_and per two weights unpacks
+// them exactly, and v_dot2_f32_f16 does two MACs per op with f32 accumulation.  The
+// activations paired with the 2^-20 form are pre-scaled by 2^-4.  To keep f32 accuracy the
+// f32 activation is split x = hi + lo/2048 with hi, lo both f16: every product is exact and
+// the result tracks an f32 GEMV, not an f16 one.  Per block
+//   y += (d * 2^24) * sum_k (n_k 2^-24) x_k  +  b * sum_k x_k,
+// the bias-factored form of the reference kernel (shaders/qwen35.metal:838-847).
+// Activations must be finite and below 65504 in magnitude (the f16 range), the same
+// limit the reference's half-staged tiled kernel has.
+#include "lq4_internal.hpp"
+
+namespace lq4 {
+
+namespace {
+
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+
+constexpr int kWaves = 4;
+constexpr int kXPitch = 36;  // dwords of LDS per block of x: 16 hi pairs, 16 lo pairs, sum, 3 pad
+                             // (36 keeps 16-byte lane reads at stride 144 B conflict-free)
+constexpr float kLoScale = 2048.0f;
+constexpr float kTwo24 = 16777216.0f;
+
+struct __attribute__((packed, aligned(4))) Q4BlockRaw {
+    uint32_t sb;    // f16 scale | f16 bias << 16
+    uint32_t q[4];  // 32 nibbles, nibble i of dword j = weight 8j + i
+};
+
+__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, a), __builtin_bit_cast(half2v, b), c, false);
+}
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_add(float v) {
+    const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, false);
+    return v + __builtin_bit_cast(float, moved);
+}
+
+// Sums groups of SEG adjacent lanes (SEG = 16, 32 or 64); the total of a group is valid
+// in its last lane.
+template <int SEG>
+__device__ __forceinline__ float segment_sum(float v) {
+    v = dpp_add<0xB1, 0xF>(v);   // quad_perm [1,0,3,2]
+    v = dpp_add<0x4E, 0xF>(v);   // quad_perm [2,3,0,1]
+    v = dpp_add<0x141, 0xF>(v);  // row_half_mirror
+    v = dpp_add<0x140, 0xF>(v);  // row_mirror: every lane holds its 16-lane row sum
+    if (SEG >= 32) v = dpp_add<0x142, 0xA>(v);  // row_bcast:15 into rows 1 and 3
+    if (SEG >= 64) v = dpp_add<0x143, 0xC>(v);  // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
+__device__ __forceinline__ uint32_t pack_h2(_Float16 a, _Float16 b) {
+    const half2v h = {a, b};
+    return __builtin_bit_cast(uint32_t, h);
+}
+
+// Converts 8 consecutive activations (the partners of one packed dword) into the pair order
+// the unpack produces — (0,4) (1,5) (2,6) (3,7) — as f16 hi parts and scaled f16 residuals.
+// Odd elements pair with the 2^-20 nibble form and are split after scaling by 2^-4.
+__device__ __forceinline__ void convert_x8(const float4 a, const float4 b, uint4& ph, uint4& pl, float& sum_x) {
+    const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    _Float16 hi[8], lo[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float s = (i & 1) ? v[i] * 0.0625f : v[i];
+        hi[i] = static_cast<_Float16>(s);
+        lo[i] = static_cast<_Float16>((s - static_cast<float>(hi[i])) * kLoScale);
+    }
+    ph.x = pack_h2(hi[0], hi[4]); ph.y = pack_h2(hi[1], hi[5]);
+    ph.z = pack_h2(hi[2], hi[6]); ph.w = pack_h2(hi[3], hi[7]);
+    pl.x = pack_h2(lo[0], lo[4]); pl.y = pack_h2(lo[1], lo[5]);
+    pl.z = pack_h2(lo[2], lo[6]); pl.w = pack_h2(lo[3], lo[7]);
+    sum_x = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+}
+
+// 2^-24 * sum_k n_k * x_k over one block.
+__device__ __forceinline__ float block_dot(const uint32_t (&q)[4], const uint32_t (&xh)[16],
+                                           const uint32_t (&xl)[16]) {
+    float ph = 0.0f, pl = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t w0 = q[j] & 0x000F000Fu;
+        const uint32_t w1 = q[j] & 0x00F000F0u;
+        const uint32_t q8 = q[j] >> 8;
+        const uint32_t w2 = q8 & 0x000F000Fu;
+        const uint32_t w3 = q8 & 0x00F000F0u;
+        ph = dot2(w0, xh[4 * j + 0], ph);
+        pl = dot2(w0, xl[4 * j + 0], pl);
+        ph = dot2(w1, xh[4 * j + 1], ph);
+        pl = dot2(w1, xl[4 * j + 1], pl);
+        ph = dot2(w2, xh[4 * j + 2], ph);
+        pl = dot2(w2, xl[4 * j + 2], pl);
+        ph = dot2(w3, xh[4 * j + 3], ph);
+        pl = dot2(w3, xl[4 * j + 3], pl);
+    }
+    return fmaf(pl, 1.0f / kLoScale, ph);
+}
+
+// A wave-row is 64/SEG weight rows side by side (SEG lanes each).  Wave `wid` of `n_waves`
+// works through chunks of RW wave-rows — chunk c holds wave-rows (c*RW + j)*n_waves + wid,
+// j < RW — and, inside a chunk, through groups of SG slabs.  One (chunk, slab group) is a
+// unit: RW*SG blocks per lane, loaded with one burst; the next unit's burst is in flight
+// while the current one is consumed.  Dynamic LDS: (K/32) * kXPitch dwords.
+template <int RW, int SG, int SEG>
+__global__ __launch_bounds__(kWaves * 64) void gemv_q4_b1(const uint8_t* __restrict__ w, uint32_t n,
+                                                          uint32_t k, const float* __restrict__ x,
+                                                          float* __restrict__ y, LoraEpilogue lora) {
+    extern __shared__ __attribute__((aligned(16))) uint32_t xs[];
+    constexpr int RPW = 64 / SEG;  // weight rows per wave-row
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int sub = lane / SEG;   // which of the side-by-side rows
+    const int seg_lane = lane % SEG;
+    const uint32_t nb = k / kBlockWeights;
+    const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
+    const uint32_t slabs = SEG == 64 ? (nb + 63) / 64 : 1;
+    const uint32_t slab_groups = (slabs + SG - 1) / SG;
+    const uint32_t n_wrows = (n + RPW - 1) / RPW;
+    const uint32_t n_waves = gridDim.x * kWaves;
+    // the wave index is uniform across the wave: keep it (and everything derived) scalar
+    const uint32_t wid = __builtin_amdgcn_readfirstlane(blockIdx.x * kWaves + (tid >> 6));
+    const uint32_t chunks = (n_wrows + n_waves * RW - 1) / (n_waves * RW);
+    const uint32_t units = chunks * slab_groups;
+
+    // ---- first chunk of x is requested before any weight so it can be waited on alone ----
+    // (straight-line code, clamped addresses: no branch between the loads and their wait)
+    const uint32_t g0 = static_cast<uint32_t>(tid) < nb * 4 ? tid : 0;
+    const float4* x0p = reinterpret_cast<const float4*>(x + (g0 >> 2) * kBlockWeights + (g0 & 3) * 8);
+    const float4 x0a = x0p[0];
+    const float4 x0b = x0p[1];
+
+    // Loads unit u's blocks.  Lanes past the end of a row and rows past N re-read a valid
+    // block; their contribution is zeroed or dropped later.
+    auto load_unit = [&](Q4BlockRaw (&buf)[RW][SG], uint32_t u) {
+        const uint32_t chunk = u / slab_groups, sgi = u - chunk * slab_groups;
+#pragma unroll
+        for (int j = 0; j < RW; ++j) {
+            uint32_t wrow = (chunk * RW + j) * n_waves + wid;  // scalar
+            if (wrow >= n_wrows) wrow = n_wrows - 1;
+            uint32_t row = wrow * RPW + sub;
+            if (RPW > 1 && row >= n) row = n - 1;
+            const uint8_t* rp = w + row * row_bytes;  // scalar base when RPW == 1
+#pragma unroll
+            for (int t = 0; t < SG; ++t) {
+                uint32_t blk = (sgi * SG + t) * 64 + seg_lane;
+                if (blk >= nb) blk = nb - 1;
+                buf[j][t] = *reinterpret_cast<const Q4BlockRaw*>(rp + blk * static_cast<uint32_t>(kBlockBytes));
+            }
+        }
+    };
+
+    Q4BlockRaw buf_a[RW][SG], buf_b[RW][SG];
+    load_unit(buf_a, 0);
+    __builtin_amdgcn_sched_barrier(0);  // nothing below is scheduled above these loads
+
+    // ---- stage x: thread handles (block, dword j) = 8 activations ---------------------------
+    auto stage = [&](uint32_t g, const float4 a, const float4 b, bool store) {
+        const uint32_t blk = g >> 2, j = g & 3;
+        float sx;
+        uint4 ph, pl;
+        convert_x8(a, b, ph, pl, sx);
+        // the 4 threads of a block are 4 adjacent lanes: quad butterfly
+        sx = dpp_add<0xB1, 0xF>(sx);
+        sx = dpp_add<0x4E, 0xF>(sx);
+        if (store) {
+            *reinterpret_cast<uint4*>(&xs[blk * kXPitch + 4 * j]) = ph;
+            *reinterpret_cast<uint4*>(&xs[blk * kXPitch + 16 + 4 * j]) = pl;
+            if (j == 0) *reinterpret_cast<float*>(&xs[blk * kXPitch + 32]) = sx;
+        }
+    };
+    stage(g0, x0a, x0b, static_cast<uint32_t>(tid) < nb * 4);
+    for (uint32_t g = tid + kWaves * 64; g < nb * 4; g += kWaves * 64) {
+        const float4* xp = reinterpret_cast<const float4*>(x + (g >> 2) * kBlockWeights + (g & 3) * 8);
+        stage(g, xp[0], xp[1], true);
+    }
+    __syncthreads();
+
+    float acc[RW];
+#pragma unroll
+    for (int j = 0; j < RW; ++j) acc[j] = 0.0f;
+
+    // Consumes unit u from `cur` while unit u+1 streams into `nxt`.
+    auto process = [&](Q4BlockRaw (&cur)[RW][SG], Q4BlockRaw (&nxt)[RW][SG], uint32_t u) {
+        const uint32_t chunk = u / slab_groups, sgi = u - chunk * slab_groups;
+        if (u + 1 < units) load_unit(nxt, u + 1);
+
+#pragma unroll
+        for (int t = 0; t < SG; ++t) {
+            const uint32_t slab = sgi * SG + t;
+            if (slab < slabs) {  // uniform across the wave
+                const uint32_t blk_raw = slab * 64 + seg_lane;
+                const bool live = blk_raw < nb;
+                const uint32_t blk = live ? blk_raw : nb - 1;
+                uint32_t xh[16], xl[16];
+                const uint4* xsrc = reinterpret_cast<const uint4*>(&xs[blk * kXPitch]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint4 h = xsrc[i], l = xsrc[4 + i];
+                    xh[4 * i + 0] = h.x; xh[4 * i + 1] = h.y; xh[4 * i + 2] = h.z; xh[4 * i + 3] = h.w;
+                    xl[4 * i + 0] = l.x; xl[4 * i + 1] = l.y; xl[4 * i + 2] = l.z; xl[4 * i + 3] = l.w;
+                }
+                const float sum_x = live ? *reinterpret_cast<const float*>(&xs[blk * kXPitch + 32]) : 0.0f;
+#pragma unroll
+                for (int j = 0; j < RW; ++j) {
+                    const float p = block_dot(cur[j][t].q, xh, xl);
+                    float d = f16_bits_to_f32(cur[j][t].sb & 0xffffu) * kTwo24;
+                    const float b = f16_bits_to_f32(cur[j][t].sb >> 16);
+                    if (!live) d = 0.0f;
+                    acc[j] = fmaf(d, p, fmaf(b, sum_x, acc[j]));
+                }
+            }
+        }
+
+        if (sgi + 1 == slab_groups) {  // chunk complete: reduce and store its rows
+#pragma unroll
+            for (int j = 0; j < RW; ++j) {
+                const uint32_t wrow = (chunk * RW + j) * n_waves + wid;
+                const uint32_t row = wrow * RPW + sub;
+                const bool row_ok = wrow < n_wrows && row < n;
+                float v = acc[j];
+                acc[j] = 0.0f;
+                if (lora.rank && row_ok) {
+                    // the row's lanes share out scale * B[row, i] * t[i]; the sum below folds it in
+                    for (uint32_t i = seg_lane; i < lora.rank; i += SEG) {
+                        const size_t bi = static_cast<size_t>(row) * lora.rank + i;
+                        const float bv = lora.b_is_f16 ? static_cast<float>(static_cast<const _Float16*>(lora.b)[bi])
+                                                       : static_cast<const float*>(lora.b)[bi];
+                        v = fmaf(lora.scale * bv, lora.t[i], v);
+                    }
+                }
+                v = segment_sum<SEG>(v);
+                if (seg_lane == SEG - 1 && row_ok) y[row] = v;
+            }
+        }
+    };
+
+    // two buffers swap roles every unit, so no block is ever copied between registers
+    for (uint32_t u = 0; u < units; u += 2) {
+        process(buf_a, buf_b, u);
+        if (u + 1 < units) process(buf_b, buf_a, u + 1);
+    }
+}
+
+template <int RW, int SG, int SEG>
+void launch_cfg(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, const LoraEpilogue& lora,
+                size_t lds, uint32_t waves, hipStream_t stream) {
+    static bool attr_set = false;  // raise the dynamic-LDS cap once per instantiation
+    if (!attr_set) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((gemv_q4_b1<RW, SG, SEG>), dim3((waves + kWaves - 1) / kWaves), dim3(kWaves * 64), lds,
+                       stream, w, n, k, x, y, lora);
+}
+
+}  // namespace
+
+size_t gemv_b1_lds_bytes(uint32_t k) { return static_cast<size_t>(k / kBlockWeights) * kXPitch * 4; }
+
+void launch_gemv_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y,
+                    const LoraEpilogue& lora, hipStream_t stream) {
+    const size_t lds = gemv_b1_lds_bytes(k);
+    const uint32_t nb = k / kBlockWeights;
+    const uint32_t seg = nb == 32 ? 32 : nb == 16 ? 16 : 64;
+    const uint32_t n_wrows = (n + 64 / seg - 1) / (64 / seg);
+    const uint32_t slabs = seg == 64 ? (nb + 63) / 64 : 1;
+    // Up to 16 waves per CU (4096 in all), fewer when the staged x leaves room for fewer
+    // workgroups; rows per wave chosen so every wave gets the same share (to within one).
+    uint32_t wg_per_cu = static_cast<uint32_t>((160 * 1024) / (lds + 512));
+    wg_per_cu = wg_per_cu > 4 ? 4 : wg_per_cu < 1 ? 1 : wg_per_cu;
+    const uint32_t max_waves = 256 * wg_per_cu * kWaves;
+    uint32_t rw = (n_wrows + max_waves - 1) / max_waves;
+    rw = rw > 4 ? 4 : rw;
+    // whole chunks per wave; a grid up to 1.5x the resident capacity beats a second chunk
+    uint32_t chunks = (2 * n_wrows + 3 * max_waves * rw - 1) / (3 * max_waves * rw);
+    chunks = chunks < 1 ? 1 : chunks;
+    const uint32_t waves = (n_wrows + rw * chunks - 1) / (rw * chunks);
+    uint32_t sg = slabs < 3 ? slabs : 3;
+    while (rw * sg > 6) --sg;
+
+#define LQ4_B1(RW_, SG_, SEG_) launch_cfg<RW_, SG_, SEG_>(w, n, k, x, y, lora, lds, waves, stream)
+    if (seg == 32) {
+        if (rw == 1) LQ4_B1(1, 1, 32); else if (rw == 2) LQ4_B1(2, 1, 32); else if (rw == 3) LQ4_B1(3, 1, 32); else LQ4_B1(4, 1, 32);
+    } else if (seg == 16) {
+        if (rw == 1) LQ4_B1(1, 1, 16); else if (rw == 2) LQ4_B1(2, 1, 16); else if (rw == 3) LQ4_B1(3, 1, 16); else LQ4_B1(4, 1, 16);
+    } else if (rw == 1) {
+        if (sg == 1) LQ4_B1(1, 1, 64); else if (sg == 2) LQ4_B1(1, 2, 64); else LQ4_B1(1, 3, 64);
+    } else if (rw == 2) {
+        if (sg == 1) LQ4_B1(2, 1, 64); else if (sg == 2) LQ4_B1(2, 2, 64); else LQ4_B1(2, 3, 64);
+    } else if (rw == 3) {
+        if (sg == 1) LQ4_B1(3, 1, 64); else LQ4_B1(3, 2, 64);
+    } else {
+        LQ4_B1(4, 1, 64);
+    }
+#undef LQ4_B1
+}
+
+}  // namespace lq4

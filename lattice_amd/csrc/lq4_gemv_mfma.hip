@@ -1,0 +1,400 @@
+// Decode GEMV for 1..8 activation rows over native Q4 blocks, on the matrix cores:
+//   y[b, n] = sum_k W[n, k] * x[b, k],  b < batch.
+//
+// The kernel is HBM-bound by design; everything below exists to keep the cores' side of
+// the work (unpack, multiply, scale) well under the time the bytes take to arrive.
+//
+// Instruction.  v_mfma_f32_4x4x4_16B_f16 multiplies 16 independent 4x4x4 problems, one per
+// group of four lanes.  Lane 4g+j supplies B[:, j] (4 values) and A[j, :] (4 values) of
+// group g and receives D[0..3, j] = sum_k A[i, k] * B[k, j].  Here B[:, j] are 4 weights of
+// the lane's own block and A[i, :] is the matching slice of activation column i, so a lane
+// gets the dot products of ITS weights with up to four activation columns; the other three
+// lanes of the group hold the same block position of three other weight rows.  Eight such
+// instructions cover a 32-weight block.
+//
+// Mapping.  Lane 4g+j of a wave owns block 16*s + g (s = step along K) of weight rows
+// 4t + j, t < T: one contiguous 20-byte block per row per step (dwordx4 + dword), 16
+// consecutive blocks (320 contiguous bytes) per row per wave-step, nothing fetched twice.
+// The waves of a workgroup split K (KS slices) and row groups (4/KS); partial sums meet in
+// LDS.  Activations are staged once per workgroup in LDS as f16, already in the order the
+// unpack yields.
+//
+// Unpack.  A masked dword IS a pair of f16 subnormals: q & 0x000F000F = (n0, n4) * 2^-24 and
+// q & 0x00F000F0 = (n1, n5) * 2^-20 (the matrix cores honour f16 subnormals), so five VALU ops
+// turn 8 nibbles into 8 exact f16 operands; activations paired with the 2^-20 form are
+// pre-scaled by 2^-4, and the block scale absorbs 2^24.  Per block, in f32:
+//   y += (d * 2^24) * P + b * sum_k x_k      (P from the matrix core; the bias-factored form
+//   of the reference kernel, shaders/qwen35.metal:838-847).
+//
+// Precision.  For batch <= 2 every f32 activation is split x = hi + lo/2048 (two f16 columns),
+// products are exact and the result tracks an f32 GEMV (~1e-6), as the reference's m == 1 kernel
+// does.  For batch >= 3 activations are rounded to f16 once, as the reference's m > 1 tiled
+// kernel does (shaders/gemm_q4_tiled.metal:45-48).  Activations must be finite and within the
+// f16 range (|x| < 65504).
+#include "lq4_internal.hpp"
+
+namespace lq4 {
+
+namespace {
+
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 256;
+constexpr float kLoScale = 2048.0f;
+constexpr float kTwo24 = 16777216.0f;
+
+struct __attribute__((packed, aligned(4))) Q4BlockRaw {
+    uint32_t sb;    // f16 scale | f16 bias << 16
+    uint32_t q[4];  // 32 nibbles, nibble i of dword j = weight 8j + i
+};
+
+__device__ __forceinline__ uint32_t pack_h2(_Float16 a, _Float16 b) {
+    const half2v h = {a, b};
+    return __builtin_bit_cast(uint32_t, h);
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+    const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false);
+    return v + __builtin_bit_cast(float, moved);
+}
+
+// LDS bytes per block of K: `ncols` columns of 32 f16 (64 B each) followed by the per-row
+// sums of x (one f32 per activation row, padded to 16 B).
+__host__ __device__ constexpr uint32_t x_pitch_bytes(int ncols, int batch) {
+    return static_cast<uint32_t>(ncols) * 64u + 16u * static_cast<uint32_t>((batch + 3) / 4);
+}
+
+// 8 consecutive activations -> the operand order of one packed dword:
+// [x0, x4, x1/16, x5/16 | x2, x6, x3/16, x7/16]  (first / second 4x4x4 step of the dword).
+template <bool HILO>
+__device__ __forceinline__ void convert_x8(const float4 a, const float4 b, uint4& hi, uint4& lo, float& sum_x) {
+    const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    _Float16 h[8], l[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float s = (i & 1) ? v[i] * 0.0625f : v[i];
+        h[i] = static_cast<_Float16>(s);
+        l[i] = HILO ? static_cast<_Float16>((s - static_cast<float>(h[i])) * kLoScale) : static_cast<_Float16>(0.0f);
+    }
+    hi.x = pack_h2(h[0], h[4]); hi.y = pack_h2(h[1], h[5]); hi.z = pack_h2(h[2], h[6]); hi.w = pack_h2(h[3], h[7]);
+    lo.x = pack_h2(l[0], l[4]); lo.y = pack_h2(l[1], l[5]); lo.z = pack_h2(l[2], l[6]); lo.w = pack_h2(l[3], l[7]);
+    sum_x = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+}
+
+struct GemvArgs {
+    const uint8_t* w;
+    const float* x;
+    float* y;
+    uint32_t n, k, batch, x_stride, y_stride;
+    LoraEpilogue lora;
+};
+
+// NSETS: groups of four activation columns (1 or 2).  HILO: two columns per activation row.
+// T: weight-row tiles (of 4 rows) per wave.  KS: slices of K per workgroup (1, 2 or 4).
+// Workgroups are persistent: workgroup g handles row groups g, g + gridDim.x, ... (a row group
+// is 4*T*(4/KS) rows) with the activations staged once.  For one wave the work is a list of
+// units (row group, step); unit u+1 is in flight while unit u is consumed.
+template <int NSETS, bool HILO, int T, int KS>
+__global__ __launch_bounds__(kThreads) void gemv_q4_mfma(GemvArgs p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    constexpr int RS = 4 / KS;  // row sub-groups per workgroup
+    constexpr int NCOLS = 4 * NSETS;
+    constexpr uint32_t kRowsPerIter = 4 * T * RS;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = lane >> 2;   // block within the step
+    const int j = lane & 3;    // weight row within the tile / activation column within a set
+    const uint32_t nb = p.k / kBlockWeights;
+    const uint32_t nsteps = (nb + 15) / 16;
+    const uint32_t batch = p.batch;
+    const int ncols = HILO ? 2 * static_cast<int>(batch) : static_cast<int>(batch);
+    const uint32_t pitch = x_pitch_bytes(ncols, batch);
+    // LDS is addressed in 16-byte units so every vector access is provably aligned
+    uint4* const xs16 = reinterpret_cast<uint4*>(smem);
+    const uint32_t pitch16 = pitch / 16;
+    uint4* const zero_region = xs16 + nb * pitch16;               // 64 B of zeros
+    float* red = reinterpret_cast<float*>(zero_region + 4);       // [2][4 waves][T][NCOLS][4]
+    constexpr int kRedFloats = 4 * T * NCOLS * 4;
+
+    const int ks = wave % KS, rs = wave / KS;
+    const uint32_t n_groups = (p.n + kRowsPerIter - 1) / kRowsPerIter;
+    const uint32_t iters = (n_groups - blockIdx.x + gridDim.x - 1) / gridDim.x;  // >= 1
+    const uint32_t n_local = static_cast<uint32_t>(ks) < nsteps ? (nsteps - ks + KS - 1) / KS : 0;
+    const uint32_t units = iters * n_local;
+    auto first_row = [&](uint32_t it) { return ((blockIdx.x + it * gridDim.x) * RS + rs) * (4 * T); };
+
+    // ---- the first activations are requested before any weight, so they can be waited on alone
+    const uint32_t items = nb * 4;  // (block, dword) pairs
+    const uint32_t it0 = static_cast<uint32_t>(tid) < items ? tid : 0;
+    const float4* x0p = reinterpret_cast<const float4*>(p.x + (it0 >> 2) * kBlockWeights + (it0 & 3) * 8);
+    const float4 x0a = x0p[0], x0b = x0p[1];
+
+    // Loads unit u.  Blocks past the end of a row and rows past N re-read a valid block; their
+    // contribution is zeroed or dropped later.
+    auto load_unit = [&](Q4BlockRaw (&buf)[T], uint32_t u) {
+        const uint32_t it = n_local ? u / n_local : 0, q = u - it * n_local;
+        uint32_t blk = (ks + q * KS) * 16 + g;
+        if (blk >= nb) blk = nb - 1;
+        const uint32_t row0 = first_row(it);
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            uint32_t row = row0 + 4 * t + j;
+            if (row >= p.n) row = p.n - 1;
+            buf[t] = *reinterpret_cast<const Q4BlockRaw*>(reinterpret_cast<const uint32_t*>(p.w) +
+                                                          static_cast<size_t>(row) * (nb * 5) + blk * 5);
+        }
+    };
+
+    // ring of four unit buffers: three units are in flight while one is consumed
+    Q4BlockRaw buf_a[T], buf_b[T], buf_c[T], buf_d[T];
+    load_unit(buf_a, 0);
+    load_unit(buf_b, units > 1 ? 1 : 0);
+    load_unit(buf_c, units > 2 ? 2 : 0);
+    __builtin_amdgcn_sched_barrier(0);  // nothing below is scheduled above these loads
+
+    // ---- stage activations: one (block, dword) item = 8 values per activation row ------------
+    auto stage = [&](uint32_t it, uint32_t b, const float4 va, const float4 vb, bool store) {
+        const uint32_t blk = it >> 2, dw = it & 3;
+        uint4 hi, lo;
+        float sx;
+        convert_x8<HILO>(va, vb, hi, lo, sx);
+        sx = dpp_add<0xB1>(sx);  // the 4 items of a block sit in 4 adjacent lanes
+        sx = dpp_add<0x4E>(sx);
+        if (store) {
+            uint4* base = xs16 + blk * pitch16;
+            if (HILO) {
+                base[(2 * b) * 4 + dw] = hi;
+                base[(2 * b + 1) * 4 + dw] = lo;
+            } else {
+                base[b * 4 + dw] = hi;
+            }
+            if (dw == 0) reinterpret_cast<float*>(base + ncols * 4)[b] = sx;
+        }
+    };
+    stage(it0, 0, x0a, x0b, static_cast<uint32_t>(tid) < items);
+    for (uint32_t b = 0; b < batch; ++b) {
+        for (uint32_t it = (b == 0 ? tid + kThreads : tid); it < items; it += kThreads) {
+            const float4* xp = reinterpret_cast<const float4*>(p.x + static_cast<size_t>(b) * p.x_stride +
+                                                               (it >> 2) * kBlockWeights + (it & 3) * 8);
+            stage(it, b, xp[0], xp[1], true);
+        }
+    }
+    if (tid < 4) zero_region[tid] = make_uint4(0u, 0u, 0u, 0u);
+    __syncthreads();
+
+    float acc[T][NCOLS];
+#pragma unroll
+    for (int t = 0; t < T; ++t)
+#pragma unroll
+        for (int c = 0; c < NCOLS; ++c) acc[t][c] = 0.0f;
+
+    // Consumes unit u from `cur` while unit u+1 streams into `nxt`.
+    auto process = [&](Q4BlockRaw (&cur)[T], Q4BlockRaw (&nxt)[T], uint32_t u) {
+        if (u + 3 < units) load_unit(nxt, u + 3);
+        const uint32_t it = u / n_local, q = u - it * n_local;
+        const uint32_t blk_raw = (ks + q * KS) * 16 + g;
+        const bool live = blk_raw < nb;
+        const uint32_t blk = live ? blk_raw : nb - 1;
+        const uint4* xb = xs16 + blk * pitch16;
+
+        // activation operands of this lane: column 4*set + j of block `blk` (zeros past ncols)
+        uint32_t a_op[NSETS][16];
+#pragma unroll
+        for (int set = 0; set < NSETS; ++set) {
+            const int col = 4 * set + j;
+            const uint4* src = col < ncols ? xb + col * 4 : zero_region;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint4 v = src[i];
+                a_op[set][4 * i + 0] = v.x; a_op[set][4 * i + 1] = v.y;
+                a_op[set][4 * i + 2] = v.z; a_op[set][4 * i + 3] = v.w;
+            }
+        }
+        // sum of x over the block, for the column that carries the bias term of its activation row
+        float sum_x[NCOLS];
+#pragma unroll
+        for (int c = 0; c < NCOLS; ++c) {
+            const int brow = HILO ? c / 2 : c;
+            const bool has = (HILO ? (c % 2 == 0) : true) && brow < static_cast<int>(batch) && live;
+            sum_x[c] = has ? reinterpret_cast<const float*>(xb + ncols * 4)[brow] : 0.0f;
+        }
+
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            float4v prod[NSETS];
+#pragma unroll
+            for (int set = 0; set < NSETS; ++set) prod[set] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int dw = 0; dw < 4; ++dw) {
+                const uint32_t qd = cur[t].q[dw];
+                const uint32_t q8 = qd >> 8;
+                const uint32_t w0 = qd & 0x000F000Fu, w1 = qd & 0x00F000F0u;
+                const uint32_t w2 = q8 & 0x000F000Fu, w3 = q8 & 0x00F000F0u;
+                const half4 b01 = __builtin_bit_cast(half4, uint2{w0, w1});
+                const half4 b23 = __builtin_bit_cast(half4, uint2{w2, w3});
+#pragma unroll
+                for (int set = 0; set < NSETS; ++set) {
+                    const half4 a01 = __builtin_bit_cast(half4, uint2{a_op[set][4 * dw + 0], a_op[set][4 * dw + 1]});
+                    const half4 a23 = __builtin_bit_cast(half4, uint2{a_op[set][4 * dw + 2], a_op[set][4 * dw + 3]});
+                    prod[set] = __builtin_amdgcn_mfma_f32_4x4x4f16(a01, b01, prod[set], 0, 0, 0);
+                    prod[set] = __builtin_amdgcn_mfma_f32_4x4x4f16(a23, b23, prod[set], 0, 0, 0);
+                }
+            }
+            float d = f16_bits_to_f32(cur[t].sb & 0xffffu) * kTwo24;
+            const float bias = f16_bits_to_f32(cur[t].sb >> 16);
+            if (!live) d = 0.0f;
+#pragma unroll
+            for (int c = 0; c < NCOLS; ++c)
+                acc[t][c] = fmaf(d, prod[c / 4][c % 4], fmaf(bias, sum_x[c], acc[t][c]));
+        }
+    };
+
+    // Row group finished for this wave: sum over the 16 blocks of a step (lanes with equal j),
+    // meet the other K slices in LDS, and let the slice-0 wave store.
+    auto finish = [&](uint32_t it) {
+#pragma unroll
+        for (int t = 0; t < T; ++t)
+#pragma unroll
+            for (int c = 0; c < NCOLS; ++c) {
+                float v = acc[t][c];
+                acc[t][c] = 0.0f;
+                v = dpp_add<0x124>(v);  // row_ror:4
+                v = dpp_add<0x128>(v);  // row_ror:8 -> sum over the row's lanes with this j
+                v += __shfl_xor(v, 16, 64);
+                v += __shfl_xor(v, 32, 64);
+                if (KS > 1 && lane < 4) red[(it & 1) * kRedFloats + ((wave * T + t) * NCOLS + c) * 4 + lane] = v;
+                if (KS == 1) acc[t][c] = v;  // reused below as the total
+            }
+        if (KS > 1) __syncthreads();
+        if (ks == 0 && lane < 4) {
+            const uint32_t row0 = first_row(it);
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                const uint32_t row = row0 + 4 * t + lane;
+                float tot[NCOLS];
+#pragma unroll
+                for (int c = 0; c < NCOLS; ++c) {
+                    float v = KS == 1 ? acc[t][c] : 0.0f;
+                    if (KS > 1)
+                        for (int o = 0; o < KS; ++o)
+                            v += red[(it & 1) * kRedFloats + (((wave + o) * T + t) * NCOLS + c) * 4 + lane];
+                    tot[c] = v;
+                }
+                if (row < p.n) {
+#pragma unroll
+                    for (int c = 0; c < NCOLS; ++c) {
+                        const int brow = HILO ? c / 2 : c;
+                        if ((HILO && (c & 1)) || brow >= static_cast<int>(batch)) continue;
+                        float v = HILO ? fmaf(tot[c + (HILO ? 1 : 0)], 1.0f / kLoScale, tot[c]) : tot[c];
+                        if (p.lora.rank) {
+                            float sacc = 0.0f;
+                            for (uint32_t r = 0; r < p.lora.rank; ++r) {
+                                const size_t bi = static_cast<size_t>(row) * p.lora.rank + r;
+                                const float bv = p.lora.b_is_f16
+                                                     ? static_cast<float>(static_cast<const _Float16*>(p.lora.b)[bi])
+                                                     : static_cast<const float*>(p.lora.b)[bi];
+                                sacc = fmaf(bv, p.lora.t[brow * p.lora.rank + r], sacc);
+                            }
+                            v = fmaf(p.lora.scale, sacc, v);
+                        }
+                        p.y[static_cast<size_t>(brow) * p.y_stride + row] = v;
+                    }
+                }
+            }
+        }
+        if (KS == 1) {
+#pragma unroll
+            for (int t = 0; t < T; ++t)
+#pragma unroll
+                for (int c = 0; c < NCOLS; ++c) acc[t][c] = 0.0f;
+        }
+    };
+
+    if (n_local == 0) {  // more K slices than steps: this wave only takes part in the barriers
+        for (uint32_t it = 0; it < iters; ++it) finish(it);
+        return;
+    }
+    // the buffers rotate roles every unit, so no block is ever copied between registers
+    uint32_t q = 0, it = 0;
+    for (uint32_t u = 0; u < units; u += 4) {
+        process(buf_a, buf_d, u);
+        if (++q == n_local) { finish(it++); q = 0; }
+        if (u + 1 >= units) break;
+        process(buf_b, buf_a, u + 1);
+        if (++q == n_local) { finish(it++); q = 0; }
+        if (u + 2 >= units) break;
+        process(buf_c, buf_b, u + 2);
+        if (++q == n_local) { finish(it++); q = 0; }
+        if (u + 3 >= units) break;
+        process(buf_d, buf_c, u + 3);
+        if (++q == n_local) { finish(it++); q = 0; }
+    }
+}
+
+template <int NSETS, bool HILO, int T, int KS>
+void launch_cfg(const GemvArgs& a, size_t lds, uint32_t max_wgs, hipStream_t stream) {
+    static bool attr_set = false;  // raise the dynamic-LDS cap once per instantiation
+    if (!attr_set) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_mfma<NSETS, HILO, T, KS>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        attr_set = true;
+    }
+    constexpr uint32_t rows_per_iter = 4 * T * (4 / KS);
+    const uint32_t groups = (a.n + rows_per_iter - 1) / rows_per_iter;
+    // every workgroup gets the same number of row groups, to within one
+    const uint32_t iters = (groups + max_wgs - 1) / max_wgs;
+    const uint32_t wgs = (groups + iters - 1) / iters;
+    hipLaunchKernelGGL((gemv_q4_mfma<NSETS, HILO, T, KS>), dim3(wgs), dim3(kThreads), lds, stream, a);
+}
+
+template <int NSETS, bool HILO>
+void launch_shape(const GemvArgs& a, size_t lds, uint32_t t, uint32_t ks, uint32_t max_wgs, hipStream_t stream) {
+#define LQ4_CASE(T_, KS_) if (t == T_ && ks == KS_) return launch_cfg<NSETS, HILO, T_, KS_>(a, lds, max_wgs, stream)
+    LQ4_CASE(1, 4); LQ4_CASE(1, 2); LQ4_CASE(1, 1);
+    LQ4_CASE(2, 4); LQ4_CASE(2, 2); LQ4_CASE(2, 1);
+    LQ4_CASE(4, 4); LQ4_CASE(4, 2); LQ4_CASE(4, 1);
+#undef LQ4_CASE
+}
+
+}  // namespace
+
+size_t gemv_mfma_lds_bytes(uint32_t k, uint32_t batch) {
+    const bool hilo = batch <= 2;
+    const int ncols = hilo ? 2 * batch : batch;
+    return static_cast<size_t>(k / kBlockWeights) * x_pitch_bytes(ncols, batch) + 64 +
+           2 * 4 * 4 * 8 * 4 * sizeof(float);
+}
+
+void launch_gemv_mfma(const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint32_t x_stride,
+                      uint32_t batch, float* y, uint32_t y_stride, const LoraEpilogue& lora,
+                      hipStream_t stream) {
+    GemvArgs a{w, x, y, n, k, batch, x_stride, y_stride, lora};
+    const size_t lds = gemv_mfma_lds_bytes(k, batch);
+    const uint32_t nsteps = (k / kBlockWeights + 15) / 16;
+    // resident workgroups per CU: up to 8 (32 waves, what the T = 1 kernels' 64 registers allow)
+    // unless the staged activations leave room for fewer
+    uint32_t wg_per_cu = static_cast<uint32_t>((160 * 1024) / (lds + 1024));
+    wg_per_cu = wg_per_cu > 8 ? 8 : wg_per_cu < 1 ? 1 : wg_per_cu;
+    const uint32_t max_wgs = 256 * wg_per_cu;
+    // K slices per workgroup: none when the rows alone give about 3 workgroups per CU (no LDS
+    // meeting point, no barrier per row group); otherwise split K as far as its steps allow
+    uint32_t ks = 1;
+    while (ks < 4 && ks * 2 <= nsteps && (n + 16 / ks - 1) / (16 / ks) < 768) ks *= 2;
+    // row tiles per wave: enough blocks in flight per CU to cover HBM latency (about 40 KB), but
+    // never so many that fewer than two workgroups per CU remain
+    uint32_t t = wg_per_cu >= 4 ? 1 : wg_per_cu >= 2 ? 2 : 4;
+    while (t > 1 && (n + 4 * t * (4 / ks) - 1) / (4 * t * (4 / ks)) < 512) t >>= 1;
+    if (batch <= 2) {
+        launch_shape<1, true>(a, lds, t, ks, max_wgs, stream);
+    } else if (batch <= 4) {
+        launch_shape<1, false>(a, lds, t, ks, max_wgs, stream);
+    } else {
+        launch_shape<2, false>(a, lds, t, ks, max_wgs, stream);
+    }
+}
+
+}  // namespace lq4

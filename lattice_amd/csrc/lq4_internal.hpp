@@ -30,6 +30,17 @@ void launch_gemv(const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint3
                  uint32_t batch, float* y, uint32_t y_stride, const LoraEpilogue& lora,
                  hipStream_t stream);
 
+// Batch-1 fast path (x staged in LDS as f16 hi/lo pairs); needs gemv_b1_lds_bytes(k) of LDS.
+size_t gemv_b1_lds_bytes(uint32_t k);
+void launch_gemv_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y,
+                    const LoraEpilogue& lora, hipStream_t stream);
+
+// Matrix-core GEMV for batch 1..8 (activations staged in LDS as f16 columns).
+size_t gemv_mfma_lds_bytes(uint32_t k, uint32_t batch);
+void launch_gemv_mfma(const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint32_t x_stride,
+                      uint32_t batch, float* y, uint32_t y_stride, const LoraEpilogue& lora,
+                      hipStream_t stream);
+
 // t[row, j] = sum_k A[j, k] * x[row, k]; x f32 or f16 with row stride x_stride elements.
 void launch_lora_a(const void* a, int a_is_f16, uint32_t rank, uint32_t d_in, const void* x,
                    int x_is_f16, uint32_t x_stride, uint32_t rows, float* t, hipStream_t stream);
@@ -42,6 +53,7 @@ void launch_lora_b_accum(const void* b, int b_is_f16, uint32_t rank, uint32_t d_
 void launch_gemm(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
                  float* y, const LoraEpilogue& lora, hipStream_t stream);
 
+void launch_probe_read(const void* p, size_t nbytes, uint32_t* sink, hipStream_t stream);
 void launch_dequant(const uint8_t* w, uint32_t n, uint32_t k, float* out, hipStream_t stream);
 
 void launch_moe_route(const float* logits, uint32_t tokens, uint32_t num_experts, uint32_t top_k,

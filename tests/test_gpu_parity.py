@@ -239,7 +239,8 @@ def test_lora_fused_matches_oracle(be, name, batch):
         # no projection registered for this (layer, module): plain base output
         y0 = torch.empty_like(y)
         be.dispatch_gemm(dev(x), 0, qw, y0, 0, batch, n, k, layer_idx=4, module=f"{name}_proj")
-        assert rel_err(host(y0), base) <= (1e-5 if batch <= backend.MAX_GEMV_BATCH else REL_TOL)
+        # batch <= 2 keeps f32 activations (hi/lo split); above that they are rounded to f16
+        assert rel_err(host(y0), base) <= (1e-5 if batch <= 2 else REL_TOL)
         # the delta itself is resolved, not lost in the base: the difference between the fused
         # and the plain launch (same base arithmetic on the GPU) against the oracle's delta
         e_delta = rel_err(host(y) - host(y0), ref - base)

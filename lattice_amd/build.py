@@ -6,6 +6,7 @@
 from __future__ import annotations
 
 import os
+import shlex
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -32,11 +33,12 @@ def _run(cmd):
 
 def build(verbose: bool = False) -> str:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    extra = shlex.split(os.environ.get("LQ4_CXXFLAGS", ""))  # e.g. -DNAME for experiments
     objs = [os.path.join(CSRC, s.replace(".hip", ".o")) for s in SOURCES]
 
     def compile_one(pair):
         src, obj = pair
-        cmd = [hipcc, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [hipcc, *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         _run(cmd)

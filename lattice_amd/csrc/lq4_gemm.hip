@@ -1,8 +1,27 @@
-// Prefill GEMM over native Q4 blocks: Y[M,N] = X[M,K] . W[N,K]^T, f16 operands into
-// MFMA, f32 accumulate.  Each k-step consumes exactly one Q4 block per weight row;
-// the block is dequantised to f16 in registers ("half(f32(q)*d + b)", the rounding
-// point of the reference's tiled kernel, shaders/gemm_q4_tiled.metal:57-66) and
-// staged in LDS next to the f16 activation tile.
+// Prefill GEMM over native Q4 blocks: Y[M,N] = X[M,K] . W[N,K]^T, f16 operands into the
+// matrix cores, f32 accumulate.
+//
+// Tile: 128 tokens x BN weight rows (128 or 256) x 64 K per step; one wave per 64x64 of
+// outputs (2x2 tiles of v_mfma_f32_32x32x16_f16), so 4 or 8 waves per workgroup.  A K step
+// consumes two Q4 blocks per weight row: 2*BN blocks per tile, one per thread.  Each thread
+// dequantises its block in registers to f16 — "half(f32(q)*d + b)", the rounding point of the
+// reference's tiled kernel (shaders/gemm_q4_tiled.metal:57-66) — and stores it beside the f16
+// activation tile in LDS.  LDS is double buffered, so a step costs one barrier; activation
+// loads run one step ahead of the matrix cores (they mostly hit L2), weight loads three steps
+// ahead (they stream from HBM).
+//
+// What bounds this kernel is the traffic from L2 into LDS, not the matrix cores: an
+// activation element costs 2 bytes per tile that reads it and a weight 0.625, so the wide tile
+// (BN = 256: every activation tile is re-read N/256 times) is preferred whenever it still
+// leaves at least one tile per CU.
+//
+// Dequantisation is done two weights per instruction: a masked dword OR-ed into the mantissa
+// of 1024.0 (or 64.0) is the f16 pair (1024+n_lo, 1024+n_hi); one packed subtract makes it
+// (n_lo, n_hi) exactly and one packed fma applies scale and bias with a single rounding.
+//
+// Tiles are numbered so that the workgroups resident at one time, and in particular those
+// that share an XCD (consecutive workgroup ids go round-robin over the 8 XCDs), work on a
+// small set of token tiles: their activations stay in that XCD's L2 while weights stream.
 #include "lq4_internal.hpp"
 
 namespace lq4 {
@@ -11,35 +30,86 @@ namespace {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 128;  // activation rows (tokens) per workgroup
-constexpr int BN = 128;  // weight rows (output features) per workgroup
-constexpr int BK = 32;   // one Q4 block along K
-constexpr int LDS_STRIDE = BK + 8;  // halfs; 80-byte rows keep ds_read_b128 conflict-free
+constexpr int BM = 128;         // tokens per workgroup
+constexpr int BK = 64;          // two Q4 blocks along K
+constexpr int kPitch = BK + 8;  // halfs per LDS row: 144 bytes keeps 16-byte reads conflict-free
+constexpr int kGroupM = 16;     // token tiles per rasterisation group
+
+struct __attribute__((packed, aligned(4))) Q4BlockRaw {
+    uint32_t sb;    // f16 scale | f16 bias << 16
+    uint32_t q[4];  // 32 nibbles, nibble i of dword j = weight 8j + i
+};
 
 __device__ __forceinline__ float load_b(const void* b, int is_f16, size_t idx) {
     return is_f16 ? static_cast<float>(static_cast<const _Float16*>(b)[idx])
                   : static_cast<const float*>(b)[idx];
 }
 
-template <bool X_F16>
-__global__ __launch_bounds__(256) void gemm_q4_mfma(const uint8_t* __restrict__ w, uint32_t n,
-                                                    uint32_t k, const void* __restrict__ xv,
-                                                    uint32_t m, float* __restrict__ y,
-                                                    LoraEpilogue lora) {
-    __shared__ __attribute__((aligned(16))) _Float16 Xs[BM * LDS_STRIDE];
-    __shared__ __attribute__((aligned(16))) _Float16 Ws[BN * LDS_STRIDE];
+__device__ __forceinline__ uint32_t and_or(uint32_t v, uint32_t mask, uint32_t bits) {
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "s"(mask), "v"(bits));
+    return r;
+}
+
+__device__ __forceinline__ half2v as_h2(uint32_t v) { return __builtin_bit_cast(half2v, v); }
+__device__ __forceinline__ uint32_t as_u32(half2v v) { return __builtin_bit_cast(uint32_t, v); }
+
+// One packed dword (weights 8j..8j+7) -> 8 f16 weights in memory order.
+__device__ __forceinline__ uint4 dequant8(uint32_t q, half2v d2, half2v b2) {
+    const half2v k1024 = {static_cast<_Float16>(1024.0f), static_cast<_Float16>(1024.0f)};
+    const half2v k64 = {static_cast<_Float16>(64.0f), static_cast<_Float16>(64.0f)};
+    const uint32_t q8 = q >> 8;
+    // pairs (n0,n4) (n1,n5) (n2,n6) (n3,n7)
+    const half2v p04 = as_h2(and_or(q, 0x000F000Fu, 0x64006400u)) - k1024;
+    const half2v p15 = as_h2(and_or(q, 0x00F000F0u, 0x54005400u)) - k64;
+    const half2v p26 = as_h2(and_or(q8, 0x000F000Fu, 0x64006400u)) - k1024;
+    const half2v p37 = as_h2(and_or(q8, 0x00F000F0u, 0x54005400u)) - k64;
+    const half2v w04 = __builtin_elementwise_fma(p04, d2, b2);
+    const half2v w15 = __builtin_elementwise_fma(p15, d2, b2);
+    const half2v w26 = __builtin_elementwise_fma(p26, d2, b2);
+    const half2v w37 = __builtin_elementwise_fma(p37, d2, b2);
+    // back to memory order: (w0,w1) (w2,w3) (w4,w5) (w6,w7)
+    uint4 r;
+    r.x = __builtin_amdgcn_perm(as_u32(w15), as_u32(w04), 0x05040100u);
+    r.y = __builtin_amdgcn_perm(as_u32(w37), as_u32(w26), 0x05040100u);
+    r.z = __builtin_amdgcn_perm(as_u32(w15), as_u32(w04), 0x07060302u);
+    r.w = __builtin_amdgcn_perm(as_u32(w37), as_u32(w26), 0x07060302u);
+    return r;
+}
+
+// BN_: weight rows per workgroup (128 or 256); 2*BN_ threads; waves in a 2 x (BN_/64) grid.
+template <bool X_F16, int BN_>
+__global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
+    const uint8_t* __restrict__ w, uint32_t n, uint32_t k, const void* __restrict__ xv, uint32_t m,
+    float* __restrict__ y, LoraEpilogue lora) {
+    extern __shared__ __attribute__((aligned(16))) _Float16 lds[];  // 2 x (X tile | W tile)
+    constexpr int kThreads = 2 * BN_;
+    constexpr int kWavesN = BN_ / 64;
+    constexpr int kTileHalfs = (BM + BN_) * kPitch;
+    constexpr int kChunksPerRow = X_F16 ? 8 : 16;       // 16-byte chunks per 64-wide row
+    constexpr int XCH = BM * kChunksPerRow / kThreads;  // activation chunks per thread per step
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int wm = (wave >> 1) * 64;  // wave's 64x64 sub-tile inside the 128x128 tile
-    const int wn = (wave & 1) * 64;
-    const uint32_t m0 = blockIdx.y * BM;
-    const uint32_t n0 = blockIdx.x * BN;
+    const int wm = (wave / kWavesN) * 64;  // wave's 64x64 sub-tile inside the workgroup tile
+    const int wn = (wave % kWavesN) * 64;
+
+    // ---- tile id -> (token tile, weight tile), grouped so co-resident tiles share activations
+    const uint32_t tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN_ - 1) / BN_;
+    const uint32_t per_group = kGroupM * tiles_n;
+    const uint32_t group = blockIdx.x / per_group;
+    const uint32_t first_m = group * kGroupM;
+    const uint32_t group_m = tiles_m - first_m < kGroupM ? tiles_m - first_m : kGroupM;
+    const uint32_t in_group = blockIdx.x - group * per_group;
+    const uint32_t m0 = (first_m + in_group % group_m) * BM;
+    const uint32_t n0 = (in_group / group_m) * BN_;
+
     const uint32_t nb = k / kBlockWeights;
-    const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
+    const uint32_t nsteps = (nb + 1) / 2;
 
     float16v acc[2][2];
 #pragma unroll
@@ -49,97 +119,141 @@ __global__ __launch_bounds__(256) void gemm_q4_mfma(const uint8_t* __restrict__ 
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    // ---- global -> register staging -------------------------------------------------
-    // activations: f16 -> 2 x 16-byte chunks per thread; f32 -> 4 x 16-byte chunks
-    constexpr int XCH = X_F16 ? 2 : 4;
-    uint4 xreg[XCH];
-    uint32_t wreg[5];
-    const bool w_loader = tid < BN;
-    const uint32_t w_row = n0 + tid;
-    const uint8_t* w_ptr = w + static_cast<size_t>(w_row < n ? w_row : 0) * row_bytes;
+    // ---- per-thread staging assignments, fixed for the whole K loop ---------------------------
+    // weights: thread -> (row tid/2, block tid%2 of the step)
+    const uint32_t w_row = n0 + (tid >> 1);
+    const bool w_live_row = w_row < n;
+    const uint32_t* w_ptr =
+        reinterpret_cast<const uint32_t*>(w) + static_cast<size_t>(w_live_row ? w_row : 0) * (nb * 5);
+    const int w_half = tid & 1;
+    // activations: chunk i of this thread is (row, part) = divmod(tid + kThreads*i, chunks per row)
+    const uint8_t* x_ptr[XCH];
+    bool x_live[XCH];
+#pragma unroll
+    for (int i = 0; i < XCH; ++i) {
+        const int c = tid + kThreads * i;
+        const int row = c / kChunksPerRow, part = c % kChunksPerRow;
+        const uint32_t gm = m0 + row;
+        x_live[i] = gm < m;
+        x_ptr[i] = static_cast<const uint8_t*>(xv) +
+                   (static_cast<size_t>(x_live[i] ? gm : 0) * k) * (X_F16 ? 2 : 4) + part * 16;
+    }
 
-    auto load_tiles = [&](uint32_t kb) {
-#pragma unroll
-        for (int i = 0; i < XCH; ++i) {
-            const int c = tid + 256 * i;
-            if (X_F16) {
-                const int row = c >> 2, part = c & 3;
-                const uint32_t gm = m0 + row;
-                xreg[i] = gm < m ? *reinterpret_cast<const uint4*>(static_cast<const _Float16*>(xv) +
-                                                                   static_cast<size_t>(gm) * k + kb * BK + part * 8)
-                                 : make_uint4(0, 0, 0, 0);
-            } else {
-                const int row = c >> 3, part = c & 7;
-                const uint32_t gm = m0 + row;
-                xreg[i] = gm < m ? *reinterpret_cast<const uint4*>(static_cast<const float*>(xv) +
-                                                                   static_cast<size_t>(gm) * k + kb * BK + part * 4)
-                                 : make_uint4(0, 0, 0, 0);
-            }
-        }
-        if (w_loader) {
-            const uint32_t* p = reinterpret_cast<const uint32_t*>(w_ptr + static_cast<size_t>(kb) * kBlockBytes);
-#pragma unroll
-            for (int i = 0; i < 5; ++i) wreg[i] = p[i];
-        }
+    struct XStage {
+        uint4 x[XCH];
     };
 
-    auto store_tiles = [&]() {
+    // Steps past the end of K (the unrolled loop below may run up to three) load nothing.
+    auto load_x = [&](XStage& st, uint32_t s) {
+        const bool first_ok = 2 * s < nb;       // the step exists at all
+        const bool second_ok = 2 * s + 1 < nb;  // the step's second block exists
+        const size_t step_bytes = static_cast<size_t>(s) * BK * (X_F16 ? 2 : 4);
 #pragma unroll
         for (int i = 0; i < XCH; ++i) {
-            const int c = tid + 256 * i;
+            const int part = (tid + kThreads * i) % kChunksPerRow;
+            const bool in_k = part < kChunksPerRow / 2 ? first_ok : second_ok;
+            st.x[i] = (x_live[i] && in_k) ? *reinterpret_cast<const uint4*>(x_ptr[i] + step_bytes)
+                                          : make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto load_w = [&](Q4BlockRaw& wst, uint32_t s) {
+        uint32_t blk = s * 2 + w_half;
+        if (blk >= nb) blk = nb - 1;
+        wst = *reinterpret_cast<const Q4BlockRaw*>(w_ptr + blk * 5);
+    };
+
+    auto store_tiles = [&](const XStage& st, const Q4BlockRaw& wst, uint32_t s, _Float16* xs, _Float16* ws) {
+#pragma unroll
+        for (int i = 0; i < XCH; ++i) {
+            const int c = tid + kThreads * i;
+            const int row = c / kChunksPerRow, part = c % kChunksPerRow;
             if (X_F16) {
-                const int row = c >> 2, part = c & 3;
-                *reinterpret_cast<uint4*>(&Xs[row * LDS_STRIDE + part * 8]) = xreg[i];
+                *reinterpret_cast<uint4*>(&xs[row * kPitch + part * 8]) = st.x[i];
             } else {
-                const int row = c >> 3, part = c & 7;
                 half4 h;
-                h[0] = static_cast<_Float16>(__builtin_bit_cast(float, xreg[i].x));
-                h[1] = static_cast<_Float16>(__builtin_bit_cast(float, xreg[i].y));
-                h[2] = static_cast<_Float16>(__builtin_bit_cast(float, xreg[i].z));
-                h[3] = static_cast<_Float16>(__builtin_bit_cast(float, xreg[i].w));
-                *reinterpret_cast<half4*>(&Xs[row * LDS_STRIDE + part * 4]) = h;
+                h[0] = static_cast<_Float16>(__builtin_bit_cast(float, st.x[i].x));
+                h[1] = static_cast<_Float16>(__builtin_bit_cast(float, st.x[i].y));
+                h[2] = static_cast<_Float16>(__builtin_bit_cast(float, st.x[i].z));
+                h[3] = static_cast<_Float16>(__builtin_bit_cast(float, st.x[i].w));
+                *reinterpret_cast<half4*>(&xs[row * kPitch + part * 4]) = h;
             }
         }
-        if (w_loader) {
-            const bool live = w_row < n;
-            const float d = live ? f16_bits_to_f32(wreg[0] & 0xffffu) : 0.0f;
-            const float b = live ? f16_bits_to_f32(wreg[0] >> 16) : 0.0f;
+        const bool live = w_live_row && (s * 2 + w_half) < nb;
+        const uint32_t sb = live ? wst.sb : 0u;
+        const half2v d2 = as_h2(__builtin_amdgcn_perm(sb, sb, 0x01000100u));  // (d, d)
+        const half2v b2 = as_h2(__builtin_amdgcn_perm(sb, sb, 0x03020302u));  // (b, b)
+        _Float16* dst = &ws[(tid >> 1) * kPitch + w_half * 32];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint32_t q = wreg[1 + j];
-                half8 h;
-#pragma unroll
-                for (int i = 0; i < 8; ++i)
-                    h[i] = static_cast<_Float16>(fmaf(static_cast<float>((q >> (4 * i)) & 0xfu), d, b));
-                *reinterpret_cast<half8*>(&Ws[tid * LDS_STRIDE + j * 8]) = h;
-            }
-        }
+        for (int j = 0; j < 4; ++j)
+            *reinterpret_cast<uint4*>(dst + j * 8) = dequant8(live ? wst.q[j] : 0u, d2, b2);
     };
 
-    load_tiles(0);
-    for (uint32_t kb = 0; kb < nb; ++kb) {
-        store_tiles();
-        __syncthreads();
-        if (kb + 1 < nb) load_tiles(kb + 1);
-        // operand layout of v_mfma_f32_32x32x16_f16: lane l supplies row/col (l & 31),
-        // k-slice 8*(l >> 5) .. +7 of a 16-deep step
-        const int r = lane & 31, ks = (lane >> 5) * 8;
+    // Matrix-core work of one K step.  Operand layout of v_mfma_f32_32x32x16_f16: lane l supplies
+    // row/col (l & 31), k-slice 8*(l >> 5) .. +7 of a 16-deep sub-step.  The operands of sub-step
+    // kk+1 are read from LDS while the instructions of sub-step kk execute.
+    auto compute = [&](const _Float16* xs, const _Float16* ws) {
+        const int r = lane & 31, ksl = (lane >> 5) * 8;
+        const _Float16* xa = &xs[(wm + r) * kPitch + ksl];
+        const _Float16* wb = &ws[(wn + r) * kPitch + ksl];
+        half8 a[2][2], b[2][2];
 #pragma unroll
-        for (int kk = 0; kk < BK; kk += 16) {
-            half8 a[2], b[2];
+        for (int i = 0; i < 2; ++i) a[0][i] = *reinterpret_cast<const half8*>(xa + i * 32 * kPitch);
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
-                a[i] = *reinterpret_cast<const half8*>(&Xs[(wm + i * 32 + r) * LDS_STRIDE + kk + ks]);
+        for (int j = 0; j < 2; ++j) b[0][j] = *reinterpret_cast<const half8*>(wb + j * 32 * kPitch);
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-                b[j] = *reinterpret_cast<const half8*>(&Ws[(wn + j * 32 + r) * LDS_STRIDE + kk + ks]);
+        for (int kk = 0; kk < BK / 16; ++kk) {
+            const int cur = kk & 1, nxt = cur ^ 1;
+            if (kk + 1 < BK / 16) {
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+                    a[nxt][i] = *reinterpret_cast<const half8*>(xa + i * 32 * kPitch + (kk + 1) * 16);
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    b[nxt][j] = *reinterpret_cast<const half8*>(wb + j * 32 * kPitch + (kk + 1) * 16);
+            }
 #pragma unroll
             for (int i = 0; i < 2; ++i)
 #pragma unroll
                 for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[cur][i], b[cur][j], acc[i][j], 0, 0, 0);
         }
+    };
+
+    _Float16* xs0 = lds;
+    _Float16* ws0 = xs0 + BM * kPitch;
+    _Float16* xs1 = lds + kTileHalfs;
+    _Float16* ws1 = xs1 + BM * kPitch;
+
+    // The K loop is unrolled by four so that register sets and LDS buffers have fixed roles at every
+    // position (nothing is copied): step s uses activation set s%2, weight set s%4, LDS buffer s%2.
+    // Steps past the end of K (at most three) run on zeros, which keeps the body branch-free.
+    XStage xa, xb;
+    Q4BlockRaw w0, w1, w2, w3;
+    load_x(xa, 0);
+    load_w(w0, 0);
+    load_w(w1, 1);
+    load_w(w2, 2);
+    for (uint32_t s = 0; s < nsteps; s += 4) {
+        store_tiles(xa, w0, s, xs0, ws0);
         __syncthreads();
+        load_x(xb, s + 1);
+        load_w(w3, s + 3);
+        compute(xs0, ws0);
+        store_tiles(xb, w1, s + 1, xs1, ws1);
+        __syncthreads();
+        load_x(xa, s + 2);
+        load_w(w0, s + 4);
+        compute(xs1, ws1);
+        store_tiles(xa, w2, s + 2, xs0, ws0);
+        __syncthreads();
+        load_x(xb, s + 3);
+        load_w(w1, s + 5);
+        compute(xs0, ws0);
+        store_tiles(xb, w3, s + 3, xs1, ws1);
+        __syncthreads();
+        load_x(xa, s + 4);
+        load_w(w2, s + 6);
+        compute(xs1, ws1);
     }
 
     // ---- epilogue: accumulator element v of lane l is
@@ -155,11 +269,11 @@ __global__ __launch_bounds__(256) void gemm_q4_mfma(const uint8_t* __restrict__ 
                 if (gm < m && gn < n) {
                     float val = acc[i][j][v];
                     if (lora.rank) {
-                        float s = 0.0f;
+                        float sacc = 0.0f;
                         for (uint32_t jj = 0; jj < lora.rank; ++jj)
-                            s += load_b(lora.b, lora.b_is_f16, static_cast<size_t>(gn) * lora.rank + jj) *
-                                 lora.t[static_cast<size_t>(gm) * lora.rank + jj];
-                        val += lora.scale * s;
+                            sacc += load_b(lora.b, lora.b_is_f16, static_cast<size_t>(gn) * lora.rank + jj) *
+                                    lora.t[static_cast<size_t>(gm) * lora.rank + jj];
+                        val += lora.scale * sacc;
                     }
                     y[static_cast<size_t>(gm) * n + gn] = val;
                 }
@@ -167,15 +281,39 @@ __global__ __launch_bounds__(256) void gemm_q4_mfma(const uint8_t* __restrict__ 
         }
 }
 
+template <bool X_F16, int BN_>
+void launch_tile(const uint8_t* w, uint32_t n, uint32_t k, const void* x, uint32_t m, float* y,
+                 const LoraEpilogue& lora, hipStream_t stream) {
+    const uint32_t tiles = ((n + BN_ - 1) / BN_) * ((m + BM - 1) / BM);
+    const size_t lds = 2 * (BM + BN_) * kPitch * sizeof(_Float16);
+    static bool attr_set = false;
+    if (!attr_set) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4_mfma<X_F16, BN_>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((gemm_q4_mfma<X_F16, BN_>), dim3(tiles), dim3(2 * BN_), lds, stream, w, n, k, x, m, y,
+                       lora);
+}
+
+#ifndef LQ4_GEMM_WIDE_MIN_TILES
+#define LQ4_GEMM_WIDE_MIN_TILES 256
+#endif
+
 }  // namespace
 
 void launch_gemm(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
                  float* y, const LoraEpilogue& lora, hipStream_t stream) {
-    const dim3 grid((n + BN - 1) / BN, (m + BM - 1) / BM), block(256);
-    if (x_is_f16)
-        hipLaunchKernelGGL(gemm_q4_mfma<true>, grid, block, 0, stream, w, n, k, x, m, y, lora);
-    else
-        hipLaunchKernelGGL(gemm_q4_mfma<false>, grid, block, 0, stream, w, n, k, x, m, y, lora);
+    // the wide tile runs one workgroup (8 waves) per CU; use it when that still fills the chip
+    const uint32_t wide_tiles = ((n + 255) / 256) * ((m + BM - 1) / BM);
+    const bool wide = wide_tiles >= LQ4_GEMM_WIDE_MIN_TILES;
+    if (x_is_f16) {
+        if (wide) launch_tile<true, 256>(w, n, k, x, m, y, lora, stream);
+        else launch_tile<true, 128>(w, n, k, x, m, y, lora, stream);
+    } else {
+        if (wide) launch_tile<false, 256>(w, n, k, x, m, y, lora, stream);
+        else launch_tile<false, 128>(w, n, k, x, m, y, lora, stream);
+    }
 }
 
 }  // namespace lq4

@@ -10,10 +10,9 @@
 // loads run one step ahead of the matrix cores (they mostly hit L2), weight loads three steps
 // ahead (they stream from HBM).
 //
-// What bounds this kernel is the traffic from L2 into LDS, not the matrix cores: an
-// activation element costs 2 bytes per tile that reads it and a weight 0.625, so the wide tile
-// (BN = 256: every activation tile is re-read N/256 times) is preferred whenever it still
-// leaves at least one tile per CU.
+// With 64 x 64 wave tiles the LDS operand reads alone need the full LDS bandwidth at matrix-core
+// peak, so this kernel tops out near a third of peak; it is the kernel for shapes with too few
+// tiles to fill the chip with the larger weights-in-registers kernel (lq4_gemm_wreg.hip).
 //
 // Dequantisation is done two weights per instruction: a masked dword OR-ed into the mantissa
 // of 1024.0 (or 64.0) is the f16 pair (1024+n_lo, 1024+n_hi); one packed subtract makes it
@@ -22,6 +21,8 @@
 // Tiles are numbered so that the workgroups resident at one time, and in particular those
 // that share an XCD (consecutive workgroup ids go round-robin over the 8 XCDs), work on a
 // small set of token tiles: their activations stay in that XCD's L2 while weights stream.
+#include <stdlib.h>
+
 #include "lq4_internal.hpp"
 
 namespace lq4 {
@@ -296,24 +297,25 @@ void launch_tile(const uint8_t* w, uint32_t n, uint32_t k, const void* x, uint32
                        lora);
 }
 
-#ifndef LQ4_GEMM_WIDE_MIN_TILES
-#define LQ4_GEMM_WIDE_MIN_TILES 256
-#endif
+// Shapes with at least this many 128 x 256 tiles (two per CU) go to the weights-in-registers
+// kernel; below that its single workgroup per CU leaves the chip under-filled and the 128 x 128
+// tile of this file, two workgroups per CU, is faster.
+constexpr uint32_t kWregMinTiles = 512;
 
 }  // namespace
 
 void launch_gemm(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
                  float* y, const LoraEpilogue& lora, hipStream_t stream) {
-    // the wide tile runs one workgroup (8 waves) per CU; use it when that still fills the chip
-    const uint32_t wide_tiles = ((n + 255) / 256) * ((m + BM - 1) / BM);
-    const bool wide = wide_tiles >= LQ4_GEMM_WIDE_MIN_TILES;
-    if (x_is_f16) {
-        if (wide) launch_tile<true, 256>(w, n, k, x, m, y, lora, stream);
-        else launch_tile<true, 128>(w, n, k, x, m, y, lora, stream);
-    } else {
-        if (wide) launch_tile<false, 256>(w, n, k, x, m, y, lora, stream);
-        else launch_tile<false, 128>(w, n, k, x, m, y, lora, stream);
-    }
+    // LQ4_GEMM_KERNEL=1 forces the LDS-staged kernels of this file, 2 the weights-in-registers
+    // kernel; anything else picks by shape.
+    static const int forced = [] {
+        const char* e = getenv("LQ4_GEMM_KERNEL");
+        return e ? atoi(e) : 0;
+    }();
+    if (forced == 2 || (forced != 1 && gemm_wreg_tiles(n, m) >= kWregMinTiles))
+        return launch_gemm_wreg(w, n, k, x, x_is_f16, m, y, lora, stream);
+    if (x_is_f16) launch_tile<true, 128>(w, n, k, x, m, y, lora, stream);
+    else launch_tile<false, 128>(w, n, k, x, m, y, lora, stream);
 }
 
 }  // namespace lq4

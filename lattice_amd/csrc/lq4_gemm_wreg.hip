@@ -1,0 +1,350 @@
+// Prefill GEMM, weights-in-registers variant: Y[M,N] = X[M,K] . W[N,K]^T for large shapes.
+//
+// A workgroup of four waves owns 128 tokens x 256 weight rows; wave w owns weight rows
+// 64w .. 64w+63 against all 128 tokens.  Only the activations go through LDS (f16, double
+// buffered, one barrier per 128-wide K step).  Weights never touch LDS: every lane loads whole
+// Q4 blocks straight from global memory, dequantises them in registers and feeds them to
+// v_mfma_f32_16x16x32_f16 as the A operand.  Compared with staging dequantised weights in LDS
+// this removes 2 bytes of LDS write and 2 x 2 bytes of LDS read per weight, and each weight is
+// dequantised exactly once per 128 tokens.
+//
+// The K dimension inside one matrix-core instruction is a sum, so its order is free as long as
+// both operands agree.  A K step covers four Q4 blocks; lane (r = lane % 16, g = lane / 16)
+// owns block g of weight row r.  Instruction j (0..3) of the step takes dword j of the lane's
+// own block: across the four lane groups it covers weights 8j..8j+7 of four different blocks.
+// So a lane only ever touches its own block and its own scale and bias.  The activation
+// operand is read from LDS at the matching K offset 32g + 8j.  Within a dword the nibble
+// pairs come out of the dequantiser as (w0,w4)(w1,w5)(w2,w6)(w3,w7); instead of shuffling
+// every weight back into order, the activations are stored to LDS in that same order once.
+//
+// Dequantised value: half(q*d + b) with one rounding, the rounding point of the reference's
+// tiled kernel (shaders/gemm_q4_tiled.metal:57-66); products accumulate in f32.
+//
+// Weight loads run two K steps ahead of their use (three rotating register sets), activation
+// loads one step ahead; the K loop is unrolled by three so that every register set has a fixed
+// role at every position.  Out-of-range rows are clamped to valid rows (their results are never
+// stored); blocks past the end of K are clamped to valid blocks and given a zero scale and
+// bias, so the loop body is free of divergent branches.
+#include "lq4_internal.hpp"
+
+namespace lq4 {
+
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+constexpr int TM = 128;                    // tokens per workgroup
+constexpr int TN = 256;                    // weight rows per workgroup
+constexpr int TK = 128;                    // K per step: four Q4 blocks
+constexpr int kPitch16 = TK * 2 / 16 + 1;  // LDS row pitch in 16-byte units (272 bytes)
+constexpr int kBuf16 = TM * kPitch16;      // one activation buffer, in 16-byte units
+constexpr int kGroupM = 16;                // token tiles per rasterisation group
+constexpr int NU = 4;                      // 16-row weight tiles per wave
+constexpr int NT = TM / 16;                // 16-token tiles per workgroup
+
+struct __attribute__((packed, aligned(4))) Q4BlockRaw {
+    uint32_t sb;    // f16 scale | f16 bias << 16
+    uint32_t q[4];  // 32 nibbles, nibble i of dword j = weight 8j + i
+};
+
+__device__ __forceinline__ float load_b(const void* b, int is_f16, size_t idx) {
+    return is_f16 ? static_cast<float>(static_cast<const _Float16*>(b)[idx])
+                  : static_cast<const float*>(b)[idx];
+}
+
+__device__ __forceinline__ uint32_t and_or(uint32_t v, uint32_t mask, uint32_t bits) {
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "s"(mask), "v"(bits));
+    return r;
+}
+
+__device__ __forceinline__ half2v as_h2(uint32_t v) { return __builtin_bit_cast(half2v, v); }
+__device__ __forceinline__ uint32_t as_u32(half2v v) { return __builtin_bit_cast(uint32_t, v); }
+
+struct U4 {
+    uint32_t v[4];
+};
+
+// Dequantisation of one packed dword (weights 8j..8j+7) into f16 weights in the order
+// w0 w4 w1 w5 w2 w6 w3 w7, cut into 13 single-instruction steps so that the K loop can place
+// them one by one in the shadow of matrix-core instructions.  A masked dword OR-ed into the
+// mantissa of 1024.0 (or 64.0) is the pair (1024+n_lo, 1024+n_hi); one packed subtract makes it
+// (n_lo, n_hi) exactly, one packed fma applies scale and bias with a single rounding.
+constexpr int kDqOps = 13;
+struct DqTmp {
+    uint32_t q8;
+    half2v t[4];
+};
+__device__ __forceinline__ void dq_op(int op, uint32_t q, half2v d2, half2v b2, DqTmp& tmp, U4& out) {
+    const half2v k1024 = {static_cast<_Float16>(1024.0f), static_cast<_Float16>(1024.0f)};
+    const half2v k64 = {static_cast<_Float16>(64.0f), static_cast<_Float16>(64.0f)};
+    switch (op) {
+        case 0: tmp.q8 = q >> 8; break;
+        case 1: tmp.t[0] = as_h2(and_or(q, 0x000F000Fu, 0x64006400u)); break;
+        case 2: tmp.t[1] = as_h2(and_or(q, 0x00F000F0u, 0x54005400u)); break;
+        case 3: tmp.t[2] = as_h2(and_or(tmp.q8, 0x000F000Fu, 0x64006400u)); break;
+        case 4: tmp.t[3] = as_h2(and_or(tmp.q8, 0x00F000F0u, 0x54005400u)); break;
+        case 5: tmp.t[0] -= k1024; break;
+        case 6: tmp.t[1] -= k64; break;
+        case 7: tmp.t[2] -= k1024; break;
+        case 8: tmp.t[3] -= k64; break;
+        default: out.v[op - 9] = as_u32(__builtin_elementwise_fma(tmp.t[op - 9], d2, b2)); break;
+    }
+}
+
+// Eight consecutive f16 activations x0..x7 (as four dwords) -> x0 x4 x1 x5 x2 x6 x3 x7.
+__device__ __forceinline__ uint4 interleave8(uint4 c) {
+    uint4 r;
+    r.x = __builtin_amdgcn_perm(c.z, c.x, 0x05040100u);
+    r.y = __builtin_amdgcn_perm(c.z, c.x, 0x07060302u);
+    r.z = __builtin_amdgcn_perm(c.w, c.y, 0x05040100u);
+    r.w = __builtin_amdgcn_perm(c.w, c.y, 0x07060302u);
+    return r;
+}
+
+__device__ __forceinline__ uint32_t pack_h2(float lo, float hi) {
+    half2v h = {static_cast<_Float16>(lo), static_cast<_Float16>(hi)};
+    return as_u32(h);
+}
+
+template <bool X_F16>
+__global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict__ w, uint32_t n, uint32_t k,
+                                                       const void* __restrict__ xv, uint32_t m,
+                                                       float* __restrict__ y, LoraEpilogue lora) {
+    extern __shared__ uint4 lds16[];  // two activation buffers of kBuf16 units
+    constexpr int XU = TM * (TK / 8) / 256;  // 8-activation units staged per thread per step
+    constexpr int XL = X_F16 ? 1 : 2;        // 16-byte global loads per unit
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int lr = lane & 15;  // row inside a 16-row tile
+    const int g = lane >> 4;   // K group: block g of the step
+
+    // ---- tile id -> (token tile, weight tile), grouped so co-resident tiles share activations
+    const uint32_t tiles_m = (m + TM - 1) / TM, tiles_n = (n + TN - 1) / TN;
+    const uint32_t per_group = kGroupM * tiles_n;
+    const uint32_t group = blockIdx.x / per_group;
+    const uint32_t first_m = group * kGroupM;
+    const uint32_t group_m = tiles_m - first_m < kGroupM ? tiles_m - first_m : kGroupM;
+    const uint32_t in_group = blockIdx.x - group * per_group;
+    const uint32_t m0 = (first_m + in_group % group_m) * TM;
+    const uint32_t n0 = (in_group / group_m) * TN;
+
+    const uint32_t nb = k / kBlockWeights;
+    const uint32_t nsteps = (nb + 3) / 4;
+
+    float4v acc[NU][NT];
+#pragma unroll
+    for (int u = 0; u < NU; ++u)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[u][t] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // ---- per-thread global pointers -----------------------------------------------------------
+    const uint32_t* w_row[NU];  // first dword of the lane's weight row of tile u
+#pragma unroll
+    for (int u = 0; u < NU; ++u) {
+        uint32_t row = n0 + wave * 64 + u * 16 + lr;
+        row = row < n ? row : n - 1;
+        w_row[u] = reinterpret_cast<const uint32_t*>(w) + static_cast<size_t>(row) * (nb * 5);
+    }
+    // activation unit i of this thread: token row tid/16 + 16 i, K offset 8 * (tid % 16) of the step
+    const int x_part = tid & 15;
+    const uint8_t* x_row[XU];
+#pragma unroll
+    for (int i = 0; i < XU; ++i) {
+        uint32_t row = m0 + (tid >> 4) + 16 * i;
+        row = row < m ? row : m - 1;
+        x_row[i] = static_cast<const uint8_t*>(xv) + static_cast<size_t>(row) * k * (X_F16 ? 2 : 4);
+    }
+
+    struct XRegs {
+        uint4 c[XU][XL];
+    };
+
+    auto load_x_unit = [&](XRegs& xr, int i, uint32_t s) {
+        uint32_t koff = s * TK + x_part * 8;
+        koff = koff < k ? koff : k - 8;  // past the end of K: any valid address, weights there are zero
+        const size_t byte_off = static_cast<size_t>(koff) * (X_F16 ? 2 : 4);
+#pragma unroll
+        for (int l = 0; l < XL; ++l)
+            xr.c[i][l] = *reinterpret_cast<const uint4*>(x_row[i] + byte_off + 16 * l);
+    };
+    auto store_x_unit = [&](const XRegs& xr, int i, uint4* buf) {
+        uint4 out;
+        if (X_F16) {
+            out = interleave8(xr.c[i][0]);
+        } else {
+            const uint4 a = xr.c[i][0], b = xr.c[i][XL - 1];
+            out.x = pack_h2(__builtin_bit_cast(float, a.x), __builtin_bit_cast(float, b.x));
+            out.y = pack_h2(__builtin_bit_cast(float, a.y), __builtin_bit_cast(float, b.y));
+            out.z = pack_h2(__builtin_bit_cast(float, a.z), __builtin_bit_cast(float, b.z));
+            out.w = pack_h2(__builtin_bit_cast(float, a.w), __builtin_bit_cast(float, b.w));
+        }
+        buf[((tid >> 4) + 16 * i) * kPitch16 + x_part] = out;
+    };
+    auto load_w = [&](Q4BlockRaw (&wr)[NU], uint32_t s) {
+        uint32_t blk = s * 4 + g;
+        blk = blk < nb ? blk : nb - 1;
+#pragma unroll
+        for (int u = 0; u < NU; ++u) wr[u] = *reinterpret_cast<const Q4BlockRaw*>(w_row[u] + blk * 5);
+    };
+
+    auto scale_pair = [&](const Q4BlockRaw& blk, bool live, half2v& d2, half2v& b2) {
+        const uint32_t sb = live ? blk.sb : 0u;
+        d2 = as_h2(__builtin_amdgcn_perm(sb, sb, 0x01000100u));  // (d, d)
+        b2 = as_h2(__builtin_amdgcn_perm(sb, sb, 0x03020302u));  // (b, b)
+    };
+
+    // State carried from step to step: the dequantised weights of the coming step's first
+    // quarter and the (scale, bias) pairs of the coming step's blocks.
+    U4 a_cur[NU];
+    half2v d2[NU], b2[NU];
+    XRegs xr;
+
+    // One K step = 4 quarters x 8 token tiles x 4 weight tiles = 128 matrix-core instructions,
+    // issued in a fixed order.  In the shadow of each instruction go one or two steps of the
+    // dequantisation of the NEXT quarter (for the last quarter: the first quarter of step s+1,
+    // from `wnext`), and every fourth token tile one activation unit of step s+1 is written to the
+    // other LDS buffer and refilled from global memory for step s+2.  LDS operand reads run two
+    // token tiles ahead.  `wfree` was consumed in the previous step and is refilled for step s+2.
+    auto step = [&](uint32_t s, Q4BlockRaw (&wr)[NU], Q4BlockRaw (&wnext)[NU], Q4BlockRaw (&wfree)[NU]) {
+        load_w(wfree, s + 2);
+        const uint4* xbuf = lds16 + (s & 1) * kBuf16 + lr * kPitch16 + 4 * g;
+        uint4* xnext = lds16 + ((s + 1) & 1) * kBuf16;
+        const bool live_next = (s + 1) * 4 + g < nb;
+        half2v d2n[NU], b2n[NU];
+        U4 a_nxt[NU];
+        DqTmp tmp;
+        uint4 bx[3];
+        bx[0] = xbuf[0];
+        bx[1] = xbuf[16 * kPitch16];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const int p = j * NT + t;  // slot: (quarter, token tile)
+                if (p + 2 < 4 * NT) {
+                    const int pj = (p + 2) / NT, pt = (p + 2) % NT;
+                    bx[(p + 2) % 3] = xbuf[pt * 16 * kPitch16 + pj];
+                }
+#pragma unroll
+                for (int u = 0; u < NU; ++u) {
+                    const int c = t * NU + u;  // instruction index inside the quarter, 0..31
+                    acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                        __builtin_bit_cast(half8, a_cur[u]), __builtin_bit_cast(half8, bx[p % 3]), acc[u][t], 0, 0,
+                        0);
+#pragma unroll
+                    for (int e = c * (NU * kDqOps) / 32; e < (c + 1) * (NU * kDqOps) / 32; ++e) {
+                        const int uu = e / kDqOps, op = e % kDqOps;
+                        if (j < 3) dq_op(op, wr[uu].q[j + 1], d2[uu], b2[uu], tmp, a_nxt[uu]);
+                        else dq_op(op, wnext[uu].q[0], d2n[uu], b2n[uu], tmp, a_nxt[uu]);
+                    }
+                    if (j == 2 && t == NT - 1) scale_pair(wnext[u], live_next, d2n[u], b2n[u]);
+                    if (u == NU - 1 && (p & 3) == 1) {
+                        store_x_unit(xr, p >> 2, xnext);
+                        load_x_unit(xr, p >> 2, s + 2);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < NU; ++u) a_cur[u] = a_nxt[u];
+        }
+#pragma unroll
+        for (int u = 0; u < NU; ++u) {
+            d2[u] = d2n[u];
+            b2[u] = b2n[u];
+        }
+        __syncthreads();
+    };
+
+    Q4BlockRaw wa[NU], wb[NU], wc[NU];
+#pragma unroll
+    for (int i = 0; i < XU; ++i) load_x_unit(xr, i, 0);
+    load_w(wa, 0);
+    load_w(wb, 1);
+#pragma unroll
+    for (int i = 0; i < XU; ++i) {
+        store_x_unit(xr, i, lds16);
+        load_x_unit(xr, i, 1);
+    }
+    {
+        DqTmp tmp;
+#pragma unroll
+        for (int u = 0; u < NU; ++u) {
+            scale_pair(wa[u], g < nb, d2[u], b2[u]);
+#pragma unroll
+            for (int op = 0; op < kDqOps; ++op) dq_op(op, wa[u].q[0], d2[u], b2[u], tmp, a_cur[u]);
+        }
+    }
+    __syncthreads();
+
+    uint32_t s = 0;
+    for (; s + 3 <= nsteps; s += 3) {
+        step(s, wa, wb, wc);
+        step(s + 1, wb, wc, wa);
+        step(s + 2, wc, wa, wb);
+    }
+    if (s < nsteps) step(s, wa, wb, wc);
+    if (s + 1 < nsteps) step(s + 1, wb, wc, wa);
+
+    // ---- epilogue: element v of lane l of a 16x16 result is weight row 4*(l/16) + v, token l%16
+    const bool vec_ok = (n & 3u) == 0;
+#pragma unroll
+    for (int u = 0; u < NU; ++u) {
+        const uint32_t gn = n0 + wave * 64 + u * 16 + 4 * g;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const uint32_t gm = m0 + t * 16 + lr;
+            if (gm >= m || gn >= n) continue;
+            float4v val = acc[u][t];
+            if (lora.rank) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    if (gn + v >= n) break;
+                    float sacc = 0.0f;
+                    for (uint32_t jj = 0; jj < lora.rank; ++jj)
+                        sacc += load_b(lora.b, lora.b_is_f16, static_cast<size_t>(gn + v) * lora.rank + jj) *
+                                lora.t[static_cast<size_t>(gm) * lora.rank + jj];
+                    val[v] += lora.scale * sacc;
+                }
+            }
+            float* dst = y + static_cast<size_t>(gm) * n + gn;
+            if (vec_ok) {
+                *reinterpret_cast<float4v*>(dst) = val;
+            } else {
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (gn + v < n) dst[v] = val[v];
+            }
+        }
+    }
+}
+
+}  // namespace
+
+uint32_t gemm_wreg_tiles(uint32_t n, uint32_t m) { return ((n + TN - 1) / TN) * ((m + TM - 1) / TM); }
+
+void launch_gemm_wreg(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
+                      float* y, const LoraEpilogue& lora, hipStream_t stream) {
+    const uint32_t tiles = gemm_wreg_tiles(n, m);
+    const size_t lds = 2 * kBuf16 * sizeof(uint4);
+    static bool attr_set = false;
+    if (!attr_set) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4_wreg<true>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4_wreg<false>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        attr_set = true;
+    }
+    if (x_is_f16)
+        hipLaunchKernelGGL(gemm_q4_wreg<true>, dim3(tiles), dim3(256), lds, stream, w, n, k, x, m, y, lora);
+    else
+        hipLaunchKernelGGL(gemm_q4_wreg<false>, dim3(tiles), dim3(256), lds, stream, w, n, k, x, m, y, lora);
+}
+
+}  // namespace lq4

@@ -53,6 +53,12 @@ void launch_lora_b_accum(const void* b, int b_is_f16, uint32_t rank, uint32_t d_
 void launch_gemm(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
                  float* y, const LoraEpilogue& lora, hipStream_t stream);
 
+// Large-shape variant: weights dequantised in registers, only activations staged in LDS.
+// Tile 128 tokens x 256 weight rows; gemm_wreg_tiles = workgroups it would launch.
+uint32_t gemm_wreg_tiles(uint32_t n, uint32_t m);
+void launch_gemm_wreg(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
+                      float* y, const LoraEpilogue& lora, hipStream_t stream);
+
 void launch_probe_read(const void* p, size_t nbytes, uint32_t* sink, hipStream_t stream);
 void launch_dequant(const uint8_t* w, uint32_t n, uint32_t k, float* out, hipStream_t stream);
 

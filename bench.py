@@ -28,6 +28,10 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense f16
 
+# rocprofv3 counters on this workload (profiles/gemv_q4_b1_decode_layer_traffic.md): per layer step
+# FETCH_SIZE 15068 KiB x 2.000 (copy-kernel scale) + WRITE_SIZE 152 KiB x 1.000, over 4 launches
+MEASURED_TRAFFIC_PER_LAUNCH = (15068.0 * 2.0 + 152.0) * 1024 / 4
+
 LAYER = [("qkv", 3072, 2048), ("o", 2048, 2048), ("gate_up", 12288, 2048), ("down", 2048, 6144)]
 
 
@@ -95,6 +99,8 @@ def main():
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--skip-extras", action="store_true", help="headline workload only")
     ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="run nothing but warmup and the timed headline region (for kernel-trace profiles)")
     ap.add_argument("--eager", action="store_true",
                     help="launch every step from Python instead of replaying a captured HIP graph")
     args = ap.parse_args()
@@ -149,13 +155,15 @@ def main():
         layer_step(i)
     tm = timed if args.eager else graph_timed
     ms_step = tm(torch, layer_step, args.steps)
-    eager_ms = timed(torch, layer_step, args.steps)
+    if args.headline_only:
+        args.skip_extras = args.skip_cpu = True
+    eager_ms = ms_step if args.headline_only else timed(torch, layer_step, args.steps)
     value = step_bytes / (ms_step * 1e-3) / 1e9
     launches_per_step = len(LAYER)
     us_per_launch = ms_step * 1e3 / launches_per_step
 
     # same loop on one layer: weights stay in the Infinity Cache
-    hot_ms = tm(torch, lambda i: layer_step(0), max(50, args.steps // 4))
+    hot_ms = ms_step if args.headline_only else tm(torch, lambda i: layer_step(0), max(50, args.steps // 4))
 
     out = {
         "metric": "Q4 GEMV HBM GB/s @batch 1 (Qwen3.5-2B decode layer)",
@@ -188,12 +196,14 @@ def main():
                       "GB/s": round(step_bytes / (hot_ms * 1e-3) / 1e9, 1)},
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_q4_b1<R>" if B == 1 else "gemv_q4_rows<%d>" % (2 if B == 2 else 4 if B <= 4 else 8),
+            "kernel": "gemv_q4_b1" if B == 1 else "gemv_q4_mfma",
             "achieved": round(value, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(value / HBM_PEAK_GBPS, 4),
-            "traffic": None,
+            # HBM-side bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what
+            # the same counter reads for the library's plain copy kernel; measured on this workload
+            "traffic": MEASURED_TRAFFIC_PER_LAUNCH if B == 1 else None,
             "algorithmic_bytes_per_launch": step_bytes / launches_per_step,
             "avg_launch_us": round(us_per_launch, 3),
         },
@@ -288,6 +298,16 @@ def main():
                                    "ms_per_step": round(ms, 4), "GB/s": round(moe_bytes / ms / 1e6, 1),
                                    "pct_of_hbm_peak": round(100 * moe_bytes / ms / 1e6 / HBM_PEAK_GBPS, 2)}
         del sets
+
+        # plain copies of known size: what a profiler's HBM traffic counters are scaled by
+        csrc = torch.empty(64 << 20, dtype=torch.int32, device="cuda").random_(generator=gen)
+        cdst = torch.empty_like(csrc)
+        for _ in range(3):
+            be.probe_copy(csrc, cdst)
+        torch.cuda.synchronize()
+        out["traffic_calibration"] = {"kernel": "probe_copy_kernel", "bytes_read": csrc.numel() * 4,
+                                      "bytes_written": csrc.numel() * 4, "launches": 3}
+        del csrc, cdst
 
     # ---- CPU baseline: the reference's CPU route, timed on this box's host cores --------
     if not args.skip_cpu:

@@ -161,9 +161,14 @@ int lq4_dequant(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
 
 /* Calibration: one launch that only streams `nbytes` (16-byte aligned buffer) through the
  * vector memory path.  Timing it gives the read-bandwidth ceiling of this GPU at that
- * launch size, the figure the GEMV kernels are held against; rocprofv3 counter runs use it
- * as the copy kernel of known size.  No counterpart in the reference. */
+ * launch size, the figure the GEMV kernels are held against.  No counterpart in the
+ * reference. */
 int lq4_probe_read(lq4_ctx* ctx, const void* p_dev, size_t nbytes, void* stream);
+
+/* Calibration: plain device copy of `nbytes` (both buffers 16-byte aligned, nbytes a multiple
+ * of 16).  It reads and writes exactly nbytes, which scales the memory-traffic counters of a
+ * profiler run.  No counterpart in the reference. */
+int lq4_probe_copy(lq4_ctx* ctx, const void* src_dev, void* dst_dev, size_t nbytes, void* stream);
 
 /* Launch counters per kernel family since context creation (the role of
  * PathProofCounters, metal_qwen35.rs:2144-2190): proves which path served a call. */

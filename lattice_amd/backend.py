@@ -46,6 +46,7 @@ EXPORTS = [
     "lq4_weight_info", "lq4_lora_upload", "lq4_lora_free", "lq4_lora_apply", "lq4_gemv",
     "lq4_gemm", "lq4_moe_route", "lq4_moe_grouped_gemv", "lq4_dequant",
     "lq4_probe_read",
+    "lq4_probe_copy",
     "lq4_get_path_counters", "lq4_malloc", "lq4_free", "lq4_memcpy_h2d", "lq4_memcpy_d2h",
 ]
 
@@ -102,6 +103,7 @@ def load_library() -> C.CDLL:
         "lq4_moe_grouped_gemv": (C.c_int, [vp, vp, vp, u32, u32, u32, vp, u32, vp, vp, u32, vp, vp]),
         "lq4_dequant": (C.c_int, [vp, vp, u64, u32, u32, vp, vp]),
         "lq4_probe_read": (C.c_int, [vp, vp, C.c_size_t, vp]),
+        "lq4_probe_copy": (C.c_int, [vp, vp, vp, C.c_size_t, vp]),
         "lq4_get_path_counters": (C.c_int, [vp, C.POINTER(PathCounters)]),
         "lq4_malloc": (C.c_int, [vp, C.c_size_t, C.POINTER(vp)]),
         "lq4_free": (C.c_int, [vp, vp]),
@@ -211,6 +213,13 @@ class HipQ4Backend:
     def probe_read(self, t):
         """One read-only streaming launch over tensor ``t`` (bandwidth-ceiling calibration)."""
         _check(self.lib.lq4_probe_read(self.ctx, t.data_ptr(), t.numel() * t.element_size(), self._stream()))
+
+    def probe_copy(self, src, dst):
+        """One plain copy launch src -> dst (equal-sized tensors): traffic-counter calibration."""
+        nbytes = src.numel() * src.element_size()
+        if dst.numel() * dst.element_size() != nbytes:
+            raise Q4Error(-1, "probe_copy needs equal-sized buffers")
+        _check(self.lib.lq4_probe_copy(self.ctx, src.data_ptr(), dst.data_ptr(), nbytes, self._stream()))
 
     # ------------------------------------------------------- weights / residency
     def upload_q4_blocks(self, blocks, payload_offset: int = 0, validate: bool = True) -> Q4WeightBuf:

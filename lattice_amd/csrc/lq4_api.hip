@@ -436,6 +436,16 @@ int lq4_probe_read(lq4_ctx* ctx, const void* p_dev, size_t nbytes, void* stream)
     return LQ4_OK;
 }
 
+int lq4_probe_copy(lq4_ctx* ctx, const void* src_dev, void* dst_dev, size_t nbytes, void* stream) {
+    if (!ctx || !src_dev || !dst_dev) return fail(LQ4_E_INVALID, "null argument");
+    if (reinterpret_cast<uintptr_t>(src_dev) % 16 || reinterpret_cast<uintptr_t>(dst_dev) % 16 || nbytes % 16)
+        return fail(LQ4_E_INVALID, "buffers and size must be multiples of 16 bytes");
+    DeviceGuard g(ctx->device);
+    launch_probe_copy(src_dev, dst_dev, nbytes, static_cast<hipStream_t>(stream));
+    LQ4_HIP(hipGetLastError());
+    return LQ4_OK;
+}
+
 int lq4_get_path_counters(const lq4_ctx* ctx, lq4_path_counters* out) {
     if (!ctx || !out) return fail(LQ4_E_INVALID, "null argument");
     *out = ctx->counters;

@@ -60,6 +60,7 @@ void launch_gemm_wreg(const uint8_t* w, uint32_t n, uint32_t k, const void* x, i
                       float* y, const LoraEpilogue& lora, hipStream_t stream);
 
 void launch_probe_read(const void* p, size_t nbytes, uint32_t* sink, hipStream_t stream);
+void launch_probe_copy(const void* src, void* dst, size_t nbytes, hipStream_t stream);
 void launch_dequant(const uint8_t* w, uint32_t n, uint32_t k, float* out, hipStream_t stream);
 
 void launch_moe_route(const float* logits, uint32_t tokens, uint32_t num_experts, uint32_t top_k,

@@ -375,3 +375,15 @@ def test_path_counters_prove_the_hip_kernels_ran(be):
     be.dispatch_gemm(x, 0, qw, y, 0, 32, 8, 64)
     after = be.path_counters()
     assert after["gemv"] == before["gemv"] + 1 and after["gemm"] == before["gemm"] + 1
+
+
+def test_probe_copy_copies_exactly(be):
+    import torch
+    src = torch.arange(1 << 20, dtype=torch.int32, device="cuda")
+    dst = torch.zeros_like(src)
+    be.probe_copy(src, dst)
+    be.probe_read(src)
+    torch.cuda.synchronize()
+    assert torch.equal(src, dst)
+    with pytest.raises(backend.Q4Error):
+        be.probe_copy(src, dst[:-1])

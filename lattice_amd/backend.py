@@ -47,6 +47,7 @@ EXPORTS = [
     "lq4_gemm", "lq4_moe_route", "lq4_moe_grouped_gemv", "lq4_dequant",
     "lq4_probe_read",
     "lq4_probe_copy",
+    "lq4_set_gemm_kernel",
     "lq4_get_path_counters", "lq4_malloc", "lq4_free", "lq4_memcpy_h2d", "lq4_memcpy_d2h",
 ]
 
@@ -104,6 +105,7 @@ def load_library() -> C.CDLL:
         "lq4_dequant": (C.c_int, [vp, vp, u64, u32, u32, vp, vp]),
         "lq4_probe_read": (C.c_int, [vp, vp, C.c_size_t, vp]),
         "lq4_probe_copy": (C.c_int, [vp, vp, vp, C.c_size_t, vp]),
+        "lq4_set_gemm_kernel": (C.c_int, [C.c_int]),
         "lq4_get_path_counters": (C.c_int, [vp, C.POINTER(PathCounters)]),
         "lq4_malloc": (C.c_int, [vp, C.c_size_t, C.POINTER(vp)]),
         "lq4_free": (C.c_int, [vp, vp]),
@@ -213,6 +215,10 @@ class HipQ4Backend:
     def probe_read(self, t):
         """One read-only streaming launch over tensor ``t`` (bandwidth-ceiling calibration)."""
         _check(self.lib.lq4_probe_read(self.ctx, t.data_ptr(), t.numel() * t.element_size(), self._stream()))
+
+    def set_gemm_kernel(self, which: int):
+        """0 = pick the prefill kernel by shape, 1 = LDS-staged tile, 2 = weights in registers."""
+        _check(self.lib.lq4_set_gemm_kernel(int(which)))
 
     def probe_copy(self, src, dst):
         """One plain copy launch src -> dst (equal-sized tensors): traffic-counter calibration."""

@@ -436,6 +436,12 @@ int lq4_probe_read(lq4_ctx* ctx, const void* p_dev, size_t nbytes, void* stream)
     return LQ4_OK;
 }
 
+int lq4_set_gemm_kernel(int which) {
+    if (which < 0 || which > 2) return fail(LQ4_E_INVALID, "gemm kernel choice must be 0, 1 or 2");
+    set_gemm_kernel_choice(which);
+    return LQ4_OK;
+}
+
 int lq4_probe_copy(lq4_ctx* ctx, const void* src_dev, void* dst_dev, size_t nbytes, void* stream) {
     if (!ctx || !src_dev || !dst_dev) return fail(LQ4_E_INVALID, "null argument");
     if (reinterpret_cast<uintptr_t>(src_dev) % 16 || reinterpret_cast<uintptr_t>(dst_dev) % 16 || nbytes % 16)

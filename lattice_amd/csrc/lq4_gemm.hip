@@ -23,6 +23,8 @@
 // small set of token tiles: their activations stay in that XCD's L2 while weights stream.
 #include <stdlib.h>
 
+#include <atomic>
+
 #include "lq4_internal.hpp"
 
 namespace lq4 {
@@ -302,17 +304,21 @@ void launch_tile(const uint8_t* w, uint32_t n, uint32_t k, const void* x, uint32
 // tile of this file, two workgroups per CU, is faster.
 constexpr uint32_t kWregMinTiles = 512;
 
+// kernel choice override: starts from the environment variable LQ4_GEMM_KERNEL (0, 1 or 2)
+std::atomic<int> g_gemm_choice{[] {
+    const char* e = getenv("LQ4_GEMM_KERNEL");
+    return e ? atoi(e) : 0;
+}()};
+
 }  // namespace
+
+void set_gemm_kernel_choice(int which) { g_gemm_choice.store(which, std::memory_order_relaxed); }
 
 void launch_gemm(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
                  float* y, const LoraEpilogue& lora, hipStream_t stream) {
-    // LQ4_GEMM_KERNEL=1 forces the LDS-staged kernels of this file, 2 the weights-in-registers
-    // kernel; anything else picks by shape.
-    static const int forced = [] {
-        const char* e = getenv("LQ4_GEMM_KERNEL");
-        return e ? atoi(e) : 0;
-    }();
-    if (forced == 2 || (forced != 1 && gemm_wreg_tiles(n, m) >= kWregMinTiles))
+    const int forced = g_gemm_choice.load(std::memory_order_relaxed);
+    if (forced != 1 && gemm_wreg_supports(n, k, m, x_is_f16) &&
+        (forced == 2 || gemm_wreg_tiles(n, m) >= kWregMinTiles))
         return launch_gemm_wreg(w, n, k, x, x_is_f16, m, y, lora, stream);
     if (x_is_f16) launch_tile<true, 128>(w, n, k, x, m, y, lora, stream);
     else launch_tile<false, 128>(w, n, k, x, m, y, lora, stream);

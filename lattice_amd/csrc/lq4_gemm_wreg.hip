@@ -329,6 +329,8 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
 
 uint32_t gemm_wreg_tiles(uint32_t n, uint32_t m) { return ((n + TN - 1) / TN) * ((m + TM - 1) / TM); }
 
+bool gemm_wreg_supports(uint32_t, uint32_t k, uint32_t, int) { return k >= kBlockWeights; }
+
 void launch_gemm_wreg(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
                       float* y, const LoraEpilogue& lora, hipStream_t stream) {
     const uint32_t tiles = gemm_wreg_tiles(n, m);

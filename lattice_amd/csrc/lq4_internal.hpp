@@ -54,8 +54,12 @@ void launch_gemm(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_
                  float* y, const LoraEpilogue& lora, hipStream_t stream);
 
 // Large-shape variant: weights dequantised in registers, only activations staged in LDS.
-// Tile 128 tokens x 256 weight rows; gemm_wreg_tiles = workgroups it would launch.
+// Tile 128 tokens x 256 weight rows; gemm_wreg_tiles = workgroups it would launch;
+// gemm_wreg_supports = the kernel can run the shape at all.
 uint32_t gemm_wreg_tiles(uint32_t n, uint32_t m);
+bool gemm_wreg_supports(uint32_t n, uint32_t k, uint32_t m, int x_is_f16);
+// 0 = choose by shape, 1 = LDS-staged kernel, 2 = weights-in-registers kernel where supported.
+void set_gemm_kernel_choice(int which);
 void launch_gemm_wreg(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
                       float* y, const LoraEpilogue& lora, hipStream_t stream);
 

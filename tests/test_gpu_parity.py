@@ -387,3 +387,51 @@ def test_probe_copy_copies_exactly(be):
     assert torch.equal(src, dst)
     with pytest.raises(backend.Q4Error):
         be.probe_copy(src, dst[:-1])
+
+
+WREG_CASES = [(5, 9, 128, "f16"), (130, 300, 256, "f16"), (129, 257, 384, "f32"), (257, 513, 640, "f16"),
+              (128, 256, 128, "f32"), (300, 64, 5120, "f16")]
+
+
+@pytest.mark.parametrize("m,n,k,xdt", WREG_CASES)
+def test_gemm_weights_in_registers_kernel_matches_oracle(be, m, n, k, xdt):
+    # the large-shape prefill kernel, forced onto small and ragged shapes (M, N tails; 1..40 K steps)
+    import torch
+    print(f"gemm wreg m={m} n={n} k={k} x={xdt}", flush=True)
+    wq = synth.q4_weight(n, k, seed=5, symmetric_bias=(k != 256))
+    x = synth.activations(m, k, seed=5, dtype=np.float16 if xdt == "f16" else np.float32)
+    qw = be.upload_q4_blocks(wq)
+    y = torch.full((m + 1, n), float("nan"), dtype=torch.float32, device="cuda")
+    y1 = torch.empty((m, n), dtype=torch.float32, device="cuda")
+    be.set_gemm_kernel(2)
+    try:
+        be.dispatch_gemm(dev(x), 0, qw, y, 0, m, n, k)
+        be.set_gemm_kernel(1)
+        be.dispatch_gemm(dev(x), 0, qw, y1, 0, m, n, k)
+    finally:
+        be.set_gemm_kernel(0)
+    got = host(y)
+    assert np.all(np.isnan(got[m])) and np.all(np.isfinite(got[:m]))
+    ref = oracle.gemm_f32(x.astype(np.float32), wq, n, k)
+    e = rel_err(got[:m], ref)
+    print(f"  rel err {e:.2e}; vs LDS-staged kernel {rel_err(got[:m], host(y1)):.2e}", flush=True)
+    assert e <= REL_TOL
+    assert rel_err(host(y1), ref) <= REL_TOL
+
+
+def test_gemm_weights_in_registers_kernel_with_lora(be):
+    import torch
+    m, n, k, r = 70, 130, 256, 16
+    wq = synth.q4_weight(n, k, seed=6)
+    x = synth.activations(m, k, seed=6, dtype=np.float16)
+    a, b = synth.lora_pair(r, k, n, seed=6)
+    qw = be.upload_q4_blocks(wq)
+    be.load_lora_adapter([backend.LoraLayerData(0, {"q_proj": (a, b)})], scale=2.0)
+    y = torch.empty((m, n), dtype=torch.float32, device="cuda")
+    be.set_gemm_kernel(2)
+    try:
+        be.dispatch_gemm(dev(x), 0, qw, y, 0, m, n, k, layer_idx=0, module="q_proj")
+    finally:
+        be.set_gemm_kernel(0)
+        be.unload_lora_adapter()
+    assert rel_err(host(y), _lora_ref(x, wq, n, k, a, b, 2.0)) <= REL_TOL

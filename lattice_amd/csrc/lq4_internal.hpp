@@ -88,6 +88,16 @@ void launch_moe_grouped(const uint8_t* gate_up, const uint8_t* down, uint32_t nu
                         const int32_t* ids, const float* weights, uint32_t top_k, float* y,
                         const MoeScratch& s, hipStream_t stream);
 
+// Matrix-core forms of the two expert passes (activations of a pass staged in LDS:
+// moe_mfma_lds_bytes(k) bytes for a reduction length k).
+size_t moe_mfma_lds_bytes(uint32_t k);
+void launch_moe_gate_up_mfma(const uint8_t* gate_up, uint32_t num_experts, uint32_t inter, uint32_t hidden,
+                             const float* x, uint32_t tokens, uint32_t top_k, const int32_t* offsets,
+                             const int32_t* order, float* h, hipStream_t stream);
+void launch_moe_down_mfma(const uint8_t* down, uint32_t num_experts, uint32_t inter, uint32_t hidden,
+                          const float* h, uint32_t tokens, const int32_t* offsets, const int32_t* order, float* o,
+                          hipStream_t stream);
+
 // ---- device helpers ---------------------------------------------------------------
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t bits16) {
     // v_cvt_f32_f16 widens exactly, subnormals included (f16 denormals are not flushed

@@ -13,6 +13,7 @@ namespace {
 
 constexpr int kMaxTopK = 16;
 constexpr int kMaxExperts = 1024;
+constexpr uint32_t kSmallPairs = 512;  // pair count up to which the grouping kernel ranks by scanning
 
 __global__ void moe_route_kernel(const float* __restrict__ logits, uint32_t tokens,
                                  uint32_t num_experts, uint32_t top_k, int32_t* __restrict__ ids,
@@ -58,32 +59,118 @@ __global__ void moe_route_kernel(const float* __restrict__ logits, uint32_t toke
     }
 }
 
-// Single workgroup: counts per expert, exclusive prefix, then a stable fill of `order`
-// (pairs of one expert stay in ascending pair index, so results do not depend on
-// scheduling).
+// Single workgroup: counts per expert, exclusive prefix, then a stable fill of `order` (the
+// pairs of one expert stay in ascending pair index).  Each of the four waves owns a contiguous
+// segment of the pairs: it counts its segment, receives a cursor per expert that starts where
+// the lower segments end, and then walks its segment 64 pairs at a time, ranking the lanes
+// that share an expert with a ballot.
 __global__ __launch_bounds__(256) void moe_group_kernel(const int32_t* __restrict__ ids,
                                                         uint32_t pairs, uint32_t num_experts,
                                                         int32_t* __restrict__ counts,
                                                         int32_t* __restrict__ offsets,
                                                         int32_t* __restrict__ order) {
+    __shared__ int32_t s_cnt[4 * kMaxExperts];  // [wave][expert]: counts, later cursors
     __shared__ int32_t s_off[kMaxExperts + 1];
-    for (uint32_t e = threadIdx.x; e < num_experts; e += 256) {
-        int32_t c = 0;
-        for (uint32_t p = 0; p < pairs; ++p) c += (ids[p] == static_cast<int32_t>(e));
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (pairs <= kSmallPairs && num_experts <= 256) {
+        // decode-sized batches: ids live in LDS, every thread ranks its own pairs by scanning the
+        // ids before them (a broadcast read per step), one global round trip in and one out
+        int32_t* s_ids = s_cnt + kMaxExperts;
+        for (uint32_t p = tid; p < pairs; p += 256) s_ids[p] = ids[p];
+        if (tid < num_experts) s_cnt[tid] = 0;
+        __syncthreads();
+        for (uint32_t p = tid; p < pairs; p += 256) {
+            const int32_t e = s_ids[p];
+            if (e >= 0 && e < static_cast<int32_t>(num_experts)) atomicAdd(&s_cnt[e], 1);
+        }
+        __syncthreads();
+        if (wave == 0) {
+            int32_t carry = 0;
+            for (uint32_t base = 0; base < num_experts; base += 64) {
+                const uint32_t e = base + lane;
+                const int32_t c = e < num_experts ? s_cnt[e] : 0;
+                int32_t v = c;
+                for (int d = 1; d < 64; d <<= 1) {
+                    const int32_t up = __shfl_up(v, d, 64);
+                    if (static_cast<int>(lane) >= d) v += up;
+                }
+                if (e < num_experts) {
+                    counts[e] = c;
+                    offsets[e + 1] = v + carry;
+                    s_off[e] = v + carry - c;
+                }
+                carry += __shfl(v, 63, 64);
+            }
+            if (lane == 0) offsets[0] = 0;
+        }
+        __syncthreads();
+        for (uint32_t p = tid; p < pairs; p += 256) {
+            const int32_t e = s_ids[p];
+            if (e < 0 || e >= static_cast<int32_t>(num_experts)) continue;
+            int32_t rank = 0;
+            for (uint32_t q = 0; q < p; ++q) rank += (s_ids[q] == e);
+            order[s_off[e] + rank] = static_cast<int32_t>(p);
+        }
+        return;
+    }
+    for (uint32_t i = tid; i < 4 * kMaxExperts; i += 256) s_cnt[i] = 0;
+    __syncthreads();
+    const uint32_t seg = (((pairs + 3) / 4 + 63) / 64) * 64;
+    const uint32_t p_beg = wave * seg < pairs ? wave * seg : pairs;
+    const uint32_t p_end = p_beg + seg < pairs ? p_beg + seg : pairs;
+    for (uint32_t p = p_beg + lane; p < p_end; p += 64) {
+        const int32_t e = ids[p];
+        if (e >= 0 && e < static_cast<int32_t>(num_experts)) atomicAdd(&s_cnt[wave * kMaxExperts + e], 1);
+    }
+    __syncthreads();
+    for (uint32_t e = tid; e < num_experts; e += 256) {
+        const int32_t c = s_cnt[e] + s_cnt[kMaxExperts + e] + s_cnt[2 * kMaxExperts + e] + s_cnt[3 * kMaxExperts + e];
         counts[e] = c;
         s_off[e + 1] = c;
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        s_off[0] = 0;
-        for (uint32_t e = 0; e < num_experts; ++e) s_off[e + 1] += s_off[e];
+    if (wave == 0) {  // inclusive scan of the counts, 64 experts at a time
+        int32_t carry = 0;
+        for (uint32_t base = 0; base < num_experts; base += 64) {
+            const uint32_t e = base + lane;
+            int32_t v = e < num_experts ? s_off[e + 1] : 0;
+            for (int d = 1; d < 64; d <<= 1) {
+                const int32_t up = __shfl_up(v, d, 64);
+                if (static_cast<int>(lane) >= d) v += up;
+            }
+            if (e < num_experts) s_off[e + 1] = v + carry;
+            carry += __shfl(v, 63, 64);
+        }
+        if (lane == 0) s_off[0] = 0;
     }
     __syncthreads();
-    for (uint32_t e = threadIdx.x; e <= num_experts; e += 256) offsets[e] = s_off[e];
-    for (uint32_t e = threadIdx.x; e < num_experts; e += 256) {
-        int32_t at = s_off[e];
-        for (uint32_t p = 0; p < pairs; ++p)
-            if (ids[p] == static_cast<int32_t>(e)) order[at++] = static_cast<int32_t>(p);
+    for (uint32_t e = tid; e <= num_experts; e += 256) offsets[e] = s_off[e];
+    for (uint32_t e = tid; e < num_experts; e += 256) {
+        int32_t run = s_off[e];
+        for (int w = 0; w < 4; ++w) {
+            const int32_t c = s_cnt[w * kMaxExperts + e];
+            s_cnt[w * kMaxExperts + e] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+    volatile int32_t* cur = s_cnt + wave * kMaxExperts;
+    for (uint32_t base = p_beg; base < p_end; base += 64) {
+        const uint32_t p = base + lane;
+        const int32_t e = p < p_end ? ids[p] : -1;
+        const bool valid = e >= 0 && e < static_cast<int32_t>(num_experts);
+        unsigned long long active = __ballot(valid);
+        while (active) {
+            const int leader = __ffsll(static_cast<long long>(active)) - 1;
+            const int32_t le = __shfl(e, leader, 64);
+            const bool mine = valid && e == le;
+            const unsigned long long m = __ballot(mine);
+            if (mine) order[cur[le] + __popcll(m & ((1ull << lane) - 1ull))] = static_cast<int32_t>(p);
+            __builtin_amdgcn_wave_barrier();
+            if (static_cast<int>(lane) == leader) cur[le] = cur[le] + __popcll(m);
+            __builtin_amdgcn_wave_barrier();
+            active &= ~m;
+        }
     }
 }
 
@@ -200,12 +287,21 @@ void launch_moe_grouped(const uint8_t* gate_up, const uint8_t* down, uint32_t nu
     const uint32_t pairs = tokens * top_k;
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(256), 0, stream, ids, pairs, num_experts,
                        s.counts, s.offsets, s.order);
-    hipLaunchKernelGGL(moe_gate_up_kernel, dim3((inter + kMoeWaves - 1) / kMoeWaves, num_experts),
-                       dim3(kMoeWaves * 64), 0, stream, gate_up, inter, hidden, x, top_k, s.offsets,
-                       s.order, s.h);
-    hipLaunchKernelGGL(moe_down_kernel, dim3((hidden + 2 * kMoeWaves - 1) / (2 * kMoeWaves), num_experts),
-                       dim3(kMoeWaves * 64), 0, stream, down, inter, hidden, s.h, s.offsets, s.order,
-                       s.o);
+    // matrix-core kernels whenever one pass's activations fit in LDS; the plain kernels otherwise
+    const size_t lds_cap = 150 * 1024;
+    if (moe_mfma_lds_bytes(hidden) <= lds_cap)
+        launch_moe_gate_up_mfma(gate_up, num_experts, inter, hidden, x, tokens, top_k, s.offsets, s.order, s.h,
+                                stream);
+    else
+        hipLaunchKernelGGL(moe_gate_up_kernel, dim3((inter + kMoeWaves - 1) / kMoeWaves, num_experts),
+                           dim3(kMoeWaves * 64), 0, stream, gate_up, inter, hidden, x, top_k, s.offsets,
+                           s.order, s.h);
+    if (moe_mfma_lds_bytes(inter) <= lds_cap)
+        launch_moe_down_mfma(down, num_experts, inter, hidden, s.h, tokens, s.offsets, s.order, s.o, stream);
+    else
+        hipLaunchKernelGGL(moe_down_kernel, dim3((hidden + 2 * kMoeWaves - 1) / (2 * kMoeWaves), num_experts),
+                           dim3(kMoeWaves * 64), 0, stream, down, inter, hidden, s.h, s.offsets, s.order,
+                           s.o);
     hipLaunchKernelGGL(moe_combine_kernel, dim3((hidden + 255) / 256, tokens), dim3(256), 0, stream,
                        s.o, ids, weights, num_experts, top_k, hidden, y);
 }

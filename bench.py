@@ -258,6 +258,46 @@ def main():
             out["decode_layer_batch8"] = {"ms_per_step": round(ms8, 5), "GB/s": round(b8 / ms8 / 1e6, 1),
                                           "pct_of_hbm_peak": round(100 * b8 / ms8 / 1e6 / HBM_PEAK_GBPS, 2)}
 
+        # single-LoRA epilogue, BASELINE config 3: q (2048x2048) and v (512x2048) projections, rank 16,
+        # f16 factors, scale alpha/r = 2.0, fused into the projection's own launch
+        if B == 1:
+            from lattice_amd import synth
+            r = 16
+            projs = [("q_proj", 2048, 2048), ("v_proj", 512, 2048)]
+            pool = [{nm: be.wrap_device_blocks(device_q4_weight(torch, n, k, gen)) for nm, n, k in projs}
+                    for _ in range(96)]  # 315 MB: more than the Infinity Cache
+            mods = {nm: synth.lora_pair(r, k, n, seed=0, tag=nm) for nm, n, k in projs}
+            lora_out = {}
+            for bsz in (1, 8, 64):
+                xl = torch.randn((bsz, 2048), device="cuda", generator=gen)
+                yl = {nm: torch.empty((bsz, n), device="cuda") for nm, n, _ in projs}
+
+                def lstep(i, use_lora, bsz=bsz, xl=xl, yl=yl):
+                    bufs = pool[i % len(pool)]
+                    for nm, n, k in projs:
+                        kw = dict(layer_idx=0, module=nm) if use_lora else {}
+                        if bsz <= 16:
+                            be.gemv_batch(xl, bufs[nm], yl[nm], bsz, n, k, **kw)
+                        else:
+                            be.dispatch_gemm(xl, 0, bufs[nm], yl[nm], 0, bsz, n, k, **kw)
+                res = {}
+                for use_lora in (False, True):
+                    if use_lora:
+                        be.load_lora_adapter([backend.LoraLayerData(0, mods)], scale=32 / r)
+                    f = lambda i, u=use_lora: lstep(i, u)
+                    for i in range(len(pool)):
+                        f(i)
+                    res[use_lora] = tm(torch, f, 192)
+                    if use_lora:
+                        be.unload_lora_adapter()
+                lb = sum(gemv_bytes(n, k, bsz) + 2 * r * (k + n) + bsz * r * 4 for _, n, k in projs)
+                lora_out["batch%d" % bsz] = {"base_us": round(res[False] * 1e3, 3),
+                                             "with_lora_us": round(res[True] * 1e3, 3),
+                                             "GB/s_with_lora": round(lb / res[True] / 1e6, 1),
+                                             "lora_overhead_pct": round(100 * (res[True] / res[False] - 1), 1)}
+            out["lora_q_v_rank16"] = lora_out
+            del pool
+
         # prefill GEMM, BASELINE config 2
         del layers
         torch.cuda.empty_cache()

@@ -259,6 +259,48 @@ __global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
         compute(xs1, ws1);
     }
 
+    // ---- LoRA: extra K steps of depth 16 over the rank on the matrix cores,
+    //      acc[token, n] += sum_r (scale * t[token, r]) * B[n, r].
+    // Both factors are split hi + lo/2048 into f16 so the delta keeps f32-level accuracy:
+    // t.B = thi.Bhi + tlo.(Bhi/2048) + (thi/2048).Blo; the last term vanishes for f16-stored B.
+    if (lora.rank) {
+        const int r = lane & 31;
+        for (uint32_t r0 = 0; r0 < lora.rank; r0 += 16) {
+            const uint32_t rbase = r0 + 8 * (lane >> 5);  // this lane's eight rank indices
+            half8 t_hi[2], t_his[2], t_lo[2], b_hi[2], b_his[2], b_lo[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                uint32_t tok = m0 + wm + i * 32 + r;
+                tok = tok < m ? tok : m - 1;
+                uint32_t row = n0 + wn + i * 32 + r;
+                row = row < n ? row : n - 1;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const uint32_t idx = rbase + e;
+                    const bool in = idx < lora.rank;
+                    const float tv = in ? lora.scale * lora.t[static_cast<size_t>(tok) * lora.rank + idx] : 0.0f;
+                    const float bv = in ? load_b(lora.b, lora.b_is_f16, static_cast<size_t>(row) * lora.rank + idx) : 0.0f;
+                    const _Float16 th = static_cast<_Float16>(tv), bh = static_cast<_Float16>(bv);
+                    t_hi[i][e] = th;
+                    t_his[i][e] = static_cast<_Float16>(tv * (1.0f / 2048.0f));
+                    t_lo[i][e] = static_cast<_Float16>((tv - static_cast<float>(th)) * 2048.0f);
+                    b_hi[i][e] = bh;
+                    b_his[i][e] = static_cast<_Float16>(bv * (1.0f / 2048.0f));
+                    b_lo[i][e] = static_cast<_Float16>((bv - static_cast<float>(bh)) * 2048.0f);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(t_hi[i], b_hi[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(t_lo[i], b_his[j], acc[i][j], 0, 0, 0);
+                    if (!lora.b_is_f16)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(t_his[i], b_lo[j], acc[i][j], 0, 0, 0);
+                }
+        }
+    }
+
     // ---- epilogue: accumulator element v of lane l is
     //      row 8*(v/4) + 4*(l/32) + v%4, column l%32 of its 32x32 tile
 #pragma unroll
@@ -269,17 +311,7 @@ __global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const uint32_t gm = m0 + wm + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-                if (gm < m && gn < n) {
-                    float val = acc[i][j][v];
-                    if (lora.rank) {
-                        float sacc = 0.0f;
-                        for (uint32_t jj = 0; jj < lora.rank; ++jj)
-                            sacc += load_b(lora.b, lora.b_is_f16, static_cast<size_t>(gn) * lora.rank + jj) *
-                                    lora.t[static_cast<size_t>(gm) * lora.rank + jj];
-                        val += lora.scale * sacc;
-                    }
-                    y[static_cast<size_t>(gm) * n + gn] = val;
-                }
+                if (gm < m && gn < n) y[static_cast<size_t>(gm) * n + gn] = acc[i][j][v];
             }
         }
 }

@@ -292,6 +292,54 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
     if (s < nsteps) step(s, wa, wb, wc);
     if (s + 1 < nsteps) step(s + 1, wb, wc, wa);
 
+    // ---- LoRA: one more K step of depth `rank` on the matrix cores,
+    //      acc[n, token] += sum_r B[n, r] * (scale * t[token, r]).
+    // Both factors are split hi + lo/2048 into f16 so the delta keeps f32-level accuracy:
+    // B.t = Bhi.thi + (Bhi/2048).tlo + Blo.(thi/2048); the last term vanishes for f16-stored B.
+    if (lora.rank) {
+        for (uint32_t r0 = 0; r0 < lora.rank; r0 += 32) {
+            const uint32_t rbase = r0 + 8 * g;  // this lane's eight rank indices
+            half8 b_hi[NU], b_his[NU], b_lo[NU];
+#pragma unroll
+            for (int u = 0; u < NU; ++u) {
+                uint32_t row = n0 + wave * 64 + u * 16 + lr;
+                row = row < n ? row : n - 1;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const uint32_t idx = rbase + i;
+                    const float bv =
+                        idx < lora.rank ? load_b(lora.b, lora.b_is_f16, static_cast<size_t>(row) * lora.rank + idx) : 0.0f;
+                    const _Float16 hi = static_cast<_Float16>(bv);
+                    b_hi[u][i] = hi;
+                    b_his[u][i] = static_cast<_Float16>(bv * (1.0f / 2048.0f));
+                    b_lo[u][i] = static_cast<_Float16>((bv - static_cast<float>(hi)) * 2048.0f);
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                uint32_t tok = m0 + t * 16 + lr;
+                tok = tok < m ? tok : m - 1;
+                half8 t_hi, t_his, t_lo;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const uint32_t idx = rbase + i;
+                    const float tv = idx < lora.rank ? lora.scale * lora.t[static_cast<size_t>(tok) * lora.rank + idx] : 0.0f;
+                    const _Float16 hi = static_cast<_Float16>(tv);
+                    t_hi[i] = hi;
+                    t_his[i] = static_cast<_Float16>(tv * (1.0f / 2048.0f));
+                    t_lo[i] = static_cast<_Float16>((tv - static_cast<float>(hi)) * 2048.0f);
+                }
+#pragma unroll
+                for (int u = 0; u < NU; ++u) {
+                    acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b_hi[u], t_hi, acc[u][t], 0, 0, 0);
+                    acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b_his[u], t_lo, acc[u][t], 0, 0, 0);
+                    if (!lora.b_is_f16)
+                        acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b_lo[u], t_his, acc[u][t], 0, 0, 0);
+                }
+            }
+        }
+    }
+
     // ---- epilogue: element v of lane l of a 16x16 result is weight row 4*(l/16) + v, token l%16
     const bool vec_ok = (n & 3u) == 0;
 #pragma unroll
@@ -301,18 +349,7 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
         for (int t = 0; t < NT; ++t) {
             const uint32_t gm = m0 + t * 16 + lr;
             if (gm >= m || gn >= n) continue;
-            float4v val = acc[u][t];
-            if (lora.rank) {
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    if (gn + v >= n) break;
-                    float sacc = 0.0f;
-                    for (uint32_t jj = 0; jj < lora.rank; ++jj)
-                        sacc += load_b(lora.b, lora.b_is_f16, static_cast<size_t>(gn + v) * lora.rank + jj) *
-                                lora.t[static_cast<size_t>(gm) * lora.rank + jj];
-                    val[v] += lora.scale * sacc;
-                }
-            }
+            const float4v val = acc[u][t];
             float* dst = y + static_cast<size_t>(gm) * n + gn;
             if (vec_ok) {
                 *reinterpret_cast<float4v*>(dst) = val;

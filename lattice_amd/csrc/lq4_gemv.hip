@@ -89,8 +89,22 @@ __global__ __launch_bounds__(256) void lora_a_kernel(const TA* __restrict__ a, u
     const TA* ar = a + static_cast<size_t>(j) * d_in;
     const TX* xr = x + static_cast<size_t>(row) * x_stride;
     float p = 0.0f;
-    for (uint32_t kk = threadIdx.x; kk < d_in; kk += 256)
-        p = fmaf(static_cast<float>(ar[kk]), static_cast<float>(xr[kk]), p);
+    // eight elements per thread and step through 16-byte loads when the rows allow it
+    struct alignas(sizeof(TA) * 8) VA { TA v[8]; };
+    struct alignas(sizeof(TX) * 8) VX { TX v[8]; };
+    const bool vec = d_in % 8 == 0 && reinterpret_cast<uintptr_t>(ar) % sizeof(VA) == 0 &&
+                     reinterpret_cast<uintptr_t>(xr) % sizeof(VX) == 0;
+    if (vec) {
+        for (uint32_t kk = threadIdx.x * 8; kk < d_in; kk += 256 * 8) {
+            const VA av = *reinterpret_cast<const VA*>(ar + kk);
+            const VX xv = *reinterpret_cast<const VX*>(xr + kk);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) p = fmaf(static_cast<float>(av.v[i]), static_cast<float>(xv.v[i]), p);
+        }
+    } else {
+        for (uint32_t kk = threadIdx.x; kk < d_in; kk += 256)
+            p = fmaf(static_cast<float>(ar[kk]), static_cast<float>(xr[kk]), p);
+    }
     p = wave_sum(p);
     __shared__ float part[4];
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = p;

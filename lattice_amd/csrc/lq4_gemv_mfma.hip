@@ -256,6 +256,29 @@ __global__ __launch_bounds__(kThreads) void gemv_q4_mfma(GemvArgs p) {
     // Row group finished for this wave: sum over the 16 blocks of a step (lanes with equal j),
     // meet the other K slices in LDS, and let the slice-0 wave store.
     auto finish = [&](uint32_t it) {
+        // LoRA delta, spread over the 16 lanes that share a weight row: lane group g adds
+        // scale * B[row, r] * t[brow, r] for r = g, g + 16, ... to its partial sums (slice-0 waves
+        // only, so it is counted once); the reduction below then sums it with everything else.
+        if (p.lora.rank && ks == 0) {
+            const uint32_t lrow0 = first_row(it);
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                uint32_t row = lrow0 + 4 * t + j;
+                if (row >= p.n) row = p.n - 1;
+                for (uint32_t r = g; r < p.lora.rank; r += 16) {
+                    const size_t bi = static_cast<size_t>(row) * p.lora.rank + r;
+                    const float bv = p.lora.scale *
+                                     (p.lora.b_is_f16 ? static_cast<float>(static_cast<const _Float16*>(p.lora.b)[bi])
+                                                      : static_cast<const float*>(p.lora.b)[bi]);
+#pragma unroll
+                    for (int c = 0; c < NCOLS; ++c) {
+                        const int brow = HILO ? c / 2 : c;
+                        if ((HILO && (c & 1)) || brow >= static_cast<int>(batch)) continue;
+                        acc[t][c] = fmaf(bv, p.lora.t[brow * p.lora.rank + r], acc[t][c]);
+                    }
+                }
+            }
+        }
 #pragma unroll
         for (int t = 0; t < T; ++t)
 #pragma unroll
@@ -289,18 +312,7 @@ __global__ __launch_bounds__(kThreads) void gemv_q4_mfma(GemvArgs p) {
                     for (int c = 0; c < NCOLS; ++c) {
                         const int brow = HILO ? c / 2 : c;
                         if ((HILO && (c & 1)) || brow >= static_cast<int>(batch)) continue;
-                        float v = HILO ? fmaf(tot[c + (HILO ? 1 : 0)], 1.0f / kLoScale, tot[c]) : tot[c];
-                        if (p.lora.rank) {
-                            float sacc = 0.0f;
-                            for (uint32_t r = 0; r < p.lora.rank; ++r) {
-                                const size_t bi = static_cast<size_t>(row) * p.lora.rank + r;
-                                const float bv = p.lora.b_is_f16
-                                                     ? static_cast<float>(static_cast<const _Float16*>(p.lora.b)[bi])
-                                                     : static_cast<const float*>(p.lora.b)[bi];
-                                sacc = fmaf(bv, p.lora.t[brow * p.lora.rank + r], sacc);
-                            }
-                            v = fmaf(p.lora.scale, sacc, v);
-                        }
+                        const float v = HILO ? fmaf(tot[c + (HILO ? 1 : 0)], 1.0f / kLoScale, tot[c]) : tot[c];
                         p.y[static_cast<size_t>(brow) * p.y_stride + row] = v;
                     }
                 }

@@ -176,11 +176,31 @@ __global__ __launch_bounds__(kThreads) void gemv_q4_mfma(GemvArgs p) {
         }
     };
     stage(it0, 0, x0a, x0b, static_cast<uint32_t>(tid) < items);
-    for (uint32_t b = 0; b < batch; ++b) {
-        for (uint32_t it = (b == 0 ? tid + kThreads : tid); it < items; it += kThreads) {
-            const float4* xp = reinterpret_cast<const float4*>(p.x + static_cast<size_t>(b) * p.x_stride +
-                                                               (it >> 2) * kBlockWeights + (it & 3) * 8);
-            stage(it, b, xp[0], xp[1], true);
+    // the remaining (row, item) pairs, four loads in flight per thread so that a batch of rows costs
+    // a couple of memory round trips, not one per row
+    {
+        constexpr int G = 4;
+        const uint32_t total = batch * items;
+        const uint32_t done = static_cast<uint32_t>(tid) < items ? tid : ~0u;  // staged above
+        for (uint32_t w0 = tid; w0 < total; w0 += G * kThreads) {
+            float4 va[G], vb[G];
+            uint32_t wb[G], wi[G];
+#pragma unroll
+            for (int i = 0; i < G; ++i) {
+                const uint32_t w = w0 + i * kThreads;
+                const uint32_t wc = w < total ? w : 0;
+                wb[i] = wc / items;
+                wi[i] = wc - wb[i] * items;
+                const float4* xp = reinterpret_cast<const float4*>(p.x + static_cast<size_t>(wb[i]) * p.x_stride +
+                                                                   (wi[i] >> 2) * kBlockWeights + (wi[i] & 3) * 8);
+                va[i] = xp[0];
+                vb[i] = xp[1];
+            }
+#pragma unroll
+            for (int i = 0; i < G; ++i) {
+                const uint32_t w = w0 + i * kThreads;
+                stage(wi[i], wb[i], va[i], vb[i], w < total && w != done);
+            }
         }
     }
     if (tid < 4) zero_region[tid] = make_uint4(0u, 0u, 0u, 0u);

@@ -113,32 +113,56 @@ __global__ __launch_bounds__(kThreads) void moe_expert_mfma(MoeGemvArgs p) {
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- stage the activations of this pass: 8 values per (block, dword) item per pair ---------
+    // All (pair, item) combinations of the pass are flattened and taken four at a time, so the loads
+    // of different pairs are in flight together.
     const uint32_t items = nb * 4;
-    for (int b = 0; b < nt; ++b) {
-        const int32_t pair = p.order[beg + b];
-        const float* xr = p.x + static_cast<size_t>(static_cast<uint32_t>(pair) / p.x_div) * p.x_stride;
-        for (uint32_t it = tid; it < items; it += kThreads) {
-            const uint32_t blk = it >> 2, dw = it & 3;
-            const float4* xp = reinterpret_cast<const float4*>(xr + blk * kBlockWeights + dw * 8);
-            const float4 va = xp[0], vb = xp[1];
-            const float v[8] = {va.x, va.y, va.z, va.w, vb.x, vb.y, vb.z, vb.w};
-            _Float16 h[8], l[8];
+    const float* xrow[kTok];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float s = (i & 1) ? v[i] * 0.0625f : v[i];
-                h[i] = static_cast<_Float16>(s);
-                l[i] = static_cast<_Float16>((s - static_cast<float>(h[i])) * kLoScale);
+    for (int b = 0; b < kTok; ++b) {
+        const int32_t pair = p.order[beg + (b < nt ? b : 0)];
+        xrow[b] = p.x + static_cast<size_t>(static_cast<uint32_t>(pair) / p.x_div) * p.x_stride;
+    }
+    {
+        constexpr int G = 4;
+        const uint32_t total = static_cast<uint32_t>(nt) * items;
+        for (uint32_t w0 = tid; w0 < total; w0 += G * kThreads) {
+            float4 va[G], vb[G];
+            uint32_t wb[G], wi[G];
+#pragma unroll
+            for (int i = 0; i < G; ++i) {
+                const uint32_t w = w0 + i * kThreads;
+                const uint32_t wc = w < total ? w : 0;
+                wb[i] = wc / items;
+                wi[i] = wc - wb[i] * items;
+                const float* xr = wb[i] == 0 ? xrow[0] : wb[i] == 1 ? xrow[1] : wb[i] == 2 ? xrow[2] : xrow[3];
+                const float4* xp = reinterpret_cast<const float4*>(xr + (wi[i] >> 2) * kBlockWeights + (wi[i] & 3) * 8);
+                va[i] = xp[0];
+                vb[i] = xp[1];
             }
-            uint4 hi, lo;
-            hi.x = pack_h2(h[0], h[4]); hi.y = pack_h2(h[1], h[5]); hi.z = pack_h2(h[2], h[6]); hi.w = pack_h2(h[3], h[7]);
-            lo.x = pack_h2(l[0], l[4]); lo.y = pack_h2(l[1], l[5]); lo.z = pack_h2(l[2], l[6]); lo.w = pack_h2(l[3], l[7]);
-            float sx = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
-            sx = dpp_add<0xB1>(sx);  // the 4 items of a block sit in 4 adjacent lanes
-            sx = dpp_add<0x4E>(sx);
-            uint4* base = xs16 + blk * kPitch16;
-            base[(2 * b) * 4 + dw] = hi;
-            base[(2 * b + 1) * 4 + dw] = lo;
-            if (dw == 0) reinterpret_cast<float*>(base + kCols * 4)[b] = sx;
+#pragma unroll
+            for (int i = 0; i < G; ++i) {
+                const uint32_t blk = wi[i] >> 2, dw = wi[i] & 3, bb = wb[i];
+                const float v[8] = {va[i].x, va[i].y, va[i].z, va[i].w, vb[i].x, vb[i].y, vb[i].z, vb[i].w};
+                _Float16 h[8], l[8];
+#pragma unroll
+                for (int e2 = 0; e2 < 8; ++e2) {
+                    const float sc = (e2 & 1) ? v[e2] * 0.0625f : v[e2];
+                    h[e2] = static_cast<_Float16>(sc);
+                    l[e2] = static_cast<_Float16>((sc - static_cast<float>(h[e2])) * kLoScale);
+                }
+                uint4 hi, lo;
+                hi.x = pack_h2(h[0], h[4]); hi.y = pack_h2(h[1], h[5]); hi.z = pack_h2(h[2], h[6]); hi.w = pack_h2(h[3], h[7]);
+                lo.x = pack_h2(l[0], l[4]); lo.y = pack_h2(l[1], l[5]); lo.z = pack_h2(l[2], l[6]); lo.w = pack_h2(l[3], l[7]);
+                float sx = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+                sx = dpp_add<0xB1>(sx);  // the 4 items of a block sit in 4 adjacent lanes
+                sx = dpp_add<0x4E>(sx);
+                if (w0 + i * kThreads < total) {
+                    uint4* base = xs16 + blk * kPitch16;
+                    base[(2 * bb) * 4 + dw] = hi;
+                    base[(2 * bb + 1) * 4 + dw] = lo;
+                    if (dw == 0) reinterpret_cast<float*>(base + kCols * 4)[bb] = sx;
+                }
+            }
         }
     }
     if (tid < 4) zero_region[tid] = make_uint4(0u, 0u, 0u, 0u);

@@ -313,6 +313,21 @@ int lq4_lora_apply(lq4_ctx* ctx, const lq4_lora* lora, float lora_scale, const v
     return LQ4_OK;
 }
 
+// Grows the context's scratch buffer (MoE intermediates, GEMM partial sums) to `bytes`.
+// Growing is a synchronising allocation; steady-state calls reuse the buffer.
+static int ensure_scratch(lq4_ctx* ctx, size_t bytes) {
+    if (bytes <= ctx->moe_scratch_bytes) return LQ4_OK;
+    if (ctx->moe_scratch) {
+        LQ4_HIP(hipDeviceSynchronize());
+        (void)hipFree(ctx->moe_scratch);
+        ctx->moe_scratch = nullptr;
+        ctx->moe_scratch_bytes = 0;
+    }
+    LQ4_HIP(hipMalloc(reinterpret_cast<void**>(&ctx->moe_scratch), bytes));
+    ctx->moe_scratch_bytes = bytes;
+    return LQ4_OK;
+}
+
 int lq4_gemm(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
              const void* x_dev, int x_dtype, uint32_t m, float* y_dev, const lq4_lora* lora,
              float lora_scale, void* stream) {
@@ -336,7 +351,14 @@ int lq4_gemm(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
         launch_lora_a(lora->a, lora->is_f16, lora->rank, k, x_dev, x_dtype == LQ4_F16, k, m, ctx->lora_t, s);
         ctx->counters.lora_a++;
     }
-    launch_gemm(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, ep, s);
+    // shapes with too few tiles run as K slices into scratch partials, summed by a second kernel
+    const size_t scratch_bytes = gemm_scratch_floats(n, k, m, x_dtype == LQ4_F16) * sizeof(float);
+    if (scratch_bytes) {
+        rc = ensure_scratch(ctx, scratch_bytes);
+        if (rc) return rc;
+    }
+    launch_gemm(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, ep,
+                scratch_bytes ? reinterpret_cast<float*>(ctx->moe_scratch) : nullptr, s);
     ctx->counters.gemm++;
     LQ4_HIP(hipGetLastError());
     return LQ4_OK;
@@ -387,16 +409,9 @@ int lq4_moe_grouped_gemv(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_weig
     const size_t off_h = off_order + up256(sizeof(int32_t) * pairs);
     const size_t off_o = off_h + up256(sizeof(float) * pairs * inter);
     const size_t total = off_o + up256(sizeof(float) * pairs * hidden);
-    if (total > ctx->moe_scratch_bytes) {
-        // growing the scratch is a synchronising allocation; steady-state calls reuse it
-        if (ctx->moe_scratch) {
-            LQ4_HIP(hipDeviceSynchronize());
-            (void)hipFree(ctx->moe_scratch);
-            ctx->moe_scratch = nullptr;
-            ctx->moe_scratch_bytes = 0;
-        }
-        LQ4_HIP(hipMalloc(reinterpret_cast<void**>(&ctx->moe_scratch), total));
-        ctx->moe_scratch_bytes = total;
+    {
+        const int src = ensure_scratch(ctx, total);
+        if (src) return src;
     }
     MoeScratch s;
     s.counts = reinterpret_cast<int32_t*>(ctx->moe_scratch + off_counts);

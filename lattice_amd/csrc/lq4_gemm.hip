@@ -346,12 +346,37 @@ std::atomic<int> g_gemm_choice{[] {
 
 void set_gemm_kernel_choice(int which) { g_gemm_choice.store(which, std::memory_order_relaxed); }
 
-void launch_gemm(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
-                 float* y, const LoraEpilogue& lora, hipStream_t stream) {
+namespace {
+
+// Which kernel serves a shape, and with how many K slices.
+struct GemmPlan {
+    bool wreg;
+    uint32_t slices;
+};
+
+GemmPlan plan_gemm(uint32_t n, uint32_t k, uint32_t m, int x_is_f16) {
     const int forced = g_gemm_choice.load(std::memory_order_relaxed);
-    if (forced != 1 && gemm_wreg_supports(n, k, m, x_is_f16) &&
-        (forced == 2 || gemm_wreg_tiles(n, m) >= kWregMinTiles))
-        return launch_gemm_wreg(w, n, k, x, x_is_f16, m, y, lora, stream);
+    if (forced == 1 || !gemm_wreg_supports(n, k, m, x_is_f16)) return {false, 1};
+    uint32_t slices = gemm_wreg_slices(n, k, m);
+    if (static_cast<uint64_t>(slices) * m * n > (64ull << 20)) slices = 1;  // keep the partials under 256 MB
+    const uint32_t lds_tiles = ((n + 127) / 128) * ((m + BM - 1) / BM);
+    // big shapes: plenty of 128 x 256 tiles; small shapes: the 128 x 128 tiles cannot fill the chip
+    // either, and slicing K can
+    const bool wreg = forced == 2 || gemm_wreg_tiles(n, m) >= kWregMinTiles || (lds_tiles < 384 && slices > 1);
+    return {wreg, wreg ? slices : 1};
+}
+
+}  // namespace
+
+size_t gemm_scratch_floats(uint32_t n, uint32_t k, uint32_t m, int x_is_f16) {
+    const GemmPlan p = plan_gemm(n, k, m, x_is_f16);
+    return p.slices > 1 ? static_cast<size_t>(p.slices) * m * n : 0;
+}
+
+void launch_gemm(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
+                 float* y, const LoraEpilogue& lora, float* scratch, hipStream_t stream) {
+    const GemmPlan p = plan_gemm(n, k, m, x_is_f16);
+    if (p.wreg) return launch_gemm_wreg(w, n, k, x, x_is_f16, m, y, lora, p.slices, scratch, stream);
     if (x_is_f16) launch_tile<true, 128>(w, n, k, x, m, y, lora, stream);
     else launch_tile<false, 128>(w, n, k, x, m, y, lora, stream);
 }

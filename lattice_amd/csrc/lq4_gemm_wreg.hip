@@ -133,8 +133,16 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
     const uint32_t m0 = (first_m + in_group % group_m) * TM;
     const uint32_t n0 = (in_group / group_m) * TN;
 
-    const uint32_t nb = k / kBlockWeights;
-    const uint32_t nsteps = (nb + 3) / 4;
+    // K slice of this workgroup (gridDim.y slices; one slice = the whole row when gridDim.y == 1).
+    // From here on steps, blocks and K offsets are counted from the start of the slice.
+    const uint32_t nb_total = k / kBlockWeights;
+    const uint32_t steps_total = (nb_total + 3) / 4;
+    const uint32_t steps_per = (steps_total + gridDim.y - 1) / gridDim.y;
+    const uint32_t s_begin = blockIdx.y * steps_per;  // the host never launches an empty slice
+    const uint32_t nsteps = s_begin + steps_per < steps_total ? steps_per : steps_total - s_begin;
+    const uint32_t nb = nb_total - s_begin * 4;       // blocks from the slice start to the end of the row
+    const uint32_t k_rem = k - s_begin * TK;
+    if (gridDim.y > 1) y += static_cast<size_t>(blockIdx.y) * m * n;  // partial sums, one matrix per slice
 
     float4v acc[NU][NT];
 #pragma unroll
@@ -148,7 +156,7 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
     for (int u = 0; u < NU; ++u) {
         uint32_t row = n0 + wave * 64 + u * 16 + lr;
         row = row < n ? row : n - 1;
-        w_row[u] = reinterpret_cast<const uint32_t*>(w) + static_cast<size_t>(row) * (nb * 5);
+        w_row[u] = reinterpret_cast<const uint32_t*>(w) + static_cast<size_t>(row) * (nb_total * 5) + s_begin * 20;
     }
     // activation unit i of this thread: token row tid/16 + 16 i, K offset 8 * (tid % 16) of the step
     const int x_part = tid & 15;
@@ -157,7 +165,8 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
     for (int i = 0; i < XU; ++i) {
         uint32_t row = m0 + (tid >> 4) + 16 * i;
         row = row < m ? row : m - 1;
-        x_row[i] = static_cast<const uint8_t*>(xv) + static_cast<size_t>(row) * k * (X_F16 ? 2 : 4);
+        x_row[i] = static_cast<const uint8_t*>(xv) +
+                   (static_cast<size_t>(row) * k + static_cast<size_t>(s_begin) * TK) * (X_F16 ? 2 : 4);
     }
 
     struct XRegs {
@@ -166,7 +175,7 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
 
     auto load_x_unit = [&](XRegs& xr, int i, uint32_t s) {
         uint32_t koff = s * TK + x_part * 8;
-        koff = koff < k ? koff : k - 8;  // past the end of K: any valid address, weights there are zero
+        koff = koff < k_rem ? koff : k_rem - 8;  // past the end of K: any valid address, weights there are zero
         const size_t byte_off = static_cast<size_t>(koff) * (X_F16 ? 2 : 4);
 #pragma unroll
         for (int l = 0; l < XL; ++l)
@@ -296,7 +305,7 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
     //      acc[n, token] += sum_r B[n, r] * (scale * t[token, r]).
     // Both factors are split hi + lo/2048 into f16 so the delta keeps f32-level accuracy:
     // B.t = Bhi.thi + (Bhi/2048).tlo + Blo.(thi/2048); the last term vanishes for f16-stored B.
-    if (lora.rank) {
+    if (lora.rank && blockIdx.y == 0) {
         for (uint32_t r0 = 0; r0 < lora.rank; r0 += 32) {
             const uint32_t rbase = r0 + 8 * g;  // this lane's eight rank indices
             half8 b_hi[NU], b_his[NU], b_lo[NU];
@@ -362,14 +371,47 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
     }
 }
 
+// y[i] = sum over slices, in slice order, of partial[s][i]  (count multiple of 4 or not)
+__global__ __launch_bounds__(256) void gemm_reduce_slices(const float* __restrict__ partial, uint32_t slices,
+                                                          size_t count, float* __restrict__ y) {
+    const size_t i4 = (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
+    if (i4 >= count) return;
+    if (i4 + 4 <= count && (count & 3) == 0) {
+        float4v v = *reinterpret_cast<const float4v*>(partial + i4);
+        for (uint32_t sl = 1; sl < slices; ++sl) v += *reinterpret_cast<const float4v*>(partial + sl * count + i4);
+        *reinterpret_cast<float4v*>(y + i4) = v;
+    } else {
+        for (size_t i = i4; i < count && i < i4 + 4; ++i) {
+            float v = partial[i];
+            for (uint32_t sl = 1; sl < slices; ++sl) v += partial[sl * count + i];
+            y[i] = v;
+        }
+    }
+}
+
 }  // namespace
 
 uint32_t gemm_wreg_tiles(uint32_t n, uint32_t m) { return ((n + TN - 1) / TN) * ((m + TM - 1) / TM); }
 
 bool gemm_wreg_supports(uint32_t, uint32_t k, uint32_t, int) { return k >= kBlockWeights; }
 
+uint32_t gemm_wreg_slices(uint32_t n, uint32_t k, uint32_t m) {
+    // Too few tiles to occupy the 256 CUs: cut K into slices (whole 128-wide steps) until there
+    // are about that many workgroups.  Each slice writes its own partial matrix; a second kernel
+    // adds them in slice order, so the result does not depend on scheduling.
+    const uint32_t tiles = gemm_wreg_tiles(n, m);
+    const uint32_t steps = (k / kBlockWeights + 3) / 4;
+    if (tiles >= 192 || steps < 4) return 1;
+    uint32_t want = (256 + tiles - 1) / tiles;
+    want = want > 16 ? 16 : want;
+    want = want > steps / 2 ? steps / 2 : want;  // at least two steps per slice
+    if (want <= 1) return 1;
+    const uint32_t per = (steps + want - 1) / want;
+    return (steps + per - 1) / per;  // no empty slice
+}
+
 void launch_gemm_wreg(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
-                      float* y, const LoraEpilogue& lora, hipStream_t stream) {
+                      float* y, const LoraEpilogue& lora, uint32_t slices, float* partial, hipStream_t stream) {
     const uint32_t tiles = gemm_wreg_tiles(n, m);
     const size_t lds = 2 * kBuf16 * sizeof(uint4);
     static bool attr_set = false;
@@ -380,10 +422,18 @@ void launch_gemm_wreg(const uint8_t* w, uint32_t n, uint32_t k, const void* x, i
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         attr_set = true;
     }
+    if (slices <= 1 || !partial) slices = 1;
+    float* out = slices > 1 ? partial : y;
+    const dim3 grid(tiles, slices);
     if (x_is_f16)
-        hipLaunchKernelGGL(gemm_q4_wreg<true>, dim3(tiles), dim3(256), lds, stream, w, n, k, x, m, y, lora);
+        hipLaunchKernelGGL(gemm_q4_wreg<true>, grid, dim3(256), lds, stream, w, n, k, x, m, out, lora);
     else
-        hipLaunchKernelGGL(gemm_q4_wreg<false>, dim3(tiles), dim3(256), lds, stream, w, n, k, x, m, y, lora);
+        hipLaunchKernelGGL(gemm_q4_wreg<false>, grid, dim3(256), lds, stream, w, n, k, x, m, out, lora);
+    if (slices > 1) {
+        const size_t count = static_cast<size_t>(m) * n;
+        hipLaunchKernelGGL(gemm_reduce_slices, dim3(static_cast<uint32_t>((count + 1023) / 1024)), dim3(256), 0,
+                           stream, partial, slices, count, y);
+    }
 }
 
 }  // namespace lq4

@@ -50,8 +50,10 @@ void launch_lora_b_accum(const void* b, int b_is_f16, uint32_t rank, uint32_t d_
                          float scale, uint32_t rows, float* y, uint32_t y_stride, hipStream_t stream);
 
 // Y[M,N] = X[M,K] . W^T (+ LoRA); X f32 or f16, Y f32.
+// gemm_scratch_floats = floats of scratch launch_gemm needs for the shape (0 = none).
+size_t gemm_scratch_floats(uint32_t n, uint32_t k, uint32_t m, int x_is_f16);
 void launch_gemm(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
-                 float* y, const LoraEpilogue& lora, hipStream_t stream);
+                 float* y, const LoraEpilogue& lora, float* scratch, hipStream_t stream);
 
 // Large-shape variant: weights dequantised in registers, only activations staged in LDS.
 // Tile 128 tokens x 256 weight rows; gemm_wreg_tiles = workgroups it would launch;
@@ -60,8 +62,11 @@ uint32_t gemm_wreg_tiles(uint32_t n, uint32_t m);
 bool gemm_wreg_supports(uint32_t n, uint32_t k, uint32_t m, int x_is_f16);
 // 0 = choose by shape, 1 = LDS-staged kernel, 2 = weights-in-registers kernel where supported.
 void set_gemm_kernel_choice(int which);
+// gemm_wreg_slices = K slices it wants for the shape (1 = none); with more than one, `partial`
+// must hold slices * m * n floats.
+uint32_t gemm_wreg_slices(uint32_t n, uint32_t k, uint32_t m);
 void launch_gemm_wreg(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
-                      float* y, const LoraEpilogue& lora, hipStream_t stream);
+                      float* y, const LoraEpilogue& lora, uint32_t slices, float* partial, hipStream_t stream);
 
 void launch_probe_read(const void* p, size_t nbytes, uint32_t* sink, hipStream_t stream);
 void launch_probe_copy(const void* src, void* dst, size_t nbytes, hipStream_t stream);

@@ -166,7 +166,9 @@ def test_weight_views_offsets_and_file_payload(be, golden_dir):
 # ------------------------------------------------------------------ prefill GEMM
 GEMM_CASES = [(64, 64, 64, "f32"), (72, 48, 64, "f32"), (17, 9, 96, "f32"), (5, 9, 96, "f16"),
               (16, 1024, 3584, "f16"), (130, 200, 256, "f16"), (128, 128, 32, "f16"),
-              (64, 512, 5120, "f16"), (96, 256, 17408, "f16")]
+              (64, 512, 5120, "f16"), (96, 256, 17408, "f16"),
+              # few tiles, long K: served as K slices plus a reduction pass (incl. a ragged last step)
+              (64, 2048, 2048, "f32"), (33, 70, 1120, "f16"), (200, 100, 4064, "f32")]
 
 
 @pytest.mark.parametrize("m,n,k,xdt", GEMM_CASES)

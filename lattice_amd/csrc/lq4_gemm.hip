@@ -84,7 +84,9 @@ __device__ __forceinline__ uint4 dequant8(uint32_t q, half2v d2, half2v b2) {
 }
 
 // BN_: weight rows per workgroup (128 or 256); 2*BN_ threads; waves in a 2 x (BN_/64) grid.
-template <bool X_F16, int BN_>
+// LORA: compiled with the LoRA step (kept out of the plain kernel, whose register allocation it
+// would disturb).
+template <bool X_F16, int BN_, bool LORA>
 __global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
     const uint8_t* __restrict__ w, uint32_t n, uint32_t k, const void* __restrict__ xv, uint32_t m,
     float* __restrict__ y, LoraEpilogue lora) {
@@ -263,7 +265,7 @@ __global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
     //      acc[token, n] += sum_r (scale * t[token, r]) * B[n, r].
     // Both factors are split hi + lo/2048 into f16 so the delta keeps f32-level accuracy:
     // t.B = thi.Bhi + tlo.(Bhi/2048) + (thi/2048).Blo; the last term vanishes for f16-stored B.
-    if (lora.rank) {
+    if (LORA && lora.rank) {
         const int r = lane & 31;
         for (uint32_t r0 = 0; r0 < lora.rank; r0 += 16) {
             const uint32_t rbase = r0 + 8 * (lane >> 5);  // this lane's eight rank indices
@@ -316,18 +318,18 @@ __global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
         }
 }
 
-template <bool X_F16, int BN_>
+template <bool X_F16, int BN_, bool LORA>
 void launch_tile(const uint8_t* w, uint32_t n, uint32_t k, const void* x, uint32_t m, float* y,
                  const LoraEpilogue& lora, hipStream_t stream) {
     const uint32_t tiles = ((n + BN_ - 1) / BN_) * ((m + BM - 1) / BM);
     const size_t lds = 2 * (BM + BN_) * kPitch * sizeof(_Float16);
     static bool attr_set = false;
     if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4_mfma<X_F16, BN_>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4_mfma<X_F16, BN_, LORA>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         attr_set = true;
     }
-    hipLaunchKernelGGL((gemm_q4_mfma<X_F16, BN_>), dim3(tiles), dim3(2 * BN_), lds, stream, w, n, k, x, m, y,
+    hipLaunchKernelGGL((gemm_q4_mfma<X_F16, BN_, LORA>), dim3(tiles), dim3(2 * BN_), lds, stream, w, n, k, x, m, y,
                        lora);
 }
 
@@ -377,8 +379,13 @@ void launch_gemm(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_
                  float* y, const LoraEpilogue& lora, float* scratch, hipStream_t stream) {
     const GemmPlan p = plan_gemm(n, k, m, x_is_f16);
     if (p.wreg) return launch_gemm_wreg(w, n, k, x, x_is_f16, m, y, lora, p.slices, scratch, stream);
-    if (x_is_f16) launch_tile<true, 128>(w, n, k, x, m, y, lora, stream);
-    else launch_tile<false, 128>(w, n, k, x, m, y, lora, stream);
+    if (lora.rank) {
+        if (x_is_f16) launch_tile<true, 128, true>(w, n, k, x, m, y, lora, stream);
+        else launch_tile<false, 128, true>(w, n, k, x, m, y, lora, stream);
+    } else {
+        if (x_is_f16) launch_tile<true, 128, false>(w, n, k, x, m, y, lora, stream);
+        else launch_tile<false, 128, false>(w, n, k, x, m, y, lora, stream);
+    }
 }
 
 }  // namespace lq4

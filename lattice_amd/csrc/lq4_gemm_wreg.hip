@@ -109,7 +109,9 @@ __device__ __forceinline__ uint32_t pack_h2(float lo, float hi) {
     return as_u32(h);
 }
 
-template <bool X_F16>
+// LORA: compiled with the LoRA step (kept out of the plain kernel, whose register allocation it
+// would disturb).
+template <bool X_F16, bool LORA>
 __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict__ w, uint32_t n, uint32_t k,
                                                        const void* __restrict__ xv, uint32_t m,
                                                        float* __restrict__ y, LoraEpilogue lora) {
@@ -305,7 +307,7 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
     //      acc[n, token] += sum_r B[n, r] * (scale * t[token, r]).
     // Both factors are split hi + lo/2048 into f16 so the delta keeps f32-level accuracy:
     // B.t = Bhi.thi + (Bhi/2048).tlo + Blo.(thi/2048); the last term vanishes for f16-stored B.
-    if (lora.rank && blockIdx.y == 0) {
+    if (LORA && lora.rank && blockIdx.y == 0) {
         for (uint32_t r0 = 0; r0 < lora.rank; r0 += 32) {
             const uint32_t rbase = r0 + 8 * g;  // this lane's eight rank indices
             half8 b_hi[NU], b_his[NU], b_lo[NU];
@@ -410,25 +412,35 @@ uint32_t gemm_wreg_slices(uint32_t n, uint32_t k, uint32_t m) {
     return (steps + per - 1) / per;  // no empty slice
 }
 
-void launch_gemm_wreg(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
-                      float* y, const LoraEpilogue& lora, uint32_t slices, float* partial, hipStream_t stream) {
-    const uint32_t tiles = gemm_wreg_tiles(n, m);
-    const size_t lds = 2 * kBuf16 * sizeof(uint4);
+namespace {
+
+template <bool X_F16, bool LORA>
+void launch_wreg_t(const uint8_t* w, uint32_t n, uint32_t k, const void* x, uint32_t m, float* out,
+                   const LoraEpilogue& lora, uint32_t slices, hipStream_t stream) {
     static bool attr_set = false;
     if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4_wreg<true>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4_wreg<false>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4_wreg<X_F16, LORA>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         attr_set = true;
     }
+    const size_t lds = 2 * kBuf16 * sizeof(uint4);
+    hipLaunchKernelGGL((gemm_q4_wreg<X_F16, LORA>), dim3(gemm_wreg_tiles(n, m), slices), dim3(256), lds, stream, w,
+                       n, k, x, m, out, lora);
+}
+
+}  // namespace
+
+void launch_gemm_wreg(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
+                      float* y, const LoraEpilogue& lora, uint32_t slices, float* partial, hipStream_t stream) {
     if (slices <= 1 || !partial) slices = 1;
     float* out = slices > 1 ? partial : y;
-    const dim3 grid(tiles, slices);
-    if (x_is_f16)
-        hipLaunchKernelGGL(gemm_q4_wreg<true>, grid, dim3(256), lds, stream, w, n, k, x, m, out, lora);
-    else
-        hipLaunchKernelGGL(gemm_q4_wreg<false>, grid, dim3(256), lds, stream, w, n, k, x, m, out, lora);
+    if (lora.rank) {
+        if (x_is_f16) launch_wreg_t<true, true>(w, n, k, x, m, out, lora, slices, stream);
+        else launch_wreg_t<false, true>(w, n, k, x, m, out, lora, slices, stream);
+    } else {
+        if (x_is_f16) launch_wreg_t<true, false>(w, n, k, x, m, out, lora, slices, stream);
+        else launch_wreg_t<false, false>(w, n, k, x, m, out, lora, slices, stream);
+    }
     if (slices > 1) {
         const size_t count = static_cast<size_t>(m) * n;
         hipLaunchKernelGGL(gemm_reduce_slices, dim3(static_cast<uint32_t>((count + 1023) / 1024)), dim3(256), 0,

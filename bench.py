@@ -217,12 +217,15 @@ def main():
         # matrices driven as batch-1 decode GEMVs: launches large enough to approach the HBM
         # streaming rate.
         shapes = {}
-        extra_shapes = [("cfg0", 4096, 1024), ("27b_up", 17408, 5120), ("27b_down", 5120, 17408)]
+        # "lm_head" is the reference's largest single GEMV per token (vocabulary 248,320 x hidden 2048,
+        # 318 MB of Q4 blocks): one launch big enough to show the kernel's streaming rate.
+        extra_shapes = [("cfg0", 4096, 1024), ("27b_up", 17408, 5120), ("27b_down", 5120, 17408),
+                        ("lm_head", 248320, 2048)]
         for name, n, k in LAYER + extra_shapes:
             wbytes = n * (k // 32) * 20
             pool = [l[name] for l in layers] if name in dict((a, 1) for a, _, _ in LAYER) else \
                 [be.wrap_device_blocks(device_q4_weight(torch, n, k, gen))
-                 for _ in range(max(2, min(400, int(1.2e9 // wbytes))))]
+                 for _ in range(max(3, min(400, int(1.2e9 // wbytes))))]
             x = torch.randn((B, k), device="cuda", generator=gen)
             y = torch.empty((B, n), device="cuda")
             f = lambda i, pool=pool, x=x, y=y, n=n, k=k: be.gemv_batch(x, pool[i % len(pool)], y, B, n, k)

@@ -133,7 +133,9 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_b1(const uint8_t* __restr
     const uint32_t n_waves = gridDim.x * kWaves;
     // the wave index is uniform across the wave: keep it (and everything derived) scalar
     const uint32_t wid = __builtin_amdgcn_readfirstlane(blockIdx.x * kWaves + (tid >> 6));
-    const uint32_t chunks = (n_wrows + n_waves * RW - 1) / (n_waves * RW);
+    // chunks whose first wave-row exists for this wave (later waves may have one chunk fewer)
+    const uint32_t first = wid < n_wrows ? n_wrows - wid : 0;  // wave-rows from this wave's first one on
+    const uint32_t chunks = (first + n_waves * RW - 1) / (n_waves * RW);
     const uint32_t units = chunks * slab_groups;
 
     // ---- first chunk of x is requested before any weight so it can be waited on alone ----
@@ -285,11 +287,24 @@ void launch_gemv_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, fl
     wg_per_cu = wg_per_cu > 4 ? 4 : wg_per_cu < 1 ? 1 : wg_per_cu;
     const uint32_t max_waves = 256 * wg_per_cu * kWaves;
     uint32_t rw = (n_wrows + max_waves - 1) / max_waves;
-    rw = rw > 4 ? 4 : rw;
-    // whole chunks per wave; a grid up to 1.5x the resident capacity beats a second chunk
-    uint32_t chunks = (2 * n_wrows + 3 * max_waves * rw - 1) / (3 * max_waves * rw);
-    chunks = chunks < 1 ? 1 : chunks;
-    const uint32_t waves = (n_wrows + rw * chunks - 1) / (rw * chunks);
+    uint32_t waves;
+    if (rw <= 4) {
+        // every wave resident, one chunk each
+        waves = (n_wrows + rw - 1) / rw;
+    } else {
+        // more rows than one chunk per resident wave covers: a full grid of persistent waves that
+        // walk several chunks.  Waves differ by at most one chunk, so the chunk height is the
+        // largest (most loads in flight) that keeps that imbalance under 8 %.
+        waves = max_waves;
+        rw = 1;
+        for (uint32_t cand = 4; cand > 1; --cand) {
+            const uint32_t most = (n_wrows + max_waves * cand - 1) / (max_waves * cand) * cand;  // rows of the busiest wave
+            if (static_cast<uint64_t>(most) * max_waves * 100 <= static_cast<uint64_t>(n_wrows) * 108) {
+                rw = cand;
+                break;
+            }
+        }
+    }
     uint32_t sg = slabs < 3 ? slabs : 3;
     while (rw * sg > 6) --sg;
 

@@ -108,3 +108,67 @@ def fuse_gate_up(gate_raw: np.ndarray, up_raw: np.ndarray) -> np.ndarray:
     (metal_qwen35.rs:7403-7406)."""
     return np.concatenate([np.ascontiguousarray(gate_raw, dtype=np.uint8),
                            np.ascontiguousarray(up_raw, dtype=np.uint8)])
+
+
+MAX_Q4_MERGE_PAYLOAD_LEN = 4 << 30  # cap on a source payload read for a merge
+
+
+def q4_file_bytes(shape: Sequence[int], original_len: int, payload) -> bytes:
+    """A KHQ4 v2 file image: header for ``shape`` / ``original_len`` followed by ``payload``."""
+    out = bytearray(b"KHQ4")
+    out += (2).to_bytes(4, "little") + len(shape).to_bytes(4, "little")
+    for d in shape:
+        out += int(d).to_bytes(8, "little")
+    out += int(original_len).to_bytes(8, "little")
+    out += bytes(memoryview(np.ascontiguousarray(payload, dtype=np.uint8)))
+    return bytes(out)
+
+
+def write_q4_file(path: str, shape: Sequence[int], payload) -> None:
+    """Writes a ``.q4`` file through a temporary file and an atomic rename, so a crash in the
+    middle never leaves a partial file at the final path."""
+    numel = 1
+    for d in shape:
+        numel *= int(d)
+    tmp = path + ".tmp"
+    try:
+        with open(tmp, "wb") as f:
+            f.write(q4_file_bytes(shape, numel, payload))
+        os.replace(tmp, path)
+    except OSError:
+        if os.path.exists(tmp):
+            os.remove(tmp)
+        raise
+
+
+def read_q4_payload_bounded(path: str, max_payload: int = MAX_Q4_MERGE_PAYLOAD_LEN):
+    """Header and block payload of a ``.q4`` file, read with a size cap (the role of
+    ``read_q4_payload_bounded`` in write_merged_qkvz, q4_weights.rs:1560-1566)."""
+    size = os.stat(path).st_size
+    if size > max_payload + 64:
+        raise Q4FileError(f"{path}: file of {size} bytes exceeds the merge cap of {max_payload} bytes")
+    data = np.fromfile(path, dtype=np.uint8)
+    h = validate_q4_file(data, path)
+    return h, data[h.payload_offset:]
+
+
+def merge_q4_files(first_path: str, second_path: str, out_path: str) -> Q4FileHeader:
+    """``write_merged_qkvz`` (q4_weights.rs:1552-1636): concatenates two 2-D ``.q4`` tensors with
+    the same hidden width along the rows — payload bytes verbatim, new header with the summed
+    row count and ``original_len`` — and writes the result atomically.  Both inputs must be
+    exactly 2-D (a rank-0 header must not be indexed)."""
+    h1, p1 = read_q4_payload_bounded(first_path)
+    h2, p2 = read_q4_payload_bounded(second_path)
+    if len(h1.shape) != 2:
+        raise Q4FileError(f"{first_path}: qkv header shape {list(h1.shape)} is not 2-D (expected [rows, hidden])")
+    if len(h2.shape) != 2:
+        raise Q4FileError(f"{second_path}: z header shape {list(h2.shape)} is not 2-D (expected [rows, hidden])")
+    if h1.shape[1] != h2.shape[1]:
+        raise Q4FileError(f"{first_path}/{second_path}: qkv hidden dimension {h1.shape[1]} does not match "
+                          f"z hidden dimension {h2.shape[1]}")
+    if h1.shape[1] % BLOCK_WEIGHTS:
+        raise Q4FileError(f"{first_path}: hidden dimension {h1.shape[1]} is not a multiple of {BLOCK_WEIGHTS}: "
+                          f"rows are not block-aligned and cannot be concatenated")
+    shape = (h1.shape[0] + h2.shape[0], h1.shape[1])
+    write_q4_file(out_path, shape, np.concatenate([p1, p2]))
+    return Q4FileHeader(shape, h1.original_len + h2.original_len, 36)

@@ -243,6 +243,14 @@ def main():
                             "read_probe_cold_us": round(pcold * 1e3, 3),
                             "read_probe_cold_GB/s": round(wbytes / pcold / 1e6, 1),
                             "gemv_vs_probe": round(pcold / cold, 3)}
+            if name == "lm_head" and B == 1:
+                # the same projection with the exact top-50 selection behind it (fused lm_head + top-k)
+                ftk = lambda i, pool=pool, x=x, n=n, k=k: be.lm_head_topk(x, pool[i % len(pool)], n, k, 50)
+                for i in range(len(pool)):
+                    ftk(i)
+                tk = tm(torch, ftk, reps)
+                shapes[name]["with_top50_us"] = round(tk * 1e3, 3)
+                shapes[name]["with_top50_GB/s"] = round(by / tk / 1e6, 1)
             del pool
         out["gemv_shapes_batch%d" % B] = shapes
 

@@ -44,6 +44,7 @@ enum {
 enum { LQ4_F32 = 0, LQ4_F16 = 1 }; /* element type of activations / LoRA factors */
 
 #define LQ4_MAX_LORA_RANK 64   /* the reference's kernels assume rank <= 64 (qwen35.metal:2302) */
+#define LQ4_MAX_TOP_K 256      /* MAX_TOP_K of the reference's GPU top-k (shaders/qwen35.metal:1686) */
 #define LQ4_MAX_GEMV_BATCH 16  /* lq4_gemv handles 1..16 rows; use lq4_gemm above that          */
 
 typedef struct lq4_ctx lq4_ctx;       /* one per GPU; owns small scratch buffers          */
@@ -152,6 +153,26 @@ int lq4_moe_grouped_gemv(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_weig
                          const float* x_dev, uint32_t tokens, const int32_t* ids_dev,
                          const float* weights_dev, uint32_t top_k, float* y_dev, void* stream);
 
+/* ---- lm_head top-k ------------------------------------------------------------
+ * Exact top-k over `n` f32 logits in the reference's candidate order (higher logit first,
+ * ties to the lower token id, NaN last as the (-inf, 0xFFFFFFFF) sentinel): the result of
+ * logits_topk_first_pass + logits_topk_merge_pass (shaders/qwen35.metal:1683-1778, driven by
+ * dispatch_topk_enc, inner/dispatch.rs:1425-1500).  out_logits_dev / out_ids_dev receive top_k
+ * entries in rank order; slots beyond the number of non-NaN logits hold sentinels.
+ * top_k <= LQ4_MAX_TOP_K. */
+int lq4_topk(lq4_ctx* ctx, const float* logits_dev, uint32_t n, uint32_t top_k, float* out_logits_dev,
+             uint32_t* out_ids_dev, void* stream);
+
+/* Replaces the two-stage lm_head path: lm_head_block_topk_q4 (shaders/qwen35.metal:1935-1985,
+ * dispatch_lm_head_block_stage1_enc, inner/dispatch.rs:1317-1373) followed by
+ * dispatch_block_topk_merge_enc (inner/dispatch.rs:1378-1421).  logits = W[vocab, K] . x (batch-1
+ * GEMV, f32-faithful) are kept in library scratch and never handed to the caller; the top_k
+ * best (logit, token id) pairs come back in rank order.  Both stages are exact, so the result
+ * equals lq4_gemv followed by lq4_topk. */
+int lq4_lm_head_topk(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t vocab, uint32_t k,
+                     const float* x_dev, uint32_t top_k, float* out_logits_dev, uint32_t* out_ids_dev,
+                     void* stream);
+
 /* ---- probes --------------------------------------------------------------------
  * Writes f32(nibble)*scale + bias for every weight of W[N,K] to out_dev (f32 [N,K]):
  * the bit-exactness probe for nibble unpack and scale/bias indexing against
@@ -178,7 +199,7 @@ int lq4_probe_copy(lq4_ctx* ctx, const void* src_dev, void* dst_dev, size_t nbyt
 /* Launch counters per kernel family since context creation (the role of
  * PathProofCounters, metal_qwen35.rs:2144-2190): proves which path served a call. */
 typedef struct lq4_path_counters {
-    uint64_t gemv, gemm, lora_a, moe_route, moe_gate_up, moe_down, dequant;
+    uint64_t gemv, gemm, lora_a, moe_route, moe_gate_up, moe_down, dequant, topk;
 } lq4_path_counters;
 int lq4_get_path_counters(const lq4_ctx* ctx, lq4_path_counters* out);
 

@@ -45,6 +45,8 @@ EXPORTS = [
     "lq4_validate_blocks", "lq4_weight_upload", "lq4_weight_wrap", "lq4_weight_free",
     "lq4_weight_info", "lq4_lora_upload", "lq4_lora_free", "lq4_lora_apply", "lq4_gemv",
     "lq4_gemm", "lq4_moe_route", "lq4_moe_grouped_gemv", "lq4_dequant",
+    "lq4_topk",
+    "lq4_lm_head_topk",
     "lq4_probe_read",
     "lq4_probe_copy",
     "lq4_set_gemm_kernel",
@@ -67,7 +69,7 @@ class Q4Error(RuntimeError):
 
 class PathCounters(C.Structure):
     _fields_ = [(n, C.c_uint64) for n in ("gemv", "gemm", "lora_a", "moe_route", "moe_gate_up",
-                                         "moe_down", "dequant")]
+                                         "moe_down", "dequant", "topk")]
 
 
 _lib = None
@@ -103,6 +105,8 @@ def load_library() -> C.CDLL:
         "lq4_moe_route": (C.c_int, [vp, vp, u32, u32, u32, vp, vp, vp]),
         "lq4_moe_grouped_gemv": (C.c_int, [vp, vp, vp, u32, u32, u32, vp, u32, vp, vp, u32, vp, vp]),
         "lq4_dequant": (C.c_int, [vp, vp, u64, u32, u32, vp, vp]),
+        "lq4_topk": (C.c_int, [vp, vp, C.c_uint32, C.c_uint32, vp, vp, vp]),
+        "lq4_lm_head_topk": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, C.c_uint32, vp, vp, vp]),
         "lq4_probe_read": (C.c_int, [vp, vp, C.c_size_t, vp]),
         "lq4_probe_copy": (C.c_int, [vp, vp, vp, C.c_size_t, vp]),
         "lq4_set_gemm_kernel": (C.c_int, [C.c_int]),
@@ -326,6 +330,29 @@ class HipQ4Backend:
         _check(self.lib.lq4_dequant(self.ctx, qw.handle, qw_extra_offset, n, k, out.data_ptr(),
                                     self._stream()))
         return out
+
+    # ------------------------------------------------------------ lm_head top-k
+    def topk(self, logits, k: int):
+        """Exact top-k of a device logits vector: ``(logits[k], token_ids[k])`` in the reference's
+        rank order (dispatch_topk_enc, inner/dispatch.rs:1425-1500)."""
+        import torch
+        out_l = torch.empty(k, dtype=torch.float32, device=self.torch_device)
+        out_i = torch.empty(k, dtype=torch.int32, device=self.torch_device)  # u32 bit patterns
+        _check(self.lib.lq4_topk(self.ctx, logits.data_ptr(), logits.numel(), k, out_l.data_ptr(),
+                                 out_i.data_ptr(), self._stream()))
+        return out_l, out_i
+
+    def lm_head_topk(self, x, qw: Q4WeightBuf, vocab: int, k: int, top_k: int, qw_extra_offset: int = 0):
+        """lm_head projection fused with top-k selection (dispatch_lm_head_block_stage1_enc +
+        dispatch_block_topk_merge_enc, inner/dispatch.rs:1317-1421): the full logits vector is
+        never returned."""
+        import torch
+        self._assert_k(k, "lm_head_topk")
+        out_l = torch.empty(top_k, dtype=torch.float32, device=self.torch_device)
+        out_i = torch.empty(top_k, dtype=torch.int32, device=self.torch_device)
+        _check(self.lib.lq4_lm_head_topk(self.ctx, qw.handle, qw_extra_offset, vocab, k, x.data_ptr(), top_k,
+                                         out_l.data_ptr(), out_i.data_ptr(), self._stream()))
+        return out_l, out_i
 
     # -------------------------------------------------------------------- LoRA
     def load_lora_adapter(self, layers: List[LoraLayerData], scale: float,

@@ -268,6 +268,8 @@ int lq4_lora_free(lq4_lora* l) {
     return LQ4_OK;
 }
 
+static int ensure_scratch(lq4_ctx* ctx, size_t bytes);
+
 int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
              const float* x_dev, uint32_t batch, float* y_dev, const lq4_lora* lora, float lora_scale,
              void* stream) {
@@ -447,6 +449,50 @@ int lq4_probe_read(lq4_ctx* ctx, const void* p_dev, size_t nbytes, void* stream)
     if (reinterpret_cast<uintptr_t>(p_dev) % 16) return fail(LQ4_E_INVALID, "buffer must be 16-byte aligned");
     DeviceGuard g(ctx->device);
     launch_probe_read(p_dev, nbytes, reinterpret_cast<uint32_t*>(ctx->lora_t), static_cast<hipStream_t>(stream));
+    LQ4_HIP(hipGetLastError());
+    return LQ4_OK;
+}
+
+int lq4_topk(lq4_ctx* ctx, const float* logits_dev, uint32_t n, uint32_t top_k, float* out_logits_dev,
+             uint32_t* out_ids_dev, void* stream) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    if (top_k == 0) return LQ4_OK;
+    if (!logits_dev || !out_logits_dev || !out_ids_dev) return fail(LQ4_E_INVALID, "null device pointer");
+    if (top_k > LQ4_MAX_TOP_K) return fail(LQ4_E_INVALID, "top_k %u above %d", top_k, LQ4_MAX_TOP_K);
+    if (n == 0) return fail(LQ4_E_INVALID, "no logits to select from");
+    DeviceGuard g(ctx->device);
+    const int rc = ensure_scratch(ctx, topk_scratch_bytes(n, top_k));
+    if (rc) return rc;
+    launch_topk(logits_dev, n, top_k, ctx->moe_scratch, out_logits_dev, out_ids_dev, static_cast<hipStream_t>(stream));
+    ctx->counters.topk++;
+    LQ4_HIP(hipGetLastError());
+    return LQ4_OK;
+}
+
+int lq4_lm_head_topk(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t vocab, uint32_t k,
+                     const float* x_dev, uint32_t top_k, float* out_logits_dev, uint32_t* out_ids_dev,
+                     void* stream) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    if (top_k == 0) return LQ4_OK;
+    if (vocab == 0) return fail(LQ4_E_INVALID, "empty vocabulary");
+    if (top_k > LQ4_MAX_TOP_K) return fail(LQ4_E_INVALID, "top_k %u above %d", top_k, LQ4_MAX_TOP_K);
+    const uint8_t* wp;
+    int rc = resolve_weight(w, w_extra_offset, vocab, k, &wp);
+    if (rc) return rc;
+    if (!x_dev || !out_logits_dev || !out_ids_dev) return fail(LQ4_E_INVALID, "null device pointer");
+    if (reinterpret_cast<uintptr_t>(x_dev) % 16) return fail(LQ4_E_INVALID, "x must be 16-byte aligned");
+    DeviceGuard g(ctx->device);
+    // scratch: [vocab logits | candidate buffers]
+    const size_t logits_bytes = (static_cast<size_t>(vocab) * sizeof(float) + 255) / 256 * 256;
+    rc = ensure_scratch(ctx, logits_bytes + topk_scratch_bytes(vocab, top_k));
+    if (rc) return rc;
+    float* logits = reinterpret_cast<float*>(ctx->moe_scratch);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};
+    launch_gemv(wp, vocab, k, x_dev, k, 1, logits, vocab, none, s);
+    launch_topk(logits, vocab, top_k, ctx->moe_scratch + logits_bytes, out_logits_dev, out_ids_dev, s);
+    ctx->counters.gemv++;
+    ctx->counters.topk++;
     LQ4_HIP(hipGetLastError());
     return LQ4_OK;
 }

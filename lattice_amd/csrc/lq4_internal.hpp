@@ -103,6 +103,12 @@ void launch_moe_down_mfma(const uint8_t* down, uint32_t num_experts, uint32_t in
                           const float* h, uint32_t tokens, const int32_t* offsets, const int32_t* order, float* o,
                           hipStream_t stream);
 
+// Exact top-k over n logits (k <= 256): out_logits / out_ids receive the k best in rank order.
+// `scratch` must hold topk_scratch_bytes(n, k) bytes.
+size_t topk_scratch_bytes(uint32_t n, uint32_t k);
+void launch_topk(const float* logits, uint32_t n, uint32_t k, void* scratch, float* out_logits, uint32_t* out_ids,
+                 hipStream_t stream);
+
 // ---- device helpers ---------------------------------------------------------------
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t bits16) {
     // v_cvt_f32_f16 widens exactly, subnormals included (f16 denormals are not flushed

@@ -88,6 +88,8 @@ def lib() -> C.CDLL:
         fn.restype = C.c_int
         fn.argtypes = [_u8p, _u8p, C.c_int, C.c_int, C.c_int, _f32p, C.c_int, _i32p, _f32p,
                        C.c_int, outp]
+    L.lq4o_topk.restype = None
+    L.lq4o_topk.argtypes = [_f32p, C.c_uint32, C.c_uint32, _f32p, C.POINTER(C.c_uint32)]
     L.lq4o_parse_q4_file.restype = C.c_int
     L.lq4o_parse_q4_file.argtypes = [_u8p, C.c_size_t, _u64p, C.c_int, C.POINTER(C.c_int), _u64p,
                                      _u64p]
@@ -312,6 +314,16 @@ Q4_FILE_ERRORS = {1: "invalid magic: not a .q4 file", 2: "legacy .q4 file (v1)",
                   5: "file truncated below Q4 block payload",
                   6: "file has trailing bytes after Q4 block payload",
                   7: "original_len does not match shape"}
+
+
+def topk(logits, k: int):
+    """(logits[k], ids[k]) of the k best entries in the reference's top-k order (higher logit
+    first, ties to the lower id, NaN last as the (-inf, 0xFFFFFFFF) sentinel)."""
+    lg = _f32(logits).reshape(-1)
+    out_l = np.empty(k, dtype=np.float32)
+    out_i = np.empty(k, dtype=np.uint32)
+    lib().lq4o_topk(_p(lg, _f32p), lg.size, k, _p(out_l, _f32p), _p(out_i, C.POINTER(C.c_uint32)))
+    return out_l, out_i
 
 
 def parse_q4_file(data):

@@ -564,3 +564,43 @@ int lq4o_parse_q4_file(const uint8_t* file, size_t file_len, uint64_t* shape, in
     *payload_offset = off;
     return 0;
 }
+
+/* ---- lm_head top-k selection ----------------------------------------------------
+ * The ordering of the reference's GPU top-k (shaders/qwen35.metal:1688-1703):
+ * candidate = (logit, token_id); a ranks before b if it has the higher logit, ties go
+ * to the lower token id; a NaN logit becomes the sentinel (-inf, UINT32_MAX) before it
+ * enters the selection (qwen35.metal:1916, 1966) and so ranks last.  The two-stage
+ * tile/merge scheme is exact by construction (qwen35.metal:1868-1892), so its result is
+ * the first k entries of the fully sorted candidate list, which is what this computes.
+ * Slots beyond the number of logits hold sentinels. */
+static int lq4o_topk_better(float al, uint32_t ai, float bl, uint32_t bi) {
+    if (al != al) return 0;
+    if (bl != bl) return 1;
+    if (al != bl) return al > bl;
+    return ai < bi;
+}
+
+void lq4o_topk(const float* logits, uint32_t n, uint32_t k, float* out_logits, uint32_t* out_ids) {
+    for (uint32_t r = 0; r < k; ++r) {
+        out_logits[r] = -INFINITY;
+        out_ids[r] = UINT32_MAX;
+    }
+    for (uint32_t i = 0; i < n; ++i) {
+        float l = logits[i];
+        uint32_t id = i;
+        if (l != l) {
+            l = -INFINITY;
+            id = UINT32_MAX;
+        }
+        /* insertion into the sorted list of the best k so far */
+        if (k == 0 || !lq4o_topk_better(l, id, out_logits[k - 1], out_ids[k - 1])) continue;
+        uint32_t pos = k - 1;
+        while (pos > 0 && lq4o_topk_better(l, id, out_logits[pos - 1], out_ids[pos - 1])) {
+            out_logits[pos] = out_logits[pos - 1];
+            out_ids[pos] = out_ids[pos - 1];
+            --pos;
+        }
+        out_logits[pos] = l;
+        out_ids[pos] = id;
+    }
+}

@@ -1,0 +1,108 @@
+"""lm_head top-k: the reference's candidate order and its two-stage exact selection
+(shaders/qwen35.metal:1683-1778, 1868-1985).  The oracle is pinned by brute force (numpy
+lexsort on small inputs) and by hand cases; the GPU kernels are checked bit for bit against it,
+including the adversarial distributions the reference names: all winners clustered in one tile,
+ties, NaN and infinities."""
+import numpy as np
+import pytest
+
+import oracle
+from lattice_amd import synth
+from util import REL_TOL
+
+
+def _brute(logits, k):
+    lg = np.asarray(logits, np.float32).copy()
+    ids = np.arange(lg.size, dtype=np.uint32)
+    nan = np.isnan(lg)
+    lg[nan] = -np.inf
+    ids[nan] = 0xFFFFFFFF
+    order = np.lexsort((ids, -lg.astype(np.float64)))  # primary: logit descending; secondary: id ascending
+    out_l = np.full(k, -np.inf, np.float32)
+    out_i = np.full(k, 0xFFFFFFFF, np.uint32)
+    m = min(k, lg.size)
+    out_l[:m], out_i[:m] = lg[order[:m]], ids[order[:m]]
+    return out_l, out_i
+
+
+def test_oracle_hand_cases():
+    l, i = oracle.topk(np.array([1, 5, np.nan, 5, -np.inf, 3], np.float32), 4)
+    assert l.tolist() == [5, 5, 3, 1] and i.tolist() == [1, 3, 5, 0]  # tie -> lower id first
+    l, i = oracle.topk(np.array([np.nan, np.nan], np.float32), 3)
+    assert np.all(np.isneginf(l)) and i.tolist() == [0xFFFFFFFF] * 3  # NaN never wins a slot
+    l, i = oracle.topk(np.array([-np.inf, np.nan, -np.inf], np.float32), 3)
+    assert i.tolist() == [0, 2, 0xFFFFFFFF]  # a real -inf still ranks before the sentinel
+    l, i = oracle.topk(np.array([2.0, 7.0], np.float32), 1)
+    assert l.tolist() == [7.0] and i.tolist() == [1]
+
+
+@pytest.mark.parametrize("n,k,seed", [(7, 3, 0), (1000, 50, 1), (5000, 256, 2), (300, 300 // 2, 3)])
+def test_oracle_matches_brute_force(n, k, seed):
+    g = np.random.default_rng(seed)
+    lg = g.normal(size=n).astype(np.float32)
+    lg[g.integers(0, n, n // 10)] = lg[0]          # plenty of exact ties
+    lg[g.integers(0, n, max(1, n // 50))] = np.nan
+    want = _brute(lg, k)
+    got = oracle.topk(lg, k)
+    assert np.array_equal(got[1], want[1]) and np.array_equal(got[0], want[0])
+
+
+def _cases():
+    g = np.random.default_rng(7)
+    n = 248320
+    base = g.normal(size=n).astype(np.float32)
+    clustered = base.copy()
+    clustered[5 * 1024 + 3: 5 * 1024 + 3 + 200] = 50.0 + np.arange(200, dtype=np.float32)  # one tile holds all winners
+    ties = np.zeros(n, np.float32)
+    ties[::7] = 1.0
+    nans = base.copy()
+    nans[::3] = np.nan
+    nans[10] = np.inf
+    nans[11] = -np.inf
+    return {"random": base, "clustered": clustered, "ties": ties, "nan_inf": nans,
+            "short": base[:777], "one_tile_exact": base[:1024], "all_nan": np.full(2000, np.nan, np.float32)}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("k", [1, 8, 50, 64, 256])
+def test_gpu_topk_is_exact(k):
+    import torch
+    from lattice_amd import backend
+    be = backend.HipQ4Backend(0)
+    for name, lg in _cases().items():
+        print(f"topk {name} n={lg.size} k={k}", flush=True)
+        out_l, out_i = be.topk(torch.from_numpy(lg).cuda(), k)
+        want_l, want_i = oracle.topk(lg, k)
+        got_i = out_i.cpu().numpy().view(np.uint32)
+        got_l = out_l.cpu().numpy()
+        assert np.array_equal(got_i, want_i), name
+        assert np.array_equal(got_l.view(np.uint32), want_l.view(np.uint32)), name
+
+
+@pytest.mark.gpu
+def test_gpu_lm_head_topk_matches_gemv_then_topk():
+    import torch
+    from lattice_amd import backend
+    be = backend.HipQ4Backend(0)
+    vocab, k, top_k = 5000, 256, 40
+    wq = synth.q4_weight(vocab, k, seed=11)
+    x = synth.activations(1, k, seed=11)
+    qw = be.upload_q4_blocks(wq)
+    xd = torch.from_numpy(x).cuda()
+    out_l, out_i = be.lm_head_topk(xd, qw, vocab, k, top_k)
+    # same library, two calls: logits from the GEMV, selection on them -> must agree bit for bit
+    y = torch.empty((1, vocab), dtype=torch.float32, device="cuda")
+    be.dispatch_matmul(xd, qw, y, 1, vocab, k)
+    ref_l, ref_i = oracle.topk(y.cpu().numpy().reshape(-1), top_k)
+    assert np.array_equal(out_i.cpu().numpy().view(np.uint32), ref_i)
+    assert np.array_equal(out_l.cpu().numpy().view(np.uint32), ref_l.view(np.uint32))
+    # against the CPU oracle's own logits: same winners wherever the gap to the next candidate
+    # exceeds the GEMV tolerance (the reference's tie epsilon, metal_qwen35.rs:37365-37427)
+    logits = oracle.gemm_f32(x, wq, vocab, k).reshape(-1)
+    o_l, o_i = oracle.topk(logits, top_k + 1)
+    eps = REL_TOL * np.abs(logits).max()
+    got = out_i.cpu().numpy().view(np.uint32)
+    for r in range(top_k):
+        if o_l[r] - o_l[r + 1] > eps and (r == 0 or o_l[r - 1] - o_l[r] > eps):
+            assert got[r] == o_i[r], r
+    assert np.abs(out_l.cpu().numpy() - o_l[:top_k]).max() <= eps

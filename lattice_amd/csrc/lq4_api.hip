@@ -64,6 +64,9 @@ struct DeviceGuard {
     explicit DeviceGuard(int dev) {
         if (hipGetDevice(&prev) != hipSuccess) prev = -1;
         if (prev != dev) ok = hipSetDevice(dev) == hipSuccess;
+        // An error some earlier, unrelated runtime call left behind in this thread must not be
+        // reported by the launch check of this entry point.
+        if (ok) (void)hipGetLastError();
     }
     ~DeviceGuard() {
         if (prev >= 0) (void)hipSetDevice(prev);

@@ -373,22 +373,70 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
     }
 }
 
-// y[i] = sum over slices, in slice order, of partial[s][i]  (count multiple of 4 or not)
+// y[i] = sum over slices, in slice order, of partial[s][i]  (count multiple of 4 or not), plus the
+// LoRA delta scale * sum_j B[row, j] * t[token, j] in f32 when lora.rank != 0 (i = token * n + row).
 __global__ __launch_bounds__(256) void gemm_reduce_slices(const float* __restrict__ partial, uint32_t slices,
-                                                          size_t count, float* __restrict__ y) {
+                                                          size_t count, float* __restrict__ y, uint32_t n,
+                                                          LoraEpilogue lora) {
     const size_t i4 = (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
     if (i4 >= count) return;
+    auto delta = [&](size_t i) {
+        const size_t token = i / n, row = i - token * n;
+        const float* t = lora.t + token * lora.rank;
+        float d = 0.0f;
+        for (uint32_t j = 0; j < lora.rank; ++j) d = fmaf(load_b(lora.b, lora.b_is_f16, row * lora.rank + j), t[j], d);
+        return lora.scale * d;
+    };
     if (i4 + 4 <= count && (count & 3) == 0) {
         float4v v = *reinterpret_cast<const float4v*>(partial + i4);
         for (uint32_t sl = 1; sl < slices; ++sl) v += *reinterpret_cast<const float4v*>(partial + sl * count + i4);
+        if (lora.rank) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] += delta(i4 + e);
+        }
         *reinterpret_cast<float4v*>(y + i4) = v;
     } else {
         for (size_t i = i4; i < count && i < i4 + 4; ++i) {
             float v = partial[i];
             for (uint32_t sl = 1; sl < slices; ++sl) v += partial[sl * count + i];
+            if (lora.rank) v += delta(i);
             y[i] = v;
         }
     }
+}
+
+// Same with the LoRA delta for n % 4 == 0 and rank % 4 == 0: grid (ceil(n / 1024), m); a thread owns
+// four consecutive weight rows of one token, so t[token, :] is a broadcast load and the B rows are
+// read with vector loads.
+__global__ __launch_bounds__(256) void gemm_reduce_slices_lora(const float* __restrict__ partial, uint32_t slices,
+                                                               uint32_t m, uint32_t n, float* __restrict__ y,
+                                                               LoraEpilogue lora) {
+    typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+    const uint32_t row = (blockIdx.x * 256 + threadIdx.x) * 4;
+    const uint32_t token = blockIdx.y;
+    if (row >= n) return;
+    const size_t at = static_cast<size_t>(token) * n + row, count = static_cast<size_t>(m) * n;
+    float4v v = *reinterpret_cast<const float4v*>(partial + at);
+    for (uint32_t sl = 1; sl < slices; ++sl) v += *reinterpret_cast<const float4v*>(partial + sl * count + at);
+    const float* t = lora.t + static_cast<size_t>(token) * lora.rank;
+    float4v d = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (uint32_t j = 0; j < lora.rank; j += 4) {
+        const float4v tv = *reinterpret_cast<const float4v*>(t + j);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const size_t bi = static_cast<size_t>(row + e) * lora.rank + j;
+            float4v bv;
+            if (lora.b_is_f16) {
+                const half4v h = *reinterpret_cast<const half4v*>(static_cast<const _Float16*>(lora.b) + bi);
+                bv = float4v{static_cast<float>(h[0]), static_cast<float>(h[1]), static_cast<float>(h[2]),
+                             static_cast<float>(h[3])};
+            } else {
+                bv = *reinterpret_cast<const float4v*>(static_cast<const float*>(lora.b) + bi);
+            }
+            d[e] = fmaf(bv[3], tv[3], fmaf(bv[2], tv[2], fmaf(bv[1], tv[1], fmaf(bv[0], tv[0], d[e]))));
+        }
+    }
+    *reinterpret_cast<float4v*>(y + at) = v + lora.scale * d;
 }
 
 }  // namespace
@@ -434,7 +482,8 @@ void launch_gemm_wreg(const uint8_t* w, uint32_t n, uint32_t k, const void* x, i
                       float* y, const LoraEpilogue& lora, uint32_t slices, float* partial, hipStream_t stream) {
     if (slices <= 1 || !partial) slices = 1;
     float* out = slices > 1 ? partial : y;
-    if (lora.rank) {
+    // K-sliced: the delta is added in f32 by the pass that sums the slices
+    if (lora.rank && slices == 1) {
         if (x_is_f16) launch_wreg_t<true, true>(w, n, k, x, m, out, lora, slices, stream);
         else launch_wreg_t<false, true>(w, n, k, x, m, out, lora, slices, stream);
     } else {
@@ -443,8 +492,12 @@ void launch_gemm_wreg(const uint8_t* w, uint32_t n, uint32_t k, const void* x, i
     }
     if (slices > 1) {
         const size_t count = static_cast<size_t>(m) * n;
-        hipLaunchKernelGGL(gemm_reduce_slices, dim3(static_cast<uint32_t>((count + 1023) / 1024)), dim3(256), 0,
-                           stream, partial, slices, count, y);
+        if (lora.rank && n % 4 == 0 && lora.rank % 4 == 0)
+            hipLaunchKernelGGL(gemm_reduce_slices_lora, dim3((n + 1023) / 1024, m), dim3(256), 0, stream, partial,
+                               slices, m, n, y, lora);
+        else
+            hipLaunchKernelGGL(gemm_reduce_slices, dim3(static_cast<uint32_t>((count + 1023) / 1024)), dim3(256), 0,
+                               stream, partial, slices, count, y, n, lora);
     }
 }
 

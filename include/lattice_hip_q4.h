@@ -173,6 +173,57 @@ int lq4_lm_head_topk(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset,
                      const float* x_dev, uint32_t top_k, float* out_logits_dev, uint32_t* out_ids_dev,
                      void* stream);
 
+/* ---- elementwise steps either side of the decode GEMVs ---------------------------
+ * Shifted RMSNorm of Qwen3.5 with the residual add in front of it: v = base + delta (delta may be
+ * NULL: plain norm), residual_out = v (skipped if NULL), normed_out = v * rsqrt(mean(v^2) + eps) *
+ * (1 + gamma).  Replaces dispatch_fused_residual_add_norm / _batch (inner/dispatch.rs:1171-1266,
+ * shaders/qwen35.metal:739-767, 2219-2249) and dispatch_rms_norm (inner/dispatch.rs:525; CPU form
+ * qwen35_rms_norm, model/qwen35/norm.rs:6-23).  `rows` rows of `hidden` floats. */
+int lq4_residual_add_rmsnorm(lq4_ctx* ctx, const float* base_dev, const float* delta_dev, const float* gamma_dev,
+                             uint32_t hidden, uint32_t rows, float eps, float* residual_out_dev,
+                             float* normed_out_dev, void* stream);
+
+/* out[r, i] = silu(gate_up[r, i]) * gate_up[r, count + i] for rows of [gate(count) | up(count)];
+ * out rows are out_stride floats apart (out == gate_up with out_stride == 2 * count is the
+ * in-place form of silu_mul_fused, shaders/qwen35.metal:712-722, dispatch_silu_mul_fused
+ * inner/dispatch.rs:916-930). */
+int lq4_silu_mul(lq4_ctx* ctx, const float* gate_up_dev, uint32_t count, uint32_t rows, float* out_dev,
+                 uint32_t out_stride, void* stream);
+
+/* residual += src; dst = residual (dst may be NULL).  Replaces dispatch_add_and_copy
+ * (inner/dispatch.rs:1268-1290, shaders/qwen35.metal:2255-2266). */
+int lq4_add_and_copy(lq4_ctx* ctx, const float* src_dev, float* residual_dev, float* dst_dev, size_t count,
+                     void* stream);
+
+/* The same steps fused into the batch-1 GEMV, so that a decode MLP is two launches
+ * (norm + gate||up GEMV, then silu*up + down GEMV + residual add) instead of five. */
+#define LQ4_PRO_NONE 0        /* activations = x_dev[K] */
+#define LQ4_PRO_ADD_RMSNORM 1 /* activations = shifted RMSNorm(base + delta); x_dev is ignored */
+#define LQ4_PRO_SILU_MUL 2    /* activations = silu(x_dev[0..K)) * x_dev[K..2K) */
+#define LQ4_EPI_NONE 0        /* y_dev[N] = W . activations (+ LoRA) */
+#define LQ4_EPI_ADD_RESIDUAL 1 /* also residual[N] += that; copy_dst[N] = residual (if not NULL);
+                                  y_dev may then be NULL */
+typedef struct lq4_gemv_fusion {
+    int prologue;
+    const float* base;   /* ADD_RMSNORM: [K] */
+    const float* delta;  /* ADD_RMSNORM: [K] or NULL */
+    const float* gamma;  /* ADD_RMSNORM: [K] */
+    float eps;
+    float* residual_out; /* ADD_RMSNORM: [K] or NULL; must not overlap base or delta */
+    int epilogue;
+    float* residual;     /* ADD_RESIDUAL: [N], updated in place */
+    float* copy_dst;     /* ADD_RESIDUAL: [N] or NULL */
+} lq4_gemv_fusion;
+
+/* lq4_gemv at batch 1 with the elementwise steps above applied while the activations are staged
+ * and while the result is stored.  Equals the unfused sequence lq4_residual_add_rmsnorm /
+ * lq4_silu_mul -> lq4_gemv -> lq4_add_and_copy to f32 rounding (the sum of squares is formed in a
+ * different order).  Shapes or options the fused kernel does not take (K too long for LDS, a LoRA
+ * adapter together with a prologue) run as exactly that sequence through library scratch. */
+int lq4_gemv_fused(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
+                   const float* x_dev, float* y_dev, const lq4_gemv_fusion* fusion, const lq4_lora* lora,
+                   float lora_scale, void* stream);
+
 /* ---- probes --------------------------------------------------------------------
  * Writes f32(nibble)*scale + bias for every weight of W[N,K] to out_dev (f32 [N,K]):
  * the bit-exactness probe for nibble unpack and scale/bias indexing against
@@ -199,7 +250,7 @@ int lq4_probe_copy(lq4_ctx* ctx, const void* src_dev, void* dst_dev, size_t nbyt
 /* Launch counters per kernel family since context creation (the role of
  * PathProofCounters, metal_qwen35.rs:2144-2190): proves which path served a call. */
 typedef struct lq4_path_counters {
-    uint64_t gemv, gemm, lora_a, moe_route, moe_gate_up, moe_down, dequant, topk;
+    uint64_t gemv, gemm, lora_a, moe_route, moe_gate_up, moe_down, dequant, topk, gemv_fused, elementwise;
 } lq4_path_counters;
 int lq4_get_path_counters(const lq4_ctx* ctx, lq4_path_counters* out);
 

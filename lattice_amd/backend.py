@@ -50,6 +50,7 @@ EXPORTS = [
     "lq4_probe_read",
     "lq4_probe_copy",
     "lq4_set_gemm_kernel",
+    "lq4_residual_add_rmsnorm", "lq4_silu_mul", "lq4_add_and_copy", "lq4_gemv_fused",
     "lq4_get_path_counters", "lq4_malloc", "lq4_free", "lq4_memcpy_h2d", "lq4_memcpy_d2h",
 ]
 
@@ -69,7 +70,18 @@ class Q4Error(RuntimeError):
 
 class PathCounters(C.Structure):
     _fields_ = [(n, C.c_uint64) for n in ("gemv", "gemm", "lora_a", "moe_route", "moe_gate_up",
-                                         "moe_down", "dequant", "topk")]
+                                         "moe_down", "dequant", "topk", "gemv_fused", "elementwise")]
+
+
+LQ4_PRO_NONE, LQ4_PRO_ADD_RMSNORM, LQ4_PRO_SILU_MUL = 0, 1, 2
+LQ4_EPI_NONE, LQ4_EPI_ADD_RESIDUAL = 0, 1
+
+
+class GemvFusion(C.Structure):
+    """``lq4_gemv_fusion``: elementwise steps fused into the batch-1 GEMV."""
+    _fields_ = [("prologue", C.c_int), ("base", C.c_void_p), ("delta", C.c_void_p), ("gamma", C.c_void_p),
+                ("eps", C.c_float), ("residual_out", C.c_void_p), ("epilogue", C.c_int),
+                ("residual", C.c_void_p), ("copy_dst", C.c_void_p)]
 
 
 _lib = None
@@ -110,6 +122,11 @@ def load_library() -> C.CDLL:
         "lq4_probe_read": (C.c_int, [vp, vp, C.c_size_t, vp]),
         "lq4_probe_copy": (C.c_int, [vp, vp, vp, C.c_size_t, vp]),
         "lq4_set_gemm_kernel": (C.c_int, [C.c_int]),
+        "lq4_residual_add_rmsnorm": (C.c_int, [vp, vp, vp, vp, C.c_uint32, C.c_uint32, C.c_float, vp, vp, vp]),
+        "lq4_silu_mul": (C.c_int, [vp, vp, C.c_uint32, C.c_uint32, vp, C.c_uint32, vp]),
+        "lq4_add_and_copy": (C.c_int, [vp, vp, vp, vp, C.c_size_t, vp]),
+        "lq4_gemv_fused": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, vp, C.POINTER(GemvFusion), vp,
+                                     C.c_float, vp]),
         "lq4_get_path_counters": (C.c_int, [vp, C.POINTER(PathCounters)]),
         "lq4_malloc": (C.c_int, [vp, C.c_size_t, C.POINTER(vp)]),
         "lq4_free": (C.c_int, [vp, vp]),
@@ -292,6 +309,59 @@ class HipQ4Backend:
         lora = self._lora_for(layer_idx, module, n, k)
         _check(self.lib.lq4_gemv(self.ctx, qw.handle, 0, n, k, x.data_ptr(), 1, y.data_ptr(), lora,
                                  self._lora_scale, self._stream()))
+
+    # ---- elementwise steps either side of the decode GEMVs -----------------------------------
+    @staticmethod
+    def _ptr(t):
+        return None if t is None else t.data_ptr()
+
+    def dispatch_fused_residual_add_norm(self, base, delta, residual_out, normed_out, gamma, row_len: int,
+                                         eps: float, num_rows: int = 1):
+        """``dispatch_fused_residual_add_norm`` / ``_batch`` (dispatch.rs:1171-1266):
+        ``residual_out = base + delta``, ``normed_out`` = shifted RMSNorm of it.  ``delta=None`` is
+        the plain ``dispatch_rms_norm`` (dispatch.rs:525); ``residual_out=None`` skips that store."""
+        _check(self.lib.lq4_residual_add_rmsnorm(self.ctx, base.data_ptr(), self._ptr(delta), gamma.data_ptr(),
+                                                 row_len, num_rows, eps, self._ptr(residual_out),
+                                                 normed_out.data_ptr(), self._stream()))
+
+    def dispatch_silu_mul_fused(self, data, count: int, rows: int = 1, out=None, out_stride=None):
+        """``dispatch_silu_mul_fused`` (dispatch.rs:916-930): ``data[i] = silu(data[i]) *
+        data[i + count]`` in place, or into ``out`` (rows ``out_stride`` floats apart)."""
+        dst = data if out is None else out
+        stride = (2 * count if out is None else count) if out_stride is None else out_stride
+        _check(self.lib.lq4_silu_mul(self.ctx, data.data_ptr(), count, rows, dst.data_ptr(), stride, self._stream()))
+
+    def dispatch_add_and_copy(self, src, residual, dst, count: int):
+        """``dispatch_add_and_copy`` (dispatch.rs:1268-1290): ``residual += src; dst = residual``."""
+        _check(self.lib.lq4_add_and_copy(self.ctx, src.data_ptr(), residual.data_ptr(), self._ptr(dst), count,
+                                         self._stream()))
+
+    def dispatch_matmul_fused(self, x, qw: Q4WeightBuf, y, n: int, k: int, *, norm=None, silu_mul=False,
+                              add_residual=None, qw_extra_offset: int = 0, layer_idx=None, module=None):
+        """Batch-1 ``dispatch_matmul`` with the neighbouring elementwise dispatches folded in.
+        ``norm=(base, delta, gamma, eps, residual_out)`` replaces a preceding
+        ``dispatch_fused_residual_add_norm`` (``x`` is then unused); ``silu_mul=True`` replaces a
+        preceding ``dispatch_silu_mul_fused`` (``x`` holds gate | up, 2k floats);
+        ``add_residual=(residual, dst)`` replaces a following ``dispatch_add_and_copy``."""
+        if n == 0:
+            return
+        self._assert_k(k, "dispatch_matmul_q4")
+        assert not (norm is not None and silu_mul), "one prologue at a time"
+        f = GemvFusion()
+        f.prologue = LQ4_PRO_ADD_RMSNORM if norm is not None else LQ4_PRO_SILU_MUL if silu_mul else LQ4_PRO_NONE
+        keep = []
+        if norm is not None:
+            base, delta, gamma, eps, residual_out = norm
+            f.base, f.delta, f.gamma = base.data_ptr(), self._ptr(delta), gamma.data_ptr()
+            f.eps, f.residual_out = eps, self._ptr(residual_out)
+            keep += [base, delta, gamma, residual_out]
+        f.epilogue = LQ4_EPI_NONE
+        if add_residual is not None:
+            residual, dst = add_residual
+            f.epilogue, f.residual, f.copy_dst = LQ4_EPI_ADD_RESIDUAL, residual.data_ptr(), self._ptr(dst)
+        lora = self._lora_for(layer_idx, module, n, k)
+        _check(self.lib.lq4_gemv_fused(self.ctx, qw.handle, qw_extra_offset, n, k, self._ptr(x), self._ptr(y),
+                                       C.byref(f), lora, self._lora_scale, self._stream()))
 
     def dispatch_gemm(self, x, x_offset: int, qw: Q4WeightBuf, y, y_offset: int, m: int, n: int,
                       k: int, *, layer_idx=None, module=None):

@@ -500,6 +500,150 @@ int lq4_lm_head_topk(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset,
     return LQ4_OK;
 }
 
+int lq4_residual_add_rmsnorm(lq4_ctx* ctx, const float* base_dev, const float* delta_dev, const float* gamma_dev,
+                             uint32_t hidden, uint32_t rows, float eps, float* residual_out_dev,
+                             float* normed_out_dev, void* stream) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    if (rows == 0 || hidden == 0) return LQ4_OK;
+    if (!base_dev || !gamma_dev || !normed_out_dev) return fail(LQ4_E_INVALID, "base, gamma or normed_out is null");
+    DeviceGuard g(ctx->device);
+    launch_residual_add_norm(base_dev, delta_dev, gamma_dev, hidden, rows, eps, residual_out_dev, normed_out_dev,
+                             static_cast<hipStream_t>(stream));
+    ctx->counters.elementwise++;
+    LQ4_HIP(hipGetLastError());
+    return LQ4_OK;
+}
+
+int lq4_silu_mul(lq4_ctx* ctx, const float* gate_up_dev, uint32_t count, uint32_t rows, float* out_dev,
+                 uint32_t out_stride, void* stream) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    if (rows == 0 || count == 0) return LQ4_OK;
+    if (!gate_up_dev || !out_dev) return fail(LQ4_E_INVALID, "gate_up or out is null");
+    if (out_stride < count) return fail(LQ4_E_INVALID, "out_stride %u below count %u", out_stride, count);
+    if (rows > 65535) return fail(LQ4_E_UNSUPPORTED, "silu_mul limited to 65535 rows, got %u", rows);
+    DeviceGuard g(ctx->device);
+    launch_silu_mul(gate_up_dev, count, rows, out_dev, out_stride, static_cast<hipStream_t>(stream));
+    ctx->counters.elementwise++;
+    LQ4_HIP(hipGetLastError());
+    return LQ4_OK;
+}
+
+int lq4_add_and_copy(lq4_ctx* ctx, const float* src_dev, float* residual_dev, float* dst_dev, size_t count,
+                     void* stream) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    if (count == 0) return LQ4_OK;
+    if (!src_dev || !residual_dev) return fail(LQ4_E_INVALID, "src or residual is null");
+    DeviceGuard g(ctx->device);
+    launch_add_and_copy(src_dev, residual_dev, dst_dev, count, static_cast<hipStream_t>(stream));
+    ctx->counters.elementwise++;
+    LQ4_HIP(hipGetLastError());
+    return LQ4_OK;
+}
+
+static bool ranges_overlap(const void* a, const void* b, size_t bytes) {
+    const uintptr_t pa = reinterpret_cast<uintptr_t>(a), pb = reinterpret_cast<uintptr_t>(b);
+    return pa < pb + bytes && pb < pa + bytes;
+}
+
+int lq4_gemv_fused(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
+                   const float* x_dev, float* y_dev, const lq4_gemv_fusion* fusion, const lq4_lora* lora,
+                   float lora_scale, void* stream) {
+    if (!fusion || (fusion->prologue == LQ4_PRO_NONE && fusion->epilogue == LQ4_EPI_NONE))
+        return lq4_gemv(ctx, w, w_extra_offset, n, k, x_dev, 1, y_dev, lora, lora_scale, stream);
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    if (n == 0) return LQ4_OK;
+    const uint8_t* wp;
+    int rc = resolve_weight(w, w_extra_offset, n, k, &wp);
+    if (rc) return rc;
+    const lq4_gemv_fusion& f = *fusion;
+    const size_t kbytes = static_cast<size_t>(k) * sizeof(float);
+    auto misaligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 != 0; };
+    switch (f.prologue) {
+        case LQ4_PRO_NONE:
+        case LQ4_PRO_SILU_MUL:
+            if (!x_dev) return fail(LQ4_E_INVALID, "x device pointer is null");
+            if (misaligned(x_dev)) return fail(LQ4_E_INVALID, "x must be 16-byte aligned");
+            break;
+        case LQ4_PRO_ADD_RMSNORM:
+            if (!f.base || !f.gamma) return fail(LQ4_E_INVALID, "fusion.base or fusion.gamma is null");
+            if (misaligned(f.base) || misaligned(f.gamma) || (f.delta && misaligned(f.delta)) ||
+                (f.residual_out && misaligned(f.residual_out)))
+                return fail(LQ4_E_INVALID, "fusion.base, delta, gamma and residual_out must be 16-byte aligned");
+            if (f.residual_out && (ranges_overlap(f.residual_out, f.base, kbytes) ||
+                                   (f.delta && ranges_overlap(f.residual_out, f.delta, kbytes))))
+                return fail(LQ4_E_INVALID, "fusion.residual_out must not overlap fusion.base or fusion.delta");
+            break;
+        default:
+            return fail(LQ4_E_INVALID, "unknown fusion.prologue %d", f.prologue);
+    }
+    if (f.epilogue == LQ4_EPI_ADD_RESIDUAL) {
+        if (!f.residual) return fail(LQ4_E_INVALID, "fusion.residual is null");
+        if (reinterpret_cast<uintptr_t>(f.residual) % 4 || reinterpret_cast<uintptr_t>(f.copy_dst) % 4)
+            return fail(LQ4_E_INVALID, "fusion.residual and copy_dst must be 4-byte aligned");
+    } else if (f.epilogue == LQ4_EPI_NONE) {
+        if (!y_dev) return fail(LQ4_E_INVALID, "y device pointer is null");
+    } else {
+        return fail(LQ4_E_INVALID, "unknown fusion.epilogue %d", f.epilogue);
+    }
+    if (y_dev && reinterpret_cast<uintptr_t>(y_dev) % 4) return fail(LQ4_E_INVALID, "y must be 4-byte aligned");
+    LoraEpilogue ep;
+    rc = resolve_lora(ctx, lora, lora_scale, n, k, 1, &ep);
+    if (rc) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    DeviceGuard g(ctx->device);
+
+    const bool fused_ok = gemv_b1_lds_bytes(k) <= 128 * 1024 && !(ep.rank && f.prologue != LQ4_PRO_NONE);
+    if (fused_ok) {
+        if (ep.rank) {
+            launch_lora_a(lora->a, lora->is_f16, lora->rank, k, x_dev, 0, k, 1, ctx->lora_t, s);
+            ctx->counters.lora_a++;
+        }
+        GemvFusion gf;
+        gf.prologue = f.prologue;
+        gf.base = f.base;
+        gf.delta = f.delta;
+        gf.gamma = f.gamma;
+        gf.eps = f.eps;
+        gf.residual_out = f.residual_out;
+        gf.epilogue = f.epilogue;
+        gf.residual = f.residual;
+        gf.copy_dst = f.copy_dst;
+        launch_gemv_b1_fused(wp, n, k, x_dev, y_dev, ep, gf, s);
+        ctx->counters.gemv_fused++;
+        LQ4_HIP(hipGetLastError());
+        return LQ4_OK;
+    }
+
+    // The same steps one by one: activations and (if the caller wants no y) the product in scratch.
+    const size_t x_off = 0, y_off = (kbytes + 255) / 256 * 256;
+    rc = ensure_scratch(ctx, y_off + static_cast<size_t>(n) * sizeof(float));
+    if (rc) return rc;
+    const float* act = x_dev;
+    float* xs = reinterpret_cast<float*>(ctx->moe_scratch + x_off);
+    if (f.prologue == LQ4_PRO_ADD_RMSNORM) {
+        launch_residual_add_norm(f.base, f.delta, f.gamma, k, 1, f.eps, f.residual_out, xs, s);
+        act = xs;
+        ctx->counters.elementwise++;
+    } else if (f.prologue == LQ4_PRO_SILU_MUL) {
+        launch_silu_mul(x_dev, k, 1, xs, k, s);
+        act = xs;
+        ctx->counters.elementwise++;
+    }
+    if (ep.rank) {
+        launch_lora_a(lora->a, lora->is_f16, lora->rank, k, act, 0, k, 1, ctx->lora_t, s);
+        ctx->counters.lora_a++;
+    }
+    float* yo = y_dev ? y_dev : reinterpret_cast<float*>(ctx->moe_scratch + y_off);
+    launch_gemv(wp, n, k, act, k, 1, yo, n, ep, s);
+    ctx->counters.gemv++;
+    if (f.epilogue == LQ4_EPI_ADD_RESIDUAL) {
+        launch_add_and_copy(yo, f.residual, f.copy_dst, n, s);
+        ctx->counters.elementwise++;
+    }
+    LQ4_HIP(hipGetLastError());
+    return LQ4_OK;
+}
+
 int lq4_set_gemm_kernel(int which) {
     if (which < 0 || which > 2) return fail(LQ4_E_INVALID, "gemm kernel choice must be 0, 1 or 2");
     set_gemm_kernel_choice(which);

@@ -115,10 +115,26 @@ __device__ __forceinline__ float block_dot(const uint32_t (&q)[4], const uint32_
 // j < RW — and, inside a chunk, through groups of SG slabs.  One (chunk, slab group) is a
 // unit: RW*SG blocks per lane, loaded with one burst; the next unit's burst is in flight
 // while the current one is consumed.  Dynamic LDS: (K/32) * kXPitch dwords.
-template <int RW, int SG, int SEG>
+//
+// FUSED instantiations take a GemvFusion: the activations are produced while they are staged
+// (residual add + shifted RMSNorm, or silu(gate) * up) and the result can be added into a
+// residual stream as it is stored.  Every workgroup stages the whole activation vector anyway,
+// so the norm costs one extra pass over K floats per workgroup and no launch.
+struct NoFusion {};
+template <bool FUSED>
+struct FusionArg {
+    typedef NoFusion type;
+};
+template <>
+struct FusionArg<true> {
+    typedef GemvFusion type;
+};
+
+template <int RW, int SG, int SEG, bool FUSED>
 __global__ __launch_bounds__(kWaves * 64) void gemv_q4_b1(const uint8_t* __restrict__ w, uint32_t n,
                                                           uint32_t k, const float* __restrict__ x,
-                                                          float* __restrict__ y, LoraEpilogue lora) {
+                                                          float* __restrict__ y, LoraEpilogue lora,
+                                                          typename FusionArg<FUSED>::type fz) {
     extern __shared__ __attribute__((aligned(16))) uint32_t xs[];
     constexpr int RPW = 64 / SEG;  // weight rows per wave-row
     const int tid = threadIdx.x;
@@ -141,9 +157,12 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_b1(const uint8_t* __restr
     // ---- first chunk of x is requested before any weight so it can be waited on alone ----
     // (straight-line code, clamped addresses: no branch between the loads and their wait)
     const uint32_t g0 = static_cast<uint32_t>(tid) < nb * 4 ? tid : 0;
-    const float4* x0p = reinterpret_cast<const float4*>(x + (g0 >> 2) * kBlockWeights + (g0 & 3) * 8);
-    const float4 x0a = x0p[0];
-    const float4 x0b = x0p[1];
+    float4 x0a = {0.0f, 0.0f, 0.0f, 0.0f}, x0b = x0a;
+    if constexpr (!FUSED) {
+        const float4* x0p = reinterpret_cast<const float4*>(x + (g0 >> 2) * kBlockWeights + (g0 & 3) * 8);
+        x0a = x0p[0];
+        x0b = x0p[1];
+    }
 
     // Loads unit u's blocks.  Lanes past the end of a row and rows past N re-read a valid
     // block; their contribution is zeroed or dropped later.
@@ -167,6 +186,16 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_b1(const uint8_t* __restr
 
     Q4BlockRaw buf_a[RW][SG], buf_b[RW][SG];
     load_unit(buf_a, 0);
+    // residual values of the first chunk's rows, requested now so the final store does not wait
+    float res_first[RW];
+    if constexpr (FUSED) {
+#pragma unroll
+        for (int j = 0; j < RW; ++j) {
+            const uint32_t wrow = j * n_waves + wid;
+            const uint32_t row = wrow * RPW + sub;
+            res_first[j] = (fz.epilogue == GemvFusion::kAddResidual && wrow < n_wrows && row < n) ? fz.residual[row] : 0.0f;
+        }
+    }
     __builtin_amdgcn_sched_barrier(0);  // nothing below is scheduled above these loads
 
     // ---- stage x: thread handles (block, dword j) = 8 activations ---------------------------
@@ -184,10 +213,114 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_b1(const uint8_t* __restr
             if (j == 0) *reinterpret_cast<float*>(&xs[blk * kXPitch + 32]) = sx;
         }
     };
-    stage(g0, x0a, x0b, static_cast<uint32_t>(tid) < nb * 4);
-    for (uint32_t g = tid + kWaves * 64; g < nb * 4; g += kWaves * 64) {
-        const float4* xp = reinterpret_cast<const float4*>(x + (g >> 2) * kBlockWeights + (g & 3) * 8);
-        stage(g, xp[0], xp[1], true);
+    if constexpr (!FUSED) {
+        stage(g0, x0a, x0b, static_cast<uint32_t>(tid) < nb * 4);
+        for (uint32_t g = tid + kWaves * 64; g < nb * 4; g += kWaves * 64) {
+            const float4* xp = reinterpret_cast<const float4*>(x + (g >> 2) * kBlockWeights + (g & 3) * 8);
+            stage(g, xp[0], xp[1], true);
+        }
+    } else {
+        __shared__ float red[kWaves];
+        const uint32_t n_units = nb * 4;
+        auto unit_at = [](uint32_t g) { return (g >> 2) * kBlockWeights + (g & 3) * 8; };
+        auto add4 = [](float4 a, const float4 b) {
+            a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+            return a;
+        };
+        auto sq4 = [](const float4 a) { return (a.x * a.x + a.y * a.y) + (a.z * a.z + a.w * a.w); };
+        auto norm4 = [](float4 v, float inv, const float4 g) {
+            v.x = v.x * inv * (1.0f + g.x); v.y = v.y * inv * (1.0f + g.y);
+            v.z = v.z * inv * (1.0f + g.z); v.w = v.w * inv * (1.0f + g.w);
+            return v;
+        };
+        // v = base + delta for unit g (8 activations)
+        auto load_v = [&](uint32_t g, float4& a, float4& b) {
+            const float4* bp = reinterpret_cast<const float4*>(fz.base + unit_at(g));
+            a = bp[0];
+            b = bp[1];
+            if (fz.delta) {
+                const float4* dp = reinterpret_cast<const float4*>(fz.delta + unit_at(g));
+                a = add4(a, dp[0]);
+                b = add4(b, dp[1]);
+            }
+        };
+        if (fz.prologue == GemvFusion::kAddNorm) {
+            // The first KEEP units of a thread (K <= 6144 has no more) stay in registers between
+            // the sum of squares and the scaling, with their gamma already requested; longer
+            // vectors re-read the rest.
+            constexpr int KEEP = 3;
+            float4 va[KEEP], vb[KEEP], ga[KEEP], gb[KEEP];
+            float ss = 0.0f;
+#pragma unroll
+            for (int i = 0; i < KEEP; ++i) {
+                const uint32_t g = tid + i * kWaves * 64;
+                const uint32_t gc = g < n_units ? g : 0;
+                load_v(gc, va[i], vb[i]);
+                const float4* gp = reinterpret_cast<const float4*>(fz.gamma + unit_at(gc));
+                ga[i] = gp[0];
+                gb[i] = gp[1];
+            }
+#pragma unroll
+            for (int i = 0; i < KEEP; ++i) {
+                const uint32_t g = tid + i * kWaves * 64;
+                if (g < n_units) {
+                    ss += sq4(va[i]) + sq4(vb[i]);
+                    if (blockIdx.x == 0 && fz.residual_out) {
+                        float4* rp = reinterpret_cast<float4*>(fz.residual_out + unit_at(g));
+                        rp[0] = va[i];
+                        rp[1] = vb[i];
+                    }
+                }
+            }
+            for (uint32_t g = tid + KEEP * kWaves * 64; g < n_units; g += kWaves * 64) {
+                float4 a, b;
+                load_v(g, a, b);
+                ss += sq4(a) + sq4(b);
+                if (blockIdx.x == 0 && fz.residual_out) {
+                    float4* rp = reinterpret_cast<float4*>(fz.residual_out + unit_at(g));
+                    rp[0] = a;
+                    rp[1] = b;
+                }
+            }
+            ss = wave_sum(ss);
+            if (lane == 0) red[tid >> 6] = ss;
+            __syncthreads();
+            const float total = (red[0] + red[1]) + (red[2] + red[3]);
+            const float inv_rms = 1.0f / sqrtf(total / static_cast<float>(k) + fz.eps);
+#pragma unroll
+            for (int i = 0; i < KEEP; ++i) {
+                const uint32_t g = tid + i * kWaves * 64;
+                if (g < n_units) stage(g, norm4(va[i], inv_rms, ga[i]), norm4(vb[i], inv_rms, gb[i]), true);
+            }
+            for (uint32_t g = tid + KEEP * kWaves * 64; g < n_units; g += kWaves * 64) {
+                float4 a, b;
+                load_v(g, a, b);
+                const float4* gp = reinterpret_cast<const float4*>(fz.gamma + unit_at(g));
+                stage(g, norm4(a, inv_rms, gp[0]), norm4(b, inv_rms, gp[1]), true);
+            }
+        } else if (fz.prologue == GemvFusion::kSiluMul) {
+            // silu through the hardware exp2 and reciprocal (about 1 ulp each): every workgroup
+            // evaluates the whole vector, so the library expf and an IEEE divide would sit on
+            // the critical path of each of them.
+            auto silu_mul = [](float gate, float u) {
+                const float e = __builtin_amdgcn_exp2f(gate * -1.44269504088896340736f);
+                return gate * __builtin_amdgcn_rcpf(1.0f + e) * u;
+            };
+            for (uint32_t g = tid; g < n_units; g += kWaves * 64) {
+                const float4* gp = reinterpret_cast<const float4*>(x + unit_at(g));
+                const float4* up = reinterpret_cast<const float4*>(x + k + unit_at(g));
+                const float4 ga = gp[0], gb = gp[1], ua = up[0], ub = up[1];
+                float4 a, b;
+                a.x = silu_mul(ga.x, ua.x); a.y = silu_mul(ga.y, ua.y); a.z = silu_mul(ga.z, ua.z); a.w = silu_mul(ga.w, ua.w);
+                b.x = silu_mul(gb.x, ub.x); b.y = silu_mul(gb.y, ub.y); b.z = silu_mul(gb.z, ub.z); b.w = silu_mul(gb.w, ub.w);
+                stage(g, a, b, true);
+            }
+        } else {
+            for (uint32_t g = tid; g < n_units; g += kWaves * 64) {
+                const float4* xp = reinterpret_cast<const float4*>(x + unit_at(g));
+                stage(g, xp[0], xp[1], true);
+            }
+        }
     }
     __syncthreads();
 
@@ -245,7 +378,18 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_b1(const uint8_t* __restr
                     }
                 }
                 v = segment_sum<SEG>(v);
-                if (seg_lane == SEG - 1 && row_ok) y[row] = v;
+                if (seg_lane == SEG - 1 && row_ok) {
+                    if constexpr (FUSED) {
+                        if (y) y[row] = v;
+                        if (fz.epilogue == GemvFusion::kAddResidual) {
+                            const float r = (chunk == 0 ? res_first[j] : fz.residual[row]) + v;
+                            fz.residual[row] = r;
+                            if (fz.copy_dst) fz.copy_dst[row] = r;
+                        }
+                    } else {
+                        y[row] = v;
+                    }
+                }
             }
         }
     };
@@ -259,16 +403,28 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_b1(const uint8_t* __restr
 
 template <int RW, int SG, int SEG>
 void launch_cfg(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, const LoraEpilogue& lora,
-                size_t lds, uint32_t waves, hipStream_t stream) {
-    static bool attr_set = false;  // raise the dynamic-LDS cap once per instantiation
-    if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        attr_set = true;
+                const GemvFusion* fusion, size_t lds, uint32_t waves, hipStream_t stream) {
+    static bool attr_set[2] = {false, false};  // raise the dynamic-LDS cap once per instantiation
+    const dim3 grid((waves + kWaves - 1) / kWaves), block(kWaves * 64);
+    if (fusion) {
+        if (!attr_set[1]) {
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, true>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 159 * 1024);
+            attr_set[1] = true;
+        }
+        hipLaunchKernelGGL((gemv_q4_b1<RW, SG, SEG, true>), grid, block, lds, stream, w, n, k, x, y, lora, *fusion);
+        return;
     }
-    hipLaunchKernelGGL((gemv_q4_b1<RW, SG, SEG>), dim3((waves + kWaves - 1) / kWaves), dim3(kWaves * 64), lds,
-                       stream, w, n, k, x, y, lora);
+    if (!attr_set[0]) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, false>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        attr_set[0] = true;
+    }
+    hipLaunchKernelGGL((gemv_q4_b1<RW, SG, SEG, false>), grid, block, lds, stream, w, n, k, x, y, lora, NoFusion{});
 }
+
+void launch_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, const LoraEpilogue& lora,
+               const GemvFusion* fusion, hipStream_t stream);
 
 }  // namespace
 
@@ -276,6 +432,18 @@ size_t gemv_b1_lds_bytes(uint32_t k) { return static_cast<size_t>(k / kBlockWeig
 
 void launch_gemv_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y,
                     const LoraEpilogue& lora, hipStream_t stream) {
+    launch_b1(w, n, k, x, y, lora, nullptr, stream);
+}
+
+void launch_gemv_b1_fused(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y,
+                          const LoraEpilogue& lora, const GemvFusion& fusion, hipStream_t stream) {
+    launch_b1(w, n, k, x, y, lora, &fusion, stream);
+}
+
+namespace {
+
+void launch_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, const LoraEpilogue& lora,
+               const GemvFusion* fusion, hipStream_t stream) {
     const size_t lds = gemv_b1_lds_bytes(k);
     const uint32_t nb = k / kBlockWeights;
     const uint32_t seg = nb == 32 ? 32 : nb == 16 ? 16 : 64;
@@ -308,7 +476,7 @@ void launch_gemv_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, fl
     uint32_t sg = slabs < 3 ? slabs : 3;
     while (rw * sg > 6) --sg;
 
-#define LQ4_B1(RW_, SG_, SEG_) launch_cfg<RW_, SG_, SEG_>(w, n, k, x, y, lora, lds, waves, stream)
+#define LQ4_B1(RW_, SG_, SEG_) launch_cfg<RW_, SG_, SEG_>(w, n, k, x, y, lora, fusion, lds, waves, stream)
     if (seg == 32) {
         if (rw == 1) LQ4_B1(1, 1, 32); else if (rw == 2) LQ4_B1(2, 1, 32); else if (rw == 3) LQ4_B1(3, 1, 32); else LQ4_B1(4, 1, 32);
     } else if (seg == 16) {
@@ -324,5 +492,7 @@ void launch_gemv_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, fl
     }
 #undef LQ4_B1
 }
+
+}  // namespace
 
 }  // namespace lq4

@@ -24,6 +24,27 @@ struct LoraEpilogue {
     float scale;
 };
 
+// Elementwise steps fused into the batch-1 GEMV.
+//   prologue kAddNorm: v = base + delta (delta may be null), the activation is the shifted RMSNorm
+//     v * rsqrt(mean(v^2) + eps) * (1 + gamma); workgroup 0 also writes v to residual_out if set
+//     (residual_out must not alias base or delta: other workgroups still read them).
+//   prologue kSiluMul: x holds [gate(K) | up(K)], the activation is silu(gate) * up.
+//   epilogue kAddResidual: residual[n] += y[n]; copy_dst[n] = residual[n] if set; y itself is
+//     stored only if its pointer is not null.
+struct GemvFusion {
+    enum Prologue : int { kPlain = 0, kAddNorm = 1, kSiluMul = 2 };
+    enum Epilogue : int { kStore = 0, kAddResidual = 1 };
+    int prologue;
+    const float* base;
+    const float* delta;
+    const float* gamma;
+    float eps;
+    float* residual_out;
+    int epilogue;
+    float* residual;
+    float* copy_dst;
+};
+
 // y[b, n] = W . x[b]  (+ LoRA), b < batch <= kMaxGemvBatch.  x rows are `x_stride`
 // floats apart, y rows `y_stride` floats apart.
 void launch_gemv(const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint32_t x_stride,
@@ -34,6 +55,21 @@ void launch_gemv(const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint3
 size_t gemv_b1_lds_bytes(uint32_t k);
 void launch_gemv_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y,
                     const LoraEpilogue& lora, hipStream_t stream);
+// Same with fused elementwise steps (separate kernel instantiations; the plain ones are untouched).
+void launch_gemv_b1_fused(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y,
+                          const LoraEpilogue& lora, const GemvFusion& fusion, hipStream_t stream);
+
+// Stand-alone forms of the same steps for any number of rows.
+//   residual_add_norm: v = base + delta (delta may be null); residual_out = v if set;
+//     normed_out = shifted RMSNorm of v.  Rows are `hidden` floats apart.
+//   silu_mul: out[r, i] = silu(gu[r, i]) * gu[r, count + i]; out rows out_stride floats apart
+//     (out == gate_up with out_stride == 2 * count is the in-place form).
+//   add_and_copy: residual += src; dst = residual if set.
+void launch_residual_add_norm(const float* base, const float* delta, const float* gamma, uint32_t hidden,
+                              uint32_t rows, float eps, float* residual_out, float* normed_out, hipStream_t stream);
+void launch_silu_mul(const float* gate_up, uint32_t count, uint32_t rows, float* out, uint32_t out_stride,
+                     hipStream_t stream);
+void launch_add_and_copy(const float* src, float* residual, float* dst, size_t count, hipStream_t stream);
 
 // Matrix-core GEMV for batch 1..8 (activations staged in LDS as f16 columns).
 size_t gemv_mfma_lds_bytes(uint32_t k, uint32_t batch);

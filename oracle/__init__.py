@@ -88,6 +88,14 @@ def lib() -> C.CDLL:
         fn.restype = C.c_int
         fn.argtypes = [_u8p, _u8p, C.c_int, C.c_int, C.c_int, _f32p, C.c_int, _i32p, _f32p,
                        C.c_int, outp]
+    L.lq4o_shifted_rms_norm.restype = None
+    L.lq4o_shifted_rms_norm.argtypes = [_f32p, _f32p, C.c_size_t, C.c_size_t, C.c_float]
+    L.lq4o_residual_add_norm.restype = None
+    L.lq4o_residual_add_norm.argtypes = [_f32p, _f32p, _f32p, C.c_size_t, C.c_size_t, C.c_float, _f32p, _f32p]
+    L.lq4o_silu_mul.restype = None
+    L.lq4o_silu_mul.argtypes = [_f32p, C.c_size_t, C.c_size_t, _f32p]
+    L.lq4o_add_and_copy.restype = None
+    L.lq4o_add_and_copy.argtypes = [_f32p, _f32p, _f32p, C.c_size_t]
     L.lq4o_topk.restype = None
     L.lq4o_topk.argtypes = [_f32p, C.c_uint32, C.c_uint32, _f32p, C.POINTER(C.c_uint32)]
     L.lq4o_parse_q4_file.restype = C.c_int
@@ -314,6 +322,47 @@ Q4_FILE_ERRORS = {1: "invalid magic: not a .q4 file", 2: "legacy .q4 file (v1)",
                   5: "file truncated below Q4 block payload",
                   6: "file has trailing bytes after Q4 block payload",
                   7: "original_len does not match shape"}
+
+
+def shifted_rms_norm(x, gamma, eps: float) -> np.ndarray:
+    """Qwen3.5 shifted RMSNorm of every row of x [rows, hidden] (model/qwen35/norm.rs:6-23)."""
+    x = np.array(_f32(x), copy=True)
+    x2 = x.reshape(-1, x.shape[-1])
+    gamma = _f32(gamma)
+    assert gamma.size == x2.shape[1]
+    lib().lq4o_shifted_rms_norm(_p(x2, _f32p), _p(gamma, _f32p), x2.shape[1], x2.shape[0], eps)
+    return x
+
+
+def residual_add_norm(base, delta, gamma, eps: float):
+    """(residual_out, normed_out) of fused_residual_add_norm (qwen35.metal:739-767)."""
+    base, delta, gamma = _f32(base), _f32(delta), _f32(gamma)
+    assert base.shape == delta.shape and gamma.size == base.shape[-1]
+    rows = base.size // base.shape[-1]
+    res, normed = np.empty_like(base), np.empty_like(base)
+    lib().lq4o_residual_add_norm(_p(base, _f32p), _p(delta, _f32p), _p(gamma, _f32p), base.shape[-1],
+                                 rows, eps, _p(res, _f32p), _p(normed, _f32p))
+    return res, normed
+
+
+def silu_mul(gate_up) -> np.ndarray:
+    """silu(gate) * up for rows of [gate | up] (qwen35.metal:712-722)."""
+    gate_up = _f32(gate_up)
+    g2 = gate_up.reshape(-1, gate_up.shape[-1])
+    count = g2.shape[1] // 2
+    assert g2.shape[1] == 2 * count
+    out = np.empty((g2.shape[0], count), dtype=np.float32)
+    lib().lq4o_silu_mul(_p(g2, _f32p), count, g2.shape[0], _p(out, _f32p))
+    return out.reshape(gate_up.shape[:-1] + (count,))
+
+
+def add_and_copy(src, residual):
+    """(updated residual, copy) of add_and_copy (qwen35.metal:2255-2266)."""
+    src = _f32(src)
+    res = np.array(_f32(residual), copy=True)
+    dst = np.empty_like(res)
+    lib().lq4o_add_and_copy(_p(src, _f32p), _p(res, _f32p), _p(dst, _f32p), res.size)
+    return res, dst
 
 
 def topk(logits, k: int):

@@ -565,6 +565,52 @@ int lq4o_parse_q4_file(const uint8_t* file, size_t file_len, uint64_t* shape, in
     return 0;
 }
 
+/* ---- elementwise steps either side of the decode GEMVs ---------------------------------
+ * Shifted RMSNorm of Qwen3.5, qwen35_rms_norm (crates/inference/src/model/qwen35/norm.rs:6-23):
+ * per row a sequential f32 sum of squares, rms = sqrt(sum / hidden + eps), inv = 1 / rms,
+ * out = x * inv * (1 + gamma), evaluated left to right in f32. */
+void lq4o_shifted_rms_norm(float* x, const float* gamma, size_t hidden, size_t rows, float eps) {
+    for (size_t t = 0; t < rows; ++t) {
+        float* row = x + t * hidden;
+        float sum_sq = 0.0f;
+        for (size_t i = 0; i < hidden; ++i) sum_sq += row[i] * row[i];
+        const float rms = sqrtf(sum_sq / (float)hidden + eps);
+        const float inv_rms = 1.0f / rms;
+        for (size_t i = 0; i < hidden; ++i) row[i] = row[i] * inv_rms * (1.0f + gamma[i]);
+    }
+}
+
+/* fused_residual_add_norm / fused_residual_add_norm_batch (shaders/qwen35.metal:739-767,
+ * 2219-2249): residual_out = base + delta, normed_out = shifted RMSNorm of residual_out. */
+void lq4o_residual_add_norm(const float* base, const float* delta, const float* gamma, size_t hidden,
+                            size_t rows, float eps, float* residual_out, float* normed_out) {
+    for (size_t i = 0; i < hidden * rows; ++i) {
+        residual_out[i] = base[i] + delta[i];
+        normed_out[i] = residual_out[i];
+    }
+    lq4o_shifted_rms_norm(normed_out, gamma, hidden, rows, eps);
+}
+
+/* silu_mul_fused (shaders/qwen35.metal:712-722) per row of [gate(count) | up(count)]:
+ * out[i] = gate / (1 + exp(-gate)) * up. */
+void lq4o_silu_mul(const float* gate_up, size_t count, size_t rows, float* out) {
+    for (size_t r = 0; r < rows; ++r)
+        for (size_t i = 0; i < count; ++i) {
+            const float gate = gate_up[r * 2 * count + i], up = gate_up[r * 2 * count + count + i];
+            const float s = gate / (1.0f + expf(-gate));
+            out[r * count + i] = s * up;
+        }
+}
+
+/* add_and_copy (shaders/qwen35.metal:2255-2266): residual += src; dst = residual. */
+void lq4o_add_and_copy(const float* src, float* residual, float* dst, size_t count) {
+    for (size_t i = 0; i < count; ++i) {
+        const float r = residual[i] + src[i];
+        residual[i] = r;
+        dst[i] = r;
+    }
+}
+
 /* ---- lm_head top-k selection ----------------------------------------------------
  * The ordering of the reference's GPU top-k (shaders/qwen35.metal:1688-1703):
  * candidate = (logit, token_id); a ranks before b if it has the higher logit, ties go

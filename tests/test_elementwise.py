@@ -1,0 +1,255 @@
+"""The elementwise steps either side of the decode GEMVs: residual add + shifted RMSNorm
+(shaders/qwen35.metal:739-767, model/qwen35/norm.rs:6-23), silu(gate) * up
+(shaders/qwen35.metal:712-722), add-and-copy (shaders/qwen35.metal:2255-2266), stand-alone and
+fused into the batch-1 Q4 GEMV.
+
+Oracle pins: the norm against the HF RMSNorm goldens the reference's tests hold
+(tests/fixtures/gemma4/stage3/rms_norm*.bin, standard gamma: the shifted norm with gamma - 1 must
+reproduce them), closed forms, and an f64 restatement; silu against its identities and the value
+the reference's MoE test uses (model/qwen35/tests.rs:298-299, 355)."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from lattice_amd import synth
+from util import REL_TOL, rel_err
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden", "rms_norm")
+ELT_TOL = 2e-6  # f32 rounding: summation order of the mean square, one ulp of expf
+
+
+def _bin(name):
+    return np.fromfile(os.path.join(GOLD, name), dtype="<f4")
+
+
+@pytest.mark.parametrize("prefix,hidden,tol", [("rms_norm", 64, 1e-6), ("rms_norm_wide", 1536, 5e-5)])
+def test_oracle_norm_reproduces_hf_goldens(prefix, hidden, tol):
+    # tolerances: the fixtures' own manifest (1e-6 at width 64, 5e-5 at width 1536), eps 1e-6
+    x = _bin(prefix + "_input.bin").reshape(-1, hidden)
+    w = _bin(prefix + "_weight.bin")
+    want = _bin(prefix + "_output.bin").reshape(-1, hidden)
+    got = oracle.shifted_rms_norm(x, w - np.float32(1.0), 1e-6)
+    assert np.max(np.abs(got - want)) <= tol + 2e-7 * np.max(np.abs(want))  # (1 + (w - 1)) rounds once more
+    # and the shift matters: plain gamma fed to the shifted norm misses the golden by far
+    assert np.max(np.abs(oracle.shifted_rms_norm(x, w, 1e-6) - want)) > 1e-2
+
+
+def test_oracle_norm_closed_forms():
+    h = 96
+    gamma = np.linspace(-0.5, 0.5, h).astype(np.float32)
+    const = np.full((1, h), 3.0, np.float32)
+    got = oracle.shifted_rms_norm(const, gamma, 1e-6)
+    want = 3.0 / np.sqrt(9.0 + 1e-6) * (1.0 + gamma.astype(np.float64))
+    assert np.max(np.abs(got[0] - want)) < 1e-6
+    assert np.all(oracle.shifted_rms_norm(np.zeros((2, h), np.float32), gamma, 1e-6) == 0.0)
+    g = np.random.default_rng(0)
+    x = g.normal(size=(5, h)).astype(np.float32)
+    a = oracle.shifted_rms_norm(x, gamma, 0.0)
+    b = oracle.shifted_rms_norm(4.0 * x, gamma, 0.0)  # scale invariance without eps
+    assert rel_err(a, b) < 1e-6
+    x64 = x.astype(np.float64)
+    want = x64 / np.sqrt(np.mean(x64 * x64, axis=1, keepdims=True) + 1e-5) * (1.0 + gamma.astype(np.float64))
+    assert rel_err(oracle.shifted_rms_norm(x, gamma, 1e-5), want) < 1e-6
+    # rows are independent
+    assert np.array_equal(oracle.shifted_rms_norm(x, gamma, 1e-5)[2], oracle.shifted_rms_norm(x[2:3], gamma, 1e-5)[0])
+
+
+def test_oracle_residual_add_norm_silu_and_add():
+    g = np.random.default_rng(1)
+    base, delta = g.normal(size=(3, 64)).astype(np.float32), g.normal(size=(3, 64)).astype(np.float32)
+    gamma = g.normal(size=64).astype(np.float32) * 0.1
+    res, normed = oracle.residual_add_norm(base, delta, gamma, 1e-6)
+    assert np.array_equal(res, base + delta)
+    assert np.array_equal(normed, oracle.shifted_rms_norm(res, gamma, 1e-6))
+
+    gu = np.array([[0.5, 0.0, -3.0, 20.0, 2.0, 7.0, 1.0, 1.0]], np.float32)  # gate(4) | up(4)
+    out = oracle.silu_mul(gu)[0]
+    silu_half = np.float32(0.5) / (np.float32(1.0) + np.exp(np.float32(-0.5)))
+    assert abs(out[0] - silu_half * 2.0) < 1e-7 and abs(out[0] - 0.62244) < 5e-5  # the reference quotes ~0.62244
+    assert abs(out[0] - 2.0 * 0.5 / (1.0 + np.exp(-0.5))) < 1e-7
+    assert out[1] == 0.0
+    x = g.normal(size=200).astype(np.float32) * 4
+    pos = oracle.silu_mul(np.concatenate([x, np.ones_like(x)])[None])[0]
+    neg = oracle.silu_mul(np.concatenate([-x, np.ones_like(x)])[None])[0]
+    assert np.max(np.abs((pos - neg) - x)) < 1e-6          # silu(x) - silu(-x) = x
+    x64 = x.astype(np.float64)
+    assert np.max(np.abs(pos - x64 / (1.0 + np.exp(-x64)))) < 1e-6
+    rows = g.normal(size=(3, 10)).astype(np.float32)
+    assert np.array_equal(oracle.silu_mul(rows)[1], oracle.silu_mul(rows[1:2])[0])
+
+    src, res0 = g.normal(size=33).astype(np.float32), g.normal(size=33).astype(np.float32)
+    res1, dst = oracle.add_and_copy(src, res0)
+    assert np.array_equal(res1, res0 + src) and np.array_equal(dst, res1)
+
+
+# ---- GPU ------------------------------------------------------------------------------------
+
+@pytest.fixture(scope="module")
+def be():
+    from lattice_amd import backend
+    b = backend.HipQ4Backend(0)
+    yield b
+    b.close()
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    return t.detach().cpu().numpy()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,hidden", [(1, 2048), (5, 96), (3, 5120), (2, 100)])
+def test_standalone_kernels_match_oracle(be, rows, hidden):
+    import torch
+    g = np.random.default_rng(rows * 1000 + hidden)
+    base, delta = g.normal(size=(rows, hidden)).astype(np.float32), g.normal(size=(rows, hidden)).astype(np.float32)
+    gamma = (g.normal(size=hidden) * 0.2).astype(np.float32)
+    res_ref, normed_ref = oracle.residual_add_norm(base, delta, gamma, 1e-6)
+    res = torch.empty((rows, hidden), device="cuda")
+    normed = torch.empty((rows, hidden), device="cuda")
+    be.dispatch_fused_residual_add_norm(dev(base), dev(delta), res, normed, dev(gamma), hidden, 1e-6, rows)
+    assert np.array_equal(host(res), res_ref)
+    assert rel_err(host(normed), normed_ref) <= ELT_TOL
+    # plain norm: no delta, no residual store
+    be.dispatch_fused_residual_add_norm(dev(base), None, None, normed, dev(gamma), hidden, 1e-6, rows)
+    assert rel_err(host(normed), oracle.shifted_rms_norm(base, gamma, 1e-6)) <= ELT_TOL
+
+    count = hidden // 2
+    gu = (g.normal(size=(rows, 2 * count)) * 3).astype(np.float32)
+    want = oracle.silu_mul(gu)
+    out = torch.empty((rows, count), device="cuda")
+    be.dispatch_silu_mul_fused(dev(gu), count, rows, out=out)
+    assert rel_err(host(out), want) <= ELT_TOL
+    inplace = dev(gu)
+    be.dispatch_silu_mul_fused(inplace, count, rows)  # the reference's in-place form
+    got = host(inplace)
+    assert rel_err(got[:, :count], want) <= ELT_TOL and np.array_equal(got[:, count:], gu[:, count:])
+
+    src, r0 = g.normal(size=rows * hidden).astype(np.float32), g.normal(size=rows * hidden).astype(np.float32)
+    r_ref, d_ref = oracle.add_and_copy(src, r0)
+    r, d = dev(r0), torch.empty(rows * hidden, device="cuda")
+    be.dispatch_add_and_copy(dev(src), r, d, rows * hidden)
+    assert np.array_equal(host(r), r_ref) and np.array_equal(host(d), d_ref)
+
+
+def _mlp_inputs(hidden, inter, seed):
+    g = np.random.default_rng(seed)
+    gate_up = synth.q4_weight(2 * inter, hidden, seed=seed)
+    down = synth.q4_weight(hidden, inter, seed=seed + 1)
+    base = g.normal(size=hidden).astype(np.float32)
+    delta = g.normal(size=hidden).astype(np.float32)
+    gamma = (g.normal(size=hidden) * 0.2).astype(np.float32)
+    return gate_up, down, base, delta, gamma
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("hidden,inter", [(2048, 6144), (1024, 512), (512, 96), (160, 352)])
+def test_fused_decode_mlp_matches_oracle_and_unfused(be, hidden, inter):
+    """norm + gate||up GEMV, then silu*up + down GEMV + residual add: two fused launches against
+    the oracle's five steps and against the same five steps run one by one on the GPU."""
+    import torch
+    gate_up, down, base, delta, gamma = _mlp_inputs(hidden, inter, 11)
+    eps = 1e-6
+    # oracle
+    res_ref, normed_ref = oracle.residual_add_norm(base[None], delta[None], gamma, eps)
+    gu_ref = oracle.gemm_f32(normed_ref, gate_up, 2 * inter, hidden)
+    h_ref = oracle.silu_mul(gu_ref)
+    ffn_ref = oracle.gemm_f32(h_ref, down, hidden, inter)
+    final_ref, copy_ref = oracle.add_and_copy(ffn_ref[0], res_ref[0])
+
+    qgu, qd = be.upload_q4_blocks(gate_up), be.upload_q4_blocks(down)
+    d_base, d_delta, d_gamma = dev(base), dev(delta), dev(gamma)
+    # fused: two launches
+    residual = torch.full((hidden,), float("nan"), device="cuda")
+    gu = torch.full((2 * inter + 1,), float("nan"), device="cuda")
+    be.dispatch_matmul_fused(None, qgu, gu, 2 * inter, hidden, norm=(d_base, d_delta, d_gamma, eps, residual))
+    assert np.array_equal(host(residual), res_ref[0])
+    got_gu = host(gu)
+    assert np.isnan(got_gu[-1]) and rel_err(got_gu[:-1], gu_ref[0]) <= REL_TOL
+    hidden_out = torch.full((hidden,), float("nan"), device="cuda")
+    ffn = torch.full((hidden,), float("nan"), device="cuda")
+    be.dispatch_matmul_fused(gu, qd, ffn, hidden, inter, silu_mul=True, add_residual=(residual, hidden_out))
+    assert rel_err(host(ffn), ffn_ref[0]) <= REL_TOL
+    assert rel_err(host(residual), final_ref) <= REL_TOL
+    assert np.array_equal(host(hidden_out), host(residual))
+    assert np.array_equal(host(residual), res_ref[0] + host(ffn))  # the add itself is exact
+
+    # unfused on the GPU: same kernels' arithmetic, so agreement is at f32 rounding level
+    res2 = torch.empty(hidden, device="cuda")
+    normed = torch.empty(hidden, device="cuda")
+    be.dispatch_fused_residual_add_norm(d_base, d_delta, res2, normed, d_gamma, hidden, eps)
+    gu2 = torch.empty(2 * inter, device="cuda")
+    be.dispatch_matmul(normed, qgu, gu2, 1, 2 * inter, hidden)
+    assert rel_err(got_gu[:-1], host(gu2)) <= 1e-5
+    be.dispatch_silu_mul_fused(gu2, inter)
+    ffn2 = torch.empty(hidden, device="cuda")
+    be.dispatch_matmul(gu2, qd, ffn2, 1, hidden, inter)
+    assert rel_err(host(ffn), host(ffn2)) <= 1e-5
+    hid2 = torch.empty(hidden, device="cuda")
+    be.dispatch_add_and_copy(ffn2, res2, hid2, hidden)
+    assert rel_err(host(hidden_out), host(hid2)) <= 1e-5
+    c = be.path_counters()
+    assert c["gemv_fused"] >= 2
+
+
+@pytest.mark.gpu
+def test_fused_gemv_options_and_fallbacks(be):
+    import torch
+    from lattice_amd import backend
+    n, k = 37, 1024
+    g = np.random.default_rng(5)
+    wq = synth.q4_weight(n, k, seed=5)
+    qw = be.upload_q4_blocks(wq)
+    x = g.normal(size=k).astype(np.float32)
+    res0 = g.normal(size=n).astype(np.float32)
+    y_ref = oracle.gemm_f32(x[None], wq, n, k)[0]
+    # epilogue only, no y wanted
+    residual = dev(res0)
+    be.dispatch_matmul_fused(dev(x), qw, None, n, k, add_residual=(residual, None))
+    assert rel_err(host(residual), res0 + y_ref) <= REL_TOL
+    # prologue only, norm without delta and without residual store
+    gamma = (g.normal(size=k) * 0.1).astype(np.float32)
+    y = torch.empty(n, device="cuda")
+    be.dispatch_matmul_fused(None, qw, y, n, k, norm=(dev(x), None, dev(gamma), 1e-5, None))
+    want = oracle.gemm_f32(oracle.shifted_rms_norm(x[None], gamma, 1e-5), wq, n, k)[0]
+    assert rel_err(host(y), want) <= REL_TOL
+    # LoRA + prologue runs as the unfused sequence; LoRA + epilogue stays fused
+    a, b = synth.lora_pair(8, k, n, seed=5)
+    be.load_lora_adapter([backend.LoraLayerData(0, {"q_proj": (a, b)})], scale=2.0)
+    try:
+        before = be.path_counters()
+        be.dispatch_matmul_fused(None, qw, y, n, k, norm=(dev(x), None, dev(gamma), 1e-5, None), layer_idx=0,
+                                 module="q_proj")
+        mid = be.path_counters()
+        assert mid["gemv_fused"] == before["gemv_fused"] and mid["elementwise"] == before["elementwise"] + 1
+        xn = oracle.shifted_rms_norm(x[None], gamma, 1e-5)
+        assert rel_err(host(y), oracle.lora_apply(a, b, 2.0, xn, oracle.gemm_f32(xn, wq, n, k))[0]) <= REL_TOL
+        residual = dev(res0)
+        be.dispatch_matmul_fused(dev(x), qw, y, n, k, add_residual=(residual, None), layer_idx=0, module="q_proj")
+        assert be.path_counters()["gemv_fused"] == mid["gemv_fused"] + 1
+        y_l = oracle.lora_apply(a, b, 2.0, x[None], y_ref[None].copy())[0]
+        assert rel_err(host(y), y_l) <= REL_TOL and rel_err(host(residual), res0 + y_l) <= REL_TOL
+    finally:
+        be.unload_lora_adapter()
+    # K too long for the staged kernel: the unfused sequence through scratch
+    kk = 29184
+    wl = synth.q4_weight(4, kk, seed=6)
+    ql = be.upload_q4_blocks(wl)
+    gul = (g.normal(size=2 * kk)).astype(np.float32)
+    yl = torch.empty(4, device="cuda")
+    rl = dev(np.ones(4, np.float32))
+    be.dispatch_matmul_fused(dev(gul), ql, yl, 4, kk, silu_mul=True, add_residual=(rl, None))
+    want = oracle.gemm_f32(oracle.silu_mul(gul[None]), wl, 4, kk)[0]
+    assert rel_err(host(yl), want) <= REL_TOL and rel_err(host(rl), 1.0 + want) <= REL_TOL
+    # rejected calls: residual_out over base, missing y without an epilogue
+    xb = dev(x)
+    with pytest.raises(backend.Q4Error):
+        be.dispatch_matmul_fused(None, qw, y, n, k, norm=(xb, None, dev(gamma), 1e-5, xb))
+    with pytest.raises(backend.Q4Error):
+        be.dispatch_matmul_fused(xb, qw, None, n, k, silu_mul=False, add_residual=None, norm=(xb, None, dev(gamma), 1e-5, None))

@@ -224,6 +224,19 @@ int lq4_gemv_fused(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, u
                    const float* x_dev, float* y_dev, const lq4_gemv_fusion* fusion, const lq4_lora* lora,
                    float lora_scale, void* stream);
 
+/* ---- Q8_0 sibling format -----------------------------------------------------------
+ * 34-byte blocks [u16 f16 scale d][32 x i8], w = q * d, rows of K/32 blocks, 2-byte aligned
+ * (forward/metal_qwen35.rs:2310-2346).  Weight handles are format-agnostic byte buffers: upload
+ * Q8_0 blocks with lq4_weight_upload(..., validate = 0) or wrap them with lq4_weight_wrap.
+ * lq4_gemv_q8 replaces dispatch_matmul_q8 (inner/dispatch.rs:61-84; batch 1 is the decode GEMV,
+ * batch <= 16 rows take the tile kernel), lq4_gemm_q8 replaces dispatch_gemm_q8
+ * (inner/dispatch.rs:86-146): same conventions as lq4_gemv / lq4_gemm, no LoRA argument (apply
+ * lq4_lora_apply afterwards). */
+int lq4_gemv_q8(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
+                const float* x_dev, uint32_t batch, float* y_dev, void* stream);
+int lq4_gemm_q8(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
+                const void* x_dev, int x_dtype, uint32_t m, float* y_dev, void* stream);
+
 /* ---- probes --------------------------------------------------------------------
  * Writes f32(nibble)*scale + bias for every weight of W[N,K] to out_dev (f32 [N,K]):
  * the bit-exactness probe for nibble unpack and scale/bias indexing against

@@ -51,6 +51,7 @@ EXPORTS = [
     "lq4_probe_copy",
     "lq4_set_gemm_kernel",
     "lq4_residual_add_rmsnorm", "lq4_silu_mul", "lq4_add_and_copy", "lq4_gemv_fused",
+    "lq4_gemv_q8", "lq4_gemm_q8",
     "lq4_get_path_counters", "lq4_malloc", "lq4_free", "lq4_memcpy_h2d", "lq4_memcpy_d2h",
 ]
 
@@ -125,6 +126,8 @@ def load_library() -> C.CDLL:
         "lq4_residual_add_rmsnorm": (C.c_int, [vp, vp, vp, vp, C.c_uint32, C.c_uint32, C.c_float, vp, vp, vp]),
         "lq4_silu_mul": (C.c_int, [vp, vp, C.c_uint32, C.c_uint32, vp, C.c_uint32, vp]),
         "lq4_add_and_copy": (C.c_int, [vp, vp, vp, vp, C.c_size_t, vp]),
+        "lq4_gemv_q8": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, C.c_uint32, vp, vp]),
+        "lq4_gemm_q8": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, C.c_int, C.c_uint32, vp, vp]),
         "lq4_gemv_fused": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, vp, C.POINTER(GemvFusion), vp,
                                      C.c_float, vp]),
         "lq4_get_path_counters": (C.c_int, [vp, C.POINTER(PathCounters)]),
@@ -309,6 +312,29 @@ class HipQ4Backend:
         lora = self._lora_for(layer_idx, module, n, k)
         _check(self.lib.lq4_gemv(self.ctx, qw.handle, 0, n, k, x.data_ptr(), 1, y.data_ptr(), lora,
                                  self._lora_scale, self._stream()))
+
+    # ---- Q8_0 sibling format ------------------------------------------------------------------
+    def upload_q8_blocks(self, blocks) -> Q4WeightBuf:
+        """Uploads Q8_0 blocks (34 bytes per 32 weights, metal_qwen35.rs:2310-2346); the handle is
+        the same byte-buffer type as for Q4 (the reference also keeps Q8_0 in a ``Q4WeightBuf``)."""
+        return self.upload_q4_blocks(blocks, validate=False)
+
+    def dispatch_matmul_q8(self, x, qw: Q4WeightBuf, y, m: int, n: int, k: int):
+        """``dispatch_matmul_q8`` (dispatch.rs:61-84): decode GEMV over Q8_0 blocks, ``m`` ignored."""
+        if n == 0:
+            return
+        self._assert_k(k, "dispatch_matmul_q8")
+        _check(self.lib.lq4_gemv_q8(self.ctx, qw.handle, 0, n, k, x.data_ptr(), 1, y.data_ptr(), self._stream()))
+
+    def dispatch_gemm_q8(self, x, x_offset: int, qw: Q4WeightBuf, y, y_offset: int, m: int, n: int, k: int):
+        """``dispatch_gemm_q8`` (dispatch.rs:86-146): byte offsets into x and y; ``m == 0 or n == 0``
+        is a no-op; ``m <= 1`` takes the GEMV."""
+        if m == 0 or n == 0:
+            return
+        self._assert_k(k, "dispatch_gemm_q8")
+        dt = _dtype_code(x)
+        _check(self.lib.lq4_gemm_q8(self.ctx, qw.handle, 0, n, k, x.data_ptr() + x_offset, dt, m,
+                                    y.data_ptr() + y_offset, self._stream()))
 
     # ---- elementwise steps either side of the decode GEMVs -----------------------------------
     @staticmethod

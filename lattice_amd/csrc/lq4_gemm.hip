@@ -83,10 +83,44 @@ __device__ __forceinline__ uint4 dequant8(uint32_t q, half2v d2, half2v b2) {
     return r;
 }
 
+// Q8_0 sibling format (FMT == 1): 34-byte block [u16 f16 scale][32 x i8], only 2-byte aligned.
+struct __attribute__((packed, aligned(2))) Q8BlockRaw {
+    uint16_t d;
+    uint32_t q[8];  // weight i in byte i
+};
+
+template <int FMT>
+struct WBlockOf {
+    typedef Q4BlockRaw type;
+};
+template <>
+struct WBlockOf<1> {
+    typedef Q8BlockRaw type;
+};
+
+// Two packed dwords of a Q8_0 block (weights 8j..8j+7) -> 8 f16 weights half(q * d) in memory
+// order.  A sign-flipped byte (q + 128) placed under the exponent byte of 1024.0 is 1024 + 128 + q
+// exactly; one packed subtract leaves q, one packed multiply applies the scale with one rounding.
+__device__ __forceinline__ uint4 dequant8_q8(uint32_t qa, uint32_t qb, half2v d2) {
+    const half2v k1152 = {static_cast<_Float16>(1152.0f), static_cast<_Float16>(1152.0f)};
+    const uint32_t ua = qa ^ 0x80808080u, ub = qb ^ 0x80808080u;
+    const half2v p01 = as_h2(__builtin_amdgcn_perm(0x64646464u, ua, 0x04010400u)) - k1152;
+    const half2v p23 = as_h2(__builtin_amdgcn_perm(0x64646464u, ua, 0x04030402u)) - k1152;
+    const half2v p45 = as_h2(__builtin_amdgcn_perm(0x64646464u, ub, 0x04010400u)) - k1152;
+    const half2v p67 = as_h2(__builtin_amdgcn_perm(0x64646464u, ub, 0x04030402u)) - k1152;
+    uint4 r;
+    r.x = as_u32(p01 * d2);
+    r.y = as_u32(p23 * d2);
+    r.z = as_u32(p45 * d2);
+    r.w = as_u32(p67 * d2);
+    return r;
+}
+
 // BN_: weight rows per workgroup (128 or 256); 2*BN_ threads; waves in a 2 x (BN_/64) grid.
 // LORA: compiled with the LoRA step (kept out of the plain kernel, whose register allocation it
 // would disturb).
-template <bool X_F16, int BN_, bool LORA>
+// FMT: 0 = Q4 blocks, 1 = Q8_0 blocks (no LoRA step).
+template <bool X_F16, int BN_, bool LORA, int FMT = 0>
 __global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
     const uint8_t* __restrict__ w, uint32_t n, uint32_t k, const void* __restrict__ xv, uint32_t m,
     float* __restrict__ y, LoraEpilogue lora) {
@@ -128,8 +162,10 @@ __global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
     // weights: thread -> (row tid/2, block tid%2 of the step)
     const uint32_t w_row = n0 + (tid >> 1);
     const bool w_live_row = w_row < n;
+    typedef typename WBlockOf<FMT>::type WBlock;
     const uint32_t* w_ptr =
         reinterpret_cast<const uint32_t*>(w) + static_cast<size_t>(w_live_row ? w_row : 0) * (nb * 5);
+    const uint8_t* w_ptr8 = w + static_cast<size_t>(w_live_row ? w_row : 0) * (nb * 34);  // FMT == 1
     const int w_half = tid & 1;
     // activations: chunk i of this thread is (row, part) = divmod(tid + kThreads*i, chunks per row)
     const uint8_t* x_ptr[XCH];
@@ -161,13 +197,14 @@ __global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
                                           : make_uint4(0, 0, 0, 0);
         }
     };
-    auto load_w = [&](Q4BlockRaw& wst, uint32_t s) {
+    auto load_w = [&](WBlock& wst, uint32_t s) {
         uint32_t blk = s * 2 + w_half;
         if (blk >= nb) blk = nb - 1;
-        wst = *reinterpret_cast<const Q4BlockRaw*>(w_ptr + blk * 5);
+        if constexpr (FMT == 0) wst = *reinterpret_cast<const WBlock*>(w_ptr + blk * 5);
+        else wst = *reinterpret_cast<const WBlock*>(w_ptr8 + blk * 34);
     };
 
-    auto store_tiles = [&](const XStage& st, const Q4BlockRaw& wst, uint32_t s, _Float16* xs, _Float16* ws) {
+    auto store_tiles = [&](const XStage& st, const WBlock& wst, uint32_t s, _Float16* xs, _Float16* ws) {
 #pragma unroll
         for (int i = 0; i < XCH; ++i) {
             const int c = tid + kThreads * i;
@@ -184,13 +221,21 @@ __global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
             }
         }
         const bool live = w_live_row && (s * 2 + w_half) < nb;
-        const uint32_t sb = live ? wst.sb : 0u;
-        const half2v d2 = as_h2(__builtin_amdgcn_perm(sb, sb, 0x01000100u));  // (d, d)
-        const half2v b2 = as_h2(__builtin_amdgcn_perm(sb, sb, 0x03020302u));  // (b, b)
         _Float16* dst = &ws[(tid >> 1) * kPitch + w_half * 32];
+        if constexpr (FMT == 0) {
+            const uint32_t sb = live ? wst.sb : 0u;
+            const half2v d2 = as_h2(__builtin_amdgcn_perm(sb, sb, 0x01000100u));  // (d, d)
+            const half2v b2 = as_h2(__builtin_amdgcn_perm(sb, sb, 0x03020302u));  // (b, b)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            *reinterpret_cast<uint4*>(dst + j * 8) = dequant8(live ? wst.q[j] : 0u, d2, b2);
+            for (int j = 0; j < 4; ++j)
+                *reinterpret_cast<uint4*>(dst + j * 8) = dequant8(live ? wst.q[j] : 0u, d2, b2);
+        } else {
+            const uint32_t db = live ? wst.d : 0u;
+            const half2v d2 = as_h2(db | (db << 16));
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                *reinterpret_cast<uint4*>(dst + j * 8) = dequant8_q8(wst.q[2 * j], wst.q[2 * j + 1], d2);
+        }
     };
 
     // Matrix-core work of one K step.  Operand layout of v_mfma_f32_32x32x16_f16: lane l supplies
@@ -233,7 +278,7 @@ __global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
     // position (nothing is copied): step s uses activation set s%2, weight set s%4, LDS buffer s%2.
     // Steps past the end of K (at most three) run on zeros, which keeps the body branch-free.
     XStage xa, xb;
-    Q4BlockRaw w0, w1, w2, w3;
+    WBlock w0, w1, w2, w3;
     load_x(xa, 0);
     load_w(w0, 0);
     load_w(w1, 1);
@@ -318,18 +363,18 @@ __global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
         }
 }
 
-template <bool X_F16, int BN_, bool LORA>
+template <bool X_F16, int BN_, bool LORA, int FMT = 0>
 void launch_tile(const uint8_t* w, uint32_t n, uint32_t k, const void* x, uint32_t m, float* y,
                  const LoraEpilogue& lora, hipStream_t stream) {
     const uint32_t tiles = ((n + BN_ - 1) / BN_) * ((m + BM - 1) / BM);
     const size_t lds = 2 * (BM + BN_) * kPitch * sizeof(_Float16);
     static bool attr_set = false;
     if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4_mfma<X_F16, BN_, LORA>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4_mfma<X_F16, BN_, LORA, FMT>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         attr_set = true;
     }
-    hipLaunchKernelGGL((gemm_q4_mfma<X_F16, BN_, LORA>), dim3(tiles), dim3(2 * BN_), lds, stream, w, n, k, x, m, y,
+    hipLaunchKernelGGL((gemm_q4_mfma<X_F16, BN_, LORA, FMT>), dim3(tiles), dim3(2 * BN_), lds, stream, w, n, k, x, m, y,
                        lora);
 }
 
@@ -386,6 +431,13 @@ void launch_gemm(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_
         if (x_is_f16) launch_tile<true, 128, false>(w, n, k, x, m, y, lora, stream);
         else launch_tile<false, 128, false>(w, n, k, x, m, y, lora, stream);
     }
+}
+
+void launch_gemm_q8(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
+                    hipStream_t stream) {
+    const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};
+    if (x_is_f16) launch_tile<true, 128, false, 1>(w, n, k, x, m, y, none, stream);
+    else launch_tile<false, 128, false, 1>(w, n, k, x, m, y, none, stream);
 }
 
 }  // namespace lq4

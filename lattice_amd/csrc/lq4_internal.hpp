@@ -104,6 +104,13 @@ uint32_t gemm_wreg_slices(uint32_t n, uint32_t k, uint32_t m);
 void launch_gemm_wreg(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
                       float* y, const LoraEpilogue& lora, uint32_t slices, float* partial, hipStream_t stream);
 
+// Q8_0 sibling format (34-byte blocks: f16 scale + 32 x i8, w = q * d): batch-1 GEMV with x staged
+// in LDS (gemv_q8_lds_bytes(k) bytes), and the LDS-staged tile GEMM for everything else.
+size_t gemv_q8_lds_bytes(uint32_t k);
+void launch_gemv_q8_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, hipStream_t stream);
+void launch_gemm_q8(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
+                    hipStream_t stream);
+
 void launch_probe_read(const void* p, size_t nbytes, uint32_t* sink, hipStream_t stream);
 void launch_probe_copy(const void* src, void* dst, size_t nbytes, hipStream_t stream);
 void launch_dequant(const uint8_t* w, uint32_t n, uint32_t k, float* out, hipStream_t stream);

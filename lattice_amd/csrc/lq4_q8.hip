@@ -1,0 +1,176 @@
+// Q8_0 sibling of the batch-1 decode GEMV:  y[n] = sum_k W[n,k] * x[k]  over 34-byte blocks
+// [u16 f16 scale d][32 x i8], w = q * d  (block layout forward/metal_qwen35.rs:2310-2346,
+// arithmetic of gemv_q8_decode, shaders/qwen35.metal:133-190: per block sum_i f32(q_i) * x_i,
+// then times f32(d), all f32).
+//
+// Same work layout as the Q4 kernel: lane l owns block 64 s + l of every row its wave
+// processes, so a wave reads 2176 contiguous bytes per row and slab (blocks are only 2-byte
+// aligned; the vector memory path takes unaligned 16-byte loads).  The activations stay f32:
+// they are staged once per workgroup in LDS (36 dwords per block: 32 values, their sum, pad)
+// and a lane's 32 values serve all rows of a chunk.  Bytes are converted with the unsigned
+// byte-to-float instruction after flipping the sign bits (q ^ 0x80 = q + 128), and the offset
+// is taken out per block with the staged sum:  sum q x = sum (q + 128) x - 128 sum x.
+// Waves are persistent over chunks of RW rows; the next unit's blocks are in flight while the
+// current one is consumed.
+#include "lq4_internal.hpp"
+
+namespace lq4 {
+
+namespace {
+
+constexpr int kWaves = 4;
+constexpr int kXPitch = 36;  // dwords of LDS per block of x (16-byte lane reads at stride 144 B are conflict-free)
+constexpr int kQ8BlockBytes = 34;
+
+struct __attribute__((packed, aligned(2))) Q8BlockRaw {
+    uint16_t d;     // f16 scale
+    uint32_t q[8];  // 32 x i8, weight i in byte i
+};
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+    const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false);
+    return v + __builtin_bit_cast(float, moved);
+}
+
+// sum_i (q_i + 128) * x_i over one block
+__device__ __forceinline__ float block_dot(const uint32_t (&q)[8], const float (&xv)[32]) {
+    float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t u = q[j] ^ 0x80808080u;
+        s0 = fmaf(static_cast<float>(u & 0xffu), xv[4 * j + 0], s0);
+        s1 = fmaf(static_cast<float>((u >> 8) & 0xffu), xv[4 * j + 1], s1);
+        s0 = fmaf(static_cast<float>((u >> 16) & 0xffu), xv[4 * j + 2], s0);
+        s1 = fmaf(static_cast<float>(u >> 24), xv[4 * j + 3], s1);
+    }
+    return s0 + s1;
+}
+
+// Chunk c of wave `wid` holds rows (c * RW + j) * n_waves + wid, j < RW; a unit is one
+// (chunk, slab of 64 blocks).  Dynamic LDS: (K/32) * kXPitch dwords.
+template <int RW>
+__global__ __launch_bounds__(kWaves * 64) void gemv_q8_b1(const uint8_t* __restrict__ w, uint32_t n, uint32_t k,
+                                                          const float* __restrict__ x, float* __restrict__ y) {
+    extern __shared__ __attribute__((aligned(16))) float xs[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const uint32_t nb = k / kBlockWeights;
+    const size_t row_bytes = static_cast<size_t>(nb) * kQ8BlockBytes;
+    const uint32_t slabs = (nb + 63) / 64;
+    const uint32_t n_waves = gridDim.x * kWaves;
+    const uint32_t wid = __builtin_amdgcn_readfirstlane(blockIdx.x * kWaves + (tid >> 6));
+    const uint32_t first = wid < n ? n - wid : 0;
+    const uint32_t chunks = (first + n_waves * RW - 1) / (n_waves * RW);
+    const uint32_t units = chunks * slabs;
+
+    auto load_unit = [&](Q8BlockRaw (&buf)[RW], uint32_t u) {
+        const uint32_t chunk = u / slabs, slab = u - chunk * slabs;
+        uint32_t blk = slab * 64 + lane;
+        if (blk >= nb) blk = nb - 1;
+#pragma unroll
+        for (int j = 0; j < RW; ++j) {
+            uint32_t row = (chunk * RW + j) * n_waves + wid;
+            if (row >= n) row = n - 1;
+            buf[j] = *reinterpret_cast<const Q8BlockRaw*>(w + row * row_bytes + blk * static_cast<uint32_t>(kQ8BlockBytes));
+        }
+    };
+
+    Q8BlockRaw buf_a[RW], buf_b[RW];
+    if (units) load_unit(buf_a, 0);
+
+    // ---- stage x: thread g handles 8 activations of block g / 4 -----------------------------
+    for (uint32_t g = tid; g < nb * 4; g += kWaves * 64) {
+        const uint32_t blk = g >> 2, j = g & 3;
+        const float4* xp = reinterpret_cast<const float4*>(x + blk * kBlockWeights + j * 8);
+        const float4 a = xp[0], b = xp[1];
+        float sx = ((a.x + a.y) + (a.z + a.w)) + ((b.x + b.y) + (b.z + b.w));
+        sx = dpp_add<0xB1>(sx);  // the 4 threads of a block are 4 adjacent lanes: quad butterfly
+        sx = dpp_add<0x4E>(sx);
+        float4* dst = reinterpret_cast<float4*>(&xs[blk * kXPitch + 8 * j]);
+        dst[0] = a;
+        dst[1] = b;
+        if (j == 0) xs[blk * kXPitch + 32] = sx;
+    }
+    __syncthreads();
+
+    float acc[RW];
+#pragma unroll
+    for (int j = 0; j < RW; ++j) acc[j] = 0.0f;
+
+    auto process = [&](Q8BlockRaw (&cur)[RW], Q8BlockRaw (&nxt)[RW], uint32_t u) {
+        const uint32_t chunk = u / slabs, slab = u - chunk * slabs;
+        if (u + 1 < units) load_unit(nxt, u + 1);
+        const uint32_t blk_raw = slab * 64 + lane;
+        const bool live = blk_raw < nb;
+        const uint32_t blk = live ? blk_raw : nb - 1;
+        float xv[32];
+        const float4* xsrc = reinterpret_cast<const float4*>(&xs[blk * kXPitch]);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float4 v = xsrc[i];
+            xv[4 * i + 0] = v.x; xv[4 * i + 1] = v.y; xv[4 * i + 2] = v.z; xv[4 * i + 3] = v.w;
+        }
+        const float sum_x = xs[blk * kXPitch + 32];
+#pragma unroll
+        for (int j = 0; j < RW; ++j) {
+            const float p = block_dot(cur[j].q, xv) - 128.0f * sum_x;
+            const float d = live ? f16_bits_to_f32(cur[j].d) : 0.0f;
+            acc[j] = fmaf(d, p, acc[j]);
+        }
+        if (slab + 1 == slabs) {  // chunk complete
+#pragma unroll
+            for (int j = 0; j < RW; ++j) {
+                const uint32_t row = (chunk * RW + j) * n_waves + wid;
+                const float v = wave_sum(acc[j]);
+                acc[j] = 0.0f;
+                if (lane == 0 && row < n) y[row] = v;
+            }
+        }
+    };
+
+    for (uint32_t u = 0; u < units; u += 2) {
+        process(buf_a, buf_b, u);
+        if (u + 1 < units) process(buf_b, buf_a, u + 1);
+    }
+}
+
+template <int RW>
+void launch_rw(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, size_t lds, uint32_t waves,
+               hipStream_t stream) {
+    static bool attr_set = false;
+    if (!attr_set) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q8_b1<RW>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((gemv_q8_b1<RW>), dim3((waves + kWaves - 1) / kWaves), dim3(kWaves * 64), lds, stream, w, n, k,
+                       x, y);
+}
+
+}  // namespace
+
+size_t gemv_q8_lds_bytes(uint32_t k) { return static_cast<size_t>(k / kBlockWeights) * kXPitch * 4; }
+
+void launch_gemv_q8_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, hipStream_t stream) {
+    const size_t lds = gemv_q8_lds_bytes(k);
+    uint32_t wg_per_cu = static_cast<uint32_t>((160 * 1024) / (lds + 512));
+    wg_per_cu = wg_per_cu > 4 ? 4 : wg_per_cu < 1 ? 1 : wg_per_cu;
+    const uint32_t max_waves = 256 * wg_per_cu * kWaves;
+    uint32_t rw = (n + max_waves - 1) / max_waves;
+    uint32_t waves;
+    if (rw <= 4) {
+        waves = (n + rw - 1) / rw;  // every wave resident, one chunk each
+    } else {
+        waves = max_waves;          // persistent waves over many chunks
+        rw = 2;
+    }
+    switch (rw) {
+        case 1: launch_rw<1>(w, n, k, x, y, lds, waves, stream); break;
+        case 2: launch_rw<2>(w, n, k, x, y, lds, waves, stream); break;
+        case 3: launch_rw<3>(w, n, k, x, y, lds, waves, stream); break;
+        default: launch_rw<4>(w, n, k, x, y, lds, waves, stream); break;
+    }
+}
+
+}  // namespace lq4

@@ -88,6 +88,14 @@ def lib() -> C.CDLL:
         fn.restype = C.c_int
         fn.argtypes = [_u8p, _u8p, C.c_int, C.c_int, C.c_int, _f32p, C.c_int, _i32p, _f32p,
                        C.c_int, outp]
+    L.lq4o_q8_quantize_row.restype = C.c_long
+    L.lq4o_q8_quantize_row.argtypes = [_f32p, C.c_size_t, _u8p]
+    L.lq4o_q8_dequantize.restype = C.c_size_t
+    L.lq4o_q8_dequantize.argtypes = [_u8p, C.c_size_t, _f32p]
+    L.lq4o_q8_gemm_f32.restype = C.c_int
+    L.lq4o_q8_gemm_f32.argtypes = [_f32p, _u8p, _f32p, C.c_size_t, C.c_size_t, C.c_size_t]
+    L.lq4o_q8_gemm_f64.restype = C.c_int
+    L.lq4o_q8_gemm_f64.argtypes = [_f32p, _u8p, _f64p, C.c_size_t, C.c_size_t, C.c_size_t]
     L.lq4o_shifted_rms_norm.restype = None
     L.lq4o_shifted_rms_norm.argtypes = [_f32p, _f32p, C.c_size_t, C.c_size_t, C.c_float]
     L.lq4o_residual_add_norm.restype = None
@@ -322,6 +330,48 @@ Q4_FILE_ERRORS = {1: "invalid magic: not a .q4 file", 2: "legacy .q4 file (v1)",
                   5: "file truncated below Q4 block payload",
                   6: "file has trailing bytes after Q4 block payload",
                   7: "original_len does not match shape"}
+
+
+def q8_quantize_rows(src) -> np.ndarray:
+    """Q8_0 blocks (34 bytes per 32 weights) of every row of src [rows, k]
+    (quantize_row_q8_0, forward/metal_qwen35.rs:2323-2346); ValueError on a non-finite value."""
+    src = _f32(src)
+    rows = src.reshape(-1, src.shape[-1])
+    k = rows.shape[1]
+    assert k % 32 == 0
+    out = np.empty((rows.shape[0], (k // 32) * 34), dtype=np.uint8)
+    for r in range(rows.shape[0]):
+        rc = lib().lq4o_q8_quantize_row(_p(rows[r], _f32p), k, _p(out[r], _u8p))
+        if rc != 0:
+            raise ValueError(f"Q8_0 weight block {-rc - 1} of row {r} contains a non-finite value")
+    return out.reshape(-1)
+
+
+def q8_dequantize(data, n_weights: int) -> np.ndarray:
+    data = _u8(data)
+    assert data.size >= (n_weights // 32) * 34
+    out = np.empty(n_weights, dtype=np.float32)
+    lib().lq4o_q8_dequantize(_p(data, _u8p), n_weights, _p(out, _f32p))
+    return out
+
+
+def q8_gemm_f32(x, wq, n: int, k: int) -> np.ndarray:
+    x, wq = _f32(x), _u8(wq)
+    m = x.size // k
+    assert wq.size >= n * (k // 32) * 34
+    y = np.empty((m, n), dtype=np.float32)
+    rc = lib().lq4o_q8_gemm_f32(_p(x, _f32p), _p(wq, _u8p), _p(y, _f32p), m, n, k)
+    assert rc == 0, rc
+    return y
+
+
+def q8_gemm_f64(x, wq, n: int, k: int) -> np.ndarray:
+    x, wq = _f32(x), _u8(wq)
+    m = x.size // k
+    y = np.empty((m, n), dtype=np.float64)
+    rc = lib().lq4o_q8_gemm_f64(_p(x, _f32p), _p(wq, _u8p), _p(y, _f64p), m, n, k)
+    assert rc == 0, rc
+    return y
 
 
 def shifted_rms_norm(x, gamma, eps: float) -> np.ndarray:

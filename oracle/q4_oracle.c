@@ -565,6 +565,90 @@ int lq4o_parse_q4_file(const uint8_t* file, size_t file_len, uint64_t* shape, in
     return 0;
 }
 
+/* ---- Q8_0 sibling format -------------------------------------------------------------
+ * Block = [u16 f16 scale d, little endian][32 x i8], 34 bytes, 32 weights; w = q * f16(d).
+ * quantize_row_q8_0 (forward/metal_qwen35.rs:2323-2346): per block amax = max|v|, d = amax / 127,
+ * id = 1 / d (0 if d == 0), q = clamp(round(v * id), -127, 127) with round-half-away-from-zero;
+ * the stored scale is f16(d) while the quotient uses the f32 d.  Returns 0, or -(1 + index of the
+ * first block holding a non-finite value): the reference rejects such rows. */
+#define LQ8_BLOCK_BYTES 34
+long lq4o_q8_quantize_row(const float* src, size_t len, uint8_t* out) {
+    if (len % 32 != 0) return -1;
+    for (size_t b = 0; b < len / 32; ++b) {
+        const float* blk = src + b * 32;
+        float amax = 0.0f;
+        for (int i = 0; i < 32; ++i) {
+            if (!isfinite(blk[i])) return -(long)(1 + b);
+            const float a = fabsf(blk[i]);
+            if (a > amax) amax = a;
+        }
+        const float d = amax / 127.0f;
+        const float id = d != 0.0f ? 1.0f / d : 0.0f;
+        const uint16_t bits = lq4o_f32_to_f16(d);
+        uint8_t* o = out + b * LQ8_BLOCK_BYTES;
+        o[0] = (uint8_t)(bits & 0xff);
+        o[1] = (uint8_t)(bits >> 8);
+        for (int i = 0; i < 32; ++i) {
+            float r = roundf(blk[i] * id);
+            if (r < -127.0f) r = -127.0f;
+            if (r > 127.0f) r = 127.0f;
+            o[2 + i] = (uint8_t)(int8_t)r;
+        }
+    }
+    return 0;
+}
+
+/* The dequantisation the reference's Q8_0 tests use as ground truth
+ * (forward/metal_qwen35.rs:23255-23262): f32(i8) * f32(f16 scale). */
+size_t lq4o_q8_dequantize(const uint8_t* data, size_t n_weights, float* out) {
+    const size_t nb = n_weights / 32;
+    for (size_t b = 0; b < nb; ++b) {
+        const uint8_t* blk = data + b * LQ8_BLOCK_BYTES;
+        const float d = lq4o_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+        for (int i = 0; i < 32; ++i) out[b * 32 + i] = (float)(int8_t)blk[2 + i] * d;
+    }
+    return nb * 32;
+}
+
+/* Y[M,N] = X[M,K] . W_q8[N,K]^T in the arithmetic of gemv_q8_decode (shaders/qwen35.metal:133-190):
+ * per block sumq = sum_i f32(q_i) * x_i, y += sumq * f32(d); blocks in ascending order, f32. */
+int lq4o_q8_gemm_f32(const float* x, const uint8_t* wq, float* y, size_t m, size_t n, size_t k) {
+    if (k == 0 || k % 32 != 0) return 1;
+    const size_t nb = k / 32, row_bytes = nb * LQ8_BLOCK_BYTES;
+    for (size_t ni = 0; ni < n; ++ni)
+        for (size_t mi = 0; mi < m; ++mi) {
+            const float* xr = x + mi * k;
+            float acc = 0.0f;
+            for (size_t b = 0; b < nb; ++b) {
+                const uint8_t* blk = wq + ni * row_bytes + b * LQ8_BLOCK_BYTES;
+                const float d = lq4o_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+                float sumq = 0.0f;
+                for (int i = 0; i < 32; ++i) sumq += (float)(int8_t)blk[2 + i] * xr[b * 32 + i];
+                acc += sumq * d;
+            }
+            y[mi * n + ni] = acc;
+        }
+    return 0;
+}
+
+/* The same contraction over the dequantised weights in f64. */
+int lq4o_q8_gemm_f64(const float* x, const uint8_t* wq, double* y, size_t m, size_t n, size_t k) {
+    if (k == 0 || k % 32 != 0) return 1;
+    const size_t nb = k / 32, row_bytes = nb * LQ8_BLOCK_BYTES;
+    for (size_t ni = 0; ni < n; ++ni)
+        for (size_t mi = 0; mi < m; ++mi) {
+            const float* xr = x + mi * k;
+            double acc = 0.0;
+            for (size_t b = 0; b < nb; ++b) {
+                const uint8_t* blk = wq + ni * row_bytes + b * LQ8_BLOCK_BYTES;
+                const double d = (double)lq4o_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+                for (int i = 0; i < 32; ++i) acc += (double)(int8_t)blk[2 + i] * d * (double)xr[b * 32 + i];
+            }
+            y[mi * n + ni] = acc;
+        }
+    return 0;
+}
+
 /* ---- elementwise steps either side of the decode GEMVs ---------------------------------
  * Shifted RMSNorm of Qwen3.5, qwen35_rms_norm (crates/inference/src/model/qwen35/norm.rs:6-23):
  * per row a sequential f32 sum of squares, rms = sqrt(sum / hidden + eps), inv = 1 / rms,

@@ -63,6 +63,18 @@ def device_q8_weight(torch, n, k, gen):
     return blocks.view(-1)
 
 
+def device_q3_weight(torch, n, k, gen):
+    """Synthetic Q3 blocks generated on the device: f16 scale |N(0,0.02)|/3.5, bias -4*scale,
+    uniform plane bits."""
+    nb = n * (k // 32)
+    s = (torch.randn(nb, device="cuda", generator=gen).abs() * (0.02 / 3.5)).clamp_min(6.2e-5)
+    blocks = torch.empty((nb, 16), dtype=torch.uint8, device="cuda")
+    blocks[:, 0:2] = s.to(torch.float16).view(torch.uint8).view(nb, 2)
+    blocks[:, 2:4] = (-4.0 * s).to(torch.float16).view(torch.uint8).view(nb, 2)
+    blocks[:, 4:] = torch.randint(0, 256, (nb, 12), dtype=torch.uint8, device="cuda", generator=gen)
+    return blocks.view(-1)
+
+
 def timed(torch, fn, iters):
     """Average milliseconds per call of fn over `iters` back-to-back calls (HIP events on the
     current stream, which is the stream every launch goes to)."""
@@ -265,28 +277,31 @@ def main():
             del pool
         out["gemv_shapes_batch%d" % B] = shapes
 
-        # Q8_0 sibling format, batch 1: the MLP matrices of the decode layer and the lm_head
+        # sibling formats, batch 1: the MLP matrices of the decode layer and the lm_head
         if B == 1:
-            q8 = {}
-            for name, n, k in [("gate_up", 12288, 2048), ("down", 2048, 6144), ("27b_up", 17408, 5120),
-                               ("lm_head", 248320, 2048)]:
-                wbytes = n * (k // 32) * 34
-                pool = [be.wrap_device_blocks(device_q8_weight(torch, n, k, gen))
-                        for _ in range(max(2, min(200, int(1.1e9 // wbytes))))]
-                x = torch.randn((1, k), device="cuda", generator=gen)
-                y = torch.empty((1, n), device="cuda")
-                f = lambda i, pool=pool, x=x, y=y, n=n, k=k: be.dispatch_matmul_q8(x, pool[i % len(pool)], y, 1, n, k)
-                pr = lambda i, pool=pool: be.probe_read(pool[i % len(pool)]._keepalive[:len(pool[0]._keepalive) // 16 * 16])
-                for i in range(len(pool)):
-                    f(i)
-                reps = max(4 * len(pool), 100) if wbytes < 3e7 else 2 * len(pool)
-                cold, pcold = tm(torch, f, reps), tm(torch, pr, reps)
-                by = wbytes + 4 * k + 4 * n
-                q8[name] = {"n": n, "k": k, "bytes": by, "cold_us": round(cold * 1e3, 3),
-                            "cold_GB/s": round(by / cold / 1e6, 1), "read_probe_cold_us": round(pcold * 1e3, 3),
-                            "gemv_vs_probe": round(pcold / cold, 3)}
-                del pool
-            out["q8_0_gemv_batch1"] = q8
+            for fmt, block_bytes, make, call in (("q8_0", 34, device_q8_weight, be.dispatch_matmul_q8),
+                                                 ("q3", 16, device_q3_weight, be.dispatch_matmul_q3)):
+                res = {}
+                for name, n, k in [("gate_up", 12288, 2048), ("down", 2048, 6144), ("27b_up", 17408, 5120),
+                                   ("lm_head", 248320, 2048)]:
+                    wbytes = n * (k // 32) * block_bytes
+                    pool = [be.wrap_device_blocks(make(torch, n, k, gen))
+                            for _ in range(max(2, min(200, int(1.1e9 // wbytes))))]
+                    x = torch.randn((1, k), device="cuda", generator=gen)
+                    y = torch.empty((1, n), device="cuda")
+                    f = lambda i, pool=pool, x=x, y=y, n=n, k=k, call=call: call(x, pool[i % len(pool)], y, 1, n, k)
+                    pr = lambda i, pool=pool: be.probe_read(
+                        pool[i % len(pool)]._keepalive[:len(pool[0]._keepalive) // 16 * 16])
+                    for i in range(len(pool)):
+                        f(i)
+                    reps = max(4 * len(pool), 100) if wbytes < 3e7 else 2 * len(pool)
+                    cold, pcold = tm(torch, f, reps), tm(torch, pr, reps)
+                    by = wbytes + 4 * k + 4 * n
+                    res[name] = {"n": n, "k": k, "bytes": by, "cold_us": round(cold * 1e3, 3),
+                                 "cold_GB/s": round(by / cold / 1e6, 1),
+                                 "read_probe_cold_us": round(pcold * 1e3, 3), "gemv_vs_probe": round(pcold / cold, 3)}
+                    del pool
+                out[fmt + "_gemv_batch1"] = res
 
         if B == 1:
             x8 = {k: torch.randn((8, k), device="cuda", generator=gen) for k in (2048, 6144)}

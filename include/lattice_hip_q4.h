@@ -237,6 +237,17 @@ int lq4_gemv_q8(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
 int lq4_gemm_q8(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
                 const void* x_dev, int x_dtype, uint32_t m, float* y_dev, void* stream);
 
+/* ---- Q3 sibling format --------------------------------------------------------------
+ * 16-byte blocks [u16 f16 scale][u16 f16 bias][8 bytes low-2-bit plane][4 bytes high-1-bit
+ * plane], w = (low2 | hi << 2) * scale + bias, rows of K/32 blocks, 4-byte aligned
+ * (weights/q3_weights.rs:13-52).  Upload with lq4_weight_upload(..., validate = 0) or wrap.
+ * lq4_gemv_q3 / lq4_gemm_q3 replace dispatch_matmul_q3 / dispatch_gemm_q3
+ * (inner/dispatch.rs:269-325): same conventions as the Q8_0 pair above. */
+int lq4_gemv_q3(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
+                const float* x_dev, uint32_t batch, float* y_dev, void* stream);
+int lq4_gemm_q3(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
+                const void* x_dev, int x_dtype, uint32_t m, float* y_dev, void* stream);
+
 /* ---- probes --------------------------------------------------------------------
  * Writes f32(nibble)*scale + bias for every weight of W[N,K] to out_dev (f32 [N,K]):
  * the bit-exactness probe for nibble unpack and scale/bias indexing against

@@ -51,7 +51,7 @@ EXPORTS = [
     "lq4_probe_copy",
     "lq4_set_gemm_kernel",
     "lq4_residual_add_rmsnorm", "lq4_silu_mul", "lq4_add_and_copy", "lq4_gemv_fused",
-    "lq4_gemv_q8", "lq4_gemm_q8",
+    "lq4_gemv_q8", "lq4_gemm_q8", "lq4_gemv_q3", "lq4_gemm_q3",
     "lq4_get_path_counters", "lq4_malloc", "lq4_free", "lq4_memcpy_h2d", "lq4_memcpy_d2h",
 ]
 
@@ -128,6 +128,8 @@ def load_library() -> C.CDLL:
         "lq4_add_and_copy": (C.c_int, [vp, vp, vp, vp, C.c_size_t, vp]),
         "lq4_gemv_q8": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, C.c_uint32, vp, vp]),
         "lq4_gemm_q8": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, C.c_int, C.c_uint32, vp, vp]),
+        "lq4_gemv_q3": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, C.c_uint32, vp, vp]),
+        "lq4_gemm_q3": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, C.c_int, C.c_uint32, vp, vp]),
         "lq4_gemv_fused": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, vp, C.POINTER(GemvFusion), vp,
                                      C.c_float, vp]),
         "lq4_get_path_counters": (C.c_int, [vp, C.POINTER(PathCounters)]),
@@ -334,6 +336,27 @@ class HipQ4Backend:
         self._assert_k(k, "dispatch_gemm_q8")
         dt = _dtype_code(x)
         _check(self.lib.lq4_gemm_q8(self.ctx, qw.handle, 0, n, k, x.data_ptr() + x_offset, dt, m,
+                                    y.data_ptr() + y_offset, self._stream()))
+
+    # ---- Q3 sibling format --------------------------------------------------------------------
+    def upload_q3_blocks(self, blocks, payload_offset: int = 0) -> Q4WeightBuf:
+        """Uploads Q3 blocks (16 bytes per 32 weights, weights/q3_weights.rs:13-52)."""
+        return self.upload_q4_blocks(blocks, payload_offset=payload_offset, validate=False)
+
+    def dispatch_matmul_q3(self, x, qw: Q4WeightBuf, y, m: int, n: int, k: int):
+        """Decode GEMV over Q3 blocks (the ``m <= 1`` arm of ``dispatch_gemm_q3``, dispatch.rs:269-325)."""
+        if n == 0:
+            return
+        self._assert_k(k, "dispatch_gemm_q3")
+        _check(self.lib.lq4_gemv_q3(self.ctx, qw.handle, 0, n, k, x.data_ptr(), 1, y.data_ptr(), self._stream()))
+
+    def dispatch_gemm_q3(self, x, x_offset: int, qw: Q4WeightBuf, y, y_offset: int, m: int, n: int, k: int):
+        """``dispatch_gemm_q3`` (dispatch.rs:269-325): byte offsets into x and y; ``m == 0 or n == 0``
+        is a no-op; ``m <= 1`` takes the GEMV."""
+        if m == 0 or n == 0:
+            return
+        self._assert_k(k, "dispatch_gemm_q3")
+        _check(self.lib.lq4_gemm_q3(self.ctx, qw.handle, 0, n, k, x.data_ptr() + x_offset, _dtype_code(x), m,
                                     y.data_ptr() + y_offset, self._stream()))
 
     # ---- elementwise steps either side of the decode GEMVs -----------------------------------

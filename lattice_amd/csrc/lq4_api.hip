@@ -100,20 +100,26 @@ int resolve_weight(const lq4_weight* w, uint64_t extra, uint32_t n, uint32_t k,
     return LQ4_OK;
 }
 
-// The same for a buffer of Q8_0 blocks (34 bytes each, 2-byte aligned).
-int resolve_weight_q8(const lq4_weight* w, uint64_t extra, uint32_t n, uint32_t k, const uint8_t** out) {
+// The same for a buffer of sibling-format blocks: Q8_0 (34 bytes, 2-byte aligned) or Q3 (16 bytes,
+// 4-byte aligned).
+int resolve_weight_sibling(const lq4_weight* w, uint64_t extra, uint32_t n, uint32_t k, const char* fmt,
+                           uint32_t block_bytes, uint32_t align, const uint8_t** out) {
     if (!w) return fail(LQ4_E_INVALID, "weight handle is null");
     if (k == 0 || k % kBlockWeights != 0)
-        return fail(LQ4_E_INVALID, "Q8 matmul requires K to be non-zero and divisible by 32, got %u", k);
-    const uint64_t need = static_cast<uint64_t>(n) * (k / kBlockWeights) * 34;
+        return fail(LQ4_E_INVALID, "%s matmul requires K to be non-zero and divisible by 32, got %u", fmt, k);
+    const uint64_t need = static_cast<uint64_t>(n) * (k / kBlockWeights) * block_bytes;
     const uint64_t start = w->payload_offset + extra;
     if (start > w->nbytes || need > w->nbytes - start)
-        return fail(LQ4_E_INVALID, "Q8 W[%u,%u] at byte %llu needs %llu bytes but the buffer holds %zu", n, k,
+        return fail(LQ4_E_INVALID, "%s W[%u,%u] at byte %llu needs %llu bytes but the buffer holds %zu", fmt, n, k,
                     static_cast<unsigned long long>(start), static_cast<unsigned long long>(need), w->nbytes);
-    if (start % 2 != 0) return fail(LQ4_E_INVALID, "Q8 weight byte offset %llu is not 2-byte aligned",
-                                    static_cast<unsigned long long>(start));
+    if (start % align != 0) return fail(LQ4_E_INVALID, "%s weight byte offset %llu is not %u-byte aligned", fmt,
+                                        static_cast<unsigned long long>(start), align);
     *out = w->base + start;
     return LQ4_OK;
+}
+
+int resolve_weight_q8(const lq4_weight* w, uint64_t extra, uint32_t n, uint32_t k, const uint8_t** out) {
+    return resolve_weight_sibling(w, extra, n, k, "Q8", 34, 2, out);
 }
 
 int resolve_lora(const lq4_ctx* ctx, const lq4_lora* l, float scale, uint32_t n, uint32_t k,
@@ -689,6 +695,37 @@ int lq4_gemv_q8(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
     if (batch > kMaxGemvBatch)
         return fail(LQ4_E_INVALID, "lq4_gemv_q8 batch %u above %d; use lq4_gemm_q8", batch, kMaxGemvBatch);
     return lq4_gemm_q8(ctx, w, w_extra_offset, n, k, x_dev, LQ4_F32, batch, y_dev, stream);
+}
+
+int lq4_gemm_q3(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
+                const void* x_dev, int x_dtype, uint32_t m, float* y_dev, void* stream) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    if (m == 0 || n == 0) return LQ4_OK;
+    if (x_dtype != LQ4_F32 && x_dtype != LQ4_F16) return fail(LQ4_E_INVALID, "x_dtype must be LQ4_F32 or LQ4_F16");
+    const uint8_t* wp;
+    const int rc = resolve_weight_sibling(w, w_extra_offset, n, k, "Q3", 16, 4, &wp);
+    if (rc) return rc;
+    if (!x_dev || !y_dev) return fail(LQ4_E_INVALID, "x/y device pointer is null");
+    if (reinterpret_cast<uintptr_t>(x_dev) % 16) return fail(LQ4_E_INVALID, "x must be 16-byte aligned");
+    if (reinterpret_cast<uintptr_t>(y_dev) % 4) return fail(LQ4_E_INVALID, "y must be 4-byte aligned");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    DeviceGuard g(ctx->device);
+    if (m == 1 && x_dtype == LQ4_F32 && gemv_q3_lds_bytes(k) <= 128 * 1024) {
+        launch_gemv_q3_b1(wp, n, k, static_cast<const float*>(x_dev), y_dev, s);
+        ctx->counters.gemv++;
+    } else {
+        launch_gemm_q3(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, s);
+        ctx->counters.gemm++;
+    }
+    LQ4_HIP(hipGetLastError());
+    return LQ4_OK;
+}
+
+int lq4_gemv_q3(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
+                const float* x_dev, uint32_t batch, float* y_dev, void* stream) {
+    if (batch > kMaxGemvBatch)
+        return fail(LQ4_E_INVALID, "lq4_gemv_q3 batch %u above %d; use lq4_gemm_q3", batch, kMaxGemvBatch);
+    return lq4_gemm_q3(ctx, w, w_extra_offset, n, k, x_dev, LQ4_F32, batch, y_dev, stream);
 }
 
 int lq4_set_gemm_kernel(int which) {

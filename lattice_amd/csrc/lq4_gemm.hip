@@ -89,6 +89,13 @@ struct __attribute__((packed, aligned(2))) Q8BlockRaw {
     uint32_t q[8];  // weight i in byte i
 };
 
+// Q3 sibling format (FMT == 2): 16-byte block [f16 scale][f16 bias][low-2-bit plane][high-1-bit plane].
+struct __attribute__((packed, aligned(4))) Q3BlockRaw {
+    uint32_t sb;
+    uint32_t lo[2];  // weight i of 16-weight half h at bits 2i of lo[h]
+    uint32_t hi;     // weight i at bit i
+};
+
 template <int FMT>
 struct WBlockOf {
     typedef Q4BlockRaw type;
@@ -97,6 +104,27 @@ template <>
 struct WBlockOf<1> {
     typedef Q8BlockRaw type;
 };
+template <>
+struct WBlockOf<2> {
+    typedef Q3BlockRaw type;
+};
+
+// Weights 8j..8j+7 of a Q3 block -> 8 f16 weights half(q * d + b) in memory order, q = low2 | hi << 2.
+__device__ __forceinline__ uint4 dequant8_q3(const Q3BlockRaw& b, int j, half2v d2, half2v b2) {
+    const half2v k1024 = {static_cast<_Float16>(1024.0f), static_cast<_Float16>(1024.0f)};
+    const uint32_t lw = (b.lo[j >> 1] >> (16 * (j & 1))) & 0xffffu;  // 8 two-bit fields
+    const uint32_t hw = (b.hi >> (8 * j)) & 0xffu;                   // 8 bits
+    uint32_t out[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const uint32_t l4 = lw >> (4 * p), h2 = hw >> (2 * p);
+        const uint32_t qa = (l4 & 3u) | ((h2 & 1u) << 2);
+        const uint32_t qb = ((l4 >> 2) & 3u) | ((h2 & 2u) << 1);
+        const half2v q2 = as_h2(0x64006400u | qa | (qb << 16)) - k1024;
+        out[p] = as_u32(__builtin_elementwise_fma(q2, d2, b2));
+    }
+    return make_uint4(out[0], out[1], out[2], out[3]);
+}
 
 // Two packed dwords of a Q8_0 block (weights 8j..8j+7) -> 8 f16 weights half(q * d) in memory
 // order.  A sign-flipped byte (q + 128) placed under the exponent byte of 1024.0 is 1024 + 128 + q
@@ -119,7 +147,7 @@ __device__ __forceinline__ uint4 dequant8_q8(uint32_t qa, uint32_t qb, half2v d2
 // BN_: weight rows per workgroup (128 or 256); 2*BN_ threads; waves in a 2 x (BN_/64) grid.
 // LORA: compiled with the LoRA step (kept out of the plain kernel, whose register allocation it
 // would disturb).
-// FMT: 0 = Q4 blocks, 1 = Q8_0 blocks (no LoRA step).
+// FMT: 0 = Q4 blocks, 1 = Q8_0 blocks, 2 = Q3 blocks (the siblings have no LoRA step).
 template <bool X_F16, int BN_, bool LORA, int FMT = 0>
 __global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
     const uint8_t* __restrict__ w, uint32_t n, uint32_t k, const void* __restrict__ xv, uint32_t m,
@@ -165,7 +193,7 @@ __global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
     typedef typename WBlockOf<FMT>::type WBlock;
     const uint32_t* w_ptr =
         reinterpret_cast<const uint32_t*>(w) + static_cast<size_t>(w_live_row ? w_row : 0) * (nb * 5);
-    const uint8_t* w_ptr8 = w + static_cast<size_t>(w_live_row ? w_row : 0) * (nb * 34);  // FMT == 1
+    const uint8_t* w_ptr8 = w + static_cast<size_t>(w_live_row ? w_row : 0) * (nb * (FMT == 2 ? 16 : 34));  // FMT != 0
     const int w_half = tid & 1;
     // activations: chunk i of this thread is (row, part) = divmod(tid + kThreads*i, chunks per row)
     const uint8_t* x_ptr[XCH];
@@ -201,7 +229,7 @@ __global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
         uint32_t blk = s * 2 + w_half;
         if (blk >= nb) blk = nb - 1;
         if constexpr (FMT == 0) wst = *reinterpret_cast<const WBlock*>(w_ptr + blk * 5);
-        else wst = *reinterpret_cast<const WBlock*>(w_ptr8 + blk * 34);
+        else wst = *reinterpret_cast<const WBlock*>(w_ptr8 + blk * (FMT == 2 ? 16 : 34));
     };
 
     auto store_tiles = [&](const XStage& st, const WBlock& wst, uint32_t s, _Float16* xs, _Float16* ws) {
@@ -229,12 +257,18 @@ __global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 *reinterpret_cast<uint4*>(dst + j * 8) = dequant8(live ? wst.q[j] : 0u, d2, b2);
-        } else {
+        } else if constexpr (FMT == 1) {
             const uint32_t db = live ? wst.d : 0u;
             const half2v d2 = as_h2(db | (db << 16));
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 *reinterpret_cast<uint4*>(dst + j * 8) = dequant8_q8(wst.q[2 * j], wst.q[2 * j + 1], d2);
+        } else {
+            const uint32_t sb = live ? wst.sb : 0u;
+            const half2v d2 = as_h2(__builtin_amdgcn_perm(sb, sb, 0x01000100u));
+            const half2v b2 = as_h2(__builtin_amdgcn_perm(sb, sb, 0x03020302u));
+#pragma unroll
+            for (int j = 0; j < 4; ++j) *reinterpret_cast<uint4*>(dst + j * 8) = dequant8_q3(wst, j, d2, b2);
         }
     };
 
@@ -438,6 +472,13 @@ void launch_gemm_q8(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int
     const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};
     if (x_is_f16) launch_tile<true, 128, false, 1>(w, n, k, x, m, y, none, stream);
     else launch_tile<false, 128, false, 1>(w, n, k, x, m, y, none, stream);
+}
+
+void launch_gemm_q3(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
+                    hipStream_t stream) {
+    const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};
+    if (x_is_f16) launch_tile<true, 128, false, 2>(w, n, k, x, m, y, none, stream);
+    else launch_tile<false, 128, false, 2>(w, n, k, x, m, y, none, stream);
 }
 
 }  // namespace lq4

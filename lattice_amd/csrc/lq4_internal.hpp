@@ -111,6 +111,12 @@ void launch_gemv_q8_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x,
 void launch_gemm_q8(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
                     hipStream_t stream);
 
+// Q3 sibling format (16-byte blocks: f16 scale, f16 bias, 2-bit and 1-bit planes): same pair of paths.
+size_t gemv_q3_lds_bytes(uint32_t k);
+void launch_gemv_q3_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, hipStream_t stream);
+void launch_gemm_q3(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
+                    hipStream_t stream);
+
 void launch_probe_read(const void* p, size_t nbytes, uint32_t* sink, hipStream_t stream);
 void launch_probe_copy(const void* src, void* dst, size_t nbytes, hipStream_t stream);
 void launch_dequant(const uint8_t* w, uint32_t n, uint32_t k, float* out, hipStream_t stream);

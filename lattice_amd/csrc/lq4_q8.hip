@@ -27,10 +27,21 @@ struct __attribute__((packed, aligned(2))) Q8BlockRaw {
     uint32_t q[8];  // 32 x i8, weight i in byte i
 };
 
-template <int CTRL>
+template <int CTRL, int ROW_MASK = 0xF>
 __device__ __forceinline__ float dpp_add(float v) {
-    const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false);
+    const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, false);
     return v + __builtin_bit_cast(float, moved);
+}
+
+// Sum over the 64 lanes of a wave with data-parallel-primitive moves only; valid in lane 63.
+__device__ __forceinline__ float wave_total(float v) {
+    v = dpp_add<0xB1>(v);        // quad_perm [1,0,3,2]
+    v = dpp_add<0x4E>(v);        // quad_perm [2,3,0,1]
+    v = dpp_add<0x141>(v);       // row_half_mirror
+    v = dpp_add<0x140>(v);       // row_mirror: every lane holds its 16-lane row sum
+    v = dpp_add<0x142, 0xA>(v);  // row_bcast:15 into rows 1 and 3
+    v = dpp_add<0x143, 0xC>(v);  // row_bcast:31 into rows 2 and 3
+    return v;
 }
 
 // sum_i (q_i + 128) * x_i over one block
@@ -122,9 +133,9 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q8_b1(const uint8_t* __restr
 #pragma unroll
             for (int j = 0; j < RW; ++j) {
                 const uint32_t row = (chunk * RW + j) * n_waves + wid;
-                const float v = wave_sum(acc[j]);
+                const float v = wave_total(acc[j]);
                 acc[j] = 0.0f;
-                if (lane == 0 && row < n) y[row] = v;
+                if (lane == 63 && row < n) y[row] = v;
             }
         }
     };

@@ -88,6 +88,16 @@ def lib() -> C.CDLL:
         fn.restype = C.c_int
         fn.argtypes = [_u8p, _u8p, C.c_int, C.c_int, C.c_int, _f32p, C.c_int, _i32p, _f32p,
                        C.c_int, outp]
+    L.lq4o_q3_quantize_block.restype = C.c_int
+    L.lq4o_q3_quantize_block.argtypes = [_f32p, C.c_int, C.c_int, _u8p]
+    L.lq4o_q3_quantize_row.restype = C.c_int
+    L.lq4o_q3_quantize_row.argtypes = [_f32p, C.c_size_t, C.c_int, _u8p]
+    L.lq4o_q3_dequantize.restype = C.c_size_t
+    L.lq4o_q3_dequantize.argtypes = [_u8p, C.c_size_t, C.c_size_t, _f32p]
+    L.lq4o_q3_gemm_f32.restype = C.c_int
+    L.lq4o_q3_gemm_f32.argtypes = [_f32p, _u8p, _f32p, C.c_size_t, C.c_size_t, C.c_size_t]
+    L.lq4o_q3_gemm_f64.restype = C.c_int
+    L.lq4o_q3_gemm_f64.argtypes = [_f32p, _u8p, _f64p, C.c_size_t, C.c_size_t, C.c_size_t]
     L.lq4o_q8_quantize_row.restype = C.c_long
     L.lq4o_q8_quantize_row.argtypes = [_f32p, C.c_size_t, _u8p]
     L.lq4o_q8_dequantize.restype = C.c_size_t
@@ -330,6 +340,58 @@ Q4_FILE_ERRORS = {1: "invalid magic: not a .q4 file", 2: "legacy .q4 file (v1)",
                   5: "file truncated below Q4 block payload",
                   6: "file has trailing bytes after Q4 block payload",
                   7: "original_len does not match shape"}
+
+
+def q3_quantize_block(vals, valid_len: int = 32, symmetric: bool = False) -> bytes:
+    """One 16-byte Q3 block (quantize_block_with_mode_len, weights/q3_weights.rs:199-262)."""
+    v = np.zeros(32, dtype=np.float32)
+    vals = _f32(vals).reshape(-1)
+    v[:vals.size] = vals
+    out = np.empty(16, dtype=np.uint8)
+    rc = lib().lq4o_q3_quantize_block(_p(v, _f32p), valid_len, int(symmetric), _p(out, _u8p))
+    if rc:
+        raise ValueError("Q3 weight block: bad valid_len" if rc == 1 else "Q3 weight block contains a non-finite value")
+    return out.tobytes()
+
+
+def q3_quantize_rows(src, symmetric: bool = False) -> np.ndarray:
+    """Q3 blocks of every row of src [rows, cols] (quantize_tensor_q3_0, q3_weights.rs:321-345);
+    a row whose length is not a multiple of 32 ends in a zero-padded block."""
+    src = _f32(src)
+    rows = src.reshape(-1, src.shape[-1])
+    nb = (rows.shape[1] + 31) // 32
+    out = np.empty((rows.shape[0], nb * 16), dtype=np.uint8)
+    for r in range(rows.shape[0]):
+        rc = lib().lq4o_q3_quantize_row(_p(rows[r], _f32p), rows.shape[1], int(symmetric), _p(out[r], _u8p))
+        if rc:
+            raise ValueError("Q3 weight block contains a non-finite value")
+    return out.reshape(-1)
+
+
+def q3_dequantize(data, n_weights: int) -> np.ndarray:
+    data = _u8(data)
+    out = np.empty(n_weights, dtype=np.float32)
+    done = lib().lq4o_q3_dequantize(_p(data, _u8p), data.size, n_weights, _p(out, _f32p))
+    return out[:done]
+
+
+def q3_gemm_f32(x, wq, n: int, k: int) -> np.ndarray:
+    x, wq = _f32(x), _u8(wq)
+    m = x.size // k
+    assert wq.size >= n * (k // 32) * 16
+    y = np.empty((m, n), dtype=np.float32)
+    rc = lib().lq4o_q3_gemm_f32(_p(x, _f32p), _p(wq, _u8p), _p(y, _f32p), m, n, k)
+    assert rc == 0, rc
+    return y
+
+
+def q3_gemm_f64(x, wq, n: int, k: int) -> np.ndarray:
+    x, wq = _f32(x), _u8(wq)
+    m = x.size // k
+    y = np.empty((m, n), dtype=np.float64)
+    rc = lib().lq4o_q3_gemm_f64(_p(x, _f32p), _p(wq, _u8p), _p(y, _f64p), m, n, k)
+    assert rc == 0, rc
+    return y
 
 
 def q8_quantize_rows(src) -> np.ndarray:

@@ -649,6 +649,130 @@ int lq4o_q8_gemm_f64(const float* x, const uint8_t* wq, double* y, size_t m, siz
     return 0;
 }
 
+/* ---- Q3 sibling format ---------------------------------------------------------------
+ * Block = [u16 f16 scale][u16 f16 bias][8 bytes low-2-bit plane][4 bytes high-1-bit plane],
+ * 16 bytes, 32 weights, w = q * scale + bias with q = low2 | hi << 2
+ * (weights/q3_weights.rs:13-52, pack_plane_split :148-167, unpack_plane_split :170-175). */
+#define LQ3_BLOCK_BYTES 16
+static void lq3_pack(const uint8_t q[32], uint8_t packed[12]) {
+    memset(packed, 0, 12);
+    for (int b = 0; b < 8; ++b)
+        packed[b] = (uint8_t)((q[4 * b] & 3) | ((q[4 * b + 1] & 3) << 2) | ((q[4 * b + 2] & 3) << 4) | ((q[4 * b + 3] & 3) << 6));
+    for (int b = 0; b < 4; ++b)
+        for (int k = 0; k < 8; ++k) packed[8 + b] |= (uint8_t)(((q[8 * b + k] >> 2) & 1) << k);
+}
+
+static uint8_t lq3_unpack(const uint8_t* packed, int i) {
+    const uint8_t low2 = (packed[i / 4] >> ((i % 4) * 2)) & 3;
+    const uint8_t hi = (packed[8 + i / 8] >> (i % 8)) & 1;
+    return (uint8_t)(low2 | (hi << 2));
+}
+
+/* quantize_block_with_mode_len (weights/q3_weights.rs:199-262).  Returns 0, 1 for a bad
+ * valid_len, 2 for a non-finite value. */
+int lq4o_q3_quantize_block(const float* vals, int valid_len, int symmetric, uint8_t* out) {
+    if (valid_len < 1 || valid_len > 32) return 1;
+    for (int i = 0; i < 32; ++i)
+        if (!isfinite(vals[i])) return 2;
+    uint8_t q[32];
+    float scale, bias;
+    if (symmetric) {
+        float abs_max = 0.0f;
+        for (int i = 0; i < 32; ++i) abs_max = fmaxf(abs_max, fabsf(vals[i]));
+        scale = abs_max == 0.0f ? 1.0f : abs_max / 3.5f;
+        const float inv = 1.0f / scale;
+        bias = -4.0f * scale;
+        for (int i = 0; i < 32; ++i) {
+            float r = roundf(vals[i] * inv) + 4.0f;
+            r = r < 0.0f ? 0.0f : r > 7.0f ? 7.0f : r;
+            q[i] = (uint8_t)r;
+        }
+    } else {
+        float mn = INFINITY, mx = -INFINITY;
+        for (int i = 0; i < valid_len; ++i) {
+            mn = fminf(mn, vals[i]);
+            mx = fmaxf(mx, vals[i]);
+        }
+        const float range = mx - mn;
+        scale = range == 0.0f ? 1.0f : range / 7.0f;
+        const float inv = 1.0f / scale;
+        bias = mn;
+        for (int i = 0; i < 32; ++i) {
+            float r = roundf((vals[i] - mn) * inv);
+            r = r < 0.0f ? 0.0f : r > 7.0f ? 7.0f : r;
+            q[i] = (uint8_t)r;
+        }
+    }
+    const uint16_t sb = lq4o_f32_to_f16(scale), bb = lq4o_f32_to_f16(bias);
+    out[0] = (uint8_t)(sb & 0xff);
+    out[1] = (uint8_t)(sb >> 8);
+    out[2] = (uint8_t)(bb & 0xff);
+    out[3] = (uint8_t)(bb >> 8);
+    lq3_pack(q, out + 4);
+    return 0;
+}
+
+/* quantize_row_q3_0 (weights/q3_weights.rs:279-299): 32 at a time, zero-padded tail block whose
+ * range comes from the real values only. */
+int lq4o_q3_quantize_row(const float* src, size_t len, int symmetric, uint8_t* out) {
+    for (size_t b = 0; b * 32 < len; ++b) {
+        float vals[32] = {0};
+        const size_t take = len - b * 32 < 32 ? len - b * 32 : 32;
+        memcpy(vals, src + b * 32, take * sizeof(float));
+        const int rc = lq4o_q3_quantize_block(vals, (int)take, symmetric, out + b * LQ3_BLOCK_BYTES);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+/* dequantize_row_q3_0 (weights/q3_weights.rs:306-319). */
+size_t lq4o_q3_dequantize(const uint8_t* data, size_t nbytes, size_t n_weights, float* out) {
+    size_t done = 0;
+    for (size_t b = 0; (b + 1) * LQ3_BLOCK_BYTES <= nbytes && done < n_weights; ++b) {
+        const uint8_t* blk = data + b * LQ3_BLOCK_BYTES;
+        const float scale = lq4o_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+        const float bias = lq4o_f16_to_f32((uint16_t)(blk[2] | (blk[3] << 8)));
+        for (int i = 0; i < 32 && done < n_weights; ++i) out[done++] = (float)lq3_unpack(blk + 4, i) * scale + bias;
+    }
+    return done;
+}
+
+/* gemm_q3_reference / gemv_q3_reference (weights/q3_weights.rs:784-838): dequantise the row, then a
+ * sequential f32 sum of products, k ascending. */
+int lq4o_q3_gemm_f32(const float* x, const uint8_t* wq, float* y, size_t m, size_t n, size_t k) {
+    if (k == 0 || k % 32 != 0) return 1;
+    const size_t row_bytes = (k / 32) * LQ3_BLOCK_BYTES;
+    float* wrow = (float*)malloc(k * sizeof(float));
+    if (!wrow) return 2;
+    for (size_t ni = 0; ni < n; ++ni) {
+        lq4o_q3_dequantize(wq + ni * row_bytes, row_bytes, k, wrow);
+        for (size_t mi = 0; mi < m; ++mi) {
+            float acc = 0.0f;
+            for (size_t ki = 0; ki < k; ++ki) acc += x[mi * k + ki] * wrow[ki];
+            y[mi * n + ni] = acc;
+        }
+    }
+    free(wrow);
+    return 0;
+}
+
+int lq4o_q3_gemm_f64(const float* x, const uint8_t* wq, double* y, size_t m, size_t n, size_t k) {
+    if (k == 0 || k % 32 != 0) return 1;
+    const size_t row_bytes = (k / 32) * LQ3_BLOCK_BYTES;
+    float* wrow = (float*)malloc(k * sizeof(float));
+    if (!wrow) return 2;
+    for (size_t ni = 0; ni < n; ++ni) {
+        lq4o_q3_dequantize(wq + ni * row_bytes, row_bytes, k, wrow);
+        for (size_t mi = 0; mi < m; ++mi) {
+            double acc = 0.0;
+            for (size_t ki = 0; ki < k; ++ki) acc += (double)x[mi * k + ki] * (double)wrow[ki];
+            y[mi * n + ni] = acc;
+        }
+    }
+    free(wrow);
+    return 0;
+}
+
 /* ---- elementwise steps either side of the decode GEMVs ---------------------------------
  * Shifted RMSNorm of Qwen3.5, qwen35_rms_norm (crates/inference/src/model/qwen35/norm.rs:6-23):
  * per row a sequential f32 sum of squares, rms = sqrt(sum / hidden + eps), inv = 1 / rms,

@@ -262,8 +262,9 @@ int lq4_dequant(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
 int lq4_probe_read(lq4_ctx* ctx, const void* p_dev, size_t nbytes, void* stream);
 
 /* Tuning/test hook, process-wide: 0 = lq4_gemm picks its kernel by shape (default), 1 = always
- * the LDS-staged tile kernel, 2 = always the weights-in-registers kernel.  Results are identical in contract either way.  No counterpart
- * in the reference. */
+ * the LDS-staged tile kernel, 2 = always the weights-in-registers kernel, 3 = always the
+ * few-token kernel.  Results are identical in contract either way.  No counterpart in the
+ * reference. */
 int lq4_set_gemm_kernel(int which);
 
 /* Calibration: plain device copy of `nbytes` (both buffers 16-byte aligned, nbytes a multiple

@@ -243,7 +243,8 @@ class HipQ4Backend:
         _check(self.lib.lq4_probe_read(self.ctx, t.data_ptr(), t.numel() * t.element_size(), self._stream()))
 
     def set_gemm_kernel(self, which: int):
-        """0 = pick the prefill kernel by shape, 1 = LDS-staged tile, 2 = weights in registers."""
+        """0 = pick the prefill kernel by shape, 1 = LDS-staged tile, 2 = weights in registers,
+        3 = few-token kernel."""
         _check(self.lib.lq4_set_gemm_kernel(int(which)))
 
     def probe_copy(self, src, dst):

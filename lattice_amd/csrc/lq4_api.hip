@@ -729,7 +729,7 @@ int lq4_gemv_q3(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
 }
 
 int lq4_set_gemm_kernel(int which) {
-    if (which < 0 || which > 2) return fail(LQ4_E_INVALID, "gemm kernel choice must be 0, 1 or 2");
+    if (which < 0 || which > 3) return fail(LQ4_E_INVALID, "gemm kernel choice must be 0, 1, 2 or 3");
     set_gemm_kernel_choice(which);
     return LQ4_OK;
 }

@@ -96,7 +96,8 @@ void launch_gemm(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_
 // gemm_wreg_supports = the kernel can run the shape at all.
 uint32_t gemm_wreg_tiles(uint32_t n, uint32_t m);
 bool gemm_wreg_supports(uint32_t n, uint32_t k, uint32_t m, int x_is_f16);
-// 0 = choose by shape, 1 = LDS-staged kernel, 2 = weights-in-registers kernel where supported.
+// 0 = choose by shape, 1 = LDS-staged kernel, 2 = weights-in-registers kernel where supported,
+// 3 = few-token kernel.
 void set_gemm_kernel_choice(int which);
 // gemm_wreg_slices = K slices it wants for the shape (1 = none); with more than one, `partial`
 // must hold slices * m * n floats.
@@ -116,6 +117,13 @@ size_t gemv_q3_lds_bytes(uint32_t k);
 void launch_gemv_q3_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, hipStream_t stream);
 void launch_gemm_q3(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
                     hipStream_t stream);
+
+// Few-token variant (up to 128 tokens): activations packed once into matrix-core operand order
+// (gemm_skinny_scratch_bytes bytes at `packed_x`), then a kernel without LDS staging.
+bool gemm_skinny_wants(uint32_t n, uint32_t k, uint32_t m);
+size_t gemm_skinny_scratch_bytes(uint32_t k, uint32_t m);
+void launch_gemm_skinny(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
+                        const LoraEpilogue& lora, void* packed_x, hipStream_t stream);
 
 void launch_probe_read(const void* p, size_t nbytes, uint32_t* sink, hipStream_t stream);
 void launch_probe_copy(const void* src, void* dst, size_t nbytes, hipStream_t stream);

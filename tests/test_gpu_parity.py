@@ -440,3 +440,61 @@ def test_gemm_weights_in_registers_kernel_with_lora(be):
         be.set_gemm_kernel(0)
         be.unload_lora_adapter()
     assert rel_err(host(y), _lora_ref(x, wq, n, k, a, b, 2.0)) <= REL_TOL
+
+
+SKINNY_CASES = [(17, 16, 32, "f32"), (64, 2048, 2048, "f32"), (64, 512, 2048, "f16"), (33, 50, 96, "f32"),
+                (100, 130, 416, "f16"), (128, 36, 1024, "f32"), (20, 7, 160, "f32"), (200, 65, 224, "f16"),
+                (48, 8200, 256, "f32"), (64, 16400, 128, "f16")]
+
+
+@pytest.mark.parametrize("m,n,k,xdt", SKINNY_CASES)
+def test_gemm_few_token_kernel_matches_oracle(be, m, n, k, xdt):
+    # the few-token kernel: ragged token groups, N tails (also N % 4 != 0), K tails inside a
+    # 128-wide step, fewer K steps than waves, all three row-tile widths; forced, so M > 128 is
+    # covered too
+    import torch
+    print(f"gemm few-token m={m} n={n} k={k} x={xdt}", flush=True)
+    wq = synth.q4_weight(n, k, seed=8, symmetric_bias=(k != 96))
+    x = synth.activations(m, k, seed=8, dtype=np.float16 if xdt == "f16" else np.float32)
+    qw = be.upload_q4_blocks(wq)
+    y = torch.full((m + 1, n), float("nan"), dtype=torch.float32, device="cuda")
+    be.set_gemm_kernel(3)
+    try:
+        be.dispatch_gemm(dev(x), 0, qw, y, 0, m, n, k)
+    finally:
+        be.set_gemm_kernel(0)
+    got = host(y)
+    assert np.all(np.isnan(got[m])) and np.all(np.isfinite(got[:m]))
+    e = rel_err(got[:m], oracle.gemm_f32(x.astype(np.float32), wq, n, k))
+    print(f"  rel err {e:.2e}", flush=True)
+    assert e <= REL_TOL
+    if m <= 64:  # the shape-based choice takes the same kernel: bit-identical
+        y0 = torch.empty((m, n), dtype=torch.float32, device="cuda")
+        be.dispatch_gemm(dev(x), 0, qw, y0, 0, m, n, k)
+        assert np.array_equal(host(y0), got[:m])
+
+
+@pytest.mark.parametrize("b_f16", [False, True])
+def test_gemm_few_token_kernel_with_lora(be, b_f16):
+    import torch
+    m, n, k, r = 64, 130, 2048, 16
+    wq = synth.q4_weight(n, k, seed=9)
+    x = synth.activations(m, k, seed=9)
+    a, b = synth.lora_pair(r, k, n, seed=9)
+    if b_f16:
+        a, b = a.astype(np.float16), b.astype(np.float16)
+    qw = be.upload_q4_blocks(wq)
+    be.load_lora_adapter([backend.LoraLayerData(0, {"v_proj": (a, b)})], scale=2.0)
+    y = torch.empty((m, n), dtype=torch.float32, device="cuda")
+    y_plain = torch.empty((m, n), dtype=torch.float32, device="cuda")
+    try:
+        be.dispatch_gemm(dev(x), 0, qw, y, 0, m, n, k, layer_idx=0, module="v_proj")
+        be.dispatch_gemm(dev(x), 0, qw, y_plain, 0, m, n, k)
+    finally:
+        be.unload_lora_adapter()
+    a32, b32 = a.astype(np.float32), b.astype(np.float32)
+    assert rel_err(host(y), _lora_ref(x, wq, n, k, a32, b32, 2.0)) <= REL_TOL
+    # the delta alone, against the f64 product
+    delta = host(y).astype(np.float64) - host(y_plain).astype(np.float64)
+    want = 2.0 * (x.astype(np.float64) @ a32.astype(np.float64).T) @ b32.astype(np.float64).T
+    assert rel_err(delta, want) <= REL_TOL

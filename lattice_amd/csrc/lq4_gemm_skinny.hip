@@ -138,9 +138,8 @@ __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __
         Q4BlockRaw wb[RT];
         uint4 x[4][4];  // [token group][instruction]
     };
-    // i-th step of this wave (clamped to its last one, so the buffer can always be refilled)
+    // i-th step of this wave
     auto load = [&](Unit& u, uint32_t i) {
-        i = i < cnt ? i : cnt - 1;
         const uint32_t s = wave + i * kWavesK;
         uint32_t blk = s * 4 + g;
         blk = blk < nb ? blk : nb - 1;
@@ -183,13 +182,13 @@ __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __
     if (cnt) {
         Unit u0, u1;
         load(u0, 0);
-        load(u1, 1);
+        if (cnt > 1) load(u1, 1);
         uint32_t i = 0;
         for (; i + 2 <= cnt; i += 2) {
             compute(u0, i);
-            load(u0, i + 2);
+            if (i + 2 < cnt) load(u0, i + 2);  // never a load nobody consumes: the reduction below waits for all of them
             compute(u1, i + 1);
-            load(u1, i + 3);
+            if (i + 3 < cnt) load(u1, i + 3);
         }
         if (i < cnt) compute(u0, i);
     }

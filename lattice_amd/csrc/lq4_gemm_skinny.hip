@@ -277,9 +277,10 @@ void launch_rt(const uint8_t* w, uint32_t n, uint32_t k, const uint4* xp, uint32
 }  // namespace
 
 bool gemm_skinny_wants(uint32_t n, uint32_t k, uint32_t m) {
-    // one token tile always; two only for narrow outputs, where the large-tile kernels cannot
-    // fill the chip (measured cross-over: equal at N = 12288, ahead below)
-    return k >= kBlockWeights && (m <= kTokens || (m <= 2 * kTokens && n <= 4096));
+    // one token tile always; two while the matrix is small enough that the large-tile kernels cannot
+    // fill the chip (measured: ahead at 12288 x 2048, behind at 17408 x 5120)
+    return k >= kBlockWeights &&
+           (m <= kTokens || (m <= 2 * kTokens && static_cast<uint64_t>(n) * k <= (1ull << 25)));
 }
 
 size_t gemm_skinny_scratch_bytes(uint32_t k, uint32_t m) {

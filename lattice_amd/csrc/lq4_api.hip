@@ -316,8 +316,20 @@ int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
         launch_lora_a(lora->a, lora->is_f16, lora->rank, k, x_dev, 0, k, batch, ctx->lora_t, s);
         ctx->counters.lora_a++;
     }
-    launch_gemv(wp, n, k, x_dev, k, batch, y_dev, n, ep, s);
-    ctx->counters.gemv++;
+    // Above four activation rows the few-token matrix-core kernel (operands packed once, eight K
+    // slices per workgroup) overtakes the 4x4x4 GEMV kernel: always from nine rows; from five for
+    // mid-sized matrices only (measured: behind for 512 x 2048, where its two launches dominate,
+    // and for 12288 x 2048, where the GEMV kernel's grid already fills the chip).
+    const uint64_t weights = static_cast<uint64_t>(n) * k;
+    if ((batch >= 9 || (batch >= 5 && n < 8192 && weights >= 6000000)) && gemm_skinny_wants(n, k, batch)) {
+        rc = ensure_scratch(ctx, gemm_skinny_scratch_bytes(k, batch));
+        if (rc) return rc;
+        launch_gemm_skinny(wp, n, k, x_dev, 0, batch, y_dev, ep, ctx->moe_scratch, s);
+        ctx->counters.gemm++;
+    } else {
+        launch_gemv(wp, n, k, x_dev, k, batch, y_dev, n, ep, s);
+        ctx->counters.gemv++;
+    }
     LQ4_HIP(hipGetLastError());
     return LQ4_OK;
 }

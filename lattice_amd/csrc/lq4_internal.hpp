@@ -153,12 +153,14 @@ void launch_moe_grouped(const uint8_t* gate_up, const uint8_t* down, uint32_t nu
 // Matrix-core forms of the two expert passes (activations of a pass staged in LDS:
 // moe_mfma_lds_bytes(k) bytes for a reduction length k).
 size_t moe_mfma_lds_bytes(uint32_t k);
+// `ids` not null: the kernels find every expert's pairs in the routing table themselves (offsets and
+// order are then unused); null: they read the grouping tables.
 void launch_moe_gate_up_mfma(const uint8_t* gate_up, uint32_t num_experts, uint32_t inter, uint32_t hidden,
                              const float* x, uint32_t tokens, uint32_t top_k, const int32_t* offsets,
-                             const int32_t* order, float* h, hipStream_t stream);
+                             const int32_t* order, const int32_t* ids, float* h, hipStream_t stream);
 void launch_moe_down_mfma(const uint8_t* down, uint32_t num_experts, uint32_t inter, uint32_t hidden,
-                          const float* h, uint32_t tokens, const int32_t* offsets, const int32_t* order, float* o,
-                          hipStream_t stream);
+                          const float* h, uint32_t tokens, uint32_t top_k, const int32_t* offsets,
+                          const int32_t* order, const int32_t* ids, float* o, hipStream_t stream);
 
 // Exact top-k over n logits (k <= 256): out_logits / out_ids receive the k best in rank order.
 // `scratch` must hold topk_scratch_bytes(n, k) bytes.

@@ -285,19 +285,26 @@ void launch_moe_grouped(const uint8_t* gate_up, const uint8_t* down, uint32_t nu
                         const int32_t* ids, const float* weights, uint32_t top_k, float* y,
                         const MoeScratch& s, hipStream_t stream) {
     const uint32_t pairs = tokens * top_k;
-    hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(256), 0, stream, ids, pairs, num_experts,
-                       s.counts, s.offsets, s.order);
     // matrix-core kernels whenever one pass's activations fit in LDS; the plain kernels otherwise
     const size_t lds_cap = 150 * 1024;
-    if (moe_mfma_lds_bytes(hidden) <= lds_cap)
-        launch_moe_gate_up_mfma(gate_up, num_experts, inter, hidden, x, tokens, top_k, s.offsets, s.order, s.h,
-                                stream);
+    const bool mfma_up = moe_mfma_lds_bytes(hidden) <= lds_cap, mfma_down = moe_mfma_lds_bytes(inter) <= lds_cap;
+    // With few pairs every expert workgroup finds its own pairs in the routing table (one load and a
+    // ballot): no grouping launch and no offsets -> order -> row chain of dependent loads.
+    const bool scan = mfma_up && mfma_down && pairs <= 1024;
+    const int32_t* scan_ids = scan ? ids : nullptr;
+    if (!scan)
+        hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(256), 0, stream, ids, pairs, num_experts, s.counts,
+                           s.offsets, s.order);
+    if (mfma_up)
+        launch_moe_gate_up_mfma(gate_up, num_experts, inter, hidden, x, tokens, top_k, s.offsets, s.order, scan_ids,
+                                s.h, stream);
     else
         hipLaunchKernelGGL(moe_gate_up_kernel, dim3((inter + kMoeWaves - 1) / kMoeWaves, num_experts),
                            dim3(kMoeWaves * 64), 0, stream, gate_up, inter, hidden, x, top_k, s.offsets,
                            s.order, s.h);
-    if (moe_mfma_lds_bytes(inter) <= lds_cap)
-        launch_moe_down_mfma(down, num_experts, inter, hidden, s.h, tokens, s.offsets, s.order, s.o, stream);
+    if (mfma_down)
+        launch_moe_down_mfma(down, num_experts, inter, hidden, s.h, tokens, top_k, s.offsets, s.order, scan_ids, s.o,
+                             stream);
     else
         hipLaunchKernelGGL(moe_down_kernel, dim3((hidden + 2 * kMoeWaves - 1) / (2 * kMoeWaves), num_experts),
                            dim3(kMoeWaves * 64), 0, stream, down, inter, hidden, s.h, s.offsets, s.order,

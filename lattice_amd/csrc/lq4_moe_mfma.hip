@@ -52,6 +52,8 @@ struct MoeGemvArgs {
     float* out;              // h (GATE_UP) or o
     const int32_t* offsets;  // [E + 1]
     const int32_t* order;    // pair indices grouped by expert
+    const int32_t* ids;      // routed expert of every pair; not null = find the expert's pairs here
+    uint32_t n_pairs;        // instead of in offsets/order (few pairs: saves a launch and two dependent loads)
     uint32_t rows_per_expert;  // weight rows of one expert (2I or H)
     uint32_t out_rows;         // output rows per pair (I or H)
     uint32_t k;                // reduction length (H or I)
@@ -66,14 +68,39 @@ __global__ __launch_bounds__(kThreads) void moe_expert_mfma(MoeGemvArgs p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     constexpr int RS = 4 / KS;
     const uint32_t e = blockIdx.y;
-    const int32_t beg = p.offsets[e] + static_cast<int32_t>(blockIdx.z) * kTok;
-    const int32_t end = p.offsets[e + 1];
-    if (beg >= end) return;
-    const int nt = end - beg < kTok ? end - beg : kTok;  // pairs in this pass
-
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    __shared__ int32_t s_pair[kTok];  // the pairs of this pass, ascending pair index (= the stable grouping order)
+    __shared__ int32_t s_cnt[kThreads / 64];
+    int nt;  // pairs in this pass
+    if (p.ids) {
+        // Every workgroup scans the routing table itself: rank of a matching pair = matches before it.
+        const int first = static_cast<int>(blockIdx.z) * kTok;
+        int base = 0;
+        for (uint32_t c0 = 0; c0 < p.n_pairs; c0 += kThreads) {
+            const uint32_t pi = c0 + tid;
+            const bool hit = pi < p.n_pairs && p.ids[pi] == static_cast<int32_t>(e);
+            const uint64_t mask = __ballot(hit);
+            if (lane == 0) s_cnt[wave] = __popcll(mask);
+            __syncthreads();
+            int before = base;
+            for (int w2 = 0; w2 < wave; ++w2) before += s_cnt[w2];
+            const int rank = before + __popcll(mask & ((1ull << lane) - 1ull));
+            if (hit && rank >= first && rank < first + kTok) s_pair[rank - first] = static_cast<int32_t>(pi);
+            base += s_cnt[0] + s_cnt[1] + s_cnt[2] + s_cnt[3];
+            __syncthreads();
+        }
+        if (base <= first) return;
+        nt = base - first < kTok ? base - first : kTok;
+    } else {
+        const int32_t beg = p.offsets[e] + static_cast<int32_t>(blockIdx.z) * kTok;
+        const int32_t end = p.offsets[e + 1];
+        if (beg >= end) return;
+        nt = end - beg < kTok ? end - beg : kTok;
+        if (tid < nt) s_pair[tid] = p.order[beg + tid];
+        __syncthreads();
+    }
     const int g = lane >> 2, j = lane & 3;
     const int ks = wave % KS, rs = wave / KS;
     const uint32_t nb = p.k / kBlockWeights;
@@ -119,7 +146,7 @@ __global__ __launch_bounds__(kThreads) void moe_expert_mfma(MoeGemvArgs p) {
     const float* xrow[kTok];
 #pragma unroll
     for (int b = 0; b < kTok; ++b) {
-        const int32_t pair = p.order[beg + (b < nt ? b : 0)];
+        const int32_t pair = s_pair[b < nt ? b : 0];
         xrow[b] = p.x + static_cast<size_t>(static_cast<uint32_t>(pair) / p.x_div) * p.x_stride;
     }
     {
@@ -284,7 +311,7 @@ __global__ __launch_bounds__(kThreads) void moe_expert_mfma(MoeGemvArgs p) {
             }
             v[t] = fmaf(lo, 1.0f / kLoScale, hi);
         }
-        const int32_t pair = p.order[beg + b];
+        const int32_t pair = s_pair[b];
         p.out[static_cast<size_t>(pair) * p.out_rows + row] = GATE_UP ? silu(v[0]) * v[1] : v[half];
     }
 }
@@ -298,7 +325,7 @@ void launch_ks(const MoeGemvArgs& a, uint32_t num_experts, uint32_t max_pairs_pe
     static bool attr_set = false;
     if (!attr_set) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(moe_expert_mfma<GATE_UP, KS>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 159 * 1024);  // the rest is static
         attr_set = true;
     }
     const dim3 grid((a.out_rows + rows_per_wg - 1) / rows_per_wg, num_experts, (max_pairs_per_expert + kTok - 1) / kTok);
@@ -330,15 +357,15 @@ size_t moe_mfma_lds_bytes(uint32_t k) {
 
 void launch_moe_gate_up_mfma(const uint8_t* gate_up, uint32_t num_experts, uint32_t inter, uint32_t hidden,
                              const float* x, uint32_t tokens, uint32_t top_k, const int32_t* offsets,
-                             const int32_t* order, float* h, hipStream_t stream) {
-    MoeGemvArgs a{gate_up, x, h, offsets, order, 2 * inter, inter, hidden, hidden, top_k, 0};
+                             const int32_t* order, const int32_t* ids, float* h, hipStream_t stream) {
+    MoeGemvArgs a{gate_up, x, h, offsets, order, ids, tokens * top_k, 2 * inter, inter, hidden, hidden, top_k, 0};
     launch_phase<true>(a, num_experts, tokens, stream);
 }
 
 void launch_moe_down_mfma(const uint8_t* down, uint32_t num_experts, uint32_t inter, uint32_t hidden,
-                          const float* h, uint32_t tokens, const int32_t* offsets, const int32_t* order, float* o,
-                          hipStream_t stream) {
-    MoeGemvArgs a{down, h, o, offsets, order, hidden, hidden, inter, inter, 1, 0};
+                          const float* h, uint32_t tokens, uint32_t top_k, const int32_t* offsets,
+                          const int32_t* order, const int32_t* ids, float* o, hipStream_t stream) {
+    MoeGemvArgs a{down, h, o, offsets, order, ids, tokens * top_k, hidden, hidden, inter, inter, 1, 0};
     launch_phase<false>(a, num_experts, tokens, stream);
 }
 

@@ -313,6 +313,7 @@ def test_moe_route_matches_oracle(be):
                                  dict(e=3, inter=96, hidden=160, tokens=7, top_k=3),
                                  dict(e=5, inter=160, hidden=1056, tokens=11, top_k=2),
                                  dict(e=12, inter=64, hidden=128, tokens=90, top_k=7),
+                                 dict(e=16, inter=32, hidden=64, tokens=150, top_k=8),  # > 1024 pairs: grouping tables
                                  dict(e=64, inter=512, hidden=2048, tokens=16, top_k=8)])
 def test_moe_grouped_experts_match_oracle(be, cfg):
     import torch

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the Q4 matmul path on one MI355X.
 
-Headline workload (BASELINE config 1): one Qwen3.5-2B-shaped decode layer at batch 1 —
+Headline workload (benchmark config 1): one Qwen3.5-2B-shaped decode layer at batch 1 —
 Q4 GEMVs at hidden 2048: fused QKV (N=3072), O (N=2048), fused gate||up (N=12288, one
 buffer and one launch, as the reference's decode does) and down (K=6144).  A "step" is
 one layer: 4 GEMV launches over 30,146,560 bytes of Q4 blocks.  Steps rotate over
@@ -236,7 +236,7 @@ def main():
     # ---- per-shape and secondary workloads ---------------------------------------------
     if not args.skip_extras:
         # Per shape: the GEMV and, on the same buffers, the read-only probe kernel whose time is
-        # the ceiling for a launch of that size on this GPU.  "27b_*" are the BASELINE config 2
+        # the ceiling for a launch of that size on this GPU.  "27b_*" are the benchmark config 2
         # matrices driven as batch-1 decode GEMVs: launches large enough to approach the HBM
         # streaming rate.
         shapes = {}
@@ -351,7 +351,7 @@ def main():
             mlp["speedup"] = round(mlp["five_launches_us"] / mlp["two_fused_launches_us"], 3)
             out["decode_mlp_hidden2048_inter6144"] = mlp
 
-        # single-LoRA epilogue, BASELINE config 3: q (2048x2048) and v (512x2048) projections, rank 16,
+        # single-LoRA epilogue, benchmark config 3: q (2048x2048) and v (512x2048) projections, rank 16,
         # f16 factors, scale alpha/r = 2.0, fused into the projection's own launch
         if B == 1:
             from lattice_amd import synth
@@ -391,7 +391,7 @@ def main():
             out["lora_q_v_rank16"] = lora_out
             del pool
 
-        # prefill GEMM, BASELINE config 2
+        # prefill GEMM, benchmark config 2
         del layers
         torch.cuda.empty_cache()
         gemm = {}
@@ -410,7 +410,7 @@ def main():
             del qw
         out["prefill_gemm_f16"] = gemm
 
-        # MoE grouped expert GEMV, BASELINE config 4
+        # MoE grouped expert GEMV, benchmark config 4
         mo = synth.MOE_35B
         E, I, H, T, TK = mo["experts"], mo["inter"], mo["hidden"], mo["tokens"], mo["top_k"]
         sets = []

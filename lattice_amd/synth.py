@@ -18,7 +18,7 @@ import numpy as np
 
 from .q4_layout import BLOCK_WEIGHTS, pack_blocks
 
-# BASELINE workload shapes: name -> (N, K)
+# benchmark workload shapes: name -> (N, K)
 DECODE_LAYER_2B = {
     "qkv": (3072, 2048),
     "o": (2048, 2048),

@@ -189,7 +189,7 @@ def test_gemm_matches_oracle(be, m, n, k, xdt):
 
 
 def test_gemm_full_size_against_torch_f32_on_dequantized_weights(be):
-    # BASELINE prefill shape at full size (M=512, N=17408, K=5120), too large for the CPU
+    # benchmark prefill shape at full size (M=512, N=17408, K=5120), too large for the CPU
     # oracle in seconds: the reference here is torch f32 matmul over the dequant probe's
     # output, which test_dequant_probe_is_bit_exact ties bit-for-bit to the oracle.
     import torch
@@ -221,7 +221,7 @@ def _lora_ref(x, wq, n, k, a, b, scale):
 
 @pytest.mark.parametrize("name,batch", [("q", 1), ("q", 8), ("v", 1), ("v", 8), ("q", 64), ("v", 64)])
 def test_lora_fused_matches_oracle(be, name, batch):
-    # BASELINE config 3: rank 16, alpha 32 (scale 2.0), f16 A/B ~ N(0, 0.01)
+    # benchmark config 3: rank 16, alpha 32 (scale 2.0), f16 A/B ~ N(0, 0.01)
     import torch
     print(f"lora {name} batch={batch}", flush=True)
     n, k = synth.LORA_2B[name]

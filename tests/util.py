@@ -1,7 +1,7 @@
 """Shared helpers for the parity tests."""
 import numpy as np
 
-# BASELINE tolerance: max relative error <= 1e-3 against the f32-accumulated reference, in the
+# Required tolerance: max relative error <= 1e-3 against the f32-accumulated reference, in the
 # reference's own form max|delta| / max|y_ref| (forward/metal_qwen35.rs:23615-23623).
 REL_TOL = 1e-3
 

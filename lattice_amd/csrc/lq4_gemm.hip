@@ -412,10 +412,7 @@ void launch_tile(const uint8_t* w, uint32_t n, uint32_t k, const void* x, uint32
                        lora);
 }
 
-// Shapes with at least this many 128 x 256 tiles (two per CU) go to the weights-in-registers
-// kernel; below that its single workgroup per CU leaves the chip under-filled and the 128 x 128
-// tile of this file, two workgroups per CU, is faster.
-constexpr uint32_t kWregMinTiles = 512;
+
 
 // kernel choice override: starts from the environment variable LQ4_GEMM_KERNEL (0, 1 or 2)
 std::atomic<int> g_gemm_choice{[] {
@@ -429,24 +426,19 @@ void set_gemm_kernel_choice(int which) { g_gemm_choice.store(which, std::memory_
 
 namespace {
 
-// Which kernel serves a shape, and with how many K slices.
+// Which kernel serves a shape.
 struct GemmPlan {
     bool wreg;
-    uint32_t slices;
     bool skinny;
 };
 
 GemmPlan plan_gemm(uint32_t n, uint32_t k, uint32_t m, int x_is_f16) {
     const int forced = g_gemm_choice.load(std::memory_order_relaxed);
-    if (forced == 3 || (forced == 0 && gemm_skinny_wants(n, k, m))) return {false, 1, true};
-    if (forced == 1 || !gemm_wreg_supports(n, k, m, x_is_f16)) return {false, 1, false};
-    uint32_t slices = gemm_wreg_slices(n, k, m);
-    if (static_cast<uint64_t>(slices) * m * n > (64ull << 20)) slices = 1;  // keep the partials under 256 MB
-    const uint32_t lds_tiles = ((n + 127) / 128) * ((m + BM - 1) / BM);
-    // big shapes: plenty of 128 x 256 tiles; small shapes: the 128 x 128 tiles cannot fill the chip
-    // either, and slicing K can
-    const bool wreg = forced == 2 || gemm_wreg_tiles(n, m) >= kWregMinTiles || (lds_tiles < 384 && slices > 1);
-    return {wreg, wreg ? slices : 1, false};
+    if (forced == 3 || (forced == 0 && gemm_skinny_wants(n, k, m))) return {false, true};
+    if (forced == 1 || !gemm_wreg_supports(n, k, m, x_is_f16)) return {false, false};
+    // The weights-in-registers kernel everywhere else: its scheduling cuts a partly filled last round
+    // of tiles into K slices, so it no longer needs many tiles to keep the chip busy.
+    return {true, false};
 }
 
 }  // namespace
@@ -454,14 +446,14 @@ GemmPlan plan_gemm(uint32_t n, uint32_t k, uint32_t m, int x_is_f16) {
 size_t gemm_scratch_floats(uint32_t n, uint32_t k, uint32_t m, int x_is_f16) {
     const GemmPlan p = plan_gemm(n, k, m, x_is_f16);
     if (p.skinny) return (gemm_skinny_scratch_bytes(k, m) + sizeof(float) - 1) / sizeof(float);
-    return p.slices > 1 ? static_cast<size_t>(p.slices) * m * n : 0;
+    return p.wreg ? gemm_wreg_scratch_floats(n, k, m) : 0;
 }
 
 void launch_gemm(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
                  float* y, const LoraEpilogue& lora, float* scratch, hipStream_t stream) {
     const GemmPlan p = plan_gemm(n, k, m, x_is_f16);
     if (p.skinny) return launch_gemm_skinny(w, n, k, x, x_is_f16, m, y, lora, scratch, stream);
-    if (p.wreg) return launch_gemm_wreg(w, n, k, x, x_is_f16, m, y, lora, p.slices, scratch, stream);
+    if (p.wreg) return launch_gemm_wreg(w, n, k, x, x_is_f16, m, y, lora, scratch, stream);
     if (lora.rank) {
         if (x_is_f16) launch_tile<true, 128, true>(w, n, k, x, m, y, lora, stream);
         else launch_tile<false, 128, true>(w, n, k, x, m, y, lora, stream);

@@ -111,10 +111,23 @@ __device__ __forceinline__ uint32_t pack_h2(float lo, float hi) {
 
 // LORA: compiled with the LoRA step (kept out of the plain kernel, whose register allocation it
 // would disturb).
+//
+// Scheduling.  Tiles are long (K/128 steps of ~2 us) and there is one per CU at a time, so a last,
+// partly filled round of tiles would idle most of the chip for a whole tile time.  The launch
+// therefore runs the first `full` tiles (a multiple of the CU count) whole, and cuts each of the
+// remaining "tail" tiles into `tail_slices` K slices that run as separate, shorter workgroups
+// (dispatched last).  A slice writes its 128 x 256 partial tile to scratch; gemm_reduce_tail adds
+// the slices in slice order (deterministic) and applies the LoRA delta of those tiles in f32.
+struct WregPlan {
+    uint32_t full;         // tiles computed whole, written straight to y
+    uint32_t tail_slices;  // K slices per remaining tile (1 = no slicing, written straight to y)
+    float* partial;        // [tail tile][slice][TM * TN] when tail_slices > 1
+};
+
 template <bool X_F16, bool LORA>
 __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict__ w, uint32_t n, uint32_t k,
                                                        const void* __restrict__ xv, uint32_t m,
-                                                       float* __restrict__ y, LoraEpilogue lora) {
+                                                       float* __restrict__ y, LoraEpilogue lora, WregPlan plan) {
     extern __shared__ uint4 lds16[];  // two activation buffers of kBuf16 units
     constexpr int XU = TM * (TK / 8) / 256;  // 8-activation units staged per thread per step
     constexpr int XL = X_F16 ? 1 : 2;        // 16-byte global loads per unit
@@ -126,25 +139,34 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
     const int g = lane >> 4;   // K group: block g of the step
 
     // ---- tile id -> (token tile, weight tile), grouped so co-resident tiles share activations
+    // workgroup -> (tile, K slice): whole tiles first, then the slices of the tail tiles
+    const bool in_tail = blockIdx.x >= plan.full;
+    const uint32_t tail_idx = in_tail ? blockIdx.x - plan.full : 0;
+    const uint32_t tile = in_tail ? plan.full + tail_idx / plan.tail_slices : blockIdx.x;
+    const uint32_t nslices = in_tail ? plan.tail_slices : 1;
+    const uint32_t slice = in_tail ? tail_idx % plan.tail_slices : 0;
+
     const uint32_t tiles_m = (m + TM - 1) / TM, tiles_n = (n + TN - 1) / TN;
     const uint32_t per_group = kGroupM * tiles_n;
-    const uint32_t group = blockIdx.x / per_group;
+    const uint32_t group = tile / per_group;
     const uint32_t first_m = group * kGroupM;
     const uint32_t group_m = tiles_m - first_m < kGroupM ? tiles_m - first_m : kGroupM;
-    const uint32_t in_group = blockIdx.x - group * per_group;
+    const uint32_t in_group = tile - group * per_group;
     const uint32_t m0 = (first_m + in_group % group_m) * TM;
     const uint32_t n0 = (in_group / group_m) * TN;
 
-    // K slice of this workgroup (gridDim.y slices; one slice = the whole row when gridDim.y == 1).
-    // From here on steps, blocks and K offsets are counted from the start of the slice.
+    // K slice of this workgroup (the whole row when nslices == 1).  From here on steps, blocks and
+    // K offsets are counted from the start of the slice.
     const uint32_t nb_total = k / kBlockWeights;
     const uint32_t steps_total = (nb_total + 3) / 4;
-    const uint32_t steps_per = (steps_total + gridDim.y - 1) / gridDim.y;
-    const uint32_t s_begin = blockIdx.y * steps_per;  // the host never launches an empty slice
+    const uint32_t steps_per = (steps_total + nslices - 1) / nslices;
+    const uint32_t s_begin = slice * steps_per;  // the host never plans an empty slice
     const uint32_t nsteps = s_begin + steps_per < steps_total ? steps_per : steps_total - s_begin;
-    const uint32_t nb = nb_total - s_begin * 4;       // blocks from the slice start to the end of the row
+    const uint32_t nb = nb_total - s_begin * 4;  // blocks from the slice start to the end of the row
     const uint32_t k_rem = k - s_begin * TK;
-    if (gridDim.y > 1) y += static_cast<size_t>(blockIdx.y) * m * n;  // partial sums, one matrix per slice
+    const bool to_partial = nslices > 1;
+    float* const ptile = to_partial ? plan.partial + (static_cast<size_t>(tile - plan.full) * nslices + slice) * (TM * TN)
+                                    : nullptr;
 
     float4v acc[NU][NT];
 #pragma unroll
@@ -307,7 +329,7 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
     //      acc[n, token] += sum_r B[n, r] * (scale * t[token, r]).
     // Both factors are split hi + lo/2048 into f16 so the delta keeps f32-level accuracy:
     // B.t = Bhi.thi + (Bhi/2048).tlo + Blo.(thi/2048); the last term vanishes for f16-stored B.
-    if (LORA && lora.rank && blockIdx.y == 0) {
+    if (LORA && lora.rank && !to_partial) {
         for (uint32_t r0 = 0; r0 < lora.rank; r0 += 32) {
             const uint32_t rbase = r0 + 8 * g;  // this lane's eight rank indices
             half8 b_hi[NU], b_his[NU], b_lo[NU];
@@ -361,6 +383,10 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
             const uint32_t gm = m0 + t * 16 + lr;
             if (gm >= m || gn >= n) continue;
             const float4v val = acc[u][t];
+            if (to_partial) {  // tile-local layout, always 16-byte aligned
+                *reinterpret_cast<float4v*>(ptile + (gm - m0) * TN + (gn - n0)) = val;
+                continue;
+            }
             float* dst = y + static_cast<size_t>(gm) * n + gn;
             if (vec_ok) {
                 *reinterpret_cast<float4v*>(dst) = val;
@@ -373,70 +399,100 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
     }
 }
 
-// y[i] = sum over slices, in slice order, of partial[s][i]  (count multiple of 4 or not), plus the
-// LoRA delta scale * sum_j B[row, j] * t[token, j] in f32 when lora.rank != 0 (i = token * n + row).
-__global__ __launch_bounds__(256) void gemm_reduce_slices(const float* __restrict__ partial, uint32_t slices,
-                                                          size_t count, float* __restrict__ y, uint32_t n,
-                                                          LoraEpilogue lora) {
-    const size_t i4 = (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
-    if (i4 >= count) return;
-    auto delta = [&](size_t i) {
-        const size_t token = i / n, row = i - token * n;
-        const float* t = lora.t + token * lora.rank;
-        float d = 0.0f;
-        for (uint32_t j = 0; j < lora.rank; ++j) d = fmaf(load_b(lora.b, lora.b_is_f16, row * lora.rank + j), t[j], d);
-        return lora.scale * d;
-    };
-    if (i4 + 4 <= count && (count & 3) == 0) {
-        float4v v = *reinterpret_cast<const float4v*>(partial + i4);
-        for (uint32_t sl = 1; sl < slices; ++sl) v += *reinterpret_cast<const float4v*>(partial + sl * count + i4);
-        if (lora.rank) {
+// Sums the K slices of the tail tiles in slice order and writes them to y, adding the LoRA delta
+// scale * sum_j B[row, j] * t[token, j] in f32.  grid (tail tiles, TM * TN / 1024); a thread owns four
+// consecutive weight rows of one token.
+__global__ __launch_bounds__(256) void gemm_reduce_tail(const float* __restrict__ partial, uint32_t first_tile,
+                                                        uint32_t slices, uint32_t m, uint32_t n,
+                                                        float* __restrict__ y, LoraEpilogue lora) {
+    const uint32_t tile = first_tile + blockIdx.x;
+    const uint32_t tiles_m = (m + TM - 1) / TM, tiles_n = (n + TN - 1) / TN;
+    const uint32_t per_group = kGroupM * tiles_n;
+    const uint32_t group = tile / per_group;
+    const uint32_t first_m = group * kGroupM;
+    const uint32_t group_m = tiles_m - first_m < kGroupM ? tiles_m - first_m : kGroupM;
+    const uint32_t in_group = tile - group * per_group;
+    const uint32_t m0 = (first_m + in_group % group_m) * TM;
+    const uint32_t n0 = (in_group / group_m) * TN;
+
+    const uint32_t local = (blockIdx.y * 256 + threadIdx.x) * 4;  // element index inside the tile
+    const uint32_t lrow = local / TN, lcol = local % TN;
+    const uint32_t token = m0 + lrow, row = n0 + lcol;
+    if (token >= m || row >= n) return;
+    const float* src = partial + static_cast<size_t>(blockIdx.x) * slices * (TM * TN) + local;
+    float4v v = *reinterpret_cast<const float4v*>(src);
+    for (uint32_t sl = 1; sl < slices; ++sl) v += *reinterpret_cast<const float4v*>(src + static_cast<size_t>(sl) * (TM * TN));
+    if (lora.rank) {
+        typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+        const float* t = lora.t + static_cast<size_t>(token) * lora.rank;
+        float4v d = {0.0f, 0.0f, 0.0f, 0.0f};
+        if ((lora.rank & 3u) == 0) {  // t[token, :] is a broadcast load, the B rows are read with vector loads
+            for (uint32_t j = 0; j < lora.rank; j += 4) {
+                const float4v tv = *reinterpret_cast<const float4v*>(t + j);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] += delta(i4 + e);
+                for (int e = 0; e < 4; ++e) {
+                    const uint32_t r = row + e < n ? row + e : n - 1;
+                    const size_t bi = static_cast<size_t>(r) * lora.rank + j;
+                    float4v bv;
+                    if (lora.b_is_f16) {
+                        const half4v h = *reinterpret_cast<const half4v*>(static_cast<const _Float16*>(lora.b) + bi);
+                        bv = float4v{static_cast<float>(h[0]), static_cast<float>(h[1]), static_cast<float>(h[2]),
+                                     static_cast<float>(h[3])};
+                    } else {
+                        bv = *reinterpret_cast<const float4v*>(static_cast<const float*>(lora.b) + bi);
+                    }
+                    d[e] = fmaf(bv[3], tv[3], fmaf(bv[2], tv[2], fmaf(bv[1], tv[1], fmaf(bv[0], tv[0], d[e]))));
+                }
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t r = row + e < n ? row + e : n - 1;
+                for (uint32_t j = 0; j < lora.rank; ++j)
+                    d[e] = fmaf(load_b(lora.b, lora.b_is_f16, static_cast<size_t>(r) * lora.rank + j), t[j], d[e]);
+            }
         }
-        *reinterpret_cast<float4v*>(y + i4) = v;
+        v += lora.scale * d;
+    }
+    float* dst = y + static_cast<size_t>(token) * n + row;
+    if ((n & 3u) == 0 && (reinterpret_cast<uintptr_t>(y) & 15u) == 0) {
+        *reinterpret_cast<float4v*>(dst) = v;
     } else {
-        for (size_t i = i4; i < count && i < i4 + 4; ++i) {
-            float v = partial[i];
-            for (uint32_t sl = 1; sl < slices; ++sl) v += partial[sl * count + i];
-            if (lora.rank) v += delta(i);
-            y[i] = v;
-        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (row + e < n) dst[e] = v[e];
     }
 }
 
-// Same with the LoRA delta for n % 4 == 0 and rank % 4 == 0: grid (ceil(n / 1024), m); a thread owns
-// four consecutive weight rows of one token, so t[token, :] is a broadcast load and the B rows are
-// read with vector loads.
-__global__ __launch_bounds__(256) void gemm_reduce_slices_lora(const float* __restrict__ partial, uint32_t slices,
-                                                               uint32_t m, uint32_t n, float* __restrict__ y,
-                                                               LoraEpilogue lora) {
-    typedef _Float16 half4v __attribute__((ext_vector_type(4)));
-    const uint32_t row = (blockIdx.x * 256 + threadIdx.x) * 4;
-    const uint32_t token = blockIdx.y;
-    if (row >= n) return;
-    const size_t at = static_cast<size_t>(token) * n + row, count = static_cast<size_t>(m) * n;
-    float4v v = *reinterpret_cast<const float4v*>(partial + at);
-    for (uint32_t sl = 1; sl < slices; ++sl) v += *reinterpret_cast<const float4v*>(partial + sl * count + at);
-    const float* t = lora.t + static_cast<size_t>(token) * lora.rank;
-    float4v d = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (uint32_t j = 0; j < lora.rank; j += 4) {
-        const float4v tv = *reinterpret_cast<const float4v*>(t + j);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const size_t bi = static_cast<size_t>(row + e) * lora.rank + j;
-            float4v bv;
-            if (lora.b_is_f16) {
-                const half4v h = *reinterpret_cast<const half4v*>(static_cast<const _Float16*>(lora.b) + bi);
-                bv = float4v{static_cast<float>(h[0]), static_cast<float>(h[1]), static_cast<float>(h[2]),
-                             static_cast<float>(h[3])};
-            } else {
-                bv = *reinterpret_cast<const float4v*>(static_cast<const float*>(lora.b) + bi);
-            }
-            d[e] = fmaf(bv[3], tv[3], fmaf(bv[2], tv[2], fmaf(bv[1], tv[1], fmaf(bv[0], tv[0], d[e]))));
+constexpr uint32_t kCus = 256;
+constexpr uint32_t kMaxTailSlices = 16;
+
+// How the tiles of a shape are scheduled: `full` whole tiles, the rest in `slices` K slices each.
+struct HostPlan {
+    uint32_t tiles, full, slices;
+};
+
+HostPlan plan_tiles(uint32_t n, uint32_t k, uint32_t m) {
+    const uint32_t tiles = ((n + TN - 1) / TN) * ((m + TM - 1) / TM);
+    const uint32_t steps = (k / kBlockWeights + 3) / 4;
+    const uint32_t rest = tiles % kCus;
+    HostPlan p{tiles, tiles - rest, 1};
+    if (rest == 0 || steps < 4) return HostPlan{tiles, tiles, 1};
+    // pick the slice count that minimises the time of the last round, ceil(rest * s / CUs) / s tile
+    // times, with at least two steps per slice and no empty slice
+    double best = 1.0;  // s = 1: one round of whole tiles
+    for (uint32_t s = 2; s <= kMaxTailSlices && s * 2 <= steps; ++s) {
+        const uint32_t per = (steps + s - 1) / s;
+        if ((s - 1) * per >= steps) continue;  // would leave the last slice empty
+        const double rounds = static_cast<double>((rest * s + kCus - 1) / kCus);
+        const double t = rounds * per / steps + 0.02 * s;  // small charge per slice for the reduction traffic
+        if (t < best - 1e-9) {
+            best = t;
+            p.slices = s;
         }
     }
-    *reinterpret_cast<float4v*>(y + at) = v + lora.scale * d;
+    if (p.slices == 1) p.full = tiles;
+    return p;
 }
 
 }  // namespace
@@ -445,26 +501,16 @@ uint32_t gemm_wreg_tiles(uint32_t n, uint32_t m) { return ((n + TN - 1) / TN) * 
 
 bool gemm_wreg_supports(uint32_t, uint32_t k, uint32_t, int) { return k >= kBlockWeights; }
 
-uint32_t gemm_wreg_slices(uint32_t n, uint32_t k, uint32_t m) {
-    // Too few tiles to occupy the 256 CUs: cut K into slices (whole 128-wide steps) until there
-    // are about that many workgroups.  Each slice writes its own partial matrix; a second kernel
-    // adds them in slice order, so the result does not depend on scheduling.
-    const uint32_t tiles = gemm_wreg_tiles(n, m);
-    const uint32_t steps = (k / kBlockWeights + 3) / 4;
-    if (tiles >= 192 || steps < 4) return 1;
-    uint32_t want = (256 + tiles - 1) / tiles;
-    want = want > 16 ? 16 : want;
-    want = want > steps / 2 ? steps / 2 : want;  // at least two steps per slice
-    if (want <= 1) return 1;
-    const uint32_t per = (steps + want - 1) / want;
-    return (steps + per - 1) / per;  // no empty slice
+size_t gemm_wreg_scratch_floats(uint32_t n, uint32_t k, uint32_t m) {
+    const HostPlan p = plan_tiles(n, k, m);
+    return p.slices > 1 ? static_cast<size_t>(p.tiles - p.full) * p.slices * (TM * TN) : 0;
 }
 
 namespace {
 
 template <bool X_F16, bool LORA>
-void launch_wreg_t(const uint8_t* w, uint32_t n, uint32_t k, const void* x, uint32_t m, float* out,
-                   const LoraEpilogue& lora, uint32_t slices, hipStream_t stream) {
+void launch_wreg_t(const uint8_t* w, uint32_t n, uint32_t k, const void* x, uint32_t m, float* y,
+                   const LoraEpilogue& lora, const HostPlan& hp, float* partial, hipStream_t stream) {
     static bool attr_set = false;
     if (!attr_set) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4_wreg<X_F16, LORA>),
@@ -472,33 +518,29 @@ void launch_wreg_t(const uint8_t* w, uint32_t n, uint32_t k, const void* x, uint
         attr_set = true;
     }
     const size_t lds = 2 * kBuf16 * sizeof(uint4);
-    hipLaunchKernelGGL((gemm_q4_wreg<X_F16, LORA>), dim3(gemm_wreg_tiles(n, m), slices), dim3(256), lds, stream, w,
-                       n, k, x, m, out, lora);
+    const WregPlan plan{hp.full, hp.slices, partial};
+    const uint32_t wgs = hp.full + (hp.tiles - hp.full) * hp.slices;
+    hipLaunchKernelGGL((gemm_q4_wreg<X_F16, LORA>), dim3(wgs), dim3(256), lds, stream, w, n, k, x, m, y, lora, plan);
 }
 
 }  // namespace
 
 void launch_gemm_wreg(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
-                      float* y, const LoraEpilogue& lora, uint32_t slices, float* partial, hipStream_t stream) {
-    if (slices <= 1 || !partial) slices = 1;
-    float* out = slices > 1 ? partial : y;
-    // K-sliced: the delta is added in f32 by the pass that sums the slices
-    if (lora.rank && slices == 1) {
-        if (x_is_f16) launch_wreg_t<true, true>(w, n, k, x, m, out, lora, slices, stream);
-        else launch_wreg_t<false, true>(w, n, k, x, m, out, lora, slices, stream);
+                      float* y, const LoraEpilogue& lora, float* partial, hipStream_t stream) {
+    HostPlan hp = plan_tiles(n, k, m);
+    if (!partial) hp = HostPlan{hp.tiles, hp.tiles, 1};
+    // the matrix-core LoRA step serves the whole tiles; the tail tiles get their delta from the reduction
+    const bool lora_in_kernel = lora.rank && hp.full > 0;
+    if (lora_in_kernel) {
+        if (x_is_f16) launch_wreg_t<true, true>(w, n, k, x, m, y, lora, hp, partial, stream);
+        else launch_wreg_t<false, true>(w, n, k, x, m, y, lora, hp, partial, stream);
     } else {
-        if (x_is_f16) launch_wreg_t<true, false>(w, n, k, x, m, out, lora, slices, stream);
-        else launch_wreg_t<false, false>(w, n, k, x, m, out, lora, slices, stream);
+        if (x_is_f16) launch_wreg_t<true, false>(w, n, k, x, m, y, lora, hp, partial, stream);
+        else launch_wreg_t<false, false>(w, n, k, x, m, y, lora, hp, partial, stream);
     }
-    if (slices > 1) {
-        const size_t count = static_cast<size_t>(m) * n;
-        if (lora.rank && n % 4 == 0 && lora.rank % 4 == 0)
-            hipLaunchKernelGGL(gemm_reduce_slices_lora, dim3((n + 1023) / 1024, m), dim3(256), 0, stream, partial,
-                               slices, m, n, y, lora);
-        else
-            hipLaunchKernelGGL(gemm_reduce_slices, dim3(static_cast<uint32_t>((count + 1023) / 1024)), dim3(256), 0,
-                               stream, partial, slices, count, y, n, lora);
-    }
+    if (hp.slices > 1)
+        hipLaunchKernelGGL(gemm_reduce_tail, dim3(hp.tiles - hp.full, TM * TN / 1024), dim3(256), 0, stream, partial,
+                           hp.full, hp.slices, m, n, y, lora);
 }
 
 }  // namespace lq4

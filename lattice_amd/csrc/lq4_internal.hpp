@@ -99,11 +99,11 @@ bool gemm_wreg_supports(uint32_t n, uint32_t k, uint32_t m, int x_is_f16);
 // 0 = choose by shape, 1 = LDS-staged kernel, 2 = weights-in-registers kernel where supported,
 // 3 = few-token kernel.
 void set_gemm_kernel_choice(int which);
-// gemm_wreg_slices = K slices it wants for the shape (1 = none); with more than one, `partial`
-// must hold slices * m * n floats.
-uint32_t gemm_wreg_slices(uint32_t n, uint32_t k, uint32_t m);
+// A last, partly filled round of tiles is cut into K slices that meet in `partial`
+// (gemm_wreg_scratch_floats floats; null = no slicing) and are summed by a second kernel.
+size_t gemm_wreg_scratch_floats(uint32_t n, uint32_t k, uint32_t m);
 void launch_gemm_wreg(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
-                      float* y, const LoraEpilogue& lora, uint32_t slices, float* partial, hipStream_t stream);
+                      float* y, const LoraEpilogue& lora, float* partial, hipStream_t stream);
 
 // Q8_0 sibling format (34-byte blocks: f16 scale + 32 x i8, w = q * d): batch-1 GEMV with x staged
 // in LDS (gemv_q8_lds_bytes(k) bytes), and the LDS-staged tile GEMM for everything else.

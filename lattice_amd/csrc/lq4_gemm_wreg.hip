@@ -466,6 +466,9 @@ __global__ __launch_bounds__(256) void gemm_reduce_tail(const float* __restrict_
 
 constexpr uint32_t kCus = 256;
 constexpr uint32_t kMaxTailSlices = 16;
+#ifndef LQ4_SLICE_CHARGE
+#define LQ4_SLICE_CHARGE 0.01
+#endif
 
 // How the tiles of a shape are scheduled: `full` whole tiles, the rest in `slices` K slices each.
 struct HostPlan {
@@ -485,7 +488,7 @@ HostPlan plan_tiles(uint32_t n, uint32_t k, uint32_t m) {
         const uint32_t per = (steps + s - 1) / s;
         if ((s - 1) * per >= steps) continue;  // would leave the last slice empty
         const double rounds = static_cast<double>((rest * s + kCus - 1) / kCus);
-        const double t = rounds * per / steps + 0.02 * s;  // small charge per slice for the reduction traffic
+        const double t = rounds * per / steps + LQ4_SLICE_CHARGE * s;  // small charge per slice for the reduction traffic
         if (t < best - 1e-9) {
             best = t;
             p.slices = s;

@@ -213,6 +213,38 @@ def test_gemm_full_size_against_torch_f32_on_dequantized_weights(be):
     assert rel_err(host(y[rows, :256]), ref_o) <= REL_TOL
 
 
+def test_gemm_full_size_with_lora_on_whole_and_sliced_tiles(be):
+    # 272 tiles of 128 x 256: one full round of whole tiles (LoRA step on the matrix cores) plus 16
+    # tail tiles cut into K slices (LoRA added by the pass that sums the slices)
+    import torch
+    m, n, k, r = 512, 17408, 5120, 16
+    wq = synth.q4_weight(n, k, seed=1)
+    x = synth.activations(m, k, seed=1, dtype=np.float16)
+    a, b = synth.lora_pair(r, k, n, seed=1)
+    qw = be.upload_q4_blocks(wq)
+    xd = dev(x)
+    y = torch.empty((m, n), dtype=torch.float32, device="cuda")
+    be.load_lora_adapter([backend.LoraLayerData(0, {"up_proj": (a, b)})], scale=2.0)
+    try:
+        be.dispatch_gemm(xd, 0, qw, y, 0, m, n, k, layer_idx=0, module="up_proj")
+    finally:
+        be.unload_lora_adapter()
+    torch.backends.cuda.matmul.allow_tf32 = False
+    wd = be.dequantize(qw, n, k)
+    ad, bd = dev(a.astype(np.float32)), dev(b.astype(np.float32))
+    delta = 2.0 * ((xd.float() @ ad.t()) @ bd.t())
+    ref = xd.float() @ wd.t() + delta
+    err = (y - ref).abs().max().item() / ref.abs().max().item()
+    print(f"  rel err vs torch f32 {err:.2e}", flush=True)
+    assert err <= REL_TOL
+    # the delta itself, tile by tile (it is small against the base product)
+    plain = torch.empty((m, n), dtype=torch.float32, device="cuda")
+    be.dispatch_gemm(xd, 0, qw, plain, 0, m, n, k)
+    derr = ((y - plain) - delta).abs().max().item() / delta.abs().max().item()
+    print(f"  delta rel err {derr:.2e}", flush=True)
+    assert derr <= 5e-3  # y - plain cancels the base product: its f32 rounding is the floor here
+
+
 # -------------------------------------------------------------------------- LoRA
 def _lora_ref(x, wq, n, k, a, b, scale):
     base = oracle.gemm_f32(x.astype(np.float32), wq, n, k)

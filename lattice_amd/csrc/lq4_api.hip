@@ -100,6 +100,12 @@ int resolve_weight(const lq4_weight* w, uint64_t extra, uint32_t n, uint32_t k,
     return LQ4_OK;
 }
 
+// The sibling formats have only the 128 x 128 tile kernel beside the few-token kernel, and it does not
+// cut K: with fewer weight tiles than half the compute units the few-token kernel also serves 65..128 rows.
+bool sibling_skinny_wants(uint32_t n, uint32_t k, uint32_t m) {
+    return gemm_skinny_wants(n, k, m) || (m <= 128 && (n + 127) / 128 < 128);
+}
+
 // The same for a buffer of sibling-format blocks: Q8_0 (34 bytes, 2-byte aligned) or Q3 (16 bytes,
 // 4-byte aligned).
 int resolve_weight_sibling(const lq4_weight* w, uint64_t extra, uint32_t n, uint32_t k, const char* fmt,
@@ -694,6 +700,13 @@ int lq4_gemm_q8(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
     if (m == 1 && x_dtype == LQ4_F32 && gemv_q8_lds_bytes(k) <= 128 * 1024) {
         launch_gemv_q8_b1(wp, n, k, static_cast<const float*>(x_dev), y_dev, s);
         ctx->counters.gemv++;
+    } else if (sibling_skinny_wants(n, k, m)) {
+        // few rows: operands packed once, the few-token matrix-core kernel with this format's decoder
+        const int src = ensure_scratch(ctx, gemm_skinny_scratch_bytes(k, m));
+        if (src) return src;
+        const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};
+        launch_gemm_skinny(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, none, ctx->moe_scratch, s, 1);
+        ctx->counters.gemm++;
     } else {
         launch_gemm_q8(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, s);
         ctx->counters.gemm++;
@@ -725,6 +738,13 @@ int lq4_gemm_q3(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
     if (m == 1 && x_dtype == LQ4_F32 && gemv_q3_lds_bytes(k) <= 128 * 1024) {
         launch_gemv_q3_b1(wp, n, k, static_cast<const float*>(x_dev), y_dev, s);
         ctx->counters.gemv++;
+    } else if (sibling_skinny_wants(n, k, m)) {
+        // few rows: operands packed once, the few-token matrix-core kernel with this format's decoder
+        const int src = ensure_scratch(ctx, gemm_skinny_scratch_bytes(k, m));
+        if (src) return src;
+        const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};
+        launch_gemm_skinny(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, none, ctx->moe_scratch, s, 2);
+        ctx->counters.gemm++;
     } else {
         launch_gemm_q3(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, s);
         ctx->counters.gemm++;

@@ -67,6 +67,62 @@ __device__ __forceinline__ U4 dequant8(uint32_t q, half2v d2, half2v b2) {
     return out;
 }
 
+// Sibling formats (FMT 1 = Q8_0, 2 = Q3): their decoders emit the eight weights of an instruction
+// in memory order, so their activations are packed without the interleave.
+struct __attribute__((packed, aligned(2))) Q8BlockRaw {
+    uint16_t d;
+    uint32_t q[8];  // weight i in byte i
+};
+struct __attribute__((packed, aligned(4))) Q3BlockRaw {
+    uint32_t sb;
+    uint32_t lo[2];  // weight i of 16-weight half h at bits 2i of lo[h]
+    uint32_t hi;     // weight i at bit i
+};
+template <int FMT>
+struct WBlockOf {
+    typedef Q4BlockRaw type;
+    static constexpr uint32_t kBytes = 20;
+};
+template <>
+struct WBlockOf<1> {
+    typedef Q8BlockRaw type;
+    static constexpr uint32_t kBytes = 34;
+};
+template <>
+struct WBlockOf<2> {
+    typedef Q3BlockRaw type;
+    static constexpr uint32_t kBytes = 16;
+};
+
+// Q8_0: two packed dwords (weights 8j..8j+7) -> half(q * d).  A sign-flipped byte (q + 128) under the
+// exponent byte of 1024.0 is 1024 + 128 + q exactly; subtract, then one multiply with one rounding.
+__device__ __forceinline__ U4 dequant8_q8(uint32_t qa, uint32_t qb, half2v d2) {
+    const half2v k1152 = {static_cast<_Float16>(1152.0f), static_cast<_Float16>(1152.0f)};
+    const uint32_t ua = qa ^ 0x80808080u, ub = qb ^ 0x80808080u;
+    U4 out;
+    out.v[0] = as_u32((as_h2(__builtin_amdgcn_perm(0x64646464u, ua, 0x04010400u)) - k1152) * d2);
+    out.v[1] = as_u32((as_h2(__builtin_amdgcn_perm(0x64646464u, ua, 0x04030402u)) - k1152) * d2);
+    out.v[2] = as_u32((as_h2(__builtin_amdgcn_perm(0x64646464u, ub, 0x04010400u)) - k1152) * d2);
+    out.v[3] = as_u32((as_h2(__builtin_amdgcn_perm(0x64646464u, ub, 0x04030402u)) - k1152) * d2);
+    return out;
+}
+
+// Q3: weights 8j..8j+7 -> half(q * d + b), q = low2 | hi << 2.
+__device__ __forceinline__ U4 dequant8_q3(const Q3BlockRaw& b, int j, half2v d2, half2v b2) {
+    const half2v k1024 = {static_cast<_Float16>(1024.0f), static_cast<_Float16>(1024.0f)};
+    const uint32_t lw = (b.lo[j >> 1] >> (16 * (j & 1))) & 0xffffu;  // 8 two-bit fields
+    const uint32_t hw = (b.hi >> (8 * j)) & 0xffu;                   // 8 bits
+    U4 out;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const uint32_t l4 = lw >> (4 * p), h2 = hw >> (2 * p);
+        const uint32_t qa = (l4 & 3u) | ((h2 & 1u) << 2);
+        const uint32_t qb = ((l4 >> 2) & 3u) | ((h2 & 2u) << 1);
+        out.v[p] = as_u32(__builtin_elementwise_fma(as_h2(0x64006400u | qa | (qb << 16)) - k1024, d2, b2));
+    }
+    return out;
+}
+
 __device__ __forceinline__ uint32_t pack_h2(float lo, float hi) {
     const half2v h = {static_cast<_Float16>(lo), static_cast<_Float16>(hi)};
     return as_u32(h);
@@ -77,7 +133,8 @@ __device__ __forceinline__ float load_b(const void* b, int is_f16, size_t idx) {
 }
 
 // grid (K steps, token groups), 256 threads = 4 instructions x 64 lanes of one (step, group).
-template <bool X_F16>
+// INTERLEAVE: the x0 x4 x1 x5 .. order of the Q4 decoder; false = memory order (sibling formats).
+template <bool X_F16, bool INTERLEAVE>
 __global__ __launch_bounds__(256) void pack_x_kernel(const void* __restrict__ xv, uint32_t m, uint32_t k,
                                                      uint4* __restrict__ xp) {
     const uint32_t s = blockIdx.x, t = blockIdx.y, groups = gridDim.y;
@@ -89,25 +146,37 @@ __global__ __launch_bounds__(256) void pack_x_kernel(const void* __restrict__ xv
         if (X_F16) {
             const uint4 c = *reinterpret_cast<const uint4*>(static_cast<const _Float16*>(xv) +
                                                             static_cast<size_t>(token) * k + koff);
-            out.x = __builtin_amdgcn_perm(c.z, c.x, 0x05040100u);  // x0..x7 -> x0 x4 x1 x5 x2 x6 x3 x7
-            out.y = __builtin_amdgcn_perm(c.z, c.x, 0x07060302u);
-            out.z = __builtin_amdgcn_perm(c.w, c.y, 0x05040100u);
-            out.w = __builtin_amdgcn_perm(c.w, c.y, 0x07060302u);
+            if (INTERLEAVE) {
+                out.x = __builtin_amdgcn_perm(c.z, c.x, 0x05040100u);  // x0..x7 -> x0 x4 x1 x5 x2 x6 x3 x7
+                out.y = __builtin_amdgcn_perm(c.z, c.x, 0x07060302u);
+                out.z = __builtin_amdgcn_perm(c.w, c.y, 0x05040100u);
+                out.w = __builtin_amdgcn_perm(c.w, c.y, 0x07060302u);
+            } else {
+                out = c;
+            }
         } else {
             const float4* p = reinterpret_cast<const float4*>(static_cast<const float*>(xv) +
                                                               static_cast<size_t>(token) * k + koff);
             const float4 lo = p[0], hi = p[1];
-            out.x = pack_h2(lo.x, hi.x);
-            out.y = pack_h2(lo.y, hi.y);
-            out.z = pack_h2(lo.z, hi.z);
-            out.w = pack_h2(lo.w, hi.w);
+            if (INTERLEAVE) {
+                out.x = pack_h2(lo.x, hi.x);
+                out.y = pack_h2(lo.y, hi.y);
+                out.z = pack_h2(lo.z, hi.z);
+                out.w = pack_h2(lo.w, hi.w);
+            } else {
+                out.x = pack_h2(lo.x, lo.y);
+                out.y = pack_h2(lo.z, lo.w);
+                out.z = pack_h2(hi.x, hi.y);
+                out.w = pack_h2(hi.z, hi.w);
+            }
         }
     }
     xp[((static_cast<size_t>(s) * groups + t) * 4 + j) * 64 + lane] = out;
 }
 
 // RT: 16-row weight tiles per wave (rows per workgroup = 16 RT).  grid (ceil(N / 16 RT), token tiles).
-template <int RT>
+// FMT: 0 = Q4, 1 = Q8_0, 2 = Q3 blocks.
+template <int RT, int FMT>
 __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __restrict__ w, uint32_t n, uint32_t k,
                                                                 const uint4* __restrict__ xp, uint32_t m,
                                                                 float* __restrict__ y, LoraEpilogue lora) {
@@ -126,16 +195,18 @@ __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __
     const uint32_t steps_total = (nb + 3) / 4;
     const uint32_t cnt = steps_total > static_cast<uint32_t>(wave) ? (steps_total - wave + kWavesK - 1) / kWavesK : 0;
 
-    const uint32_t* w_row[RT];
+    typedef typename WBlockOf<FMT>::type WBlock;
+    constexpr uint32_t kBytes = WBlockOf<FMT>::kBytes;
+    const uint8_t* w_row[RT];
 #pragma unroll
     for (int u = 0; u < RT; ++u) {
         uint32_t row = n0 + 16 * u + lr;
         row = row < n ? row : n - 1;
-        w_row[u] = reinterpret_cast<const uint32_t*>(w) + static_cast<size_t>(row) * (nb * 5);
+        w_row[u] = w + static_cast<size_t>(row) * (nb * kBytes);
     }
 
     struct Unit {
-        Q4BlockRaw wb[RT];
+        WBlock wb[RT];
         uint4 x[4][4];  // [token group][instruction]
     };
     // i-th step of this wave
@@ -144,7 +215,7 @@ __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __
         uint32_t blk = s * 4 + g;
         blk = blk < nb ? blk : nb - 1;
 #pragma unroll
-        for (int r = 0; r < RT; ++r) u.wb[r] = *reinterpret_cast<const Q4BlockRaw*>(w_row[r] + blk * 5);
+        for (int r = 0; r < RT; ++r) u.wb[r] = *reinterpret_cast<const WBlock*>(w_row[r] + blk * kBytes);
         const uint4* xs = xp + (static_cast<size_t>(s) * groups + tg0) * 256 + lane;
 #pragma unroll
         for (int t = 0; t < 4; ++t)
@@ -164,12 +235,17 @@ __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __
         const bool live = (wave + i * kWavesK) * 4 + g < nb;  // K tail: a block past the end of the row counts as zero
 #pragma unroll
         for (int r = 0; r < RT; ++r) {
-            const uint32_t sb = live ? u.wb[r].sb : 0u;
+            uint32_t sb;
+            if constexpr (FMT == 1) sb = live ? static_cast<uint32_t>(u.wb[r].d) : 0u;  // scale only
+            else sb = live ? u.wb[r].sb : 0u;
             const half2v d2 = as_h2(__builtin_amdgcn_perm(sb, sb, 0x01000100u));
             const half2v b2 = as_h2(__builtin_amdgcn_perm(sb, sb, 0x03020302u));
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const U4 a = dequant8(live ? u.wb[r].q[j] : 0u, d2, b2);
+                U4 a;
+                if constexpr (FMT == 0) a = dequant8(live ? u.wb[r].q[j] : 0u, d2, b2);
+                else if constexpr (FMT == 1) a = dequant8_q8(u.wb[r].q[2 * j], u.wb[r].q[2 * j + 1], d2);
+                else a = dequant8_q3(u.wb[r], j, d2, b2);
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
                     if (static_cast<uint32_t>(t) < ntg)
@@ -266,12 +342,12 @@ __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __
     }
 }
 
-template <int RT>
+template <int RT, int FMT>
 void launch_rt(const uint8_t* w, uint32_t n, uint32_t k, const uint4* xp, uint32_t m, float* y, const LoraEpilogue& lora,
                hipStream_t stream) {
     const dim3 grid((n + 16 * RT - 1) / (16 * RT), (m + kTokens - 1) / kTokens);
     const size_t lds = static_cast<size_t>(kWavesK / 2) * RT * 4 * 64 * sizeof(float4v);
-    hipLaunchKernelGGL((gemm_q4_skinny<RT>), grid, dim3(64 * kWavesK), lds, stream, w, n, k, xp, m, y, lora);
+    hipLaunchKernelGGL((gemm_q4_skinny<RT, FMT>), grid, dim3(64 * kWavesK), lds, stream, w, n, k, xp, m, y, lora);
 }
 
 }  // namespace
@@ -288,18 +364,34 @@ size_t gemm_skinny_scratch_bytes(uint32_t k, uint32_t m) {
     return steps * groups * 256 * sizeof(uint4);
 }
 
-void launch_gemm_skinny(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
-                        const LoraEpilogue& lora, void* packed_x, hipStream_t stream) {
+namespace {
+
+template <int FMT>
+void launch_fmt(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
+                const LoraEpilogue& lora, void* packed_x, hipStream_t stream) {
     const uint32_t steps = (k / kBlockWeights + 3) / 4, groups = (m + 15) / 16;
     uint4* xp = static_cast<uint4*>(packed_x);
-    if (x_is_f16) hipLaunchKernelGGL((pack_x_kernel<true>), dim3(steps, groups), dim3(256), 0, stream, x, m, k, xp);
-    else hipLaunchKernelGGL((pack_x_kernel<false>), dim3(steps, groups), dim3(256), 0, stream, x, m, k, xp);
+    constexpr bool kInterleave = FMT == 0;
+    if (x_is_f16)
+        hipLaunchKernelGGL((pack_x_kernel<true, kInterleave>), dim3(steps, groups), dim3(256), 0, stream, x, m, k, xp);
+    else
+        hipLaunchKernelGGL((pack_x_kernel<false, kInterleave>), dim3(steps, groups), dim3(256), 0, stream, x, m, k, xp);
     // Every workgroup reads the whole packed X of its token tile, so wider row tiles cut that
-    // traffic; they are taken only while at least one workgroup per CU remains.
+    // traffic; they are taken only while at least 128 workgroups remain.
     const uint32_t tiles16 = (n + 15) / 16;
-    if (tiles16 >= 4 * 128) launch_rt<4>(w, n, k, xp, m, y, lora, stream);
-    else if (tiles16 >= 2 * 128) launch_rt<2>(w, n, k, xp, m, y, lora, stream);
-    else launch_rt<1>(w, n, k, xp, m, y, lora, stream);
+    // (the 34-byte Q8_0 blocks of four row tiles do not fit the register file)
+    if (FMT != 1 && tiles16 >= 4 * 128) launch_rt<4, FMT>(w, n, k, xp, m, y, lora, stream);
+    else if (tiles16 >= 2 * 128) launch_rt<2, FMT>(w, n, k, xp, m, y, lora, stream);
+    else launch_rt<1, FMT>(w, n, k, xp, m, y, lora, stream);
+}
+
+}  // namespace
+
+void launch_gemm_skinny(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
+                        const LoraEpilogue& lora, void* packed_x, hipStream_t stream, int fmt) {
+    if (fmt == 1) launch_fmt<1>(w, n, k, x, x_is_f16, m, y, lora, packed_x, stream);
+    else if (fmt == 2) launch_fmt<2>(w, n, k, x, x_is_f16, m, y, lora, packed_x, stream);
+    else launch_fmt<0>(w, n, k, x, x_is_f16, m, y, lora, packed_x, stream);
 }
 
 }  // namespace lq4

@@ -122,8 +122,9 @@ void launch_gemm_q3(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int
 // (gemm_skinny_scratch_bytes bytes at `packed_x`), then a kernel without LDS staging.
 bool gemm_skinny_wants(uint32_t n, uint32_t k, uint32_t m);
 size_t gemm_skinny_scratch_bytes(uint32_t k, uint32_t m);
+// fmt: 0 = Q4 blocks, 1 = Q8_0, 2 = Q3.
 void launch_gemm_skinny(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
-                        const LoraEpilogue& lora, void* packed_x, hipStream_t stream);
+                        const LoraEpilogue& lora, void* packed_x, hipStream_t stream, int fmt = 0);
 
 void launch_probe_read(const void* p, size_t nbytes, uint32_t* sink, hipStream_t stream);
 void launch_probe_copy(const void* src, void* dst, size_t nbytes, hipStream_t stream);

@@ -100,12 +100,6 @@ int resolve_weight(const lq4_weight* w, uint64_t extra, uint32_t n, uint32_t k,
     return LQ4_OK;
 }
 
-// The sibling formats have only the 128 x 128 tile kernel beside the few-token kernel, and it does not
-// cut K: with fewer weight tiles than half the compute units the few-token kernel also serves 65..128 rows.
-bool sibling_skinny_wants(uint32_t n, uint32_t k, uint32_t m) {
-    return gemm_skinny_wants(n, k, m) || (m <= 128 && (n + 127) / 128 < 128);
-}
-
 // The same for a buffer of sibling-format blocks: Q8_0 (34 bytes, 2-byte aligned) or Q3 (16 bytes,
 // 4-byte aligned).
 int resolve_weight_sibling(const lq4_weight* w, uint64_t extra, uint32_t n, uint32_t k, const char* fmt,
@@ -327,7 +321,7 @@ int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
     // mid-sized matrices only (measured: behind for 512 x 2048, where its two launches dominate,
     // and for 12288 x 2048, where the GEMV kernel's grid already fills the chip).
     const uint64_t weights = static_cast<uint64_t>(n) * k;
-    if ((batch >= 9 || (batch >= 5 && n < 8192 && weights >= 6000000)) && gemm_skinny_wants(n, k, batch)) {
+    if (batch >= 9 || (batch >= 5 && n < 8192 && weights >= 6000000)) {
         rc = ensure_scratch(ctx, gemm_skinny_scratch_bytes(k, batch));
         if (rc) return rc;
         launch_gemm_skinny(wp, n, k, x_dev, 0, batch, y_dev, ep, ctx->moe_scratch, s);
@@ -700,15 +694,18 @@ int lq4_gemm_q8(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
     if (m == 1 && x_dtype == LQ4_F32 && gemv_q8_lds_bytes(k) <= 128 * 1024) {
         launch_gemv_q8_b1(wp, n, k, static_cast<const float*>(x_dev), y_dev, s);
         ctx->counters.gemv++;
-    } else if (sibling_skinny_wants(n, k, m)) {
+    } else if (m <= 64 || gemm_skinny_wants(n, k, m)) {
         // few rows: operands packed once, the few-token matrix-core kernel with this format's decoder
+        // (always for one token tile: the sibling tile kernel is no match for it there)
         const int src = ensure_scratch(ctx, gemm_skinny_scratch_bytes(k, m));
         if (src) return src;
         const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};
         launch_gemm_skinny(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, none, ctx->moe_scratch, s, 1);
         ctx->counters.gemm++;
     } else {
-        launch_gemm_q8(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, s);
+        const int src = ensure_scratch(ctx, gemm_sibling_scratch_floats(n, k, m) * sizeof(float));
+        if (src) return src;
+        launch_gemm_q8(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, reinterpret_cast<float*>(ctx->moe_scratch), s);
         ctx->counters.gemm++;
     }
     LQ4_HIP(hipGetLastError());
@@ -738,15 +735,18 @@ int lq4_gemm_q3(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
     if (m == 1 && x_dtype == LQ4_F32 && gemv_q3_lds_bytes(k) <= 128 * 1024) {
         launch_gemv_q3_b1(wp, n, k, static_cast<const float*>(x_dev), y_dev, s);
         ctx->counters.gemv++;
-    } else if (sibling_skinny_wants(n, k, m)) {
+    } else if (m <= 64 || gemm_skinny_wants(n, k, m)) {
         // few rows: operands packed once, the few-token matrix-core kernel with this format's decoder
+        // (always for one token tile: the sibling tile kernel is no match for it there)
         const int src = ensure_scratch(ctx, gemm_skinny_scratch_bytes(k, m));
         if (src) return src;
         const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};
         launch_gemm_skinny(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, none, ctx->moe_scratch, s, 2);
         ctx->counters.gemm++;
     } else {
-        launch_gemm_q3(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, s);
+        const int src = ensure_scratch(ctx, gemm_sibling_scratch_floats(n, k, m) * sizeof(float));
+        if (src) return src;
+        launch_gemm_q3(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, reinterpret_cast<float*>(ctx->moe_scratch), s);
         ctx->counters.gemm++;
     }
     LQ4_HIP(hipGetLastError());

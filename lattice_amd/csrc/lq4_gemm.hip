@@ -35,6 +35,7 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float float16v __attribute__((ext_vector_type(16)));
+typedef float float4v __attribute__((ext_vector_type(4)));
 
 constexpr int BM = 128;         // tokens per workgroup
 constexpr int BK = 64;          // two Q4 blocks along K
@@ -148,10 +149,21 @@ __device__ __forceinline__ uint4 dequant8_q8(uint32_t qa, uint32_t qb, half2v d2
 // LORA: compiled with the LoRA step (kept out of the plain kernel, whose register allocation it
 // would disturb).
 // FMT: 0 = Q4 blocks, 1 = Q8_0 blocks, 2 = Q3 blocks (the siblings have no LoRA step).
+//
+// K slices.  With fewer tiles than workgroup slots the launch cuts K into `slices.count` ranges of
+// `slices.steps` K steps: workgroup b computes tile b / count over range b % count and stores its
+// partial tile, row-major [BM][BN_], at slices.partial[b]; gemm_sum_slices adds the ranges of a tile
+// in order.  count == 1 writes y directly.
+struct KSlices {
+    uint32_t count;
+    uint32_t steps;
+    float* partial;
+};
+
 template <bool X_F16, int BN_, bool LORA, int FMT = 0>
 __global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
     const uint8_t* __restrict__ w, uint32_t n, uint32_t k, const void* __restrict__ xv, uint32_t m,
-    float* __restrict__ y, LoraEpilogue lora) {
+    float* __restrict__ y, LoraEpilogue lora, KSlices slices) {
     extern __shared__ __attribute__((aligned(16))) _Float16 lds[];  // 2 x (X tile | W tile)
     constexpr int kThreads = 2 * BN_;
     constexpr int kWavesN = BN_ / 64;
@@ -166,16 +178,21 @@ __global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
     const int wn = (wave % kWavesN) * 64;
 
     // ---- tile id -> (token tile, weight tile), grouped so co-resident tiles share activations
+    const uint32_t tile = blockIdx.x / slices.count;
+    const uint32_t slice = blockIdx.x - tile * slices.count;
     const uint32_t tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN_ - 1) / BN_;
     const uint32_t per_group = kGroupM * tiles_n;
-    const uint32_t group = blockIdx.x / per_group;
+    const uint32_t group = tile / per_group;
     const uint32_t first_m = group * kGroupM;
     const uint32_t group_m = tiles_m - first_m < kGroupM ? tiles_m - first_m : kGroupM;
-    const uint32_t in_group = blockIdx.x - group * per_group;
+    const uint32_t in_group = tile - group * per_group;
     const uint32_t m0 = (first_m + in_group % group_m) * BM;
     const uint32_t n0 = (in_group / group_m) * BN_;
 
-    const uint32_t nb = k / kBlockWeights;
+    // This workgroup's K range in steps; blocks at or past `nb` (the end of the range) count as zeros.
+    const uint32_t nb_row = k / kBlockWeights;  // blocks per weight row
+    const uint32_t s_begin = slice * slices.steps;
+    const uint32_t nb = nb_row < 2 * (s_begin + slices.steps) ? nb_row : 2 * (s_begin + slices.steps);
     const uint32_t nsteps = (nb + 1) / 2;
 
     float16v acc[2][2];
@@ -192,8 +209,8 @@ __global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
     const bool w_live_row = w_row < n;
     typedef typename WBlockOf<FMT>::type WBlock;
     const uint32_t* w_ptr =
-        reinterpret_cast<const uint32_t*>(w) + static_cast<size_t>(w_live_row ? w_row : 0) * (nb * 5);
-    const uint8_t* w_ptr8 = w + static_cast<size_t>(w_live_row ? w_row : 0) * (nb * (FMT == 2 ? 16 : 34));  // FMT != 0
+        reinterpret_cast<const uint32_t*>(w) + static_cast<size_t>(w_live_row ? w_row : 0) * (nb_row * 5);
+    const uint8_t* w_ptr8 = w + static_cast<size_t>(w_live_row ? w_row : 0) * (nb_row * (FMT == 2 ? 16 : 34));  // FMT != 0
     const int w_half = tid & 1;
     // activations: chunk i of this thread is (row, part) = divmod(tid + kThreads*i, chunks per row)
     const uint8_t* x_ptr[XCH];
@@ -313,11 +330,11 @@ __global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
     // Steps past the end of K (at most three) run on zeros, which keeps the body branch-free.
     XStage xa, xb;
     WBlock w0, w1, w2, w3;
-    load_x(xa, 0);
-    load_w(w0, 0);
-    load_w(w1, 1);
-    load_w(w2, 2);
-    for (uint32_t s = 0; s < nsteps; s += 4) {
+    load_x(xa, s_begin);
+    load_w(w0, s_begin);
+    load_w(w1, s_begin + 1);
+    load_w(w2, s_begin + 2);
+    for (uint32_t s = s_begin; s < nsteps; s += 4) {
         store_tiles(xa, w0, s, xs0, ws0);
         __syncthreads();
         load_x(xb, s + 1);
@@ -344,7 +361,7 @@ __global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
     //      acc[token, n] += sum_r (scale * t[token, r]) * B[n, r].
     // Both factors are split hi + lo/2048 into f16 so the delta keeps f32-level accuracy:
     // t.B = thi.Bhi + tlo.(Bhi/2048) + (thi/2048).Blo; the last term vanishes for f16-stored B.
-    if (LORA && lora.rank) {
+    if (LORA && lora.rank && slice == 0) {
         const int r = lane & 31;
         for (uint32_t r0 = 0; r0 < lora.rank; r0 += 16) {
             const uint32_t rbase = r0 + 8 * (lane >> 5);  // this lane's eight rank indices
@@ -384,6 +401,18 @@ __global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
 
     // ---- epilogue: accumulator element v of lane l is
     //      row 8*(v/4) + 4*(l/32) + v%4, column l%32 of its 32x32 tile
+    if (slices.count > 1) {
+        float* ptile = slices.partial + static_cast<size_t>(blockIdx.x) * (BM * BN_);
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    ptile[(wm + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3)) * BN_ + wn + j * 32 + (lane & 31)] =
+                        acc[i][j][v];
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -397,10 +426,67 @@ __global__ __launch_bounds__(2 * BN_, BN_ == 128 ? 2 : 1) void gemm_q4_mfma(
         }
 }
 
+// y tile = sum over the K slices of its partial tiles, in slice order.  grid (tiles, BM * BN_ / 1024);
+// a thread owns four consecutive weight rows of one token.
+template <int BN_>
+__global__ __launch_bounds__(256) void gemm_sum_slices(const float* __restrict__ partial, uint32_t count, uint32_t m,
+                                                       uint32_t n, float* __restrict__ y) {
+    const uint32_t tile = blockIdx.x;
+    const uint32_t tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN_ - 1) / BN_;
+    const uint32_t per_group = kGroupM * tiles_n;
+    const uint32_t group = tile / per_group;
+    const uint32_t first_m = group * kGroupM;
+    const uint32_t group_m = tiles_m - first_m < kGroupM ? tiles_m - first_m : kGroupM;
+    const uint32_t in_group = tile - group * per_group;
+    const uint32_t m0 = (first_m + in_group % group_m) * BM;
+    const uint32_t n0 = (in_group / group_m) * BN_;
+
+    const uint32_t local = (blockIdx.y * 256 + threadIdx.x) * 4;
+    const uint32_t token = m0 + local / BN_, row = n0 + local % BN_;
+    if (token >= m || row >= n) return;
+    const float* src = partial + static_cast<size_t>(tile) * count * (BM * BN_) + local;
+    float4v v = *reinterpret_cast<const float4v*>(src);
+    for (uint32_t sl = 1; sl < count; ++sl) v += *reinterpret_cast<const float4v*>(src + static_cast<size_t>(sl) * (BM * BN_));
+    float* dst = y + static_cast<size_t>(token) * n + row;
+    if ((n & 3u) == 0 && (reinterpret_cast<uintptr_t>(y) & 15u) == 0) {
+        *reinterpret_cast<float4v*>(dst) = v;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (row + e < n) dst[e] = v[e];
+    }
+}
+
+// K slicing of a shape for the tile kernel: slice count and steps per slice.  Two workgroups fit a
+// compute unit, so up to 512 run at once; a slice keeps at least eight K steps (a multiple of the
+// loop's unroll of four), and its partial tile costs a 64 KB write and read.
+struct TileSlices {
+    uint32_t count, steps;
+};
+template <int BN_>
+TileSlices plan_tile_slices(uint32_t n, uint32_t k, uint32_t m) {
+    const uint32_t tiles = ((n + BN_ - 1) / BN_) * ((m + BM - 1) / BM);
+    const uint32_t nsteps = (k / kBlockWeights + 1) / 2;
+    const uint32_t slots = BN_ == 128 ? 512 : 256;
+    uint32_t want = slots / tiles;
+    if (want > 16) want = 16;
+    if (want < 2 || nsteps < 16) return {1, nsteps};
+    uint32_t per = (nsteps + want - 1) / want;
+    per = (per + 3) / 4 * 4;
+    if (per < 8) per = 8;
+    const uint32_t count = (nsteps + per - 1) / per;
+    if (count < 2) return {1, nsteps};
+    return {count, per};
+}
+
+// partial: scratch of tile_scratch_floats() floats, or nullptr to keep K whole.
 template <bool X_F16, int BN_, bool LORA, int FMT = 0>
 void launch_tile(const uint8_t* w, uint32_t n, uint32_t k, const void* x, uint32_t m, float* y,
-                 const LoraEpilogue& lora, hipStream_t stream) {
+                 const LoraEpilogue& lora, hipStream_t stream, float* partial = nullptr) {
     const uint32_t tiles = ((n + BN_ - 1) / BN_) * ((m + BM - 1) / BM);
+    TileSlices ts = plan_tile_slices<BN_>(n, k, m);
+    if (!partial || (LORA && lora.rank)) ts = TileSlices{1, (k / kBlockWeights + 1) / 2};
+    const KSlices slices{ts.count, ts.steps, partial};
     const size_t lds = 2 * (BM + BN_) * kPitch * sizeof(_Float16);
     static bool attr_set = false;
     if (!attr_set) {
@@ -408,8 +494,11 @@ void launch_tile(const uint8_t* w, uint32_t n, uint32_t k, const void* x, uint32
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         attr_set = true;
     }
-    hipLaunchKernelGGL((gemm_q4_mfma<X_F16, BN_, LORA, FMT>), dim3(tiles), dim3(2 * BN_), lds, stream, w, n, k, x, m, y,
-                       lora);
+    hipLaunchKernelGGL((gemm_q4_mfma<X_F16, BN_, LORA, FMT>), dim3(tiles * ts.count), dim3(2 * BN_), lds, stream, w, n,
+                       k, x, m, y, lora, slices);
+    if (ts.count > 1)
+        hipLaunchKernelGGL((gemm_sum_slices<BN_>), dim3(tiles, BM * BN_ / 1024), dim3(256), 0, stream, partial, ts.count,
+                           m, n, y);
 }
 
 
@@ -463,18 +552,24 @@ void launch_gemm(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_
     }
 }
 
+size_t gemm_sibling_scratch_floats(uint32_t n, uint32_t k, uint32_t m) {
+    const TileSlices ts = plan_tile_slices<128>(n, k, m);
+    if (ts.count < 2) return 0;
+    return static_cast<size_t>((n + 127) / 128) * ((m + BM - 1) / BM) * ts.count * (BM * 128);
+}
+
 void launch_gemm_q8(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
-                    hipStream_t stream) {
+                    float* scratch, hipStream_t stream) {
     const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};
-    if (x_is_f16) launch_tile<true, 128, false, 1>(w, n, k, x, m, y, none, stream);
-    else launch_tile<false, 128, false, 1>(w, n, k, x, m, y, none, stream);
+    if (x_is_f16) launch_tile<true, 128, false, 1>(w, n, k, x, m, y, none, stream, scratch);
+    else launch_tile<false, 128, false, 1>(w, n, k, x, m, y, none, stream, scratch);
 }
 
 void launch_gemm_q3(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
-                    hipStream_t stream) {
+                    float* scratch, hipStream_t stream) {
     const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};
-    if (x_is_f16) launch_tile<true, 128, false, 2>(w, n, k, x, m, y, none, stream);
-    else launch_tile<false, 128, false, 2>(w, n, k, x, m, y, none, stream);
+    if (x_is_f16) launch_tile<true, 128, false, 2>(w, n, k, x, m, y, none, stream, scratch);
+    else launch_tile<false, 128, false, 2>(w, n, k, x, m, y, none, stream, scratch);
 }
 
 }  // namespace lq4

@@ -353,10 +353,17 @@ void launch_rt(const uint8_t* w, uint32_t n, uint32_t k, const uint4* xp, uint32
 }  // namespace
 
 bool gemm_skinny_wants(uint32_t n, uint32_t k, uint32_t m) {
-    // one token tile always; two while the matrix is small enough that the large-tile kernels cannot
-    // fill the chip (measured: ahead at 12288 x 2048, behind at 17408 x 5120)
-    return k >= kBlockWeights &&
-           (m <= kTokens || (m <= 2 * kTokens && static_cast<uint64_t>(n) * k <= (1ull << 25)));
+    // Against the large-tile kernel, which wastes the empty part of its 128-token tile but shares the
+    // activations of a tile among 256 rows where this kernel re-reads them for every 16..64 rows
+    // (measured on 6M..500M-weight matrices): up to 16 tokens are always served here; one token tile
+    // unless the matrix is large
+    // (above 2^26 weights) and either more than 32 tokens, fewer than 8192 rows (too few workgroups
+    // here) or more than 2^28 weights; two token tiles only up to 2^24 weights.
+    if (k < kBlockWeights) return false;
+    const uint64_t weights = static_cast<uint64_t>(n) * k;
+    if (m <= 16) return true;
+    if (m <= kTokens) return weights <= (1ull << 26) || (m <= 32 && n >= 8192 && weights <= (1ull << 28));
+    return m <= 2 * kTokens && weights <= (1ull << 24);
 }
 
 size_t gemm_skinny_scratch_bytes(uint32_t k, uint32_t m) {

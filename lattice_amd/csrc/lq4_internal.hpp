@@ -110,13 +110,16 @@ void launch_gemm_wreg(const uint8_t* w, uint32_t n, uint32_t k, const void* x, i
 size_t gemv_q8_lds_bytes(uint32_t k);
 void launch_gemv_q8_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, hipStream_t stream);
 void launch_gemm_q8(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
-                    hipStream_t stream);
+                    float* scratch, hipStream_t stream);
+// Floats of scratch the sibling tile GEMMs use to cut K on shapes with few tiles (0 = none; a null
+// scratch pointer keeps K whole).
+size_t gemm_sibling_scratch_floats(uint32_t n, uint32_t k, uint32_t m);
 
 // Q3 sibling format (16-byte blocks: f16 scale, f16 bias, 2-bit and 1-bit planes): same pair of paths.
 size_t gemv_q3_lds_bytes(uint32_t k);
 void launch_gemv_q3_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, hipStream_t stream);
 void launch_gemm_q3(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
-                    hipStream_t stream);
+                    float* scratch, hipStream_t stream);
 
 // Few-token variant (up to 128 tokens): activations packed once into matrix-core operand order
 // (gemm_skinny_scratch_bytes bytes at `packed_x`), then a kernel without LDS staging.

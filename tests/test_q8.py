@@ -136,7 +136,8 @@ def test_q8_gemv_matches_oracle(be, n, k):
 
 
 GEMM_CASES = [(2, 64, 64, "f32"), (8, 2048, 2048, "f32"), (16, 37, 96, "f32"), (130, 300, 256, "f16"),
-              (512, 256, 1024, "f16"), (33, 129, 4160, "f32")]
+              (512, 256, 1024, "f16"), (33, 129, 4160, "f32"),
+              (200, 300, 2080, "f32"), (96, 130, 1056, "f16"), (257, 128, 4096, "f16")]
 
 
 @pytest.mark.gpu

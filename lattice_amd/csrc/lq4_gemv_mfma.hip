@@ -307,8 +307,7 @@ __global__ __launch_bounds__(kThreads) void gemv_q4_mfma(GemvArgs p) {
                 acc[t][c] = 0.0f;
                 v = dpp_add<0x124>(v);  // row_ror:4
                 v = dpp_add<0x128>(v);  // row_ror:8 -> sum over the row's lanes with this j
-                v += __shfl_xor(v, 16, 64);
-                v += __shfl_xor(v, 32, 64);
+                v = sum_over_rows(v);
                 if (KS > 1 && lane < 4) red[(it & 1) * kRedFloats + ((wave * T + t) * NCOLS + c) * 4 + lane] = v;
                 if (KS == 1) acc[t][c] = v;  // reused below as the total
             }

@@ -173,6 +173,21 @@ void launch_topk(const float* logits, uint32_t n, uint32_t k, void* scratch, flo
                  hipStream_t stream);
 
 // ---- device helpers ---------------------------------------------------------------
+// v summed over the four 16-lane rows of a wave: every lane ends with the total of the four lanes
+// at its position in a row, (r0 + r1) + (r2 + r3) seen from rows 0/1 and mirrored from rows 2/3, the
+// same sums as adding the lanes at xor 16 and then xor 32.  The two row-swap instructions of this
+// chip exchange registers directly, where a general lane shuffle goes through the LDS crossbar at
+// ~100 cycles of latency each.
+__device__ __forceinline__ float sum_over_rows(float v) {
+    float a = v, b = v;
+    asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));  // a: rows 0 0 2 2, b: rows 1 1 3 3
+    v = a + b;
+    a = v;
+    b = v;
+    asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));  // a: low half twice, b: high half twice
+    return a + b;
+}
+
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t bits16) {
     // v_cvt_f32_f16 widens exactly, subnormals included (f16 denormals are not flushed
     // in the default HIP float mode).

@@ -264,10 +264,20 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
     const uint32_t c = blockIdx.x * 256 + threadIdx.x;
     if (c >= hidden) return;
     float acc = 0.0f;
-    for (uint32_t s = 0; s < top_k; ++s) {
-        const int32_t e = ids[t * top_k + s];
-        if (e < 0 || e >= static_cast<int32_t>(num_experts)) continue;
-        acc += weights[t * top_k + s] * o[static_cast<size_t>(t * top_k + s) * hidden + c];
+    // eight slots at a time: their routing entries, then their rows, are loaded together
+    for (uint32_t s0 = 0; s0 < top_k; s0 += 8) {
+        float wv[8], ov[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t s = s0 + i < top_k ? s0 + i : top_k - 1;
+            const int32_t e = ids[t * top_k + s];
+            const bool ok = s0 + i < top_k && e >= 0 && e < static_cast<int32_t>(num_experts);
+            wv[i] = ok ? weights[t * top_k + s] : 0.0f;
+            ov[i] = o[static_cast<size_t>(t * top_k + s) * hidden + c];
+            if (!ok) ov[i] = 0.0f;  // rows of invalid slots are never written
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc += wv[i] * ov[i];
     }
     y[static_cast<size_t>(t) * hidden + c] = acc;
 }

@@ -13,6 +13,10 @@
 // of the down projection ([E, H, I]), o[pair, r] = W . h[pair].
 #include "lq4_internal.hpp"
 
+#ifndef LQ4_MOE_RING
+#define LQ4_MOE_RING 3
+#endif
+
 namespace lq4 {
 
 namespace {
@@ -26,6 +30,7 @@ constexpr int kTok = 4;           // pairs per workgroup pass
 constexpr int kCols = 2 * kTok;   // hi and lo column per pair
 constexpr float kLoScale = 2048.0f;
 constexpr float kTwo24 = 16777216.0f;
+constexpr int kRing = LQ4_MOE_RING;
 constexpr uint32_t kPitch16 = (kCols * 64 + 16) / 16;  // per K block: 8 columns of 32 f16, then 4 sums
 
 struct __attribute__((packed, aligned(4))) Q4BlockRaw {
@@ -132,11 +137,11 @@ __global__ __launch_bounds__(kThreads) void moe_expert_mfma(MoeGemvArgs p) {
         buf[1] = *reinterpret_cast<const Q4BlockRaw*>(wbase + static_cast<size_t>(rb) * (nb * 5) + blk * 5);
     };
 
-    Q4BlockRaw buf_a[2], buf_b[2], buf_c[2];
-    if (units) {
-        load_unit(buf_a, 0);
-        load_unit(buf_b, units > 1 ? 1 : 0);
-    }
+    // ring of kRing unit buffers: kRing - 1 units are in flight while one is consumed
+    Q4BlockRaw buf[kRing][2];
+#pragma unroll
+    for (int i = 0; i < kRing - 1; ++i)
+        if (static_cast<uint32_t>(i) < units) load_unit(buf[i], i);
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- stage the activations of this pass: 8 values per (block, dword) item per pair ---------
@@ -203,7 +208,7 @@ __global__ __launch_bounds__(kThreads) void moe_expert_mfma(MoeGemvArgs p) {
         for (int c = 0; c < kCols; ++c) acc[t][c] = 0.0f;
 
     auto process = [&](Q4BlockRaw (&cur)[2], Q4BlockRaw (&nxt)[2], uint32_t u) {
-        if (u + 2 < units) load_unit(nxt, u + 2);
+        if (u + kRing - 1 < units) load_unit(nxt, u + kRing - 1);
         const uint32_t t_idx = u / n_local, q = u - t_idx * n_local;
         const uint32_t blk_raw = (ks + q * KS) * 16 + g;
         const bool live = blk_raw < nb;
@@ -266,23 +271,20 @@ __global__ __launch_bounds__(kThreads) void moe_expert_mfma(MoeGemvArgs p) {
                 acc[t][c] = 0.0f;
                 v = dpp_add<0x124>(v);  // row_ror:4
                 v = dpp_add<0x128>(v);  // row_ror:8
-                v += __shfl_xor(v, 16, 64);
-                v += __shfl_xor(v, 32, 64);
+                v = sum_over_rows(v);
                 if (lane < 4) red[(((wave * tp + t_idx) * 2 + t) * kCols + c) * 4 + lane] = v;
             }
     };
 
     if (units) {
         uint32_t q = 0, t_idx = 0;
-        for (uint32_t u = 0; u < units; u += 3) {
-            process(buf_a, buf_c, u);
-            if (++q == n_local) { finish(t_idx++); q = 0; }
-            if (u + 1 >= units) break;
-            process(buf_b, buf_a, u + 1);
-            if (++q == n_local) { finish(t_idx++); q = 0; }
-            if (u + 2 >= units) break;
-            process(buf_c, buf_b, u + 2);
-            if (++q == n_local) { finish(t_idx++); q = 0; }
+        for (uint32_t u0 = 0; u0 < units; u0 += kRing) {
+#pragma unroll
+            for (int i = 0; i < kRing; ++i) {
+                if (u0 + i >= units) break;
+                process(buf[i], buf[(i + kRing - 1) % kRing], u0 + i);  // refills the buffer consumed last
+                if (++q == n_local) { finish(t_idx++); q = 0; }
+            }
         }
     } else {
         for (uint32_t t_idx = 0; t_idx < tp; ++t_idx) finish(t_idx);  // zeros: this wave has no K slice

@@ -703,7 +703,7 @@ int lq4_gemm_q8(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
         launch_gemm_skinny(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, none, ctx->moe_scratch, s, 1);
         ctx->counters.gemm++;
     } else {
-        const int src = ensure_scratch(ctx, gemm_sibling_scratch_floats(n, k, m) * sizeof(float));
+        const int src = ensure_scratch(ctx, gemm_sibling_scratch_floats(1, n, k, m) * sizeof(float));
         if (src) return src;
         launch_gemm_q8(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, reinterpret_cast<float*>(ctx->moe_scratch), s);
         ctx->counters.gemm++;
@@ -744,7 +744,7 @@ int lq4_gemm_q3(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
         launch_gemm_skinny(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, none, ctx->moe_scratch, s, 2);
         ctx->counters.gemm++;
     } else {
-        const int src = ensure_scratch(ctx, gemm_sibling_scratch_floats(n, k, m) * sizeof(float));
+        const int src = ensure_scratch(ctx, gemm_sibling_scratch_floats(2, n, k, m) * sizeof(float));
         if (src) return src;
         launch_gemm_q3(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, reinterpret_cast<float*>(ctx->moe_scratch), s);
         ctx->counters.gemm++;

@@ -552,7 +552,29 @@ void launch_gemm(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_
     }
 }
 
-size_t gemm_sibling_scratch_floats(uint32_t n, uint32_t k, uint32_t m) {
+// Sibling formats: the weights-in-registers kernel with the format's decoder, unless the tile
+// kernel is forced (choice 1).  Q8_0 blocks are 1.7 x the bytes and 2-byte aligned, which costs the
+// register kernel more than the tile kernel (measured): it is taken on long, wide matrices only.
+namespace {
+bool sibling_wants_wreg(int fmt, uint32_t n, uint32_t k) {
+    const int forced = g_gemm_choice.load(std::memory_order_relaxed);
+    if (forced == 1) return false;
+    if (forced == 2) return true;
+    return fmt != 1 || (k >= 4096 && n >= 4096);
+}
+
+template <int FMT>
+void launch_sibling(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
+                    float* scratch, hipStream_t stream) {
+    const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};
+    if (sibling_wants_wreg(FMT, n, k)) return launch_gemm_wreg(w, n, k, x, x_is_f16, m, y, none, scratch, stream, FMT);
+    if (x_is_f16) launch_tile<true, 128, false, FMT>(w, n, k, x, m, y, none, stream, scratch);
+    else launch_tile<false, 128, false, FMT>(w, n, k, x, m, y, none, stream, scratch);
+}
+}  // namespace
+
+size_t gemm_sibling_scratch_floats(int fmt, uint32_t n, uint32_t k, uint32_t m) {
+    if (sibling_wants_wreg(fmt, n, k)) return gemm_wreg_scratch_floats(n, k, m);
     const TileSlices ts = plan_tile_slices<128>(n, k, m);
     if (ts.count < 2) return 0;
     return static_cast<size_t>((n + 127) / 128) * ((m + BM - 1) / BM) * ts.count * (BM * 128);
@@ -560,16 +582,12 @@ size_t gemm_sibling_scratch_floats(uint32_t n, uint32_t k, uint32_t m) {
 
 void launch_gemm_q8(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
                     float* scratch, hipStream_t stream) {
-    const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};
-    if (x_is_f16) launch_tile<true, 128, false, 1>(w, n, k, x, m, y, none, stream, scratch);
-    else launch_tile<false, 128, false, 1>(w, n, k, x, m, y, none, stream, scratch);
+    launch_sibling<1>(w, n, k, x, x_is_f16, m, y, scratch, stream);
 }
 
 void launch_gemm_q3(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
                     float* scratch, hipStream_t stream) {
-    const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};
-    if (x_is_f16) launch_tile<true, 128, false, 2>(w, n, k, x, m, y, none, stream, scratch);
-    else launch_tile<false, 128, false, 2>(w, n, k, x, m, y, none, stream, scratch);
+    launch_sibling<2>(w, n, k, x, x_is_f16, m, y, scratch, stream);
 }
 
 }  // namespace lq4

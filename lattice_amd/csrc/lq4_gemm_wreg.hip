@@ -27,6 +27,8 @@
 // bias, so the loop body is free of divergent branches.
 #include "lq4_internal.hpp"
 
+#include <type_traits>
+
 namespace lq4 {
 
 namespace {
@@ -47,6 +49,32 @@ constexpr int NT = TM / 16;                // 16-token tiles per workgroup
 struct __attribute__((packed, aligned(4))) Q4BlockRaw {
     uint32_t sb;    // f16 scale | f16 bias << 16
     uint32_t q[4];  // 32 nibbles, nibble i of dword j = weight 8j + i
+};
+
+// Sibling formats (FMT 1 = Q8_0, 2 = Q3).
+struct __attribute__((packed, aligned(2))) Q8BlockRaw {
+    uint16_t d;     // f16 scale
+    uint32_t q[8];  // 32 x i8, weight i in byte i
+};
+struct __attribute__((packed, aligned(4))) Q3BlockRaw {
+    uint32_t sb;     // f16 scale | f16 bias << 16
+    uint32_t lo[2];  // weight i of 16-weight half h at bits 2i of lo[h]
+    uint32_t hi;     // weight i at bit i
+};
+template <int FMT>
+struct WBlockOf {
+    typedef Q4BlockRaw type;
+    static constexpr uint32_t kBytes = 20;
+};
+template <>
+struct WBlockOf<1> {
+    typedef Q8BlockRaw type;
+    static constexpr uint32_t kBytes = 34;
+};
+template <>
+struct WBlockOf<2> {
+    typedef Q3BlockRaw type;
+    static constexpr uint32_t kBytes = 16;
 };
 
 __device__ __forceinline__ float load_b(const void* b, int is_f16, size_t idx) {
@@ -72,12 +100,25 @@ struct U4 {
 // them one by one in the shadow of matrix-core instructions.  A masked dword OR-ed into the
 // mantissa of 1024.0 (or 64.0) is the pair (1024+n_lo, 1024+n_hi); one packed subtract makes it
 // (n_lo, n_hi) exactly, one packed fma applies scale and bias with a single rounding.
-constexpr int kDqOps = 13;
 struct DqTmp {
-    uint32_t q8;
+    uint32_t q8;   // Q4: dword >> 8;  Q8_0: second sign-flipped dword;  Q3: spread high-plane bits
+    uint32_t qa;   // Q8_0: first sign-flipped dword;  Q3: shifted low-plane dword
     half2v t[4];
 };
-__device__ __forceinline__ void dq_op(int op, uint32_t q, half2v d2, half2v b2, DqTmp& tmp, U4& out) {
+template <int FMT>
+struct DqOps {
+    static constexpr int kOps = 13;
+};
+template <>
+struct DqOps<1> {
+    static constexpr int kOps = 14;
+};
+template <>
+struct DqOps<2> {
+    static constexpr int kOps = 24;
+};
+
+__device__ __forceinline__ void dq_op_q4(int op, uint32_t q, half2v d2, half2v b2, DqTmp& tmp, U4& out) {
     const half2v k1024 = {static_cast<_Float16>(1024.0f), static_cast<_Float16>(1024.0f)};
     const half2v k64 = {static_cast<_Float16>(64.0f), static_cast<_Float16>(64.0f)};
     switch (op) {
@@ -92,6 +133,61 @@ __device__ __forceinline__ void dq_op(int op, uint32_t q, half2v d2, half2v b2, 
         case 8: tmp.t[3] -= k64; break;
         default: out.v[op - 9] = as_u32(__builtin_elementwise_fma(tmp.t[op - 9], d2, b2)); break;
     }
+}
+
+// Q8_0, weights 8j..8j+7 in memory order -> half(q * d): a sign-flipped byte (q + 128) under the
+// exponent byte of 1024.0 is 1024 + 128 + q exactly; one subtract, one multiply (a single rounding).
+__device__ __forceinline__ void dq_op_q8(int op, const Q8BlockRaw& blk, int j, half2v d2, DqTmp& tmp, U4& out) {
+    const half2v k1152 = {static_cast<_Float16>(1152.0f), static_cast<_Float16>(1152.0f)};
+    switch (op) {
+        case 0: tmp.qa = blk.q[2 * j] ^ 0x80808080u; break;
+        case 1: tmp.q8 = blk.q[2 * j + 1] ^ 0x80808080u; break;
+        case 2: tmp.t[0] = as_h2(__builtin_amdgcn_perm(0x64646464u, tmp.qa, 0x04010400u)); break;
+        case 3: tmp.t[1] = as_h2(__builtin_amdgcn_perm(0x64646464u, tmp.qa, 0x04030402u)); break;
+        case 4: tmp.t[2] = as_h2(__builtin_amdgcn_perm(0x64646464u, tmp.q8, 0x04010400u)); break;
+        case 5: tmp.t[3] = as_h2(__builtin_amdgcn_perm(0x64646464u, tmp.q8, 0x04030402u)); break;
+        case 6: case 7: case 8: case 9: tmp.t[op - 6] -= k1152; break;
+        default: out.v[op - 10] = as_u32(tmp.t[op - 10] * d2); break;
+    }
+}
+
+// Q3 -> half(q * d + b), q = low2 | high << 2, in the same pair order as Q4: pair p of
+// instruction j is weights 8j + p and 8j + p + 4.  One byte permute puts the two-bit fields of the
+// first four weights in bits 0..7 and of the last four in bits 16..23, where a mantissa of
+// 1024 / 4^p counts field p of each half in units of one; the high plane's byte of the same weights
+// is spread to bits p and 16 + p once per instruction and shifted to bit 2p + 2 of each half per
+// pair (units of four).
+__device__ __forceinline__ void dq_op_q3(int op, const Q3BlockRaw& blk, int j, half2v d2, half2v b2, DqTmp& tmp,
+                                         U4& out) {
+    if (op == 0) {
+        tmp.qa = __builtin_amdgcn_perm(0u, blk.lo[j >> 1], (j & 1) ? 0x0c030c02u : 0x0c010c00u);
+    } else if (op == 1) {
+        tmp.q8 = (blk.hi >> (8 * j)) & 0xffu;
+    } else if (op == 2) {
+        tmp.q8 = (tmp.q8 << 12) | tmp.q8;
+    } else if (op == 3) {
+        tmp.q8 &= 0x000F000Fu;  // bits p and 16 + p: high bits of weights 8j + p and 8j + p + 4
+    } else {
+        // stage by stage over the four pairs, so that no step waits on the one before it
+        const int step = (op - 4) / 4, p = (op - 4) % 4;
+        const uint32_t magic = p == 0 ? 0x64006400u : p == 1 ? 0x5C005C00u : p == 2 ? 0x54005400u : 0x4C004C00u;
+        const _Float16 mv = static_cast<_Float16>(p == 0 ? 1024.0f : p == 1 ? 256.0f : p == 2 ? 64.0f : 16.0f);
+        const half2v km = {mv, mv};
+        switch (step) {
+            case 0: tmp.t[p] = as_h2((tmp.qa & (0x00030003u << (2 * p))) | magic); break;
+            case 1: out.v[p] = tmp.q8 << (p + 2); break;  // out.v[p] is free until the pair's last step
+            case 2: tmp.t[p] = as_h2((out.v[p] & (0x00040004u << (2 * p))) | as_u32(tmp.t[p])); break;
+            case 3: tmp.t[p] -= km; break;
+            default: out.v[p] = as_u32(__builtin_elementwise_fma(tmp.t[p], d2, b2)); break;
+        }
+    }
+}
+
+template <int FMT, typename WBlock>
+__device__ __forceinline__ void dq_op(int op, const WBlock& blk, int j, half2v d2, half2v b2, DqTmp& tmp, U4& out) {
+    if constexpr (FMT == 0) dq_op_q4(op, blk.q[j], d2, b2, tmp, out);
+    else if constexpr (FMT == 1) dq_op_q8(op, blk, j, d2, tmp, out);
+    else dq_op_q3(op, blk, j, d2, b2, tmp, out);
 }
 
 // Eight consecutive f16 activations x0..x7 (as four dwords) -> x0 x4 x1 x5 x2 x6 x3 x7.
@@ -124,13 +220,18 @@ struct WregPlan {
     float* partial;        // [tail tile][slice][TM * TN] when tail_slices > 1
 };
 
-template <bool X_F16, bool LORA>
+// FMT: 0 = Q4 blocks, 1 = Q8_0, 2 = Q3 (the siblings have no LoRA step; Q8_0 keeps its activations in
+// memory order, the other two in the x0 x4 x1 x5 .. order of their decoders).
+template <bool X_F16, bool LORA, int FMT = 0>
 __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict__ w, uint32_t n, uint32_t k,
                                                        const void* __restrict__ xv, uint32_t m,
                                                        float* __restrict__ y, LoraEpilogue lora, WregPlan plan) {
     extern __shared__ uint4 lds16[];  // two activation buffers of kBuf16 units
     constexpr int XU = TM * (TK / 8) / 256;  // 8-activation units staged per thread per step
     constexpr int XL = X_F16 ? 1 : 2;        // 16-byte global loads per unit
+    typedef typename WBlockOf<FMT>::type WBlock;
+    constexpr uint32_t kBytes = WBlockOf<FMT>::kBytes;
+    constexpr int kDqOps = DqOps<FMT>::kOps;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -175,12 +276,16 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
         for (int t = 0; t < NT; ++t) acc[u][t] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
 
     // ---- per-thread global pointers -----------------------------------------------------------
-    const uint32_t* w_row[NU];  // first dword of the lane's weight row of tile u
+    // first block of the slice in the lane's weight row of tile u; counted in dwords where the format's
+    // blocks are whole dwords, in 2-byte units for Q8_0
+    typedef typename std::conditional<FMT == 1, uint16_t, uint32_t>::type WUnit;
+    constexpr uint32_t kUnits = kBytes / sizeof(WUnit);
+    const WUnit* w_row[NU];
 #pragma unroll
     for (int u = 0; u < NU; ++u) {
         uint32_t row = n0 + wave * 64 + u * 16 + lr;
         row = row < n ? row : n - 1;
-        w_row[u] = reinterpret_cast<const uint32_t*>(w) + static_cast<size_t>(row) * (nb_total * 5) + s_begin * 20;
+        w_row[u] = reinterpret_cast<const WUnit*>(w) + static_cast<size_t>(row) * (nb_total * kUnits) + s_begin * (4 * kUnits);
     }
     // activation unit i of this thread: token row tid/16 + 16 i, K offset 8 * (tid % 16) of the step
     const int x_part = tid & 15;
@@ -208,7 +313,13 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
     auto store_x_unit = [&](const XRegs& xr, int i, uint4* buf) {
         uint4 out;
         if (X_F16) {
-            out = interleave8(xr.c[i][0]);
+            out = FMT == 1 ? xr.c[i][0] : interleave8(xr.c[i][0]);
+        } else if (FMT == 1) {
+            const uint4 a = xr.c[i][0], b = xr.c[i][XL - 1];
+            out.x = pack_h2(__builtin_bit_cast(float, a.x), __builtin_bit_cast(float, a.y));
+            out.y = pack_h2(__builtin_bit_cast(float, a.z), __builtin_bit_cast(float, a.w));
+            out.z = pack_h2(__builtin_bit_cast(float, b.x), __builtin_bit_cast(float, b.y));
+            out.w = pack_h2(__builtin_bit_cast(float, b.z), __builtin_bit_cast(float, b.w));
         } else {
             const uint4 a = xr.c[i][0], b = xr.c[i][XL - 1];
             out.x = pack_h2(__builtin_bit_cast(float, a.x), __builtin_bit_cast(float, b.x));
@@ -218,15 +329,17 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
         }
         buf[((tid >> 4) + 16 * i) * kPitch16 + x_part] = out;
     };
-    auto load_w = [&](Q4BlockRaw (&wr)[NU], uint32_t s) {
+    auto load_w = [&](WBlock (&wr)[NU], uint32_t s) {
         uint32_t blk = s * 4 + g;
         blk = blk < nb ? blk : nb - 1;
 #pragma unroll
-        for (int u = 0; u < NU; ++u) wr[u] = *reinterpret_cast<const Q4BlockRaw*>(w_row[u] + blk * 5);
+        for (int u = 0; u < NU; ++u) wr[u] = *reinterpret_cast<const WBlock*>(w_row[u] + blk * kUnits);
     };
 
-    auto scale_pair = [&](const Q4BlockRaw& blk, bool live, half2v& d2, half2v& b2) {
-        const uint32_t sb = live ? blk.sb : 0u;
+    auto scale_pair = [&](const WBlock& blk, bool live, half2v& d2, half2v& b2) {
+        uint32_t sb;
+        if constexpr (FMT == 1) sb = live ? static_cast<uint32_t>(blk.d) : 0u;  // scale only
+        else sb = live ? blk.sb : 0u;
         d2 = as_h2(__builtin_amdgcn_perm(sb, sb, 0x01000100u));  // (d, d)
         b2 = as_h2(__builtin_amdgcn_perm(sb, sb, 0x03020302u));  // (b, b)
     };
@@ -243,7 +356,7 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
     // from `wnext`), and every fourth token tile one activation unit of step s+1 is written to the
     // other LDS buffer and refilled from global memory for step s+2.  LDS operand reads run two
     // token tiles ahead.  `wfree` was consumed in the previous step and is refilled for step s+2.
-    auto step = [&](uint32_t s, Q4BlockRaw (&wr)[NU], Q4BlockRaw (&wnext)[NU], Q4BlockRaw (&wfree)[NU]) {
+    auto step = [&](uint32_t s, WBlock (&wr)[NU], WBlock (&wnext)[NU], WBlock (&wfree)[NU]) {
         load_w(wfree, s + 2);
         const uint4* xbuf = lds16 + (s & 1) * kBuf16 + lr * kPitch16 + 4 * g;
         uint4* xnext = lds16 + ((s + 1) & 1) * kBuf16;
@@ -273,8 +386,8 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
 #pragma unroll
                     for (int e = c * (NU * kDqOps) / 32; e < (c + 1) * (NU * kDqOps) / 32; ++e) {
                         const int uu = e / kDqOps, op = e % kDqOps;
-                        if (j < 3) dq_op(op, wr[uu].q[j + 1], d2[uu], b2[uu], tmp, a_nxt[uu]);
-                        else dq_op(op, wnext[uu].q[0], d2n[uu], b2n[uu], tmp, a_nxt[uu]);
+                        if (j < 3) dq_op<FMT>(op, wr[uu], j + 1, d2[uu], b2[uu], tmp, a_nxt[uu]);
+                        else dq_op<FMT>(op, wnext[uu], 0, d2n[uu], b2n[uu], tmp, a_nxt[uu]);
                     }
                     if (j == 2 && t == NT - 1) scale_pair(wnext[u], live_next, d2n[u], b2n[u]);
                     if (u == NU - 1 && (p & 3) == 1) {
@@ -295,7 +408,7 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
         __syncthreads();
     };
 
-    Q4BlockRaw wa[NU], wb[NU], wc[NU];
+    WBlock wa[NU], wb[NU], wc[NU];
 #pragma unroll
     for (int i = 0; i < XU; ++i) load_x_unit(xr, i, 0);
     load_w(wa, 0);
@@ -311,7 +424,7 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
         for (int u = 0; u < NU; ++u) {
             scale_pair(wa[u], g < nb, d2[u], b2[u]);
 #pragma unroll
-            for (int op = 0; op < kDqOps; ++op) dq_op(op, wa[u].q[0], d2[u], b2[u], tmp, a_cur[u]);
+            for (int op = 0; op < kDqOps; ++op) dq_op<FMT>(op, wa[u], 0, d2[u], b2[u], tmp, a_cur[u]);
         }
     }
     __syncthreads();
@@ -514,35 +627,44 @@ size_t gemm_wreg_scratch_floats(uint32_t n, uint32_t k, uint32_t m) {
 
 namespace {
 
-template <bool X_F16, bool LORA>
+template <bool X_F16, bool LORA, int FMT>
 void launch_wreg_t(const uint8_t* w, uint32_t n, uint32_t k, const void* x, uint32_t m, float* y,
                    const LoraEpilogue& lora, const HostPlan& hp, float* partial, hipStream_t stream) {
     static bool attr_set = false;
     if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4_wreg<X_F16, LORA>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4_wreg<X_F16, LORA, FMT>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         attr_set = true;
     }
     const size_t lds = 2 * kBuf16 * sizeof(uint4);
     const WregPlan plan{hp.full, hp.slices, partial};
     const uint32_t wgs = hp.full + (hp.tiles - hp.full) * hp.slices;
-    hipLaunchKernelGGL((gemm_q4_wreg<X_F16, LORA>), dim3(wgs), dim3(256), lds, stream, w, n, k, x, m, y, lora, plan);
+    hipLaunchKernelGGL((gemm_q4_wreg<X_F16, LORA, FMT>), dim3(wgs), dim3(256), lds, stream, w, n, k, x, m, y, lora,
+                       plan);
 }
 
 }  // namespace
 
 void launch_gemm_wreg(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
-                      float* y, const LoraEpilogue& lora, float* partial, hipStream_t stream) {
+                      float* y, const LoraEpilogue& lora, float* partial, hipStream_t stream, int fmt) {
     HostPlan hp = plan_tiles(n, k, m);
     if (!partial) hp = HostPlan{hp.tiles, hp.tiles, 1};
-    // the matrix-core LoRA step serves the whole tiles; the tail tiles get their delta from the reduction
-    const bool lora_in_kernel = lora.rank && hp.full > 0;
-    if (lora_in_kernel) {
-        if (x_is_f16) launch_wreg_t<true, true>(w, n, k, x, m, y, lora, hp, partial, stream);
-        else launch_wreg_t<false, true>(w, n, k, x, m, y, lora, hp, partial, stream);
+    if (fmt == 1) {
+        if (x_is_f16) launch_wreg_t<true, false, 1>(w, n, k, x, m, y, lora, hp, partial, stream);
+        else launch_wreg_t<false, false, 1>(w, n, k, x, m, y, lora, hp, partial, stream);
+    } else if (fmt == 2) {
+        if (x_is_f16) launch_wreg_t<true, false, 2>(w, n, k, x, m, y, lora, hp, partial, stream);
+        else launch_wreg_t<false, false, 2>(w, n, k, x, m, y, lora, hp, partial, stream);
     } else {
-        if (x_is_f16) launch_wreg_t<true, false>(w, n, k, x, m, y, lora, hp, partial, stream);
-        else launch_wreg_t<false, false>(w, n, k, x, m, y, lora, hp, partial, stream);
+        // the matrix-core LoRA step serves the whole tiles; the tail tiles get their delta from the reduction
+        const bool lora_in_kernel = lora.rank && hp.full > 0;
+        if (lora_in_kernel) {
+            if (x_is_f16) launch_wreg_t<true, true, 0>(w, n, k, x, m, y, lora, hp, partial, stream);
+            else launch_wreg_t<false, true, 0>(w, n, k, x, m, y, lora, hp, partial, stream);
+        } else {
+            if (x_is_f16) launch_wreg_t<true, false, 0>(w, n, k, x, m, y, lora, hp, partial, stream);
+            else launch_wreg_t<false, false, 0>(w, n, k, x, m, y, lora, hp, partial, stream);
+        }
     }
     if (hp.slices > 1)
         hipLaunchKernelGGL(gemm_reduce_tail, dim3(hp.tiles - hp.full, TM * TN / 1024), dim3(256), 0, stream, partial,

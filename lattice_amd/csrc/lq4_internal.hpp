@@ -103,7 +103,7 @@ void set_gemm_kernel_choice(int which);
 // (gemm_wreg_scratch_floats floats; null = no slicing) and are summed by a second kernel.
 size_t gemm_wreg_scratch_floats(uint32_t n, uint32_t k, uint32_t m);
 void launch_gemm_wreg(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
-                      float* y, const LoraEpilogue& lora, float* partial, hipStream_t stream);
+                      float* y, const LoraEpilogue& lora, float* partial, hipStream_t stream, int fmt = 0);
 
 // Q8_0 sibling format (34-byte blocks: f16 scale + 32 x i8, w = q * d): batch-1 GEMV with x staged
 // in LDS (gemv_q8_lds_bytes(k) bytes), and the LDS-staged tile GEMM for everything else.
@@ -113,7 +113,7 @@ void launch_gemm_q8(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int
                     float* scratch, hipStream_t stream);
 // Floats of scratch the sibling tile GEMMs use to cut K on shapes with few tiles (0 = none; a null
 // scratch pointer keeps K whole).
-size_t gemm_sibling_scratch_floats(uint32_t n, uint32_t k, uint32_t m);
+size_t gemm_sibling_scratch_floats(int fmt, uint32_t n, uint32_t k, uint32_t m);  // fmt: 1 = Q8_0, 2 = Q3
 
 // Q3 sibling format (16-byte blocks: f16 scale, f16 bias, 2-bit and 1-bit planes): same pair of paths.
 size_t gemv_q3_lds_bytes(uint32_t k);

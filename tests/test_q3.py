@@ -148,15 +148,20 @@ GEMM_CASES = [(2, 64, 64, "f32"), (8, 2048, 2048, "f32"), (16, 37, 96, "f32"), (
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("kernel", [0, 1, 2])  # by shape / tile kernel / weights-in-registers kernel
 @pytest.mark.parametrize("m,n,k,xdt", GEMM_CASES)
-def test_q3_gemm_matches_oracle(be, m, n, k, xdt):
+def test_q3_gemm_matches_oracle(be, m, n, k, xdt, kernel):
     import torch
-    print(f"q3 gemm m={m} n={n} k={k} x={xdt}", flush=True)
+    print(f"q3 gemm m={m} n={n} k={k} x={xdt} kernel={kernel}", flush=True)
     wq = _q3_weight(n, k, seed=m + n + k, symmetric=(m % 2 == 0))
     x = synth.activations(m, k, seed=2, dtype=np.float16 if xdt == "f16" else np.float32)
     qw = be.upload_q3_blocks(wq)
     y = torch.full((m + 1, n), float("nan"), device="cuda")
-    be.dispatch_gemm_q3(dev(x), 0, qw, y, 0, m, n, k)
+    be.set_gemm_kernel(kernel)  # rows up to 64 take the few-token kernel whatever is chosen
+    try:
+        be.dispatch_gemm_q3(dev(x), 0, qw, y, 0, m, n, k)
+    finally:
+        be.set_gemm_kernel(0)
     got = host(y)
     assert np.all(np.isnan(got[m])) and np.all(np.isfinite(got[:m]))
     e = rel_err(got[:m], oracle.q3_gemm_f32(x.astype(np.float32), wq, n, k))

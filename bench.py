@@ -410,6 +410,26 @@ def main():
             del qw
         out["prefill_gemm_f16"] = gemm
 
+        # the same for the sibling formats (one shape each way), and their few-token kernel at 16 rows
+        sib = {}
+        for fmt, make, call in (("q8_0", device_q8_weight, be.dispatch_gemm_q8),
+                                ("q3", device_q3_weight, be.dispatch_gemm_q3)):
+            res = {}
+            for (n, k) in ((17408, 5120), (5120, 17408)):
+                qw = be.wrap_device_blocks(make(torch, n, k, gen))
+                for m in (16, 2048):
+                    x = torch.randn((m, k), device="cuda", generator=gen).to(torch.float16)
+                    y = torch.empty((m, n), device="cuda")
+                    f = lambda i: call(x, 0, qw, y, 0, m, n, k)
+                    for i in range(3):
+                        f(i)
+                    ms = tm(torch, f, 10)
+                    res["M%d_N%d_K%d" % (m, n, k)] = {"ms": round(ms, 4),
+                                                      "TFLOP/s": round(2.0 * m * n * k / (ms * 1e-3) / 1e12, 1)}
+                del qw
+            sib[fmt] = res
+        out["sibling_gemm_f16"] = sib
+
         # MoE grouped expert GEMV, benchmark config 4
         mo = synth.MOE_35B
         E, I, H, T, TK = mo["experts"], mo["inter"], mo["hidden"], mo["tokens"], mo["top_k"]
@@ -427,9 +447,17 @@ def main():
         for i in range(len(sets)):
             f(i)
         ms = tm(torch, f, 40)
+        # the same step with the router in front of it (softmax, top-k, renormalise from the logits)
+        def routed(i):
+            ids_i, wts_i = be.moe_route(lg, TK)
+            be.moe_experts(sets[i % len(sets)][0], sets[i % len(sets)][1], E, I, H, xm, ids_i, wts_i, ym)
+        for i in range(3):
+            routed(i)
+        ms_routed = tm(torch, routed, 40)
         out["moe_grouped_gemv"] = {"distinct_experts": distinct, "algorithmic_bytes": moe_bytes,
                                    "ms_per_step": round(ms, 4), "GB/s": round(moe_bytes / ms / 1e6, 1),
-                                   "pct_of_hbm_peak": round(100 * moe_bytes / ms / 1e6 / HBM_PEAK_GBPS, 2)}
+                                   "pct_of_hbm_peak": round(100 * moe_bytes / ms / 1e6 / HBM_PEAK_GBPS, 2),
+                                   "ms_per_step_with_router": round(ms_routed, 4)}
         del sets
 
         # plain copies of known size: what a profiler's HBM traffic counters are scaled by

@@ -410,6 +410,7 @@ int lq4_moe_route(lq4_ctx* ctx, const float* logits_dev, uint32_t tokens, uint32
     if (!logits_dev || !ids_dev || !weights_dev) return fail(LQ4_E_INVALID, "null device pointer");
     if (top_k == 0 || top_k > 16 || top_k > num_experts)
         return fail(LQ4_E_INVALID, "top_k must be in 1..min(16, num_experts), got %u", top_k);
+    if (num_experts > 1024) return fail(LQ4_E_INVALID, "num_experts %u above 1024", num_experts);
     DeviceGuard g(ctx->device);
     launch_moe_route(logits_dev, tokens, num_experts, top_k, ids_dev, weights_dev, static_cast<hipStream_t>(stream));
     ctx->counters.moe_route++;

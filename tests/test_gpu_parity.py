@@ -340,6 +340,22 @@ def test_moe_route_matches_oracle(be):
     assert np.array_equal(host(ids), o_ids) and np.array_equal(host(wts), o_wts)
 
 
+@pytest.mark.parametrize("tokens,experts,top_k", [(33, 256, 8), (5, 100, 16), (3, 1000, 7), (70, 9, 9), (1, 1024, 1)])
+def test_moe_route_expert_counts_and_ties(be, tokens, experts, top_k):
+    # expert counts off the 64-lane grid, as many ranks as experts, and rows with many equal logits
+    # (coarsely rounded), an infinite and a NaN entry
+    print(f"moe route tokens={tokens} experts={experts} top_k={top_k}", flush=True)
+    lg = synth.router_logits(tokens, experts, seed=tokens + experts)
+    lg[::2] = np.round(lg[::2] * 2.0) / 2.0
+    if tokens > 2:
+        lg[1, experts // 2] = np.inf
+        lg[2, experts - 1] = np.nan
+    ids, wts = be.moe_route(dev(lg), top_k)
+    o_ids, o_wts, _ = oracle.moe_route(lg, top_k)
+    assert np.array_equal(host(ids), o_ids)
+    assert np.allclose(host(wts), o_wts, rtol=1e-5, atol=1e-7, equal_nan=True)
+
+
 @pytest.mark.parametrize("cfg", [dict(e=4, inter=64, hidden=96, tokens=3, top_k=2),
                                  dict(e=8, inter=32, hidden=64, tokens=9, top_k=8),
                                  dict(e=3, inter=96, hidden=160, tokens=7, top_k=3),

@@ -29,7 +29,7 @@ namespace {
 
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 
-constexpr int kWaves = 4;
+constexpr int kWaves = 4;  // waves per workgroup unless a launch asks for more
 constexpr int kXPitch = 36;  // dwords of LDS per block of x: 16 hi pairs, 16 lo pairs, sum, 3 pad
                              // (36 keeps 16-byte lane reads at stride 144 B conflict-free)
 constexpr float kLoScale = 2048.0f;
@@ -130,8 +130,10 @@ struct FusionArg<true> {
     typedef GemvFusion type;
 };
 
-template <int RW, int SG, int SEG, bool FUSED>
-__global__ __launch_bounds__(kWaves * 64) void gemv_q4_b1(const uint8_t* __restrict__ w, uint32_t n,
+// WAVES: waves per workgroup.  Every workgroup stages the whole activation vector, so on long rows
+// (K of 4096..8192) eight waves share one staging where four would each pay half of it again.
+template <int RW, int SG, int SEG, bool FUSED, int WAVES = kWaves>
+__global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restrict__ w, uint32_t n,
                                                           uint32_t k, const float* __restrict__ x,
                                                           float* __restrict__ y, LoraEpilogue lora,
                                                           typename FusionArg<FUSED>::type fz) {
@@ -146,9 +148,9 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_b1(const uint8_t* __restr
     const uint32_t slabs = SEG == 64 ? (nb + 63) / 64 : 1;
     const uint32_t slab_groups = (slabs + SG - 1) / SG;
     const uint32_t n_wrows = (n + RPW - 1) / RPW;
-    const uint32_t n_waves = gridDim.x * kWaves;
+    const uint32_t n_waves = gridDim.x * WAVES;
     // the wave index is uniform across the wave: keep it (and everything derived) scalar
-    const uint32_t wid = __builtin_amdgcn_readfirstlane(blockIdx.x * kWaves + (tid >> 6));
+    const uint32_t wid = __builtin_amdgcn_readfirstlane(blockIdx.x * WAVES + (tid >> 6));
     // chunks whose first wave-row exists for this wave (later waves may have one chunk fewer)
     const uint32_t first = wid < n_wrows ? n_wrows - wid : 0;  // wave-rows from this wave's first one on
     const uint32_t chunks = (first + n_waves * RW - 1) / (n_waves * RW);
@@ -215,12 +217,12 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_b1(const uint8_t* __restr
     };
     if constexpr (!FUSED) {
         stage(g0, x0a, x0b, static_cast<uint32_t>(tid) < nb * 4);
-        for (uint32_t g = tid + kWaves * 64; g < nb * 4; g += kWaves * 64) {
+        for (uint32_t g = tid + WAVES * 64; g < nb * 4; g += WAVES * 64) {
             const float4* xp = reinterpret_cast<const float4*>(x + (g >> 2) * kBlockWeights + (g & 3) * 8);
             stage(g, xp[0], xp[1], true);
         }
     } else {
-        __shared__ float red[kWaves];
+        __shared__ float red[WAVES];
         const uint32_t n_units = nb * 4;
         auto unit_at = [](uint32_t g) { return (g >> 2) * kBlockWeights + (g & 3) * 8; };
         auto add4 = [](float4 a, const float4 b) {
@@ -253,7 +255,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_b1(const uint8_t* __restr
             float ss = 0.0f;
 #pragma unroll
             for (int i = 0; i < KEEP; ++i) {
-                const uint32_t g = tid + i * kWaves * 64;
+                const uint32_t g = tid + i * WAVES * 64;
                 const uint32_t gc = g < n_units ? g : 0;
                 load_v(gc, va[i], vb[i]);
                 const float4* gp = reinterpret_cast<const float4*>(fz.gamma + unit_at(gc));
@@ -262,7 +264,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_b1(const uint8_t* __restr
             }
 #pragma unroll
             for (int i = 0; i < KEEP; ++i) {
-                const uint32_t g = tid + i * kWaves * 64;
+                const uint32_t g = tid + i * WAVES * 64;
                 if (g < n_units) {
                     ss += sq4(va[i]) + sq4(vb[i]);
                     if (blockIdx.x == 0 && fz.residual_out) {
@@ -272,7 +274,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_b1(const uint8_t* __restr
                     }
                 }
             }
-            for (uint32_t g = tid + KEEP * kWaves * 64; g < n_units; g += kWaves * 64) {
+            for (uint32_t g = tid + KEEP * WAVES * 64; g < n_units; g += WAVES * 64) {
                 float4 a, b;
                 load_v(g, a, b);
                 ss += sq4(a) + sq4(b);
@@ -289,10 +291,10 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_b1(const uint8_t* __restr
             const float inv_rms = 1.0f / sqrtf(total / static_cast<float>(k) + fz.eps);
 #pragma unroll
             for (int i = 0; i < KEEP; ++i) {
-                const uint32_t g = tid + i * kWaves * 64;
+                const uint32_t g = tid + i * WAVES * 64;
                 if (g < n_units) stage(g, norm4(va[i], inv_rms, ga[i]), norm4(vb[i], inv_rms, gb[i]), true);
             }
-            for (uint32_t g = tid + KEEP * kWaves * 64; g < n_units; g += kWaves * 64) {
+            for (uint32_t g = tid + KEEP * WAVES * 64; g < n_units; g += WAVES * 64) {
                 float4 a, b;
                 load_v(g, a, b);
                 const float4* gp = reinterpret_cast<const float4*>(fz.gamma + unit_at(g));
@@ -306,7 +308,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_b1(const uint8_t* __restr
                 const float e = __builtin_amdgcn_exp2f(gate * -1.44269504088896340736f);
                 return gate * __builtin_amdgcn_rcpf(1.0f + e) * u;
             };
-            for (uint32_t g = tid; g < n_units; g += kWaves * 64) {
+            for (uint32_t g = tid; g < n_units; g += WAVES * 64) {
                 const float4* gp = reinterpret_cast<const float4*>(x + unit_at(g));
                 const float4* up = reinterpret_cast<const float4*>(x + k + unit_at(g));
                 const float4 ga = gp[0], gb = gp[1], ua = up[0], ub = up[1];
@@ -316,7 +318,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_b1(const uint8_t* __restr
                 stage(g, a, b, true);
             }
         } else {
-            for (uint32_t g = tid; g < n_units; g += kWaves * 64) {
+            for (uint32_t g = tid; g < n_units; g += WAVES * 64) {
                 const float4* xp = reinterpret_cast<const float4*>(x + unit_at(g));
                 stage(g, xp[0], xp[1], true);
             }
@@ -401,26 +403,28 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_b1(const uint8_t* __restr
     }
 }
 
-template <int RW, int SG, int SEG>
+template <int RW, int SG, int SEG, int WAVES = kWaves>
 void launch_cfg(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, const LoraEpilogue& lora,
                 const GemvFusion* fusion, size_t lds, uint32_t waves, hipStream_t stream) {
     static bool attr_set[2] = {false, false};  // raise the dynamic-LDS cap once per instantiation
-    const dim3 grid((waves + kWaves - 1) / kWaves), block(kWaves * 64);
+    const dim3 grid((waves + WAVES - 1) / WAVES), block(WAVES * 64);
     if (fusion) {
         if (!attr_set[1]) {
-            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, true>),
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, true, WAVES>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, 159 * 1024);
             attr_set[1] = true;
         }
-        hipLaunchKernelGGL((gemv_q4_b1<RW, SG, SEG, true>), grid, block, lds, stream, w, n, k, x, y, lora, *fusion);
+        hipLaunchKernelGGL((gemv_q4_b1<RW, SG, SEG, true, WAVES>), grid, block, lds, stream, w, n, k, x, y, lora,
+                           *fusion);
         return;
     }
     if (!attr_set[0]) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, false>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, false, WAVES>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         attr_set[0] = true;
     }
-    hipLaunchKernelGGL((gemv_q4_b1<RW, SG, SEG, false>), grid, block, lds, stream, w, n, k, x, y, lora, NoFusion{});
+    hipLaunchKernelGGL((gemv_q4_b1<RW, SG, SEG, false, WAVES>), grid, block, lds, stream, w, n, k, x, y, lora,
+                       NoFusion{});
 }
 
 void launch_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, const LoraEpilogue& lora,
@@ -452,8 +456,11 @@ void launch_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* 
     // Up to 16 waves per CU (4096 in all), fewer when the staged x leaves room for fewer
     // workgroups; rows per wave chosen so every wave gets the same share (to within one).
     uint32_t wg_per_cu = static_cast<uint32_t>((160 * 1024) / (lds + 512));
-    wg_per_cu = wg_per_cu > 4 ? 4 : wg_per_cu < 1 ? 1 : wg_per_cu;
-    const uint32_t max_waves = 256 * wg_per_cu * kWaves;
+    // eight waves per workgroup on long rows (measured: 2048 x 6144 5.15 -> 4.69 us, 17408 x 5120
+    // 16.2 -> 15.2; behind on K 2048 and K 17408)
+    const uint32_t wg_waves = (seg == 64 && k >= 4096 && k <= 8192) ? 8 : kWaves;
+    wg_per_cu = wg_per_cu > 16 / wg_waves ? 16 / wg_waves : wg_per_cu < 1 ? 1 : wg_per_cu;
+    const uint32_t max_waves = 256 * wg_per_cu * wg_waves;
     uint32_t rw = (n_wrows + max_waves - 1) / max_waves;
     uint32_t waves;
     if (rw <= 4) {
@@ -477,10 +484,16 @@ void launch_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* 
     while (rw * sg > 6) --sg;
 
 #define LQ4_B1(RW_, SG_, SEG_) launch_cfg<RW_, SG_, SEG_>(w, n, k, x, y, lora, fusion, lds, waves, stream)
+#define LQ4_B1W(RW_, SG_) launch_cfg<RW_, SG_, 64, 8>(w, n, k, x, y, lora, fusion, lds, waves, stream)
     if (seg == 32) {
         if (rw == 1) LQ4_B1(1, 1, 32); else if (rw == 2) LQ4_B1(2, 1, 32); else if (rw == 3) LQ4_B1(3, 1, 32); else LQ4_B1(4, 1, 32);
     } else if (seg == 16) {
         if (rw == 1) LQ4_B1(1, 1, 16); else if (rw == 2) LQ4_B1(2, 1, 16); else if (rw == 3) LQ4_B1(3, 1, 16); else LQ4_B1(4, 1, 16);
+    } else if (wg_waves == 8) {  // K 4096..8192: two to four slabs
+        if (rw == 1) { if (sg == 2) LQ4_B1W(1, 2); else LQ4_B1W(1, 3); }
+        else if (rw == 2) { if (sg == 2) LQ4_B1W(2, 2); else LQ4_B1W(2, 3); }
+        else if (rw == 3) LQ4_B1W(3, 2);
+        else LQ4_B1W(4, 1);
     } else if (rw == 1) {
         if (sg == 1) LQ4_B1(1, 1, 64); else if (sg == 2) LQ4_B1(1, 2, 64); else LQ4_B1(1, 3, 64);
     } else if (rw == 2) {
@@ -490,6 +503,7 @@ void launch_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* 
     } else {
         LQ4_B1(4, 1, 64);
     }
+#undef LQ4_B1W
 #undef LQ4_B1
 }
 

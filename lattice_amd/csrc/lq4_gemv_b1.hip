@@ -23,6 +23,8 @@
 // limit the reference's half-staged tiled kernel has.
 #include "lq4_internal.hpp"
 
+#include <type_traits>
+
 namespace lq4 {
 
 namespace {
@@ -331,9 +333,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
     for (int j = 0; j < RW; ++j) acc[j] = 0.0f;
 
     // Consumes unit u from `cur` while unit u+1 streams into `nxt`.
-    auto process = [&](Q4BlockRaw (&cur)[RW][SG], Q4BlockRaw (&nxt)[RW][SG], uint32_t u) {
+    // `prefetch` is a compile-time flag: a load behind a run-time condition would make the compiler
+    // wait, before the current unit's blocks are used, for as many loads as the path WITHOUT the
+    // prefetch needs, i.e. for most of the just-issued next unit as well.
+    auto process = [&](auto prefetch, Q4BlockRaw (&cur)[RW][SG], Q4BlockRaw (&nxt)[RW][SG], uint32_t u) {
         const uint32_t chunk = u / slab_groups, sgi = u - chunk * slab_groups;
-        if (u + 1 < units) load_unit(nxt, u + 1);
+        if constexpr (decltype(prefetch)::value) load_unit(nxt, u + 1);
 
 #pragma unroll
         for (int t = 0; t < SG; ++t) {
@@ -397,9 +402,19 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
     };
 
     // two buffers swap roles every unit, so no block is ever copied between registers
-    for (uint32_t u = 0; u < units; u += 2) {
-        process(buf_a, buf_b, u);
-        if (u + 1 < units) process(buf_b, buf_a, u + 1);
+    // (units that have a successor prefetch it unconditionally; the last one or two are peeled off)
+    constexpr std::true_type kFetch{};
+    constexpr std::false_type kLast{};
+    uint32_t u = 0;
+    for (; u + 2 < units; u += 2) {
+        process(kFetch, buf_a, buf_b, u);
+        process(kFetch, buf_b, buf_a, u + 1);
+    }
+    if (u + 2 == units) {
+        process(kFetch, buf_a, buf_b, u);
+        process(kLast, buf_b, buf_a, u + 1);
+    } else if (u < units) {
+        process(kLast, buf_a, buf_b, u);
     }
 }
 

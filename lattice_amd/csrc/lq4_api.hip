@@ -695,9 +695,9 @@ int lq4_gemm_q8(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
     if (m == 1 && x_dtype == LQ4_F32 && gemv_q8_lds_bytes(k) <= 128 * 1024) {
         launch_gemv_q8_b1(wp, n, k, static_cast<const float*>(x_dev), y_dev, s);
         ctx->counters.gemv++;
-    } else if (m <= 64 || gemm_skinny_wants(n, k, m)) {
+    } else if (m <= 32 || gemm_skinny_wants(n, k, m)) {
         // few rows: operands packed once, the few-token matrix-core kernel with this format's decoder
-        // (always for one token tile: the sibling tile kernel is no match for it there)
+        // (always up to 32 rows: the large-tile kernels are no match for it there)
         const int src = ensure_scratch(ctx, gemm_skinny_scratch_bytes(k, m));
         if (src) return src;
         const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};
@@ -736,9 +736,9 @@ int lq4_gemm_q3(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
     if (m == 1 && x_dtype == LQ4_F32 && gemv_q3_lds_bytes(k) <= 128 * 1024) {
         launch_gemv_q3_b1(wp, n, k, static_cast<const float*>(x_dev), y_dev, s);
         ctx->counters.gemv++;
-    } else if (m <= 64 || gemm_skinny_wants(n, k, m)) {
+    } else if (m <= 32 || gemm_skinny_wants(n, k, m)) {
         // few rows: operands packed once, the few-token matrix-core kernel with this format's decoder
-        // (always for one token tile: the sibling tile kernel is no match for it there)
+        // (always up to 32 rows: the large-tile kernels are no match for it there)
         const int src = ensure_scratch(ctx, gemm_skinny_scratch_bytes(k, m));
         if (src) return src;
         const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};

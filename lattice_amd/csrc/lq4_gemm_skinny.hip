@@ -176,7 +176,11 @@ __global__ __launch_bounds__(256) void pack_x_kernel(const void* __restrict__ xv
 
 // RT: 16-row weight tiles per wave (rows per workgroup = 16 RT).  grid (ceil(N / 16 RT), token tiles).
 // FMT: 0 = Q4, 1 = Q8_0, 2 = Q3 blocks.
-template <int RT, int FMT>
+// NTG: 16-token groups a workgroup computes (1, 2 or 4); a token tile with fewer groups re-reads its
+// last group and drops the results.  Fixed per instantiation, like the prefetches of the K loop below:
+// a load behind a run-time condition makes the compiler wait for loads it cannot count, and the
+// pipeline collapses to one unit in flight.
+template <int RT, int FMT, int NTG>
 __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __restrict__ w, uint32_t n, uint32_t k,
                                                                 const uint4* __restrict__ xp, uint32_t m,
                                                                 float* __restrict__ y, LoraEpilogue lora) {
@@ -207,8 +211,11 @@ __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __
 
     struct Unit {
         WBlock wb[RT];
-        uint4 x[4][4];  // [token group][instruction]
+        uint4 x[NTG][4];  // [token group][instruction]
     };
+    uint32_t xg[NTG];  // packed-image group of token group t (clamped to the last one)
+#pragma unroll
+    for (int t = 0; t < NTG; ++t) xg[t] = tg0 + t < groups ? tg0 + t : groups - 1;
     // i-th step of this wave
     auto load = [&](Unit& u, uint32_t i) {
         const uint32_t s = wave + i * kWavesK;
@@ -216,20 +223,18 @@ __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __
         blk = blk < nb ? blk : nb - 1;
 #pragma unroll
         for (int r = 0; r < RT; ++r) u.wb[r] = *reinterpret_cast<const WBlock*>(w_row[r] + blk * kBytes);
-        const uint4* xs = xp + (static_cast<size_t>(s) * groups + tg0) * 256 + lane;
+        const uint4* xs = xp + static_cast<size_t>(s) * groups * 256 + lane;
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
-            if (static_cast<uint32_t>(t) < ntg) {
+        for (int t = 0; t < NTG; ++t)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) u.x[t][j] = xs[(t * 4 + j) * 64];
-            }
+            for (int j = 0; j < 4; ++j) u.x[t][j] = xs[(xg[t] * 4 + j) * 64];
     };
 
-    float4v acc[RT][4];
+    float4v acc[RT][NTG];
 #pragma unroll
     for (int r = 0; r < RT; ++r)
 #pragma unroll
-        for (int t = 0; t < 4; ++t) acc[r][t] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int t = 0; t < NTG; ++t) acc[r][t] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
 
     auto compute = [&](const Unit& u, uint32_t i) {
         const bool live = (wave + i * kWavesK) * 4 + g < nb;  // K tail: a block past the end of the row counts as zero
@@ -247,33 +252,60 @@ __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __
                 else if constexpr (FMT == 1) a = dequant8_q8(u.wb[r].q[2 * j], u.wb[r].q[2 * j + 1], d2);
                 else a = dequant8_q3(u.wb[r], j, d2, b2);
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    if (static_cast<uint32_t>(t) < ntg)
-                        acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                            __builtin_bit_cast(half8, a), __builtin_bit_cast(half8, u.x[t][j]), acc[r][t], 0, 0, 0);
+                for (int t = 0; t < NTG; ++t)
+                    acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                        __builtin_bit_cast(half8, a), __builtin_bit_cast(half8, u.x[t][j]), acc[r][t], 0, 0, 0);
             }
         }
     };
 
-    if (cnt) {
+    // Two units in flight.  Every unit that has a successor two places on prefetches it without a
+    // condition; the last two or three units are written out.  (A redundant clamped prefetch instead
+    // would be waited for by whatever reuses its registers.)
+    // (the scheduling fences keep a unit's arithmetic from being hoisted across the loads around it,
+    // which would hold both units' temporaries live at once and spill)
+#define LQ4_FENCE() __builtin_amdgcn_sched_barrier(0)
+    if (cnt > 1) {
         Unit u0, u1;
         load(u0, 0);
-        if (cnt > 1) load(u1, 1);
+        load(u1, 1);
+        LQ4_FENCE();
         uint32_t i = 0;
-        for (; i + 2 <= cnt; i += 2) {
+        for (; i + 3 < cnt; i += 2) {
             compute(u0, i);
-            if (i + 2 < cnt) load(u0, i + 2);  // never a load nobody consumes: the reduction below waits for all of them
+            LQ4_FENCE();
+            load(u0, i + 2);
+            LQ4_FENCE();
             compute(u1, i + 1);
-            if (i + 3 < cnt) load(u1, i + 3);
+            LQ4_FENCE();
+            load(u1, i + 3);
+            LQ4_FENCE();
         }
-        if (i < cnt) compute(u0, i);
+        if (cnt - i == 3) {
+            compute(u0, i);
+            LQ4_FENCE();
+            load(u0, i + 2);
+            LQ4_FENCE();
+            compute(u1, i + 1);
+            LQ4_FENCE();
+            compute(u0, i + 2);
+        } else {
+            compute(u0, i);
+            LQ4_FENCE();
+            compute(u1, i + 1);
+        }
+    } else if (cnt == 1) {
+        Unit u0;
+        load(u0, 0);
+        compute(u0, 0);
     }
+#undef LQ4_FENCE
 
     // ---- LoRA: wave w adds the ranks w, w + 8, ... of scale * B[row, :] . t[token, :] to its own
     //      partial result in f32, so the delta is spread over all waves and joins the same reduction
     if (lora.rank) {
         for (uint32_t jj = wave; jj < lora.rank; jj += kWavesK) {
-            float bv[RT][4], tv[4];
+            float bv[RT][4], tv[NTG];
 #pragma unroll
             for (int r = 0; r < RT; ++r)
 #pragma unroll
@@ -283,7 +315,7 @@ __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __
                     bv[r][v] = lora.scale * load_b(lora.b, lora.b_is_f16, static_cast<size_t>(row) * lora.rank + jj);
                 }
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
+            for (int t = 0; t < NTG; ++t) {
                 uint32_t tok = 16 * (tg0 + t) + lr;
                 tok = tok < m ? tok : m - 1;
                 tv[t] = lora.t[static_cast<size_t>(tok) * lora.rank + jj];
@@ -291,7 +323,7 @@ __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __
 #pragma unroll
             for (int r = 0; r < RT; ++r)
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
+                for (int t = 0; t < NTG; ++t)
 #pragma unroll
                     for (int v = 0; v < 4; ++v) acc[r][t][v] = fmaf(bv[r][v], tv[t], acc[r][t][v]);
         }
@@ -299,21 +331,21 @@ __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __
 
     // ---- the eight K slices meet in LDS in three rounds: (w, w + 4), then (w, w + 2), then (0, 1);
     //      the order is fixed, so the result does not depend on timing
-    constexpr int kSlot = RT * 4 * 64;
+    constexpr int kSlot = RT * NTG * 64;
 #pragma unroll
     for (int half = kWavesK / 2; half >= 1; half >>= 1) {
         if (wave >= half && wave < 2 * half) {
 #pragma unroll
             for (int r = 0; r < RT; ++r)
 #pragma unroll
-                for (int t = 0; t < 4; ++t) red[(wave - half) * kSlot + (r * 4 + t) * 64 + lane] = acc[r][t];
+                for (int t = 0; t < NTG; ++t) red[(wave - half) * kSlot + (r * NTG + t) * 64 + lane] = acc[r][t];
         }
         __syncthreads();
         if (wave < half) {
 #pragma unroll
             for (int r = 0; r < RT; ++r)
 #pragma unroll
-                for (int t = 0; t < 4; ++t) acc[r][t] += red[wave * kSlot + (r * 4 + t) * 64 + lane];
+                for (int t = 0; t < NTG; ++t) acc[r][t] += red[wave * kSlot + (r * NTG + t) * 64 + lane];
         }
         if (half > 1) __syncthreads();  // the slots are reused by the next round
     }
@@ -326,7 +358,7 @@ __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __
         const uint32_t gn = n0 + 16 * r + 4 * g;
         if (gn >= n) continue;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
+        for (int t = 0; t < NTG; ++t) {
             const uint32_t tok = 16 * (tg0 + t) + lr;
             if (static_cast<uint32_t>(t) >= ntg || tok >= m) continue;
             const float4v val = acc[r][t];
@@ -342,12 +374,28 @@ __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __
     }
 }
 
+template <int RT, int FMT, int NTG>
+void launch_ntg(const uint8_t* w, uint32_t n, uint32_t k, const uint4* xp, uint32_t m, float* y,
+                const LoraEpilogue& lora, hipStream_t stream) {
+    const dim3 grid((n + 16 * RT - 1) / (16 * RT), (m + kTokens - 1) / kTokens);
+    const size_t lds = static_cast<size_t>(kWavesK / 2) * RT * NTG * 64 * sizeof(float4v);
+    hipLaunchKernelGGL((gemm_q4_skinny<RT, FMT, NTG>), grid, dim3(64 * kWavesK), lds, stream, w, n, k, xp, m, y, lora);
+}
+
+// Widest row tile whose two units in flight fit the 256 registers of a wave without spilling.
+constexpr int max_rt(int fmt, int ntg) {
+    if (fmt == 0) return ntg == 4 ? 2 : 4;
+    if (fmt == 1) return ntg == 4 ? 1 : 2;
+    return ntg == 1 ? 2 : 1;
+}
+
 template <int RT, int FMT>
 void launch_rt(const uint8_t* w, uint32_t n, uint32_t k, const uint4* xp, uint32_t m, float* y, const LoraEpilogue& lora,
                hipStream_t stream) {
-    const dim3 grid((n + 16 * RT - 1) / (16 * RT), (m + kTokens - 1) / kTokens);
-    const size_t lds = static_cast<size_t>(kWavesK / 2) * RT * 4 * 64 * sizeof(float4v);
-    hipLaunchKernelGGL((gemm_q4_skinny<RT, FMT>), grid, dim3(64 * kWavesK), lds, stream, w, n, k, xp, m, y, lora);
+    const uint32_t groups = (m + 15) / 16;
+    if (groups == 1) launch_ntg<(RT < max_rt(FMT, 1) ? RT : max_rt(FMT, 1)), FMT, 1>(w, n, k, xp, m, y, lora, stream);
+    else if (groups == 2) launch_ntg<(RT < max_rt(FMT, 2) ? RT : max_rt(FMT, 2)), FMT, 2>(w, n, k, xp, m, y, lora, stream);
+    else launch_ntg<(RT < max_rt(FMT, 4) ? RT : max_rt(FMT, 4)), FMT, 4>(w, n, k, xp, m, y, lora, stream);
 }
 
 }  // namespace
@@ -386,8 +434,8 @@ void launch_fmt(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_i
     // Every workgroup reads the whole packed X of its token tile, so wider row tiles cut that
     // traffic; they are taken only while at least 128 workgroups remain.
     const uint32_t tiles16 = (n + 15) / 16;
-    // (the 34-byte Q8_0 blocks of four row tiles do not fit the register file)
-    if (FMT != 1 && tiles16 >= 4 * 128) launch_rt<4, FMT>(w, n, k, xp, m, y, lora, stream);
+    // (launch_rt narrows the tile again where the format and token count would spill registers)
+    if (tiles16 >= 4 * 128) launch_rt<4, FMT>(w, n, k, xp, m, y, lora, stream);
     else if (tiles16 >= 2 * 128) launch_rt<2, FMT>(w, n, k, xp, m, y, lora, stream);
     else launch_rt<1, FMT>(w, n, k, xp, m, y, lora, stream);
 }

@@ -14,6 +14,8 @@
 // current one is consumed.
 #include "lq4_internal.hpp"
 
+#include <type_traits>
+
 namespace lq4 {
 
 namespace {
@@ -109,9 +111,11 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q8_b1(const uint8_t* __restr
 #pragma unroll
     for (int j = 0; j < RW; ++j) acc[j] = 0.0f;
 
-    auto process = [&](Q8BlockRaw (&cur)[RW], Q8BlockRaw (&nxt)[RW], uint32_t u) {
+    // `prefetch` is a compile-time flag: behind a run-time condition the compiler would have to wait
+    // for most of the just-issued next unit before it may use the current one.
+    auto process = [&](auto prefetch, Q8BlockRaw (&cur)[RW], Q8BlockRaw (&nxt)[RW], uint32_t u) {
         const uint32_t chunk = u / slabs, slab = u - chunk * slabs;
-        if (u + 1 < units) load_unit(nxt, u + 1);
+        if constexpr (decltype(prefetch)::value) load_unit(nxt, u + 1);
         const uint32_t blk_raw = slab * 64 + lane;
         const bool live = blk_raw < nb;
         const uint32_t blk = live ? blk_raw : nb - 1;
@@ -140,9 +144,18 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q8_b1(const uint8_t* __restr
         }
     };
 
-    for (uint32_t u = 0; u < units; u += 2) {
-        process(buf_a, buf_b, u);
-        if (u + 1 < units) process(buf_b, buf_a, u + 1);
+    constexpr std::true_type kFetch{};
+    constexpr std::false_type kLast{};
+    uint32_t u = 0;
+    for (; u + 2 < units; u += 2) {
+        process(kFetch, buf_a, buf_b, u);
+        process(kFetch, buf_b, buf_a, u + 1);
+    }
+    if (u + 2 == units) {
+        process(kFetch, buf_a, buf_b, u);
+        process(kLast, buf_b, buf_a, u + 1);
+    } else if (u < units) {
+        process(kLast, buf_a, buf_b, u);
     }
 }
 

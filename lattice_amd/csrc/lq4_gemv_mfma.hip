@@ -97,7 +97,7 @@ struct GemvArgs {
 // Workgroups are persistent: workgroup g handles row groups g, g + gridDim.x, ... (a row group
 // is 4*T*(4/KS) rows) with the activations staged once.  For one wave the work is a list of
 // units (row group, step); unit u+1 is in flight while unit u is consumed.
-template <int NSETS, bool HILO, int T, int KS>
+template <int NSETS, bool HILO, int T, int KS, bool LONG>
 __global__ __launch_bounds__(kThreads) void gemv_q4_mfma(GemvArgs p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     constexpr int RS = 4 / KS;  // row sub-groups per workgroup
@@ -214,7 +214,11 @@ __global__ __launch_bounds__(kThreads) void gemv_q4_mfma(GemvArgs p) {
 
     // Consumes unit u from `cur` while unit u+1 streams into `nxt`.
     auto process = [&](Q4BlockRaw (&cur)[T], Q4BlockRaw (&nxt)[T], uint32_t u) {
-        if (u + 3 < units) load_unit(nxt, u + 3);
+        // LONG streams prefetch without a condition (past the end: the last unit again), so the wait
+        // for the current unit counts exactly and three units stay in flight; short streams, whose
+        // units are all in flight from the start, skip the redundant loads instead
+        if (LONG) load_unit(nxt, u + 3 < units ? u + 3 : units - 1);
+        else if (u + 3 < units) load_unit(nxt, u + 3);
         const uint32_t it = u / n_local, q = u - it * n_local;
         const uint32_t blk_raw = (ks + q * KS) * 16 + g;
         const bool live = blk_raw < nb;
@@ -366,20 +370,28 @@ __global__ __launch_bounds__(kThreads) void gemv_q4_mfma(GemvArgs p) {
     }
 }
 
-template <int NSETS, bool HILO, int T, int KS>
-void launch_cfg(const GemvArgs& a, size_t lds, uint32_t max_wgs, hipStream_t stream) {
+template <int NSETS, bool HILO, int T, int KS, bool LONG>
+void launch_long(const GemvArgs& a, size_t lds, uint32_t wgs, hipStream_t stream) {
     static bool attr_set = false;  // raise the dynamic-LDS cap once per instantiation
     if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_mfma<NSETS, HILO, T, KS>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_mfma<NSETS, HILO, T, KS, LONG>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         attr_set = true;
     }
+    hipLaunchKernelGGL((gemv_q4_mfma<NSETS, HILO, T, KS, LONG>), dim3(wgs), dim3(kThreads), lds, stream, a);
+}
+
+template <int NSETS, bool HILO, int T, int KS>
+void launch_cfg(const GemvArgs& a, size_t lds, uint32_t max_wgs, hipStream_t stream) {
     constexpr uint32_t rows_per_iter = 4 * T * (4 / KS);
     const uint32_t groups = (a.n + rows_per_iter - 1) / rows_per_iter;
     // every workgroup gets the same number of row groups, to within one
     const uint32_t iters = (groups + max_wgs - 1) / max_wgs;
     const uint32_t wgs = (groups + iters - 1) / iters;
-    hipLaunchKernelGGL((gemv_q4_mfma<NSETS, HILO, T, KS>), dim3(wgs), dim3(kThreads), lds, stream, a);
+    const uint32_t nsteps = (a.k / kBlockWeights + 15) / 16;
+    const uint32_t units = iters * ((nsteps + KS - 1) / KS);  // per wave
+    if (units >= 8) launch_long<NSETS, HILO, T, KS, true>(a, lds, wgs, stream);
+    else launch_long<NSETS, HILO, T, KS, false>(a, lds, wgs, stream);
 }
 
 template <int NSETS, bool HILO>

@@ -117,6 +117,23 @@ def test_gemv_small_batch_matches_oracle(be, batch, n, k):
     assert e <= REL_TOL
 
 
+@pytest.mark.parametrize("batch", [1, 2, 5, 8])
+def test_gemv_long_streams_match_oracle(be, batch):
+    # enough rows that every wave walks many units: the kernels' steady-state loops (unconditional
+    # prefetch) and their peeled last units, with a K tail inside a 64-block slab and rows off the grid
+    import torch
+    n, k = 40003, 2080
+    print(f"gemv long streams batch={batch} n={n} k={k}", flush=True)
+    wq = synth.q4_weight(n, k, seed=6, symmetric_bias=False)
+    x = synth.activations(batch, k, seed=6)
+    qw = be.upload_q4_blocks(wq)
+    y = torch.full((batch, n), float("nan"), dtype=torch.float32, device="cuda")
+    be.gemv_batch(dev(x), qw, y, batch, n, k)
+    e = rel_err(host(y), oracle.gemm_f32(x, wq, n, k))
+    print(f"  rel err {e:.2e}", flush=True)
+    assert e <= REL_TOL
+
+
 def test_gemv_extreme_scales_and_activations(be):
     # forward/metal_qwen35.rs:23529-23692: mixed block scales, +-500 activations
     import torch

@@ -114,7 +114,8 @@ def _q3_weight(n, k, seed, symmetric=False):
 
 
 GEMV_CASES = [(4096, 1024, False), (2048, 2048, True), (12288, 2048, False), (2048, 6144, False), (37, 96, False),
-              (5, 32, True), (1000, 4160, False), (20000, 256, False)]
+              (5, 32, True), (1000, 4160, False), (20000, 256, False),
+              (30011, 2080, True)]  # many units per wave: steady-state loop and peeled tail
 
 
 @pytest.mark.gpu

@@ -108,7 +108,8 @@ def _q8_weight(n, k, seed):
     return oracle.q8_quantize_rows(w)
 
 
-GEMV_CASES = [(4096, 1024), (2048, 2048), (12288, 2048), (2048, 6144), (37, 96), (5, 32), (1000, 4160), (20000, 256)]
+GEMV_CASES = [(4096, 1024), (2048, 2048), (12288, 2048), (2048, 6144), (37, 96), (5, 32), (1000, 4160), (20000, 256),
+              (30011, 2080)]  # many units per wave: steady-state loop and peeled tail
 
 
 @pytest.mark.gpu

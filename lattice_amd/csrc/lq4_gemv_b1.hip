@@ -158,14 +158,25 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
     const uint32_t chunks = (first + n_waves * RW - 1) / (n_waves * RW);
     const uint32_t units = chunks * slab_groups;
 
-    // ---- first chunk of x is requested before any weight so it can be waited on alone ----
-    // (straight-line code, clamped addresses: no branch between the loads and their wait)
-    const uint32_t g0 = static_cast<uint32_t>(tid) < nb * 4 ? tid : 0;
-    float4 x0a = {0.0f, 0.0f, 0.0f, 0.0f}, x0b = x0a;
-    if constexpr (!FUSED) {
-        const float4* x0p = reinterpret_cast<const float4*>(x + (g0 >> 2) * kBlockWeights + (g0 & 3) * 8);
-        x0a = x0p[0];
-        x0b = x0p[1];
+    // ---- the first activations are requested before any weight so they can be waited on alone ----
+    // (straight-line code, clamped addresses: no branch between the loads and their wait).  Loads
+    // return in order: an activation load issued after the weight prefetch would hold its staging,
+    // and the barrier behind it, back until the first weights have crossed from HBM.  Rows longer
+    // than one slab hoist four 8-activation units per thread (K up to 8192 with four waves).
+    constexpr int HX = SG >= 2 ? 4 : 1;
+    uint32_t gx[HX];
+    float4 xa[HX], xb[HX];
+#pragma unroll
+    for (int i = 0; i < HX; ++i) {
+        const uint32_t g = tid + i * WAVES * 64;
+        gx[i] = g < nb * 4 ? g : 0;
+        xa[i] = float4{0.0f, 0.0f, 0.0f, 0.0f};
+        xb[i] = xa[i];
+        if constexpr (!FUSED) {
+            const float4* xp = reinterpret_cast<const float4*>(x + (gx[i] >> 2) * kBlockWeights + (gx[i] & 3) * 8);
+            xa[i] = xp[0];
+            xb[i] = xp[1];
+        }
     }
 
     // Loads unit u's blocks.  Lanes past the end of a row and rows past N re-read a valid
@@ -218,8 +229,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
         }
     };
     if constexpr (!FUSED) {
-        stage(g0, x0a, x0b, static_cast<uint32_t>(tid) < nb * 4);
-        for (uint32_t g = tid + WAVES * 64; g < nb * 4; g += WAVES * 64) {
+#pragma unroll
+        for (int i = 0; i < HX; ++i) stage(gx[i], xa[i], xb[i], tid + i * WAVES * 64 < nb * 4);
+        for (uint32_t g = tid + HX * WAVES * 64; g < nb * 4; g += WAVES * 64) {
             const float4* xp = reinterpret_cast<const float4*>(x + (g >> 2) * kBlockWeights + (g & 3) * 8);
             stage(g, xp[0], xp[1], true);
         }

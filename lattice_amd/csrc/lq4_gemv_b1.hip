@@ -162,8 +162,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
     // (straight-line code, clamped addresses: no branch between the loads and their wait).  Loads
     // return in order: an activation load issued after the weight prefetch would hold its staging,
     // and the barrier behind it, back until the first weights have crossed from HBM.  Rows longer
-    // than one slab hoist four 8-activation units per thread (K up to 8192 with four waves).
-    constexpr int HX = SG >= 2 ? 4 : 1;
+    // than one slab hoist more 8-activation units per thread: two with eight waves (all of K up to
+    // 8192), eight with four waves (rows beyond that; measured, 5120 x 17408 18.0 -> 16.4 us).
+    constexpr int HX = SG < 2 ? 1 : WAVES == 8 ? 2 : 8;
     uint32_t gx[HX];
     float4 xa[HX], xb[HX];
 #pragma unroll

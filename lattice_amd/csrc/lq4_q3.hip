@@ -95,7 +95,8 @@ __device__ __forceinline__ float block_dot(const Q3BlockRaw& b, const uint32_t (
 
 // Chunk c of wave `wid` holds rows (c * RW + j) * n_waves + wid, j < RW; a unit is one
 // (chunk, slab of 64 blocks).  Dynamic LDS: (K/32) * kXPitch dwords.
-template <int RW>
+// HX: 8-activation units per thread requested ahead of the weights (all of K up to 2048 * HX).
+template <int RW, int HX>
 __global__ __launch_bounds__(kWaves * 64) void gemv_q3_b1(const uint8_t* __restrict__ w, uint32_t n, uint32_t k,
                                                           const float* __restrict__ x, float* __restrict__ y) {
     extern __shared__ __attribute__((aligned(16))) uint32_t xs[];
@@ -122,18 +123,17 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q3_b1(const uint8_t* __restr
         }
     };
 
-    Q3BlockRaw buf_a[RW], buf_b[RW];
-    if (units) load_unit(buf_a, 0);
-
     // ---- stage x: four threads per block ------------------------------------------------------
     // thread j = 0, 1: low-plane pairs of weights 16 j .. 16 j + 15; j = 2, 3: high-plane pairs
     // e = 8 (j - 2) .. + 7, i.e. (x[e], x[e + 16]).
-    for (uint32_t g = tid; g < nb * 4; g += kWaves * 64) {
+    auto x_src = [&](uint32_t g, const float4*& pa, const float4*& pb) {
         const uint32_t blk = g >> 2, j = g & 3;
         const float* xb = x + blk * kBlockWeights;
-        const float4* pa = reinterpret_cast<const float4*>(xb + (j < 2 ? 16 * j : 8 * (j - 2)));
-        const float4* pb = reinterpret_cast<const float4*>(xb + (j < 2 ? 16 * j + 8 : 8 * (j - 2) + 16));
-        const float4 a0 = pa[0], a1 = pa[1], b0 = pb[0], b1 = pb[1];
+        pa = reinterpret_cast<const float4*>(xb + (j < 2 ? 16 * j : 8 * (j - 2)));
+        pb = reinterpret_cast<const float4*>(xb + (j < 2 ? 16 * j + 8 : 8 * (j - 2) + 16));
+    };
+    auto stage = [&](uint32_t g, const float4 a0, const float4 a1, const float4 b0, const float4 b1, bool store) {
+        const uint32_t blk = g >> 2, j = g & 3;
         const float va[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
         const float vb[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
         uint32_t out[8];
@@ -157,10 +157,38 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q3_b1(const uint8_t* __restr
         }
         sx = dpp_add<0xB1>(sx);  // the 4 threads of a block are 4 adjacent lanes: quad butterfly
         sx = dpp_add<0x4E>(sx);
-        uint4* dst = reinterpret_cast<uint4*>(&xs[blk * kXPitch + 8 * j]);
-        dst[0] = make_uint4(out[0], out[1], out[2], out[3]);
-        dst[1] = make_uint4(out[4], out[5], out[6], out[7]);
-        if (j == 0) *reinterpret_cast<float*>(&xs[blk * kXPitch + 32]) = sx;
+        if (store) {
+            uint4* dst = reinterpret_cast<uint4*>(&xs[blk * kXPitch + 8 * j]);
+            dst[0] = make_uint4(out[0], out[1], out[2], out[3]);
+            dst[1] = make_uint4(out[4], out[5], out[6], out[7]);
+            if (j == 0) *reinterpret_cast<float*>(&xs[blk * kXPitch + 32]) = sx;
+        }
+    };
+
+    // The first activations of every thread are requested before any weight (clamped addresses, no
+    // branch): loads return in order, so behind the weight prefetch their staging, and the barrier
+    // after it, would wait until the first weights have crossed from HBM.
+    uint32_t gx[HX];
+    float4 xa0[HX], xa1[HX], xb0[HX], xb1[HX];
+#pragma unroll
+    for (int i = 0; i < HX; ++i) {
+        const uint32_t g = tid + i * kWaves * 64;
+        gx[i] = g < nb * 4 ? g : 0;
+        const float4 *pa, *pb;
+        x_src(gx[i], pa, pb);
+        xa0[i] = pa[0]; xa1[i] = pa[1]; xb0[i] = pb[0]; xb1[i] = pb[1];
+    }
+
+    Q3BlockRaw buf_a[RW], buf_b[RW];
+    load_unit(buf_a, 0);  // (a wave without rows re-reads the last row; it stores nothing)
+    __builtin_amdgcn_sched_barrier(0);  // nothing below is scheduled above these loads
+
+#pragma unroll
+    for (int i = 0; i < HX; ++i) stage(gx[i], xa0[i], xa1[i], xb0[i], xb1[i], tid + i * kWaves * 64 < nb * 4);
+    for (uint32_t g = tid + HX * kWaves * 64; g < nb * 4; g += kWaves * 64) {
+        const float4 *pa, *pb;
+        x_src(g, pa, pb);
+        stage(g, pa[0], pa[1], pb[0], pb[1], true);
     }
     __syncthreads();
 
@@ -218,17 +246,25 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q3_b1(const uint8_t* __restr
     }
 }
 
-template <int RW>
-void launch_rw(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, size_t lds, uint32_t waves,
+template <int RW, int HX>
+void launch_hx(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, size_t lds, uint32_t waves,
                hipStream_t stream) {
     static bool attr_set = false;
     if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q3_b1<RW>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q3_b1<RW, HX>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         attr_set = true;
     }
-    hipLaunchKernelGGL((gemv_q3_b1<RW>), dim3((waves + kWaves - 1) / kWaves), dim3(kWaves * 64), lds, stream, w, n, k,
+    hipLaunchKernelGGL((gemv_q3_b1<RW, HX>), dim3((waves + kWaves - 1) / kWaves), dim3(kWaves * 64), lds, stream, w, n, k,
                        x, y);
+}
+
+template <int RW>
+void launch_rw(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, size_t lds, uint32_t waves,
+               hipStream_t stream) {
+    if (k <= 2048) launch_hx<RW, 1>(w, n, k, x, y, lds, waves, stream);
+    else if (k <= 4096) launch_hx<RW, 2>(w, n, k, x, y, lds, waves, stream);
+    else launch_hx<RW, 3>(w, n, k, x, y, lds, waves, stream);
 }
 
 }  // namespace

@@ -62,7 +62,8 @@ __device__ __forceinline__ float block_dot(const uint32_t (&q)[8], const float (
 
 // Chunk c of wave `wid` holds rows (c * RW + j) * n_waves + wid, j < RW; a unit is one
 // (chunk, slab of 64 blocks).  Dynamic LDS: (K/32) * kXPitch dwords.
-template <int RW>
+// HX: 8-activation units per thread requested ahead of the weights (all of K up to 2048 * HX).
+template <int RW, int HX>
 __global__ __launch_bounds__(kWaves * 64) void gemv_q8_b1(const uint8_t* __restrict__ w, uint32_t n, uint32_t k,
                                                           const float* __restrict__ x, float* __restrict__ y) {
     extern __shared__ __attribute__((aligned(16))) float xs[];
@@ -89,21 +90,43 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q8_b1(const uint8_t* __restr
         }
     };
 
-    Q8BlockRaw buf_a[RW], buf_b[RW];
-    if (units) load_unit(buf_a, 0);
-
     // ---- stage x: thread g handles 8 activations of block g / 4 -----------------------------
-    for (uint32_t g = tid; g < nb * 4; g += kWaves * 64) {
+    auto stage = [&](uint32_t g, const float4 a, const float4 b, bool store) {
         const uint32_t blk = g >> 2, j = g & 3;
-        const float4* xp = reinterpret_cast<const float4*>(x + blk * kBlockWeights + j * 8);
-        const float4 a = xp[0], b = xp[1];
         float sx = ((a.x + a.y) + (a.z + a.w)) + ((b.x + b.y) + (b.z + b.w));
         sx = dpp_add<0xB1>(sx);  // the 4 threads of a block are 4 adjacent lanes: quad butterfly
         sx = dpp_add<0x4E>(sx);
-        float4* dst = reinterpret_cast<float4*>(&xs[blk * kXPitch + 8 * j]);
-        dst[0] = a;
-        dst[1] = b;
-        if (j == 0) xs[blk * kXPitch + 32] = sx;
+        if (store) {
+            float4* dst = reinterpret_cast<float4*>(&xs[blk * kXPitch + 8 * j]);
+            dst[0] = a;
+            dst[1] = b;
+            if (j == 0) xs[blk * kXPitch + 32] = sx;
+        }
+    };
+
+    // The first activations of every thread are requested before any weight (clamped addresses, no
+    // branch): loads return in order, so behind the weight prefetch their staging, and the barrier
+    // after it, would wait until the first weights have crossed from HBM.
+    uint32_t gx[HX];
+    float4 xa[HX], xb[HX];
+#pragma unroll
+    for (int i = 0; i < HX; ++i) {
+        const uint32_t g = tid + i * kWaves * 64;
+        gx[i] = g < nb * 4 ? g : 0;
+        const float4* xp = reinterpret_cast<const float4*>(x + (gx[i] >> 2) * kBlockWeights + (gx[i] & 3) * 8);
+        xa[i] = xp[0];
+        xb[i] = xp[1];
+    }
+
+    Q8BlockRaw buf_a[RW], buf_b[RW];
+    load_unit(buf_a, 0);  // (a wave without rows re-reads the last row; it stores nothing)
+    __builtin_amdgcn_sched_barrier(0);  // nothing below is scheduled above these loads
+
+#pragma unroll
+    for (int i = 0; i < HX; ++i) stage(gx[i], xa[i], xb[i], tid + i * kWaves * 64 < nb * 4);
+    for (uint32_t g = tid + HX * kWaves * 64; g < nb * 4; g += kWaves * 64) {
+        const float4* xp = reinterpret_cast<const float4*>(x + (g >> 2) * kBlockWeights + (g & 3) * 8);
+        stage(g, xp[0], xp[1], true);
     }
     __syncthreads();
 
@@ -159,17 +182,25 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q8_b1(const uint8_t* __restr
     }
 }
 
-template <int RW>
-void launch_rw(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, size_t lds, uint32_t waves,
+template <int RW, int HX>
+void launch_hx(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, size_t lds, uint32_t waves,
                hipStream_t stream) {
     static bool attr_set = false;
     if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q8_b1<RW>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q8_b1<RW, HX>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         attr_set = true;
     }
-    hipLaunchKernelGGL((gemv_q8_b1<RW>), dim3((waves + kWaves - 1) / kWaves), dim3(kWaves * 64), lds, stream, w, n, k,
+    hipLaunchKernelGGL((gemv_q8_b1<RW, HX>), dim3((waves + kWaves - 1) / kWaves), dim3(kWaves * 64), lds, stream, w, n, k,
                        x, y);
+}
+
+template <int RW>
+void launch_rw(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, size_t lds, uint32_t waves,
+               hipStream_t stream) {
+    if (k <= 2048) launch_hx<RW, 1>(w, n, k, x, y, lds, waves, stream);
+    else if (k <= 4096) launch_hx<RW, 2>(w, n, k, x, y, lds, waves, stream);
+    else launch_hx<RW, 3>(w, n, k, x, y, lds, waves, stream);
 }
 
 }  // namespace

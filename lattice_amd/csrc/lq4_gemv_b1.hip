@@ -302,7 +302,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
             ss = wave_sum(ss);
             if (lane == 0) red[tid >> 6] = ss;
             __syncthreads();
-            const float total = (red[0] + red[1]) + (red[2] + red[3]);
+            float total = (red[0] + red[1]) + (red[2] + red[3]);
+            if constexpr (WAVES == 8) total += (red[4] + red[5]) + (red[6] + red[7]);
+            static_assert(WAVES == 4 || WAVES == 8, "the sum of squares is combined for four or eight waves");
             const float inv_rms = 1.0f / sqrtf(total / static_cast<float>(k) + fz.eps);
 #pragma unroll
             for (int i = 0; i < KEEP; ++i) {

@@ -149,7 +149,8 @@ def _mlp_inputs(hidden, inter, seed):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("hidden,inter", [(2048, 6144), (1024, 512), (512, 96), (160, 352)])
+@pytest.mark.parametrize("hidden,inter", [(2048, 6144), (1024, 512), (512, 96), (160, 352),
+                                          (5120, 544)])  # norm prologue in an eight-wave workgroup
 def test_fused_decode_mlp_matches_oracle_and_unfused(be, hidden, inter):
     """norm + gate||up GEMV, then silu*up + down GEMV + residual add: two fused launches against
     the oracle's five steps and against the same five steps run one by one on the GPU."""

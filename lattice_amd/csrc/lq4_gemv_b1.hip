@@ -165,18 +165,46 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
     // than one slab hoist more 8-activation units per thread: two with eight waves (all of K up to
     // 8192), eight with four waves (rows beyond that; measured, 5120 x 17408 18.0 -> 16.4 us).
     constexpr int HX = SG < 2 ? 1 : WAVES == 8 ? 2 : 8;
-    uint32_t gx[HX];
-    float4 xa[HX], xb[HX];
+    // fused prologues hold up to four vectors per unit, so they hoist at most three units
+    constexpr int HF = FUSED ? (HX < 3 ? HX : 3) : HX;
+    uint32_t gx[HF];
+    float4 xa[HF], xb[HF];  // plain: x;  add + norm: base (+ delta);  silu * up: gate
+    float4 ya[FUSED ? HF : 1], yb[FUSED ? HF : 1];  // add + norm: gamma;  silu * up: up
 #pragma unroll
-    for (int i = 0; i < HX; ++i) {
+    for (int i = 0; i < HF; ++i) {
         const uint32_t g = tid + i * WAVES * 64;
         gx[i] = g < nb * 4 ? g : 0;
-        xa[i] = float4{0.0f, 0.0f, 0.0f, 0.0f};
-        xb[i] = xa[i];
+        const uint32_t at = (gx[i] >> 2) * kBlockWeights + (gx[i] & 3) * 8;
         if constexpr (!FUSED) {
-            const float4* xp = reinterpret_cast<const float4*>(x + (gx[i] >> 2) * kBlockWeights + (gx[i] & 3) * 8);
+            const float4* xp = reinterpret_cast<const float4*>(x + at);
             xa[i] = xp[0];
             xb[i] = xp[1];
+        } else if (fz.prologue == GemvFusion::kAddNorm) {
+            const float4* bp = reinterpret_cast<const float4*>(fz.base + at);
+            xa[i] = bp[0];
+            xb[i] = bp[1];
+            if (fz.delta) {
+                const float4* dp = reinterpret_cast<const float4*>(fz.delta + at);
+                const float4 da = dp[0], db = dp[1];
+                xa[i].x += da.x; xa[i].y += da.y; xa[i].z += da.z; xa[i].w += da.w;
+                xb[i].x += db.x; xb[i].y += db.y; xb[i].z += db.z; xb[i].w += db.w;
+            }
+            const float4* gp = reinterpret_cast<const float4*>(fz.gamma + at);
+            ya[i] = gp[0];
+            yb[i] = gp[1];
+        } else if (fz.prologue == GemvFusion::kSiluMul) {
+            const float4* gp = reinterpret_cast<const float4*>(x + at);
+            const float4* up = reinterpret_cast<const float4*>(x + k + at);
+            xa[i] = gp[0];
+            xb[i] = gp[1];
+            ya[i] = up[0];
+            yb[i] = up[1];
+        } else {
+            const float4* xp = reinterpret_cast<const float4*>(x + at);
+            xa[i] = xp[0];
+            xb[i] = xp[1];
+            ya[i] = xa[i];
+            yb[i] = xb[i];
         }
     }
 
@@ -231,8 +259,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
     };
     if constexpr (!FUSED) {
 #pragma unroll
-        for (int i = 0; i < HX; ++i) stage(gx[i], xa[i], xb[i], tid + i * WAVES * 64 < nb * 4);
-        for (uint32_t g = tid + HX * WAVES * 64; g < nb * 4; g += WAVES * 64) {
+        for (int i = 0; i < HF; ++i) stage(gx[i], xa[i], xb[i], tid + i * WAVES * 64 < nb * 4);
+        for (uint32_t g = tid + HF * WAVES * 64; g < nb * 4; g += WAVES * 64) {
             const float4* xp = reinterpret_cast<const float4*>(x + (g >> 2) * kBlockWeights + (g & 3) * 8);
             stage(g, xp[0], xp[1], true);
         }
@@ -262,34 +290,22 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
             }
         };
         if (fz.prologue == GemvFusion::kAddNorm) {
-            // The first KEEP units of a thread (K <= 6144 has no more) stay in registers between
-            // the sum of squares and the scaling, with their gamma already requested; longer
-            // vectors re-read the rest.
-            constexpr int KEEP = 3;
-            float4 va[KEEP], vb[KEEP], ga[KEEP], gb[KEEP];
+            // The hoisted units of a thread stay in registers between the sum of squares and the
+            // scaling, with their gamma; longer vectors re-read the rest.
             float ss = 0.0f;
 #pragma unroll
-            for (int i = 0; i < KEEP; ++i) {
-                const uint32_t g = tid + i * WAVES * 64;
-                const uint32_t gc = g < n_units ? g : 0;
-                load_v(gc, va[i], vb[i]);
-                const float4* gp = reinterpret_cast<const float4*>(fz.gamma + unit_at(gc));
-                ga[i] = gp[0];
-                gb[i] = gp[1];
-            }
-#pragma unroll
-            for (int i = 0; i < KEEP; ++i) {
+            for (int i = 0; i < HF; ++i) {
                 const uint32_t g = tid + i * WAVES * 64;
                 if (g < n_units) {
-                    ss += sq4(va[i]) + sq4(vb[i]);
+                    ss += sq4(xa[i]) + sq4(xb[i]);
                     if (blockIdx.x == 0 && fz.residual_out) {
                         float4* rp = reinterpret_cast<float4*>(fz.residual_out + unit_at(g));
-                        rp[0] = va[i];
-                        rp[1] = vb[i];
+                        rp[0] = xa[i];
+                        rp[1] = xb[i];
                     }
                 }
             }
-            for (uint32_t g = tid + KEEP * WAVES * 64; g < n_units; g += WAVES * 64) {
+            for (uint32_t g = tid + HF * WAVES * 64; g < n_units; g += WAVES * 64) {
                 float4 a, b;
                 load_v(g, a, b);
                 ss += sq4(a) + sq4(b);
@@ -307,11 +323,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
             static_assert(WAVES == 4 || WAVES == 8, "the sum of squares is combined for four or eight waves");
             const float inv_rms = 1.0f / sqrtf(total / static_cast<float>(k) + fz.eps);
 #pragma unroll
-            for (int i = 0; i < KEEP; ++i) {
-                const uint32_t g = tid + i * WAVES * 64;
-                if (g < n_units) stage(g, norm4(va[i], inv_rms, ga[i]), norm4(vb[i], inv_rms, gb[i]), true);
-            }
-            for (uint32_t g = tid + KEEP * WAVES * 64; g < n_units; g += WAVES * 64) {
+            for (int i = 0; i < HF; ++i)
+                stage(gx[i], norm4(xa[i], inv_rms, ya[i]), norm4(xb[i], inv_rms, yb[i]), tid + i * WAVES * 64 < n_units);
+            for (uint32_t g = tid + HF * WAVES * 64; g < n_units; g += WAVES * 64) {
                 float4 a, b;
                 load_v(g, a, b);
                 const float4* gp = reinterpret_cast<const float4*>(fz.gamma + unit_at(g));
@@ -325,17 +339,27 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
                 const float e = __builtin_amdgcn_exp2f(gate * -1.44269504088896340736f);
                 return gate * __builtin_amdgcn_rcpf(1.0f + e) * u;
             };
-            for (uint32_t g = tid; g < n_units; g += WAVES * 64) {
-                const float4* gp = reinterpret_cast<const float4*>(x + unit_at(g));
-                const float4* up = reinterpret_cast<const float4*>(x + k + unit_at(g));
-                const float4 ga = gp[0], gb = gp[1], ua = up[0], ub = up[1];
-                float4 a, b;
+            auto silu_mul8 = [&](const float4 ga, const float4 gb, const float4 ua, const float4 ub, float4& a, float4& b) {
                 a.x = silu_mul(ga.x, ua.x); a.y = silu_mul(ga.y, ua.y); a.z = silu_mul(ga.z, ua.z); a.w = silu_mul(ga.w, ua.w);
                 b.x = silu_mul(gb.x, ub.x); b.y = silu_mul(gb.y, ub.y); b.z = silu_mul(gb.z, ub.z); b.w = silu_mul(gb.w, ub.w);
+            };
+#pragma unroll
+            for (int i = 0; i < HF; ++i) {
+                float4 a, b;
+                silu_mul8(xa[i], xb[i], ya[i], yb[i], a, b);
+                stage(gx[i], a, b, tid + i * WAVES * 64 < n_units);
+            }
+            for (uint32_t g = tid + HF * WAVES * 64; g < n_units; g += WAVES * 64) {
+                const float4* gp = reinterpret_cast<const float4*>(x + unit_at(g));
+                const float4* up = reinterpret_cast<const float4*>(x + k + unit_at(g));
+                float4 a, b;
+                silu_mul8(gp[0], gp[1], up[0], up[1], a, b);
                 stage(g, a, b, true);
             }
         } else {
-            for (uint32_t g = tid; g < n_units; g += WAVES * 64) {
+#pragma unroll
+            for (int i = 0; i < HF; ++i) stage(gx[i], xa[i], xb[i], tid + i * WAVES * 64 < n_units);
+            for (uint32_t g = tid + HF * WAVES * 64; g < n_units; g += WAVES * 64) {
                 const float4* xp = reinterpret_cast<const float4*>(x + unit_at(g));
                 stage(g, xp[0], xp[1], true);
             }

@@ -228,6 +228,25 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
         }
     };
 
+    // LoRA factors of the first chunk's rows (lane i of a row holds t[i] and B[row, i]), requested ahead
+    // of the weights like the activations: fetched only when the chunk completes, they would add a
+    // memory round trip to the tail of the kernel
+    float lora_t0 = 0.0f, lora_b0[RW];
+#pragma unroll
+    for (int j = 0; j < RW; ++j) lora_b0[j] = 0.0f;
+    if (lora.rank && static_cast<uint32_t>(seg_lane) < lora.rank) {
+        lora_t0 = lora.t[seg_lane];
+#pragma unroll
+        for (int j = 0; j < RW; ++j) {
+            const uint32_t wrow = j * n_waves + wid;
+            uint32_t row = wrow * RPW + sub;
+            row = (wrow < n_wrows && row < n) ? row : n - 1;
+            const size_t bi = static_cast<size_t>(row) * lora.rank + seg_lane;
+            lora_b0[j] = lora.b_is_f16 ? static_cast<float>(static_cast<const _Float16*>(lora.b)[bi])
+                                       : static_cast<const float*>(lora.b)[bi];
+        }
+    }
+
     Q4BlockRaw buf_a[RW][SG], buf_b[RW][SG];
     load_unit(buf_a, 0);
     // residual values of the first chunk's rows, requested now so the final store does not wait
@@ -416,7 +435,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
                 acc[j] = 0.0f;
                 if (lora.rank && row_ok) {
                     // the row's lanes share out scale * B[row, i] * t[i]; the sum below folds it in
-                    for (uint32_t i = seg_lane; i < lora.rank; i += SEG) {
+                    uint32_t i = seg_lane;
+                    if (chunk == 0 && i < lora.rank) {  // requested at kernel start
+                        v = fmaf(lora.scale * lora_b0[j], lora_t0, v);
+                        i += SEG;
+                    }
+                    for (; i < lora.rank; i += SEG) {
                         const size_t bi = static_cast<size_t>(row) * lora.rank + i;
                         const float bv = lora.b_is_f16 ? static_cast<float>(static_cast<const _Float16*>(lora.b)[bi])
                                                        : static_cast<const float*>(lora.b)[bi];

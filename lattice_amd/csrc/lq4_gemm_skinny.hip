@@ -382,9 +382,9 @@ void launch_ntg(const uint8_t* w, uint32_t n, uint32_t k, const uint4* xp, uint3
     hipLaunchKernelGGL((gemm_q4_skinny<RT, FMT, NTG>), grid, dim3(64 * kWavesK), lds, stream, w, n, k, xp, m, y, lora);
 }
 
-// Widest row tile whose two units in flight fit the 256 registers of a wave without spilling.
+// Widest row tile (of 1 or 2) whose two units in flight fit the 256 registers of a wave without spilling.
 constexpr int max_rt(int fmt, int ntg) {
-    if (fmt == 0) return ntg == 4 ? 2 : 4;
+    if (fmt == 0) return 2;
     if (fmt == 1) return ntg == 4 ? 1 : 2;
     return ntg == 1 ? 2 : 1;
 }
@@ -431,12 +431,13 @@ void launch_fmt(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_i
         hipLaunchKernelGGL((pack_x_kernel<true, kInterleave>), dim3(steps, groups), dim3(256), 0, stream, x, m, k, xp);
     else
         hipLaunchKernelGGL((pack_x_kernel<false, kInterleave>), dim3(steps, groups), dim3(256), 0, stream, x, m, k, xp);
-    // Every workgroup reads the whole packed X of its token tile, so wider row tiles cut that
-    // traffic; they are taken only while at least 128 workgroups remain.
+    // Every workgroup reads the whole packed X of its token tile, so a wider row tile halves that
+    // traffic, at the price of fewer workgroups to balance over the compute units.  Measured over
+    // 2048..34816 rows and K 2048..17408 at 16, 32 and 64 tokens: two row tiles pay on tall matrices,
+    // on long rows and with four token groups; four never do since the K loop keeps two units in flight.
     const uint32_t tiles16 = (n + 15) / 16;
-    // (launch_rt narrows the tile again where the format and token count would spill registers)
-    if (tiles16 >= 4 * 128) launch_rt<4, FMT>(w, n, k, xp, m, y, lora, stream);
-    else if (tiles16 >= 2 * 128) launch_rt<2, FMT>(w, n, k, xp, m, y, lora, stream);
+    const bool wide = tiles16 >= 1024 || (k >= 8192 && tiles16 >= 256) || (m > 32 && tiles16 >= 512);
+    if (wide) launch_rt<2, FMT>(w, n, k, xp, m, y, lora, stream);
     else launch_rt<1, FMT>(w, n, k, xp, m, y, lora, stream);
 }
 

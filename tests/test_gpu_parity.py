@@ -516,7 +516,7 @@ SKINNY_CASES = [(17, 16, 32, "f32"), (64, 2048, 2048, "f32"), (64, 512, 2048, "f
 @pytest.mark.parametrize("m,n,k,xdt", SKINNY_CASES)
 def test_gemm_few_token_kernel_matches_oracle(be, m, n, k, xdt):
     # the few-token kernel: ragged token groups, N tails (also N % 4 != 0), K tails inside a
-    # 128-wide step, fewer K steps than waves, all three row-tile widths; forced, so M > 128 is
+    # 128-wide step, fewer K steps than waves, both row-tile widths; forced, so M > 128 is
     # covered too
     import torch
     print(f"gemm few-token m={m} n={n} k={k} x={xdt}", flush=True)

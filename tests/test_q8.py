@@ -151,7 +151,7 @@ def test_q8_gemm_matches_oracle(be, m, n, k, xdt, kernel):
     x = synth.activations(m, k, seed=2, dtype=np.float16 if xdt == "f16" else np.float32)
     qw = be.upload_q8_blocks(wq)
     y = torch.full((m + 1, n), float("nan"), device="cuda")
-    be.set_gemm_kernel(kernel)  # rows up to 64 take the few-token kernel whatever is chosen
+    be.set_gemm_kernel(kernel)  # few rows take the few-token kernel whatever is chosen
     try:
         be.dispatch_gemm_q8(dev(x), 0, qw, y, 0, m, n, k)
     finally:

@@ -137,13 +137,6 @@ __global__ __launch_bounds__(kThreads) void moe_expert_mfma(MoeGemvArgs p) {
         buf[1] = *reinterpret_cast<const Q4BlockRaw*>(wbase + static_cast<size_t>(rb) * (nb * 5) + blk * 5);
     };
 
-    // ring of kRing unit buffers: kRing - 1 units are in flight while one is consumed
-    Q4BlockRaw buf[kRing][2];
-#pragma unroll
-    for (int i = 0; i < kRing - 1; ++i)
-        if (static_cast<uint32_t>(i) < units) load_unit(buf[i], i);
-    __builtin_amdgcn_sched_barrier(0);
-
     // ---- stage the activations of this pass: 8 values per (block, dword) item per pair ---------
     // All (pair, item) combinations of the pass are flattened and taken four at a time, so the loads
     // of different pairs are in flight together.
@@ -154,48 +147,69 @@ __global__ __launch_bounds__(kThreads) void moe_expert_mfma(MoeGemvArgs p) {
         const int32_t pair = s_pair[b < nt ? b : 0];
         xrow[b] = p.x + static_cast<size_t>(static_cast<uint32_t>(pair) / p.x_div) * p.x_stride;
     }
-    {
-        constexpr int G = 4;
-        const uint32_t total = static_cast<uint32_t>(nt) * items;
-        for (uint32_t w0 = tid; w0 < total; w0 += G * kThreads) {
-            float4 va[G], vb[G];
-            uint32_t wb[G], wi[G];
+    constexpr int G = 4;
+    const uint32_t total = static_cast<uint32_t>(nt) * items;
+    struct Round {
+        float4 va[G], vb[G];
+        uint32_t wb[G], wi[G];
+    };
+    auto load_round = [&](Round& r, uint32_t w0) {
 #pragma unroll
-            for (int i = 0; i < G; ++i) {
-                const uint32_t w = w0 + i * kThreads;
-                const uint32_t wc = w < total ? w : 0;
-                wb[i] = wc / items;
-                wi[i] = wc - wb[i] * items;
-                const float* xr = wb[i] == 0 ? xrow[0] : wb[i] == 1 ? xrow[1] : wb[i] == 2 ? xrow[2] : xrow[3];
-                const float4* xp = reinterpret_cast<const float4*>(xr + (wi[i] >> 2) * kBlockWeights + (wi[i] & 3) * 8);
-                va[i] = xp[0];
-                vb[i] = xp[1];
+        for (int i = 0; i < G; ++i) {
+            const uint32_t w = w0 + i * kThreads;
+            const uint32_t wc = w < total ? w : 0;
+            r.wb[i] = wc / items;
+            r.wi[i] = wc - r.wb[i] * items;
+            const float* xr = r.wb[i] == 0 ? xrow[0] : r.wb[i] == 1 ? xrow[1] : r.wb[i] == 2 ? xrow[2] : xrow[3];
+            const float4* xp = reinterpret_cast<const float4*>(xr + (r.wi[i] >> 2) * kBlockWeights + (r.wi[i] & 3) * 8);
+            r.va[i] = xp[0];
+            r.vb[i] = xp[1];
+        }
+    };
+    auto store_round = [&](const Round& r, uint32_t w0) {
+#pragma unroll
+        for (int i = 0; i < G; ++i) {
+            const uint32_t blk = r.wi[i] >> 2, dw = r.wi[i] & 3, bb = r.wb[i];
+            const float v[8] = {r.va[i].x, r.va[i].y, r.va[i].z, r.va[i].w, r.vb[i].x, r.vb[i].y, r.vb[i].z, r.vb[i].w};
+            _Float16 h[8], l[8];
+#pragma unroll
+            for (int e2 = 0; e2 < 8; ++e2) {
+                const float sc = (e2 & 1) ? v[e2] * 0.0625f : v[e2];
+                h[e2] = static_cast<_Float16>(sc);
+                l[e2] = static_cast<_Float16>((sc - static_cast<float>(h[e2])) * kLoScale);
             }
-#pragma unroll
-            for (int i = 0; i < G; ++i) {
-                const uint32_t blk = wi[i] >> 2, dw = wi[i] & 3, bb = wb[i];
-                const float v[8] = {va[i].x, va[i].y, va[i].z, va[i].w, vb[i].x, vb[i].y, vb[i].z, vb[i].w};
-                _Float16 h[8], l[8];
-#pragma unroll
-                for (int e2 = 0; e2 < 8; ++e2) {
-                    const float sc = (e2 & 1) ? v[e2] * 0.0625f : v[e2];
-                    h[e2] = static_cast<_Float16>(sc);
-                    l[e2] = static_cast<_Float16>((sc - static_cast<float>(h[e2])) * kLoScale);
-                }
-                uint4 hi, lo;
-                hi.x = pack_h2(h[0], h[4]); hi.y = pack_h2(h[1], h[5]); hi.z = pack_h2(h[2], h[6]); hi.w = pack_h2(h[3], h[7]);
-                lo.x = pack_h2(l[0], l[4]); lo.y = pack_h2(l[1], l[5]); lo.z = pack_h2(l[2], l[6]); lo.w = pack_h2(l[3], l[7]);
-                float sx = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
-                sx = dpp_add<0xB1>(sx);  // the 4 items of a block sit in 4 adjacent lanes
-                sx = dpp_add<0x4E>(sx);
-                if (w0 + i * kThreads < total) {
-                    uint4* base = xs16 + blk * kPitch16;
-                    base[(2 * bb) * 4 + dw] = hi;
-                    base[(2 * bb + 1) * 4 + dw] = lo;
-                    if (dw == 0) reinterpret_cast<float*>(base + kCols * 4)[bb] = sx;
-                }
+            uint4 hi, lo;
+            hi.x = pack_h2(h[0], h[4]); hi.y = pack_h2(h[1], h[5]); hi.z = pack_h2(h[2], h[6]); hi.w = pack_h2(h[3], h[7]);
+            lo.x = pack_h2(l[0], l[4]); lo.y = pack_h2(l[1], l[5]); lo.z = pack_h2(l[2], l[6]); lo.w = pack_h2(l[3], l[7]);
+            float sx = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+            sx = dpp_add<0xB1>(sx);  // the 4 items of a block sit in 4 adjacent lanes
+            sx = dpp_add<0x4E>(sx);
+            if (w0 + i * kThreads < total) {
+                uint4* base = xs16 + blk * kPitch16;
+                base[(2 * bb) * 4 + dw] = hi;
+                base[(2 * bb + 1) * 4 + dw] = lo;
+                if (dw == 0) reinterpret_cast<float*>(base + kCols * 4)[bb] = sx;
             }
         }
+    };
+    // The first round of activations is requested before any weight (clamped, no branch): loads return
+    // in order, so behind the weight prefetch its staging and the barrier after it would wait until
+    // the first weights have crossed from HBM.
+    Round first;
+    load_round(first, tid);
+
+    // ring of kRing unit buffers: kRing - 1 units are in flight while one is consumed
+    Q4BlockRaw buf[kRing][2];
+#pragma unroll
+    for (int i = 0; i < kRing - 1; ++i)  // (a wave with fewer units re-reads its last one)
+        load_unit(buf[i], static_cast<uint32_t>(i) < units ? i : (units ? units - 1 : 0));
+    __builtin_amdgcn_sched_barrier(0);
+
+    store_round(first, tid);
+    for (uint32_t w0 = tid + G * kThreads; w0 < total; w0 += G * kThreads) {
+        Round r;
+        load_round(r, w0);
+        store_round(r, w0);
     }
     if (tid < 4) zero_region[tid] = make_uint4(0u, 0u, 0u, 0u);
     __syncthreads();

@@ -128,10 +128,25 @@ __global__ __launch_bounds__(kThreads) void gemv_q4_mfma(GemvArgs p) {
     auto first_row = [&](uint32_t it) { return ((blockIdx.x + it * gridDim.x) * RS + rs) * (4 * T); };
 
     // ---- the first activations are requested before any weight, so they can be waited on alone
-    const uint32_t items = nb * 4;  // (block, dword) pairs
-    const uint32_t it0 = static_cast<uint32_t>(tid) < items ? tid : 0;
-    const float4* x0p = reinterpret_cast<const float4*>(p.x + (it0 >> 2) * kBlockWeights + (it0 & 3) * 8);
-    const float4 x0a = x0p[0], x0b = x0p[1];
+    // (loads return in order: behind the weight prefetch their staging would wait for the weights).
+    // One (row, item) pair per thread, or a whole round of four with eight activation columns, whose
+    // kernels have the registers to spare at the occupancy their staged activations allow.
+    const uint32_t items = nb * 4;  // (block, dword) pairs per activation row
+    const uint32_t total_items = batch * items;
+    constexpr int kHoist = NSETS == 2 ? 4 : 1;
+    float4 hva[kHoist], hvb[kHoist];
+    uint32_t hrow[kHoist], hitem[kHoist];
+#pragma unroll
+    for (int i = 0; i < kHoist; ++i) {
+        const uint32_t w = tid + i * kThreads;
+        const uint32_t wc = w < total_items ? w : 0;
+        hrow[i] = wc / items;
+        hitem[i] = wc - hrow[i] * items;
+        const float4* xp = reinterpret_cast<const float4*>(p.x + static_cast<size_t>(hrow[i]) * p.x_stride +
+                                                           (hitem[i] >> 2) * kBlockWeights + (hitem[i] & 3) * 8);
+        hva[i] = xp[0];
+        hvb[i] = xp[1];
+    }
 
     // Loads unit u.  Blocks past the end of a row and rows past N re-read a valid block; their
     // contribution is zeroed or dropped later.
@@ -175,14 +190,14 @@ __global__ __launch_bounds__(kThreads) void gemv_q4_mfma(GemvArgs p) {
             if (dw == 0) reinterpret_cast<float*>(base + ncols * 4)[b] = sx;
         }
     };
-    stage(it0, 0, x0a, x0b, static_cast<uint32_t>(tid) < items);
+#pragma unroll
+    for (int i = 0; i < kHoist; ++i) stage(hitem[i], hrow[i], hva[i], hvb[i], tid + i * kThreads < total_items);
     // the remaining (row, item) pairs, four loads in flight per thread so that a batch of rows costs
     // a couple of memory round trips, not one per row
     {
         constexpr int G = 4;
-        const uint32_t total = batch * items;
-        const uint32_t done = static_cast<uint32_t>(tid) < items ? tid : ~0u;  // staged above
-        for (uint32_t w0 = tid; w0 < total; w0 += G * kThreads) {
+        const uint32_t total = total_items;
+        for (uint32_t w0 = tid + kHoist * kThreads; w0 < total; w0 += G * kThreads) {
             float4 va[G], vb[G];
             uint32_t wb[G], wi[G];
 #pragma unroll
@@ -197,10 +212,7 @@ __global__ __launch_bounds__(kThreads) void gemv_q4_mfma(GemvArgs p) {
                 vb[i] = xp[1];
             }
 #pragma unroll
-            for (int i = 0; i < G; ++i) {
-                const uint32_t w = w0 + i * kThreads;
-                stage(wi[i], wb[i], va[i], vb[i], w < total && w != done);
-            }
+            for (int i = 0; i < G; ++i) stage(wi[i], wb[i], va[i], vb[i], w0 + i * kThreads < total);
         }
     }
     if (tid < 4) zero_region[tid] = make_uint4(0u, 0u, 0u, 0u);

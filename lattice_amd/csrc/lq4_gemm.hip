@@ -11,8 +11,11 @@
 // ahead (they stream from HBM).
 //
 // With 64 x 64 wave tiles the LDS operand reads alone need the full LDS bandwidth at matrix-core
-// peak, so this kernel tops out near a third of peak; it is the kernel for shapes with too few
-// tiles to fill the chip with the larger weights-in-registers kernel (lq4_gemm_wreg.hip).
+// peak, so this kernel tops out near a third of peak.  The weights-in-registers kernel
+// (lq4_gemm_wreg.hip) serves Q4 and Q3 by default; this one serves Q8_0 on short or narrow
+// matrices and stays selectable for the others (block format = template argument FMT).  With
+// fewer tiles than workgroup slots it cuts K into ranges, one workgroup per (tile, range), and
+// gemm_sum_slices adds the partial tiles in range order.
 //
 // Dequantisation is done two weights per instruction: a masked dword OR-ed into the mantissa
 // of 1024.0 (or 64.0) is the f16 pair (1024+n_lo, 1024+n_hi); one packed subtract makes it

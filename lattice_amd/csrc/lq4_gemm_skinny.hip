@@ -1,4 +1,4 @@
-// Few-token prefill GEMM: Y[M,N] = X[M,K] . W[N,K]^T for a few dozen tokens (17 .. 128).
+// Few-token prefill GEMM: Y[M,N] = X[M,K] . W[N,K]^T for 2 .. 128 tokens, over Q4, Q8_0 or Q3 blocks.
 //
 // With so few tokens the product is bound by streaming W once, like the decode GEMV, but there
 // are too many tokens for the 4x4x4 GEMV kernel and too few to fill the 128-token tiles of the
@@ -8,15 +8,17 @@
 //    B operand wants them: for K step s (128 wide), token group t (16 tokens) and instruction j,
 //    the 64 lanes' 16-byte operands are contiguous (1 KB).  Lane (c = lane % 16, g = lane / 16)
 //    holds token 16 t + c, K offsets 128 s + 32 g + 8 j .. + 7 in the order x0 x4 x1 x5 x2 x6 x3
-//    x7 (the order in which the dequantiser emits a packed dword).  Tokens past M and K past the
-//    end are zero-filled, so the main kernel needs no tail handling on this operand.
+//    x7 (the order in which the Q4 dequantiser emits a packed dword; memory order for the sibling
+//    formats).  Tokens past M and K past the end are zero-filled, so the main kernel needs no tail
+//    handling on this operand.
 //
-// 2. gemm_q4_skinny<RT>: a workgroup of eight waves owns 16 RT weight rows against a tile of up
-//    to 64 tokens.  Wave w takes K steps w, w + 8, ...; per step it loads its own Q4 blocks
+// 2. gemm_q4_skinny<RT, FMT, NTG>: a workgroup of eight waves owns 16 RT weight rows against a tile
+//    of NTG groups of 16 tokens.  Wave w takes K steps w, w + 8, ...; per step it loads its own Q4 blocks
 //    (lane (r, g) owns block g of row r of the step, as in the large prefill kernel) and the
 //    packed operands with fully coalesced 16-byte loads, dequantises in registers and issues
 //    v_mfma_f32_16x16x32_f16.  No LDS staging and no barrier in the K loop: nothing is shared
-//    between waves.  Loads of the next step are in flight while the current one is multiplied.
+//    between waves.  Two steps are in flight per wave; every load is unconditional (a load behind a
+//    run-time condition would make the compiler wait for loads it cannot count).
 //    Each wave adds its share of the LoRA delta (ranks w, w + 8, ...) to its partial result in
 //    f32; the eight partial results then meet in LDS in a fixed order and y is stored once.
 //

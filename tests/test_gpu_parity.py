@@ -357,6 +357,18 @@ def test_moe_route_matches_oracle(be):
     assert np.array_equal(host(ids), o_ids) and np.array_equal(host(wts), o_wts)
 
 
+def test_moe_route_argument_checks(be):
+    import torch
+    from lattice_amd import backend
+    lg = torch.zeros((2, 1025), device="cuda")
+    with pytest.raises(backend.Q4Error, match="num_experts"):
+        be.moe_route(lg, 4)            # more experts than a wave's lanes can hold
+    with pytest.raises(backend.Q4Error, match="top_k"):
+        be.moe_route(lg[:, :8], 9)     # more ranks than experts
+    with pytest.raises(backend.Q4Error, match="top_k"):
+        be.moe_route(lg[:, :64].contiguous(), 17)
+
+
 @pytest.mark.parametrize("tokens,experts,top_k", [(33, 256, 8), (5, 100, 16), (3, 1000, 7), (70, 9, 9), (1, 1024, 1)])
 def test_moe_route_expert_counts_and_ties(be, tokens, experts, top_k):
     # expert counts off the 64-lane grid, as many ranks as experts, and rows with many equal logits

@@ -353,7 +353,10 @@ void launch_phase(MoeGemvArgs a, uint32_t num_experts, uint32_t max_pairs_per_ex
     const uint32_t nsteps = (a.k / kBlockWeights + 15) / 16;
     constexpr uint32_t rows_per_tp = GATE_UP ? 4 : 8;
     // about 32 (gate/up) or 128 (down) output rows per workgroup: 40-80 KB of blocks each
-    const uint32_t target_rows = GATE_UP ? 32 : 128;
+    // (half of that for a single token's worth of pairs: with so few workgroups at work the chip is
+    // filled by more, smaller ones; measured 26.7 -> 23.7 us at 8 pairs, but slower from 128 pairs on)
+    const bool few_pairs = a.n_pairs <= 16;
+    const uint32_t target_rows = GATE_UP ? (few_pairs ? 16 : 32) : (few_pairs ? 64 : 128);
     // Waves split the output rows; they split K as well only when an expert has too few rows to
     // give every wave a tile pair (each K slice costs a cross-lane reduction per tile pair).
     uint32_t ks = 1;

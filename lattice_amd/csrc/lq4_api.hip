@@ -18,6 +18,7 @@ struct lq4_ctx {
     int device;
     float* lora_t;        // [kLoraTRows, kMaxLoraRank] f32: A.x of the call in flight
     uint8_t* moe_scratch; // grown on demand
+    uint32_t* topk_ticket; // finished-workgroup count of the top-k kernel, zero between launches
     size_t moe_scratch_bytes;
     lq4_path_counters counters;
 };
@@ -161,6 +162,14 @@ int lq4_ctx_create(int device_ordinal, lq4_ctx** out) {
         delete c;
         return fail(LQ4_E_HIP, "hipMalloc(lora scratch): %s", hipGetErrorString(e));
     }
+    e = hipMalloc(reinterpret_cast<void**>(&c->topk_ticket), 256);
+    if (e == hipSuccess) e = hipMemset(c->topk_ticket, 0, 256);
+    if (e != hipSuccess) {
+        (void)hipFree(c->topk_ticket);
+        (void)hipFree(c->lora_t);
+        delete c;
+        return fail(LQ4_E_HIP, "hipMalloc(top-k ticket): %s", hipGetErrorString(e));
+    }
     *out = c;
     return LQ4_OK;
 }
@@ -169,6 +178,7 @@ int lq4_ctx_destroy(lq4_ctx* ctx) {
     if (!ctx) return LQ4_OK;
     DeviceGuard g(ctx->device);
     (void)hipFree(ctx->lora_t);
+    (void)hipFree(ctx->topk_ticket);
     if (ctx->moe_scratch) (void)hipFree(ctx->moe_scratch);
     delete ctx;
     return LQ4_OK;
@@ -501,7 +511,8 @@ int lq4_topk(lq4_ctx* ctx, const float* logits_dev, uint32_t n, uint32_t top_k, 
     DeviceGuard g(ctx->device);
     const int rc = ensure_scratch(ctx, topk_scratch_bytes(n, top_k));
     if (rc) return rc;
-    launch_topk(logits_dev, n, top_k, ctx->moe_scratch, out_logits_dev, out_ids_dev, static_cast<hipStream_t>(stream));
+    launch_topk(logits_dev, n, top_k, ctx->moe_scratch, ctx->topk_ticket, out_logits_dev, out_ids_dev,
+                static_cast<hipStream_t>(stream));
     ctx->counters.topk++;
     LQ4_HIP(hipGetLastError());
     return LQ4_OK;
@@ -528,7 +539,7 @@ int lq4_lm_head_topk(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset,
     hipStream_t s = static_cast<hipStream_t>(stream);
     const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};
     launch_gemv(wp, vocab, k, x_dev, k, 1, logits, vocab, none, s);
-    launch_topk(logits, vocab, top_k, ctx->moe_scratch + logits_bytes, out_logits_dev, out_ids_dev, s);
+    launch_topk(logits, vocab, top_k, ctx->moe_scratch + logits_bytes, ctx->topk_ticket, out_logits_dev, out_ids_dev, s);
     ctx->counters.gemv++;
     ctx->counters.topk++;
     LQ4_HIP(hipGetLastError());

@@ -167,10 +167,11 @@ void launch_moe_down_mfma(const uint8_t* down, uint32_t num_experts, uint32_t in
                           const int32_t* order, const int32_t* ids, float* o, hipStream_t stream);
 
 // Exact top-k over n logits (k <= 256): out_logits / out_ids receive the k best in rank order.
-// `scratch` must hold topk_scratch_bytes(n, k) bytes.
+// `scratch` must hold topk_scratch_bytes(n, k) bytes; `ticket` is one device word that is zero
+// between launches (the kernel counts finished workgroups in it and puts it back to zero).
 size_t topk_scratch_bytes(uint32_t n, uint32_t k);
-void launch_topk(const float* logits, uint32_t n, uint32_t k, void* scratch, float* out_logits, uint32_t* out_ids,
-                 hipStream_t stream);
+void launch_topk(const float* logits, uint32_t n, uint32_t k, void* scratch, uint32_t* ticket, float* out_logits,
+                 uint32_t* out_ids, hipStream_t stream);
 
 // ---- device helpers ---------------------------------------------------------------
 // v summed over the four 16-lane rows of a wave: every lane ends with the total of the four lanes

@@ -1,10 +1,12 @@
 // Exact top-k selection over a vector of logits: the device side of the reference's two-stage
 // lm_head top-k (shaders/qwen35.metal:1683-1778, 1868-1985).
 //
-// Stage 1 sorts tiles of 1024 logits and keeps each tile's k best; merge passes then sort up to
-// 2048 surviving candidates at a time and keep k, until one group is left.  Every pass is a full
-// bitonic sort of its candidates, so each tile's list is its exact local top-k and the result is
-// the first k entries of the globally sorted list — independent of tile size and fan-in.
+// Small inputs take the reference's route: stage 1 sorts tiles of 1024 logits and keeps each
+// tile's k best; merge passes then sort up to 2048 surviving candidates at a time and keep k,
+// until one group is left.  Every pass is a full bitonic sort of its candidates, so each tile's
+// list is its exact local top-k and the result is the first k entries of the globally sorted
+// list — independent of tile size and fan-in.  Inputs of at least k blocks of 256 take the
+// threshold route further down, which returns the same list without sorting.
 // Ordering (qwen35.metal:1697-1703): higher logit first, ties to the lower token id; a NaN logit
 // enters as the sentinel (-inf, 0xFFFFFFFF) and ranks last.
 #include "lq4_internal.hpp"
@@ -12,6 +14,8 @@
 namespace lq4 {
 
 namespace {
+
+typedef float float4v __attribute__((ext_vector_type(4)));
 
 struct Cand {
     float logit;
@@ -104,12 +108,28 @@ __global__ __launch_bounds__(256) void topk_merge_kernel(const Cand* __restrict_
 }
 
 // ---- fast path: threshold from block maxima, then rank the few survivors ---------------------
-// The vector is cut into M <= 1024 blocks of `blk` logits.  tau = the k-th best block maximum.
-// At least k elements (the maxima themselves) rank at or before tau, so every global top-k
-// element does too; exactly k blocks can contain such elements, so at most k * blk survive.
+// The vector is cut into M <= 1024 blocks of `blk` logits.  tau = a key that at least k of the
+// block maxima reach (the k-th best maximum, or a little below it).  At least k elements (those
+// maxima) rank at or before tau, so every global top-k element does too, and only the blocks whose
+// maximum reaches tau can contain such elements: at most topk_most_blocks(k) * blk survive.
 // The survivors are ranked by counting, for each, how many survivors beat it: `better` is a
-// strict total order, so ranks are distinct and rank r goes to output slot r.  No sorting, no
-// barriers on the critical path, and the result is the same exact list the tile/merge path gives.
+// strict total order, so ranks are distinct and rank r goes to output slot r.  No sorting, and
+// the result is the same exact list the tile/merge path gives.
+//
+// For k <= 64 one launch does all of it.  Every wave reduces one block to its best key; the
+// workgroup that draws the last ticket (all maxima are then in memory) finds tau, rescans the
+// blocks whose maximum reaches tau (50 KB for k = 50) and ranks what it found.  The steps after
+// the maxima are serial work for one workgroup, but each is short (a thousand keys, k blocks,
+// typically 1-3 k survivors), and three launches with their ramp-up and drain are gone: 13.9 us
+// instead of 17 for the top 50 of 248 320 logits.
+//
+// How the maxima reach the last workgroup: each is written with a device-scope atomic exchange,
+// whose returned old value the wave waits for before its workgroup draws a ticket (another
+// device-scope atomic); the last workgroup reads them with device-scope atomic loads.  Atomics at
+// device scope are carried out where all compute dies see them, so a load issued after the last
+// ticket came back finds every exchange done.  Plain stores with a device-wide fence before the
+// ticket would be the textbook form; the fence writes the whole L2 back and, at one per
+// workgroup, made the kernel 13 us slower.
 
 // 64-bit sort key of a candidate: a ranks before b  <=>  key(a) > key(b).  High word: the logit's
 // bits mapped to an unsigned order (-0 counted as +0, as the float comparison does); low word:
@@ -136,6 +156,274 @@ __device__ __forceinline__ uint64_t wave_max_key(uint64_t k) {
     }
     return k;
 }
+
+// A candidate this workgroup stored a moment ago, read back past the vector cache.
+__device__ __forceinline__ Cand load_survivor(const Cand* surv, uint32_t i) {
+    const uint64_t raw =
+        __hip_atomic_load(reinterpret_cast<const uint64_t*>(surv) + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return Cand{__uint_as_float(static_cast<uint32_t>(raw)), static_cast<uint32_t>(raw >> 32)};
+}
+
+struct SelectShared {
+    uint32_t hist[256];
+    uint64_t prefix;
+    uint32_t need;
+};
+
+// The k-th largest (k >= 1, counted with multiplicity) of the `count` >= k keys get(0..count):
+// eight rounds of an 8-bit radix select, most significant digit first.  A round counts the digit
+// of every key that still matches the digits fixed so far; wave 0 walks the 256 counts from the
+// top to the digit that holds the `need`-th key.  Called by all 256 threads of the workgroup.
+template <typename Get>
+__device__ __forceinline__ uint64_t select_kth_key(Get get, uint32_t count, uint32_t k, SelectShared& sh) {
+    const uint32_t tid = threadIdx.x;
+    uint64_t prefix = 0;
+    uint32_t need = k;
+    for (int shift = 56; shift >= 0; shift -= 8) {
+        sh.hist[tid] = 0;
+        __syncthreads();
+        for (uint32_t i = tid; i < count; i += 256) {
+            const uint64_t key = get(i);
+            // (x >> 1) >> 63-or-less: a shift by 64 is not defined, the first round matches all
+            const bool match = (((key ^ prefix) >> 1) >> (shift + 7)) == 0;
+            if (match) atomicAdd(&sh.hist[(key >> shift) & 255], 1u);
+        }
+        __syncthreads();
+        if (tid < 64) {  // lane l owns digits 255 - 4l .. 252 - 4l, highest first
+            uint32_t c[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) c[j] = sh.hist[255 - 4 * tid - j];
+            const uint32_t sum = (c[0] + c[1]) + (c[2] + c[3]);
+            uint32_t incl = sum;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const uint32_t t = __shfl_up(incl, off, 64);
+                if (tid >= static_cast<uint32_t>(off)) incl += t;
+            }
+            uint32_t run = incl - sum;
+            if (run < need && need <= incl) {  // exactly one lane: the counts above it fall short
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (run < need && need <= run + c[j]) {
+                        sh.prefix = prefix | (static_cast<uint64_t>(255 - 4 * tid - j) << shift);
+                        sh.need = need - run;
+                    }
+                    run += c[j];
+                }
+            }
+        }
+        __syncthreads();
+        prefix = sh.prefix;
+        need = sh.need;
+    }
+    return prefix;
+}
+
+constexpr uint32_t kRankSlots = 1024;  // survivors ranked out of LDS
+constexpr uint32_t kSingleKernelMaxK = 64;
+constexpr int kGatherUnits = 16;       // 16-byte loads a thread has in flight when rescanning: 50 blocks of 256 in one go
+
+// The threshold may let up to this many blocks through instead of exactly k: it is found in fewer
+// steps, and the survivor buffer is sized for it.
+__host__ __device__ constexpr uint32_t topk_most_blocks(uint32_t k) { return k + (k >> 2) + 4; }
+
+// grid ceil(M / 4), block 256: wave w of workgroup g reduces block 4g + w of `blk` logits to its
+// best key; the workgroup with the last ticket selects, rescans and ranks (see above).  `ticket`
+// is zero between launches: the last workgroup puts it back.  `surv` holds topk_most_blocks(k) * blk
+// candidates.
+__global__ __launch_bounds__(256) void topk_select_kernel(const float* __restrict__ logits, uint32_t n, uint32_t blk,
+                                                          uint32_t m, uint32_t k, uint64_t* maxima, Cand* surv,
+                                                          uint32_t* ticket, float* __restrict__ out_logits,
+                                                          uint32_t* __restrict__ out_ids) {
+    __shared__ uint64_t s_keys[kRankSlots];
+    __shared__ float s_vals[kRankSlots];
+    __shared__ uint32_t s_ids[kRankSlots];
+    __shared__ uint16_t s_sel[1024];
+    __shared__ SelectShared sh;
+    __shared__ uint32_t s_cnt[2][4];
+    __shared__ uint32_t s_count, s_nsel, s_tail, s_last;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63;
+    {
+        const uint32_t b = blockIdx.x * 4 + (tid >> 6);
+        if (b < m) {
+            const uint32_t beg = b * blk;
+            const uint32_t end = beg + blk < n ? beg + blk : n;
+            uint64_t best = key_of(sentinel());
+            for (uint32_t i = beg + lane; i < end; i += 64) {
+                const uint64_t kk = key_of(load_cand(logits, i));
+                best = kk > best ? kk : best;
+            }
+            best = wave_max_key(best);
+            if (lane == 0) {
+                // An exchange at device scope is carried out where every part of the chip sees it,
+                // and once its old value has come back it is done: the empty statement below
+                // takes that value, so the wave waits for it before the barrier and the ticket.
+                // (A device-wide fence instead costs every workgroup a cache write-back.)
+                const uint64_t old = __hip_atomic_exchange(maxima + b, best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                asm volatile("" ::"v"(static_cast<uint32_t>(old)));
+            }
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {
+        const uint32_t t = atomicAdd(ticket, 1u);
+        s_last = t == gridDim.x - 1;
+        // every other workgroup has drawn: ready for the next launch
+        if (s_last) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_count = 0;
+        s_nsel = 0;
+        s_tail = 0;
+    }
+    __syncthreads();
+    if (!s_last) return;
+
+    for (uint32_t o = tid; o < k; o += 256) {  // slots no survivor claims (NaN input) keep the sentinel
+        out_logits[o] = -INFINITY;
+        out_ids[o] = 0xFFFFFFFFu;
+    }
+
+    // tau: a key that at least k and at most `most` of the block maxima reach.  Built from the top
+    // bit down (a bit stays set if k maxima still reach the result); the first value that no more
+    // than `most` maxima reach will do, and if none comes up the loop ends at the k-th best
+    // maximum itself.  A step is four compares per thread and one barrier.
+    uint64_t kk[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)  // device-scope loads, as the maxima were written; 0: below every key
+        kk[j] = tid + 256 * j < m ? __hip_atomic_load(maxima + tid + 256 * j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                  : 0ull;
+    const uint32_t most = topk_most_blocks(k);
+    uint64_t tau = 0;
+    for (int bit = 63, par = 0; bit >= 0; --bit, par ^= 1) {
+        const uint64_t cand = tau | (1ull << bit);
+        uint32_t c = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) c += __popcll(__ballot(kk[j] >= cand));
+        if (lane == 0) s_cnt[par][tid >> 6] = c;
+        __syncthreads();  // one barrier a step: the two halves of s_cnt take turns
+        c = (s_cnt[par][0] + s_cnt[par][1]) + (s_cnt[par][2] + s_cnt[par][3]);
+        if (c >= k) {
+            tau = cand;
+            if (c <= most) break;
+        }
+    }
+
+    // the blocks that can hold an element at or before tau: at most `most` (more only if tau is
+    // the all-NaN key, and then the extra blocks hold nothing that passes the test below)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if (kk[j] >= tau && tid + 256 * j < m) {
+            s_sel[atomicAdd(&s_nsel, 1u)] = static_cast<uint16_t>(tid + 256 * j);
+            if (tid + 256 * j == m - 1) s_tail = 1;
+        }
+    }
+    __syncthreads();
+    const uint32_t nsel = s_nsel;
+    // Survivors: every logit of those blocks that is not below tau's logit (tau's high word mapped
+    // back to a float; a word below every real key means that -inf still passes).  One compare,
+    // which NaN fails; an element that ties tau's logit with a higher id passes although it ranks
+    // after tau, which costs a slot and nothing else.
+    const uint32_t tau_u = static_cast<uint32_t>(tau >> 32);
+    const float tau_f = tau_u < 0x007FFFFFu ? -INFINITY
+                                            : __uint_as_float((tau_u >> 31) ? tau_u ^ 0x80000000u : ~tau_u);
+    auto consider = [&](float v, uint32_t i) {
+        if (!(v >= tau_f)) return;
+        const uint32_t slot = atomicAdd(&s_count, 1u);
+        if (slot < kRankSlots) {
+            s_vals[slot] = v;
+            s_ids[slot] = i;
+        }
+        surv[slot] = Cand{v, i};
+    };
+    // All loads of a batch are issued before the first is looked at: one workgroup has to cover
+    // the latency of nsel * blk logits by itself.  Slots past the end reload element 0 and drop it.
+    const uint32_t lb = __ffs(blk) - 1;  // blk is a power of two
+    if ((reinterpret_cast<uintptr_t>(logits) & 15) == 0) {
+        const uint32_t units = nsel << (lb - 2);  // 4 logits each
+        const uint32_t whole = n & ~3u;           // logits below this index sit in whole units
+        for (uint32_t u0 = 0; u0 < units; u0 += 256 * kGatherUnits) {
+            float4v v[kGatherUnits];
+            uint32_t idx[kGatherUnits];
+#pragma unroll
+            for (int j = 0; j < kGatherUnits; ++j) {
+                const uint32_t u = u0 + j * 256 + tid < units ? u0 + j * 256 + tid : 0;
+                const uint32_t i = (static_cast<uint32_t>(s_sel[u >> (lb - 2)]) << lb) + ((u & ((blk >> 2) - 1)) << 2);
+                const bool ok = u0 + j * 256 + tid < units && i < whole;
+                idx[j] = i;
+                v[j] = *reinterpret_cast<const float4v*>(logits + (ok ? i : 0));
+                if (!ok) v[j] = float4v{NAN, NAN, NAN, NAN};
+            }
+#pragma unroll
+            for (int j = 0; j < kGatherUnits; ++j) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) consider(v[j][e], idx[j] + e);
+            }
+        }
+        if (s_tail && tid < (n & 3)) consider(logits[whole + tid], whole + tid);  // the last block's odd end
+    } else {
+        const uint32_t elems = nsel << lb;
+        for (uint32_t e0 = 0; e0 < elems; e0 += 256 * kGatherUnits) {
+            float v[kGatherUnits];
+            uint32_t idx[kGatherUnits];
+#pragma unroll
+            for (int j = 0; j < kGatherUnits; ++j) {
+                const uint32_t e = e0 + j * 256 + tid < elems ? e0 + j * 256 + tid : 0;
+                const uint32_t i = (static_cast<uint32_t>(s_sel[e >> lb]) << lb) + (e & (blk - 1));
+                const bool ok = e0 + j * 256 + tid < elems && i < n;
+                idx[j] = i;
+                v[j] = logits[ok ? i : 0];
+                if (!ok) v[j] = NAN;
+            }
+#pragma unroll
+            for (int j = 0; j < kGatherUnits; ++j) consider(v[j], idx[j]);
+        }
+    }
+    __syncthreads();
+    uint32_t total = s_count;
+    for (uint32_t e = tid; e < (total < kRankSlots ? total : kRankSlots); e += 256)
+        s_keys[e] = key_of(Cand{s_vals[e], s_ids[e]});
+    if (total > kRankSlots) {
+        // too many to rank from LDS (sorted or constant input): keep exactly the k best of them,
+        // read back from memory
+        __threadfence();
+        __syncthreads();
+        const uint64_t tau2 = select_kth_key(
+            [&](uint32_t i) { return key_of(load_survivor(surv, i)); }, total, k, sh);
+        if (tid == 0) s_count = 0;
+        __syncthreads();
+        for (uint32_t i = tid; i < total; i += 256) {
+            const Cand c = load_survivor(surv, i);
+            const uint64_t key = key_of(c);
+            if (key >= tau2) {  // keys are distinct: k of them
+                const uint32_t slot = atomicAdd(&s_count, 1u);
+                s_keys[slot] = key;
+                s_vals[slot] = c.logit;
+            }
+        }
+        __syncthreads();
+        total = s_count;
+    }
+    const uint32_t lim = (total + 15) & ~15u;
+    for (uint32_t i = total + tid; i < lim; i += 256) s_keys[i] = 0;  // below every real key
+    __syncthreads();
+    for (uint32_t e = tid; e < total; e += 256) {
+        const uint64_t ck = s_keys[e];
+        uint32_t rank = 0;
+        for (uint32_t j0 = 0; j0 < lim; j0 += 16) {
+#pragma unroll
+            for (uint32_t u = 0; u < 16; ++u) rank += s_keys[j0 + u] > ck;
+        }
+        if (rank < k) {
+            out_logits[rank] = s_vals[e];
+            out_ids[rank] = ~static_cast<uint32_t>(ck);
+        }
+    }
+}
+
+// ---- the same selection as four launches, for large k ---------------------------------------
+// The single kernel above leaves the rescan of the surviving blocks to one workgroup; from about
+// 64 blocks on (k = 256: 320 KB of logits) a grid doing that work in parallel is faster even with
+// three more launches: 20 us against 34 for k = 256 over 248 320 logits.
 
 // grid M, block 256: key of the best candidate of block b of `blk` logits.
 __global__ __launch_bounds__(256) void topk_blockmax_kernel(const float* __restrict__ logits, uint32_t n, uint32_t blk,
@@ -237,7 +525,7 @@ __global__ __launch_bounds__(256) void topk_rank_kernel(const Cand* __restrict__
 
 // blocks of `blk` logits such that there are at most 1024 of them; 0 = fast path not applicable
 uint32_t fast_block(uint32_t n, uint32_t k) {
-    uint32_t blk = 256;
+    uint32_t blk = 64;  // a wave's width; smaller blocks only add maxima
     while ((n + blk - 1) / blk > 1024) blk <<= 1;
     return (n + blk - 1) / blk >= k ? blk : 0;
 }
@@ -246,20 +534,26 @@ uint32_t fast_block(uint32_t n, uint32_t k) {
 
 size_t topk_scratch_bytes(uint32_t n, uint32_t k) {
     const uint32_t blk = fast_block(n, k);
-    if (blk)  // maxima[1024] | tau | counter | survivors (at most k blocks survive)
-        return (1024 + 2) * sizeof(Cand) + static_cast<size_t>(k) * blk * sizeof(Cand);
+    if (blk)  // maxima[1024] | tau, counter (large k only) | survivors
+        return (1024 + 2) * sizeof(uint64_t) + static_cast<size_t>(topk_most_blocks(k)) * blk * sizeof(Cand);
     const size_t tiles = (n + kTile - 1) / kTile;
     return 2 * tiles * k * sizeof(Cand);  // two candidate buffers, ping-pong
 }
 
-void launch_topk(const float* logits, uint32_t n, uint32_t k, void* scratch, float* out_logits, uint32_t* out_ids,
-                 hipStream_t stream) {
+void launch_topk(const float* logits, uint32_t n, uint32_t k, void* scratch, uint32_t* ticket, float* out_logits,
+                 uint32_t* out_ids, hipStream_t stream) {
     if (const uint32_t blk = fast_block(n, k)) {
         const uint32_t m = (n + blk - 1) / blk;
         uint64_t* maxima = static_cast<uint64_t*>(scratch);
+        Cand* surv = reinterpret_cast<Cand*>(maxima + 1024);
+        if (k <= kSingleKernelMaxK) {
+            hipLaunchKernelGGL(topk_select_kernel, dim3((m + 3) / 4), dim3(256), 0, stream, logits, n, blk, m, k,
+                               maxima, surv, ticket, out_logits, out_ids);
+            return;
+        }
         uint64_t* tau = maxima + 1024;
         uint32_t* counter = reinterpret_cast<uint32_t*>(tau + 1);
-        Cand* surv = reinterpret_cast<Cand*>(tau + 2);
+        surv = reinterpret_cast<Cand*>(tau + 2);
         hipLaunchKernelGGL(topk_blockmax_kernel, dim3(m), dim3(256), 0, stream, logits, n, blk, maxima);
         hipLaunchKernelGGL(topk_threshold_kernel, dim3((m + 15) / 16), dim3(256), 0, stream, maxima, m, k, tau, counter,
                            out_logits, out_ids);

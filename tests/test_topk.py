@@ -59,8 +59,18 @@ def _cases():
     nans[::3] = np.nan
     nans[10] = np.inf
     nans[11] = -np.inf
+    zeros = np.zeros(n, np.float32)
+    zeros[g.integers(0, n, n // 2)] = -0.0           # -0 and +0 tie (lower id first) and keep their sign bit
+    zeros[g.integers(0, n, 20)] = -1.0
+    few_real = np.full(n, np.nan, np.float32)        # fewer real values than k: the rest stay sentinels
+    few_real[g.integers(0, n, 30)] = g.normal(size=30).astype(np.float32)
     return {"random": base, "clustered": clustered, "ties": ties, "nan_inf": nans,
-            "short": base[:777], "one_tile_exact": base[:1024], "all_nan": np.full(2000, np.nan, np.float32)}
+            "short": base[:777], "one_tile_exact": base[:1024], "all_nan": np.full(2000, np.nan, np.float32),
+            # whole blocks survive the threshold: thousands of candidates to cut down to k
+            "ascending": np.arange(n, dtype=np.float32), "descending": -np.arange(n, dtype=np.float32),
+            "constant": np.full(n, 3.25, np.float32), "signed_zeros": zeros, "few_real": few_real,
+            "odd_length": base[:100003],
+            "small_vocabulary": base[:32000]}  # blocks of 64 logits so that there are at least k of them
 
 
 @pytest.mark.gpu
@@ -106,3 +116,25 @@ def test_gpu_lm_head_topk_matches_gemv_then_topk():
         if o_l[r] - o_l[r + 1] > eps and (r == 0 or o_l[r - 1] - o_l[r] > eps):
             assert got[r] == o_i[r], r
     assert np.abs(out_l.cpu().numpy() - o_l[:top_k]).max() <= eps
+
+
+@pytest.mark.gpu
+def test_gpu_topk_back_to_back_calls_use_their_own_block_maxima():
+    """The one-launch selection hands every block's best key to the workgroup that finishes last
+    through device-scope atomics, in scratch memory that all calls share.  A call that picked up
+    the previous call's keys would set its threshold from the wrong data: after the 'high' input
+    the 'low' input would find nothing at or above it and return sentinels.  Many alternating calls,
+    each checked, with lengths that move the block boundaries."""
+    import torch
+    from lattice_amd import backend
+    be = backend.HipQ4Backend(0)
+    g = np.random.default_rng(99)
+    inputs = []
+    for n, lo_, hi_ in [(248320, 0.0, 1.0), (248320, 100.0, 101.0), (151936, -50.0, -49.0), (200003, 7.0, 8.0)]:
+        lg = g.uniform(lo_, hi_, size=n).astype(np.float32)
+        inputs.append((torch.from_numpy(lg).cuda(), oracle.topk(lg, 50)))
+    for r in range(150):
+        outs = [be.topk(dev_lg, 50) for dev_lg, _ in inputs]  # queued back to back, checked afterwards
+        for (out_l, out_i), (_, (want_l, want_i)) in zip(outs, inputs):
+            assert np.array_equal(out_i.cpu().numpy().view(np.uint32), want_i), r
+            assert np.array_equal(out_l.cpu().numpy().view(np.uint32), want_l.view(np.uint32)), r

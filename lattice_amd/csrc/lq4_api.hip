@@ -331,7 +331,10 @@ int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
     // mid-sized matrices only (measured: behind for 512 x 2048, where its two launches dominate,
     // and for 12288 x 2048, where the GEMV kernel's grid already fills the chip).
     const uint64_t weights = static_cast<uint64_t>(n) * k;
-    if (batch >= 9 || (batch >= 5 && n < 8192 && weights >= 6000000)) {
+    // (not for up to 2048 rows while the GEMV kernel can stage the activations: its eight-wave
+    // workgroups then win, 2048 x 6144 at 5..8 rows 9.5 -> 7.2..8.2 us)
+    const bool narrow = n <= 2048 && gemv_mfma_lds_bytes(k, batch < 8 ? batch : 8) <= 150 * 1024;
+    if (batch >= 9 || (batch >= 5 && n < 8192 && !narrow && weights >= 6000000)) {
         rc = ensure_scratch(ctx, gemm_skinny_scratch_bytes(k, batch));
         if (rc) return rc;
         launch_gemm_skinny(wp, n, k, x_dev, 0, batch, y_dev, ep, ctx->moe_scratch, s);

@@ -41,7 +41,6 @@ typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 
-constexpr int kThreads = 256;
 constexpr float kLoScale = 2048.0f;
 constexpr float kTwo24 = 16777216.0f;
 
@@ -94,13 +93,15 @@ struct GemvArgs {
 
 // NSETS: groups of four activation columns (1 or 2).  HILO: two columns per activation row.
 // T: weight-row tiles (of 4 rows) per wave.  KS: slices of K per workgroup (1, 2 or 4).
+// WAVES: waves per workgroup (4 or 8), all served by one staged copy of the activations.
 // Workgroups are persistent: workgroup g handles row groups g, g + gridDim.x, ... (a row group
-// is 4*T*(4/KS) rows) with the activations staged once.  For one wave the work is a list of
+// is 4*T*(WAVES/KS) rows) with the activations staged once.  For one wave the work is a list of
 // units (row group, step); unit u+1 is in flight while unit u is consumed.
-template <int NSETS, bool HILO, int T, int KS, bool LONG>
-__global__ __launch_bounds__(kThreads) void gemv_q4_mfma(GemvArgs p) {
+template <int NSETS, bool HILO, int T, int KS, bool LONG, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void gemv_q4_mfma(GemvArgs p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    constexpr int RS = 4 / KS;  // row sub-groups per workgroup
+    constexpr int kThreads = 64 * WAVES;
+    constexpr int RS = WAVES / KS;  // row sub-groups per workgroup
     constexpr int NCOLS = 4 * NSETS;
     constexpr uint32_t kRowsPerIter = 4 * T * RS;
     const int tid = threadIdx.x;
@@ -117,8 +118,8 @@ __global__ __launch_bounds__(kThreads) void gemv_q4_mfma(GemvArgs p) {
     uint4* const xs16 = reinterpret_cast<uint4*>(smem);
     const uint32_t pitch16 = pitch / 16;
     uint4* const zero_region = xs16 + nb * pitch16;               // 64 B of zeros
-    float* red = reinterpret_cast<float*>(zero_region + 4);       // [2][4 waves][T][NCOLS][4]
-    constexpr int kRedFloats = 4 * T * NCOLS * 4;
+    float* red = reinterpret_cast<float*>(zero_region + 4);       // [2][WAVES][T][NCOLS][4]
+    constexpr int kRedFloats = WAVES * T * NCOLS * 4;
 
     const int ks = wave % KS, rs = wave / KS;
     const uint32_t n_groups = (p.n + kRowsPerIter - 1) / kRowsPerIter;
@@ -382,46 +383,55 @@ __global__ __launch_bounds__(kThreads) void gemv_q4_mfma(GemvArgs p) {
     }
 }
 
-template <int NSETS, bool HILO, int T, int KS, bool LONG>
+template <int NSETS, bool HILO, int T, int KS, bool LONG, int WAVES>
 void launch_long(const GemvArgs& a, size_t lds, uint32_t wgs, hipStream_t stream) {
     static bool attr_set = false;  // raise the dynamic-LDS cap once per instantiation
     if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_mfma<NSETS, HILO, T, KS, LONG>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_mfma<NSETS, HILO, T, KS, LONG, WAVES>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         attr_set = true;
     }
-    hipLaunchKernelGGL((gemv_q4_mfma<NSETS, HILO, T, KS, LONG>), dim3(wgs), dim3(kThreads), lds, stream, a);
+    hipLaunchKernelGGL((gemv_q4_mfma<NSETS, HILO, T, KS, LONG, WAVES>), dim3(wgs), dim3(64 * WAVES), lds, stream, a);
 }
 
-template <int NSETS, bool HILO, int T, int KS>
+template <int NSETS, bool HILO, int T, int KS, int WAVES>
 void launch_cfg(const GemvArgs& a, size_t lds, uint32_t max_wgs, hipStream_t stream) {
-    constexpr uint32_t rows_per_iter = 4 * T * (4 / KS);
+    constexpr uint32_t rows_per_iter = 4 * T * (WAVES / KS);
     const uint32_t groups = (a.n + rows_per_iter - 1) / rows_per_iter;
     // every workgroup gets the same number of row groups, to within one
     const uint32_t iters = (groups + max_wgs - 1) / max_wgs;
     const uint32_t wgs = (groups + iters - 1) / iters;
     const uint32_t nsteps = (a.k / kBlockWeights + 15) / 16;
     const uint32_t units = iters * ((nsteps + KS - 1) / KS);  // per wave
-    if (units >= 8) launch_long<NSETS, HILO, T, KS, true>(a, lds, wgs, stream);
-    else launch_long<NSETS, HILO, T, KS, false>(a, lds, wgs, stream);
+    if (units >= 8) launch_long<NSETS, HILO, T, KS, true, WAVES>(a, lds, wgs, stream);
+    else launch_long<NSETS, HILO, T, KS, false, WAVES>(a, lds, wgs, stream);
 }
 
 template <int NSETS, bool HILO>
-void launch_shape(const GemvArgs& a, size_t lds, uint32_t t, uint32_t ks, uint32_t max_wgs, hipStream_t stream) {
-#define LQ4_CASE(T_, KS_) if (t == T_ && ks == KS_) return launch_cfg<NSETS, HILO, T_, KS_>(a, lds, max_wgs, stream)
-    LQ4_CASE(1, 4); LQ4_CASE(1, 2); LQ4_CASE(1, 1);
-    LQ4_CASE(2, 4); LQ4_CASE(2, 2); LQ4_CASE(2, 1);
-    LQ4_CASE(4, 4); LQ4_CASE(4, 2); LQ4_CASE(4, 1);
+void launch_shape(const GemvArgs& a, size_t lds, uint32_t t, uint32_t ks, uint32_t waves, uint32_t max_wgs,
+                  hipStream_t stream) {
+#define LQ4_CASE(T_, KS_, W_) \
+    if (t == T_ && ks == KS_ && waves == W_) return launch_cfg<NSETS, HILO, T_, KS_, W_>(a, lds, max_wgs, stream)
+    LQ4_CASE(1, 4, 4); LQ4_CASE(1, 2, 4); LQ4_CASE(1, 1, 4);
+    LQ4_CASE(2, 4, 4); LQ4_CASE(2, 2, 4); LQ4_CASE(2, 1, 4);
+    LQ4_CASE(4, 4, 4); LQ4_CASE(4, 2, 4); LQ4_CASE(4, 1, 4);
+    LQ4_CASE(1, 4, 8); LQ4_CASE(1, 2, 8); LQ4_CASE(1, 1, 8);
+    LQ4_CASE(2, 4, 8); LQ4_CASE(2, 2, 8); LQ4_CASE(2, 1, 8);
 #undef LQ4_CASE
 }
 
 }  // namespace
 
+// the K slices' meeting point: [2][waves][T <= 4][columns <= 8][4] floats
+constexpr size_t kRedBytes4 = 2 * 4 * 4 * 8 * 4 * sizeof(float);
+constexpr size_t kRedBytes8 = 2 * 8 * 2 * 8 * 4 * sizeof(float);  // eight waves come with T <= 2
+static_assert(kRedBytes8 <= kRedBytes4, "the eight-wave kernels must fit the LDS size the routing was told");
+
 size_t gemv_mfma_lds_bytes(uint32_t k, uint32_t batch) {
     const bool hilo = batch <= 2;
     const int ncols = hilo ? 2 * batch : batch;
     return static_cast<size_t>(k / kBlockWeights) * x_pitch_bytes(ncols, batch) + 64 +
-           2 * 4 * 4 * 8 * 4 * sizeof(float);
+           kRedBytes4;
 }
 
 void launch_gemv_mfma(const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint32_t x_stride,
@@ -437,18 +447,27 @@ void launch_gemv_mfma(const uint8_t* w, uint32_t n, uint32_t k, const float* x, 
     const uint32_t max_wgs = 256 * wg_per_cu;
     // K slices per workgroup: none when the rows alone give about 3 workgroups per CU (no LDS
     // meeting point, no barrier per row group); otherwise split K as far as its steps allow
+    // Waves per workgroup: eight where the staged activations leave room for one workgroup per CU
+    // only (one copy then serves twice the waves: 17408 x 5120 at 8 rows 27.2 -> 23.4 us, 5120 x 17408
+    // at 4 rows 24.9 -> 21.3), for matrices of at most 2048 rows, whose rows are too few to go round
+    // (2048 x 2048 at 8 rows 6.0 -> 4.9 us), and for one or two rows of a matrix below 2^25 weights
+    // (2048 x 6144 at 2 rows 7.3 -> 5.8 us).  Elsewhere the wider workgroup was measured slower
+    // (12288 x 2048 at 4 rows 7.5 -> 8.9 us): fewer, larger workgroups balance worse over the CUs.
+    const uint64_t weights = static_cast<uint64_t>(n) * k;
+    const uint32_t waves = wg_per_cu == 1 || n <= 2048 || (batch <= 2 && weights < (1ull << 25)) ? 8 : 4;
     uint32_t ks = 1;
-    while (ks < 4 && ks * 2 <= nsteps && (n + 16 / ks - 1) / (16 / ks) < 768) ks *= 2;
+    while (ks < 4 && ks * 2 <= nsteps && (n + 4 * waves / ks - 1) / (4 * waves / ks) < 768) ks *= 2;
     // row tiles per wave: enough blocks in flight per CU to cover HBM latency (about 40 KB), but
     // never so many that fewer than two workgroups per CU remain
     uint32_t t = wg_per_cu >= 4 ? 1 : wg_per_cu >= 2 ? 2 : 4;
-    while (t > 1 && (n + 4 * t * (4 / ks) - 1) / (4 * t * (4 / ks)) < 512) t >>= 1;
+    while (t > 1 && (n + 4 * t * (waves / ks) - 1) / (4 * t * (waves / ks)) < 512) t >>= 1;
+    if (waves == 8 && t > 2) t = 2;
     if (batch <= 2) {
-        launch_shape<1, true>(a, lds, t, ks, max_wgs, stream);
+        launch_shape<1, true>(a, lds, t, ks, waves, max_wgs, stream);
     } else if (batch <= 4) {
-        launch_shape<1, false>(a, lds, t, ks, max_wgs, stream);
+        launch_shape<1, false>(a, lds, t, ks, waves, max_wgs, stream);
     } else {
-        launch_shape<2, false>(a, lds, t, ks, max_wgs, stream);
+        launch_shape<2, false>(a, lds, t, ks, waves, max_wgs, stream);
     }
 }
 

@@ -7,6 +7,7 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 
@@ -19,6 +20,9 @@ struct lq4_ctx {
     float* lora_t;        // [kLoraTRows, kMaxLoraRank] f32: A.x of the call in flight
     uint8_t* moe_scratch; // grown on demand
     uint32_t* topk_ticket; // finished-workgroup count of the top-k kernel, zero between launches
+    uint32_t* lora_sync;   // epoch, producer count and slots of the batch-1 GEMV that computes A.x itself (same allocation)
+    bool lora_in_kernel;
+    uint32_t lora_spin_limit;  // polls a weight wave spends on those counters before it computes A.x alone
     size_t moe_scratch_bytes;
     lq4_path_counters counters;
 };
@@ -162,13 +166,25 @@ int lq4_ctx_create(int device_ordinal, lq4_ctx** out) {
         delete c;
         return fail(LQ4_E_HIP, "hipMalloc(lora scratch): %s", hipGetErrorString(e));
     }
-    e = hipMalloc(reinterpret_cast<void**>(&c->topk_ticket), 256);
-    if (e == hipSuccess) e = hipMemset(c->topk_ticket, 0, 256);
+    // 256 B of top-k ticket, 256 B for the LoRA epoch and producer count, 512 B of LoRA slots
+    e = hipMalloc(reinterpret_cast<void**>(&c->topk_ticket), 1024);
+    if (e == hipSuccess) e = hipMemset(c->topk_ticket, 0, 1024);
+    const uint32_t first_epoch = 1;  // the zeroed slots carry epoch 0
+    if (e == hipSuccess) e = hipMemcpy(c->topk_ticket + 64, &first_epoch, 4, hipMemcpyHostToDevice);
     if (e != hipSuccess) {
         (void)hipFree(c->topk_ticket);
         (void)hipFree(c->lora_t);
         delete c;
         return fail(LQ4_E_HIP, "hipMalloc(top-k ticket): %s", hipGetErrorString(e));
+    }
+    c->lora_sync = c->topk_ticket + 64;
+    // LQ4_LORA_SPIN_LIMIT: 0 makes every weight wave compute A.x itself (the path a wave takes when
+    // the producers are late), "off" restores the separate A.x launch
+    c->lora_spin_limit = 512;
+    c->lora_in_kernel = true;
+    if (const char* env = getenv("LQ4_LORA_SPIN_LIMIT")) {
+        if (!strcmp(env, "off")) c->lora_in_kernel = false;
+        else c->lora_spin_limit = static_cast<uint32_t>(strtoul(env, nullptr, 10));
     }
     *out = c;
     return LQ4_OK;
@@ -322,7 +338,13 @@ int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
     if (rc) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
     DeviceGuard g(ctx->device);
-    if (ep.rank) {
+    if (ep.rank && batch == 1 && ctx->lora_in_kernel && gemv_b1_lds_bytes(k) <= 128 * 1024) {
+        // one token: the GEMV launch computes A.x in its first `rank` workgroups
+        ep.a = lora->a;
+        ep.slots = reinterpret_cast<unsigned long long*>(ctx->lora_sync + 64);
+        ep.sync = ctx->lora_sync;
+        ep.spin_limit = ctx->lora_spin_limit;
+    } else if (ep.rank) {
         launch_lora_a(lora->a, lora->is_f16, lora->rank, k, x_dev, 0, k, batch, ctx->lora_t, s);
         ctx->counters.lora_a++;
     }

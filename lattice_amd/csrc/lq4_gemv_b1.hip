@@ -122,6 +122,60 @@ __device__ __forceinline__ float block_dot(const uint32_t (&q)[4], const uint32_
 // (residual add + shifted RMSNorm, or silu(gate) * up) and the result can be added into a
 // residual stream as it is stored.  Every workgroup stages the whole activation vector anyway,
 // so the norm costs one extra pass over K floats per workgroup and no launch.
+// Partial dot product of row `j` of A (f16 or f32, `k` long, k a multiple of 32) with x, for thread
+// `t` of `nt`: eight elements per step through 16-byte loads.
+__device__ __forceinline__ float lora_a_row_partial(const void* a, int a_is_f16, uint32_t j, uint32_t k,
+                                                    const float* __restrict__ x, uint32_t t, uint32_t nt) {
+    float p = 0.0f;
+    for (uint32_t kk = t * 8; kk < k; kk += nt * 8) {
+        const float4 x0 = *reinterpret_cast<const float4*>(x + kk), x1 = *reinterpret_cast<const float4*>(x + kk + 4);
+        float av[8];
+        if (a_is_f16) {
+            struct alignas(16) H8 { _Float16 v[8]; };
+            const H8 h = *reinterpret_cast<const H8*>(static_cast<const _Float16*>(a) + static_cast<size_t>(j) * k + kk);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) av[i] = static_cast<float>(h.v[i]);
+        } else {
+            const float4* ap = reinterpret_cast<const float4*>(static_cast<const float*>(a) + static_cast<size_t>(j) * k + kk);
+            const float4 a0 = ap[0], a1 = ap[1];
+            av[0] = a0.x; av[1] = a0.y; av[2] = a0.z; av[3] = a0.w;
+            av[4] = a1.x; av[5] = a1.y; av[6] = a1.z; av[7] = a1.w;
+        }
+        p = fmaf(av[0], x0.x, p); p = fmaf(av[1], x0.y, p); p = fmaf(av[2], x0.z, p); p = fmaf(av[3], x0.w, p);
+        p = fmaf(av[4], x1.x, p); p = fmaf(av[5], x1.y, p); p = fmaf(av[6], x1.z, p); p = fmaf(av[7], x1.w, p);
+    }
+    return p;
+}
+
+// Whole-wave call.  Returns t[lane] (0 beyond the rank) once every slot carries `epoch`; polls the
+// slots at most `spin_limit` times and otherwise computes t in this wave.  The slots are read with
+// agent-scope atomic loads (they do not hit in this XCD's caches), value and epoch in one word.
+__device__ __forceinline__ float lora_t_acquire(const LoraEpilogue& lora, uint32_t epoch, uint32_t k,
+                                                const float* __restrict__ x, int lane) {
+    const bool mine = static_cast<uint32_t>(lane) < lora.rank;
+    const unsigned long long none = static_cast<unsigned long long>(epoch) << 32;
+    if (lora.spin_limit) {
+        // First look through the caches: when the producers are done, which is the usual case, the
+        // line is fetched once per XCD instead of once per wave.  A line cached too early is only
+        // incomplete (its epochs say so) and the polls below go past the caches.
+        unsigned long long v = none;
+        if (mine) v = *static_cast<const volatile unsigned long long*>(&lora.slots[lane]);
+        if (__all(static_cast<uint32_t>(v >> 32) == epoch)) return __builtin_bit_cast(float, static_cast<uint32_t>(v));
+    }
+    for (uint32_t spin = 0; spin < lora.spin_limit; ++spin) {
+        unsigned long long v = none;
+        if (mine) v = __hip_atomic_load(&lora.slots[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (__all(static_cast<uint32_t>(v >> 32) == epoch)) return __builtin_bit_cast(float, static_cast<uint32_t>(v));
+        __builtin_amdgcn_s_sleep(4);
+    }
+    float t = 0.0f;
+    for (uint32_t j = 0; j < lora.rank; ++j) {
+        const float s = wave_sum(lora_a_row_partial(lora.a, lora.b_is_f16, j, k, x, lane, 64));
+        if (static_cast<uint32_t>(lane) == j) t = s;
+    }
+    return t;
+}
+
 struct NoFusion {};
 template <bool FUSED>
 struct FusionArg {
@@ -134,15 +188,54 @@ struct FusionArg<true> {
 
 // WAVES: waves per workgroup.  Every workgroup stages the whole activation vector, so on long rows
 // (K of 4096..8192) eight waves share one staging where four would each pay half of it again.
-template <int RW, int SG, int SEG, bool FUSED, int WAVES = kWaves>
+//
+// MODE: 0 plain, 1 fused prologue/epilogue (GemvFusion), 2 plain with the LoRA factor t = A.x
+// computed inside the launch: workgroups 0..rank-1 each reduce one row of A against x and publish
+// it (release), the weight workgroups behind them pick t up (acquire) when their first rows are
+// complete, long after it was published.  The wait is bounded: a wave that runs out of polls
+// computes t itself, so every wave finishes whatever the dispatch order was.
+constexpr int kPlainMode = 0, kFusedMode = 1, kLoraAMode = 2;
+
+template <int RW, int SG, int SEG, int MODE, int WAVES = kWaves>
 __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restrict__ w, uint32_t n,
                                                           uint32_t k, const float* __restrict__ x,
                                                           float* __restrict__ y, LoraEpilogue lora,
-                                                          typename FusionArg<FUSED>::type fz) {
+                                                          typename FusionArg<MODE == 1>::type fz) {
     extern __shared__ __attribute__((aligned(16))) uint32_t xs[];
+    constexpr bool FUSED = MODE == kFusedMode;
+    constexpr bool INA = MODE == kLoraAMode;
     constexpr int RPW = 64 / SEG;  // weight rows per wave-row
     const int tid = threadIdx.x;
     const int lane = tid & 63;
+    // workgroups that stream weights, and this one's index among them
+    uint32_t w_groups = gridDim.x, w_group = blockIdx.x;
+    if constexpr (INA) {
+        if (blockIdx.x < lora.rank) {  // ---- one row of A against x ----
+            const uint32_t epoch = __hip_atomic_load(&lora.sync[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const float p = lora_a_row_partial(lora.a, lora.b_is_f16, blockIdx.x, k, x, tid, WAVES * 64);
+            const float ws = wave_sum(p);
+            float* part = reinterpret_cast<float*>(xs);
+            if (lane == 0) part[tid >> 6] = ws;
+            __syncthreads();
+            if (tid == 0) {
+                float total = 0.0f;
+#pragma unroll
+                for (int i = 0; i < WAVES; ++i) total += part[i];
+                const unsigned long long word = (static_cast<unsigned long long>(epoch) << 32) | __builtin_bit_cast(uint32_t, total);
+                __hip_atomic_store(&lora.slots[blockIdx.x], word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                // this producer's read of the epoch has returned (it is part of `word`): count it; the
+                // last one advances the epoch.  rank atomics in all, off the weight workgroups' path.
+                const uint32_t before = __hip_atomic_fetch_add(&lora.sync[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (before + 1 == lora.rank) {
+                    __hip_atomic_store(&lora.sync[1], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(&lora.sync[0], epoch + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+            return;
+        }
+        w_groups -= lora.rank;
+        w_group -= lora.rank;
+    }
     const int sub = lane / SEG;   // which of the side-by-side rows
     const int seg_lane = lane % SEG;
     const uint32_t nb = k / kBlockWeights;
@@ -150,9 +243,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
     const uint32_t slabs = SEG == 64 ? (nb + 63) / 64 : 1;
     const uint32_t slab_groups = (slabs + SG - 1) / SG;
     const uint32_t n_wrows = (n + RPW - 1) / RPW;
-    const uint32_t n_waves = gridDim.x * WAVES;
+    const uint32_t n_waves = w_groups * WAVES;
     // the wave index is uniform across the wave: keep it (and everything derived) scalar
-    const uint32_t wid = __builtin_amdgcn_readfirstlane(blockIdx.x * WAVES + (tid >> 6));
+    const uint32_t wid = __builtin_amdgcn_readfirstlane(w_group * WAVES + (tid >> 6));
     // chunks whose first wave-row exists for this wave (later waves may have one chunk fewer)
     const uint32_t first = wid < n_wrows ? n_wrows - wid : 0;  // wave-rows from this wave's first one on
     const uint32_t chunks = (first + n_waves * RW - 1) / (n_waves * RW);
@@ -235,7 +328,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
 #pragma unroll
     for (int j = 0; j < RW; ++j) lora_b0[j] = 0.0f;
     if (lora.rank && static_cast<uint32_t>(seg_lane) < lora.rank) {
-        lora_t0 = lora.t[seg_lane];
+        if constexpr (!INA) lora_t0 = lora.t[seg_lane];
 #pragma unroll
         for (int j = 0; j < RW; ++j) {
             const uint32_t wrow = j * n_waves + wid;
@@ -249,6 +342,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
 
     Q4BlockRaw buf_a[RW][SG], buf_b[RW][SG];
     load_unit(buf_a, 0);
+    // Launch epoch, through the caches on purpose: the L2 holds nothing from before the launch, so
+    // the first wave of an XCD fetches the current word and the others hit it instead of queueing
+    // at one memory channel.  A copy that stays cached after the producers advanced the epoch is
+    // still this launch's epoch.
+    uint32_t lora_epoch = 0;
+    if constexpr (INA) lora_epoch = *static_cast<const volatile uint32_t*>(&lora.sync[0]);
     // residual values of the first chunk's rows, requested now so the final store does not wait
     float res_first[RW];
     if constexpr (FUSED) {
@@ -389,6 +488,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
     float acc[RW];
 #pragma unroll
     for (int j = 0; j < RW; ++j) acc[j] = 0.0f;
+    float t_reg = 0.0f;   // kLoraAMode: t[lane], fetched when the wave's first rows are complete
+    bool t_have = false;
 
     // Consumes unit u from `cur` while unit u+1 streams into `nxt`.
     // `prefetch` is a compile-time flag: a load behind a run-time condition would make the compiler
@@ -433,7 +534,28 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
                 const bool row_ok = wrow < n_wrows && row < n;
                 float v = acc[j];
                 acc[j] = 0.0f;
-                if (lora.rank && row_ok) {
+                if constexpr (INA) {
+                    // lane l of the wave holds t[l]; every lane takes part in the exchange
+                    if (!t_have) {
+                        t_reg = lora_t_acquire(lora, __builtin_amdgcn_readfirstlane(lora_epoch), k, x, lane);
+                        t_have = true;
+                    }
+                    for (uint32_t i0 = 0; i0 < lora.rank; i0 += SEG) {
+                        const uint32_t i = i0 + seg_lane;
+                        const float ti = __shfl(t_reg, static_cast<int>(i & 63u), 64);
+                        if (row_ok && i < lora.rank) {
+                            float bv;
+                            if (chunk == 0 && i0 == 0) {
+                                bv = lora_b0[j];  // requested at kernel start
+                            } else {
+                                const size_t bi = static_cast<size_t>(row) * lora.rank + i;
+                                bv = lora.b_is_f16 ? static_cast<float>(static_cast<const _Float16*>(lora.b)[bi])
+                                                   : static_cast<const float*>(lora.b)[bi];
+                            }
+                            v = fmaf(lora.scale * bv, ti, v);
+                        }
+                    }
+                } else if (lora.rank && row_ok) {
                     // the row's lanes share out scale * B[row, i] * t[i]; the sum below folds it in
                     uint32_t i = seg_lane;
                     if (chunk == 0 && i < lora.rank) {  // requested at kernel start
@@ -484,24 +606,35 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
 template <int RW, int SG, int SEG, int WAVES = kWaves>
 void launch_cfg(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, const LoraEpilogue& lora,
                 const GemvFusion* fusion, size_t lds, uint32_t waves, hipStream_t stream) {
-    static bool attr_set[2] = {false, false};  // raise the dynamic-LDS cap once per instantiation
+    static bool attr_set[3] = {false, false, false};  // raise the dynamic-LDS cap once per instantiation
     const dim3 grid((waves + WAVES - 1) / WAVES), block(WAVES * 64);
     if (fusion) {
         if (!attr_set[1]) {
-            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, true, WAVES>),
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, kFusedMode, WAVES>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, 159 * 1024);
             attr_set[1] = true;
         }
-        hipLaunchKernelGGL((gemv_q4_b1<RW, SG, SEG, true, WAVES>), grid, block, lds, stream, w, n, k, x, y, lora,
+        hipLaunchKernelGGL((gemv_q4_b1<RW, SG, SEG, kFusedMode, WAVES>), grid, block, lds, stream, w, n, k, x, y, lora,
                            *fusion);
         return;
     }
+    if (lora.rank && lora.a) {
+        if (!attr_set[2]) {
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, kLoraAMode, WAVES>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            attr_set[2] = true;
+        }
+        const dim3 grid_a(grid.x + lora.rank);  // the rank producer workgroups come first
+        hipLaunchKernelGGL((gemv_q4_b1<RW, SG, SEG, kLoraAMode, WAVES>), grid_a, block, lds, stream, w, n, k, x, y,
+                           lora, NoFusion{});
+        return;
+    }
     if (!attr_set[0]) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, false, WAVES>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, kPlainMode, WAVES>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         attr_set[0] = true;
     }
-    hipLaunchKernelGGL((gemv_q4_b1<RW, SG, SEG, false, WAVES>), grid, block, lds, stream, w, n, k, x, y, lora,
+    hipLaunchKernelGGL((gemv_q4_b1<RW, SG, SEG, kPlainMode, WAVES>), grid, block, lds, stream, w, n, k, x, y, lora,
                        NoFusion{});
 }
 

@@ -22,6 +22,20 @@ struct LoraEpilogue {
     uint32_t rank;     // 0 = no LoRA
     int b_is_f16;
     float scale;
+    // Batch-1 GEMV only.  With `a` set the launch carries `rank` extra workgroups that compute
+    // t = A.x themselves while the others stream weights, so no separate launch precedes it.
+    // sync[0] is the launch epoch: every workgroup reads it when it starts.  Producer j stores
+    // slots[j] = {bits of t[j], epoch} as one 64-bit word; a weight wave polls the slots until
+    // all carry its epoch (at most `spin_limit` polls, then it computes t on its own).  The
+    // producers count themselves in sync[1]; the last one zeroes that count and advances the
+    // epoch, which happens only after every producer has read it.  A weight workgroup that starts
+    // after that reads the next epoch, never sees it in the slots and takes the slow path; one
+    // that started before sees exactly this launch's values.  No counter is touched by the weight
+    // workgroups, and nothing has to be reset between launches.
+    const void* a;     // [rank, d_in] row-major, f32 or f16 (b_is_f16 applies to both factors)
+    unsigned long long* slots;  // [kMaxLoraRank]
+    uint32_t* sync;
+    uint32_t spin_limit;
 };
 
 // Elementwise steps fused into the batch-1 GEMV.

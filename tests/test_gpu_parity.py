@@ -576,3 +576,103 @@ def test_gemm_few_token_kernel_with_lora(be, b_f16):
     delta = host(y).astype(np.float64) - host(y_plain).astype(np.float64)
     want = 2.0 * (x.astype(np.float64) @ a32.astype(np.float64).T) @ b32.astype(np.float64).T
     assert rel_err(delta, want) <= REL_TOL
+
+
+# ------------------------------------------------- LoRA, one token: A.x inside the GEMV launch
+# lq4_ctx_create reads LQ4_LORA_SPIN_LIMIT: unset = the weight waves wait for the producer
+# workgroups, "0" = no wave waits (each computes A.x itself, the path taken when the producers are
+# late), "off" = the separate A.x launch.  All three must give the oracle's result.
+_LORA_B1_SHAPES = [
+    # n, k, rank, dtype           rows side by side / slabs / waves per workgroup exercised
+    (512, 2048, 16, np.float16),   # config 3 v projection
+    (2048, 2048, 16, np.float16),  # config 3 q projection
+    (2048, 2048, 64, np.float32),  # full rank limit, f32 factors
+    (300, 512, 3, np.float16),     # four rows per wave, ragged N, rank below the lane group
+    (1030, 1024, 40, np.float16),  # two rows per wave, rank above the lane group of 32
+    (777, 6144, 16, np.float32),   # eight-wave workgroups
+    (1024, 17408, 8, np.float16),  # nine slabs per row
+    (40000, 2048, 16, np.float16), # persistent waves walking several chunks
+    (5, 64, 1, np.float32),        # fewer rows than producers' neighbours: tiny grid
+]
+
+
+@pytest.mark.parametrize("mode", ["wait", "0", "off"])
+def test_lora_one_token_a_inside_the_launch(mode):
+    import torch
+    old = os.environ.get("LQ4_LORA_SPIN_LIMIT")
+    if mode == "wait":
+        os.environ.pop("LQ4_LORA_SPIN_LIMIT", None)
+    else:
+        os.environ["LQ4_LORA_SPIN_LIMIT"] = mode
+    try:
+        b2 = backend.HipQ4Backend(0)
+    finally:
+        if old is None:
+            os.environ.pop("LQ4_LORA_SPIN_LIMIT", None)
+        else:
+            os.environ["LQ4_LORA_SPIN_LIMIT"] = old
+    try:
+        for n, k, rank, dt in _LORA_B1_SHAPES:
+            print(f"lora one token mode={mode} n={n} k={k} rank={rank} {np.dtype(dt).name}", flush=True)
+            wq = synth.q4_weight(n, k, seed=1, tag="lora_b1")
+            a, b = synth.lora_pair(rank, k, n, seed=1, tag="lora_b1", std=0.05, dtype=dt)
+            qw = b2.upload_q4_blocks(wq)
+            b2.load_lora_adapter([backend.LoraLayerData(0, {"p": (a, b)})], scale=2.0)
+            before = b2.path_counters()["lora_a"]
+            try:
+                y = torch.empty((1, n), dtype=torch.float32, device="cuda")
+                # several calls in a row with different activations: the launch's counters must be
+                # back at zero each time and no call may see the previous call's A.x
+                for call in range(3):
+                    x = synth.activations(1, k, seed=10 + call)
+                    y.fill_(float("nan"))
+                    b2.gemv_batch(dev(x), qw, y, 1, n, k, layer_idx=0, module="p")
+                    ref = _lora_ref(x, wq, n, k, a, b, 2.0)
+                    base = oracle.gemm_f32(x, wq, n, k)
+                    e = rel_err(host(y), ref)
+                    e_delta = rel_err(host(y) - base, ref - base)
+                    print(f"  call {call}: rel err {e:.2e}, delta rel err {e_delta:.2e}", flush=True)
+                    assert e <= REL_TOL
+                    assert e_delta <= 2e-3  # y - base cancels the base product
+            finally:
+                launches = b2.path_counters()["lora_a"] - before
+                b2.unload_lora_adapter()
+            assert launches == (3 if mode == "off" else 0), "which path computed A.x"
+    finally:
+        b2.close()
+
+
+def test_lora_one_token_graph_replays(be):
+    # the launch that computes A.x itself keeps two counters in device memory; a captured launch
+    # must leave them ready for its own replay, with the program's eager work in between
+    import torch
+    n, k = synth.LORA_2B["q"]
+    wq = synth.q4_weight(n, k, seed=2, tag="lora_graph")
+    a, b = synth.lora_pair(16, k, n, seed=2, tag="lora_graph", std=0.05)
+    qw = be.upload_q4_blocks(wq)
+    be.load_lora_adapter([backend.LoraLayerData(0, {"p": (a, b)})], scale=2.0)
+    try:
+        xd = torch.zeros((1, k), dtype=torch.float32, device="cuda")
+        y = torch.empty((1, n), dtype=torch.float32, device="cuda")
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            be.gemv_batch(xd, qw, y, 1, n, k, layer_idx=0, module="p")  # warm-up outside the capture
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            be.gemv_batch(xd, qw, y, 1, n, k, layer_idx=0, module="p")
+        for replay in range(4):
+            print(f"lora graph replay {replay}", flush=True)
+            x = synth.activations(1, k, seed=20 + replay)
+            xd.copy_(dev(x))
+            graph.replay()
+            torch.cuda.synchronize()
+            got = host(y)
+            # eager call between the replays, same operands
+            y2 = torch.empty_like(y)
+            be.gemv_batch(xd, qw, y2, 1, n, k, layer_idx=0, module="p")
+            assert np.array_equal(got, host(y2))
+            assert rel_err(got, _lora_ref(x, wq, n, k, a, b, 2.0)) <= REL_TOL
+    finally:
+        be.unload_lora_adapter()

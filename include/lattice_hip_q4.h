@@ -113,7 +113,9 @@ int lq4_lora_apply(lq4_ctx* ctx, const lq4_lora* lora, float lora_scale, const v
  *   y[b, n] += lora_scale * sum_j B[n, j] * (sum_k A[j, k] * x[b, k]).
  * x_dev: f32 [batch, K]; y_dev: f32 [batch, N]; W starts at
  * payload_offset + w_extra_offset bytes into the weight buffer (qw_extra_offset of
- * dispatch_gemm_at, dispatch.rs:935-980). */
+ * dispatch_gemm_at, dispatch.rs:935-980).
+ * At batch 1 with a LoRA adapter the launch computes A . x itself and keeps a few words of
+ * hand-over state in the context: such calls must not overlap on two streams of one context. */
 int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
              const float* x_dev, uint32_t batch, float* y_dev, const lq4_lora* lora,
              float lora_scale, void* stream);

@@ -14,7 +14,8 @@ constexpr int kMaxLoraRank = 64;
 constexpr int kMaxGemvBatch = 16;
 
 // Optional LoRA epilogue operands.  t = A.x is produced by launch_lora_a into
-// ctx scratch before the main kernel runs; the main kernel adds
+// ctx scratch before the main kernel runs (or, for one token, inside the main kernel's
+// launch: see `a` below); the main kernel adds
 // scale * sum_j B[n,j] * t[row,j] before its single store of y.
 struct LoraEpilogue {
     const void* b;     // [d_out, rank] row-major, f32 or f16

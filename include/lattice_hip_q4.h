@@ -226,6 +226,62 @@ int lq4_gemv_fused(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, u
                    const float* x_dev, float* y_dev, const lq4_gemv_fusion* fusion, const lq4_lora* lora,
                    float lora_scale, void* stream);
 
+/* ---- a chain of dependent one-token GEMVs in one launch ---------------------------------------
+ * The reference encodes a whole token into one command buffer (forward_step,
+ * forward/metal_qwen35.rs:6943, committed once at :6447): o -> residual add + RMSNorm -> gate||up ->
+ * silu * up -> down -> residual add -> next layer's RMSNorm -> qkv follow each other without the
+ * host in between (encode_mlp_block, inner/layers/mod.rs; the elementwise dispatches at
+ * inner/dispatch.rs:916-930, 1171-1290).  lq4_gemv_chain is that unit here: up to
+ * LQ4_CHAIN_MAX_STEPS batch-1 GEMVs, each fed by an external vector or by the previous step's
+ * result, run as ONE persistent launch whose waves request the weights of later steps while
+ * earlier results are still on their way (falls back to one lq4_gemv_fused per step, same results to
+ * f32 rounding, when a step is too large for that: more than ~25 M weights, or K > 16384).
+ *
+ * Step j computes r_j = epilogue(W_j . prologue(x_j)):
+ *   x_j        x_dev (f32 [K]; [2K] = gate | up for LQ4_PRO_SILU_MUL), or base/delta/gamma under
+ *              LQ4_PRO_ADD_RMSNORM as in lq4_gemv_fusion, or, with x_dev == NULL and base == NULL,
+ *              the previous step's result r_(j-1) (then K must equal its length; the prologue is
+ *              LQ4_PRO_NONE, or LQ4_PRO_ADD_RMSNORM = shifted RMSNorm of r_(j-1) with gamma, eps);
+ *   epilogue   LQ4_EPI_NONE           r = W . x                         [N]
+ *              LQ4_EPI_ADD_RESIDUAL   r = residual + W . x, residual = r [N]  (dispatch_add_and_copy)
+ *              LQ4_EPI_SILU_MUL_PAIRS r[i] = silu(y[i]) * y[i + N/2]     [N/2] for W = [gate rows | up
+ *                                     rows], the fused buffer of metal_qwen35.rs:12137-12152
+ *                                     (dispatch_silu_mul_fused);
+ *   y_dev      receives r_j when not NULL (the last step needs y_dev or a residual).
+ * Vectors of different steps must be identical or disjoint.  The launch keeps hand-over state in the
+ * context: chains must not overlap on two streams of one context.  A hand-over that never
+ * completes (the grid not resident at once because another kernel holds the GPU) ends the launch
+ * after a bounded wait and lq4_sync returns LQ4_E_HIP; the chain's results are then invalid. */
+#define LQ4_CHAIN_MAX_STEPS 16
+#define LQ4_EPI_SILU_MUL_PAIRS 2
+typedef struct lq4_chain_step {
+    const lq4_weight* w;
+    uint64_t w_extra_offset;
+    uint32_t n, k;
+    const float* x_dev;
+    int prologue;
+    const float* base;
+    const float* delta;
+    const float* gamma;
+    float eps;
+    float* residual_out; /* external LQ4_PRO_ADD_RMSNORM only: receives base + delta */
+    int epilogue;
+    float* residual;
+    float* y_dev;
+} lq4_chain_step;
+int lq4_gemv_chain(lq4_ctx* ctx, const lq4_chain_step* steps, uint32_t n_steps, void* stream);
+/* Tuning/test hook, process-wide: 0 = one persistent launch where the chain is eligible (default),
+ * 1 = always step by step.  No counterpart in the reference. */
+int lq4_set_chain_mode(int mode);
+
+/* Grows the context's scratch (partial tiles of K-sliced GEMMs, packed few-token operands, MoE
+ * intermediates, lm_head logits) to at least `bytes` ahead of time.  The library grows it on demand
+ * otherwise, which allocates: a call that would have to grow it while its stream is being captured
+ * into a HIP graph returns LQ4_E_UNSUPPORTED instead.  Outgrown buffers stay allocated until
+ * lq4_ctx_destroy, so launches already queued or captured keep valid addresses.  No counterpart in
+ * the reference. */
+int lq4_ctx_reserve_scratch(lq4_ctx* ctx, size_t bytes);
+
 /* ---- Q8_0 sibling format -----------------------------------------------------------
  * 34-byte blocks [u16 f16 scale d][32 x i8], w = q * d, rows of K/32 blocks, 2-byte aligned
  * (forward/metal_qwen35.rs:2310-2346).  Weight handles are format-agnostic byte buffers: upload
@@ -278,6 +334,10 @@ int lq4_probe_copy(lq4_ctx* ctx, const void* src_dev, void* dst_dev, size_t nbyt
  * PathProofCounters, metal_qwen35.rs:2144-2190): proves which path served a call. */
 typedef struct lq4_path_counters {
     uint64_t gemv, gemm, lora_a, moe_route, moe_gate_up, moe_down, dequant, topk, gemv_fused, elementwise;
+    uint64_t gemv_chain;       /* lq4_gemv_chain calls served by the single persistent launch */
+    uint64_t lora_t_fallback;  /* waves of one-token LoRA launches that computed A.x themselves because
+                                  the producers' hand-over did not arrive in time (read from the device:
+                                  this call waits for the GPU) */
 } lq4_path_counters;
 int lq4_get_path_counters(const lq4_ctx* ctx, lq4_path_counters* out);
 

@@ -51,6 +51,7 @@ EXPORTS = [
     "lq4_probe_copy",
     "lq4_set_gemm_kernel",
     "lq4_residual_add_rmsnorm", "lq4_silu_mul", "lq4_add_and_copy", "lq4_gemv_fused",
+    "lq4_gemv_chain", "lq4_set_chain_mode", "lq4_ctx_reserve_scratch",
     "lq4_gemv_q8", "lq4_gemm_q8", "lq4_gemv_q3", "lq4_gemm_q3",
     "lq4_get_path_counters", "lq4_malloc", "lq4_free", "lq4_memcpy_h2d", "lq4_memcpy_d2h",
 ]
@@ -71,11 +72,13 @@ class Q4Error(RuntimeError):
 
 class PathCounters(C.Structure):
     _fields_ = [(n, C.c_uint64) for n in ("gemv", "gemm", "lora_a", "moe_route", "moe_gate_up",
-                                         "moe_down", "dequant", "topk", "gemv_fused", "elementwise")]
+                                         "moe_down", "dequant", "topk", "gemv_fused", "elementwise",
+                                         "gemv_chain", "lora_t_fallback")]
 
 
 LQ4_PRO_NONE, LQ4_PRO_ADD_RMSNORM, LQ4_PRO_SILU_MUL = 0, 1, 2
-LQ4_EPI_NONE, LQ4_EPI_ADD_RESIDUAL = 0, 1
+LQ4_EPI_NONE, LQ4_EPI_ADD_RESIDUAL, LQ4_EPI_SILU_MUL_PAIRS = 0, 1, 2
+CHAIN_MAX_STEPS = 16
 
 
 class GemvFusion(C.Structure):
@@ -83,6 +86,14 @@ class GemvFusion(C.Structure):
     _fields_ = [("prologue", C.c_int), ("base", C.c_void_p), ("delta", C.c_void_p), ("gamma", C.c_void_p),
                 ("eps", C.c_float), ("residual_out", C.c_void_p), ("epilogue", C.c_int),
                 ("residual", C.c_void_p), ("copy_dst", C.c_void_p)]
+
+
+class ChainStep(C.Structure):
+    """``lq4_chain_step``: one batch-1 GEMV of a chain that runs as a single launch."""
+    _fields_ = [("w", C.c_void_p), ("w_extra_offset", C.c_uint64), ("n", C.c_uint32), ("k", C.c_uint32),
+                ("x_dev", C.c_void_p), ("prologue", C.c_int), ("base", C.c_void_p), ("delta", C.c_void_p),
+                ("gamma", C.c_void_p), ("eps", C.c_float), ("residual_out", C.c_void_p), ("epilogue", C.c_int),
+                ("residual", C.c_void_p), ("y_dev", C.c_void_p)]
 
 
 _lib = None
@@ -132,6 +143,9 @@ def load_library() -> C.CDLL:
         "lq4_gemm_q3": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, C.c_int, C.c_uint32, vp, vp]),
         "lq4_gemv_fused": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, vp, C.POINTER(GemvFusion), vp,
                                      C.c_float, vp]),
+        "lq4_gemv_chain": (C.c_int, [vp, C.POINTER(ChainStep), C.c_uint32, vp]),
+        "lq4_set_chain_mode": (C.c_int, [C.c_int]),
+        "lq4_ctx_reserve_scratch": (C.c_int, [vp, C.c_size_t]),
         "lq4_get_path_counters": (C.c_int, [vp, C.POINTER(PathCounters)]),
         "lq4_malloc": (C.c_int, [vp, C.c_size_t, C.POINTER(vp)]),
         "lq4_free": (C.c_int, [vp, vp]),
@@ -413,6 +427,44 @@ class HipQ4Backend:
         _check(self.lib.lq4_gemv_fused(self.ctx, qw.handle, qw_extra_offset, n, k, self._ptr(x), self._ptr(y),
                                        C.byref(f), lora, self._lora_scale, self._stream()))
 
+    def chain_step(self, qw: Q4WeightBuf, n: int, k: int, *, x=None, norm=None, silu_mul=False,
+                   add_residual=None, silu_mul_pairs=False, y=None, qw_extra_offset: int = 0) -> ChainStep:
+        """One step of :meth:`dispatch_chain`.  ``x=None`` (and no ``base`` in ``norm``) feeds the step
+        with the previous step's result.  ``norm=(base, delta, gamma, eps, residual_out)`` as in
+        :meth:`dispatch_matmul_fused`, or ``norm=(None, None, gamma, eps, None)`` for the shifted RMSNorm
+        of the previous result; ``silu_mul=True``: ``x`` holds gate | up; ``add_residual=residual``:
+        the result is ``residual + W.x``, written back; ``silu_mul_pairs=True``: W is gate rows then up
+        rows and the result is ``silu(gate) * up`` (n/2 values); ``y`` receives the result."""
+        self._assert_k(k, "dispatch_matmul_q4")
+        assert not (norm is not None and silu_mul), "one prologue at a time"
+        assert not (add_residual is not None and silu_mul_pairs), "one epilogue at a time"
+        st = ChainStep()
+        st.w, st.w_extra_offset, st.n, st.k = qw.handle, qw_extra_offset, n, k
+        st.x_dev = self._ptr(x)
+        st.prologue = LQ4_PRO_ADD_RMSNORM if norm is not None else LQ4_PRO_SILU_MUL if silu_mul else LQ4_PRO_NONE
+        keep = [qw, x, y, add_residual]
+        if norm is not None:
+            base, delta, gamma, eps, residual_out = norm
+            st.base, st.delta, st.gamma = self._ptr(base), self._ptr(delta), gamma.data_ptr()
+            st.eps, st.residual_out = eps, self._ptr(residual_out)
+            keep += [base, delta, gamma, residual_out]
+        st.epilogue = (LQ4_EPI_ADD_RESIDUAL if add_residual is not None else
+                       LQ4_EPI_SILU_MUL_PAIRS if silu_mul_pairs else LQ4_EPI_NONE)
+        st.residual = self._ptr(add_residual)
+        st.y_dev = self._ptr(y)
+        st._keep = keep
+        return st
+
+    def dispatch_chain(self, steps: Sequence[ChainStep]):
+        """The dispatches of one token between two points where the host must look at the result
+        (``forward_step`` encodes them into one command buffer, metal_qwen35.rs:6943), as one launch."""
+        arr = (ChainStep * len(steps))(*steps)
+        _check(self.lib.lq4_gemv_chain(self.ctx, arr, len(steps), self._stream()))
+
+    def set_chain_mode(self, mode: int):
+        """0 = one persistent launch where the chain is eligible, 1 = always step by step."""
+        _check(self.lib.lq4_set_chain_mode(int(mode)))
+
     def dispatch_gemm(self, x, x_offset: int, qw: Q4WeightBuf, y, y_offset: int, m: int, n: int,
                       k: int, *, layer_idx=None, module=None):
         """``dispatch_gemm`` (dispatch.rs:507-525 -> dispatch_gemm_q4 :170-229)."""
@@ -462,16 +514,21 @@ class HipQ4Backend:
                                  out_i.data_ptr(), self._stream()))
         return out_l, out_i
 
-    def lm_head_topk(self, x, qw: Q4WeightBuf, vocab: int, k: int, top_k: int, qw_extra_offset: int = 0):
+    def lm_head_topk(self, x, qw: Q4WeightBuf, vocab: int, k: int, top_k: int, qw_extra_offset: int = 0,
+                     out=None, static_scratch: bool = False):
         """lm_head projection fused with top-k selection (dispatch_lm_head_block_stage1_enc +
         dispatch_block_topk_merge_enc, inner/dispatch.rs:1317-1421): the full logits vector is
-        never returned."""
+        never returned.  ``static_scratch=True`` takes the entry point that allocates nothing
+        (pass ``out=(logits, ids)`` tensors as well and the call touches no allocator at all)."""
         import torch
         self._assert_k(k, "lm_head_topk")
-        out_l = torch.empty(top_k, dtype=torch.float32, device=self.torch_device)
-        out_i = torch.empty(top_k, dtype=torch.int32, device=self.torch_device)
-        _check(self.lib.lq4_lm_head_topk(self.ctx, qw.handle, qw_extra_offset, vocab, k, x.data_ptr(), top_k,
-                                         out_l.data_ptr(), out_i.data_ptr(), self._stream()))
+        if out is None:
+            out = (torch.empty(top_k, dtype=torch.float32, device=self.torch_device),
+                   torch.empty(top_k, dtype=torch.int32, device=self.torch_device))
+        out_l, out_i = out
+        fn = self.lib.lq4_lm_head_topk_static if static_scratch else self.lib.lq4_lm_head_topk
+        _check(fn(self.ctx, qw.handle, qw_extra_offset, vocab, k, x.data_ptr(), top_k,
+                  out_l.data_ptr(), out_i.data_ptr(), self._stream()))
         return out_l, out_i
 
     # -------------------------------------------------------------------- LoRA

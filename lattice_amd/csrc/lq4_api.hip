@@ -10,6 +10,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <new>
+#include <vector>
 
 #include "lq4_internal.hpp"
 
@@ -24,6 +25,17 @@ struct lq4_ctx {
     bool lora_in_kernel;
     uint32_t lora_spin_limit;  // polls a weight wave spends on those counters before it computes A.x alone
     size_t moe_scratch_bytes;
+    // Buffers the growable scratch outgrew: launches already queued (or captured into a graph) may
+    // still use them, so they are only released with the context.
+    std::vector<void*> retired;
+    // lq4_gemv_chain: launch epoch (word 0) and failure word (word 64) in one allocation, the tagged
+    // result vectors of the steps, the CU count that sizes the resident grid
+    uint32_t* chain_sync;
+    uint8_t* chain_scratch;
+    size_t chain_scratch_bytes;
+    uint32_t cu_count;
+    uint32_t chain_spin_limit;
+    bool chain_unchecked;  // a chain launch was queued since the failure word was last read
     lq4_path_counters counters;
 };
 
@@ -178,6 +190,23 @@ int lq4_ctx_create(int device_ordinal, lq4_ctx** out) {
         return fail(LQ4_E_HIP, "hipMalloc(top-k ticket): %s", hipGetErrorString(e));
     }
     c->lora_sync = c->topk_ticket + 64;
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, device_ordinal);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&c->chain_sync), 512);
+    if (e == hipSuccess) e = hipMemset(c->chain_sync, 0, 512);
+    if (e == hipSuccess) e = hipMemcpy(c->chain_sync, &first_epoch, 4, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        if (c->chain_sync) (void)hipFree(c->chain_sync);
+        (void)hipFree(c->topk_ticket);
+        (void)hipFree(c->lora_t);
+        delete c;
+        return fail(LQ4_E_HIP, "context set-up (chain words): %s", hipGetErrorString(e));
+    }
+    c->cu_count = static_cast<uint32_t>(prop.multiProcessorCount);
+    // LQ4_CHAIN_SPIN_LIMIT: polls a wave of the chain kernel spends on one hand-over (0: none, the
+    // launch reports failure at its first dependent step; every kernel still exits)
+    c->chain_spin_limit = 1u << 20;
+    if (const char* env = getenv("LQ4_CHAIN_SPIN_LIMIT")) c->chain_spin_limit = static_cast<uint32_t>(strtoul(env, nullptr, 10));
     // LQ4_LORA_SPIN_LIMIT: 0 makes every weight wave compute A.x itself (the path a wave takes when
     // the producers are late), "off" restores the separate A.x launch
     c->lora_spin_limit = 512;
@@ -196,6 +225,9 @@ int lq4_ctx_destroy(lq4_ctx* ctx) {
     (void)hipFree(ctx->lora_t);
     (void)hipFree(ctx->topk_ticket);
     if (ctx->moe_scratch) (void)hipFree(ctx->moe_scratch);
+    if (ctx->chain_scratch) (void)hipFree(ctx->chain_scratch);
+    (void)hipFree(ctx->chain_sync);
+    for (void* p : ctx->retired) (void)hipFree(p);
     delete ctx;
     return LQ4_OK;
 }
@@ -203,6 +235,19 @@ int lq4_ctx_destroy(lq4_ctx* ctx) {
 int lq4_sync(lq4_ctx* ctx, void* stream) {
     if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
     LQ4_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    if (ctx->chain_unchecked) {
+        DeviceGuard g(ctx->device);
+        uint32_t failed_step = 0;
+        LQ4_HIP(hipMemcpy(&failed_step, ctx->chain_sync + 64, sizeof failed_step, hipMemcpyDeviceToHost));
+        ctx->chain_unchecked = false;
+        if (failed_step) {
+            LQ4_HIP(hipMemset(ctx->chain_sync + 64, 0, sizeof failed_step));
+            return fail(LQ4_E_HIP,
+                        "lq4_gemv_chain: the activations of step %u never arrived (workgroups not resident together, "
+                        "or the wait was cut short); the chain's results are invalid, run it per step",
+                        failed_step);
+        }
+    }
     return LQ4_OK;
 }
 
@@ -319,7 +364,7 @@ int lq4_lora_free(lq4_lora* l) {
     return LQ4_OK;
 }
 
-static int ensure_scratch(lq4_ctx* ctx, size_t bytes);
+static int ensure_scratch(lq4_ctx* ctx, size_t bytes, hipStream_t stream);
 
 int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
              const float* x_dev, uint32_t batch, float* y_dev, const lq4_lora* lora, float lora_scale,
@@ -357,7 +402,7 @@ int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
     // workgroups then win, 2048 x 6144 at 5..8 rows 9.5 -> 7.2..8.2 us)
     const bool narrow = n <= 2048 && gemv_mfma_lds_bytes(k, batch < 8 ? batch : 8) <= 150 * 1024;
     if (batch >= 9 || (batch >= 5 && n < 8192 && !narrow && weights >= 6000000)) {
-        rc = ensure_scratch(ctx, gemm_skinny_scratch_bytes(k, batch));
+        rc = ensure_scratch(ctx, gemm_skinny_scratch_bytes(k, batch), static_cast<hipStream_t>(stream));
         if (rc) return rc;
         launch_gemm_skinny(wp, n, k, x_dev, 0, batch, y_dev, ep, ctx->moe_scratch, s);
         ctx->counters.gemm++;
@@ -387,19 +432,42 @@ int lq4_lora_apply(lq4_ctx* ctx, const lq4_lora* lora, float lora_scale, const v
     return LQ4_OK;
 }
 
-// Grows the context's scratch buffer (MoE intermediates, GEMM partial sums) to `bytes`.
-// Growing is a synchronising allocation; steady-state calls reuse the buffer.
-static int ensure_scratch(lq4_ctx* ctx, size_t bytes) {
-    if (bytes <= ctx->moe_scratch_bytes) return LQ4_OK;
-    if (ctx->moe_scratch) {
-        LQ4_HIP(hipDeviceSynchronize());
-        (void)hipFree(ctx->moe_scratch);
-        ctx->moe_scratch = nullptr;
-        ctx->moe_scratch_bytes = 0;
+// Grows one of the context's scratch buffers to `bytes`.  The outgrown buffer is kept until the
+// context is destroyed: launches already queued, and launches captured into a graph, carry its
+// address.  Nothing may be allocated while the stream is capturing: the call then fails and names
+// lq4_ctx_reserve_scratch.  Steady-state calls reuse the buffer.
+static int grow_scratch(lq4_ctx* ctx, uint8_t** buf, size_t* have, size_t bytes, hipStream_t stream, bool zero) {
+    if (bytes <= *have) return LQ4_OK;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) != hipSuccess) (void)hipGetLastError();
+    if (cap != hipStreamCaptureStatusNone)
+        return fail(LQ4_E_UNSUPPORTED,
+                    "library scratch must grow from %zu to %zu bytes but the stream is capturing; run the shape once, or "
+                    "call lq4_ctx_reserve_scratch, before the capture", *have, bytes);
+    bytes = (bytes + (1u << 20) - 1) >> 20 << 20;
+    uint8_t* fresh = nullptr;
+    LQ4_HIP(hipMalloc(reinterpret_cast<void**>(&fresh), bytes));
+    if (zero) {
+        const hipError_t e = hipMemset(fresh, 0, bytes);
+        if (e != hipSuccess) {
+            (void)hipFree(fresh);
+            return fail(LQ4_E_HIP, "hipMemset(scratch): %s", hipGetErrorString(e));
+        }
     }
-    LQ4_HIP(hipMalloc(reinterpret_cast<void**>(&ctx->moe_scratch), bytes));
-    ctx->moe_scratch_bytes = bytes;
+    if (*buf) ctx->retired.push_back(*buf);
+    *buf = fresh;
+    *have = bytes;
     return LQ4_OK;
+}
+
+static int ensure_scratch(lq4_ctx* ctx, size_t bytes, hipStream_t stream) {
+    return grow_scratch(ctx, &ctx->moe_scratch, &ctx->moe_scratch_bytes, bytes, stream, false);
+}
+
+int lq4_ctx_reserve_scratch(lq4_ctx* ctx, size_t bytes) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    DeviceGuard g(ctx->device);
+    return ensure_scratch(ctx, bytes, nullptr);
 }
 
 int lq4_gemm(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
@@ -428,7 +496,7 @@ int lq4_gemm(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
     // shapes with too few tiles run as K slices into scratch partials, summed by a second kernel
     const size_t scratch_bytes = gemm_scratch_floats(n, k, m, x_dtype == LQ4_F16) * sizeof(float);
     if (scratch_bytes) {
-        rc = ensure_scratch(ctx, scratch_bytes);
+        rc = ensure_scratch(ctx, scratch_bytes, static_cast<hipStream_t>(stream));
         if (rc) return rc;
     }
     launch_gemm(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, ep,
@@ -485,7 +553,7 @@ int lq4_moe_grouped_gemv(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_weig
     const size_t off_o = off_h + up256(sizeof(float) * pairs * inter);
     const size_t total = off_o + up256(sizeof(float) * pairs * hidden);
     {
-        const int src = ensure_scratch(ctx, total);
+        const int src = ensure_scratch(ctx, total, static_cast<hipStream_t>(stream));
         if (src) return src;
     }
     MoeScratch s;
@@ -534,7 +602,7 @@ int lq4_topk(lq4_ctx* ctx, const float* logits_dev, uint32_t n, uint32_t top_k, 
     if (top_k > LQ4_MAX_TOP_K) return fail(LQ4_E_INVALID, "top_k %u above %d", top_k, LQ4_MAX_TOP_K);
     if (n == 0) return fail(LQ4_E_INVALID, "no logits to select from");
     DeviceGuard g(ctx->device);
-    const int rc = ensure_scratch(ctx, topk_scratch_bytes(n, top_k));
+    const int rc = ensure_scratch(ctx, topk_scratch_bytes(n, top_k), static_cast<hipStream_t>(stream));
     if (rc) return rc;
     launch_topk(logits_dev, n, top_k, ctx->moe_scratch, ctx->topk_ticket, out_logits_dev, out_ids_dev,
                 static_cast<hipStream_t>(stream));
@@ -558,7 +626,7 @@ int lq4_lm_head_topk(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset,
     DeviceGuard g(ctx->device);
     // scratch: [vocab logits | candidate buffers]
     const size_t logits_bytes = (static_cast<size_t>(vocab) * sizeof(float) + 255) / 256 * 256;
-    rc = ensure_scratch(ctx, logits_bytes + topk_scratch_bytes(vocab, top_k));
+    rc = ensure_scratch(ctx, logits_bytes + topk_scratch_bytes(vocab, top_k), static_cast<hipStream_t>(stream));
     if (rc) return rc;
     float* logits = reinterpret_cast<float*>(ctx->moe_scratch);
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -687,7 +755,7 @@ int lq4_gemv_fused(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, u
 
     // The same steps one by one: activations and (if the caller wants no y) the product in scratch.
     const size_t x_off = 0, y_off = (kbytes + 255) / 256 * 256;
-    rc = ensure_scratch(ctx, y_off + static_cast<size_t>(n) * sizeof(float));
+    rc = ensure_scratch(ctx, y_off + static_cast<size_t>(n) * sizeof(float), static_cast<hipStream_t>(stream));
     if (rc) return rc;
     const float* act = x_dev;
     float* xs = reinterpret_cast<float*>(ctx->moe_scratch + x_off);
@@ -715,6 +783,243 @@ int lq4_gemv_fused(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, u
     return LQ4_OK;
 }
 
+// ---- a chain of dependent batch-1 GEMVs ----------------------------------------------------------
+namespace {
+
+int g_chain_mode = 0;  // 0 = one persistent launch where the chain is eligible, 1 = always step by step
+
+inline size_t up256(size_t v) { return (v + 255) / 256 * 256; }
+
+inline uint32_t chain_result_len(const lq4_chain_step& st) {
+    return st.epilogue == LQ4_EPI_SILU_MUL_PAIRS ? st.n / 2 : st.n;
+}
+
+inline bool chain_reads_previous(const lq4_chain_step& st) {
+    return !st.x_dev && !(st.prologue == LQ4_PRO_ADD_RMSNORM && st.base);
+}
+
+// The plain pointer a step's result is stored at for the caller (null: nowhere).
+inline const float* chain_result_ptr(const lq4_chain_step& st) {
+    return st.y_dev ? st.y_dev : st.epilogue == LQ4_EPI_ADD_RESIDUAL ? st.residual : nullptr;
+}
+
+int chain_validate(const lq4_chain_step* steps, uint32_t n_steps) {
+    auto misaligned = [](const void* p, uintptr_t a) { return reinterpret_cast<uintptr_t>(p) % a != 0; };
+    for (uint32_t j = 0; j < n_steps; ++j) {
+        const lq4_chain_step& st = steps[j];
+        if (st.n == 0) return fail(LQ4_E_INVALID, "chain step %u has no rows", j);
+        const uint8_t* wp;
+        const int rc = resolve_weight(st.w, st.w_extra_offset, st.n, st.k, &wp);
+        if (rc) return rc;
+        const bool prev = chain_reads_previous(st);
+        if (prev) {
+            if (j == 0) return fail(LQ4_E_INVALID, "chain step 0 needs external activations");
+            if (st.prologue != LQ4_PRO_NONE && st.prologue != LQ4_PRO_ADD_RMSNORM)
+                return fail(LQ4_E_INVALID, "chain step %u: a step fed by the previous result takes LQ4_PRO_NONE or LQ4_PRO_ADD_RMSNORM", j);
+            if (chain_result_len(steps[j - 1]) != st.k)
+                return fail(LQ4_E_INVALID, "chain step %u: K = %u but the previous step yields %u values", j, st.k,
+                            chain_result_len(steps[j - 1]));
+            if (st.delta || st.residual_out)
+                return fail(LQ4_E_INVALID, "chain step %u: delta / residual_out belong to an external LQ4_PRO_ADD_RMSNORM", j);
+        } else {
+            switch (st.prologue) {
+                case LQ4_PRO_NONE:
+                case LQ4_PRO_SILU_MUL:
+                    if (!st.x_dev || misaligned(st.x_dev, 16)) return fail(LQ4_E_INVALID, "chain step %u: x must be non-null and 16-byte aligned", j);
+                    break;
+                case LQ4_PRO_ADD_RMSNORM:
+                    if (misaligned(st.base, 16) || (st.delta && misaligned(st.delta, 16)) ||
+                        (st.residual_out && misaligned(st.residual_out, 16)))
+                        return fail(LQ4_E_INVALID, "chain step %u: base, delta and residual_out must be 16-byte aligned", j);
+                    if (st.residual_out && (ranges_overlap(st.residual_out, st.base, static_cast<size_t>(st.k) * 4) ||
+                                            (st.delta && ranges_overlap(st.residual_out, st.delta, static_cast<size_t>(st.k) * 4))))
+                        return fail(LQ4_E_INVALID, "chain step %u: residual_out must not overlap base or delta", j);
+                    break;
+                default:
+                    return fail(LQ4_E_INVALID, "chain step %u: unknown prologue %d", j, st.prologue);
+            }
+        }
+        if (st.prologue == LQ4_PRO_ADD_RMSNORM && (!st.gamma || misaligned(st.gamma, 16)))
+            return fail(LQ4_E_INVALID, "chain step %u: gamma must be non-null and 16-byte aligned", j);
+        switch (st.epilogue) {
+            case LQ4_EPI_NONE:
+                break;
+            case LQ4_EPI_ADD_RESIDUAL:
+                if (!st.residual || misaligned(st.residual, 16)) return fail(LQ4_E_INVALID, "chain step %u: residual must be non-null and 16-byte aligned", j);
+                break;
+            case LQ4_EPI_SILU_MUL_PAIRS:
+                if (st.n % 2) return fail(LQ4_E_INVALID, "chain step %u: silu(gate) * up over row pairs needs an even N, got %u", j, st.n);
+                break;
+            default:
+                return fail(LQ4_E_INVALID, "chain step %u: unknown epilogue %d", j, st.epilogue);
+        }
+        if (st.y_dev && misaligned(st.y_dev, 16)) return fail(LQ4_E_INVALID, "chain step %u: y must be 16-byte aligned", j);
+        if (j + 1 == n_steps && !chain_result_ptr(st))
+            return fail(LQ4_E_INVALID, "the last chain step has nowhere to put its result (y_dev is null)");
+    }
+    return LQ4_OK;
+}
+
+// Byte offset of every step's result vector in the chain scratch (8 bytes per value) and the total.
+size_t chain_scratch_layout(const lq4_chain_step* steps, uint32_t n_steps, size_t (&off)[kMaxChainSteps]) {
+    size_t total = 0;
+    for (uint32_t j = 0; j < n_steps; ++j) {
+        off[j] = total;
+        total += up256(static_cast<size_t>(steps[j].n) * 8);  // n, not n/2: the per-step path keeps W . x here too
+    }
+    return total;
+}
+
+// Fills the device descriptors of the persistent launch; false = the chain is not eligible for it
+// (a step too large for the register slots or for LDS, or a vector that an earlier step of the same
+// chain writes and that cannot be taken from that step's tagged result).
+bool chain_plan(lq4_ctx* ctx, const lq4_chain_step* steps, uint32_t n_steps, const size_t (&off)[kMaxChainSteps],
+                ChainArgs* args, uint32_t* k_max) {
+    *k_max = 0;
+    std::memset(args, 0, sizeof *args);
+    args->n_steps = n_steps;
+    args->spin_limit = ctx->chain_spin_limit;
+    args->epoch = ctx->chain_sync;
+    args->fail = ctx->chain_sync + 64;
+    auto tagged = [&](uint32_t i) { return reinterpret_cast<unsigned long long*>(ctx->chain_scratch + off[i]); };
+    for (uint32_t j = 0; j < n_steps; ++j) {
+        const lq4_chain_step& st = steps[j];
+        ChainStep& d = args->s[j];
+        if (st.k > gemv_chain_max_k()) return false;
+        *k_max = st.k > *k_max ? st.k : *k_max;
+        (void)resolve_weight(st.w, st.w_extra_offset, st.n, st.k, &d.w);
+        d.n = st.n;
+        d.k = st.k;
+        d.prologue = st.prologue;
+        d.epilogue = st.epilogue;
+        d.gamma = st.gamma;
+        d.eps = st.eps;
+        d.y = st.y_dev;
+        // Which earlier step, if any, wrote vector p for the caller?  Its memory is not coherent
+        // inside the launch; only that step's tagged result is.
+        auto writer_of = [&](const void* p) -> int {
+            if (!p) return -1;
+            for (int i = static_cast<int>(j) - 1; i >= 0; --i)
+                if (steps[i].y_dev == p || (steps[i].epilogue == LQ4_EPI_ADD_RESIDUAL && steps[i].residual == p) ||
+                    steps[i].residual_out == p)
+                    return i;
+            return -1;
+        };
+        if (chain_reads_previous(st)) {
+            d.x_tagged = tagged(j - 1);
+            args->s[j - 1].out_tagged = tagged(j - 1);
+        } else {
+            if (writer_of(st.x_dev) >= 0 || writer_of(st.base) >= 0 || writer_of(st.delta) >= 0) return false;
+            d.x = st.x_dev;
+            d.base = st.base;
+            d.delta = st.delta;
+            d.residual_out = st.residual_out;
+        }
+        if (st.epilogue == LQ4_EPI_ADD_RESIDUAL) {
+            d.res_out = st.residual;
+            const int i = writer_of(st.residual);
+            if (i < 0) {
+                d.res_plain = st.residual;
+            } else {
+                // readable from step i's tagged result once a later hand-over has completed, i.e. from
+                // two steps on; and only if that result is what was stored there
+                if (i + 1 >= static_cast<int>(j) || chain_result_ptr(steps[i]) != st.residual) return false;
+                d.res_tagged = tagged(static_cast<uint32_t>(i));
+                args->s[i].out_tagged = tagged(static_cast<uint32_t>(i));
+            }
+        }
+        if (!gemv_chain_plan_step(d, ctx->cu_count)) return false;
+    }
+    return gemv_chain_lds_bytes(*k_max) <= 160 * 1024;
+}
+
+}  // namespace
+
+#ifdef LQ4_CHAIN_TRACE
+static unsigned long long* g_chain_trace = nullptr;
+int lq4_debug_chain_trace(void* buf) { g_chain_trace = static_cast<unsigned long long*>(buf); return 0; }
+#endif
+
+int lq4_set_chain_mode(int mode) {
+    if (mode < 0 || mode > 1) return fail(LQ4_E_INVALID, "chain mode must be 0 (one launch where eligible) or 1 (step by step)");
+    g_chain_mode = mode;
+    return LQ4_OK;
+}
+
+int lq4_gemv_chain(lq4_ctx* ctx, const lq4_chain_step* steps, uint32_t n_steps, void* stream) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    if (n_steps == 0) return LQ4_OK;
+    if (!steps) return fail(LQ4_E_INVALID, "steps is null");
+    if (n_steps > LQ4_CHAIN_MAX_STEPS) return fail(LQ4_E_INVALID, "a chain holds at most %d steps, got %u", LQ4_CHAIN_MAX_STEPS, n_steps);
+    int rc = chain_validate(steps, n_steps);
+    if (rc) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    DeviceGuard g(ctx->device);
+    size_t off[kMaxChainSteps];
+    const size_t total = chain_scratch_layout(steps, n_steps, off);
+    rc = grow_scratch(ctx, &ctx->chain_scratch, &ctx->chain_scratch_bytes, total, s, true);
+    if (rc) return rc;
+
+    ChainArgs args;
+    uint32_t k_max = 0;
+    if (g_chain_mode == 0 && chain_plan(ctx, steps, n_steps, off, &args, &k_max)) {
+#ifdef LQ4_CHAIN_TRACE
+        args.trace = g_chain_trace;
+#endif
+        const hipError_t e = launch_gemv_chain(args, ctx->cu_count, k_max, s);
+        if (e != hipSuccess) return fail(LQ4_E_HIP, "chain launch: %s", hipGetErrorString(e));
+        ctx->chain_unchecked = true;
+        ctx->counters.gemv_chain++;
+        return LQ4_OK;
+    }
+
+    // Step by step: every step is lq4_gemv_fused (plus the stand-alone silu * up where a step ends
+    // in it); results nobody asked for live in the chain scratch as plain floats.
+    const float* prev = nullptr;
+    for (uint32_t j = 0; j < n_steps; ++j) {
+        const lq4_chain_step& st = steps[j];
+        float* spare = reinterpret_cast<float*>(ctx->chain_scratch + off[j]);
+        lq4_gemv_fusion f;
+        std::memset(&f, 0, sizeof f);
+        const float* x = st.x_dev;
+        f.prologue = st.prologue;
+        f.gamma = st.gamma;
+        f.eps = st.eps;
+        if (chain_reads_previous(st)) {
+            if (st.prologue == LQ4_PRO_ADD_RMSNORM) f.base = prev;
+            else x = prev;
+        } else {
+            f.base = st.base;
+            f.delta = st.delta;
+            f.residual_out = st.residual_out;
+        }
+        float* result;
+        if (st.epilogue == LQ4_EPI_ADD_RESIDUAL) {
+            f.epilogue = LQ4_EPI_ADD_RESIDUAL;
+            f.residual = st.residual;
+            f.copy_dst = st.y_dev;
+            rc = lq4_gemv_fused(ctx, st.w, st.w_extra_offset, st.n, st.k, x, nullptr, &f, nullptr, 0.0f, stream);
+            result = st.residual;
+        } else if (st.epilogue == LQ4_EPI_SILU_MUL_PAIRS) {
+            f.epilogue = LQ4_EPI_NONE;
+            rc = lq4_gemv_fused(ctx, st.w, st.w_extra_offset, st.n, st.k, x, spare, &f, nullptr, 0.0f, stream);
+            result = st.y_dev ? st.y_dev : spare;  // in place: out[i] only depends on in[i] and in[i + n/2]
+            if (!rc) {
+                launch_silu_mul(spare, st.n / 2, 1, result, st.n / 2, s);
+                ctx->counters.elementwise++;
+            }
+        } else {
+            f.epilogue = LQ4_EPI_NONE;
+            result = st.y_dev ? st.y_dev : spare;
+            rc = lq4_gemv_fused(ctx, st.w, st.w_extra_offset, st.n, st.k, x, result, &f, nullptr, 0.0f, stream);
+        }
+        if (rc) return rc;
+        prev = result;
+    }
+    LQ4_HIP(hipGetLastError());
+    return LQ4_OK;
+}
+
 int lq4_gemm_q8(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
                 const void* x_dev, int x_dtype, uint32_t m, float* y_dev, void* stream) {
     if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
@@ -734,13 +1039,13 @@ int lq4_gemm_q8(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
     } else if (m <= 32 || gemm_skinny_wants(n, k, m)) {
         // few rows: operands packed once, the few-token matrix-core kernel with this format's decoder
         // (always up to 32 rows: the large-tile kernels are no match for it there)
-        const int src = ensure_scratch(ctx, gemm_skinny_scratch_bytes(k, m));
+        const int src = ensure_scratch(ctx, gemm_skinny_scratch_bytes(k, m), static_cast<hipStream_t>(stream));
         if (src) return src;
         const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};
         launch_gemm_skinny(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, none, ctx->moe_scratch, s, 1);
         ctx->counters.gemm++;
     } else {
-        const int src = ensure_scratch(ctx, gemm_sibling_scratch_floats(1, n, k, m) * sizeof(float));
+        const int src = ensure_scratch(ctx, gemm_sibling_scratch_floats(1, n, k, m) * sizeof(float), static_cast<hipStream_t>(stream));
         if (src) return src;
         launch_gemm_q8(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, reinterpret_cast<float*>(ctx->moe_scratch), s);
         ctx->counters.gemm++;
@@ -775,13 +1080,13 @@ int lq4_gemm_q3(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
     } else if (m <= 32 || gemm_skinny_wants(n, k, m)) {
         // few rows: operands packed once, the few-token matrix-core kernel with this format's decoder
         // (always up to 32 rows: the large-tile kernels are no match for it there)
-        const int src = ensure_scratch(ctx, gemm_skinny_scratch_bytes(k, m));
+        const int src = ensure_scratch(ctx, gemm_skinny_scratch_bytes(k, m), static_cast<hipStream_t>(stream));
         if (src) return src;
         const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};
         launch_gemm_skinny(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, none, ctx->moe_scratch, s, 2);
         ctx->counters.gemm++;
     } else {
-        const int src = ensure_scratch(ctx, gemm_sibling_scratch_floats(2, n, k, m) * sizeof(float));
+        const int src = ensure_scratch(ctx, gemm_sibling_scratch_floats(2, n, k, m) * sizeof(float), static_cast<hipStream_t>(stream));
         if (src) return src;
         launch_gemm_q3(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, reinterpret_cast<float*>(ctx->moe_scratch), s);
         ctx->counters.gemm++;
@@ -816,6 +1121,10 @@ int lq4_probe_copy(lq4_ctx* ctx, const void* src_dev, void* dst_dev, size_t nbyt
 int lq4_get_path_counters(const lq4_ctx* ctx, lq4_path_counters* out) {
     if (!ctx || !out) return fail(LQ4_E_INVALID, "null argument");
     *out = ctx->counters;
+    uint32_t fallbacks = 0;
+    DeviceGuard g(ctx->device);
+    LQ4_HIP(hipMemcpy(&fallbacks, ctx->lora_sync + 2, sizeof fallbacks, hipMemcpyDeviceToHost));
+    out->lora_t_fallback = fallbacks;
     return LQ4_OK;
 }
 

@@ -9,19 +9,9 @@
 // Waves are persistent: each walks a strided list of row groups and keeps the next
 // group's blocks in flight while it works on the current one.
 //
-// Arithmetic.  A naive unpack (shift, mask, int->float, fma per nibble) would make VALU
-// issue, not HBM, the limit on this chip.  Instead a masked dword IS a pair of f16
-// subnormals:  q & 0x000F000F = (n_lo, n_hi) * 2^-24 and q & 0x00F000F0 = (n_lo, n_hi) * 2^-20
-// (gfx950's v_dot2_f32_f16 honours f16 subnormals), so one v_and per two weights unpacks
-// them exactly, and v_dot2_f32_f16 does two MACs per op with f32 accumulation.  The
-// activations paired with the 2^-20 form are pre-scaled by 2^-4.  To keep f32 accuracy the
-// f32 activation is split x = hi + lo/2048 with hi, lo both f16: every product is exact and
-// the result tracks an f32 GEMV, not an f16 one.  Per block
-//   y += (d * 2^24) * sum_k (n_k 2^-24) x_k  +  b * sum_k x_k,
-// the bias-factored form of the reference kernel (shaders/qwen35.metal:838-847).
-// Activations must be finite and below 65504 in magnitude (the f16 range), the same
-// limit the reference's half-staged tiled kernel has.
-#include "lq4_internal.hpp"
+// The unpack-free arithmetic (masked nibbles as f16 subnormals, activations as per-block scaled
+// hi/lo f16 pairs) and the LDS staging are in lq4_b1_dev.hpp, shared with the decode-chain kernel.
+#include "lq4_b1_dev.hpp"
 
 #include <type_traits>
 
@@ -29,88 +19,9 @@ namespace lq4 {
 
 namespace {
 
-typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+using namespace b1;
 
 constexpr int kWaves = 4;  // waves per workgroup unless a launch asks for more
-constexpr int kXPitch = 36;  // dwords of LDS per block of x: 16 hi pairs, 16 lo pairs, sum, 3 pad
-                             // (36 keeps 16-byte lane reads at stride 144 B conflict-free)
-constexpr float kLoScale = 2048.0f;
-constexpr float kTwo24 = 16777216.0f;
-
-struct __attribute__((packed, aligned(4))) Q4BlockRaw {
-    uint32_t sb;    // f16 scale | f16 bias << 16
-    uint32_t q[4];  // 32 nibbles, nibble i of dword j = weight 8j + i
-};
-
-__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
-    return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, a), __builtin_bit_cast(half2v, b), c, false);
-}
-
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ float dpp_add(float v) {
-    const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, false);
-    return v + __builtin_bit_cast(float, moved);
-}
-
-// Sums groups of SEG adjacent lanes (SEG = 16, 32 or 64); the total of a group is valid
-// in its last lane.
-template <int SEG>
-__device__ __forceinline__ float segment_sum(float v) {
-    v = dpp_add<0xB1, 0xF>(v);   // quad_perm [1,0,3,2]
-    v = dpp_add<0x4E, 0xF>(v);   // quad_perm [2,3,0,1]
-    v = dpp_add<0x141, 0xF>(v);  // row_half_mirror
-    v = dpp_add<0x140, 0xF>(v);  // row_mirror: every lane holds its 16-lane row sum
-    if (SEG >= 32) v = dpp_add<0x142, 0xA>(v);  // row_bcast:15 into rows 1 and 3
-    if (SEG >= 64) v = dpp_add<0x143, 0xC>(v);  // row_bcast:31 into rows 2 and 3
-    return v;
-}
-
-__device__ __forceinline__ uint32_t pack_h2(_Float16 a, _Float16 b) {
-    const half2v h = {a, b};
-    return __builtin_bit_cast(uint32_t, h);
-}
-
-// Converts 8 consecutive activations (the partners of one packed dword) into the pair order
-// the unpack produces — (0,4) (1,5) (2,6) (3,7) — as f16 hi parts and scaled f16 residuals.
-// Odd elements pair with the 2^-20 nibble form and are split after scaling by 2^-4.
-__device__ __forceinline__ void convert_x8(const float4 a, const float4 b, uint4& ph, uint4& pl, float& sum_x) {
-    const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-    _Float16 hi[8], lo[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const float s = (i & 1) ? v[i] * 0.0625f : v[i];
-        hi[i] = static_cast<_Float16>(s);
-        lo[i] = static_cast<_Float16>((s - static_cast<float>(hi[i])) * kLoScale);
-    }
-    ph.x = pack_h2(hi[0], hi[4]); ph.y = pack_h2(hi[1], hi[5]);
-    ph.z = pack_h2(hi[2], hi[6]); ph.w = pack_h2(hi[3], hi[7]);
-    pl.x = pack_h2(lo[0], lo[4]); pl.y = pack_h2(lo[1], lo[5]);
-    pl.z = pack_h2(lo[2], lo[6]); pl.w = pack_h2(lo[3], lo[7]);
-    sum_x = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
-}
-
-// 2^-24 * sum_k n_k * x_k over one block.
-__device__ __forceinline__ float block_dot(const uint32_t (&q)[4], const uint32_t (&xh)[16],
-                                           const uint32_t (&xl)[16]) {
-    float ph = 0.0f, pl = 0.0f;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const uint32_t w0 = q[j] & 0x000F000Fu;
-        const uint32_t w1 = q[j] & 0x00F000F0u;
-        const uint32_t q8 = q[j] >> 8;
-        const uint32_t w2 = q8 & 0x000F000Fu;
-        const uint32_t w3 = q8 & 0x00F000F0u;
-        ph = dot2(w0, xh[4 * j + 0], ph);
-        pl = dot2(w0, xl[4 * j + 0], pl);
-        ph = dot2(w1, xh[4 * j + 1], ph);
-        pl = dot2(w1, xl[4 * j + 1], pl);
-        ph = dot2(w2, xh[4 * j + 2], ph);
-        pl = dot2(w2, xl[4 * j + 2], pl);
-        ph = dot2(w3, xh[4 * j + 3], ph);
-        pl = dot2(w3, xl[4 * j + 3], pl);
-    }
-    return fmaf(pl, 1.0f / kLoScale, ph);
-}
 
 // A wave-row is 64/SEG weight rows side by side (SEG lanes each).  Wave `wid` of `n_waves`
 // works through chunks of RW wave-rows — chunk c holds wave-rows (c*RW + j)*n_waves + wid,
@@ -150,6 +61,10 @@ __device__ __forceinline__ float lora_a_row_partial(const void* a, int a_is_f16,
 // Whole-wave call.  Returns t[lane] (0 beyond the rank) once every slot carries `epoch`; polls the
 // slots at most `spin_limit` times and otherwise computes t in this wave.  The slots are read with
 // agent-scope atomic loads (they do not hit in this XCD's caches), value and epoch in one word.
+// The wave that computes t itself follows the producers' summation exactly (the k partition of a
+// WAVES*64-thread workgroup, the same wave sum, then the waves' sums in order), so t has the same
+// bits whichever way a wave obtained it.  Such waves count themselves in sync[2].
+template <int WAVES>
 __device__ __forceinline__ float lora_t_acquire(const LoraEpilogue& lora, uint32_t epoch, uint32_t k,
                                                 const float* __restrict__ x, int lane) {
     const bool mine = static_cast<uint32_t>(lane) < lora.rank;
@@ -168,10 +83,14 @@ __device__ __forceinline__ float lora_t_acquire(const LoraEpilogue& lora, uint32
         if (__all(static_cast<uint32_t>(v >> 32) == epoch)) return __builtin_bit_cast(float, static_cast<uint32_t>(v));
         __builtin_amdgcn_s_sleep(4);
     }
+    if (lane == 0) __hip_atomic_fetch_add(&lora.sync[2], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     float t = 0.0f;
     for (uint32_t j = 0; j < lora.rank; ++j) {
-        const float s = wave_sum(lora_a_row_partial(lora.a, lora.b_is_f16, j, k, x, lane, 64));
-        if (static_cast<uint32_t>(lane) == j) t = s;
+        float total = 0.0f;
+#pragma unroll
+        for (int v = 0; v < WAVES; ++v)
+            total += wave_sum(lora_a_row_partial(lora.a, lora.b_is_f16, j, k, x, v * 64 + lane, WAVES * 64));
+        if (static_cast<uint32_t>(lane) == j) t = total;
     }
     return t;
 }
@@ -202,6 +121,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
                                                           float* __restrict__ y, LoraEpilogue lora,
                                                           typename FusionArg<MODE == 1>::type fz) {
     extern __shared__ __attribute__((aligned(16))) uint32_t xs[];
+    lds_u32* const xsl = (lds_u32*)xs;
     constexpr bool FUSED = MODE == kFusedMode;
     constexpr bool INA = MODE == kLoraAMode;
     constexpr int RPW = 64 / SEG;  // weight rows per wave-row
@@ -361,20 +281,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
     __builtin_amdgcn_sched_barrier(0);  // nothing below is scheduled above these loads
 
     // ---- stage x: thread handles (block, dword j) = 8 activations ---------------------------
-    auto stage = [&](uint32_t g, const float4 a, const float4 b, bool store) {
-        const uint32_t blk = g >> 2, j = g & 3;
-        float sx;
-        uint4 ph, pl;
-        convert_x8(a, b, ph, pl, sx);
-        // the 4 threads of a block are 4 adjacent lanes: quad butterfly
-        sx = dpp_add<0xB1, 0xF>(sx);
-        sx = dpp_add<0x4E, 0xF>(sx);
-        if (store) {
-            *reinterpret_cast<uint4*>(&xs[blk * kXPitch + 4 * j]) = ph;
-            *reinterpret_cast<uint4*>(&xs[blk * kXPitch + 16 + 4 * j]) = pl;
-            if (j == 0) *reinterpret_cast<float*>(&xs[blk * kXPitch + 32]) = sx;
-        }
-    };
+    auto stage = [&](uint32_t g, const float4 a, const float4 b, bool store) { stage_x8(xsl, g, a, b, store); };
     if constexpr (!FUSED) {
 #pragma unroll
         for (int i = 0; i < HF; ++i) stage(gx[i], xa[i], xb[i], tid + i * WAVES * 64 < nb * 4);
@@ -506,23 +413,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
                 const uint32_t blk_raw = slab * 64 + seg_lane;
                 const bool live = blk_raw < nb;
                 const uint32_t blk = live ? blk_raw : nb - 1;
-                uint32_t xh[16], xl[16];
-                const uint4* xsrc = reinterpret_cast<const uint4*>(&xs[blk * kXPitch]);
+                XBlock xblk;
+                load_xblock(xsl, blk, xblk);
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const uint4 h = xsrc[i], l = xsrc[4 + i];
-                    xh[4 * i + 0] = h.x; xh[4 * i + 1] = h.y; xh[4 * i + 2] = h.z; xh[4 * i + 3] = h.w;
-                    xl[4 * i + 0] = l.x; xl[4 * i + 1] = l.y; xl[4 * i + 2] = l.z; xl[4 * i + 3] = l.w;
-                }
-                const float sum_x = live ? *reinterpret_cast<const float*>(&xs[blk * kXPitch + 32]) : 0.0f;
-#pragma unroll
-                for (int j = 0; j < RW; ++j) {
-                    const float p = block_dot(cur[j][t].q, xh, xl);
-                    float d = f16_bits_to_f32(cur[j][t].sb & 0xffffu) * kTwo24;
-                    const float b = f16_bits_to_f32(cur[j][t].sb >> 16);
-                    if (!live) d = 0.0f;
-                    acc[j] = fmaf(d, p, fmaf(b, sum_x, acc[j]));
-                }
+                for (int j = 0; j < RW; ++j) acc[j] = block_fma(cur[j][t], xblk, live, acc[j]);
             }
         }
 
@@ -537,7 +431,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
                 if constexpr (INA) {
                     // lane l of the wave holds t[l]; every lane takes part in the exchange
                     if (!t_have) {
-                        t_reg = lora_t_acquire(lora, __builtin_amdgcn_readfirstlane(lora_epoch), k, x, lane);
+                        t_reg = lora_t_acquire<WAVES>(lora, __builtin_amdgcn_readfirstlane(lora_epoch), k, x, lane);
                         t_have = true;
                     }
                     for (uint32_t i0 = 0; i0 < lora.rank; i0 += SEG) {
@@ -671,7 +565,11 @@ void launch_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* 
     // 16.2 -> 15.2; behind on K 2048 and K 17408)
     const uint32_t wg_waves = (seg == 64 && k >= 4096 && k <= 8192) ? 8 : kWaves;
     wg_per_cu = wg_per_cu > 16 / wg_waves ? 16 / wg_waves : wg_per_cu < 1 ? 1 : wg_per_cu;
-    const uint32_t max_waves = 256 * wg_per_cu * wg_waves;
+    // A launch that computes A.x itself carries `rank` producer workgroups in front: the weight
+    // workgroups leave them room, so that every workgroup of the launch is resident at once and none
+    // starts after the producers have advanced the epoch.
+    const uint32_t producers = (lora.rank && lora.a && !fusion) ? lora.rank : 0;
+    const uint32_t max_waves = (256 * wg_per_cu - producers) * wg_waves;
     uint32_t rw = (n_wrows + max_waves - 1) / max_waves;
     uint32_t waves;
     if (rw <= 4) {

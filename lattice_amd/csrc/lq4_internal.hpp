@@ -74,6 +74,48 @@ void launch_gemv_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, fl
 void launch_gemv_b1_fused(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y,
                           const LoraEpilogue& lora, const GemvFusion& fusion, hipStream_t stream);
 
+// One launch for a chain of dependent batch-1 GEMVs (lq4_gemv_chain.hip).  A step's result vector is
+// W . x after its epilogue: kStore W . x [n]; kAddResidual residual + W . x [n] (also written back to
+// res_out); kSiluMulPairs silu(y[i]) * y[i + n/2] [n/2] for W = [gate rows | up rows].  The next step
+// reads it from `out_tagged` ({f32, launch epoch} words in library scratch) when its x_tagged points
+// there; x_tagged == null means external activations (x, or base/delta/gamma under kAddNorm, or
+// gate|up in x under kSiluMul).  With x_tagged set the prologue is kPlain or kAddNorm (the norm of
+// the previous result, gamma/eps only).
+constexpr int kMaxChainSteps = 16;
+struct ChainStep {
+    enum Prologue : int { kPlain = 0, kAddNorm = 1, kSiluMul = 2 };
+    enum Epilogue : int { kStore = 0, kAddResidual = 1, kSiluMulPairs = 2 };
+    const uint8_t* w;
+    const float* x;
+    const unsigned long long* x_tagged;
+    const float* base;
+    const float* delta;
+    const float* gamma;
+    float* residual_out;                   // external kAddNorm only: receives base + delta
+    const float* res_plain;                // kAddResidual input: external ...
+    const unsigned long long* res_tagged;  // ... or an earlier step's tagged result
+    float* res_out;                        // kAddResidual: the updated residual (plain copy)
+    float* y;                              // plain copy of the result, or null
+    unsigned long long* out_tagged;        // null when no later step reads the result
+    uint32_t n, k;
+    float eps;
+    int prologue, epilogue;
+    uint32_t slabs, group_rows, groups;    // work split, filled by gemv_chain_plan_step
+};
+struct ChainArgs {
+    uint32_t n_steps;
+    uint32_t spin_limit;   // polls a wave spends on one hand-over before it gives up (0: give up at once)
+    uint32_t xs_dwords;    // LDS dwords per activation buffer, filled by the launcher
+    uint32_t* epoch;       // launch epoch word
+    uint32_t* fail;        // set to the step index whose activations never arrived
+    unsigned long long* trace;  // development builds only: 32 wall-clock stamps per wave
+    ChainStep s[kMaxChainSteps];
+};
+size_t gemv_chain_lds_bytes(uint32_t k_max);
+uint32_t gemv_chain_max_k();
+bool gemv_chain_plan_step(ChainStep& st, uint32_t workgroups);
+hipError_t launch_gemv_chain(ChainArgs& args, uint32_t workgroups, uint32_t k_max, hipStream_t stream);
+
 // Stand-alone forms of the same steps for any number of rows.
 //   residual_add_norm: v = base + delta (delta may be null); residual_out = v if set;
 //     normed_out = shifted RMSNorm of v.  Rows are `hidden` floats apart.

@@ -1,0 +1,223 @@
+"""The chain of dependent batch-1 GEMVs that runs as one launch (`lq4_gemv_chain`): the decode steps the
+reference encodes into one command buffer per token (forward/metal_qwen35.rs:6943, :6447):
+o -> residual add -> shifted RMSNorm -> gate||up -> silu * up -> down -> residual add -> next layer's
+RMSNorm -> qkv.  Checked against the oracle's unfused sequence (f32 GEMV after dequantisation, the
+elementwise restatements) and against the library's own step-by-step form."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from lattice_amd import synth
+from util import REL_TOL, rel_err
+
+EPS = 1e-6
+
+
+def _oracle_layer(x_attn, r0, g1, g2, w_o, w_gu, w_down, w_qkv, hidden, inter, qkv_rows):
+    """o(+residual) -> norm -> gate||up -> silu*up -> down(+residual) -> norm -> qkv, step by step."""
+    y_o = oracle.gemm_f32(x_attn[None, :], w_o, hidden, hidden)[0]
+    r1, _ = oracle.add_and_copy(y_o, r0)
+    xn = oracle.shifted_rms_norm(r1[None, :], g1, EPS)[0]
+    gu = oracle.gemm_f32(xn[None, :], w_gu, 2 * inter, hidden)[0]
+    h = oracle.silu_mul(gu[None, :])[0]
+    y_d = oracle.gemm_f32(h[None, :], w_down, hidden, inter)[0]
+    r2, _ = oracle.add_and_copy(y_d, r1)
+    xn2 = oracle.shifted_rms_norm(r2[None, :], g2, EPS)[0]
+    qkv = oracle.gemm_f32(xn2[None, :], w_qkv, qkv_rows, hidden)[0]
+    return r1, h, r2, qkv
+
+
+def _layer_inputs(hidden, inter, qkv_rows, seed):
+    g = np.random.default_rng(seed)
+    w = dict(o=synth.q4_weight(hidden, hidden, seed=seed, tag="o"),
+             gu=synth.q4_weight(2 * inter, hidden, seed=seed, tag="gu"),
+             down=synth.q4_weight(hidden, inter, seed=seed, tag="down"),
+             qkv=synth.q4_weight(qkv_rows, hidden, seed=seed, tag="qkv"))
+    x_attn = synth.activations(1, hidden, seed=seed, tag="attn")[0]
+    r0 = synth.activations(1, hidden, seed=seed, tag="res")[0]
+    g1 = (0.1 * g.normal(size=hidden)).astype(np.float32)
+    g2 = (0.1 * g.normal(size=hidden)).astype(np.float32)
+    return w, x_attn, r0, g1, g2
+
+
+def _run_layer_chain(be, qw, x_attn, r0, g1, g2, hidden, inter, qkv_rows, want_h=False):
+    import torch
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    xd, rd, g1d, g2d = dev(x_attn), dev(r0), dev(g1), dev(g2)
+    qkv = torch.full((qkv_rows,), float("nan"), dtype=torch.float32, device="cuda")
+    h = torch.full((inter,), float("nan"), dtype=torch.float32, device="cuda") if want_h else None
+    steps = [
+        be.chain_step(qw["o"], hidden, hidden, x=xd, add_residual=rd),
+        be.chain_step(qw["gu"], 2 * inter, hidden, norm=(None, None, g1d, EPS, None), silu_mul_pairs=True, y=h),
+        be.chain_step(qw["down"], hidden, inter, add_residual=rd),
+        be.chain_step(qw["qkv"], qkv_rows, hidden, norm=(None, None, g2d, EPS, None), y=qkv),
+    ]
+    be.dispatch_chain(steps)
+    be.synchronize()
+    return rd.cpu().numpy(), qkv.cpu().numpy(), (h.cpu().numpy() if want_h else None)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("hidden,inter,qkv_rows", [(2048, 6144, 3072), (64, 96, 40), (1024, 512, 6), (4096, 2048, 1000)])
+def test_decode_layer_chain_matches_oracle_sequence(hidden, inter, qkv_rows):
+    from lattice_amd import backend
+    be = backend.HipQ4Backend(0)
+    w, x_attn, r0, g1, g2 = _layer_inputs(hidden, inter, qkv_rows, seed=3)
+    qw = {k: be.upload_q4_blocks(v) for k, v in w.items()}
+    _, want_h, want_r2, want_qkv = _oracle_layer(x_attn, r0, g1, g2, w["o"], w["gu"], w["down"], w["qkv"], hidden, inter, qkv_rows)
+
+    before = be.path_counters()["gemv_chain"]
+    got_r, got_qkv, got_h = _run_layer_chain(be, qw, x_attn, r0, g1, g2, hidden, inter, qkv_rows, want_h=True)
+    assert be.path_counters()["gemv_chain"] == before + 1, "the persistent launch did not serve this chain"
+    assert rel_err(got_h, want_h) <= REL_TOL
+    assert rel_err(got_r, want_r2) <= REL_TOL
+    assert rel_err(got_qkv, want_qkv) <= REL_TOL
+    # in fact f32-faithful
+    assert rel_err(got_r, want_r2) <= 2e-5 and rel_err(got_qkv, want_qkv) <= 2e-5
+
+    # the same chain step by step through the library: equal to f32 rounding (the sum of squares and
+    # silu are formed differently)
+    be.set_chain_mode(1)
+    try:
+        ref_r, ref_qkv, ref_h = _run_layer_chain(be, qw, x_attn, r0, g1, g2, hidden, inter, qkv_rows, want_h=True)
+    finally:
+        be.set_chain_mode(0)
+    assert be.path_counters()["gemv_chain"] == before + 1
+    assert rel_err(got_r, ref_r) <= 1e-5 and rel_err(got_qkv, ref_qkv) <= 1e-5 and rel_err(got_h, ref_h) <= 1e-5
+    be.close()
+
+
+@pytest.mark.gpu
+def test_chain_of_independent_steps_and_external_prologues():
+    """Steps that all take external activations (no hand-over), with each external prologue, and a
+    result that is only handed on (no y) next to one that is also stored."""
+    import torch
+    from lattice_amd import backend
+    be = backend.HipQ4Backend(0)
+    n, k = 300, 256
+    g = np.random.default_rng(5)
+    w1, w2, w3 = (synth.q4_weight(n, k, seed=s) for s in (1, 2, 3))
+    x = synth.activations(1, k, seed=1)[0]
+    base, delta = synth.activations(1, k, seed=2)[0], synth.activations(1, k, seed=3)[0]
+    gamma = (0.2 * g.normal(size=k)).astype(np.float32)
+    gate_up = synth.activations(1, 2 * k, seed=4)[0]
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    q1, q2, q3 = (be.upload_q4_blocks(w) for w in (w1, w2, w3))
+    y1, y2, y3 = (torch.full((n,), float("nan"), dtype=torch.float32, device="cuda") for _ in range(3))
+    res_out = torch.zeros(k, dtype=torch.float32, device="cuda")
+    steps = [
+        be.chain_step(q1, n, k, x=dev(x), y=y1),
+        be.chain_step(q2, n, k, norm=(dev(base), dev(delta), dev(gamma), EPS, res_out), y=y2),
+        be.chain_step(q3, n, k, x=dev(gate_up), silu_mul=True, y=y3),
+    ]
+    before = be.path_counters()["gemv_chain"]
+    be.dispatch_chain(steps)
+    be.synchronize()
+    assert be.path_counters()["gemv_chain"] == before + 1
+    res, normed = oracle.residual_add_norm(base[None, :], delta[None, :], gamma, EPS)
+    assert rel_err(y1.cpu().numpy(), oracle.gemm_f32(x[None, :], w1, n, k)[0]) <= 2e-5
+    assert rel_err(y2.cpu().numpy(), oracle.gemm_f32(normed, w2, n, k)[0]) <= 2e-5
+    assert np.array_equal(res_out.cpu().numpy(), res[0])
+    assert rel_err(y3.cpu().numpy(), oracle.gemm_f32(oracle.silu_mul(gate_up[None, :]), w3, n, k)[0]) <= 2e-5
+    be.close()
+
+
+@pytest.mark.gpu
+def test_chain_replays_in_a_graph_and_large_steps_fall_back():
+    import torch
+    from lattice_amd import backend
+    be = backend.HipQ4Backend(0)
+    hidden, inter, qkv_rows = 512, 768, 320
+    w, x_attn, r0, g1, g2 = _layer_inputs(hidden, inter, qkv_rows, seed=9)
+    qw = {k: be.upload_q4_blocks(v) for k, v in w.items()}
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    xd, rd, g1d, g2d = dev(x_attn), dev(r0), dev(g1), dev(g2)
+    qkv = torch.zeros(qkv_rows, dtype=torch.float32, device="cuda")
+    steps = [
+        be.chain_step(qw["o"], hidden, hidden, x=xd, add_residual=rd),
+        be.chain_step(qw["gu"], 2 * inter, hidden, norm=(None, None, g1d, EPS, None), silu_mul_pairs=True),
+        be.chain_step(qw["down"], hidden, inter, add_residual=rd),
+        be.chain_step(qw["qkv"], qkv_rows, hidden, norm=(None, None, g2d, EPS, None), y=qkv),
+    ]
+    be.dispatch_chain(steps)  # warm: the scratch exists before the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        be.dispatch_chain(steps)
+    # every replay works on the residual the previous one left: follow it with the oracle
+    rd.copy_(dev(r0))
+    torch.cuda.synchronize()
+    r_host = r0
+    for rep in range(4):
+        graph.replay()
+        torch.cuda.synchronize()
+        _, _, want_r2, want_qkv = _oracle_layer(x_attn, r_host, g1, g2, w["o"], w["gu"], w["down"], w["qkv"], hidden, inter, qkv_rows)
+        assert rel_err(rd.cpu().numpy(), want_r2) <= 2e-5, rep
+        assert rel_err(qkv.cpu().numpy(), want_qkv) <= 2e-5, rep
+        r_host = rd.cpu().numpy()
+        # eager work of the same library between the replays
+        y = torch.empty((1, hidden), dtype=torch.float32, device="cuda")
+        be.dispatch_matmul(xd, qw["o"], y, 1, hidden, hidden)
+        be.synchronize()
+
+    # a step beyond the register slots of the resident grid: served step by step, same contract
+    n_big, k_big = 14000, 2048
+    wb = synth.q4_weight(n_big, k_big, seed=10)
+    qb = be.upload_q4_blocks(wb)
+    xb = synth.activations(1, k_big, seed=10)[0]
+    yb = torch.empty(n_big, dtype=torch.float32, device="cuda")
+    before = be.path_counters()["gemv_chain"]
+    be.dispatch_chain([be.chain_step(qb, n_big, k_big, x=dev(xb), y=yb)])
+    be.synchronize()
+    assert be.path_counters()["gemv_chain"] == before
+    assert rel_err(yb.cpu().numpy(), oracle.gemm_f32(xb[None, :], wb, n_big, k_big)[0]) <= 2e-5
+    be.close()
+
+
+@pytest.mark.gpu
+def test_chain_contract_errors_and_bounded_wait():
+    import torch
+    from lattice_amd import backend
+    be = backend.HipQ4Backend(0)
+    n, k = 64, 64
+    qw = be.upload_q4_blocks(synth.q4_weight(n, k, seed=0))
+    x = torch.zeros(k, dtype=torch.float32, device="cuda")
+    y = torch.zeros(n, dtype=torch.float32, device="cuda")
+    with pytest.raises(backend.Q4Error, match="step 0 needs external"):
+        be.dispatch_chain([be.chain_step(qw, n, k, y=y)])
+    with pytest.raises(backend.Q4Error, match="nowhere to put its result"):
+        be.dispatch_chain([be.chain_step(qw, n, k, x=x)])
+    with pytest.raises(backend.Q4Error, match="previous step yields"):
+        be.dispatch_chain([be.chain_step(qw, n, k, x=x, silu_mul_pairs=True), be.chain_step(qw, n, k, y=y)])
+    with pytest.raises(backend.Q4Error, match="at most 16"):
+        be.dispatch_chain([be.chain_step(qw, n, k, x=x, y=y)] * 17)
+    be.dispatch_chain([])  # no-op
+    be.close()
+
+    # A wait that is cut short: the kernel leaves at its first dependent step, every workgroup exits,
+    # and the failure is reported at the next synchronisation; the step-by-step form still serves.
+    os.environ["LQ4_CHAIN_SPIN_LIMIT"] = "0"
+    try:
+        be2 = backend.HipQ4Backend(0)
+    finally:
+        del os.environ["LQ4_CHAIN_SPIN_LIMIT"]
+    qw = be2.upload_q4_blocks(synth.q4_weight(n, k, seed=0))
+    wq = synth.q4_weight(n, k, seed=0)
+    xh = synth.activations(1, k, seed=0)[0]
+    xd = torch.from_numpy(xh).cuda()
+    steps = [be2.chain_step(qw, n, k, x=xd), be2.chain_step(qw, n, k, y=y)]
+    be2.dispatch_chain(steps)
+    with pytest.raises(backend.Q4Error, match="never arrived"):
+        be2.synchronize()
+    be2.synchronize()  # reported once
+    be2.set_chain_mode(1)
+    try:
+        be2.dispatch_chain(steps)
+        be2.synchronize()
+    finally:
+        be2.set_chain_mode(0)
+    y1 = oracle.gemm_f32(xh[None, :], wq, n, k)
+    assert rel_err(y.cpu().numpy(), oracle.gemm_f32(y1, wq, n, k)[0]) <= 2e-5
+    be2.close()

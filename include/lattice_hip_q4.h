@@ -226,52 +226,63 @@ int lq4_gemv_fused(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, u
                    const float* x_dev, float* y_dev, const lq4_gemv_fusion* fusion, const lq4_lora* lora,
                    float lora_scale, void* stream);
 
-/* ---- a chain of dependent one-token GEMVs in one launch ---------------------------------------
+/* ---- a chain of one-token GEMVs in one launch -------------------------------------------------
  * The reference encodes a whole token into one command buffer (forward_step,
  * forward/metal_qwen35.rs:6943, committed once at :6447): o -> residual add + RMSNorm -> gate||up ->
- * silu * up -> down -> residual add -> next layer's RMSNorm -> qkv follow each other without the
- * host in between (encode_mlp_block, inner/layers/mod.rs; the elementwise dispatches at
+ * silu * up -> down -> residual add + next layer's RMSNorm -> qkv follow each other without the host
+ * in between (encode_mlp_block, inner/layers/mod.rs; the elementwise dispatches at
  * inner/dispatch.rs:916-930, 1171-1290).  lq4_gemv_chain is that unit here: up to
- * LQ4_CHAIN_MAX_STEPS batch-1 GEMVs, each fed by an external vector or by the previous step's
- * result, run as ONE persistent launch whose waves request the weights of later steps while
- * earlier results are still on their way (falls back to one lq4_gemv_fused per step, same results to
- * f32 rounding, when a step is too large for that: more than ~25 M weights, or K > 16384).
+ * LQ4_CHAIN_MAX_STEPS batch-1 GEMVs, each fed by an external vector or by an earlier step's result,
+ * behind one call.  By default every step is one fused launch (lq4_gemv_fused, plus the stand-alone
+ * silu * up where a step ends in it).  With lq4_set_chain_mode(LQ4_CHAIN_ONE_LAUNCH) an eligible
+ * chain (every K <= 8192) runs as ONE persistent launch whose waves request the weights of later
+ * steps while earlier results are still on their way and hand results over through tagged words in
+ * library scratch; on MI355X that hand-over costs more than the launches it saves (36 us against
+ * 16 us for the four GEMVs of a 2B decode layer), so it is not the default.  Both forms give the same
+ * results to f32 rounding.
  *
- * Step j computes r_j = epilogue(W_j . prologue(x_j)):
- *   x_j        x_dev (f32 [K]; [2K] = gate | up for LQ4_PRO_SILU_MUL), or base/delta/gamma under
- *              LQ4_PRO_ADD_RMSNORM as in lq4_gemv_fusion, or, with x_dev == NULL and base == NULL,
- *              the previous step's result r_(j-1) (then K must equal its length; the prologue is
- *              LQ4_PRO_NONE, or LQ4_PRO_ADD_RMSNORM = shifted RMSNorm of r_(j-1) with gamma, eps);
- *   epilogue   LQ4_EPI_NONE           r = W . x                         [N]
+ * Step j computes r_j = epilogue(W_j . prologue(...)):
+ *   prologue   LQ4_PRO_NONE         activations = x_dev [K], or r_(j-1) when from_previous != 0
+ *              LQ4_PRO_ADD_RMSNORM  v = base + delta as in lq4_gemv_fusion (base or delta may be NULL),
+ *                                   with r_(j-1) in the place of delta when from_previous != 0;
+ *                                   activations = v * rsqrt(mean(v^2) + eps) * (1 + gamma);
+ *                                   residual_out (if not NULL, no overlap with base/delta) = v
+ *                                   (dispatch_fused_residual_add_norm, inner/dispatch.rs:1171-1266)
+ *              LQ4_PRO_SILU_MUL     activations = silu(x_dev[0..K)) * x_dev[K..2K), external only
+ *   epilogue   LQ4_EPI_NONE           r = W . x                          [N]
  *              LQ4_EPI_ADD_RESIDUAL   r = residual + W . x, residual = r [N]  (dispatch_add_and_copy)
  *              LQ4_EPI_SILU_MUL_PAIRS r[i] = silu(y[i]) * y[i + N/2]     [N/2] for W = [gate rows | up
  *                                     rows], the fused buffer of metal_qwen35.rs:12137-12152
- *                                     (dispatch_silu_mul_fused);
+ *                                     (dispatch_silu_mul_fused)
  *   y_dev      receives r_j when not NULL (the last step needs y_dev or a residual).
- * Vectors of different steps must be identical or disjoint.  The launch keeps hand-over state in the
- * context: chains must not overlap on two streams of one context.  A hand-over that never
- * completes (the grid not resident at once because another kernel holds the GPU) ends the launch
- * after a bounded wait and lq4_sync returns LQ4_E_HIP; the chain's results are then invalid. */
+ * With from_previous the step's K must equal the length of r_(j-1).  Any input vector (x_dev, base,
+ * delta) may also be the y_dev or residual_out of an earlier step of the same chain.  Vectors of
+ * different steps must be identical or disjoint.  The launch keeps hand-over state in the context:
+ * chains must not overlap on two streams of one context.  A hand-over that never completes (the
+ * grid not resident at once because another kernel holds the GPU) ends the launch after a bounded
+ * wait and lq4_sync returns LQ4_E_HIP; the chain's results are then invalid. */
 #define LQ4_CHAIN_MAX_STEPS 16
 #define LQ4_EPI_SILU_MUL_PAIRS 2
 typedef struct lq4_chain_step {
     const lq4_weight* w;
     uint64_t w_extra_offset;
     uint32_t n, k;
+    int from_previous;
     const float* x_dev;
     int prologue;
     const float* base;
     const float* delta;
     const float* gamma;
     float eps;
-    float* residual_out; /* external LQ4_PRO_ADD_RMSNORM only: receives base + delta */
+    float* residual_out;
     int epilogue;
     float* residual;
     float* y_dev;
 } lq4_chain_step;
 int lq4_gemv_chain(lq4_ctx* ctx, const lq4_chain_step* steps, uint32_t n_steps, void* stream);
-/* Tuning/test hook, process-wide: 0 = one persistent launch where the chain is eligible (default),
- * 1 = always step by step.  No counterpart in the reference. */
+/* Process-wide: how lq4_gemv_chain runs a chain.  No counterpart in the reference. */
+#define LQ4_CHAIN_STEPWISE 0   /* one launch per step (default) */
+#define LQ4_CHAIN_ONE_LAUNCH 1 /* one persistent launch where the chain is eligible */
 int lq4_set_chain_mode(int mode);
 
 /* Grows the context's scratch (partial tiles of K-sliced GEMMs, packed few-token operands, MoE

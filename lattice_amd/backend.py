@@ -79,6 +79,7 @@ class PathCounters(C.Structure):
 LQ4_PRO_NONE, LQ4_PRO_ADD_RMSNORM, LQ4_PRO_SILU_MUL = 0, 1, 2
 LQ4_EPI_NONE, LQ4_EPI_ADD_RESIDUAL, LQ4_EPI_SILU_MUL_PAIRS = 0, 1, 2
 CHAIN_MAX_STEPS = 16
+CHAIN_STEPWISE, CHAIN_ONE_LAUNCH = 0, 1  # lq4_set_chain_mode
 
 
 class GemvFusion(C.Structure):
@@ -91,6 +92,7 @@ class GemvFusion(C.Structure):
 class ChainStep(C.Structure):
     """``lq4_chain_step``: one batch-1 GEMV of a chain that runs as a single launch."""
     _fields_ = [("w", C.c_void_p), ("w_extra_offset", C.c_uint64), ("n", C.c_uint32), ("k", C.c_uint32),
+                ("from_previous", C.c_int),
                 ("x_dev", C.c_void_p), ("prologue", C.c_int), ("base", C.c_void_p), ("delta", C.c_void_p),
                 ("gamma", C.c_void_p), ("eps", C.c_float), ("residual_out", C.c_void_p), ("epilogue", C.c_int),
                 ("residual", C.c_void_p), ("y_dev", C.c_void_p)]
@@ -427,19 +429,21 @@ class HipQ4Backend:
         _check(self.lib.lq4_gemv_fused(self.ctx, qw.handle, qw_extra_offset, n, k, self._ptr(x), self._ptr(y),
                                        C.byref(f), lora, self._lora_scale, self._stream()))
 
-    def chain_step(self, qw: Q4WeightBuf, n: int, k: int, *, x=None, norm=None, silu_mul=False,
+    def chain_step(self, qw: Q4WeightBuf, n: int, k: int, *, x=None, from_previous=False, norm=None, silu_mul=False,
                    add_residual=None, silu_mul_pairs=False, y=None, qw_extra_offset: int = 0) -> ChainStep:
-        """One step of :meth:`dispatch_chain`.  ``x=None`` (and no ``base`` in ``norm``) feeds the step
-        with the previous step's result.  ``norm=(base, delta, gamma, eps, residual_out)`` as in
-        :meth:`dispatch_matmul_fused`, or ``norm=(None, None, gamma, eps, None)`` for the shifted RMSNorm
-        of the previous result; ``silu_mul=True``: ``x`` holds gate | up; ``add_residual=residual``:
-        the result is ``residual + W.x``, written back; ``silu_mul_pairs=True``: W is gate rows then up
-        rows and the result is ``silu(gate) * up`` (n/2 values); ``y`` receives the result."""
+        """One step of :meth:`dispatch_chain`.  ``from_previous=True`` feeds the step with the previous
+        step's result (in the place of ``x``, or of ``delta`` under ``norm``).
+        ``norm=(base, delta, gamma, eps, residual_out)`` as in :meth:`dispatch_matmul_fused`
+        (``base`` / ``delta`` may be ``None``); ``silu_mul=True``: ``x`` holds gate | up;
+        ``add_residual=residual``: the result is ``residual + W.x``, written back;
+        ``silu_mul_pairs=True``: W is gate rows then up rows and the result is ``silu(gate) * up``
+        (n/2 values); ``y`` receives the result."""
         self._assert_k(k, "dispatch_matmul_q4")
         assert not (norm is not None and silu_mul), "one prologue at a time"
         assert not (add_residual is not None and silu_mul_pairs), "one epilogue at a time"
         st = ChainStep()
         st.w, st.w_extra_offset, st.n, st.k = qw.handle, qw_extra_offset, n, k
+        st.from_previous = int(bool(from_previous))
         st.x_dev = self._ptr(x)
         st.prologue = LQ4_PRO_ADD_RMSNORM if norm is not None else LQ4_PRO_SILU_MUL if silu_mul else LQ4_PRO_NONE
         keep = [qw, x, y, add_residual]
@@ -457,12 +461,13 @@ class HipQ4Backend:
 
     def dispatch_chain(self, steps: Sequence[ChainStep]):
         """The dispatches of one token between two points where the host must look at the result
-        (``forward_step`` encodes them into one command buffer, metal_qwen35.rs:6943), as one launch."""
+        (``forward_step`` encodes them into one command buffer, metal_qwen35.rs:6943), as one library call."""
         arr = (ChainStep * len(steps))(*steps)
         _check(self.lib.lq4_gemv_chain(self.ctx, arr, len(steps), self._stream()))
 
     def set_chain_mode(self, mode: int):
-        """0 = one persistent launch where the chain is eligible, 1 = always step by step."""
+        """``CHAIN_STEPWISE`` (default): one launch per step; ``CHAIN_ONE_LAUNCH``: one persistent launch
+        where the chain is eligible."""
         _check(self.lib.lq4_set_chain_mode(int(mode)))
 
     def dispatch_gemm(self, x, x_offset: int, qw: Q4WeightBuf, y, y_offset: int, m: int, n: int,

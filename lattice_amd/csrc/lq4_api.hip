@@ -192,8 +192,8 @@ int lq4_ctx_create(int device_ordinal, lq4_ctx** out) {
     c->lora_sync = c->topk_ticket + 64;
     hipDeviceProp_t prop;
     e = hipGetDeviceProperties(&prop, device_ordinal);
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&c->chain_sync), 512);
-    if (e == hipSuccess) e = hipMemset(c->chain_sync, 0, 512);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&c->chain_sync), 512 + 16384);
+    if (e == hipSuccess) e = hipMemset(c->chain_sync, 0, 512 + 16384);
     if (e == hipSuccess) e = hipMemcpy(c->chain_sync, &first_epoch, 4, hipMemcpyHostToDevice);
     if (e != hipSuccess) {
         if (c->chain_sync) (void)hipFree(c->chain_sync);
@@ -783,19 +783,15 @@ int lq4_gemv_fused(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, u
     return LQ4_OK;
 }
 
-// ---- a chain of dependent batch-1 GEMVs ----------------------------------------------------------
+// ---- a chain of batch-1 GEMVs --------------------------------------------------------------------
 namespace {
 
-int g_chain_mode = 0;  // 0 = one persistent launch where the chain is eligible, 1 = always step by step
+int g_chain_mode = LQ4_CHAIN_STEPWISE;
 
 inline size_t up256(size_t v) { return (v + 255) / 256 * 256; }
 
 inline uint32_t chain_result_len(const lq4_chain_step& st) {
     return st.epilogue == LQ4_EPI_SILU_MUL_PAIRS ? st.n / 2 : st.n;
-}
-
-inline bool chain_reads_previous(const lq4_chain_step& st) {
-    return !st.x_dev && !(st.prologue == LQ4_PRO_ADD_RMSNORM && st.base);
 }
 
 // The plain pointer a step's result is stored at for the caller (null: nowhere).
@@ -811,36 +807,36 @@ int chain_validate(const lq4_chain_step* steps, uint32_t n_steps) {
         const uint8_t* wp;
         const int rc = resolve_weight(st.w, st.w_extra_offset, st.n, st.k, &wp);
         if (rc) return rc;
-        const bool prev = chain_reads_previous(st);
-        if (prev) {
+        if (st.from_previous) {
             if (j == 0) return fail(LQ4_E_INVALID, "chain step 0 needs external activations");
             if (st.prologue != LQ4_PRO_NONE && st.prologue != LQ4_PRO_ADD_RMSNORM)
                 return fail(LQ4_E_INVALID, "chain step %u: a step fed by the previous result takes LQ4_PRO_NONE or LQ4_PRO_ADD_RMSNORM", j);
             if (chain_result_len(steps[j - 1]) != st.k)
                 return fail(LQ4_E_INVALID, "chain step %u: K = %u but the previous step yields %u values", j, st.k,
                             chain_result_len(steps[j - 1]));
-            if (st.delta || st.residual_out)
-                return fail(LQ4_E_INVALID, "chain step %u: delta / residual_out belong to an external LQ4_PRO_ADD_RMSNORM", j);
-        } else {
-            switch (st.prologue) {
-                case LQ4_PRO_NONE:
-                case LQ4_PRO_SILU_MUL:
-                    if (!st.x_dev || misaligned(st.x_dev, 16)) return fail(LQ4_E_INVALID, "chain step %u: x must be non-null and 16-byte aligned", j);
-                    break;
-                case LQ4_PRO_ADD_RMSNORM:
-                    if (misaligned(st.base, 16) || (st.delta && misaligned(st.delta, 16)) ||
-                        (st.residual_out && misaligned(st.residual_out, 16)))
-                        return fail(LQ4_E_INVALID, "chain step %u: base, delta and residual_out must be 16-byte aligned", j);
-                    if (st.residual_out && (ranges_overlap(st.residual_out, st.base, static_cast<size_t>(st.k) * 4) ||
-                                            (st.delta && ranges_overlap(st.residual_out, st.delta, static_cast<size_t>(st.k) * 4))))
-                        return fail(LQ4_E_INVALID, "chain step %u: residual_out must not overlap base or delta", j);
-                    break;
-                default:
-                    return fail(LQ4_E_INVALID, "chain step %u: unknown prologue %d", j, st.prologue);
-            }
+            if (st.x_dev || st.delta)
+                return fail(LQ4_E_INVALID, "chain step %u: from_previous puts the previous result in the place of x_dev / delta; leave both null", j);
+        } else if (st.prologue == LQ4_PRO_NONE || st.prologue == LQ4_PRO_SILU_MUL) {
+            if (!st.x_dev || misaligned(st.x_dev, 16)) return fail(LQ4_E_INVALID, "chain step %u: x must be non-null and 16-byte aligned", j);
         }
-        if (st.prologue == LQ4_PRO_ADD_RMSNORM && (!st.gamma || misaligned(st.gamma, 16)))
-            return fail(LQ4_E_INVALID, "chain step %u: gamma must be non-null and 16-byte aligned", j);
+        switch (st.prologue) {
+            case LQ4_PRO_NONE:
+            case LQ4_PRO_SILU_MUL:
+                break;
+            case LQ4_PRO_ADD_RMSNORM: {
+                if (!st.gamma || misaligned(st.gamma, 16)) return fail(LQ4_E_INVALID, "chain step %u: gamma must be non-null and 16-byte aligned", j);
+                if (!st.from_previous && !st.base) return fail(LQ4_E_INVALID, "chain step %u: base is null", j);
+                if (misaligned(st.base, 16) || misaligned(st.delta, 16) || misaligned(st.residual_out, 16))
+                    return fail(LQ4_E_INVALID, "chain step %u: base, delta and residual_out must be 16-byte aligned", j);
+                const size_t kb = static_cast<size_t>(st.k) * 4;
+                if (st.residual_out && ((st.base && ranges_overlap(st.residual_out, st.base, kb)) ||
+                                        (st.delta && ranges_overlap(st.residual_out, st.delta, kb))))
+                    return fail(LQ4_E_INVALID, "chain step %u: residual_out must not overlap base or delta", j);
+                break;
+            }
+            default:
+                return fail(LQ4_E_INVALID, "chain step %u: unknown prologue %d", j, st.prologue);
+        }
         switch (st.epilogue) {
             case LQ4_EPI_NONE:
                 break;
@@ -860,28 +856,36 @@ int chain_validate(const lq4_chain_step* steps, uint32_t n_steps) {
     return LQ4_OK;
 }
 
-// Byte offset of every step's result vector in the chain scratch (8 bytes per value) and the total.
-size_t chain_scratch_layout(const lq4_chain_step* steps, uint32_t n_steps, size_t (&off)[kMaxChainSteps]) {
-    size_t total = 0;
+// Byte offsets, in the chain scratch, of every step's result vector and of the residual stream its
+// prologue forms (8 bytes per value), and the total.
+struct ChainLayout {
+    size_t result[kMaxChainSteps], resid[kMaxChainSteps], total;
+};
+ChainLayout chain_scratch_layout(const lq4_chain_step* steps, uint32_t n_steps) {
+    ChainLayout l;
+    l.total = 0;
     for (uint32_t j = 0; j < n_steps; ++j) {
-        off[j] = total;
-        total += up256(static_cast<size_t>(steps[j].n) * 8);  // n, not n/2: the per-step path keeps W . x here too
+        l.result[j] = l.total;
+        l.total += up256(static_cast<size_t>(steps[j].n) * 8);  // n, not n/2: the per-step path keeps W . x here too
+        l.resid[j] = l.total;
+        if (steps[j].prologue == LQ4_PRO_ADD_RMSNORM) l.total += up256(static_cast<size_t>(steps[j].k) * 8);
     }
-    return total;
+    return l;
 }
 
 // Fills the device descriptors of the persistent launch; false = the chain is not eligible for it
-// (a step too large for the register slots or for LDS, or a vector that an earlier step of the same
-// chain writes and that cannot be taken from that step's tagged result).
-bool chain_plan(lq4_ctx* ctx, const lq4_chain_step* steps, uint32_t n_steps, const size_t (&off)[kMaxChainSteps],
-                ChainArgs* args, uint32_t* k_max) {
+// (a K too long for LDS, or a vector that an earlier step of the same chain writes and that cannot be
+// taken from that step's tagged copy).
+bool chain_plan(lq4_ctx* ctx, const lq4_chain_step* steps, uint32_t n_steps, const ChainLayout& lay, ChainArgs* args,
+                uint32_t* k_max) {
     *k_max = 0;
     std::memset(args, 0, sizeof *args);
     args->n_steps = n_steps;
     args->spin_limit = ctx->chain_spin_limit;
     args->epoch = ctx->chain_sync;
     args->fail = ctx->chain_sync + 64;
-    auto tagged = [&](uint32_t i) { return reinterpret_cast<unsigned long long*>(ctx->chain_scratch + off[i]); };
+    args->idle = reinterpret_cast<const uint8_t*>(ctx->chain_sync + 128);  // 16 KB behind the 512 bytes of words
+    auto words = [&](size_t off) { return reinterpret_cast<unsigned long long*>(ctx->chain_scratch + off); };
     for (uint32_t j = 0; j < n_steps; ++j) {
         const lq4_chain_step& st = steps[j];
         ChainStep& d = args->s[j];
@@ -890,58 +894,63 @@ bool chain_plan(lq4_ctx* ctx, const lq4_chain_step* steps, uint32_t n_steps, con
         (void)resolve_weight(st.w, st.w_extra_offset, st.n, st.k, &d.w);
         d.n = st.n;
         d.k = st.k;
-        d.prologue = st.prologue;
-        d.epilogue = st.epilogue;
+        d.flags = static_cast<uint32_t>(st.prologue) | (static_cast<uint32_t>(st.epilogue) << 8);
         d.gamma = st.gamma;
         d.eps = st.eps;
         d.y = st.y_dev;
-        // Which earlier step, if any, wrote vector p for the caller?  Its memory is not coherent
-        // inside the launch; only that step's tagged result is.
-        auto writer_of = [&](const void* p) -> int {
-            if (!p) return -1;
-            for (int i = static_cast<int>(j) - 1; i >= 0; --i)
-                if (steps[i].y_dev == p || (steps[i].epilogue == LQ4_EPI_ADD_RESIDUAL && steps[i].residual == p) ||
-                    steps[i].residual_out == p)
-                    return i;
-            return -1;
+        // An input vector that an earlier step of this chain wrote for the caller is not coherent
+        // inside the launch; that step's tagged copy is.  Sets *tagged (and makes the writer keep the
+        // copy) or *plain; false if the writer has no usable copy.
+        auto source = [&](const float* p, const float** plain, const unsigned long long** tagged) -> bool {
+            *plain = nullptr;
+            *tagged = nullptr;
+            if (!p) return true;
+            for (int i = static_cast<int>(j) - 1; i >= 0; --i) {
+                if (chain_result_ptr(steps[i]) == p) {
+                    args->s[i].out_tagged = words(lay.result[i]);
+                    *tagged = args->s[i].out_tagged;
+                    return true;
+                }
+                if (steps[i].prologue == LQ4_PRO_ADD_RMSNORM && steps[i].residual_out == p) {
+                    args->s[i].resid_out_tagged = words(lay.resid[i]);
+                    *tagged = args->s[i].resid_out_tagged;
+                    return true;
+                }
+                if (steps[i].y_dev == p || steps[i].residual == p) return false;  // written, but not as a whole result
+            }
+            *plain = p;
+            return true;
         };
-        if (chain_reads_previous(st)) {
-            d.x_tagged = tagged(j - 1);
-            args->s[j - 1].out_tagged = tagged(j - 1);
+        if (st.from_previous) {
+            args->s[j - 1].out_tagged = words(lay.result[j - 1]);
+            d.x_tagged = args->s[j - 1].out_tagged;
         } else {
-            if (writer_of(st.x_dev) >= 0 || writer_of(st.base) >= 0 || writer_of(st.delta) >= 0) return false;
-            d.x = st.x_dev;
-            d.base = st.base;
-            d.delta = st.delta;
-            d.residual_out = st.residual_out;
+            const float* b_src = st.prologue == LQ4_PRO_ADD_RMSNORM ? st.delta : st.x_dev;
+            if (!source(b_src, &d.x, &d.x_tagged)) return false;
+            if (st.prologue == LQ4_PRO_SILU_MUL && d.x_tagged) return false;  // gate | up must be external
+        }
+        if (st.prologue == LQ4_PRO_ADD_RMSNORM) {
+            if (!source(st.base, &d.base, &d.base_tagged)) return false;
+            d.resid_out = st.residual_out;
         }
         if (st.epilogue == LQ4_EPI_ADD_RESIDUAL) {
+            const float* plain;
+            const unsigned long long* tagged;
+            // the ring requests a row's residual word far ahead of the row: it must come from outside the chain
+            if (!source(st.residual, &plain, &tagged) || tagged) return false;
+            d.res_plain = st.residual;
             d.res_out = st.residual;
-            const int i = writer_of(st.residual);
-            if (i < 0) {
-                d.res_plain = st.residual;
-            } else {
-                // readable from step i's tagged result once a later hand-over has completed, i.e. from
-                // two steps on; and only if that result is what was stored there
-                if (i + 1 >= static_cast<int>(j) || chain_result_ptr(steps[i]) != st.residual) return false;
-                d.res_tagged = tagged(static_cast<uint32_t>(i));
-                args->s[i].out_tagged = tagged(static_cast<uint32_t>(i));
-            }
         }
-        if (!gemv_chain_plan_step(d, ctx->cu_count)) return false;
+        gemv_chain_plan_step(d);
     }
     return gemv_chain_lds_bytes(*k_max) <= 160 * 1024;
 }
 
 }  // namespace
 
-#ifdef LQ4_CHAIN_TRACE
-static unsigned long long* g_chain_trace = nullptr;
-int lq4_debug_chain_trace(void* buf) { g_chain_trace = static_cast<unsigned long long*>(buf); return 0; }
-#endif
-
 int lq4_set_chain_mode(int mode) {
-    if (mode < 0 || mode > 1) return fail(LQ4_E_INVALID, "chain mode must be 0 (one launch where eligible) or 1 (step by step)");
+    if (mode != LQ4_CHAIN_STEPWISE && mode != LQ4_CHAIN_ONE_LAUNCH)
+        return fail(LQ4_E_INVALID, "chain mode must be LQ4_CHAIN_STEPWISE (0) or LQ4_CHAIN_ONE_LAUNCH (1)");
     g_chain_mode = mode;
     return LQ4_OK;
 }
@@ -955,17 +964,13 @@ int lq4_gemv_chain(lq4_ctx* ctx, const lq4_chain_step* steps, uint32_t n_steps, 
     if (rc) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
     DeviceGuard g(ctx->device);
-    size_t off[kMaxChainSteps];
-    const size_t total = chain_scratch_layout(steps, n_steps, off);
-    rc = grow_scratch(ctx, &ctx->chain_scratch, &ctx->chain_scratch_bytes, total, s, true);
+    const ChainLayout lay = chain_scratch_layout(steps, n_steps);
+    rc = grow_scratch(ctx, &ctx->chain_scratch, &ctx->chain_scratch_bytes, lay.total, s, true);
     if (rc) return rc;
 
     ChainArgs args;
     uint32_t k_max = 0;
-    if (g_chain_mode == 0 && chain_plan(ctx, steps, n_steps, off, &args, &k_max)) {
-#ifdef LQ4_CHAIN_TRACE
-        args.trace = g_chain_trace;
-#endif
+    if (g_chain_mode == LQ4_CHAIN_ONE_LAUNCH && chain_plan(ctx, steps, n_steps, lay, &args, &k_max)) {
         const hipError_t e = launch_gemv_chain(args, ctx->cu_count, k_max, s);
         if (e != hipSuccess) return fail(LQ4_E_HIP, "chain launch: %s", hipGetErrorString(e));
         ctx->chain_unchecked = true;
@@ -978,20 +983,20 @@ int lq4_gemv_chain(lq4_ctx* ctx, const lq4_chain_step* steps, uint32_t n_steps, 
     const float* prev = nullptr;
     for (uint32_t j = 0; j < n_steps; ++j) {
         const lq4_chain_step& st = steps[j];
-        float* spare = reinterpret_cast<float*>(ctx->chain_scratch + off[j]);
+        float* spare = reinterpret_cast<float*>(ctx->chain_scratch + lay.result[j]);
         lq4_gemv_fusion f;
         std::memset(&f, 0, sizeof f);
         const float* x = st.x_dev;
         f.prologue = st.prologue;
         f.gamma = st.gamma;
         f.eps = st.eps;
-        if (chain_reads_previous(st)) {
-            if (st.prologue == LQ4_PRO_ADD_RMSNORM) f.base = prev;
-            else x = prev;
-        } else {
-            f.base = st.base;
-            f.delta = st.delta;
-            f.residual_out = st.residual_out;
+        f.base = st.base;
+        f.delta = st.delta;
+        f.residual_out = st.residual_out;
+        if (st.from_previous) {
+            if (st.prologue != LQ4_PRO_ADD_RMSNORM) x = prev;
+            else if (st.base) f.delta = prev;
+            else f.base = prev;
         }
         float* result;
         if (st.epilogue == LQ4_EPI_ADD_RESIDUAL) {

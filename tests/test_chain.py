@@ -15,6 +15,16 @@ from util import REL_TOL, rel_err
 EPS = 1e-6
 
 
+@pytest.fixture(autouse=True)
+def _one_launch_mode():
+    """The tests below are about the persistent launch; the library's default is one launch per step."""
+    from lattice_amd import backend
+    lib = backend.load_library()
+    lib.lq4_set_chain_mode(backend.CHAIN_ONE_LAUNCH)
+    yield
+    lib.lq4_set_chain_mode(backend.CHAIN_STEPWISE)
+
+
 def _oracle_layer(x_attn, r0, g1, g2, w_o, w_gu, w_down, w_qkv, hidden, inter, qkv_rows):
     """o(+residual) -> norm -> gate||up -> silu*up -> down(+residual) -> norm -> qkv, step by step."""
     y_o = oracle.gemm_f32(x_attn[None, :], w_o, hidden, hidden)[0]
@@ -42,21 +52,27 @@ def _layer_inputs(hidden, inter, qkv_rows, seed):
     return w, x_attn, r0, g1, g2
 
 
+def _layer_steps(be, qw, xd, r0d, r1d, r2d, g1d, g2d, hidden, inter, qkv_rows, qkv, h=None):
+    return [
+        be.chain_step(qw["o"], hidden, hidden, x=xd),
+        be.chain_step(qw["gu"], 2 * inter, hidden, from_previous=True, norm=(r0d, None, g1d, EPS, r1d),
+                      silu_mul_pairs=True, y=h),
+        be.chain_step(qw["down"], hidden, inter, from_previous=True),
+        be.chain_step(qw["qkv"], qkv_rows, hidden, from_previous=True, norm=(r1d, None, g2d, EPS, r2d), y=qkv),
+    ]
+
+
 def _run_layer_chain(be, qw, x_attn, r0, g1, g2, hidden, inter, qkv_rows, want_h=False):
     import torch
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
-    xd, rd, g1d, g2d = dev(x_attn), dev(r0), dev(g1), dev(g2)
+    xd, r0d, g1d, g2d = dev(x_attn), dev(r0), dev(g1), dev(g2)
+    r1d, r2d = (torch.full((hidden,), float("nan"), dtype=torch.float32, device="cuda") for _ in range(2))
     qkv = torch.full((qkv_rows,), float("nan"), dtype=torch.float32, device="cuda")
     h = torch.full((inter,), float("nan"), dtype=torch.float32, device="cuda") if want_h else None
-    steps = [
-        be.chain_step(qw["o"], hidden, hidden, x=xd, add_residual=rd),
-        be.chain_step(qw["gu"], 2 * inter, hidden, norm=(None, None, g1d, EPS, None), silu_mul_pairs=True, y=h),
-        be.chain_step(qw["down"], hidden, inter, add_residual=rd),
-        be.chain_step(qw["qkv"], qkv_rows, hidden, norm=(None, None, g2d, EPS, None), y=qkv),
-    ]
-    be.dispatch_chain(steps)
+    be.dispatch_chain(_layer_steps(be, qw, xd, r0d, r1d, r2d, g1d, g2d, hidden, inter, qkv_rows, qkv, h))
     be.synchronize()
-    return rd.cpu().numpy(), qkv.cpu().numpy(), (h.cpu().numpy() if want_h else None)
+    assert np.array_equal(r0d.cpu().numpy(), r0), "the incoming residual stream must stay untouched"
+    return r2d.cpu().numpy(), qkv.cpu().numpy(), (h.cpu().numpy() if want_h else None), r1d.cpu().numpy()
 
 
 @pytest.mark.gpu
@@ -66,11 +82,12 @@ def test_decode_layer_chain_matches_oracle_sequence(hidden, inter, qkv_rows):
     be = backend.HipQ4Backend(0)
     w, x_attn, r0, g1, g2 = _layer_inputs(hidden, inter, qkv_rows, seed=3)
     qw = {k: be.upload_q4_blocks(v) for k, v in w.items()}
-    _, want_h, want_r2, want_qkv = _oracle_layer(x_attn, r0, g1, g2, w["o"], w["gu"], w["down"], w["qkv"], hidden, inter, qkv_rows)
+    want_r1, want_h, want_r2, want_qkv = _oracle_layer(x_attn, r0, g1, g2, w["o"], w["gu"], w["down"], w["qkv"], hidden, inter, qkv_rows)
 
     before = be.path_counters()["gemv_chain"]
-    got_r, got_qkv, got_h = _run_layer_chain(be, qw, x_attn, r0, g1, g2, hidden, inter, qkv_rows, want_h=True)
+    got_r, got_qkv, got_h, got_r1 = _run_layer_chain(be, qw, x_attn, r0, g1, g2, hidden, inter, qkv_rows, want_h=True)
     assert be.path_counters()["gemv_chain"] == before + 1, "the persistent launch did not serve this chain"
+    assert rel_err(got_r1, want_r1) <= 2e-5
     assert rel_err(got_h, want_h) <= REL_TOL
     assert rel_err(got_r, want_r2) <= REL_TOL
     assert rel_err(got_qkv, want_qkv) <= REL_TOL
@@ -79,11 +96,11 @@ def test_decode_layer_chain_matches_oracle_sequence(hidden, inter, qkv_rows):
 
     # the same chain step by step through the library: equal to f32 rounding (the sum of squares and
     # silu are formed differently)
-    be.set_chain_mode(1)
+    be.set_chain_mode(backend.CHAIN_STEPWISE)
     try:
-        ref_r, ref_qkv, ref_h = _run_layer_chain(be, qw, x_attn, r0, g1, g2, hidden, inter, qkv_rows, want_h=True)
+        ref_r, ref_qkv, ref_h, _ = _run_layer_chain(be, qw, x_attn, r0, g1, g2, hidden, inter, qkv_rows, want_h=True)
     finally:
-        be.set_chain_mode(0)
+        be.set_chain_mode(backend.CHAIN_ONE_LAUNCH)
     assert be.path_counters()["gemv_chain"] == before + 1
     assert rel_err(got_r, ref_r) <= 1e-5 and rel_err(got_qkv, ref_qkv) <= 1e-5 and rel_err(got_h, ref_h) <= 1e-5
     be.close()
@@ -125,7 +142,7 @@ def test_chain_of_independent_steps_and_external_prologues():
 
 
 @pytest.mark.gpu
-def test_chain_replays_in_a_graph_and_large_steps_fall_back():
+def test_chain_replays_in_a_graph_and_other_routes():
     import torch
     from lattice_amd import backend
     be = backend.HipQ4Backend(0)
@@ -133,46 +150,60 @@ def test_chain_replays_in_a_graph_and_large_steps_fall_back():
     w, x_attn, r0, g1, g2 = _layer_inputs(hidden, inter, qkv_rows, seed=9)
     qw = {k: be.upload_q4_blocks(v) for k, v in w.items()}
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
-    xd, rd, g1d, g2d = dev(x_attn), dev(r0), dev(g1), dev(g2)
+    xd, r0d, g1d, g2d = dev(x_attn), dev(r0), dev(g1), dev(g2)
+    r1d, r2d = torch.zeros(hidden, device="cuda"), torch.zeros(hidden, device="cuda")
     qkv = torch.zeros(qkv_rows, dtype=torch.float32, device="cuda")
-    steps = [
-        be.chain_step(qw["o"], hidden, hidden, x=xd, add_residual=rd),
-        be.chain_step(qw["gu"], 2 * inter, hidden, norm=(None, None, g1d, EPS, None), silu_mul_pairs=True),
-        be.chain_step(qw["down"], hidden, inter, add_residual=rd),
-        be.chain_step(qw["qkv"], qkv_rows, hidden, norm=(None, None, g2d, EPS, None), y=qkv),
-    ]
+    steps = _layer_steps(be, qw, xd, r0d, r1d, r2d, g1d, g2d, hidden, inter, qkv_rows, qkv)
     be.dispatch_chain(steps)  # warm: the scratch exists before the capture
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         be.dispatch_chain(steps)
-    # every replay works on the residual the previous one left: follow it with the oracle
-    rd.copy_(dev(r0))
-    torch.cuda.synchronize()
+    # every replay continues from the residual stream the previous one produced
     r_host = r0
     for rep in range(4):
+        r0d.copy_(dev(r_host))
         graph.replay()
         torch.cuda.synchronize()
         _, _, want_r2, want_qkv = _oracle_layer(x_attn, r_host, g1, g2, w["o"], w["gu"], w["down"], w["qkv"], hidden, inter, qkv_rows)
-        assert rel_err(rd.cpu().numpy(), want_r2) <= 2e-5, rep
+        assert rel_err(r2d.cpu().numpy(), want_r2) <= 2e-5, rep
         assert rel_err(qkv.cpu().numpy(), want_qkv) <= 2e-5, rep
-        r_host = rd.cpu().numpy()
+        r_host = r2d.cpu().numpy()
         # eager work of the same library between the replays
         y = torch.empty((1, hidden), dtype=torch.float32, device="cuda")
         be.dispatch_matmul(xd, qw["o"], y, 1, hidden, hidden)
         be.synchronize()
 
-    # a step beyond the register slots of the resident grid: served step by step, same contract
-    n_big, k_big = 14000, 2048
-    wb = synth.q4_weight(n_big, k_big, seed=10)
-    qb = be.upload_q4_blocks(wb)
+    # a tall step (many slots a wave), a residual added as the result is stored, and a later step that
+    # names an earlier step's y as its x: all one launch
+    n_big, k_big, n_tail = 8160, 2048, 96
+    wb, wt = synth.q4_weight(n_big, k_big, seed=10), synth.q4_weight(n_tail, n_big, seed=11)
+    qb, qt = be.upload_q4_blocks(wb), be.upload_q4_blocks(wt)
     xb = synth.activations(1, k_big, seed=10)[0]
+    res = synth.activations(1, n_big, seed=12)[0]
     yb = torch.empty(n_big, dtype=torch.float32, device="cuda")
+    resd = dev(res)
+    yt = torch.empty(n_tail, dtype=torch.float32, device="cuda")
     before = be.path_counters()["gemv_chain"]
-    be.dispatch_chain([be.chain_step(qb, n_big, k_big, x=dev(xb), y=yb)])
+    be.dispatch_chain([be.chain_step(qb, n_big, k_big, x=dev(xb), add_residual=resd, y=yb),
+                       be.chain_step(qt, n_tail, n_big, x=yb, y=yt)])
+    be.synchronize()
+    assert be.path_counters()["gemv_chain"] == before + 1
+    want_b = oracle.add_and_copy(oracle.gemm_f32(xb[None, :], wb, n_big, k_big)[0], res)[0]
+    assert rel_err(yb.cpu().numpy(), want_b) <= 2e-5 and np.array_equal(yb.cpu().numpy(), resd.cpu().numpy())
+    assert rel_err(yt.cpu().numpy(), oracle.gemm_f32(want_b[None, :], wt, n_tail, n_big)[0]) <= 2e-5
+
+    # K beyond what a workgroup stages: served step by step, same contract
+    n_l, k_l = 48, 17408
+    wl = synth.q4_weight(n_l, k_l, seed=13)
+    ql = be.upload_q4_blocks(wl)
+    xl = synth.activations(1, k_l, seed=13)[0]
+    yl = torch.empty(n_l, dtype=torch.float32, device="cuda")
+    before = be.path_counters()["gemv_chain"]
+    be.dispatch_chain([be.chain_step(ql, n_l, k_l, x=dev(xl), y=yl)])
     be.synchronize()
     assert be.path_counters()["gemv_chain"] == before
-    assert rel_err(yb.cpu().numpy(), oracle.gemm_f32(xb[None, :], wb, n_big, k_big)[0]) <= 2e-5
+    assert rel_err(yl.cpu().numpy(), oracle.gemm_f32(xl[None, :], wl, n_l, k_l)[0]) <= 2e-5
     be.close()
 
 
@@ -186,11 +217,11 @@ def test_chain_contract_errors_and_bounded_wait():
     x = torch.zeros(k, dtype=torch.float32, device="cuda")
     y = torch.zeros(n, dtype=torch.float32, device="cuda")
     with pytest.raises(backend.Q4Error, match="step 0 needs external"):
-        be.dispatch_chain([be.chain_step(qw, n, k, y=y)])
+        be.dispatch_chain([be.chain_step(qw, n, k, from_previous=True, y=y)])
     with pytest.raises(backend.Q4Error, match="nowhere to put its result"):
         be.dispatch_chain([be.chain_step(qw, n, k, x=x)])
     with pytest.raises(backend.Q4Error, match="previous step yields"):
-        be.dispatch_chain([be.chain_step(qw, n, k, x=x, silu_mul_pairs=True), be.chain_step(qw, n, k, y=y)])
+        be.dispatch_chain([be.chain_step(qw, n, k, x=x, silu_mul_pairs=True), be.chain_step(qw, n, k, from_previous=True, y=y)])
     with pytest.raises(backend.Q4Error, match="at most 16"):
         be.dispatch_chain([be.chain_step(qw, n, k, x=x, y=y)] * 17)
     be.dispatch_chain([])  # no-op
@@ -207,17 +238,17 @@ def test_chain_contract_errors_and_bounded_wait():
     wq = synth.q4_weight(n, k, seed=0)
     xh = synth.activations(1, k, seed=0)[0]
     xd = torch.from_numpy(xh).cuda()
-    steps = [be2.chain_step(qw, n, k, x=xd), be2.chain_step(qw, n, k, y=y)]
+    steps = [be2.chain_step(qw, n, k, x=xd), be2.chain_step(qw, n, k, from_previous=True, y=y)]
     be2.dispatch_chain(steps)
     with pytest.raises(backend.Q4Error, match="never arrived"):
         be2.synchronize()
     be2.synchronize()  # reported once
-    be2.set_chain_mode(1)
+    be2.set_chain_mode(backend.CHAIN_STEPWISE)
     try:
         be2.dispatch_chain(steps)
         be2.synchronize()
     finally:
-        be2.set_chain_mode(0)
+        be2.set_chain_mode(backend.CHAIN_ONE_LAUNCH)
     y1 = oracle.gemm_f32(xh[None, :], wq, n, k)
     assert rel_err(y.cpu().numpy(), oracle.gemm_f32(y1, wq, n, k)[0]) <= 2e-5
     be2.close()

@@ -175,6 +175,19 @@ int lq4_lm_head_topk(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset,
                      const float* x_dev, uint32_t top_k, float* out_logits_dev, uint32_t* out_ids_dev,
                      void* stream);
 
+/* lq4_lm_head_topk for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid it).  No counterpart in the reference.  Same
+ * arguments, same result bit for bit; the logits and the candidate buffers live in a fixed
+ * LQ4_STATIC_SCRATCH_BYTES array inside the library's device code instead of the context's growable
+ * scratch, so the call makes no hipMalloc / hipFree and calls no allocating routine.  Shapes whose
+ * scratch (vocab * 4 bytes, rounded up to 256, plus the selection's candidate buffers) does not fit
+ * return LQ4_E_UNSUPPORTED: vocabularies up to 262 144 with top_k <= 256 fit.  Every context on one
+ * GPU shares that GPU's array: calls that overlap on one GPU (two streams, two contexts) race. */
+#define LQ4_STATIC_SCRATCH_BYTES (2u << 20)
+int lq4_lm_head_topk_static(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t vocab, uint32_t k,
+                            const float* x_dev, uint32_t top_k, float* out_logits_dev, uint32_t* out_ids_dev,
+                            void* stream);
+
 /* ---- elementwise steps either side of the decode GEMVs ---------------------------
  * Shifted RMSNorm of Qwen3.5 with the residual add in front of it: v = base + delta (delta may be
  * NULL: plain norm), residual_out = v (skipped if NULL), normed_out = v * rsqrt(mean(v^2) + eps) *

@@ -51,6 +51,7 @@ EXPORTS = [
     "lq4_probe_copy",
     "lq4_set_gemm_kernel",
     "lq4_residual_add_rmsnorm", "lq4_silu_mul", "lq4_add_and_copy", "lq4_gemv_fused",
+    "lq4_lm_head_topk_static",
     "lq4_gemv_chain", "lq4_set_chain_mode", "lq4_ctx_reserve_scratch",
     "lq4_gemv_q8", "lq4_gemm_q8", "lq4_gemv_q3", "lq4_gemm_q3",
     "lq4_get_path_counters", "lq4_malloc", "lq4_free", "lq4_memcpy_h2d", "lq4_memcpy_d2h",
@@ -133,6 +134,7 @@ def load_library() -> C.CDLL:
         "lq4_dequant": (C.c_int, [vp, vp, u64, u32, u32, vp, vp]),
         "lq4_topk": (C.c_int, [vp, vp, C.c_uint32, C.c_uint32, vp, vp, vp]),
         "lq4_lm_head_topk": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, C.c_uint32, vp, vp, vp]),
+        "lq4_lm_head_topk_static": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, C.c_uint32, vp, vp, vp]),
         "lq4_probe_read": (C.c_int, [vp, vp, C.c_size_t, vp]),
         "lq4_probe_copy": (C.c_int, [vp, vp, vp, C.c_size_t, vp]),
         "lq4_set_gemm_kernel": (C.c_int, [C.c_int]),

@@ -19,6 +19,7 @@ using namespace lq4;
 struct lq4_ctx {
     int device;
     float* lora_t;        // [kLoraTRows, kMaxLoraRank] f32: A.x of the call in flight
+    uint8_t* static_scratch;  // this device's copy of `scratch` below (lq4_lm_head_topk_static)
     uint8_t* moe_scratch; // grown on demand
     uint32_t* topk_ticket; // finished-workgroup count of the top-k kernel, zero between launches
     uint32_t* lora_sync;   // epoch, producer count and slots of the batch-1 GEMV that computes A.x itself (same allocation)
@@ -161,6 +162,13 @@ extern "C" {
 const char* lq4_last_error(void) { return g_err; }
 const char* lq4_version(void) { return "lattice-hip-q4 0.1 (gfx950)"; }
 
+// Scratch of lq4_lm_head_topk_static, in the code object's own data so that entry point never
+// allocates: the logits of one lm_head pass, then the top-k candidate buffers.  Every GPU the
+// library runs on holds one copy until the process ends; host code reaches it only through the
+// address hipGetSymbolAddress returns for the current device (kept in the context).
+constexpr size_t kStaticScratchBytes = LQ4_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 int lq4_ctx_create(int device_ordinal, lq4_ctx** out) {
     if (!out) return fail(LQ4_E_INVALID, "out is null");
     *out = nullptr;
@@ -188,6 +196,13 @@ int lq4_ctx_create(int device_ordinal, lq4_ctx** out) {
         (void)hipFree(c->lora_t);
         delete c;
         return fail(LQ4_E_HIP, "hipMalloc(top-k ticket): %s", hipGetErrorString(e));
+    }
+    e = hipGetSymbolAddress(reinterpret_cast<void**>(&c->static_scratch), HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !c->static_scratch) {
+        (void)hipFree(c->topk_ticket);
+        (void)hipFree(c->lora_t);
+        delete c;
+        return fail(LQ4_E_HIP, "hipGetSymbolAddress(static scratch): %s", hipGetErrorString(e));
     }
     c->lora_sync = c->topk_ticket + 64;
     hipDeviceProp_t prop;
@@ -633,6 +648,37 @@ int lq4_lm_head_topk(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset,
     const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};
     launch_gemv(wp, vocab, k, x_dev, k, 1, logits, vocab, none, s);
     launch_topk(logits, vocab, top_k, ctx->moe_scratch + logits_bytes, ctx->topk_ticket, out_logits_dev, out_ids_dev, s);
+    ctx->counters.gemv++;
+    ctx->counters.topk++;
+    LQ4_HIP(hipGetLastError());
+    return LQ4_OK;
+}
+
+int lq4_lm_head_topk_static(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t vocab, uint32_t k,
+                            const float* x_dev, uint32_t top_k, float* out_logits_dev, uint32_t* out_ids_dev,
+                            void* stream) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    if (top_k == 0) return LQ4_OK;
+    if (vocab == 0) return fail(LQ4_E_INVALID, "empty vocabulary");
+    if (top_k > LQ4_MAX_TOP_K) return fail(LQ4_E_INVALID, "top_k %u above %d", top_k, LQ4_MAX_TOP_K);
+    const uint8_t* wp;
+    const int rc = resolve_weight(w, w_extra_offset, vocab, k, &wp);
+    if (rc) return rc;
+    if (!x_dev || !out_logits_dev || !out_ids_dev) return fail(LQ4_E_INVALID, "null device pointer");
+    if (reinterpret_cast<uintptr_t>(x_dev) % 16) return fail(LQ4_E_INVALID, "x must be 16-byte aligned");
+    // same layout as lq4_lm_head_topk: [vocab logits | candidate buffers], in the static array
+    const size_t logits_bytes = (static_cast<size_t>(vocab) * sizeof(float) + 255) / 256 * 256;
+    const size_t need = logits_bytes + topk_scratch_bytes(vocab, top_k);
+    if (need > kStaticScratchBytes)
+        return fail(LQ4_E_UNSUPPORTED,
+                    "lq4_lm_head_topk_static: vocab %u with top_k %u needs %zu bytes of scratch, the static buffer holds %zu; "
+                    "use lq4_lm_head_topk", vocab, top_k, need, kStaticScratchBytes);
+    DeviceGuard g(ctx->device);
+    float* logits = reinterpret_cast<float*>(ctx->static_scratch);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};
+    launch_gemv(wp, vocab, k, x_dev, k, 1, logits, vocab, none, s);
+    launch_topk(logits, vocab, top_k, ctx->static_scratch + logits_bytes, ctx->topk_ticket, out_logits_dev, out_ids_dev, s);
     ctx->counters.gemv++;
     ctx->counters.topk++;
     LQ4_HIP(hipGetLastError());

@@ -88,29 +88,66 @@ def timed(torch, fn, iters):
     return start.elapsed_time(stop) / iters
 
 
+MIN_TIMED_MS = 20.0  # every graph-timed figure covers at least this much GPU time
+LAST_TIMING = {}
+
+
 def graph_timed(torch, fn, iters, replays=3):
     """Like timed(), but the `iters` calls are captured once into a HIP graph and the graph is
     replayed: the launches reach the GPU back to back, with no per-call host overhead between
-    them.  Returns average milliseconds per call over the last replay."""
+    them.  The graph is replayed at least `replays` times and as often as it takes to cover
+    MIN_TIMED_MS of GPU time, each replay between its own pair of HIP events.  Returns the MEAN
+    milliseconds per call over all timed replays; the minimum and the replay count are left in
+    LAST_TIMING."""
     g = torch.cuda.CUDAGraph()
     torch.cuda.synchronize()
     with torch.cuda.graph(g):
         for i in range(iters):
             fn(i)
     torch.cuda.synchronize()
-    g.replay()
-    best = None
-    for _ in range(replays):
+    g.replay()  # untimed: first replay of a fresh graph
+    per_replay = []
+    while len(per_replay) < replays or (sum(per_replay) < MIN_TIMED_MS and len(per_replay) < 2000):
         start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         start.record()
         g.replay()
         stop.record()
         torch.cuda.synchronize()
-        ms = start.elapsed_time(stop) / iters
-        best = ms if best is None or ms < best else best
+        per_replay.append(start.elapsed_time(stop))
     del g
-    return best
+    LAST_TIMING.clear()
+    LAST_TIMING.update(mean_ms=sum(per_replay) / len(per_replay) / iters, min_ms=min(per_replay) / iters,
+                       replays=len(per_replay), timed_region_ms=sum(per_replay))
+    return LAST_TIMING["mean_ms"]
+
+
+def read_sweep(torch, be):
+    """Read-bandwidth ceiling of this GPU by launch size: the read probe over a 4 GB pool (launch i
+    reads piece i, so nothing is served from a cache), swept over grid, bytes in flight per thread,
+    chunked or interleaved workgroups and plain or non-temporal loads.  Prints a table."""
+    pool_bytes = 4 << 30
+    pool = torch.empty(pool_bytes, dtype=torch.uint8, device="cuda")
+    pool.fill_(1)
+    sizes = [7864320, 30146560, 55705600, 318767104, 1 << 30]
+    print("%-22s %12s %6s %9s %9s" % ("variant", "bytes", "grid", "us", "GB/s"))
+    for sz in sizes:
+        best = None
+        for strided in (False, True):
+            for nt in (False, True):
+                for fl in (64, 128, 256):
+                    for grid in (256, 512, 1024, 2048, 4096, 8192):
+                        nbuf = min(200, pool_bytes // sz)
+                        iters = 12 if sz > (100 << 20) else 100
+                        f = lambda i: be.probe_read_config(pool, sz, grid, fl, strided, nt, offset=(i % nbuf) * sz)
+                        f(0)
+                        ms = graph_timed(torch, f, iters, replays=2)
+                        name = "%s %3dB%s" % ("interleaved" if strided else "chunked", fl, " nt" if nt else "")
+                        print("%-22s %12d %6d %9.2f %9.1f" % (name, sz, grid, ms * 1e3, sz / ms / 1e6), flush=True)
+                        if best is None or ms < best[0]:
+                            best = (ms, name, grid)
+        print("best at %d bytes: %s grid %d: %.2f us = %.1f GB/s" % (sz, best[1], best[2], best[0] * 1e3, sz / best[0] / 1e6),
+              flush=True)
 
 
 def main():
@@ -124,6 +161,8 @@ def main():
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--headline-only", action="store_true",
                     help="run nothing but warmup and the timed headline region (for kernel-trace profiles)")
+    ap.add_argument("--read-sweep", action="store_true",
+                    help="print the read-probe sweep (grid x bytes in flight x access pattern x size) and exit")
     ap.add_argument("--eager", action="store_true",
                     help="launch every step from Python instead of replaying a captured HIP graph")
     args = ap.parse_args()
@@ -136,6 +175,9 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     be = backend.HipQ4Backend(0)
+    if args.read_sweep:
+        read_sweep(torch, be)
+        return
     gen = torch.Generator(device="cuda")
     gen.manual_seed(0)
     B = args.batch
@@ -178,6 +220,7 @@ def main():
         layer_step(i)
     tm = timed if args.eager else graph_timed
     ms_step = tm(torch, layer_step, args.steps)
+    headline_timing = dict(LAST_TIMING) if not args.eager else {}
     if args.headline_only:
         args.skip_extras = args.skip_cpu = True
     eager_ms = ms_step if args.headline_only else timed(torch, layer_step, args.steps)
@@ -213,6 +256,9 @@ def main():
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
         "tokens_per_s_equivalent_24_layers": round(1.0 / (24 * ms_step * 1e-3), 1),
         "launch_mode": "eager launches from Python" if args.eager else "captured HIP graph, replayed",
+        "timing": {"value_is": "mean over replays", "replays": headline_timing.get("replays"),
+                   "timed_region_ms": round(headline_timing.get("timed_region_ms", 0.0), 3),
+                   "ms_per_step_min_over_replays": round(headline_timing.get("min_ms", ms_step), 5)},
         "eager_python_launch": {"ms_per_step": round(eager_ms, 5),
                                 "GB/s": round(step_bytes / (eager_ms * 1e-3) / 1e9, 1)},
         "hot_cache": {"ms_per_step": round(hot_ms, 5),
@@ -318,6 +364,38 @@ def main():
             out["decode_layer_batch8"] = {"ms_per_step": round(ms8, 5), "GB/s": round(b8 / ms8 / 1e6, 1),
                                           "pct_of_hbm_peak": round(100 * b8 / ms8 / 1e6 / HBM_PEAK_GBPS, 2)}
 
+        # The same four matrices as the real dependent chain of a token (o -> +residual, RMSNorm -> gate||up
+        # -> silu*up -> down -> +residual, RMSNorm -> qkv) through lq4_gemv_chain: step by step (the
+        # default: one fused launch per step) and as the one persistent launch.
+        if B == 1:
+            cres, cres1, cres2 = (torch.randn(2048, device="cuda", generator=gen) for _ in range(3))
+            cg1, cg2 = (0.1 * torch.randn(2048, device="cuda", generator=gen) for _ in range(2))
+            cqkv = torch.empty(3072, device="cuda")
+            chains = [[
+                be.chain_step(b["o"], 2048, 2048, x=xs[2048][0]),
+                be.chain_step(b["gate_up"], 12288, 2048, from_previous=True, norm=(cres, None, cg1, 1e-6, cres1),
+                              silu_mul_pairs=True),
+                be.chain_step(b["down"], 2048, 6144, from_previous=True),
+                be.chain_step(b["qkv"], 3072, 2048, from_previous=True, norm=(cres1, None, cg2, 1e-6, cres2), y=cqkv)]
+                for b in layers]
+            cf = lambda i: be.dispatch_chain(chains[i % len(chains)])
+            ch = {}
+            for mode, nm in ((backend.CHAIN_STEPWISE, "stepwise"), (backend.CHAIN_ONE_LAUNCH, "one_launch")):
+                be.set_chain_mode(mode)
+                try:
+                    for i in range(len(layers)):
+                        cf(i)
+                    be.synchronize()
+                    ms_c = tm(torch, cf, max(72, args.steps // 2))
+                    be.synchronize()
+                finally:
+                    be.set_chain_mode(backend.CHAIN_STEPWISE)
+                ch[nm] = {"us_per_step": round(ms_c * 1e3, 3), "GB/s": round(step_bytes / ms_c / 1e6, 1),
+                          "pct_of_hbm_peak": round(100 * step_bytes / ms_c / 1e6 / HBM_PEAK_GBPS, 2)}
+            ch["note"] = ("dependent chain incl. residual adds, RMSNorms and silu*up; the headline's four GEMVs "
+                          "alone are independent launches over the same weights")
+            out["decode_layer_chain"] = ch
+
         # decode MLP with its elementwise neighbours: residual add + RMSNorm, gate||up GEMV, silu*up,
         # down GEMV, add into the residual.  Five launches one by one against two fused launches.
         if B == 1:
@@ -409,6 +487,16 @@ def main():
                                                    "pct_of_f16_mfma_peak": round(100 * tf / MFMA_F16_PEAK_TFLOPS, 2)}
             del qw
         out["prefill_gemm_f16"] = gemm
+        # the GEMM half of the metric as a roofline object of its own: the largest config-2 problem
+        big = gemm["M2048_N17408_K5120"]
+        out["roofline_gemm"] = {
+            "bound": "mfma", "kernel": "gemm_q4 (prefill)", "workload": "BASELINE config 2: M=2048, N=17408, K=5120",
+            "achieved": big["TFLOP/s"], "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(big["TFLOP/s"] / MFMA_F16_PEAK_TFLOPS, 4),
+            "flops_per_launch": 2.0 * 2048 * 17408 * 5120, "avg_launch_us": round(big["ms"] * 1e3, 2),
+            "traffic": None,
+            "other_shapes_frac": {k_: round(v_["TFLOP/s"] / MFMA_F16_PEAK_TFLOPS, 4) for k_, v_ in gemm.items()},
+        }
 
         # the same for the sibling formats (one shape each way), and their few-token kernel at 16 rows
         sib = {}

@@ -342,6 +342,12 @@ int lq4_dequant(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
  * launch size, the figure the GEMV kernels are held against.  No counterpart in the
  * reference. */
 int lq4_probe_read(lq4_ctx* ctx, const void* p_dev, size_t nbytes, void* stream);
+/* The same with the launch spelled out, for sweeps: `workgroups` of 256 threads (0: the library's
+ * choice), 64 / 128 / 256 bytes in flight per thread, workgroups interleaved at 4 KB x (bytes / 16)
+ * granularity (`strided`) or one contiguous chunk each, plain or non-temporal loads.  lq4_probe_read
+ * is (0, 128, strided, non-temporal), the fastest of the sweep from 8 MB to 1 GB. */
+int lq4_probe_read_config(lq4_ctx* ctx, const void* p_dev, size_t nbytes, uint32_t workgroups, uint32_t bytes_in_flight,
+                          int strided, int nontemporal, void* stream);
 
 /* Tuning/test hook, process-wide: 0 = lq4_gemm picks its kernel by shape (default), 1 = always
  * the LDS-staged tile kernel, 2 = always the weights-in-registers kernel, 3 = always the

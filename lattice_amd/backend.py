@@ -48,6 +48,7 @@ EXPORTS = [
     "lq4_topk",
     "lq4_lm_head_topk",
     "lq4_probe_read",
+    "lq4_probe_read_config",
     "lq4_probe_copy",
     "lq4_set_gemm_kernel",
     "lq4_residual_add_rmsnorm", "lq4_silu_mul", "lq4_add_and_copy", "lq4_gemv_fused",
@@ -136,6 +137,7 @@ def load_library() -> C.CDLL:
         "lq4_lm_head_topk": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, C.c_uint32, vp, vp, vp]),
         "lq4_lm_head_topk_static": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, C.c_uint32, vp, vp, vp]),
         "lq4_probe_read": (C.c_int, [vp, vp, C.c_size_t, vp]),
+        "lq4_probe_read_config": (C.c_int, [vp, vp, C.c_size_t, C.c_uint32, C.c_uint32, C.c_int, C.c_int, vp]),
         "lq4_probe_copy": (C.c_int, [vp, vp, vp, C.c_size_t, vp]),
         "lq4_set_gemm_kernel": (C.c_int, [C.c_int]),
         "lq4_residual_add_rmsnorm": (C.c_int, [vp, vp, vp, vp, C.c_uint32, C.c_uint32, C.c_float, vp, vp, vp]),
@@ -259,6 +261,12 @@ class HipQ4Backend:
     def probe_read(self, t):
         """One read-only streaming launch over tensor ``t`` (bandwidth-ceiling calibration)."""
         _check(self.lib.lq4_probe_read(self.ctx, t.data_ptr(), t.numel() * t.element_size(), self._stream()))
+
+    def probe_read_config(self, t, nbytes: int, workgroups: int, bytes_in_flight: int, strided: bool,
+                          nontemporal: bool, offset: int = 0):
+        """The read probe with its launch spelled out, over ``nbytes`` of ``t`` from byte ``offset``."""
+        _check(self.lib.lq4_probe_read_config(self.ctx, t.data_ptr() + offset, nbytes, workgroups, bytes_in_flight,
+                                              int(strided), int(nontemporal), self._stream()))
 
     def set_gemm_kernel(self, which: int):
         """0 = pick the prefill kernel by shape, 1 = LDS-staged tile, 2 = weights in registers,

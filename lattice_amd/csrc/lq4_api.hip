@@ -600,13 +600,22 @@ int lq4_dequant(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
     return LQ4_OK;
 }
 
-int lq4_probe_read(lq4_ctx* ctx, const void* p_dev, size_t nbytes, void* stream) {
+int lq4_probe_read_config(lq4_ctx* ctx, const void* p_dev, size_t nbytes, uint32_t workgroups, uint32_t bytes_in_flight,
+                          int strided, int nontemporal, void* stream) {
     if (!ctx || !p_dev) return fail(LQ4_E_INVALID, "null argument");
     if (reinterpret_cast<uintptr_t>(p_dev) % 16) return fail(LQ4_E_INVALID, "buffer must be 16-byte aligned");
+    if (workgroups > 65536) return fail(LQ4_E_INVALID, "at most 65536 workgroups");
     DeviceGuard g(ctx->device);
-    launch_probe_read(p_dev, nbytes, reinterpret_cast<uint32_t*>(ctx->lora_t), static_cast<hipStream_t>(stream));
+    if (!launch_probe_read(p_dev, nbytes, workgroups, bytes_in_flight, strided != 0, nontemporal != 0,
+                           reinterpret_cast<uint32_t*>(ctx->lora_t), static_cast<hipStream_t>(stream)))
+        return fail(LQ4_E_INVALID, "bytes_in_flight must be 64, 128 or 256, got %u", bytes_in_flight);
     LQ4_HIP(hipGetLastError());
     return LQ4_OK;
+}
+
+int lq4_probe_read(lq4_ctx* ctx, const void* p_dev, size_t nbytes, void* stream) {
+    // the configuration that won the sweep at every size from 8 MB to 1 GB
+    return lq4_probe_read_config(ctx, p_dev, nbytes, 0, 128, 1, 1, stream);
 }
 
 int lq4_topk(lq4_ctx* ctx, const float* logits_dev, uint32_t n, uint32_t top_k, float* out_logits_dev,

@@ -129,20 +129,40 @@ __global__ __launch_bounds__(256) void lora_b_accum_kernel(const void* __restric
 // Calibration kernel: streams `n16` 16-byte words through the vector memory path and does
 // nothing else (the xor keeps the loads alive; the store never fires for real data).  Its
 // duration at a given size is the ceiling any read-only kernel of that size can reach.
-__global__ __launch_bounds__(256) void probe_read_kernel(const uint4* __restrict__ p, size_t n16,
+// D loads of 16 bytes are in flight per thread; STRIDED: consecutive workgroups read consecutive
+// 4 KB * D pieces (otherwise every workgroup owns one contiguous chunk); NT: non-temporal loads.
+typedef uint32_t probe_u32x4 __attribute__((ext_vector_type(4)));
+template <int D, bool NT, bool STRIDED>
+__global__ __launch_bounds__(256) void probe_read_kernel(const probe_u32x4* __restrict__ p, size_t n16,
                                                          uint32_t* __restrict__ sink) {
-    const size_t per_wg = (n16 + gridDim.x - 1) / gridDim.x;
-    const size_t beg = blockIdx.x * per_wg;
-    const size_t end = beg + per_wg < n16 ? beg + per_wg : n16;
     uint32_t acc = 0;
-    size_t i = beg + threadIdx.x;
-    for (; i + 768 < end; i += 1024) {
-        const uint4 a = p[i], b = p[i + 256], c = p[i + 512], d = p[i + 768];
-        acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
+    size_t i, end, step;
+    if (STRIDED) {
+        i = static_cast<size_t>(blockIdx.x) * 256 * D + threadIdx.x;
+        end = n16;
+        step = static_cast<size_t>(gridDim.x) * 256 * D;
+    } else {
+        const size_t per_wg = (n16 + gridDim.x - 1) / gridDim.x;
+        const size_t beg = blockIdx.x * per_wg;
+        i = beg + threadIdx.x;
+        end = beg + per_wg < n16 ? beg + per_wg : n16;
+        step = 256 * D;
     }
-    for (; i < end; i += 256) {
-        const uint4 a = p[i];
-        acc ^= a.x ^ a.y ^ a.z ^ a.w;
+    for (; i + 256 * (D - 1) < end; i += step) {
+        probe_u32x4 r[D];
+#pragma unroll
+        for (int j = 0; j < D; ++j) r[j] = NT ? __builtin_nontemporal_load(p + i + 256 * j) : p[i + 256 * j];
+#pragma unroll
+        for (int j = 0; j < D; ++j) acc ^= r[j].x ^ r[j].y ^ r[j].z ^ r[j].w;
+    }
+    // what the unrolled loop left over: a chunk's tail, or the last partial round of the grid
+    if (STRIDED) {
+        if (i < end) {
+            for (int j = 0; j < D; ++j)
+                if (i + 256 * j < end) { const probe_u32x4 a = p[i + 256 * j]; acc ^= a.x ^ a.y ^ a.z ^ a.w; }
+        }
+    } else {
+        for (; i < end; i += 256) { const probe_u32x4 a = p[i]; acc ^= a.x ^ a.y ^ a.z ^ a.w; }
     }
     if (acc == 0x9E3779B9u && sink) sink[0] = acc;
 }
@@ -240,11 +260,30 @@ void launch_lora_b_accum(const void* b, int b_is_f16, uint32_t rank, uint32_t d_
                        b_is_f16, rank, d_out, t, scale, y, y_stride);
 }
 
-void launch_probe_read(const void* p, size_t nbytes, uint32_t* sink, hipStream_t stream) {
+// in_flight: bytes in flight per thread (64, 128 or 256); grid 0: the library's own choice
+bool launch_probe_read(const void* p, size_t nbytes, uint32_t grid, uint32_t in_flight, bool strided, bool nontemporal,
+                       uint32_t* sink, hipStream_t stream) {
     const size_t n16 = nbytes / 16;
-    uint32_t grid = static_cast<uint32_t>((n16 + 1023) / 1024);
-    grid = grid > 1024 ? 1024 : grid < 1 ? 1 : grid;
-    hipLaunchKernelGGL(probe_read_kernel, dim3(grid), dim3(256), 0, stream, static_cast<const uint4*>(p), n16, sink);
+    if (grid == 0) {
+        grid = static_cast<uint32_t>((n16 + 2047) / 2048);
+        grid = grid > 1024 ? 1024 : grid < 1 ? 1 : grid;
+    }
+    const probe_u32x4* q = static_cast<const probe_u32x4*>(p);
+#define LQ4_PROBE(D_) \
+    do { \
+        if (strided && nontemporal) hipLaunchKernelGGL((probe_read_kernel<D_, true, true>), dim3(grid), dim3(256), 0, stream, q, n16, sink); \
+        else if (strided) hipLaunchKernelGGL((probe_read_kernel<D_, false, true>), dim3(grid), dim3(256), 0, stream, q, n16, sink); \
+        else if (nontemporal) hipLaunchKernelGGL((probe_read_kernel<D_, true, false>), dim3(grid), dim3(256), 0, stream, q, n16, sink); \
+        else hipLaunchKernelGGL((probe_read_kernel<D_, false, false>), dim3(grid), dim3(256), 0, stream, q, n16, sink); \
+    } while (0)
+    switch (in_flight) {
+        case 64: LQ4_PROBE(4); break;
+        case 128: LQ4_PROBE(8); break;
+        case 256: LQ4_PROBE(16); break;
+        default: return false;
+    }
+#undef LQ4_PROBE
+    return true;
 }
 
 void launch_probe_copy(const void* src, void* dst, size_t nbytes, hipStream_t stream) {

@@ -236,7 +236,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
             for (int t = 0; t < SG; ++t) {
                 uint32_t blk = (sgi * SG + t) * 64 + seg_lane;
                 if (blk >= nb) blk = nb - 1;
-                buf[j][t] = *reinterpret_cast<const Q4BlockRaw*>(rp + blk * static_cast<uint32_t>(kBlockBytes));
+                // non-temporal: every block is read once, and a plain load's allocation in the caches
+                // measurably slows the stream (read probe: 4.9 -> 5.15 TB/s at 30 MB, 6.2 -> 6.8 at 318 MB)
+                const uint8_t* bp = rp + blk * static_cast<uint32_t>(kBlockBytes);
+                buf[j][t].sb = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(bp));
+                const u32x4u q = __builtin_nontemporal_load(reinterpret_cast<const u32x4u*>(bp + 4));
+                buf[j][t].q[0] = q.x; buf[j][t].q[1] = q.y; buf[j][t].q[2] = q.z; buf[j][t].q[3] = q.w;
             }
         }
     };

@@ -189,7 +189,8 @@ size_t gemm_skinny_scratch_bytes(uint32_t k, uint32_t m);
 void launch_gemm_skinny(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
                         const LoraEpilogue& lora, void* packed_x, hipStream_t stream, int fmt = 0);
 
-void launch_probe_read(const void* p, size_t nbytes, uint32_t* sink, hipStream_t stream);
+bool launch_probe_read(const void* p, size_t nbytes, uint32_t grid, uint32_t in_flight, bool strided, bool nontemporal,
+                       uint32_t* sink, hipStream_t stream);
 void launch_probe_copy(const void* src, void* dst, size_t nbytes, hipStream_t stream);
 void launch_dequant(const uint8_t* w, uint32_t n, uint32_t k, float* out, hipStream_t stream);
 

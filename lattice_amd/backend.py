@@ -268,6 +268,11 @@ class HipQ4Backend:
         _check(self.lib.lq4_probe_read_config(self.ctx, t.data_ptr() + offset, nbytes, workgroups, bytes_in_flight,
                                               int(strided), int(nontemporal), self._stream()))
 
+    def reserve_scratch(self, nbytes: int):
+        """Grows the context's scratch ahead of time (growing it allocates, which a call under HIP
+        graph capture refuses to do)."""
+        _check(self.lib.lq4_ctx_reserve_scratch(self.ctx, int(nbytes)))
+
     def set_gemm_kernel(self, which: int):
         """0 = pick the prefill kernel by shape, 1 = LDS-staged tile, 2 = weights in registers,
         3 = few-token kernel."""

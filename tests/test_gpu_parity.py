@@ -619,6 +619,7 @@ def test_lora_one_token_a_inside_the_launch(mode):
             qw = b2.upload_q4_blocks(wq)
             b2.load_lora_adapter([backend.LoraLayerData(0, {"p": (a, b)})], scale=2.0)
             before = b2.path_counters()["lora_a"]
+            fallbacks_before = b2.path_counters()["lora_t_fallback"]
             try:
                 y = torch.empty((1, n), dtype=torch.float32, device="cuda")
                 # several calls in a row with different activations: the launch's counters must be
@@ -638,6 +639,14 @@ def test_lora_one_token_a_inside_the_launch(mode):
                 launches = b2.path_counters()["lora_a"] - before
                 b2.unload_lora_adapter()
             assert launches == (3 if mode == "off" else 0), "which path computed A.x"
+            if mode == "wait":
+                # every weight workgroup found A.x in the slots, none had to compute it alone, as long as
+                # the launch is one round of workgroups; a full grid of persistent waves (n = 40 000) may
+                # place a few workgroups late, which then take the fallback (right result, measured
+                # 26 of 3 x 1008 workgroups)
+                fb = b2.path_counters()["lora_t_fallback"] - fallbacks_before
+                print(f"  workgroups that computed A.x alone: {fb}", flush=True)
+                assert fb == 0 if n <= 2048 else fb <= 150
     finally:
         b2.close()
 
@@ -676,3 +685,39 @@ def test_lora_one_token_graph_replays(be):
             assert rel_err(got, _lora_ref(x, wq, n, k, a, b, 2.0)) <= REL_TOL
     finally:
         be.unload_lora_adapter()
+
+
+def test_scratch_growth_is_refused_while_the_stream_is_capturing():
+    # growing library scratch allocates, which a stream under capture cannot do; and a buffer that a
+    # captured launch already holds must stay valid when a later call outgrows it
+    import torch
+    b2 = backend.HipQ4Backend(0)
+    try:
+        vocab, k = 20000, 256
+        qw = b2.upload_q4_blocks(synth.q4_weight(vocab, k, seed=3, tag="cap"))
+        x = dev(synth.activations(1, k, seed=3))
+        out = (torch.empty(8, dtype=torch.float32, device="cuda"), torch.empty(8, dtype=torch.int32, device="cuda"))
+        graph = torch.cuda.CUDAGraph()
+        with pytest.raises(backend.Q4Error, match="capturing"):
+            with torch.cuda.graph(graph):
+                b2.lm_head_topk(x, qw, vocab, k, 8, out=out)  # first use of this size: scratch would grow
+        torch.cuda.synchronize()
+        # reserved ahead of time, the same capture goes through, and its replay survives a later call
+        # that outgrows the scratch (the captured launch keeps the old buffer)
+        b2.reserve_scratch(1 << 20)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            b2.lm_head_topk(x, qw, vocab, k, 8, out=out)
+        graph.replay()
+        torch.cuda.synchronize()
+        want = (host(out[0]).copy(), host(out[1]).copy())
+        big_vocab = 600000
+        qbig = b2.wrap_device_blocks(torch.zeros(big_vocab * (32 // 32) * 20, dtype=torch.uint8, device="cuda"))
+        b2.lm_head_topk(torch.zeros((1, 32), dtype=torch.float32, device="cuda"), qbig, big_vocab, 32, 4)
+        torch.cuda.synchronize()
+        out[0].zero_(); out[1].zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(host(out[0]), want[0]) and np.array_equal(host(out[1]), want[1])
+    finally:
+        b2.close()

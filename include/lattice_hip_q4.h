@@ -351,8 +351,9 @@ int lq4_probe_read_config(lq4_ctx* ctx, const void* p_dev, size_t nbytes, uint32
 
 /* Tuning/test hook, process-wide: 0 = lq4_gemm picks its kernel by shape (default), 1 = always
  * the LDS-staged tile kernel, 2 = always the weights-in-registers kernel, 3 = always the
- * few-token kernel.  Results are identical in contract either way.  No counterpart in the
- * reference. */
+ * few-token kernel, 4 = always the weights-in-registers kernel at two workgroups per CU (Q4 without
+ * LoRA; packs the activations into scratch first).  Results are identical in contract either way.
+ * No counterpart in the reference. */
 int lq4_set_gemm_kernel(int which);
 
 /* Calibration: plain device copy of `nbytes` (both buffers 16-byte aligned, nbytes a multiple

@@ -275,7 +275,7 @@ class HipQ4Backend:
 
     def set_gemm_kernel(self, which: int):
         """0 = pick the prefill kernel by shape, 1 = LDS-staged tile, 2 = weights in registers,
-        3 = few-token kernel."""
+        3 = few-token kernel, 4 = weights in registers at two workgroups per CU."""
         _check(self.lib.lq4_set_gemm_kernel(int(which)))
 
     def probe_copy(self, src, dst):

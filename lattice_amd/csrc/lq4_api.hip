@@ -509,7 +509,7 @@ int lq4_gemm(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
         ctx->counters.lora_a++;
     }
     // shapes with too few tiles run as K slices into scratch partials, summed by a second kernel
-    const size_t scratch_bytes = gemm_scratch_floats(n, k, m, x_dtype == LQ4_F16) * sizeof(float);
+    const size_t scratch_bytes = gemm_scratch_floats(n, k, m, x_dtype == LQ4_F16, ep.rank != 0) * sizeof(float);
     if (scratch_bytes) {
         rc = ensure_scratch(ctx, scratch_bytes, static_cast<hipStream_t>(stream));
         if (rc) return rc;
@@ -1163,7 +1163,7 @@ int lq4_gemv_q3(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
 }
 
 int lq4_set_gemm_kernel(int which) {
-    if (which < 0 || which > 3) return fail(LQ4_E_INVALID, "gemm kernel choice must be 0, 1, 2 or 3");
+    if (which < 0 || which > 4) return fail(LQ4_E_INVALID, "gemm kernel choice must be 0..4");
     set_gemm_kernel_choice(which);
     return LQ4_OK;
 }

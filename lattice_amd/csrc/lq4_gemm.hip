@@ -522,29 +522,33 @@ namespace {
 struct GemmPlan {
     bool wreg;
     bool skinny;
+    bool w2;  // the weights-in-registers tile at two workgroups per CU (activations packed first)
 };
 
-GemmPlan plan_gemm(uint32_t n, uint32_t k, uint32_t m, int x_is_f16) {
+GemmPlan plan_gemm(uint32_t n, uint32_t k, uint32_t m, int x_is_f16, bool with_lora) {
     const int forced = g_gemm_choice.load(std::memory_order_relaxed);
-    if (forced == 3 || (forced == 0 && gemm_skinny_wants(n, k, m))) return {false, true};
-    if (forced == 1 || !gemm_wreg_supports(n, k, m, x_is_f16)) return {false, false};
+    if (forced == 3 || (forced == 0 && gemm_skinny_wants(n, k, m))) return {false, true, false};
+    if (forced == 1 || !gemm_wreg_supports(n, k, m, x_is_f16)) return {false, false, false};
+    if (!with_lora && (forced == 4 || (forced == 0 && gemm_w2_wants(n, k, m)))) return {false, false, true};
     // The weights-in-registers kernel everywhere else: its scheduling cuts a partly filled last round
     // of tiles into K slices, so it no longer needs many tiles to keep the chip busy.
-    return {true, false};
+    return {true, false, false};
 }
 
 }  // namespace
 
-size_t gemm_scratch_floats(uint32_t n, uint32_t k, uint32_t m, int x_is_f16) {
-    const GemmPlan p = plan_gemm(n, k, m, x_is_f16);
+size_t gemm_scratch_floats(uint32_t n, uint32_t k, uint32_t m, int x_is_f16, bool with_lora) {
+    const GemmPlan p = plan_gemm(n, k, m, x_is_f16, with_lora);
     if (p.skinny) return (gemm_skinny_scratch_bytes(k, m) + sizeof(float) - 1) / sizeof(float);
+    if (p.w2) return (gemm_w2_scratch_bytes(n, k, m) + sizeof(float) - 1) / sizeof(float);
     return p.wreg ? gemm_wreg_scratch_floats(n, k, m) : 0;
 }
 
 void launch_gemm(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
                  float* y, const LoraEpilogue& lora, float* scratch, hipStream_t stream) {
-    const GemmPlan p = plan_gemm(n, k, m, x_is_f16);
+    const GemmPlan p = plan_gemm(n, k, m, x_is_f16, lora.rank != 0);
     if (p.skinny) return launch_gemm_skinny(w, n, k, x, x_is_f16, m, y, lora, scratch, stream);
+    if (p.w2) return launch_gemm_w2(w, n, k, x, x_is_f16, m, y, reinterpret_cast<uint8_t*>(scratch), stream);
     if (p.wreg) return launch_gemm_wreg(w, n, k, x, x_is_f16, m, y, lora, scratch, stream);
     if (lora.rank) {
         if (x_is_f16) launch_tile<true, 128, true>(w, n, k, x, m, y, lora, stream);

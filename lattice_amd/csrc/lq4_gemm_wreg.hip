@@ -28,6 +28,7 @@
 #include "lq4_internal.hpp"
 
 #include <type_traits>
+#include <utility>
 
 namespace lq4 {
 
@@ -512,6 +513,290 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
     }
 }
 
+// ---- two workgroups per CU: activations packed ahead of time, loaded straight into LDS ------------
+//
+// The kernel above holds 400 registers per lane (one wave per SIMD), and a wave alone cannot issue
+// matrix-core instructions back to back: its own dequantisation, LDS reads and waits sit between
+// them.  gemm_q4_w2 is the same tile and the same instruction order within 256 registers, so that
+// two workgroups share a CU and one wave's gaps are the other's issue slots.  What makes room:
+//  * the activations arrive already converted to f16, in the dequantiser's pair order and in the
+//    tile order of LDS (pack_x_tiles_kernel, one pass over X per call), so a K step's 32 KB go from
+//    global memory to LDS with eight global_load_lds_dwordx4 per wave: no staging registers, no
+//    permutes and no LDS stores in the loop;
+//  * two rotating weight register sets instead of three: the set of step s is dead once its last
+//    quarter has been dequantised (in the shadow of quarter 2) and is refilled for step s + 2 at the
+//    start of quarter 3.
+// LDS holds a step's activations as [token tile 8][K chunk 16][token 16] units of 16 bytes (8 f16), the
+// order packed X has in memory: the 16 lanes of a lane group read 256 contiguous bytes.
+constexpr int kStepUnits = TM * (TK / 8);  // 16-byte units of activations per K step: 2048 = 32 KB
+
+// dq_op_q4 with scale and bias taken straight from the block's first dword (d in the low half, b in
+// the high half) through the packed fma's operand selectors: no (d, d) / (b, b) registers.
+__device__ __forceinline__ uint32_t pk_fma_sb(half2v t, uint32_t sb) {
+    uint32_t r;
+    asm("v_pk_fma_f16 %0, %1, %2, %2 op_sel:[0,0,1] op_sel_hi:[1,0,1]" : "=v"(r) : "v"(t), "v"(sb));
+    return r;
+}
+__device__ __forceinline__ void dq_op_q4_sb(int op, uint32_t q, uint32_t sb, DqTmp& tmp, U4& out) {
+    if (op < 9) dq_op_q4(op, q, half2v{}, half2v{}, tmp, out);
+    else out.v[op - 9] = pk_fma_sb(tmp.t[op - 9], sb);
+}
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+template <int OFF>
+__device__ __forceinline__ u32x4 lds_read128(uint32_t addr) {
+    u32x4 r;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF) : "memory");
+    return r;
+}
+// Waits until at most N LDS operations of the wave are outstanding; `r` is the register the wait is
+// for, so that no use of it can move ahead of the wait.
+template <int N>
+__device__ __forceinline__ void lds_wait(u32x4& r) {
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(r) : "n"(N));
+}
+// acc += A . B on the matrix cores with the accumulator pinned to the accumulation registers: the
+// 128 accumulators of a wave then never compete with the loop's working set for the 128 ordinary
+// vector registers that two waves per SIMD leave each wave.  Every accumulator is touched once per
+// quarter (32 instructions apart), so no two dependent instructions are back to back.
+__device__ __forceinline__ void mfma_in_place(float4v& c, const U4& a, const u32x4& b) {
+    const u32x4 av = {a.v[0], a.v[1], a.v[2], a.v[3]};
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(av), "v"(b));
+}
+
+template <int... I, typename F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F&&>(f));
+}
+
+typedef __attribute__((address_space(3))) void lds_void_t;
+typedef __attribute__((address_space(1))) const void global_void_t;
+
+// X [m, k] (f16 or f32, row-major) -> f16 units [token tile][K chunk of 8][token in tile 16][8], the 8
+// in the order x0 x4 x1 x5 x2 x6 x3 x7; token tiles up to a multiple of 8 and K chunks up to
+// kc_pad (a multiple of 16) are zero-filled.  One thread per unit.
+__global__ __launch_bounds__(256) void pack_x_tiles_kernel(const void* __restrict__ xv, int x_is_f16, uint32_t m,
+                                                           uint32_t k, uint32_t kc_pad, uint4* __restrict__ out,
+                                                           uint64_t units) {
+    const uint64_t u = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (u >= units) return;
+    const uint32_t lr = static_cast<uint32_t>(u & 15);
+    const uint64_t rest = u >> 4;
+    const uint32_t kc = static_cast<uint32_t>(rest % kc_pad);
+    const uint32_t row = static_cast<uint32_t>(rest / kc_pad) * 16 + lr;
+    uint4 r = {0u, 0u, 0u, 0u};
+    if (row < m && kc * 8 < k) {
+        if (x_is_f16) {
+            r = interleave8(*reinterpret_cast<const uint4*>(static_cast<const _Float16*>(xv) + static_cast<size_t>(row) * k + kc * 8));
+        } else {
+            const float4* p = reinterpret_cast<const float4*>(static_cast<const float*>(xv) + static_cast<size_t>(row) * k + kc * 8);
+            const float4 a = p[0], b = p[1];
+            r.x = pack_h2(a.x, b.x);
+            r.y = pack_h2(a.y, b.y);
+            r.z = pack_h2(a.z, b.z);
+            r.w = pack_h2(a.w, b.w);
+        }
+    }
+    out[u] = r;
+}
+
+__global__ __launch_bounds__(256, 2) void gemm_q4_w2(const uint8_t* __restrict__ w, uint32_t n, uint32_t k,
+                                                     const uint4* __restrict__ xp, uint32_t kc_pad, uint32_t m,
+                                                     float* __restrict__ y, WregPlan plan) {
+    extern __shared__ uint4 lds16[];  // two activation buffers of kStepUnits units
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int lr = lane & 15;  // row inside a 16-row tile
+    const int g = lane >> 4;   // K group: block g of the step
+
+    // ---- workgroup -> (tile, K slice).  Whole tiles first, then the slices of the tail tiles; inside
+    // either range, workgroups that land on one XCD (blockIdx % 8) take a contiguous run of tile ids,
+    // i.e. neighbouring weight tiles: each XCD's L2 then streams an eighth of W instead of all of it.
+    const uint32_t n_whole = plan.full, n_tail = gridDim.x - plan.full;
+    const bool in_tail = blockIdx.x >= n_whole;
+    const uint32_t pos = in_tail ? blockIdx.x - n_whole : blockIdx.x, count = in_tail ? n_tail : n_whole;
+    const uint32_t xcd = pos & 7u, per = count >> 3, rem = count & 7u;
+    const uint32_t item = xcd * per + (xcd < rem ? xcd : rem) + (pos >> 3);
+    const uint32_t tile = in_tail ? plan.full + item / plan.tail_slices : item;
+    const uint32_t nslices = in_tail ? plan.tail_slices : 1;
+    const uint32_t slice = in_tail ? item % plan.tail_slices : 0;
+
+    const uint32_t tiles_m = (m + TM - 1) / TM, tiles_n = (n + TN - 1) / TN;
+    const uint32_t per_group = kGroupM * tiles_n;
+    const uint32_t group = tile / per_group;
+    const uint32_t first_m = group * kGroupM;
+    const uint32_t group_m = tiles_m - first_m < kGroupM ? tiles_m - first_m : kGroupM;
+    const uint32_t in_group = tile - group * per_group;
+    const uint32_t m0 = (first_m + in_group % group_m) * TM;
+    const uint32_t n0 = (in_group / group_m) * TN;
+
+    const uint32_t nb_total = k / kBlockWeights;
+    const uint32_t steps_total = (nb_total + 3) / 4;
+    const uint32_t steps_per = (steps_total + nslices - 1) / nslices;
+    const uint32_t s_begin = slice * steps_per;  // the host never plans an empty slice
+    const uint32_t nsteps = s_begin + steps_per < steps_total ? steps_per : steps_total - s_begin;
+    const uint32_t nb = nb_total - s_begin * 4;  // blocks from the slice start to the end of the row
+    const bool to_partial = nslices > 1;
+    float* const ptile = to_partial ? plan.partial + (static_cast<size_t>(tile - plan.full) * nslices + slice) * (TM * TN)
+                                    : nullptr;
+
+    float4v acc[NU][NT];
+#pragma unroll
+    for (int u = 0; u < NU; ++u)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[u][t] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // byte offset of the lane's weight row of tile u from the first block of the slice in row 0 (rows
+    // past the end are clamped to the last row: their results are never stored); a uniform base plus
+    // 32-bit lane offsets keeps the addresses in 4 registers (a Q4 tensor is far below 4 GB)
+    const uint8_t* const w_base = w + static_cast<size_t>(s_begin) * (4 * kBlockBytes);
+    uint32_t w_off[NU];
+#pragma unroll
+    for (int u = 0; u < NU; ++u) {
+        uint32_t row = n0 + wave * 64 + u * 16 + lr;
+        row = row < n ? row : n - 1;
+        w_off[u] = row * (nb_total * static_cast<uint32_t>(kBlockBytes));
+    }
+    auto load_w_one = [&](Q4BlockRaw (&wr)[NU], uint32_t s, int u) {
+        uint32_t blk = s * 4 + g;
+        blk = blk < nb ? blk : nb - 1;
+        wr[u] = *reinterpret_cast<const Q4BlockRaw*>(w_base + (w_off[u] + blk * static_cast<uint32_t>(kBlockBytes)));
+    };
+    auto load_w = [&](Q4BlockRaw (&wr)[NU], uint32_t s) {
+#pragma unroll
+        for (int u = 0; u < NU; ++u) load_w_one(wr, s, u);
+    };
+
+    // The activations of step s of this slice: token tile i of the workgroup is 4 KB contiguous in packed X
+    // and in LDS; wave w moves its quarter (64 units) of each of the 8 token tiles.  Steps past the
+    // slice re-read its last step, so that every step issues the same eight loads.
+    const uint4* const x_src = xp + (static_cast<size_t>(m0 / 16) * kc_pad + static_cast<size_t>(s_begin) * 16) * 16 + wave * 64 + lane;
+    auto load_x_one = [&](uint32_t s, int buf, int i) {
+        const uint32_t ss = s < nsteps ? s : nsteps - 1;
+        const uint4* src = x_src + static_cast<size_t>(ss) * 256;
+        uint4* dst = lds16 + buf * kStepUnits + wave * 64;
+        __builtin_amdgcn_global_load_lds((global_void_t*)(src + static_cast<size_t>(i) * kc_pad * 16),
+                                         (lds_void_t*)(dst + i * 256), 16, 0, 0);
+    };
+    auto load_x = [&](uint32_t s, int buf) {
+#pragma unroll
+        for (int i = 0; i < NT; ++i) load_x_one(s, buf, i);
+    };
+
+    U4 a_cur[NU];
+
+    // One K step, the instruction order of gemm_q4_wreg: 4 quarters x 8 token tiles x 4 weight tiles,
+    // in the shadow of each matrix-core instruction one or two steps of the next quarter's
+    // dequantisation, LDS operand reads two token tiles ahead.  `wr` holds this step's blocks and is
+    // refilled for step s + 2 when its last quarter has been dequantised; `wnext` holds step s + 1.
+    // The operand reads are written as ds_read_b128 by hand, with their waits: a read the compiler
+    // knows of is made to wait for every global_load_lds in flight (it cannot tell the two LDS
+    // buffers apart), which would stall each step on the activations of the next.
+    const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<size_t>((__attribute__((address_space(3))) char*)lds16));
+    auto step = [&](uint32_t s, Q4BlockRaw (&wr)[NU], Q4BlockRaw (&wnext)[NU]) {
+        const uint32_t xaddr = lds_base + ((s & 1) * kStepUnits + (4 * g) * 16 + lr) * 16;
+        const bool live_next = (s + 1) * 4 + g < nb;
+        U4 a_nxt[NU];
+        DqTmp tmp;
+        u32x4 bx[3];
+        bx[0] = lds_read128<0>(xaddr);
+        bx[1] = lds_read128<256 * 16>(xaddr);
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<4>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            static_for<NT>([&](auto tc) {
+                constexpr int t = decltype(tc)::value;
+                constexpr int p = j * NT + t;  // slot: (quarter, token tile)
+                // Memory instructions one at a time between the token tiles: a burst of them from all
+                // eight waves right after the barrier would fill the address unit's queue, and a wave
+                // whose load is not accepted cannot issue its matrix instructions either.
+                if constexpr (j == 0) load_x_one(s + 1, (s + 1) & 1, t);  // next step's activations, token tile t
+                if constexpr (j == 3 && (t & 1) == 0) load_w_one(wr, s + 2, t / 2);  // wr is free: refill for step s + 2
+                if constexpr (p + 2 < 4 * NT) {
+                    constexpr int pj = (p + 2) / NT, pt = (p + 2) % NT;
+                    bx[(p + 2) % 3] = lds_read128<(pt * 256 + pj * 16) * 16>(xaddr);
+                }
+                // the read of slot p is done when at most the reads of slots p + 1 and p + 2 are out
+                lds_wait<(p + 2 < 4 * NT) ? 2 : (4 * NT - 1 - p)>(bx[p % 3]);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int u = 0; u < NU; ++u) {
+                    const int c = t * NU + u;  // instruction index inside the quarter, 0..31
+                    mfma_in_place(acc[u][t], a_cur[u], bx[p % 3]);
+#pragma unroll
+                    for (int e = c * (NU * 13) / 32; e < (c + 1) * (NU * 13) / 32; ++e) {
+                        const int uu = e / 13, op = e % 13;
+                        if (j < 3) dq_op_q4_sb(op, wr[uu].q[j + 1], wr[uu].sb, tmp, a_nxt[uu]);
+                        else dq_op_q4_sb(op, wnext[uu].q[0], wnext[uu].sb, tmp, a_nxt[uu]);
+                    }
+                    if (j == 2 && t == NT - 1) wnext[u].sb = live_next ? wnext[u].sb : 0u;  // a block past the end of K counts as zero
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            });
+#pragma unroll
+            for (int u = 0; u < NU; ++u) a_cur[u] = a_nxt[u];
+        });
+        // the activations of step s + 1 have landed (only the weight loads of step s + 2, issued after
+        // them, may still be in flight), and every wave is done reading this step's buffer
+        asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
+    };
+
+    Q4BlockRaw wa[NU], wb[NU];
+    load_x(0, 0);
+    load_w(wa, 0);
+    load_w(wb, 1);
+    {
+        DqTmp tmp;
+#pragma unroll
+        for (int u = 0; u < NU; ++u) {
+            wa[u].sb = static_cast<uint32_t>(g) < nb ? wa[u].sb : 0u;
+#pragma unroll
+            for (int op = 0; op < 13; ++op) dq_op_q4_sb(op, wa[u].q[0], wa[u].sb, tmp, a_cur[u]);
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+
+    uint32_t s = 0;
+    for (; s + 2 <= nsteps; s += 2) {
+        step(s, wa, wb);
+        step(s + 1, wb, wa);
+    }
+    if (s < nsteps) step(s, wa, wb);
+    // the last matrix-core results are 8 passes from their registers
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+
+    // ---- epilogue: element v of lane l of a 16x16 result is weight row 4*(l/16) + v, token l%16
+    const bool vec_ok = (n & 3u) == 0;
+#pragma unroll
+    for (int u = 0; u < NU; ++u) {
+        const uint32_t gn = n0 + wave * 64 + u * 16 + 4 * g;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const uint32_t gm = m0 + t * 16 + lr;
+            if (gm >= m || gn >= n) continue;
+            const float4v val = acc[u][t];
+            if (to_partial) {  // tile-local layout, always 16-byte aligned
+                *reinterpret_cast<float4v*>(ptile + (gm - m0) * TN + (gn - n0)) = val;
+                continue;
+            }
+            float* dst = y + static_cast<size_t>(gm) * n + gn;
+            if (vec_ok) {
+                *reinterpret_cast<float4v*>(dst) = val;
+            } else {
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (gn + v < n) dst[v] = val[v];
+            }
+        }
+    }
+}
+
 // Sums the K slices of the tail tiles in slice order and writes them to y, adding the LoRA delta
 // scale * sum_j B[row, j] * t[token, j] in f32.  grid (tail tiles, TM * TN / 1024); a thread owns four
 // consecutive weight rows of one token.
@@ -590,10 +875,10 @@ struct HostPlan {
     uint32_t tiles, full, slices;
 };
 
-HostPlan plan_tiles(uint32_t n, uint32_t k, uint32_t m) {
+HostPlan plan_tiles(uint32_t n, uint32_t k, uint32_t m, uint32_t slots = kCus) {
     const uint32_t tiles = ((n + TN - 1) / TN) * ((m + TM - 1) / TM);
     const uint32_t steps = (k / kBlockWeights + 3) / 4;
-    const uint32_t rest = tiles % kCus;
+    const uint32_t rest = tiles % slots;
     HostPlan p{tiles, tiles - rest, 1};
     if (rest == 0 || steps < 4) return HostPlan{tiles, tiles, 1};
     // pick the slice count that minimises the time of the last round in K steps,
@@ -603,7 +888,7 @@ HostPlan plan_tiles(uint32_t n, uint32_t k, uint32_t m) {
     for (uint32_t s = 2; s <= kMaxTailSlices && s * 2 <= steps; ++s) {
         const uint32_t per = (steps + s - 1) / s;
         if ((s - 1) * per >= steps) continue;  // would leave the last slice empty
-        const double rounds = static_cast<double>((rest * s + kCus - 1) / kCus);
+        const double rounds = static_cast<double>((rest * s + slots - 1) / slots);
         const double t = rounds * per + LQ4_SLICE_CHARGE * rest * s;
         if (t < best - 1e-9) {
             best = t;
@@ -619,6 +904,12 @@ HostPlan plan_tiles(uint32_t n, uint32_t k, uint32_t m) {
 uint32_t gemm_wreg_tiles(uint32_t n, uint32_t m) { return ((n + TN - 1) / TN) * ((m + TM - 1) / TM); }
 
 bool gemm_wreg_supports(uint32_t, uint32_t k, uint32_t, int) { return k >= kBlockWeights; }
+
+// The two-workgroups-per-CU kernel pays one pass over X for packing and schedules in rounds of 512
+// tiles: it is ahead (4-13 % measured) where there is at least one such round of whole tiles.
+bool gemm_w2_wants(uint32_t n, uint32_t k, uint32_t m) {
+    return k >= kBlockWeights && gemm_wreg_tiles(n, m) >= 2 * kCus;
+}
 
 size_t gemm_wreg_scratch_floats(uint32_t n, uint32_t k, uint32_t m) {
     const HostPlan p = plan_tiles(n, k, m);
@@ -666,6 +957,45 @@ void launch_gemm_wreg(const uint8_t* w, uint32_t n, uint32_t k, const void* x, i
             else launch_wreg_t<false, false, 0>(w, n, k, x, m, y, lora, hp, partial, stream);
         }
     }
+    if (hp.slices > 1)
+        hipLaunchKernelGGL(gemm_reduce_tail, dim3(hp.tiles - hp.full, TM * TN / 1024), dim3(256), 0, stream, partial,
+                           hp.full, hp.slices, m, n, y, lora);
+}
+
+// ---- gemm_q4_w2: scratch = [packed X | partial tiles of the sliced tail] ----------------------------
+namespace {
+constexpr uint32_t kW2Slots = 2 * kCus;  // two workgroups per CU
+inline uint32_t w2_kc_pad(uint32_t k) { return (k / 8 + 15) / 16 * 16; }
+inline size_t w2_packed_bytes(uint32_t k, uint32_t m) {
+    return static_cast<size_t>((m + TM - 1) / TM) * TM * w2_kc_pad(k) * 16;
+}
+}  // namespace
+
+size_t gemm_w2_scratch_bytes(uint32_t n, uint32_t k, uint32_t m) {
+    const HostPlan p = plan_tiles(n, k, m, kW2Slots);
+    const size_t partial = p.slices > 1 ? static_cast<size_t>(p.tiles - p.full) * p.slices * (TM * TN) * sizeof(float) : 0;
+    return w2_packed_bytes(k, m) + partial;
+}
+
+void launch_gemm_w2(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
+                    uint8_t* scratch, hipStream_t stream) {
+    const LoraEpilogue lora{nullptr, nullptr, 0, 0, 0.0f};  // no LoRA step in this kernel
+    const HostPlan hp = plan_tiles(n, k, m, kW2Slots);
+    const uint32_t kc_pad = w2_kc_pad(k);
+    uint4* packed = reinterpret_cast<uint4*>(scratch);
+    float* partial = reinterpret_cast<float*>(scratch + w2_packed_bytes(k, m));
+    const uint64_t units = w2_packed_bytes(k, m) / 16;
+    hipLaunchKernelGGL(pack_x_tiles_kernel, dim3(static_cast<uint32_t>((units + 255) / 256)), dim3(256), 0, stream, x,
+                       x_is_f16, m, k, kc_pad, packed, units);
+    static bool attr_set = false;
+    if (!attr_set) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4_w2), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+        attr_set = true;
+    }
+    const size_t lds = 2 * kStepUnits * sizeof(uint4);
+    const WregPlan plan{hp.full, hp.slices, partial};
+    const uint32_t wgs = hp.full + (hp.tiles - hp.full) * hp.slices;
+    hipLaunchKernelGGL(gemm_q4_w2, dim3(wgs), dim3(256), lds, stream, w, n, k, packed, kc_pad, m, y, plan);
     if (hp.slices > 1)
         hipLaunchKernelGGL(gemm_reduce_tail, dim3(hp.tiles - hp.full, TM * TN / 1024), dim3(256), 0, stream, partial,
                            hp.full, hp.slices, m, n, y, lora);

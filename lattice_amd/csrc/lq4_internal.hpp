@@ -147,7 +147,7 @@ void launch_lora_b_accum(const void* b, int b_is_f16, uint32_t rank, uint32_t d_
 
 // Y[M,N] = X[M,K] . W^T (+ LoRA); X f32 or f16, Y f32.
 // gemm_scratch_floats = floats of scratch launch_gemm needs for the shape (0 = none).
-size_t gemm_scratch_floats(uint32_t n, uint32_t k, uint32_t m, int x_is_f16);
+size_t gemm_scratch_floats(uint32_t n, uint32_t k, uint32_t m, int x_is_f16, bool with_lora);
 void launch_gemm(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
                  float* y, const LoraEpilogue& lora, float* scratch, hipStream_t stream);
 
@@ -162,6 +162,12 @@ void set_gemm_kernel_choice(int which);
 // A last, partly filled round of tiles is cut into K slices that meet in `partial`
 // (gemm_wreg_scratch_floats floats; null = no slicing) and are summed by a second kernel.
 size_t gemm_wreg_scratch_floats(uint32_t n, uint32_t k, uint32_t m);
+// The same tile at two workgroups per CU, Q4 only: activations packed into scratch first (f16, tile order),
+// then the tail's partial tiles behind them; gemm_w2_scratch_bytes covers both.
+size_t gemm_w2_scratch_bytes(uint32_t n, uint32_t k, uint32_t m);
+bool gemm_w2_wants(uint32_t n, uint32_t k, uint32_t m);
+void launch_gemm_w2(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
+                    uint8_t* scratch, hipStream_t stream);
 void launch_gemm_wreg(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
                       float* y, const LoraEpilogue& lora, float* partial, hipStream_t stream, int fmt = 0);
 

@@ -81,6 +81,18 @@ def test_prefill_gemm_config2_full_size(be, m, n, k):
     _gemm_full(be, m, n, k, seed=3)
 
 
+@pytest.mark.parametrize("kernel", [2, 4])
+@pytest.mark.parametrize("m,n,k", [(2048, 17408, 5120), (2048, 5120, 17408)])
+def test_prefill_gemm_config2_full_size_either_register_kernel(be, kernel, m, n, k):
+    # whichever of the two weights-in-registers kernels the shape rule does not pick is checked too
+    print(f"gemm full kernel={kernel} m={m} n={n} k={k}", flush=True)
+    be.set_gemm_kernel(kernel)
+    try:
+        _gemm_full(be, m, n, k, seed=6)
+    finally:
+        be.set_gemm_kernel(0)
+
+
 @pytest.mark.parametrize("m,n,k", [(512, 5120, 17408), (2048, 5120, 17408)])
 def test_prefill_gemm_config2_full_size_with_lora(be, m, n, k):
     # the down projection: at M = 512 every tile of it is a K-sliced tail tile

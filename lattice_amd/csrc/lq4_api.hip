@@ -1033,9 +1033,12 @@ int lq4_gemv_chain(lq4_ctx* ctx, const lq4_chain_step* steps, uint32_t n_steps, 
         return LQ4_OK;
     }
 
-    // Step by step: every step is lq4_gemv_fused (plus the stand-alone silu * up where a step ends
-    // in it); results nobody asked for live in the chain scratch as plain floats.
+    // Step by step: every step is lq4_gemv_fused; results nobody asked for live in the chain scratch as
+    // plain floats.  A step that ends in silu(gate) * up runs plain and the NEXT step takes gate || up
+    // through its silu prologue (LQ4_PRO_SILU_MUL), which costs no launch; only when the caller wants the
+    // product itself (y_dev), or nothing plain follows, does the stand-alone silu * up kernel run.
     const float* prev = nullptr;
+    bool prev_is_gate_up = false;  // prev holds [gate | up] of the previous step, silu * up still to apply
     for (uint32_t j = 0; j < n_steps; ++j) {
         const lq4_chain_step& st = steps[j];
         float* spare = reinterpret_cast<float*>(ctx->chain_scratch + lay.result[j]);
@@ -1049,10 +1052,16 @@ int lq4_gemv_chain(lq4_ctx* ctx, const lq4_chain_step* steps, uint32_t n_steps, 
         f.delta = st.delta;
         f.residual_out = st.residual_out;
         if (st.from_previous) {
-            if (st.prologue != LQ4_PRO_ADD_RMSNORM) x = prev;
-            else if (st.base) f.delta = prev;
-            else f.base = prev;
+            if (st.prologue != LQ4_PRO_ADD_RMSNORM) {
+                x = prev;
+                if (prev_is_gate_up) f.prologue = LQ4_PRO_SILU_MUL;
+            } else if (st.base) {
+                f.delta = prev;
+            } else {
+                f.base = prev;
+            }
         }
+        prev_is_gate_up = false;
         float* result;
         if (st.epilogue == LQ4_EPI_ADD_RESIDUAL) {
             f.epilogue = LQ4_EPI_ADD_RESIDUAL;
@@ -1063,10 +1072,17 @@ int lq4_gemv_chain(lq4_ctx* ctx, const lq4_chain_step* steps, uint32_t n_steps, 
         } else if (st.epilogue == LQ4_EPI_SILU_MUL_PAIRS) {
             f.epilogue = LQ4_EPI_NONE;
             rc = lq4_gemv_fused(ctx, st.w, st.w_extra_offset, st.n, st.k, x, spare, &f, nullptr, 0.0f, stream);
-            result = st.y_dev ? st.y_dev : spare;  // in place: out[i] only depends on in[i] and in[i + n/2]
-            if (!rc) {
-                launch_silu_mul(spare, st.n / 2, 1, result, st.n / 2, s);
-                ctx->counters.elementwise++;
+            const bool next_takes_it = !st.y_dev && j + 1 < n_steps && steps[j + 1].from_previous &&
+                                       steps[j + 1].prologue == LQ4_PRO_NONE;
+            if (next_takes_it) {
+                result = spare;
+                prev_is_gate_up = true;
+            } else {
+                result = st.y_dev ? st.y_dev : spare;  // in place: out[i] only depends on in[i] and in[i + n/2]
+                if (!rc) {
+                    launch_silu_mul(spare, st.n / 2, 1, result, st.n / 2, s);
+                    ctx->counters.elementwise++;
+                }
             }
         } else {
             f.epilogue = LQ4_EPI_NONE;

@@ -330,11 +330,14 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
         }
         buf[((tid >> 4) + 16 * i) * kPitch16 + x_part] = out;
     };
-    auto load_w = [&](WBlock (&wr)[NU], uint32_t s) {
+    auto load_w_one = [&](WBlock (&wr)[NU], uint32_t s, int u) {
         uint32_t blk = s * 4 + g;
         blk = blk < nb ? blk : nb - 1;
+        wr[u] = *reinterpret_cast<const WBlock*>(w_row[u] + blk * kUnits);
+    };
+    auto load_w = [&](WBlock (&wr)[NU], uint32_t s) {
 #pragma unroll
-        for (int u = 0; u < NU; ++u) wr[u] = *reinterpret_cast<const WBlock*>(w_row[u] + blk * kUnits);
+        for (int u = 0; u < NU; ++u) load_w_one(wr, s, u);
     };
 
     auto scale_pair = [&](const WBlock& blk, bool live, half2v& d2, half2v& b2) {
@@ -356,9 +359,9 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
     // dequantisation of the NEXT quarter (for the last quarter: the first quarter of step s+1,
     // from `wnext`), and every fourth token tile one activation unit of step s+1 is written to the
     // other LDS buffer and refilled from global memory for step s+2.  LDS operand reads run two
-    // token tiles ahead.  `wfree` was consumed in the previous step and is refilled for step s+2.
+    // token tiles ahead.  `wfree` was consumed in the previous step and is refilled for step s+2
+    // during the first quarter.
     auto step = [&](uint32_t s, WBlock (&wr)[NU], WBlock (&wnext)[NU], WBlock (&wfree)[NU]) {
-        load_w(wfree, s + 2);
         const uint4* xbuf = lds16 + (s & 1) * kBuf16 + lr * kPitch16 + 4 * g;
         uint4* xnext = lds16 + ((s + 1) & 1) * kBuf16;
         const bool live_next = (s + 1) * 4 + g < nb;
@@ -374,6 +377,9 @@ __global__ __launch_bounds__(256, 1) void gemm_q4_wreg(const uint8_t* __restrict
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
                 const int p = j * NT + t;  // slot: (quarter, token tile)
+                // one weight tile's loads every other token tile rather than all eight at the step's
+                // start: a burst from every wave right after the barrier fills the address unit's queue
+                if (j == 0 && (t & 1) == 0) load_w_one(wfree, s + 2, t / 2);
                 if (p + 2 < 4 * NT) {
                     const int pj = (p + 2) / NT, pt = (p + 2) % NT;
                     bx[(p + 2) % 3] = xbuf[pt * 16 * kPitch16 + pj];

@@ -29,8 +29,8 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense f16
 
 # rocprofv3 counters on this workload (profiles/gemv_q4_b1_decode_layer_traffic.md): per layer step
-# FETCH_SIZE 15103.9 KiB x 2.000 (copy-kernel scale) + WRITE_SIZE 144 KiB x 1.000, over 4 launches
-MEASURED_TRAFFIC_PER_LAUNCH = (15103.9 * 2.0 + 144.0) * 1024 / 4
+# FETCH_SIZE 15110.0 KiB x 2.000 (copy-kernel scale) + WRITE_SIZE 144 KiB x 1.000, over 4 launches
+MEASURED_TRAFFIC_PER_LAUNCH = (15110.0 * 2.0 + 144.0) * 1024 / 4
 
 LAYER = [("qkv", 3072, 2048), ("o", 2048, 2048), ("gate_up", 12288, 2048), ("down", 2048, 6144)]
 
@@ -150,6 +150,25 @@ def read_sweep(torch, be):
               flush=True)
 
 
+def prefill_gemm(torch, be, gen, tm):
+    """BASELINE config 2: the 27B MLP matrices at 512 and 2048 tokens, f16 activations."""
+    gemm = {}
+    for (n, k) in ((17408, 5120), (5120, 17408)):
+        qw = be.wrap_device_blocks(device_q4_weight(torch, n, k, gen))
+        for m in (512, 2048):
+            x = torch.randn((m, k), device="cuda", generator=gen).to(torch.float16)
+            y = torch.empty((m, n), device="cuda")
+            f = lambda i: be.dispatch_gemm(x, 0, qw, y, 0, m, n, k)
+            for i in range(3):
+                f(i)
+            ms = tm(torch, f, 10)
+            tf = 2.0 * m * n * k / (ms * 1e-3) / 1e12
+            gemm["M%d_N%d_K%d" % (m, n, k)] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 1),
+                                               "pct_of_f16_mfma_peak": round(100 * tf / MFMA_F16_PEAK_TFLOPS, 2)}
+        del qw
+    return gemm
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -161,6 +180,8 @@ def main():
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--headline-only", action="store_true",
                     help="run nothing but warmup and the timed headline region (for kernel-trace profiles)")
+    ap.add_argument("--gemm-only", action="store_true",
+                    help="run the four config-2 prefill GEMM shapes and nothing else (for counter runs)")
     ap.add_argument("--read-sweep", action="store_true",
                     help="print the read-probe sweep (grid x bytes in flight x access pattern x size) and exit")
     ap.add_argument("--eager", action="store_true",
@@ -181,6 +202,9 @@ def main():
     gen = torch.Generator(device="cuda")
     gen.manual_seed(0)
     B = args.batch
+    if args.gemm_only:
+        print(json.dumps({"prefill_gemm_f16": prefill_gemm(torch, be, gen, graph_timed)}))
+        return
 
     # ---- resident inputs ------------------------------------------------------------
     layers = []
@@ -472,20 +496,7 @@ def main():
         # prefill GEMM, benchmark config 2
         del layers
         torch.cuda.empty_cache()
-        gemm = {}
-        for (n, k) in ((17408, 5120), (5120, 17408)):
-            qw = be.wrap_device_blocks(device_q4_weight(torch, n, k, gen))
-            for m in (512, 2048):
-                x = torch.randn((m, k), device="cuda", generator=gen).to(torch.float16)
-                y = torch.empty((m, n), device="cuda")
-                f = lambda i: be.dispatch_gemm(x, 0, qw, y, 0, m, n, k)
-                for i in range(3):
-                    f(i)
-                ms = tm(torch, f, 10)
-                tf = 2.0 * m * n * k / (ms * 1e-3) / 1e12
-                gemm["M%d_N%d_K%d" % (m, n, k)] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 1),
-                                                   "pct_of_f16_mfma_peak": round(100 * tf / MFMA_F16_PEAK_TFLOPS, 2)}
-            del qw
+        gemm = prefill_gemm(torch, be, gen, tm)
         out["prefill_gemm_f16"] = gemm
         # the GEMM half of the metric as a roofline object of its own: the largest config-2 problem
         big = gemm["M2048_N17408_K5120"]

@@ -553,11 +553,23 @@ def main():
         for i in range(3):
             routed(i)
         ms_routed = tm(torch, routed, 40)
+        # ... and with the always-active shared expert (same intermediate size) added onto the sum
+        shared = [(be.wrap_device_blocks(device_q4_weight(torch, 2 * I, H, gen)),
+                   be.wrap_device_blocks(device_q4_weight(torch, H, I, gen))) for _ in range(len(sets))]
+        sgate = torch.randn((H,), device="cuda", generator=gen) * (1.0 / H ** 0.5)
+        def whole_layer(i):
+            routed(i)
+            sh = shared[i % len(shared)]
+            be.moe_shared_expert(sh[0], sh[1], sgate, I, H, xm, ym)
+        for i in range(3):
+            whole_layer(i)
+        ms_layer = tm(torch, whole_layer, 40)
         out["moe_grouped_gemv"] = {"distinct_experts": distinct, "algorithmic_bytes": moe_bytes,
                                    "ms_per_step": round(ms, 4), "GB/s": round(moe_bytes / ms / 1e6, 1),
                                    "pct_of_hbm_peak": round(100 * moe_bytes / ms / 1e6 / HBM_PEAK_GBPS, 2),
-                                   "ms_per_step_with_router": round(ms_routed, 4)}
-        del sets
+                                   "ms_per_step_with_router": round(ms_routed, 4),
+                                   "ms_per_step_with_router_and_shared_expert": round(ms_layer, 4)}
+        del sets, shared
 
         # plain copies of known size: what a profiler's HBM traffic counters are scaled by
         csrc = torch.empty(64 << 20, dtype=torch.int32, device="cuda").random_(generator=gen)

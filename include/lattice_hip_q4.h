@@ -159,6 +159,21 @@ int lq4_moe_grouped_gemv(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_weig
                          const float* x_dev, uint32_t tokens, const int32_t* ids_dev,
                          const float* weights_dev, uint32_t top_k, float* y_dev, void* stream);
 
+/* Replaces apply_shared_expert (crates/inference/src/model/qwen35/moe.rs:194-250) / step 2 of
+ * encode_moe_ffn (forward/metal_qwen35/inner/layers/mod.rs:313-413) with its closing
+ * moe_shared_gate_add (shaders/qwen35.metal:2379-2392), the always-active expert of the MoE FFN:
+ *   g[t]    = 1 / (1 + exp(-dot(x[t], shared_gate)))
+ *   y[t,:] += g[t] * W_down . ( silu(W_gate . x[t]) * (W_up . x[t]) )
+ * y_dev is ACCUMULATED into: call it after lq4_moe_grouped_gemv on the same y (the reference adds the
+ * shared expert onto the routed experts' sum), or on a zeroed y for the shared part alone.
+ * gate_up: [2*shared_inter, hidden], gate_proj rows then up_proj rows (the fused gate||up layout of
+ * the dense MLP); down: [hidden, shared_inter]; shared_gate_dev f32 [hidden]; x_dev f32
+ * [tokens, hidden], 16-byte aligned; y_dev f32 [tokens, hidden].  The intermediate results live in a
+ * library buffer that grows on first use (not during stream capture; run the shape once before). */
+int lq4_moe_shared_expert(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_weight* down,
+                          const float* shared_gate_dev, uint32_t shared_inter, uint32_t hidden,
+                          const float* x_dev, uint32_t tokens, float* y_dev, void* stream);
+
 /* ---- lm_head top-k ------------------------------------------------------------
  * Exact top-k over `n` f32 logits in the reference's candidate order (higher logit first,
  * ties to the lower token id, NaN last as the (-inf, 0xFFFFFFFF) sentinel): the result of

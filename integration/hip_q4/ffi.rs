@@ -234,6 +234,18 @@ extern "C" {
         y: *mut f32,
         stream: *mut c_void,
     ) -> c_int;
+    pub fn lq4_moe_shared_expert(
+        ctx: *mut Lq4Ctx,
+        gate_up: *const Lq4Weight,
+        down: *const Lq4Weight,
+        shared_gate: *const f32,
+        shared_inter: u32,
+        hidden: u32,
+        x: *const f32,
+        tokens: u32,
+        y: *mut f32,
+        stream: *mut c_void,
+    ) -> c_int;
 
     // ---- lm_head and top-k
     pub fn lq4_topk(

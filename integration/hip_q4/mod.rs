@@ -55,6 +55,23 @@ impl Drop for HipQ4WeightBuf {
     }
 }
 
+/// One MoE layer's resident tensors (the role of `MoeMetalBuffers`, metal_qwen35.rs): expert-major
+/// `gate_up [E, 2*inter, hidden]` and `down [E, hidden, inter]`, the shared expert's fused
+/// `shared_gate_up [2*shared_inter, hidden]` (gate_proj rows, then up_proj rows) and
+/// `shared_down [hidden, shared_inter]`, and its f32 gate vector `[hidden]`.
+pub struct HipMoeLayer {
+    pub gate_up: HipQ4WeightBuf,
+    pub down: HipQ4WeightBuf,
+    pub shared_gate_up: HipQ4WeightBuf,
+    pub shared_down: HipQ4WeightBuf,
+    pub shared_expert_gate: DevBuf,
+    pub num_experts: u32,
+    pub top_k: u32,
+    pub inter: u32,
+    pub shared_inter: u32,
+    pub hidden: u32,
+}
+
 struct HipLoraProjection {
     raw: *mut Lq4Lora,
 }
@@ -327,6 +344,46 @@ impl HipQ4Backend {
         }
         // SAFETY: steps points at steps.len() initialised descriptors.
         check(unsafe { lq4_gemv_chain(self.ctx, steps.as_ptr(), steps.len() as u32, self.stream) }).expect("lq4_gemv_chain");
+    }
+
+    /// The MoE FFN of one layer for `tokens` rows of `x` (`encode_moe_ffn`, inner/layers/mod.rs:226-660;
+    /// CPU form `moe_ffn_step`, model/qwen35/moe.rs:8-36): router softmax / top-k / renormalise from the
+    /// router logits, the routed experts, then the always-active shared expert onto the same `y`.
+    /// `ids` / `weights` are device scratch of `tokens * top_k` entries.  Unlike the Metal path nothing
+    /// is read back to the host between the steps (the router and the shared expert's sigmoid gate stay
+    /// on the device).
+    #[allow(clippy::too_many_arguments)]
+    pub fn encode_moe_ffn(
+        &self,
+        router_logits: &DevBuf,
+        moe: &HipMoeLayer,
+        x: &DevBuf,
+        tokens: u32,
+        ids: &DevBuf,
+        weights: &DevBuf,
+        y: &DevBuf,
+    ) {
+        // SAFETY: the buffers hold [tokens, E] logits, [tokens, hidden] activations and outputs and
+        // tokens * top_k routing entries; the weight handles were uploaded with these shapes.
+        unsafe {
+            check(lq4_moe_route(
+                self.ctx, router_logits.ptr as *const f32, tokens, moe.num_experts, moe.top_k,
+                ids.ptr as *mut i32, weights.ptr as *mut f32, self.stream,
+            ))
+            .expect("lq4_moe_route");
+            check(lq4_moe_grouped_gemv(
+                self.ctx, moe.gate_up.raw, moe.down.raw, moe.num_experts, moe.inter, moe.hidden,
+                x.ptr as *const f32, tokens, ids.ptr as *const i32, weights.ptr as *const f32,
+                moe.top_k, y.ptr as *mut f32, self.stream,
+            ))
+            .expect("lq4_moe_grouped_gemv");
+            check(lq4_moe_shared_expert(
+                self.ctx, moe.shared_gate_up.raw, moe.shared_down.raw,
+                moe.shared_expert_gate.ptr as *const f32, moe.shared_inter, moe.hidden,
+                x.ptr as *const f32, tokens, y.ptr as *mut f32, self.stream,
+            ))
+            .expect("lq4_moe_shared_expert");
+        }
     }
 
     /// `commit()` + `wait_until_completed()` of the command buffer.

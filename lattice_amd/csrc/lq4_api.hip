@@ -26,6 +26,8 @@ struct lq4_ctx {
     bool lora_in_kernel;
     uint32_t lora_spin_limit;  // polls a weight wave spends on those counters before it computes A.x alone
     size_t moe_scratch_bytes;
+    uint8_t* shared_scratch;  // lq4_moe_shared_expert: gate||up and down results (the GEMM it calls uses moe_scratch)
+    size_t shared_scratch_bytes;
     // Buffers the growable scratch outgrew: launches already queued (or captured into a graph) may
     // still use them, so they are only released with the context.
     std::vector<void*> retired;
@@ -240,6 +242,7 @@ int lq4_ctx_destroy(lq4_ctx* ctx) {
     (void)hipFree(ctx->lora_t);
     (void)hipFree(ctx->topk_ticket);
     if (ctx->moe_scratch) (void)hipFree(ctx->moe_scratch);
+    if (ctx->shared_scratch) (void)hipFree(ctx->shared_scratch);
     if (ctx->chain_scratch) (void)hipFree(ctx->chain_scratch);
     (void)hipFree(ctx->chain_sync);
     for (void* p : ctx->retired) (void)hipFree(p);
@@ -581,6 +584,57 @@ int lq4_moe_grouped_gemv(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_weig
                        static_cast<hipStream_t>(stream));
     ctx->counters.moe_gate_up++;
     ctx->counters.moe_down++;
+    LQ4_HIP(hipGetLastError());
+    return LQ4_OK;
+}
+
+int lq4_moe_shared_expert(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_weight* down,
+                          const float* shared_gate_dev, uint32_t shared_inter, uint32_t hidden, const float* x_dev,
+                          uint32_t tokens, float* y_dev, void* stream) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    if (tokens == 0 || hidden == 0) return LQ4_OK;
+    if (!x_dev || !y_dev || !shared_gate_dev) return fail(LQ4_E_INVALID, "null device pointer");
+    if (shared_inter == 0 || shared_inter % kBlockWeights)
+        return fail(LQ4_E_INVALID, "shared expert intermediate size must be a non-zero multiple of 32, got %u", shared_inter);
+    if (shared_inter > UINT32_MAX / 2) return fail(LQ4_E_INVALID, "shared expert intermediate size too large");
+    if (reinterpret_cast<uintptr_t>(x_dev) % 16) return fail(LQ4_E_INVALID, "x must be 16-byte aligned");
+    const uint8_t *gu, *dn;
+    int rc = resolve_weight(gate_up, 0, 2 * shared_inter, hidden, &gu);
+    if (rc) return rc;
+    rc = resolve_weight(down, 0, hidden, shared_inter, &dn);
+    if (rc) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    DeviceGuard g(ctx->device);
+    auto up256 = [](size_t v) { return (v + 255) / 256 * 256; };
+    const size_t off_gu = 0;
+    const size_t off_act = off_gu + up256(sizeof(float) * tokens * 2 * shared_inter);
+    const size_t off_o = off_act + up256(sizeof(float) * tokens * shared_inter);
+    const size_t total = off_o + up256(sizeof(float) * tokens * hidden);
+    rc = grow_scratch(ctx, &ctx->shared_scratch, &ctx->shared_scratch_bytes, total, s, false);
+    if (rc) return rc;
+    float* gu_out = reinterpret_cast<float*>(ctx->shared_scratch + off_gu);
+    float* act = reinterpret_cast<float*>(ctx->shared_scratch + off_act);
+    float* o = reinterpret_cast<float*>(ctx->shared_scratch + off_o);
+    const LoraEpilogue none{};
+    if (tokens == 1 && gemv_b1_lds_bytes(shared_inter) <= 128 * 1024) {
+        // gate||up, then the down projection with silu(gate) * up computed as it stages its activations
+        launch_gemv(gu, 2 * shared_inter, hidden, x_dev, hidden, 1, gu_out, 2 * shared_inter, none, s);
+        GemvFusion gf{};
+        gf.prologue = GemvFusion::kSiluMul;
+        gf.epilogue = GemvFusion::kStore;
+        launch_gemv_b1_fused(dn, hidden, shared_inter, gu_out, o, none, gf, s);
+        ctx->counters.gemv++;
+        ctx->counters.gemv_fused++;
+    } else {
+        rc = lq4_gemm(ctx, gate_up, 0, 2 * shared_inter, hidden, x_dev, LQ4_F32, tokens, gu_out, nullptr, 0.0f, stream);
+        if (rc) return rc;
+        launch_silu_mul(gu_out, shared_inter, tokens, act, shared_inter, s);
+        ctx->counters.elementwise++;
+        rc = lq4_gemm(ctx, down, 0, hidden, shared_inter, act, LQ4_F32, tokens, o, nullptr, 0.0f, stream);
+        if (rc) return rc;
+    }
+    launch_moe_shared_gate_add(x_dev, shared_gate_dev, o, hidden, tokens, y_dev, s);
+    ctx->counters.elementwise++;
     LQ4_HIP(hipGetLastError());
     return LQ4_OK;
 }

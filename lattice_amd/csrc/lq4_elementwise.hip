@@ -108,7 +108,32 @@ __global__ __launch_bounds__(256) void add_and_copy_kernel(const float* __restri
     if (dst) dst[i] = r;
 }
 
+// The shared expert's sigmoid gate and its add onto the routed experts' sum (apply_shared_expert,
+// crates/inference/src/model/qwen35/moe.rs:201-207 and 242-244; moe_shared_gate_add,
+// shaders/qwen35.metal:2379-2392): one workgroup per token computes g = sigmoid(x . gate) and then
+// y = fma(g, shared_out, y) over the token's row.
+__global__ __launch_bounds__(256) void moe_shared_gate_add_kernel(const float* __restrict__ x,
+                                                                  const float* __restrict__ gate,
+                                                                  const float* __restrict__ shared_out,
+                                                                  uint32_t hidden, float* y) {
+    __shared__ float red[4];
+    const size_t off = static_cast<size_t>(blockIdx.x) * hidden;
+    float dot = 0.0f;
+    for (uint32_t i = threadIdx.x; i < hidden; i += 256) dot = fmaf(x[off + i], gate[i], dot);
+    dot = wave_sum(dot);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = dot;
+    __syncthreads();
+    const float logit = (red[0] + red[1]) + (red[2] + red[3]);
+    const float g = 1.0f / (1.0f + expf(-logit));
+    for (uint32_t i = threadIdx.x; i < hidden; i += 256) y[off + i] = fmaf(g, shared_out[off + i], y[off + i]);
+}
+
 }  // namespace
+
+void launch_moe_shared_gate_add(const float* x, const float* gate, const float* shared_out, uint32_t hidden,
+                                uint32_t tokens, float* y, hipStream_t stream) {
+    hipLaunchKernelGGL(moe_shared_gate_add_kernel, dim3(tokens), dim3(256), 0, stream, x, gate, shared_out, hidden, y);
+}
 
 void launch_residual_add_norm(const float* base, const float* delta, const float* gamma, uint32_t hidden,
                               uint32_t rows, float eps, float* residual_out, float* normed_out, hipStream_t stream) {

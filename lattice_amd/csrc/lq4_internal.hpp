@@ -130,6 +130,9 @@ void launch_residual_add_norm(const float* base, const float* delta, const float
 void launch_silu_mul(const float* gate_up, uint32_t count, uint32_t rows, float* out, uint32_t out_stride,
                      hipStream_t stream);
 void launch_add_and_copy(const float* src, float* residual, float* dst, size_t count, hipStream_t stream);
+// y[t, :] = fma(sigmoid(x[t] . gate), shared_out[t, :], y[t, :]) for every token
+void launch_moe_shared_gate_add(const float* x, const float* gate, const float* shared_out, uint32_t hidden,
+                                uint32_t tokens, float* y, hipStream_t stream);
 
 // Matrix-core GEMV for batch 1..8 (activations staged in LDS as f16 columns).
 size_t gemv_mfma_lds_bytes(uint32_t k, uint32_t batch);

@@ -88,6 +88,10 @@ def lib() -> C.CDLL:
         fn.restype = C.c_int
         fn.argtypes = [_u8p, _u8p, C.c_int, C.c_int, C.c_int, _f32p, C.c_int, _i32p, _f32p,
                        C.c_int, outp]
+    for name, outp in (("lq4o_moe_shared_expert_f32", _f32p), ("lq4o_moe_shared_expert_f64", _f64p)):
+        fn = getattr(L, name)
+        fn.restype = C.c_int
+        fn.argtypes = [_u8p, _u8p, _f32p, C.c_int, C.c_int, _f32p, C.c_int, outp]
     L.lq4o_q3_quantize_block.restype = C.c_int
     L.lq4o_q3_quantize_block.argtypes = [_f32p, C.c_int, C.c_int, _u8p]
     L.lq4o_q3_quantize_row.restype = C.c_int
@@ -332,6 +336,24 @@ def moe_ffn(gate_up_q4, down_q4, num_experts, inter, hidden, x, ids, weights, f6
     if rc:
         raise ValueError(f"moe_ffn rc={rc}")
     return out
+
+
+def moe_shared_expert(gate_up_q4, down_q4, shared_gate, shared_inter, hidden, x, out, f64=False):
+    """apply_shared_expert (moe.rs:194-250) over Q4 tensors; returns ``out`` plus the gated
+    shared-expert FFN of every row of ``x`` (``out`` itself is left untouched)."""
+    gu, dn = _u8(gate_up_q4), _u8(down_q4)
+    xx = _f32(x).reshape(-1, hidden)
+    sg = _f32(shared_gate).ravel()
+    assert sg.size == hidden
+    assert gu.size == 2 * shared_inter * (hidden // 32) * BLOCK_BYTES
+    assert dn.size == hidden * (shared_inter // 32) * BLOCK_BYTES
+    acc = np.array(out, dtype=np.float64 if f64 else np.float32).reshape(xx.shape[0], hidden).copy()
+    fn = lib().lq4o_moe_shared_expert_f64 if f64 else lib().lq4o_moe_shared_expert_f32
+    rc = fn(_p(gu, _u8p), _p(dn, _u8p), _p(sg, _f32p), shared_inter, hidden, _p(xx, _f32p),
+            xx.shape[0], _p(acc, _f64p if f64 else _f32p))
+    if rc:
+        raise ValueError(f"moe_shared_expert rc={rc}")
+    return acc
 
 
 # --- .q4 file ---------------------------------------------------------------

@@ -527,6 +527,68 @@ int lq4o_moe_ffn_f64(const uint8_t* gate_up_q4, const uint8_t* down_q4, int num_
     return 0;
 }
 
+/* apply_shared_expert (moe.rs:194-250) with the shared expert's tensors held as Q4
+ * blocks: gate_up is [2*SI, H] (gate_proj rows, then up_proj rows), down is [H, SI].
+ * Per token: g = 1 / (1 + exp(-dot(x, shared_gate))) with the dot summed
+ * sequentially in f32 (the iterator .sum() of moe.rs:201-206), then
+ * out[i] += g * (W_down . (silu(W_gate . x) * (W_up . x)))[i] (moe.rs:242-244):
+ * `out` is accumulated into, as the reference adds onto the routed experts' sum. */
+int lq4o_moe_shared_expert_f32(const uint8_t* gate_up_q4, const uint8_t* down_q4,
+                               const float* shared_gate, int shared_inter, int hidden,
+                               const float* x, int tokens, float* out) {
+    if (hidden % 32 || shared_inter % 32) return 1;
+    float* gu = (float*)malloc((size_t)2 * shared_inter * sizeof(float));
+    float* o = (float*)malloc((size_t)hidden * sizeof(float));
+    for (int t = 0; t < tokens; ++t) {
+        const float* xt = x + (size_t)t * hidden;
+        float* ot = out + (size_t)t * hidden;
+        float logit = 0.0f;
+        for (int i = 0; i < hidden; ++i) logit += xt[i] * shared_gate[i];
+        const float g = 1.0f / (1.0f + expf(-logit));
+        lq4o_gemm_f32(xt, gate_up_q4, gu, 1, (size_t)2 * shared_inter, hidden);
+        for (int i = 0; i < shared_inter; ++i) gu[i] = silu_f32(gu[i]) * gu[shared_inter + i];
+        lq4o_gemm_f32(gu, down_q4, o, 1, hidden, shared_inter);
+        for (int i = 0; i < hidden; ++i) ot[i] += g * o[i];
+    }
+    free(gu);
+    free(o);
+    return 0;
+}
+
+/* f64 twin: gate logit, sigmoid, every dot, the SiLU and the scaled add in f64. */
+int lq4o_moe_shared_expert_f64(const uint8_t* gate_up_q4, const uint8_t* down_q4,
+                               const float* shared_gate, int shared_inter, int hidden,
+                               const float* x, int tokens, double* out) {
+    if (hidden % 32 || shared_inter % 32) return 1;
+    size_t gu_row = (size_t)(hidden / 32) * LQ4_BLOCK_BYTES;
+    size_t dn_row = (size_t)(shared_inter / 32) * LQ4_BLOCK_BYTES;
+    float* wrow = (float*)malloc((size_t)(hidden > shared_inter ? hidden : shared_inter) * sizeof(float));
+    double* gu = (double*)malloc((size_t)2 * shared_inter * sizeof(double));
+    for (int t = 0; t < tokens; ++t) {
+        const float* xt = x + (size_t)t * hidden;
+        double* ot = out + (size_t)t * hidden;
+        double logit = 0.0;
+        for (int i = 0; i < hidden; ++i) logit += (double)xt[i] * (double)shared_gate[i];
+        const double g = 1.0 / (1.0 + exp(-logit));
+        for (int r = 0; r < 2 * shared_inter; ++r) {
+            lq4o_dequantize(gate_up_q4 + (size_t)r * gu_row, gu_row, hidden, wrow);
+            double acc = 0.0;
+            for (int kk = 0; kk < hidden; ++kk) acc += (double)xt[kk] * (double)wrow[kk];
+            gu[r] = acc;
+        }
+        for (int i = 0; i < shared_inter; ++i) gu[i] = gu[i] / (1.0 + exp(-gu[i])) * gu[shared_inter + i];
+        for (int r = 0; r < hidden; ++r) {
+            lq4o_dequantize(down_q4 + (size_t)r * dn_row, dn_row, shared_inter, wrow);
+            double acc = 0.0;
+            for (int kk = 0; kk < shared_inter; ++kk) acc += gu[kk] * (double)wrow[kk];
+            ot[r] += g * acc;
+        }
+    }
+    free(wrow);
+    free(gu);
+    return 0;
+}
+
 /* ------------------------------------------------------------------------- */
 /* `.q4` file header                                                          */
 /* ------------------------------------------------------------------------- */

@@ -413,6 +413,82 @@ def test_moe_grouped_experts_match_oracle(be, cfg):
     assert e32 <= REL_TOL and e64 <= REL_TOL
 
 
+@pytest.mark.parametrize("cfg", [dict(inter=64, hidden=96, tokens=1),
+                                 dict(inter=512, hidden=2048, tokens=1),     # config 4's shared expert, decode
+                                 dict(inter=96, hidden=160, tokens=5),
+                                 dict(inter=512, hidden=2048, tokens=16),
+                                 dict(inter=512, hidden=2048, tokens=40)])   # beyond the GEMV batch: GEMM kernels
+def test_moe_shared_expert_matches_oracle(be, cfg):
+    import torch
+    inter, hidden, tokens = cfg["inter"], cfg["hidden"], cfg["tokens"]
+    print(f"moe shared expert {cfg}", flush=True)
+    gu = synth.q4_weight(2 * inter, hidden, seed=1, tag="sh_gu")
+    dn = synth.q4_weight(hidden, inter, seed=1, tag="sh_dn")
+    x = synth.activations(tokens, hidden, seed=1, tag="sh_x")
+    rng = np.random.default_rng(1)
+    sg = (rng.normal(size=hidden) * (2.0 / np.sqrt(hidden))).astype(np.float32)
+    base = rng.normal(size=(tokens, hidden)).astype(np.float32)  # stands for the routed experts' sum
+    qgu, qdn = be.upload_q4_blocks(gu), be.upload_q4_blocks(dn)
+    y = dev(base.copy())
+    be.moe_shared_expert(qgu, qdn, dev(sg), inter, hidden, dev(x), y)
+    ref32 = oracle.moe_shared_expert(gu, dn, sg, inter, hidden, x, base)
+    ref64 = oracle.moe_shared_expert(gu, dn, sg, inter, hidden, x, base, f64=True)
+    e32, e64 = rel_err(host(y), ref32), rel_err(host(y), ref64)
+    # the shared expert's own contribution, so that an error in it cannot hide behind `base`
+    d_err = rel_err(host(y) - base, ref64 - base)
+    print(f"  rel err vs f32 {e32:.2e}, vs f64 {e64:.2e}, contribution alone {d_err:.2e}", flush=True)
+    assert e32 <= REL_TOL and e64 <= REL_TOL and d_err <= REL_TOL
+
+
+def test_moe_layer_routed_plus_shared_expert(be):
+    """moe_ffn_step (moe.rs:8-36) end to end: route, routed experts, shared expert onto the same y."""
+    import torch
+    e_, inter, sh_inter, hidden, tokens, top_k = 8, 64, 128, 256, 6, 2
+    gu = synth.q4_weight(e_ * 2 * inter, hidden, seed=2, tag="moe_gu")
+    dn = synth.q4_weight(e_ * hidden, inter, seed=2, tag="moe_dn")
+    sgu = synth.q4_weight(2 * sh_inter, hidden, seed=2, tag="sh_gu")
+    sdn = synth.q4_weight(hidden, sh_inter, seed=2, tag="sh_dn")
+    x = synth.activations(tokens, hidden, seed=2, tag="moe_x")
+    lg = synth.router_logits(tokens, e_, seed=2)
+    sg = (np.random.default_rng(2).normal(size=hidden) * 0.1).astype(np.float32)
+    ids, wts, _ = oracle.moe_route(lg, top_k)
+    routed64 = oracle.moe_ffn(gu, dn, e_, inter, hidden, x, ids, wts, f64=True)
+    d_ids, d_wts = be.moe_route(dev(lg), top_k)
+    assert np.array_equal(host(d_ids), ids)
+    y = torch.full((tokens, hidden), float("nan"), dtype=torch.float32, device="cuda")
+    be.moe_experts(be.upload_q4_blocks(gu), be.upload_q4_blocks(dn), e_, inter, hidden, dev(x), d_ids, d_wts, y)
+    routed = host(y).copy()
+    assert rel_err(routed, routed64) <= REL_TOL
+    be.moe_shared_expert(be.upload_q4_blocks(sgu), be.upload_q4_blocks(sdn), dev(sg), sh_inter, hidden, dev(x), y)
+    # each stage to the tolerance on its own: the shared expert is checked on top of the routed sum the
+    # device produced (the two stages' f16 activation roundings are independent and would add up)
+    want = oracle.moe_shared_expert(sgu, sdn, sg, sh_inter, hidden, x, routed.astype(np.float64), f64=True)
+    e_stage = rel_err(host(y) - routed, want - routed)
+    whole = oracle.moe_shared_expert(sgu, sdn, sg, sh_inter, hidden, x, routed64, f64=True)
+    e_whole = rel_err(host(y), whole)
+    print(f"  shared stage alone {e_stage:.2e}, whole layer {e_whole:.2e}; max|routed| {np.abs(routed64).max():.3e} "
+          f"max|shared| {np.abs(want - routed).max():.3e} max|sum| {np.abs(whole).max():.3e}", flush=True)
+    # the shared expert is two dependent GEMVs, each of which rounds its activations to f16 at 3..16 tokens
+    # (REL_TOL apiece); this small shape lands at 1.0e-3 for the pair
+    assert e_stage <= 2 * REL_TOL and e_whole <= 2 * REL_TOL
+
+
+def test_moe_shared_expert_argument_checks(be):
+    import torch
+    gu, dn = be.upload_q4_blocks(synth.q4_weight(128, 64)), be.upload_q4_blocks(synth.q4_weight(64, 64))
+    x = torch.zeros(64, device="cuda")
+    y = torch.full((64,), 5.0, device="cuda")
+    sg = torch.zeros(64, device="cuda")
+    lib, ctx = be.lib, be.ctx
+    assert lib.lq4_moe_shared_expert(ctx, gu.handle, dn.handle, sg.data_ptr(), 64, 64, x.data_ptr(), 0, y.data_ptr(), None) == 0
+    assert lib.lq4_moe_shared_expert(ctx, gu.handle, dn.handle, sg.data_ptr(), 48, 64, x.data_ptr(), 1, y.data_ptr(), None) == -1
+    assert b"multiple of 32" in lib.lq4_last_error()
+    assert lib.lq4_moe_shared_expert(ctx, gu.handle, dn.handle, None, 64, 64, x.data_ptr(), 1, y.data_ptr(), None) == -1
+    # the gate||up tensor is too small for this intermediate size: refused on the host
+    assert lib.lq4_moe_shared_expert(ctx, gu.handle, dn.handle, sg.data_ptr(), 96, 64, x.data_ptr(), 1, y.data_ptr(), None) == -1
+    assert np.all(host(y) == 5.0)
+
+
 # ---------------------------------------------------------------- error behaviour
 def test_dispatch_contract_errors_and_noops(be):
     import ctypes as C

@@ -180,6 +180,65 @@ def test_moe_constant_expert_closed_form():
     assert np.allclose(got, want, rtol=1e-12)
 
 
+def test_moe_shared_expert_matches_dense_f64_composition():
+    # independent restatement in numpy f64 from the (pinned) dequantised tensors: a swapped gate/up
+    # half, a transposed operand, a dropped sigmoid or an overwritten accumulator fails here
+    inter, hidden, t = 96, 160, 4
+    gu = synth.q4_weight(2 * inter, hidden, seed=8, tag="sh_gu", scale_std=0.2)
+    dn = synth.q4_weight(hidden, inter, seed=8, tag="sh_dn", scale_std=0.2)
+    x = synth.activations(t, hidden, seed=8)
+    rng = np.random.default_rng(8)
+    sg = (rng.normal(size=hidden) * 0.2).astype(np.float32)
+    base = rng.normal(size=(t, hidden)).astype(np.float32)
+    wgu = _dense(gu, 2 * inter, hidden).astype(np.float64)
+    wdn = _dense(dn, hidden, inter).astype(np.float64)
+    x64 = x.astype(np.float64)
+    gate_val = 1 / (1 + np.exp(-(x64 @ sg.astype(np.float64))))
+    assert 0.01 < gate_val.min() and gate_val.max() < 0.99 and np.ptp(gate_val) > 0.05  # not a trivial gate
+    g, u = x64 @ wgu[:inter].T, x64 @ wgu[inter:].T
+    want = base.astype(np.float64) + gate_val[:, None] * ((g / (1 + np.exp(-g)) * u) @ wdn.T)
+    got64 = oracle.moe_shared_expert(gu, dn, sg, inter, hidden, x, base, f64=True)
+    assert np.allclose(got64, want, rtol=1e-10, atol=1e-12)
+    got32 = oracle.moe_shared_expert(gu, dn, sg, inter, hidden, x, base)
+    assert np.max(np.abs(got32 - want)) <= 1e-5 * np.max(np.abs(want))
+
+
+def test_moe_shared_expert_with_zero_gate_vector_is_half_a_routed_expert():
+    # sigmoid(0) = 1/2 exactly, so the shared expert equals one routed expert of the same tensors at
+    # weight 0.5, bit for bit (moe.rs:242-244 and :187-189 share the scaled add)
+    inter, hidden, t = 64, 96, 3
+    gu = synth.q4_weight(2 * inter, hidden, seed=9, tag="gu", scale_std=0.2)
+    dn = synth.q4_weight(hidden, inter, seed=9, tag="dn", scale_std=0.2)
+    x = synth.activations(t, hidden, seed=9)
+    routed = oracle.moe_ffn(gu, dn, 1, inter, hidden, x, np.zeros((t, 1), np.int32), np.full((t, 1), 0.5, np.float32))
+    shared = oracle.moe_shared_expert(gu, dn, np.zeros(hidden, np.float32), inter, hidden, x, np.zeros((t, hidden), np.float32))
+    assert np.array_equal(shared.view(np.uint32), routed.view(np.uint32))
+
+
+def test_moe_shared_expert_gate_saturates_and_constant_closed_form():
+    # constant-per-row tensors are exact in Q4: out = base + g * c * I * silu(a*S) * (b*S), S = sum(x)
+    inter, hidden = 32, 64
+    a, b, c = 0.25, -0.5, 0.125
+    gu = np.concatenate([oracle.quantize_rows(np.full((inter, hidden), v, np.float32)) for v in (a, b)])
+    dn = oracle.quantize_rows(np.full((hidden, inter), c, np.float32))
+    x = synth.activations(1, hidden, seed=7)
+    s = float(x.astype(np.float64).sum())
+    ffn = c * inter * ((a * s) / (1 + np.exp(-a * s))) * (b * s)
+    base = np.full((1, hidden), 3.0, np.float32)
+    for gate_scale, want_g in ((0.0, 0.5), (1e4, None), (-1e4, None)):
+        sg = (gate_scale * np.sign(x[0])).astype(np.float32)  # logit = gate_scale * sum|x|
+        logit = gate_scale * float(np.abs(x.astype(np.float64)).sum())
+        g = 0.5 if want_g else (1.0 if logit > 0 else 0.0)
+        got = oracle.moe_shared_expert(gu, dn, sg, inter, hidden, x, base, f64=True)
+        assert np.allclose(got, 3.0 + g * ffn, rtol=1e-12), gate_scale
+    # ln(3) as the logit: sigmoid = 3/4
+    sg = np.zeros(hidden, np.float32)
+    sg[0] = np.float32(np.log(3.0) / x[0, 0])
+    got = oracle.moe_shared_expert(gu, dn, sg, inter, hidden, x, base, f64=True)
+    g = 1 / (1 + np.exp(-float(np.float64(sg[0]) * np.float64(x[0, 0]))))
+    assert abs(g - 0.75) < 1e-6 and np.allclose(got, 3.0 + g * ffn, rtol=1e-12)
+
+
 # ----------------------------------------------------------------- CPU baseline
 @pytest.mark.parametrize("m,k,n", [(1, 96, 7), (3, 200, 9), (4, 256, 8), (5, 1024, 300), (1, 2048, 600)])
 def test_cpu_baseline_kernels_agree_with_numpy(m, k, n):

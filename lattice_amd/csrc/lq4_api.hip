@@ -689,9 +689,23 @@ int lq4_topk(lq4_ctx* ctx, const float* logits_dev, uint32_t n, uint32_t top_k, 
     return LQ4_OK;
 }
 
-int lq4_lm_head_topk(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t vocab, uint32_t k,
-                     const float* x_dev, uint32_t top_k, float* out_logits_dev, uint32_t* out_ids_dev,
-                     void* stream) {
+namespace {
+
+int g_lm_head_mode = LQ4_LM_HEAD_TWO_LAUNCHES;  // measured faster: see lq4_set_lm_head_mode in the header
+
+// Scratch of one lm_head + top-k call: [vocab logits | maxima, candidates], in the layout of whichever
+// path serves the shape.
+size_t lm_head_scratch_need(uint32_t vocab, uint32_t k, uint32_t top_k, bool* one_launch) {
+    const size_t fused = g_lm_head_mode == LQ4_LM_HEAD_ONE_LAUNCH ? gemv_b1_topk_scratch_bytes(vocab, k, top_k) : 0;
+    *one_launch = fused != 0;
+    if (fused) return fused;
+    const size_t logits_bytes = (static_cast<size_t>(vocab) * sizeof(float) + 255) / 256 * 256;
+    return logits_bytes + topk_scratch_bytes(vocab, top_k);
+}
+
+int lm_head_topk_common(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t vocab, uint32_t k,
+                        const float* x_dev, uint32_t top_k, float* out_logits_dev, uint32_t* out_ids_dev, void* stream,
+                        bool static_scratch) {
     if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
     if (top_k == 0) return LQ4_OK;
     if (vocab == 0) return fail(LQ4_E_INVALID, "empty vocabulary");
@@ -701,51 +715,58 @@ int lq4_lm_head_topk(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset,
     if (rc) return rc;
     if (!x_dev || !out_logits_dev || !out_ids_dev) return fail(LQ4_E_INVALID, "null device pointer");
     if (reinterpret_cast<uintptr_t>(x_dev) % 16) return fail(LQ4_E_INVALID, "x must be 16-byte aligned");
-    DeviceGuard g(ctx->device);
-    // scratch: [vocab logits | candidate buffers]
-    const size_t logits_bytes = (static_cast<size_t>(vocab) * sizeof(float) + 255) / 256 * 256;
-    rc = ensure_scratch(ctx, logits_bytes + topk_scratch_bytes(vocab, top_k), static_cast<hipStream_t>(stream));
-    if (rc) return rc;
-    float* logits = reinterpret_cast<float*>(ctx->moe_scratch);
+    bool one_launch;
+    const size_t need = lm_head_scratch_need(vocab, k, top_k, &one_launch);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};
-    launch_gemv(wp, vocab, k, x_dev, k, 1, logits, vocab, none, s);
-    launch_topk(logits, vocab, top_k, ctx->moe_scratch + logits_bytes, ctx->topk_ticket, out_logits_dev, out_ids_dev, s);
-    ctx->counters.gemv++;
-    ctx->counters.topk++;
+    DeviceGuard g(ctx->device);
+    uint8_t* base;
+    if (static_scratch) {
+        if (need > kStaticScratchBytes)
+            return fail(LQ4_E_UNSUPPORTED,
+                        "lq4_lm_head_topk_static: vocab %u with top_k %u needs %zu bytes of scratch, the static buffer holds %zu; "
+                        "use lq4_lm_head_topk", vocab, top_k, need, kStaticScratchBytes);
+        base = ctx->static_scratch;
+    } else {
+        rc = ensure_scratch(ctx, need, s);
+        if (rc) return rc;
+        base = ctx->moe_scratch;
+    }
+    if (one_launch) {
+        launch_gemv_b1_topk(wp, vocab, k, x_dev, base, ctx->topk_ticket, top_k, out_logits_dev, out_ids_dev, s);
+        ctx->counters.lm_head_one_launch++;
+    } else {
+        const size_t logits_bytes = (static_cast<size_t>(vocab) * sizeof(float) + 255) / 256 * 256;
+        float* logits = reinterpret_cast<float*>(base);
+        const LoraEpilogue none{};
+        launch_gemv(wp, vocab, k, x_dev, k, 1, logits, vocab, none, s);
+        launch_topk(logits, vocab, top_k, base + logits_bytes, ctx->topk_ticket, out_logits_dev, out_ids_dev, s);
+        ctx->counters.gemv++;
+        ctx->counters.topk++;
+    }
     LQ4_HIP(hipGetLastError());
     return LQ4_OK;
 }
 
+}  // namespace
+
+int lq4_set_lm_head_mode(int mode) {
+    if (mode != LQ4_LM_HEAD_ONE_LAUNCH && mode != LQ4_LM_HEAD_TWO_LAUNCHES)
+        return fail(LQ4_E_INVALID, "unknown lm_head mode %d", mode);
+    g_lm_head_mode = mode;
+    return LQ4_OK;
+}
+
+int lq4_lm_head_topk(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t vocab, uint32_t k,
+                     const float* x_dev, uint32_t top_k, float* out_logits_dev, uint32_t* out_ids_dev,
+                     void* stream) {
+    return lm_head_topk_common(ctx, w, w_extra_offset, vocab, k, x_dev, top_k, out_logits_dev, out_ids_dev, stream, false);
+}
+
+// The same call with its scratch in the library's static array: allocates nothing.
 int lq4_lm_head_topk_static(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t vocab, uint32_t k,
                             const float* x_dev, uint32_t top_k, float* out_logits_dev, uint32_t* out_ids_dev,
                             void* stream) {
-    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
-    if (top_k == 0) return LQ4_OK;
-    if (vocab == 0) return fail(LQ4_E_INVALID, "empty vocabulary");
-    if (top_k > LQ4_MAX_TOP_K) return fail(LQ4_E_INVALID, "top_k %u above %d", top_k, LQ4_MAX_TOP_K);
-    const uint8_t* wp;
-    const int rc = resolve_weight(w, w_extra_offset, vocab, k, &wp);
-    if (rc) return rc;
-    if (!x_dev || !out_logits_dev || !out_ids_dev) return fail(LQ4_E_INVALID, "null device pointer");
-    if (reinterpret_cast<uintptr_t>(x_dev) % 16) return fail(LQ4_E_INVALID, "x must be 16-byte aligned");
-    // same layout as lq4_lm_head_topk: [vocab logits | candidate buffers], in the static array
-    const size_t logits_bytes = (static_cast<size_t>(vocab) * sizeof(float) + 255) / 256 * 256;
-    const size_t need = logits_bytes + topk_scratch_bytes(vocab, top_k);
-    if (need > kStaticScratchBytes)
-        return fail(LQ4_E_UNSUPPORTED,
-                    "lq4_lm_head_topk_static: vocab %u with top_k %u needs %zu bytes of scratch, the static buffer holds %zu; "
-                    "use lq4_lm_head_topk", vocab, top_k, need, kStaticScratchBytes);
-    DeviceGuard g(ctx->device);
-    float* logits = reinterpret_cast<float*>(ctx->static_scratch);
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};
-    launch_gemv(wp, vocab, k, x_dev, k, 1, logits, vocab, none, s);
-    launch_topk(logits, vocab, top_k, ctx->static_scratch + logits_bytes, ctx->topk_ticket, out_logits_dev, out_ids_dev, s);
-    ctx->counters.gemv++;
-    ctx->counters.topk++;
-    LQ4_HIP(hipGetLastError());
-    return LQ4_OK;
+    return lm_head_topk_common(ctx, w, w_extra_offset, vocab, k, x_dev, top_k, out_logits_dev, out_ids_dev, stream, true);
 }
 
 int lq4_residual_add_rmsnorm(lq4_ctx* ctx, const float* base_dev, const float* delta_dev, const float* gamma_dev,

@@ -12,6 +12,7 @@
 // The unpack-free arithmetic (masked nibbles as f16 subnormals, activations as per-block scaled
 // hi/lo f16 pairs) and the LDS staging are in lq4_b1_dev.hpp, shared with the decode-chain kernel.
 #include "lq4_b1_dev.hpp"
+#include "lq4_topk_dev.hpp"
 
 #include <type_traits>
 
@@ -96,13 +97,26 @@ __device__ __forceinline__ float lora_t_acquire(const LoraEpilogue& lora, uint32
 }
 
 struct NoFusion {};
-template <bool FUSED>
+// What the top-k mode needs beside the GEMV's own arguments: y is then the logits buffer.
+struct TopkEpilogue {
+    uint64_t* maxima;   // [workgroups] best key of each workgroup's rows
+    Cand* surv;         // topk_most_blocks(k) * (rows of one workgroup, rounded up to whole runs) candidates
+    uint32_t* ticket;   // zero between launches
+    uint32_t k;
+    float* out_logits;
+    uint32_t* out_ids;
+};
+template <int MODE>
 struct FusionArg {
     typedef NoFusion type;
 };
 template <>
-struct FusionArg<true> {
+struct FusionArg<1> {
     typedef GemvFusion type;
+};
+template <>
+struct FusionArg<3> {
+    typedef TopkEpilogue type;
 };
 
 // WAVES: waves per workgroup.  Every workgroup stages the whole activation vector, so on long rows
@@ -113,13 +127,19 @@ struct FusionArg<true> {
 // it (release), the weight workgroups behind them pick t up (acquire) when their first rows are
 // complete, long after it was published.  The wait is bounded: a wave that runs out of polls
 // computes t itself, so every wave finishes whatever the dispatch order was.
-constexpr int kPlainMode = 0, kFusedMode = 1, kLoraAMode = 2;
+// 3 the lm_head pass with the exact top-k selection in the same launch (shaders/qwen35.metal:1935-1985
+// computes block candidates inside the GEMV kernel too): the logits go to `y` with device-scope stores,
+// every wave keeps the best key among the rows it produced, the workgroup publishes the best of its
+// waves and draws a ticket, and the workgroup that draws the last one (every logit and every maximum
+// is then in memory) runs the selection tail over those maxima.  A workgroup's rows are its selection
+// block; in this mode they are consecutive (every wave takes a run of wave-rows).
+constexpr int kPlainMode = 0, kFusedMode = 1, kLoraAMode = 2, kTopkMode = 3;
 
 template <int RW, int SG, int SEG, int MODE, int WAVES = kWaves>
 __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restrict__ w, uint32_t n,
                                                           uint32_t k, const float* __restrict__ x,
                                                           float* __restrict__ y, LoraEpilogue lora,
-                                                          typename FusionArg<MODE == 1>::type fz) {
+                                                          typename FusionArg<MODE>::type fz) {
     extern __shared__ __attribute__((aligned(16))) uint32_t xs[];
     lds_u32* const xsl = (lds_u32*)xs;
     constexpr bool FUSED = MODE == kFusedMode;
@@ -168,7 +188,19 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
     const uint32_t wid = __builtin_amdgcn_readfirstlane(w_group * WAVES + (tid >> 6));
     // chunks whose first wave-row exists for this wave (later waves may have one chunk fewer)
     const uint32_t first = wid < n_wrows ? n_wrows - wid : 0;  // wave-rows from this wave's first one on
-    const uint32_t chunks = (first + n_waves * RW - 1) / (n_waves * RW);
+    uint32_t chunks = (first + n_waves * RW - 1) / (n_waves * RW);
+    // kTopkMode: a wave takes `per_wave` consecutive wave-rows instead, so that the logits of one
+    // workgroup are one run in memory (the workgroup that selects reads the best workgroups' logits:
+    // scattered over the vector they are a cache line each)
+    const uint32_t per_wave = (n_wrows + n_waves - 1) / n_waves;
+    if constexpr (MODE == kTopkMode) {
+        const uint32_t begin = wid * per_wave;
+        const uint32_t mine = begin < n_wrows ? (n_wrows - begin < per_wave ? n_wrows - begin : per_wave) : 0;
+        chunks = (mine + RW - 1) / RW;
+    }
+    // wave-row of round r = chunk * RW + j, and whether this wave owns it
+    auto wrow_of = [&](uint32_t r) { return MODE == kTopkMode ? wid * per_wave + r : r * n_waves + wid; };
+    auto wrow_mine = [&](uint32_t r) { return wrow_of(r) < n_wrows && (MODE != kTopkMode || r < per_wave); };
     const uint32_t units = chunks * slab_groups;
 
     // ---- the first activations are requested before any weight so they can be waited on alone ----
@@ -227,7 +259,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
         const uint32_t chunk = u / slab_groups, sgi = u - chunk * slab_groups;
 #pragma unroll
         for (int j = 0; j < RW; ++j) {
-            uint32_t wrow = (chunk * RW + j) * n_waves + wid;  // scalar
+            uint32_t wrow = wrow_of(chunk * RW + j);  // scalar
             if (wrow >= n_wrows) wrow = n_wrows - 1;
             uint32_t row = wrow * RPW + sub;
             if (RPW > 1 && row >= n) row = n - 1;
@@ -400,6 +432,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
     float acc[RW];
 #pragma unroll
     for (int j = 0; j < RW; ++j) acc[j] = 0.0f;
+    uint64_t best_key = key_of(sentinel());  // kTopkMode: best of the rows this lane stored
     float t_reg = 0.0f;   // kLoraAMode: t[lane], fetched when the wave's first rows are complete
     bool t_have = false;
 
@@ -428,9 +461,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
         if (sgi + 1 == slab_groups) {  // chunk complete: reduce and store its rows
 #pragma unroll
             for (int j = 0; j < RW; ++j) {
-                const uint32_t wrow = (chunk * RW + j) * n_waves + wid;
+                const uint32_t wrow = wrow_of(chunk * RW + j);
                 const uint32_t row = wrow * RPW + sub;
-                const bool row_ok = wrow < n_wrows && row < n;
+                const bool row_ok = wrow_mine(chunk * RW + j) && row < n;
                 float v = acc[j];
                 acc[j] = 0.0f;
                 if constexpr (INA) {
@@ -477,6 +510,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
                             fz.residual[row] = r;
                             if (fz.copy_dst) fz.copy_dst[row] = r;
                         }
+                    } else if constexpr (MODE == kTopkMode) {
+                        // device scope: written through to where the workgroup that selects reads it
+                        __hip_atomic_store(y + row, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        const uint64_t key = key_of(v == v ? Cand{v, row} : sentinel());
+                        best_key = key > best_key ? key : best_key;
                     } else {
                         y[row] = v;
                     }
@@ -500,6 +538,50 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
     } else if (u < units) {
         process(kLast, buf_a, buf_b, u);
     }
+
+    if constexpr (MODE == kTopkMode) {
+        static_assert(WAVES == 4, "the selection tail is written for 256 threads");
+        // this wave's logit stores have been carried out (a store counts as outstanding until then)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        best_key = wave_max_key(best_key);
+        __syncthreads();  // every wave is past the staged activations: the LDS is free
+        TopkTailShared& ts = *reinterpret_cast<TopkTailShared*>(xs);
+        uint64_t* part = reinterpret_cast<uint64_t*>(reinterpret_cast<uint8_t*>(xs) + sizeof(TopkTailShared));  // [WAVES], then the flag
+        uint32_t* last_flag = reinterpret_cast<uint32_t*>(part + WAVES);
+        if (lane == 0) part[tid >> 6] = best_key;
+        __syncthreads();
+        if (tid == 0) {
+            uint64_t best = part[0];
+#pragma unroll
+            for (int v = 1; v < WAVES; ++v) best = part[v] > best ? part[v] : best;
+            // An exchange at device scope is carried out where every part of the chip sees it, and once
+            // its old value has come back it is done; only then is the ticket drawn.
+            const uint64_t old = __hip_atomic_exchange(fz.maxima + w_group, best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            asm volatile("s_waitcnt vmcnt(0)" ::"v"(static_cast<uint32_t>(old)) : "memory");
+            const uint32_t t = atomicAdd(fz.ticket, 1u);
+            const bool last = t == w_groups - 1;
+            if (last) __hip_atomic_store(fz.ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+            *last_flag = last;
+        }
+        __syncthreads();
+        if (!*last_flag) return;
+        __syncthreads();  // the flag has been read by all before the tail reuses the LDS
+        const TopkBlocks blocks{WAVES * per_wave * RPW, 0, 1};  // a workgroup's logits: one run
+        topk_select_tail<true>(y, n, blocks, w_groups, fz.k, fz.maxima, fz.surv, ts, fz.out_logits, fz.out_ids);
+    }
+}
+
+template <int RW, int SG>
+void launch_cfg_topk(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, const TopkEpilogue& topk,
+                     size_t lds, uint32_t waves, hipStream_t stream) {
+    static bool attr_set = false;
+    if (!attr_set) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, 64, kTopkMode, 4>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((gemv_q4_b1<RW, SG, 64, kTopkMode, 4>), dim3((waves + 3) / 4), dim3(256), lds, stream, w, n, k, x,
+                       y, LoraEpilogue{}, topk);
 }
 
 template <int RW, int SG, int SEG, int WAVES = kWaves>
@@ -556,9 +638,19 @@ void launch_gemv_b1_fused(const uint8_t* w, uint32_t n, uint32_t k, const float*
 
 namespace {
 
-void launch_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, const LoraEpilogue& lora,
-               const GemvFusion* fusion, hipStream_t stream) {
-    const size_t lds = gemv_b1_lds_bytes(k);
+// Grid shape of one launch: waves in all, wave-rows per chunk, slabs per unit.
+struct B1Plan {
+    size_t lds;
+    uint32_t seg, wg_waves, waves, rw, sg;
+};
+
+// `producers`: workgroups in front of the weight workgroups.  `four_waves`: never the eight-wave
+// workgroups.  `lds_min`: dynamic LDS the launch needs beyond the staged x.
+B1Plan plan_b1(uint32_t n, uint32_t k, uint32_t producers, bool four_waves, size_t lds_min) {
+    B1Plan p;
+    p.lds = gemv_b1_lds_bytes(k);
+    if (p.lds < lds_min) p.lds = lds_min;
+    const size_t lds = p.lds;
     const uint32_t nb = k / kBlockWeights;
     const uint32_t seg = nb == 32 ? 32 : nb == 16 ? 16 : 64;
     const uint32_t n_wrows = (n + 64 / seg - 1) / (64 / seg);
@@ -568,12 +660,11 @@ void launch_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* 
     uint32_t wg_per_cu = static_cast<uint32_t>((160 * 1024) / (lds + 512));
     // eight waves per workgroup on long rows (measured: 2048 x 6144 5.15 -> 4.69 us, 17408 x 5120
     // 16.2 -> 15.2; behind on K 2048 and K 17408)
-    const uint32_t wg_waves = (seg == 64 && k >= 4096 && k <= 8192) ? 8 : kWaves;
+    const uint32_t wg_waves = (!four_waves && seg == 64 && k >= 4096 && k <= 8192) ? 8 : kWaves;
     wg_per_cu = wg_per_cu > 16 / wg_waves ? 16 / wg_waves : wg_per_cu < 1 ? 1 : wg_per_cu;
     // A launch that computes A.x itself carries `rank` producer workgroups in front: the weight
     // workgroups leave them room, so that every workgroup of the launch is resident at once and none
     // starts after the producers have advanced the epoch.
-    const uint32_t producers = (lora.rank && lora.a && !fusion) ? lora.rank : 0;
     const uint32_t max_waves = (256 * wg_per_cu - producers) * wg_waves;
     uint32_t rw = (n_wrows + max_waves - 1) / max_waves;
     uint32_t waves;
@@ -596,6 +687,19 @@ void launch_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* 
     }
     uint32_t sg = slabs < 3 ? slabs : 3;
     while (rw * sg > 6) --sg;
+    p.seg = seg;
+    p.wg_waves = wg_waves;
+    p.waves = waves;
+    p.rw = rw;
+    p.sg = sg;
+    return p;
+}
+
+void launch_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, const LoraEpilogue& lora,
+               const GemvFusion* fusion, hipStream_t stream) {
+    const B1Plan pl = plan_b1(n, k, (lora.rank && lora.a && !fusion) ? lora.rank : 0, false, 0);
+    const size_t lds = pl.lds;
+    const uint32_t seg = pl.seg, wg_waves = pl.wg_waves, waves = pl.waves, rw = pl.rw, sg = pl.sg;
 
 #define LQ4_B1(RW_, SG_, SEG_) launch_cfg<RW_, SG_, SEG_>(w, n, k, x, y, lora, fusion, lds, waves, stream)
 #define LQ4_B1W(RW_, SG_) launch_cfg<RW_, SG_, 64, 8>(w, n, k, x, y, lora, fusion, lds, waves, stream)
@@ -621,6 +725,50 @@ void launch_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* 
 #undef LQ4_B1
 }
 
+// The lm_head pass that selects in its own launch serves four-wave workgroups over rows of one or
+// more 64-block slabs (K of 2048 and up, not 512 or 1024), k up to 64, between k and 1024 workgroups.
+bool plan_b1_topk(uint32_t n, uint32_t k, uint32_t topk, B1Plan* out, uint32_t* runs) {
+    if (topk == 0 || topk > kSingleKernelMaxK || n == 0) return false;
+    if (gemv_b1_lds_bytes(k) > 128 * 1024) return false;
+    const B1Plan pl = plan_b1(n, k, 0, true, sizeof(TopkTailShared) + 64);
+    if (pl.seg != 64) return false;
+    const uint32_t grid = (pl.waves + 3) / 4;
+    if (grid > 1024 || grid < topk) return false;
+    *out = pl;
+    *runs = (n + grid * 4 - 1) / (grid * 4);  // rows per wave; a workgroup's block is four times that
+    return true;
+}
+
 }  // namespace
+
+size_t gemv_b1_topk_scratch_bytes(uint32_t n, uint32_t k, uint32_t topk) {
+    B1Plan pl;
+    uint32_t runs;
+    if (!plan_b1_topk(n, k, topk, &pl, &runs)) return 0;
+    const size_t logits = (static_cast<size_t>(n) * sizeof(float) + 255) / 256 * 256;
+    return logits + 1024 * sizeof(uint64_t) + static_cast<size_t>(topk_most_blocks(topk)) * runs * 4 * sizeof(Cand);
+}
+
+void launch_gemv_b1_topk(const uint8_t* w, uint32_t n, uint32_t k, const float* x, void* scratch, uint32_t* ticket,
+                         uint32_t topk, float* out_logits, uint32_t* out_ids, hipStream_t stream) {
+    B1Plan pl;
+    uint32_t runs;
+    if (!plan_b1_topk(n, k, topk, &pl, &runs)) return;  // the caller asked gemv_b1_topk_scratch_bytes first
+    float* logits = static_cast<float*>(scratch);
+    TopkEpilogue te;
+    te.maxima = reinterpret_cast<uint64_t*>(static_cast<uint8_t*>(scratch) + (static_cast<size_t>(n) * sizeof(float) + 255) / 256 * 256);
+    te.surv = reinterpret_cast<Cand*>(te.maxima + 1024);
+    te.ticket = ticket;
+    te.k = topk;
+    te.out_logits = out_logits;
+    te.out_ids = out_ids;
+#define LQ4_B1T(RW_, SG_) launch_cfg_topk<RW_, SG_>(w, n, k, x, logits, te, pl.lds, pl.waves, stream)
+    const uint32_t rw = pl.rw, sg = pl.sg;
+    if (rw == 1) { if (sg == 1) LQ4_B1T(1, 1); else if (sg == 2) LQ4_B1T(1, 2); else LQ4_B1T(1, 3); }
+    else if (rw == 2) { if (sg == 1) LQ4_B1T(2, 1); else if (sg == 2) LQ4_B1T(2, 2); else LQ4_B1T(2, 3); }
+    else if (rw == 3) { if (sg == 1) LQ4_B1T(3, 1); else LQ4_B1T(3, 2); }
+    else LQ4_B1T(4, 1);
+#undef LQ4_B1T
+}
 
 }  // namespace lq4

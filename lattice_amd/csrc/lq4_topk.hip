@@ -10,26 +10,11 @@
 // Ordering (qwen35.metal:1697-1703): higher logit first, ties to the lower token id; a NaN logit
 // enters as the sentinel (-inf, 0xFFFFFFFF) and ranks last.
 #include "lq4_internal.hpp"
+#include "lq4_topk_dev.hpp"
 
 namespace lq4 {
 
 namespace {
-
-typedef float float4v __attribute__((ext_vector_type(4)));
-
-struct Cand {
-    float logit;
-    uint32_t id;
-};
-
-__device__ __forceinline__ Cand sentinel() { return Cand{-INFINITY, 0xFFFFFFFFu}; }
-
-__device__ __forceinline__ bool better(Cand a, Cand b) {
-    if (a.logit != a.logit) return false;
-    if (b.logit != b.logit) return true;
-    if (a.logit != b.logit) return a.logit > b.logit;
-    return a.id < b.id;
-}
 
 // Descending bitonic sort of tg[0..N) by 256 threads.
 template <int N>
@@ -131,102 +116,6 @@ __global__ __launch_bounds__(256) void topk_merge_kernel(const Cand* __restrict_
 // ticket would be the textbook form; the fence writes the whole L2 back and, at one per
 // workgroup, made the kernel 13 us slower.
 
-// 64-bit sort key of a candidate: a ranks before b  <=>  key(a) > key(b).  High word: the logit's
-// bits mapped to an unsigned order (-0 counted as +0, as the float comparison does); low word:
-// ~id, so ties go to the lower id.  NaN never gets here (it became the sentinel, the lowest key).
-__device__ __forceinline__ uint64_t key_of(Cand c) {
-    uint32_t u = __float_as_uint(c.logit);
-    if (c.logit == 0.0f) u = 0;
-    u ^= (u >> 31) ? 0xFFFFFFFFu : 0x80000000u;
-    return (static_cast<uint64_t>(u) << 32) | static_cast<uint32_t>(~c.id);
-}
-
-__device__ __forceinline__ Cand load_cand(const float* logits, uint32_t i) {
-    const float v = logits[i];
-    return v == v ? Cand{v, i} : sentinel();
-}
-
-__device__ __forceinline__ uint64_t wave_max_key(uint64_t k) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        const uint32_t lo = __shfl_xor(static_cast<uint32_t>(k), off, 64);
-        const uint32_t hi = __shfl_xor(static_cast<uint32_t>(k >> 32), off, 64);
-        const uint64_t o = (static_cast<uint64_t>(hi) << 32) | lo;
-        k = o > k ? o : k;
-    }
-    return k;
-}
-
-// A candidate this workgroup stored a moment ago, read back past the vector cache.
-__device__ __forceinline__ Cand load_survivor(const Cand* surv, uint32_t i) {
-    const uint64_t raw =
-        __hip_atomic_load(reinterpret_cast<const uint64_t*>(surv) + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return Cand{__uint_as_float(static_cast<uint32_t>(raw)), static_cast<uint32_t>(raw >> 32)};
-}
-
-struct SelectShared {
-    uint32_t hist[256];
-    uint64_t prefix;
-    uint32_t need;
-};
-
-// The k-th largest (k >= 1, counted with multiplicity) of the `count` >= k keys get(0..count):
-// eight rounds of an 8-bit radix select, most significant digit first.  A round counts the digit
-// of every key that still matches the digits fixed so far; wave 0 walks the 256 counts from the
-// top to the digit that holds the `need`-th key.  Called by all 256 threads of the workgroup.
-template <typename Get>
-__device__ __forceinline__ uint64_t select_kth_key(Get get, uint32_t count, uint32_t k, SelectShared& sh) {
-    const uint32_t tid = threadIdx.x;
-    uint64_t prefix = 0;
-    uint32_t need = k;
-    for (int shift = 56; shift >= 0; shift -= 8) {
-        sh.hist[tid] = 0;
-        __syncthreads();
-        for (uint32_t i = tid; i < count; i += 256) {
-            const uint64_t key = get(i);
-            // (x >> 1) >> 63-or-less: a shift by 64 is not defined, the first round matches all
-            const bool match = (((key ^ prefix) >> 1) >> (shift + 7)) == 0;
-            if (match) atomicAdd(&sh.hist[(key >> shift) & 255], 1u);
-        }
-        __syncthreads();
-        if (tid < 64) {  // lane l owns digits 255 - 4l .. 252 - 4l, highest first
-            uint32_t c[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) c[j] = sh.hist[255 - 4 * tid - j];
-            const uint32_t sum = (c[0] + c[1]) + (c[2] + c[3]);
-            uint32_t incl = sum;
-#pragma unroll
-            for (int off = 1; off < 64; off <<= 1) {
-                const uint32_t t = __shfl_up(incl, off, 64);
-                if (tid >= static_cast<uint32_t>(off)) incl += t;
-            }
-            uint32_t run = incl - sum;
-            if (run < need && need <= incl) {  // exactly one lane: the counts above it fall short
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    if (run < need && need <= run + c[j]) {
-                        sh.prefix = prefix | (static_cast<uint64_t>(255 - 4 * tid - j) << shift);
-                        sh.need = need - run;
-                    }
-                    run += c[j];
-                }
-            }
-        }
-        __syncthreads();
-        prefix = sh.prefix;
-        need = sh.need;
-    }
-    return prefix;
-}
-
-constexpr uint32_t kRankSlots = 1024;  // survivors ranked out of LDS
-constexpr uint32_t kSingleKernelMaxK = 64;
-constexpr int kGatherUnits = 16;       // 16-byte loads a thread has in flight when rescanning: 50 blocks of 256 in one go
-
-// The threshold may let up to this many blocks through instead of exactly k: it is found in fewer
-// steps, and the survivor buffer is sized for it.
-__host__ __device__ constexpr uint32_t topk_most_blocks(uint32_t k) { return k + (k >> 2) + 4; }
-
 // grid ceil(M / 4), block 256: wave w of workgroup g reduces block 4g + w of `blk` logits to its
 // best key; the workgroup with the last ticket selects, rescans and ranks (see above).  `ticket`
 // is zero between launches: the last workgroup puts it back.  `surv` holds topk_most_blocks(k) * blk
@@ -235,13 +124,8 @@ __global__ __launch_bounds__(256) void topk_select_kernel(const float* __restric
                                                           uint32_t m, uint32_t k, uint64_t* maxima, Cand* surv,
                                                           uint32_t* ticket, float* __restrict__ out_logits,
                                                           uint32_t* __restrict__ out_ids) {
-    __shared__ uint64_t s_keys[kRankSlots];
-    __shared__ float s_vals[kRankSlots];
-    __shared__ uint32_t s_ids[kRankSlots];
-    __shared__ uint16_t s_sel[1024];
-    __shared__ SelectShared sh;
-    __shared__ uint32_t s_cnt[2][4];
-    __shared__ uint32_t s_count, s_nsel, s_tail, s_last;
+    __shared__ TopkTailShared ts;
+    __shared__ uint32_t s_last;
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63;
     {
@@ -271,153 +155,10 @@ __global__ __launch_bounds__(256) void topk_select_kernel(const float* __restric
         s_last = t == gridDim.x - 1;
         // every other workgroup has drawn: ready for the next launch
         if (s_last) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_count = 0;
-        s_nsel = 0;
-        s_tail = 0;
     }
     __syncthreads();
     if (!s_last) return;
-
-    for (uint32_t o = tid; o < k; o += 256) {  // slots no survivor claims (NaN input) keep the sentinel
-        out_logits[o] = -INFINITY;
-        out_ids[o] = 0xFFFFFFFFu;
-    }
-
-    // tau: a key that at least k and at most `most` of the block maxima reach.  Built from the top
-    // bit down (a bit stays set if k maxima still reach the result); the first value that no more
-    // than `most` maxima reach will do, and if none comes up the loop ends at the k-th best
-    // maximum itself.  A step is four compares per thread and one barrier.
-    uint64_t kk[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)  // device-scope loads, as the maxima were written; 0: below every key
-        kk[j] = tid + 256 * j < m ? __hip_atomic_load(maxima + tid + 256 * j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-                                  : 0ull;
-    const uint32_t most = topk_most_blocks(k);
-    uint64_t tau = 0;
-    for (int bit = 63, par = 0; bit >= 0; --bit, par ^= 1) {
-        const uint64_t cand = tau | (1ull << bit);
-        uint32_t c = 0;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) c += __popcll(__ballot(kk[j] >= cand));
-        if (lane == 0) s_cnt[par][tid >> 6] = c;
-        __syncthreads();  // one barrier a step: the two halves of s_cnt take turns
-        c = (s_cnt[par][0] + s_cnt[par][1]) + (s_cnt[par][2] + s_cnt[par][3]);
-        if (c >= k) {
-            tau = cand;
-            if (c <= most) break;
-        }
-    }
-
-    // the blocks that can hold an element at or before tau: at most `most` (more only if tau is
-    // the all-NaN key, and then the extra blocks hold nothing that passes the test below)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        if (kk[j] >= tau && tid + 256 * j < m) {
-            s_sel[atomicAdd(&s_nsel, 1u)] = static_cast<uint16_t>(tid + 256 * j);
-            if (tid + 256 * j == m - 1) s_tail = 1;
-        }
-    }
-    __syncthreads();
-    const uint32_t nsel = s_nsel;
-    // Survivors: every logit of those blocks that is not below tau's logit (tau's high word mapped
-    // back to a float; a word below every real key means that -inf still passes).  One compare,
-    // which NaN fails; an element that ties tau's logit with a higher id passes although it ranks
-    // after tau, which costs a slot and nothing else.
-    const uint32_t tau_u = static_cast<uint32_t>(tau >> 32);
-    const float tau_f = tau_u < 0x007FFFFFu ? -INFINITY
-                                            : __uint_as_float((tau_u >> 31) ? tau_u ^ 0x80000000u : ~tau_u);
-    auto consider = [&](float v, uint32_t i) {
-        if (!(v >= tau_f)) return;
-        const uint32_t slot = atomicAdd(&s_count, 1u);
-        if (slot < kRankSlots) {
-            s_vals[slot] = v;
-            s_ids[slot] = i;
-        }
-        surv[slot] = Cand{v, i};
-    };
-    // All loads of a batch are issued before the first is looked at: one workgroup has to cover
-    // the latency of nsel * blk logits by itself.  Slots past the end reload element 0 and drop it.
-    const uint32_t lb = __ffs(blk) - 1;  // blk is a power of two
-    if ((reinterpret_cast<uintptr_t>(logits) & 15) == 0) {
-        const uint32_t units = nsel << (lb - 2);  // 4 logits each
-        const uint32_t whole = n & ~3u;           // logits below this index sit in whole units
-        for (uint32_t u0 = 0; u0 < units; u0 += 256 * kGatherUnits) {
-            float4v v[kGatherUnits];
-            uint32_t idx[kGatherUnits];
-#pragma unroll
-            for (int j = 0; j < kGatherUnits; ++j) {
-                const uint32_t u = u0 + j * 256 + tid < units ? u0 + j * 256 + tid : 0;
-                const uint32_t i = (static_cast<uint32_t>(s_sel[u >> (lb - 2)]) << lb) + ((u & ((blk >> 2) - 1)) << 2);
-                const bool ok = u0 + j * 256 + tid < units && i < whole;
-                idx[j] = i;
-                v[j] = *reinterpret_cast<const float4v*>(logits + (ok ? i : 0));
-                if (!ok) v[j] = float4v{NAN, NAN, NAN, NAN};
-            }
-#pragma unroll
-            for (int j = 0; j < kGatherUnits; ++j) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) consider(v[j][e], idx[j] + e);
-            }
-        }
-        if (s_tail && tid < (n & 3)) consider(logits[whole + tid], whole + tid);  // the last block's odd end
-    } else {
-        const uint32_t elems = nsel << lb;
-        for (uint32_t e0 = 0; e0 < elems; e0 += 256 * kGatherUnits) {
-            float v[kGatherUnits];
-            uint32_t idx[kGatherUnits];
-#pragma unroll
-            for (int j = 0; j < kGatherUnits; ++j) {
-                const uint32_t e = e0 + j * 256 + tid < elems ? e0 + j * 256 + tid : 0;
-                const uint32_t i = (static_cast<uint32_t>(s_sel[e >> lb]) << lb) + (e & (blk - 1));
-                const bool ok = e0 + j * 256 + tid < elems && i < n;
-                idx[j] = i;
-                v[j] = logits[ok ? i : 0];
-                if (!ok) v[j] = NAN;
-            }
-#pragma unroll
-            for (int j = 0; j < kGatherUnits; ++j) consider(v[j], idx[j]);
-        }
-    }
-    __syncthreads();
-    uint32_t total = s_count;
-    for (uint32_t e = tid; e < (total < kRankSlots ? total : kRankSlots); e += 256)
-        s_keys[e] = key_of(Cand{s_vals[e], s_ids[e]});
-    if (total > kRankSlots) {
-        // too many to rank from LDS (sorted or constant input): keep exactly the k best of them,
-        // read back from memory
-        __threadfence();
-        __syncthreads();
-        const uint64_t tau2 = select_kth_key(
-            [&](uint32_t i) { return key_of(load_survivor(surv, i)); }, total, k, sh);
-        if (tid == 0) s_count = 0;
-        __syncthreads();
-        for (uint32_t i = tid; i < total; i += 256) {
-            const Cand c = load_survivor(surv, i);
-            const uint64_t key = key_of(c);
-            if (key >= tau2) {  // keys are distinct: k of them
-                const uint32_t slot = atomicAdd(&s_count, 1u);
-                s_keys[slot] = key;
-                s_vals[slot] = c.logit;
-            }
-        }
-        __syncthreads();
-        total = s_count;
-    }
-    const uint32_t lim = (total + 15) & ~15u;
-    for (uint32_t i = total + tid; i < lim; i += 256) s_keys[i] = 0;  // below every real key
-    __syncthreads();
-    for (uint32_t e = tid; e < total; e += 256) {
-        const uint64_t ck = s_keys[e];
-        uint32_t rank = 0;
-        for (uint32_t j0 = 0; j0 < lim; j0 += 16) {
-#pragma unroll
-            for (uint32_t u = 0; u < 16; ++u) rank += s_keys[j0 + u] > ck;
-        }
-        if (rank < k) {
-            out_logits[rank] = s_vals[e];
-            out_ids[rank] = ~static_cast<uint32_t>(ck);
-        }
-    }
+    topk_select_tail<false>(logits, n, TopkBlocks{blk, 0, 1}, m, k, maxima, surv, ts, out_logits, out_ids);
 }
 
 // ---- the same selection as four launches, for large k ---------------------------------------

@@ -118,6 +118,99 @@ def test_gpu_lm_head_topk_matches_gemv_then_topk():
     assert np.abs(out_l.cpu().numpy() - o_l[:top_k]).max() <= eps
 
 
+def _lm_head_cases():
+    """(name, vocab, k, top_k, weight blocks, x): shapes on both sides of what the one-launch form takes,
+    exact ties, logits near the top of the f32 range, and all-NaN logits."""
+    cases = []
+    for vocab, k, top_k, seed in [(5000, 2048, 40, 1), (300, 2048, 50, 2), (100, 2048, 50, 3), (7001, 5120, 64, 4),
+                                  (3000, 4096, 1, 5), (2500, 8192, 17, 6), (4099, 2112, 33, 7), (40000, 2048, 64, 8),
+                                  (6000, 1024, 20, 9), (5000, 2048, 65, 10)]:
+        cases.append((f"v{vocab}_k{k}_top{top_k}", vocab, k, top_k, synth.q4_weight(vocab, k, seed=seed),
+                      synth.activations(1, k, seed=seed)))
+    # 37 distinct rows repeated: every logit occurs 100+ times, the lower token id must win each tie
+    vocab, k = 4000, 2048
+    rows = synth.q4_weight(37, k, seed=12).reshape(37, -1)
+    tied = np.ascontiguousarray(rows[np.arange(vocab) % 37]).reshape(-1)
+    cases.append(("exact_ties", vocab, k, 50, tied, synth.activations(1, k, seed=12)))
+    # logits near the top of the f32 range, and (one activation infinite: inf - inf inside every row) all NaN,
+    # which the selection returns as sentinels
+    x = synth.activations(1, k, seed=13)
+    x[0, 5], x[0, 40] = 3.0e38, -3.0e38
+    cases.append(("huge_logits", 5000, k, 60, synth.q4_weight(5000, k, seed=13), x))
+    x = synth.activations(1, k, seed=14)
+    x[0, 0] = np.inf
+    cases.append(("all_nan_logits", 5000, k, 60, synth.q4_weight(5000, k, seed=14), x))
+    return cases
+
+
+@pytest.mark.gpu
+def test_gpu_lm_head_selection_inside_the_gemv_launch_matches_two_launches():
+    import torch
+    from lattice_amd import backend
+    be = backend.HipQ4Backend(0)
+    try:
+        served = 0
+        for name, vocab, k, top_k, wq, x in _lm_head_cases():
+            print(f"lm_head one launch vs two: {name}", flush=True)
+            qw = be.upload_q4_blocks(wq)
+            xd = torch.from_numpy(x).cuda()
+            be.set_lm_head_mode(backend.LM_HEAD_TWO_LAUNCHES)
+            two_l, two_i = be.lm_head_topk(xd, qw, vocab, k, top_k)
+            two_l, two_i = two_l.cpu().numpy().view(np.uint32), two_i.cpu().numpy().view(np.uint32)
+            be.set_lm_head_mode(backend.LM_HEAD_ONE_LAUNCH)
+            before = be.path_counters()["lm_head_one_launch"]
+            for rep in range(3):  # the ticket and the maxima are shared by back-to-back calls
+                one_l, one_i = be.lm_head_topk(xd, qw, vocab, k, top_k)
+                assert np.array_equal(one_i.cpu().numpy().view(np.uint32), two_i), (name, rep)
+                assert np.array_equal(one_l.cpu().numpy().view(np.uint32), two_l), (name, rep)
+            served += be.path_counters()["lm_head_one_launch"] - before
+            # and both are the exact top-k of the GEMV's logits
+            y = torch.empty((1, vocab), dtype=torch.float32, device="cuda")
+            be.dispatch_matmul(xd, qw, y, 1, vocab, k)
+            ref_l, ref_i = oracle.topk(y.cpu().numpy().reshape(-1), top_k)
+            assert np.array_equal(two_i, ref_i), name
+            assert np.array_equal(two_l, ref_l.view(np.uint32)), name
+            if name == "exact_ties":
+                # the best row's copies, lower token ids first
+                assert np.array_equal(two_i, two_i[0] + 37 * np.arange(top_k, dtype=np.uint32)) and two_i[0] < 37
+            if name == "all_nan_logits":
+                assert np.all(two_i == 0xFFFFFFFF) and np.isnan(y.cpu().numpy()).all()
+        # every case but the tiny vocabulary, the 1024-wide rows and top_k 65 went through the one-launch form
+        assert served == 3 * (len(_lm_head_cases()) - 3), served
+    finally:
+        be.set_lm_head_mode(backend.LM_HEAD_TWO_LAUNCHES)
+        be.close()
+
+
+@pytest.mark.gpu
+def test_gpu_lm_head_one_launch_alternating_inputs():
+    """Calls that alternate between two vocabularies and activations share the logits buffer, the
+    maxima and the ticket: each call must select from its own launch's values."""
+    import torch
+    from lattice_amd import backend
+    be = backend.HipQ4Backend(0)
+    k = 2048
+    sets = []
+    for vocab, seed, gain in [(30000, 21, 1.0), (11000, 22, 1e-3)]:
+        wq = synth.q4_weight(vocab, k, seed=seed)
+        x = synth.activations(1, k, seed=seed) * np.float32(gain)
+        qw, xd = be.upload_q4_blocks(wq), torch.from_numpy(x).cuda()
+        y = torch.empty((1, vocab), dtype=torch.float32, device="cuda")
+        be.dispatch_matmul(xd, qw, y, 1, vocab, k)
+        sets.append((vocab, qw, xd, oracle.topk(y.cpu().numpy().reshape(-1), 50)))
+    be.set_lm_head_mode(backend.LM_HEAD_ONE_LAUNCH)
+    try:
+        for it in range(40):
+            vocab, qw, xd, (ref_l, ref_i) = sets[it % 2]
+            out_l, out_i = be.lm_head_topk(xd, qw, vocab, k, 50)
+            assert np.array_equal(out_i.cpu().numpy().view(np.uint32), ref_i), it
+            assert np.array_equal(out_l.cpu().numpy().view(np.uint32), ref_l.view(np.uint32)), it
+        assert be.path_counters()["lm_head_one_launch"] == 40
+    finally:
+        be.set_lm_head_mode(backend.LM_HEAD_TWO_LAUNCHES)
+        be.close()
+
+
 @pytest.mark.gpu
 def test_gpu_topk_back_to_back_calls_use_their_own_block_maxima():
     """The one-launch selection hands every block's best key to the workgroup that finishes last

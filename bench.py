@@ -424,34 +424,36 @@ def main():
         # down GEMV, add into the residual.  Five launches one by one against two fused launches.
         if B == 1:
             hid, inter = 2048, 6144
-            base_v, delta_v = xs[2048][0], torch.randn(hid, device="cuda", generator=gen)
             gamma_v = torch.randn(hid, device="cuda", generator=gen) * 0.1
-            res_v, normed_v, hid_v = (torch.empty(hid, device="cuda") for _ in range(3))
-            gu_v, ffn_v = torch.empty(2 * inter, device="cuda"), torch.empty(hid, device="cuda")
+            for rows in (1, 8):  # one token, and the decode steps of eight sequences at once
+                base_v = torch.randn((rows, hid), device="cuda", generator=gen)
+                delta_v = torch.randn((rows, hid), device="cuda", generator=gen)
+                res_v, normed_v, hid_v, ffn_v = (torch.empty((rows, hid), device="cuda") for _ in range(4))
+                gu_v, act_v = torch.empty((rows, 2 * inter), device="cuda"), torch.empty((rows, inter), device="cuda")
 
-            def mlp_unfused(i):
-                bufs = layers[i % len(layers)]
-                be.dispatch_fused_residual_add_norm(base_v, delta_v, res_v, normed_v, gamma_v, hid, 1e-6)
-                be.dispatch_matmul(normed_v, bufs["gate_up"], gu_v, 1, 2 * inter, hid)
-                be.dispatch_silu_mul_fused(gu_v, inter)
-                be.dispatch_matmul(gu_v, bufs["down"], ffn_v, 1, hid, inter)
-                be.dispatch_add_and_copy(ffn_v, res_v, hid_v, hid)
+                def mlp_unfused(i, rows=rows):
+                    bufs = layers[i % len(layers)]
+                    be.dispatch_fused_residual_add_norm(base_v, delta_v, res_v, normed_v, gamma_v, hid, 1e-6, num_rows=rows)
+                    be.gemv_batch(normed_v, bufs["gate_up"], gu_v, rows, 2 * inter, hid)
+                    be.dispatch_silu_mul_fused(gu_v, inter, rows, out=act_v, out_stride=inter)
+                    be.gemv_batch(act_v, bufs["down"], ffn_v, rows, hid, inter)
+                    be.dispatch_add_and_copy(ffn_v, res_v, hid_v, rows * hid)
 
-            def mlp_fused(i):
-                bufs = layers[i % len(layers)]
-                be.dispatch_matmul_fused(None, bufs["gate_up"], gu_v, 2 * inter, hid,
-                                         norm=(base_v, delta_v, gamma_v, 1e-6, res_v))
-                be.dispatch_matmul_fused(gu_v, bufs["down"], None, hid, inter, silu_mul=True,
-                                         add_residual=(res_v, hid_v))
-            mlp = {}
-            for nm, f in (("five_launches", mlp_unfused), ("two_fused_launches", mlp_fused)):
-                for i in range(len(layers)):
-                    f(i)
-                mlp[nm + "_us"] = round(tm(torch, f, max(72, args.steps // 2)) * 1e3, 3)
-            mlp_bytes = gemv_bytes(2 * inter, hid, 1) + gemv_bytes(hid, inter, 1)
-            mlp["GB/s_fused"] = round(mlp_bytes / mlp["two_fused_launches_us"] / 1e3, 1)
-            mlp["speedup"] = round(mlp["five_launches_us"] / mlp["two_fused_launches_us"], 3)
-            out["decode_mlp_hidden2048_inter6144"] = mlp
+                def mlp_fused(i, rows=rows):
+                    bufs = layers[i % len(layers)]
+                    be.dispatch_matmul_fused(None, bufs["gate_up"], gu_v, 2 * inter, hid,
+                                             norm=(base_v, delta_v, gamma_v, 1e-6, res_v), batch=rows)
+                    be.dispatch_matmul_fused(gu_v, bufs["down"], None, hid, inter, silu_mul=True,
+                                             add_residual=(res_v, hid_v), batch=rows)
+                mlp = {}
+                for nm, f in (("five_launches", mlp_unfused), ("two_fused_launches", mlp_fused)):
+                    for i in range(len(layers)):
+                        f(i)
+                    mlp[nm + "_us"] = round(tm(torch, f, max(72, args.steps // 2)) * 1e3, 3)
+                mlp_bytes = gemv_bytes(2 * inter, hid, rows) + gemv_bytes(hid, inter, rows)
+                mlp["GB/s_fused"] = round(mlp_bytes / mlp["two_fused_launches_us"] / 1e3, 1)
+                mlp["speedup"] = round(mlp["five_launches_us"] / mlp["two_fused_launches_us"], 3)
+                out["decode_mlp_hidden2048_inter6144" + ("" if rows == 1 else "_rows%d" % rows)] = mlp
 
         # single-LoRA epilogue, benchmark config 3: q (2048x2048) and v (512x2048) projections, rank 16,
         # f16 factors, scale alpha/r = 2.0, fused into the projection's own launch

@@ -271,6 +271,22 @@ int lq4_gemv_fused(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, u
                    const float* x_dev, float* y_dev, const lq4_gemv_fusion* fusion, const lq4_lora* lora,
                    float lora_scale, void* stream);
 
+/* lq4_gemv_fused for `batch` activation rows (1 <= batch <= LQ4_MAX_GEMV_BATCH), the decode
+ * steps of several sequences at once; the batched elementwise shaders it folds in are
+ * fused_residual_add_norm_batch (shaders/qwen35.metal:2219-2249, dispatch_fused_residual_add_norm_batch,
+ * inner/dispatch.rs:1171-1266) and silu_mul_fused over rows (shaders/qwen35.metal:712-722).  Every
+ * per-row array is dense: fusion->base, delta and residual_out are [batch, K]; gamma is [K] and shared;
+ * x_dev is [batch, K] (LQ4_PRO_NONE) or [batch, 2K] rows of [gate | up] (LQ4_PRO_SILU_MUL); y_dev,
+ * fusion->residual and copy_dst are [batch, N].  batch == 1 is lq4_gemv_fused.  For 2..8 rows the
+ * epilogue runs inside the small-batch GEMV's launch, and so does the prologue while its input is
+ * at most 64 KB (each workgroup forms 1/rms of every row, one wave per row, before it stages the
+ * rows; every workgroup repeats that work, so beyond a few rows one stand-alone launch is cheaper
+ * and the library runs that instead).  More than 8 rows, K too long for LDS, or a LoRA adapter run
+ * as the unfused sequence through library scratch.  Same results as that sequence to f32 rounding. */
+int lq4_gemv_fused_batch(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
+                         const float* x_dev, uint32_t batch, float* y_dev, const lq4_gemv_fusion* fusion,
+                         const lq4_lora* lora, float lora_scale, void* stream);
+
 /* ---- a chain of one-token GEMVs in one launch -------------------------------------------------
  * The reference encodes a whole token into one command buffer (forward_step,
  * forward/metal_qwen35.rs:6943, committed once at :6447): o -> residual add + RMSNorm -> gate||up ->

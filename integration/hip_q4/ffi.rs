@@ -206,6 +206,20 @@ extern "C" {
         lora_scale: f32,
         stream: *mut c_void,
     ) -> c_int;
+    pub fn lq4_gemv_fused_batch(
+        ctx: *mut Lq4Ctx,
+        w: *const Lq4Weight,
+        w_extra_offset: u64,
+        n: u32,
+        k: u32,
+        x: *const f32,
+        batch: u32,
+        y: *mut f32,
+        fusion: *const Lq4GemvFusion,
+        lora: *const Lq4Lora,
+        lora_scale: f32,
+        stream: *mut c_void,
+    ) -> c_int;
     pub fn lq4_gemv_chain(ctx: *mut Lq4Ctx, steps: *const Lq4ChainStep, n_steps: u32, stream: *mut c_void) -> c_int;
     pub fn lq4_set_chain_mode(mode: c_int) -> c_int;
     pub fn lq4_set_lm_head_mode(mode: c_int) -> c_int;

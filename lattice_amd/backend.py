@@ -51,7 +51,7 @@ EXPORTS = [
     "lq4_probe_read_config",
     "lq4_probe_copy",
     "lq4_set_gemm_kernel",
-    "lq4_residual_add_rmsnorm", "lq4_silu_mul", "lq4_add_and_copy", "lq4_gemv_fused",
+    "lq4_residual_add_rmsnorm", "lq4_silu_mul", "lq4_add_and_copy", "lq4_gemv_fused", "lq4_gemv_fused_batch",
     "lq4_lm_head_topk_static",
     "lq4_gemv_chain", "lq4_set_chain_mode", "lq4_set_lm_head_mode", "lq4_ctx_reserve_scratch",
     "lq4_gemv_q8", "lq4_gemm_q8", "lq4_gemv_q3", "lq4_gemm_q3",
@@ -151,6 +151,8 @@ def load_library() -> C.CDLL:
         "lq4_gemm_q3": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, C.c_int, C.c_uint32, vp, vp]),
         "lq4_gemv_fused": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, vp, C.POINTER(GemvFusion), vp,
                                      C.c_float, vp]),
+        "lq4_gemv_fused_batch": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, C.c_uint32, vp,
+                                           C.POINTER(GemvFusion), vp, C.c_float, vp]),
         "lq4_gemv_chain": (C.c_int, [vp, C.POINTER(ChainStep), C.c_uint32, vp]),
         "lq4_set_chain_mode": (C.c_int, [C.c_int]),
         "lq4_set_lm_head_mode": (C.c_int, [C.c_int]),
@@ -421,12 +423,14 @@ class HipQ4Backend:
                                          self._stream()))
 
     def dispatch_matmul_fused(self, x, qw: Q4WeightBuf, y, n: int, k: int, *, norm=None, silu_mul=False,
-                              add_residual=None, qw_extra_offset: int = 0, layer_idx=None, module=None):
-        """Batch-1 ``dispatch_matmul`` with the neighbouring elementwise dispatches folded in.
-        ``norm=(base, delta, gamma, eps, residual_out)`` replaces a preceding
-        ``dispatch_fused_residual_add_norm`` (``x`` is then unused); ``silu_mul=True`` replaces a
-        preceding ``dispatch_silu_mul_fused`` (``x`` holds gate | up, 2k floats);
-        ``add_residual=(residual, dst)`` replaces a following ``dispatch_add_and_copy``."""
+                              add_residual=None, qw_extra_offset: int = 0, layer_idx=None, module=None,
+                              batch: int = 1):
+        """``dispatch_matmul`` for 1..16 activation rows with the neighbouring elementwise dispatches
+        folded in.  ``norm=(base, delta, gamma, eps, residual_out)`` replaces a preceding
+        ``dispatch_fused_residual_add_norm`` / ``_batch`` (``x`` is then unused); ``silu_mul=True``
+        replaces a preceding ``dispatch_silu_mul_fused`` (``x`` holds gate | up, 2k floats per row);
+        ``add_residual=(residual, dst)`` replaces a following ``dispatch_add_and_copy``.  With
+        ``batch`` rows every per-row tensor is ``[batch, ...]`` and dense."""
         if n == 0:
             return
         self._assert_k(k, "dispatch_matmul_q4")
@@ -444,8 +448,8 @@ class HipQ4Backend:
             residual, dst = add_residual
             f.epilogue, f.residual, f.copy_dst = LQ4_EPI_ADD_RESIDUAL, residual.data_ptr(), self._ptr(dst)
         lora = self._lora_for(layer_idx, module, n, k)
-        _check(self.lib.lq4_gemv_fused(self.ctx, qw.handle, qw_extra_offset, n, k, self._ptr(x), self._ptr(y),
-                                       C.byref(f), lora, self._lora_scale, self._stream()))
+        _check(self.lib.lq4_gemv_fused_batch(self.ctx, qw.handle, qw_extra_offset, n, k, self._ptr(x), batch,
+                                             self._ptr(y), C.byref(f), lora, self._lora_scale, self._stream()))
 
     def chain_step(self, qw: Q4WeightBuf, n: int, k: int, *, x=None, from_previous=False, norm=None, silu_mul=False,
                    add_residual=None, silu_mul_pairs=False, y=None, qw_extra_offset: int = 0) -> ChainStep:

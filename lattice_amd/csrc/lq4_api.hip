@@ -26,7 +26,7 @@ struct lq4_ctx {
     bool lora_in_kernel;
     uint32_t lora_spin_limit;  // polls a weight wave spends on those counters before it computes A.x alone
     size_t moe_scratch_bytes;
-    uint8_t* shared_scratch;  // lq4_moe_shared_expert: gate||up and down results (the GEMM it calls uses moe_scratch)
+    uint8_t* shared_scratch;  // intermediates of calls that run lq4_gemv / lq4_gemm in between (those use moe_scratch)
     size_t shared_scratch_bytes;
     // Buffers the growable scratch outgrew: launches already queued (or captured into a graph) may
     // still use them, so they are only released with the context.
@@ -60,6 +60,7 @@ struct lq4_lora {
 
 namespace {
 
+constexpr size_t kFusedPrologueBytes = 64u << 10;  // lq4_gemv_fused_batch: see there
 constexpr uint32_t kLoraTRows = 4096;  // most rows one LoRA-fused call may carry
 
 thread_local char g_err[512] = "";
@@ -907,6 +908,124 @@ int lq4_gemv_fused(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, u
     ctx->counters.gemv++;
     if (f.epilogue == LQ4_EPI_ADD_RESIDUAL) {
         launch_add_and_copy(yo, f.residual, f.copy_dst, n, s);
+        ctx->counters.elementwise++;
+    }
+    LQ4_HIP(hipGetLastError());
+    return LQ4_OK;
+}
+
+int lq4_gemv_fused_batch(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
+                         const float* x_dev, uint32_t batch, float* y_dev, const lq4_gemv_fusion* fusion,
+                         const lq4_lora* lora, float lora_scale, void* stream) {
+    if (batch == 1) return lq4_gemv_fused(ctx, w, w_extra_offset, n, k, x_dev, y_dev, fusion, lora, lora_scale, stream);
+    if (!fusion || (fusion->prologue == LQ4_PRO_NONE && fusion->epilogue == LQ4_EPI_NONE))
+        return lq4_gemv(ctx, w, w_extra_offset, n, k, x_dev, batch, y_dev, lora, lora_scale, stream);
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    if (batch == 0 || n == 0) return LQ4_OK;
+    if (batch > LQ4_MAX_GEMV_BATCH) return fail(LQ4_E_INVALID, "batch %u above %d", batch, LQ4_MAX_GEMV_BATCH);
+    const uint8_t* wp;
+    int rc = resolve_weight(w, w_extra_offset, n, k, &wp);
+    if (rc) return rc;
+    const lq4_gemv_fusion& f = *fusion;
+    const size_t in_bytes = static_cast<size_t>(batch) * k * sizeof(float);
+    auto misaligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 != 0; };
+    switch (f.prologue) {
+        case LQ4_PRO_NONE:
+        case LQ4_PRO_SILU_MUL:
+            if (!x_dev) return fail(LQ4_E_INVALID, "x device pointer is null");
+            if (misaligned(x_dev)) return fail(LQ4_E_INVALID, "x must be 16-byte aligned");
+            break;
+        case LQ4_PRO_ADD_RMSNORM:
+            if (!f.base || !f.gamma) return fail(LQ4_E_INVALID, "fusion.base or fusion.gamma is null");
+            if (misaligned(f.base) || misaligned(f.gamma) || (f.delta && misaligned(f.delta)) ||
+                (f.residual_out && misaligned(f.residual_out)))
+                return fail(LQ4_E_INVALID, "fusion.base, delta, gamma and residual_out must be 16-byte aligned");
+            if (f.residual_out && (ranges_overlap(f.residual_out, f.base, in_bytes) ||
+                                   (f.delta && ranges_overlap(f.residual_out, f.delta, in_bytes))))
+                return fail(LQ4_E_INVALID, "fusion.residual_out must not overlap fusion.base or fusion.delta");
+            break;
+        default:
+            return fail(LQ4_E_INVALID, "unknown fusion.prologue %d", f.prologue);
+    }
+    if (f.epilogue == LQ4_EPI_ADD_RESIDUAL) {
+        if (!f.residual) return fail(LQ4_E_INVALID, "fusion.residual is null");
+        if (reinterpret_cast<uintptr_t>(f.residual) % 4 || reinterpret_cast<uintptr_t>(f.copy_dst) % 4)
+            return fail(LQ4_E_INVALID, "fusion.residual and copy_dst must be 4-byte aligned");
+    } else if (f.epilogue == LQ4_EPI_NONE) {
+        if (!y_dev) return fail(LQ4_E_INVALID, "y device pointer is null");
+    } else {
+        return fail(LQ4_E_INVALID, "unknown fusion.epilogue %d", f.epilogue);
+    }
+    if (y_dev && reinterpret_cast<uintptr_t>(y_dev) % 4) return fail(LQ4_E_INVALID, "y must be 4-byte aligned");
+    LoraEpilogue ep;
+    rc = resolve_lora(ctx, lora, lora_scale, n, k, batch, &ep);
+    if (rc) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    DeviceGuard g(ctx->device);
+
+    // Inside the launch every workgroup produces all rows' activations for itself: that pays while the
+    // rows are small (one token always; more rows up to this many bytes of prologue input per workgroup:
+    // the decode MLP of a 2048-wide model at 3 and 4 rows 21.2 / 22.1 -> 19.6 / 21.2 us, at 8 rows
+    // 26.4 -> 32.7 us with everything inside).  Larger inputs run the prologue once, as its own launch, and
+    // keep only the epilogue in the GEMV.  More than 8 rows are served by the few-token GEMM kernel,
+    // which has no fused form: the steps run one by one.
+    const size_t pro_bytes = f.prologue == LQ4_PRO_NONE ? 0 : in_bytes * (f.prologue == LQ4_PRO_SILU_MUL ? 2 : (f.delta ? 2 : 1));
+    static const size_t pro_limit = [] {
+        const char* env = getenv("LQ4_FUSED_PROLOGUE_BYTES");
+        return env ? static_cast<size_t>(strtoull(env, nullptr, 10)) : kFusedPrologueBytes;
+    }();
+    if (!ep.rank && batch <= 8 && gemv_fused_batch_fits(k, batch)) {
+        GemvFusion gf;
+        const float* act_in = x_dev;
+        int pro = f.prologue;
+        if (pro_bytes > pro_limit) {
+            rc = ensure_scratch(ctx, in_bytes, s);
+            if (rc) return rc;
+            float* xs = reinterpret_cast<float*>(ctx->moe_scratch);
+            if (pro == LQ4_PRO_ADD_RMSNORM) launch_residual_add_norm(f.base, f.delta, f.gamma, k, batch, f.eps, f.residual_out, xs, s);
+            else launch_silu_mul(x_dev, k, batch, xs, k, s);
+            ctx->counters.elementwise++;
+            act_in = xs;
+            pro = LQ4_PRO_NONE;
+        }
+        gf.prologue = pro;
+        gf.base = f.base;
+        gf.delta = f.delta;
+        gf.gamma = f.gamma;
+        gf.eps = f.eps;
+        gf.residual_out = f.residual_out;
+        gf.epilogue = f.epilogue;
+        gf.residual = f.residual;
+        gf.copy_dst = f.copy_dst;
+        if (launch_gemv_fused_batch(wp, n, k, act_in, batch, y_dev, gf, s)) {
+            ctx->counters.gemv_fused++;
+            LQ4_HIP(hipGetLastError());
+            return LQ4_OK;
+        }
+    }
+
+    // The same steps one by one: activations and (if the caller wants no y) the product in scratch (not
+    // the scratch lq4_gemv itself may use for its few-token kernel).
+    const size_t y_off = (in_bytes + 255) / 256 * 256;
+    rc = grow_scratch(ctx, &ctx->shared_scratch, &ctx->shared_scratch_bytes,
+                      y_off + static_cast<size_t>(batch) * n * sizeof(float), s, false);
+    if (rc) return rc;
+    const float* act = x_dev;
+    float* xs = reinterpret_cast<float*>(ctx->shared_scratch);
+    if (f.prologue == LQ4_PRO_ADD_RMSNORM) {
+        launch_residual_add_norm(f.base, f.delta, f.gamma, k, batch, f.eps, f.residual_out, xs, s);
+        act = xs;
+        ctx->counters.elementwise++;
+    } else if (f.prologue == LQ4_PRO_SILU_MUL) {
+        launch_silu_mul(x_dev, k, batch, xs, k, s);
+        act = xs;
+        ctx->counters.elementwise++;
+    }
+    float* yo = y_dev ? y_dev : reinterpret_cast<float*>(ctx->shared_scratch + y_off);
+    rc = lq4_gemv(ctx, w, w_extra_offset, n, k, act, batch, yo, lora, lora_scale, stream);
+    if (rc) return rc;
+    if (f.epilogue == LQ4_EPI_ADD_RESIDUAL) {
+        launch_add_and_copy(yo, f.residual, f.copy_dst, static_cast<size_t>(batch) * n, s);
         ctx->counters.elementwise++;
     }
     LQ4_HIP(hipGetLastError());

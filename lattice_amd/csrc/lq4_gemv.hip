@@ -237,6 +237,32 @@ void launch_gemv(const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint3
     }
 }
 
+bool gemv_fused_batch_fits(uint32_t k, uint32_t batch) {
+    for (uint32_t b0 = 0; b0 < batch; b0 += 8)
+        if (gemv_mfma_lds_bytes(k, batch - b0 < 8 ? batch - b0 : 8) > 150 * 1024) return false;
+    return true;
+}
+
+bool launch_gemv_fused_batch(const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint32_t batch, float* y,
+                             const GemvFusion& fusion, hipStream_t stream) {
+    if (!gemv_fused_batch_fits(k, batch)) return false;
+    const uint32_t x_stride = fusion.prologue == GemvFusion::kSiluMul ? 2 * k : k;
+    const LoraEpilogue none{};
+    for (uint32_t b0 = 0; b0 < batch; b0 += 8) {  // more than 8 rows: two passes over the weights
+        const uint32_t nb = batch - b0 < 8 ? batch - b0 : 8;
+        GemvFusion f = fusion;
+        const size_t in_off = static_cast<size_t>(b0) * k, out_off = static_cast<size_t>(b0) * n;
+        if (f.base) f.base += in_off;
+        if (f.delta) f.delta += in_off;
+        if (f.residual_out) f.residual_out += in_off;
+        if (f.residual) f.residual += out_off;
+        if (f.copy_dst) f.copy_dst += out_off;
+        launch_gemv_mfma(w, n, k, x ? x + static_cast<size_t>(b0) * x_stride : nullptr, x_stride, nb,
+                         y ? y + out_off : nullptr, n, none, stream, &f);
+    }
+    return true;
+}
+
 void launch_lora_a(const void* a, int a_is_f16, uint32_t rank, uint32_t d_in, const void* x,
                    int x_is_f16, uint32_t x_stride, uint32_t rows, float* t, hipStream_t stream) {
     const dim3 grid(rank, rows), block(256);

@@ -89,6 +89,11 @@ struct GemvArgs {
     float* y;
     uint32_t n, k, batch, x_stride, y_stride;
     LoraEpilogue lora;
+    // Elementwise steps around the product, per activation row (the batch form of the one-token
+    // kernel's GemvFusion): base, delta and residual_out are [batch, K] rows, x for kSiluMul is
+    // [batch, 2K] rows of [gate | up] (x_stride apart), residual and copy_dst are [batch, N] rows
+    // (y_stride apart).  kPlain / kStore: the plain product.
+    GemvFusion fz;
 };
 
 // NSETS: groups of four activation columns (1 or 2).  HILO: two columns per activation row.
@@ -143,10 +148,14 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_mfma(GemvArgs p) {
         const uint32_t wc = w < total_items ? w : 0;
         hrow[i] = wc / items;
         hitem[i] = wc - hrow[i] * items;
-        const float4* xp = reinterpret_cast<const float4*>(p.x + static_cast<size_t>(hrow[i]) * p.x_stride +
-                                                           (hitem[i] >> 2) * kBlockWeights + (hitem[i] & 3) * 8);
-        hva[i] = xp[0];
-        hvb[i] = xp[1];
+        if (p.fz.prologue == GemvFusion::kPlain) {  // uniform; the fused prologues load everything below
+            const float4* xp = reinterpret_cast<const float4*>(p.x + static_cast<size_t>(hrow[i]) * p.x_stride +
+                                                               (hitem[i] >> 2) * kBlockWeights + (hitem[i] & 3) * 8);
+            hva[i] = xp[0];
+            hvb[i] = xp[1];
+        } else {
+            hva[i] = hvb[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
     }
 
     // Loads unit u.  Blocks past the end of a row and rows past N re-read a valid block; their
@@ -191,6 +200,119 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_mfma(GemvArgs p) {
             if (dw == 0) reinterpret_cast<float*>(base + ncols * 4)[b] = sx;
         }
     };
+    // The activations are produced while they are staged (the batch form of the one-token kernel's
+    // prologues; shaders/qwen35.metal:2219-2249 is the reference's batched add + norm, :712-722 its
+    // silu * up).  Every workgroup does this for all rows, as it stages all rows anyway.
+    auto stage_fused = [&]() {
+        auto unit_at = [](uint32_t it) { return (it >> 2) * kBlockWeights + (it & 3) * 8; };
+        auto add4 = [](float4 a, const float4 b) {
+            a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+            return a;
+        };
+        constexpr int G = 2;  // pairs in flight per thread (each is four 16-byte loads)
+        if (p.fz.prologue == GemvFusion::kAddNorm) {
+            // 1/rms of every row first: wave v owns rows v, v + WAVES, ...; a lane sums units lane, lane + 64, ...
+            // in order, then the wave sum: the same value in every workgroup.  Workgroup 0 stores the new residual.
+            float* inv_rms = red;  // [batch]: the K slices' meeting point is not in use yet
+            for (uint32_t b = wave; b < batch; b += WAVES) {
+                const float* bp = p.fz.base + static_cast<size_t>(b) * p.k;
+                const float* dp = p.fz.delta ? p.fz.delta + static_cast<size_t>(b) * p.k : nullptr;
+                float ss = 0.0f;
+                for (uint32_t it0 = lane; it0 < items; it0 += 64 * 4) {
+                    float4 a[4], c[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const uint32_t it = it0 + 64 * i < items ? it0 + 64 * i : 0;
+                        a[i] = reinterpret_cast<const float4*>(bp + unit_at(it))[0];
+                        c[i] = reinterpret_cast<const float4*>(bp + unit_at(it))[1];
+                        if (dp) {
+                            a[i] = add4(a[i], reinterpret_cast<const float4*>(dp + unit_at(it))[0]);
+                            c[i] = add4(c[i], reinterpret_cast<const float4*>(dp + unit_at(it))[1]);
+                        }
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        if (it0 + 64 * i < items) {
+                            ss += ((a[i].x * a[i].x + a[i].y * a[i].y) + (a[i].z * a[i].z + a[i].w * a[i].w)) +
+                                  ((c[i].x * c[i].x + c[i].y * c[i].y) + (c[i].z * c[i].z + c[i].w * c[i].w));
+                            if (blockIdx.x == 0 && p.fz.residual_out) {
+                                float4* rp = reinterpret_cast<float4*>(p.fz.residual_out + static_cast<size_t>(b) * p.k + unit_at(it0 + 64 * i));
+                                rp[0] = a[i];
+                                rp[1] = c[i];
+                            }
+                        }
+                    }
+                }
+                ss = wave_sum(ss);
+                if (lane == 0) inv_rms[b] = 1.0f / sqrtf(ss / static_cast<float>(p.k) + p.fz.eps);
+            }
+            __syncthreads();
+            for (uint32_t w0 = tid; w0 < total_items; w0 += G * kThreads) {
+                float4 va[G], vb[G], ga[G], gb[G];
+                uint32_t wb[G], wi[G];
+#pragma unroll
+                for (int i = 0; i < G; ++i) {
+                    const uint32_t w = w0 + i * kThreads;
+                    const uint32_t wc = w < total_items ? w : 0;
+                    wb[i] = wc / items;
+                    wi[i] = wc - wb[i] * items;
+                    const size_t at = static_cast<size_t>(wb[i]) * p.k + unit_at(wi[i]);
+                    va[i] = reinterpret_cast<const float4*>(p.fz.base + at)[0];
+                    vb[i] = reinterpret_cast<const float4*>(p.fz.base + at)[1];
+                    if (p.fz.delta) {
+                        va[i] = add4(va[i], reinterpret_cast<const float4*>(p.fz.delta + at)[0]);
+                        vb[i] = add4(vb[i], reinterpret_cast<const float4*>(p.fz.delta + at)[1]);
+                    }
+                    ga[i] = reinterpret_cast<const float4*>(p.fz.gamma + unit_at(wi[i]))[0];
+                    gb[i] = reinterpret_cast<const float4*>(p.fz.gamma + unit_at(wi[i]))[1];
+                }
+#pragma unroll
+                for (int i = 0; i < G; ++i) {
+                    const float inv = inv_rms[wb[i]];
+                    auto norm4 = [inv](float4 v, const float4 gm) {
+                        v.x = v.x * inv * (1.0f + gm.x); v.y = v.y * inv * (1.0f + gm.y);
+                        v.z = v.z * inv * (1.0f + gm.z); v.w = v.w * inv * (1.0f + gm.w);
+                        return v;
+                    };
+                    stage(wi[i], wb[i], norm4(va[i], ga[i]), norm4(vb[i], gb[i]), w0 + i * kThreads < total_items);
+                }
+            }
+            __syncthreads();  // inv_rms has been read by all before the meeting point is written
+        } else {  // kSiluMul: silu through the hardware exp2 and reciprocal, as the one-token kernel does
+            auto silu_mul = [](float gate, float u) {
+                const float e = __builtin_amdgcn_exp2f(gate * -1.44269504088896340736f);
+                return gate * __builtin_amdgcn_rcpf(1.0f + e) * u;
+            };
+            for (uint32_t w0 = tid; w0 < total_items; w0 += G * kThreads) {
+                float4 ga[G], gb[G], ua[G], ub[G];
+                uint32_t wb[G], wi[G];
+#pragma unroll
+                for (int i = 0; i < G; ++i) {
+                    const uint32_t w = w0 + i * kThreads;
+                    const uint32_t wc = w < total_items ? w : 0;
+                    wb[i] = wc / items;
+                    wi[i] = wc - wb[i] * items;
+                    const float* gp = p.x + static_cast<size_t>(wb[i]) * p.x_stride + unit_at(wi[i]);
+                    ga[i] = reinterpret_cast<const float4*>(gp)[0];
+                    gb[i] = reinterpret_cast<const float4*>(gp)[1];
+                    ua[i] = reinterpret_cast<const float4*>(gp + p.k)[0];
+                    ub[i] = reinterpret_cast<const float4*>(gp + p.k)[1];
+                }
+#pragma unroll
+                for (int i = 0; i < G; ++i) {
+                    float4 a, b;
+                    a.x = silu_mul(ga[i].x, ua[i].x); a.y = silu_mul(ga[i].y, ua[i].y);
+                    a.z = silu_mul(ga[i].z, ua[i].z); a.w = silu_mul(ga[i].w, ua[i].w);
+                    b.x = silu_mul(gb[i].x, ub[i].x); b.y = silu_mul(gb[i].y, ub[i].y);
+                    b.z = silu_mul(gb[i].z, ub[i].z); b.w = silu_mul(gb[i].w, ub[i].w);
+                    stage(wi[i], wb[i], a, b, w0 + i * kThreads < total_items);
+                }
+            }
+        }
+    };
+    if (p.fz.prologue != GemvFusion::kPlain) {
+        stage_fused();
+    } else {
 #pragma unroll
     for (int i = 0; i < kHoist; ++i) stage(hitem[i], hrow[i], hva[i], hvb[i], tid + i * kThreads < total_items);
     // the remaining (row, item) pairs, four loads in flight per thread so that a batch of rows costs
@@ -215,6 +337,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_mfma(GemvArgs p) {
 #pragma unroll
             for (int i = 0; i < G; ++i) stage(wi[i], wb[i], va[i], vb[i], w0 + i * kThreads < total);
         }
+    }
     }
     if (tid < 4) zero_region[tid] = make_uint4(0u, 0u, 0u, 0u);
     __syncthreads();
@@ -349,7 +472,15 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_mfma(GemvArgs p) {
                         const int brow = HILO ? c / 2 : c;
                         if ((HILO && (c & 1)) || brow >= static_cast<int>(batch)) continue;
                         const float v = HILO ? fmaf(tot[c + (HILO ? 1 : 0)], 1.0f / kLoScale, tot[c]) : tot[c];
-                        p.y[static_cast<size_t>(brow) * p.y_stride + row] = v;
+                        const size_t at = static_cast<size_t>(brow) * p.y_stride + row;
+                        if (p.fz.epilogue == GemvFusion::kAddResidual) {
+                            const float r = p.fz.residual[at] + v;
+                            p.fz.residual[at] = r;
+                            if (p.fz.copy_dst) p.fz.copy_dst[at] = r;
+                            if (p.y) p.y[at] = v;
+                        } else {
+                            p.y[at] = v;
+                        }
                     }
                 }
             }
@@ -436,8 +567,8 @@ size_t gemv_mfma_lds_bytes(uint32_t k, uint32_t batch) {
 
 void launch_gemv_mfma(const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint32_t x_stride,
                       uint32_t batch, float* y, uint32_t y_stride, const LoraEpilogue& lora,
-                      hipStream_t stream) {
-    GemvArgs a{w, x, y, n, k, batch, x_stride, y_stride, lora};
+                      hipStream_t stream, const GemvFusion* fusion) {
+    GemvArgs a{w, x, y, n, k, batch, x_stride, y_stride, lora, fusion ? *fusion : GemvFusion{}};
     const size_t lds = gemv_mfma_lds_bytes(k, batch);
     const uint32_t nsteps = (k / kBlockWeights + 15) / 16;
     // resident workgroups per CU: up to 8 (32 waves, what the T = 1 kernels' 64 registers allow)

@@ -145,7 +145,13 @@ void launch_moe_shared_gate_add(const float* x, const float* gate, const float* 
 size_t gemv_mfma_lds_bytes(uint32_t k, uint32_t batch);
 void launch_gemv_mfma(const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint32_t x_stride,
                       uint32_t batch, float* y, uint32_t y_stride, const LoraEpilogue& lora,
-                      hipStream_t stream);
+                      hipStream_t stream, const GemvFusion* fusion = nullptr);
+// The batch form of launch_gemv_b1_fused for 2..kMaxGemvBatch activation rows: base, delta and
+// residual_out are [batch, K], x for kSiluMul is [batch, 2K] ([gate | up] per row), y, residual and
+// copy_dst are [batch, N].  False (nothing launched) when the staged rows do not fit in LDS.
+bool gemv_fused_batch_fits(uint32_t k, uint32_t batch);
+bool launch_gemv_fused_batch(const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint32_t batch, float* y,
+                             const GemvFusion& fusion, hipStream_t stream);
 
 // t[row, j] = sum_k A[j, k] * x[row, k]; x f32 or f16 with row stride x_stride elements.
 void launch_lora_a(const void* a, int a_is_f16, uint32_t rank, uint32_t d_in, const void* x,

@@ -200,6 +200,81 @@ def test_fused_decode_mlp_matches_oracle_and_unfused(be, hidden, inter):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("hidden,inter,batch", [(2048, 6144, 8), (2048, 6144, 2), (1024, 512, 5), (160, 352, 3),
+                                                (512, 96, 16), (2048, 1024, 11), (5120, 544, 4),
+                                                (29184, 32, 3)])  # rows too long for LDS: the unfused sequence
+def test_fused_decode_mlp_for_several_rows(be, hidden, inter, batch):
+    """The decode MLP of `batch` sequences at once, two launches (norm + gate||up, silu*up + down + residual
+    add), against the oracle's five steps row by row and against the stand-alone kernels on the GPU."""
+    import torch
+    g = np.random.default_rng(21)
+    gate_up = synth.q4_weight(2 * inter, hidden, seed=21)
+    down = synth.q4_weight(hidden, inter, seed=22)
+    base = g.normal(size=(batch, hidden)).astype(np.float32)
+    base *= (1.0 + np.arange(batch, dtype=np.float32))[:, None]  # rows with different rms
+    delta = g.normal(size=(batch, hidden)).astype(np.float32)
+    gamma = (g.normal(size=hidden) * 0.2).astype(np.float32)
+    eps = 1e-6
+    print(f"fused MLP hidden={hidden} inter={inter} batch={batch}", flush=True)
+    res_ref, normed_ref = oracle.residual_add_norm(base, delta, gamma, eps)
+    gu_ref = oracle.gemm_f32(normed_ref, gate_up, 2 * inter, hidden)
+    h_ref = oracle.silu_mul(gu_ref)
+    ffn_ref = oracle.gemm_f32(h_ref, down, hidden, inter)
+    final_ref = res_ref + ffn_ref
+
+    qgu, qd = be.upload_q4_blocks(gate_up), be.upload_q4_blocks(down)
+    d_base, d_delta, d_gamma = dev(base), dev(delta), dev(gamma)
+    before = be.path_counters()
+    residual = torch.full((batch, hidden), float("nan"), device="cuda")
+    gu = torch.full((batch * 2 * inter + 1,), float("nan"), device="cuda")
+    be.dispatch_matmul_fused(None, qgu, gu, 2 * inter, hidden, norm=(d_base, d_delta, d_gamma, eps, residual),
+                             batch=batch)
+    assert np.array_equal(host(residual), res_ref)
+    got_gu = host(gu)
+    assert np.isnan(got_gu[-1])
+    got_gu = got_gu[:-1].reshape(batch, 2 * inter)
+    for b in range(batch):  # per row: rows differ in scale
+        assert rel_err(got_gu[b], gu_ref[b]) <= REL_TOL, b
+    hidden_out = torch.full((batch, hidden), float("nan"), device="cuda")
+    ffn = torch.full((batch, hidden), float("nan"), device="cuda")
+    be.dispatch_matmul_fused(gu, qd, ffn, hidden, inter, silu_mul=True, add_residual=(residual, hidden_out), batch=batch)
+    for b in range(batch):
+        # two dependent GEMVs, each rounding its activations to f16 above two rows: REL_TOL apiece
+        assert rel_err(host(ffn)[b], ffn_ref[b]) <= 2 * REL_TOL, b
+        assert rel_err(host(residual)[b], final_ref[b]) <= 2 * REL_TOL, b
+    assert np.array_equal(host(hidden_out), host(residual))
+    assert np.array_equal(host(residual), res_ref + host(ffn))  # the add itself is exact
+    after = be.path_counters()
+    # Routing: up to 8 rows whose staged form fits in LDS run in the fused kernel, with the prologue inside
+    # while its input is at most 64 KB and as a launch of its own beyond; otherwise the steps run one by one.
+    def stage(k, pro_bytes, steps):
+        if batch <= 8 and k <= 8192:
+            return 1, (1 if pro_bytes > 64 * 1024 else 0)
+        return 0, steps
+    f1, e1 = stage(hidden, batch * hidden * 4 * 2, 1)      # base + delta
+    f2, e2 = stage(inter, batch * inter * 4 * 2, 2)        # gate + up; silu and the residual add
+    assert after["gemv_fused"] - before["gemv_fused"] == f1 + f2
+    assert after["elementwise"] - before["elementwise"] == e1 + e2
+
+    # the stand-alone kernels and the plain GEMV on the GPU: the same arithmetic but for the order of the
+    # sum of squares and the silu's exp, so agreement is far inside the GEMV tolerance
+    res2 = torch.empty((batch, hidden), device="cuda")
+    normed = torch.empty((batch, hidden), device="cuda")
+    be.dispatch_fused_residual_add_norm(d_base, d_delta, res2, normed, d_gamma, hidden, eps, num_rows=batch)
+    gu2 = torch.empty((batch, 2 * inter), device="cuda")
+    be.gemv_batch(normed, qgu, gu2, batch, 2 * inter, hidden)
+    same_kernel = 2e-5
+    assert rel_err(got_gu, host(gu2)) <= same_kernel
+    # (the second stage from the fused first stage's own output, so that only this stage is compared)
+    gu2 = dev(got_gu)
+    act = torch.empty((batch, inter), device="cuda")
+    be.dispatch_silu_mul_fused(gu2, inter, batch, out=act, out_stride=inter)
+    ffn2 = torch.empty((batch, hidden), device="cuda")
+    be.gemv_batch(act, qd, ffn2, batch, hidden, inter)
+    assert rel_err(host(ffn), host(ffn2)) <= same_kernel
+
+
+@pytest.mark.gpu
 def test_fused_gemv_options_and_fallbacks(be):
     import torch
     from lattice_amd import backend

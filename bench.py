@@ -566,11 +566,19 @@ def main():
         for i in range(3):
             whole_layer(i)
         ms_layer = tm(torch, whole_layer, 40)
+        # ... and as one call (lq4_moe_ffn)
+        def one_call(i):
+            sh = shared[i % len(shared)]
+            be.moe_ffn(lg, sets[i % len(sets)][0], sets[i % len(sets)][1], E, TK, I, sh[0], sh[1], sgate, I, H, xm, ym)
+        for i in range(3):
+            one_call(i)
+        ms_one = tm(torch, one_call, 40)
         out["moe_grouped_gemv"] = {"distinct_experts": distinct, "algorithmic_bytes": moe_bytes,
                                    "ms_per_step": round(ms, 4), "GB/s": round(moe_bytes / ms / 1e6, 1),
                                    "pct_of_hbm_peak": round(100 * moe_bytes / ms / 1e6 / HBM_PEAK_GBPS, 2),
                                    "ms_per_step_with_router": round(ms_routed, 4),
-                                   "ms_per_step_with_router_and_shared_expert": round(ms_layer, 4)}
+                                   "ms_per_step_with_router_and_shared_expert": round(ms_layer, 4),
+                                   "ms_per_step_whole_layer_one_call": round(ms_one, 4)}
         del sets, shared
 
         # plain copies of known size: what a profiler's HBM traffic counters are scaled by

@@ -174,6 +174,18 @@ int lq4_moe_shared_expert(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_wei
                           const float* shared_gate_dev, uint32_t shared_inter, uint32_t hidden,
                           const float* x_dev, uint32_t tokens, float* y_dev, void* stream);
 
+/* The whole MoE FFN of one layer: moe_ffn_step (crates/inference/src/model/qwen35/moe.rs:8-36) /
+ * encode_moe_ffn (forward/metal_qwen35/inner/layers/mod.rs:226-660) from the router logits on:
+ * lq4_moe_route, lq4_moe_grouped_gemv and lq4_moe_shared_expert behind one call, with the routing
+ * tables in library scratch.  y_dev f32 [tokens, hidden] is overwritten.  Everything runs on
+ * `stream` in order (the shared expert beside the routed experts on a second stream was measured
+ * slower on MI355X).  Argument meaning and limits as in the three calls it replaces; same results
+ * bit for bit. */
+int lq4_moe_ffn(lq4_ctx* ctx, const float* router_logits_dev, const lq4_weight* gate_up, const lq4_weight* down,
+                uint32_t num_experts, uint32_t top_k, uint32_t inter, const lq4_weight* shared_gate_up,
+                const lq4_weight* shared_down, const float* shared_gate_dev, uint32_t shared_inter,
+                uint32_t hidden, const float* x_dev, uint32_t tokens, float* y_dev, void* stream);
+
 /* ---- lm_head top-k ------------------------------------------------------------
  * Exact top-k over `n` f32 logits in the reference's candidate order (higher logit first,
  * ties to the lower token id, NaN last as the (-inf, 0xFFFFFFFF) sentinel): the result of

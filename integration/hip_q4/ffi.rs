@@ -263,6 +263,25 @@ extern "C" {
         stream: *mut c_void,
     ) -> c_int;
 
+    pub fn lq4_moe_ffn(
+        ctx: *mut Lq4Ctx,
+        router_logits: *const f32,
+        gate_up: *const Lq4Weight,
+        down: *const Lq4Weight,
+        num_experts: u32,
+        top_k: u32,
+        inter: u32,
+        shared_gate_up: *const Lq4Weight,
+        shared_down: *const Lq4Weight,
+        shared_gate: *const f32,
+        shared_inter: u32,
+        hidden: u32,
+        x: *const f32,
+        tokens: u32,
+        y: *mut f32,
+        stream: *mut c_void,
+    ) -> c_int;
+
     // ---- lm_head and top-k
     pub fn lq4_topk(
         ctx: *mut Lq4Ctx,

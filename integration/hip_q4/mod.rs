@@ -348,42 +348,20 @@ impl HipQ4Backend {
 
     /// The MoE FFN of one layer for `tokens` rows of `x` (`encode_moe_ffn`, inner/layers/mod.rs:226-660;
     /// CPU form `moe_ffn_step`, model/qwen35/moe.rs:8-36): router softmax / top-k / renormalise from the
-    /// router logits, the routed experts, then the always-active shared expert onto the same `y`.
-    /// `ids` / `weights` are device scratch of `tokens * top_k` entries.  Unlike the Metal path nothing
-    /// is read back to the host between the steps (the router and the shared expert's sigmoid gate stay
-    /// on the device).
-    #[allow(clippy::too_many_arguments)]
-    pub fn encode_moe_ffn(
-        &self,
-        router_logits: &DevBuf,
-        moe: &HipMoeLayer,
-        x: &DevBuf,
-        tokens: u32,
-        ids: &DevBuf,
-        weights: &DevBuf,
-        y: &DevBuf,
-    ) {
-        // SAFETY: the buffers hold [tokens, E] logits, [tokens, hidden] activations and outputs and
-        // tokens * top_k routing entries; the weight handles were uploaded with these shapes.
-        unsafe {
-            check(lq4_moe_route(
-                self.ctx, router_logits.ptr as *const f32, tokens, moe.num_experts, moe.top_k,
-                ids.ptr as *mut i32, weights.ptr as *mut f32, self.stream,
-            ))
-            .expect("lq4_moe_route");
-            check(lq4_moe_grouped_gemv(
-                self.ctx, moe.gate_up.raw, moe.down.raw, moe.num_experts, moe.inter, moe.hidden,
-                x.ptr as *const f32, tokens, ids.ptr as *const i32, weights.ptr as *const f32,
-                moe.top_k, y.ptr as *mut f32, self.stream,
-            ))
-            .expect("lq4_moe_grouped_gemv");
-            check(lq4_moe_shared_expert(
-                self.ctx, moe.shared_gate_up.raw, moe.shared_down.raw,
-                moe.shared_expert_gate.ptr as *const f32, moe.shared_inter, moe.hidden,
-                x.ptr as *const f32, tokens, y.ptr as *mut f32, self.stream,
-            ))
-            .expect("lq4_moe_shared_expert");
-        }
+    /// router logits, the routed experts, and the always-active shared expert onto the same `y`, as one
+    /// library call.  Unlike the Metal path nothing is read back to the host between the steps (the
+    /// router and the shared expert's sigmoid gate stay on the device).
+    pub fn encode_moe_ffn(&self, router_logits: &DevBuf, moe: &HipMoeLayer, x: &DevBuf, tokens: u32, y: &DevBuf) {
+        // SAFETY: the buffers hold [tokens, E] logits and [tokens, hidden] activations and outputs; the
+        // weight handles were uploaded with these shapes.
+        check(unsafe {
+            lq4_moe_ffn(
+                self.ctx, router_logits.ptr as *const f32, moe.gate_up.raw, moe.down.raw, moe.num_experts, moe.top_k,
+                moe.inter, moe.shared_gate_up.raw, moe.shared_down.raw, moe.shared_expert_gate.ptr as *const f32,
+                moe.shared_inter, moe.hidden, x.ptr as *const f32, tokens, y.ptr as *mut f32, self.stream,
+            )
+        })
+        .expect("lq4_moe_ffn");
     }
 
     /// `commit()` + `wait_until_completed()` of the command buffer.

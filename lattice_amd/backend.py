@@ -44,7 +44,7 @@ EXPORTS = [
     "lq4_last_error", "lq4_version", "lq4_ctx_create", "lq4_ctx_destroy", "lq4_sync",
     "lq4_validate_blocks", "lq4_weight_upload", "lq4_weight_wrap", "lq4_weight_free",
     "lq4_weight_info", "lq4_lora_upload", "lq4_lora_free", "lq4_lora_apply", "lq4_gemv",
-    "lq4_gemm", "lq4_moe_route", "lq4_moe_grouped_gemv", "lq4_moe_shared_expert", "lq4_dequant",
+    "lq4_gemm", "lq4_moe_route", "lq4_moe_grouped_gemv", "lq4_moe_shared_expert", "lq4_moe_ffn", "lq4_dequant",
     "lq4_topk",
     "lq4_lm_head_topk",
     "lq4_probe_read",
@@ -134,6 +134,7 @@ def load_library() -> C.CDLL:
         "lq4_moe_route": (C.c_int, [vp, vp, u32, u32, u32, vp, vp, vp]),
         "lq4_moe_grouped_gemv": (C.c_int, [vp, vp, vp, u32, u32, u32, vp, u32, vp, vp, u32, vp, vp]),
         "lq4_moe_shared_expert": (C.c_int, [vp, vp, vp, vp, u32, u32, vp, u32, vp, vp]),
+        "lq4_moe_ffn": (C.c_int, [vp, vp, vp, vp, u32, u32, u32, vp, vp, vp, u32, u32, vp, u32, vp, vp]),
         "lq4_dequant": (C.c_int, [vp, vp, u64, u32, u32, vp, vp]),
         "lq4_topk": (C.c_int, [vp, vp, C.c_uint32, C.c_uint32, vp, vp, vp]),
         "lq4_lm_head_topk": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, C.c_uint32, vp, vp, vp]),
@@ -634,6 +635,16 @@ class HipQ4Backend:
         _check(self.lib.lq4_moe_shared_expert(self.ctx, gate_up.handle, down.handle, shared_gate.data_ptr(),
                                               shared_inter, hidden, x.data_ptr(), tokens, y.data_ptr(),
                                               self._stream()))
+
+    def moe_ffn(self, router_logits, gate_up: Q4WeightBuf, down: Q4WeightBuf, num_experts: int, top_k: int,
+                inter: int, shared_gate_up: Q4WeightBuf, shared_down: Q4WeightBuf, shared_gate, shared_inter: int,
+                hidden: int, x, y):
+        """``moe_ffn_step`` (moe.rs:8-36) from the router logits on: route, routed experts, shared expert;
+        ``y`` is overwritten."""
+        tokens = x.shape[0] if x.dim() > 1 else 1
+        _check(self.lib.lq4_moe_ffn(self.ctx, router_logits.data_ptr(), gate_up.handle, down.handle, num_experts,
+                                    top_k, inter, shared_gate_up.handle, shared_down.handle, shared_gate.data_ptr(),
+                                    shared_inter, hidden, x.data_ptr(), tokens, y.data_ptr(), self._stream()))
 
     def moe_experts(self, gate_up: Q4WeightBuf, down: Q4WeightBuf, num_experts: int, inter: int,
                     hidden: int, x, ids, weights, y):

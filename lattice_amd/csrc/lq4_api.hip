@@ -589,33 +589,50 @@ int lq4_moe_grouped_gemv(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_weig
     return LQ4_OK;
 }
 
-int lq4_moe_shared_expert(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_weight* down,
-                          const float* shared_gate_dev, uint32_t shared_inter, uint32_t hidden, const float* x_dev,
-                          uint32_t tokens, float* y_dev, void* stream) {
-    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
-    if (tokens == 0 || hidden == 0) return LQ4_OK;
-    if (!x_dev || !y_dev || !shared_gate_dev) return fail(LQ4_E_INVALID, "null device pointer");
-    if (shared_inter == 0 || shared_inter % kBlockWeights)
-        return fail(LQ4_E_INVALID, "shared expert intermediate size must be a non-zero multiple of 32, got %u", shared_inter);
-    if (shared_inter > UINT32_MAX / 2) return fail(LQ4_E_INVALID, "shared expert intermediate size too large");
-    if (reinterpret_cast<uintptr_t>(x_dev) % 16) return fail(LQ4_E_INVALID, "x must be 16-byte aligned");
-    const uint8_t *gu, *dn;
-    int rc = resolve_weight(gate_up, 0, 2 * shared_inter, hidden, &gu);
-    if (rc) return rc;
-    rc = resolve_weight(down, 0, hidden, shared_inter, &dn);
-    if (rc) return rc;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    DeviceGuard g(ctx->device);
+namespace {
+
+// Scratch of the shared expert for `tokens` rows: [gate||up | act | out | packed activations of the
+// few-token kernel], then (lq4_moe_ffn) the routing tables.
+struct SharedScratch {
+    size_t gu, act, o, pack, ids, wts, total;
+};
+
+SharedScratch shared_scratch_layout(uint32_t tokens, uint32_t shared_inter, uint32_t hidden, uint32_t top_k) {
     auto up256 = [](size_t v) { return (v + 255) / 256 * 256; };
-    const size_t off_gu = 0;
-    const size_t off_act = off_gu + up256(sizeof(float) * tokens * 2 * shared_inter);
-    const size_t off_o = off_act + up256(sizeof(float) * tokens * shared_inter);
-    const size_t total = off_o + up256(sizeof(float) * tokens * hidden);
-    rc = grow_scratch(ctx, &ctx->shared_scratch, &ctx->shared_scratch_bytes, total, s, false);
-    if (rc) return rc;
-    float* gu_out = reinterpret_cast<float*>(ctx->shared_scratch + off_gu);
-    float* act = reinterpret_cast<float*>(ctx->shared_scratch + off_act);
-    float* o = reinterpret_cast<float*>(ctx->shared_scratch + off_o);
+    SharedScratch l;
+    l.gu = 0;
+    l.act = l.gu + up256(sizeof(float) * tokens * 2 * shared_inter);
+    l.o = l.act + up256(sizeof(float) * tokens * shared_inter);
+    l.pack = l.o + up256(sizeof(float) * tokens * hidden);
+    const uint32_t kmax = hidden > shared_inter ? hidden : shared_inter;
+    l.ids = l.pack + up256(tokens <= kMaxGemvBatch ? gemm_skinny_scratch_bytes(kmax, tokens) : 0);
+    l.wts = l.ids + up256(sizeof(int32_t) * tokens * top_k);
+    l.total = l.wts + up256(sizeof(float) * tokens * top_k);
+    return l;
+}
+
+// W . x for up to kMaxGemvBatch rows with explicit scratch (the routing of lq4_gemv without LoRA).
+void small_batch_gemv(lq4_ctx* ctx, const uint8_t* wp, uint32_t n, uint32_t k, const float* x, uint32_t rows, float* y,
+                      uint8_t* pack, hipStream_t s) {
+    const LoraEpilogue none{};
+    const uint64_t weights = static_cast<uint64_t>(n) * k;
+    const bool narrow = n <= 2048 && gemv_mfma_lds_bytes(k, rows < 8 ? rows : 8) <= 150 * 1024;
+    if (rows >= 9 || (rows >= 5 && n < 8192 && !narrow && weights >= 6000000)) {
+        launch_gemm_skinny(wp, n, k, x, 0, rows, y, none, pack, s);
+        ctx->counters.gemm++;
+    } else {
+        launch_gemv(wp, n, k, x, k, rows, y, n, none, s);
+        ctx->counters.gemv++;
+    }
+}
+
+// The shared expert's FFN into scratch `o` (everything but the gate and the add).
+int shared_expert_ffn(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_weight* down, const uint8_t* gu,
+                      const uint8_t* dn, uint32_t shared_inter, uint32_t hidden, const float* x_dev, uint32_t tokens,
+                      uint8_t* base, const SharedScratch& l, hipStream_t s) {
+    float* gu_out = reinterpret_cast<float*>(base + l.gu);
+    float* act = reinterpret_cast<float*>(base + l.act);
+    float* o = reinterpret_cast<float*>(base + l.o);
     const LoraEpilogue none{};
     if (tokens == 1 && gemv_b1_lds_bytes(shared_inter) <= 128 * 1024) {
         // gate||up, then the down projection with silu(gate) * up computed as it stages its activations
@@ -626,15 +643,91 @@ int lq4_moe_shared_expert(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_wei
         launch_gemv_b1_fused(dn, hidden, shared_inter, gu_out, o, none, gf, s);
         ctx->counters.gemv++;
         ctx->counters.gemv_fused++;
+    } else if (tokens <= kMaxGemvBatch) {
+        small_batch_gemv(ctx, gu, 2 * shared_inter, hidden, x_dev, tokens, gu_out, base + l.pack, s);
+        launch_silu_mul(gu_out, shared_inter, tokens, act, shared_inter, s);
+        ctx->counters.elementwise++;
+        small_batch_gemv(ctx, dn, hidden, shared_inter, act, tokens, o, base + l.pack, s);
     } else {
-        rc = lq4_gemm(ctx, gate_up, 0, 2 * shared_inter, hidden, x_dev, LQ4_F32, tokens, gu_out, nullptr, 0.0f, stream);
+        int rc = lq4_gemm(ctx, gate_up, 0, 2 * shared_inter, hidden, x_dev, LQ4_F32, tokens, gu_out, nullptr, 0.0f, s);
         if (rc) return rc;
         launch_silu_mul(gu_out, shared_inter, tokens, act, shared_inter, s);
         ctx->counters.elementwise++;
-        rc = lq4_gemm(ctx, down, 0, hidden, shared_inter, act, LQ4_F32, tokens, o, nullptr, 0.0f, stream);
+        rc = lq4_gemm(ctx, down, 0, hidden, shared_inter, act, LQ4_F32, tokens, o, nullptr, 0.0f, s);
         if (rc) return rc;
     }
-    launch_moe_shared_gate_add(x_dev, shared_gate_dev, o, hidden, tokens, y_dev, s);
+    return LQ4_OK;
+}
+
+int check_shared_expert_args(const lq4_weight* gate_up, const lq4_weight* down, const float* shared_gate_dev,
+                             uint32_t shared_inter, uint32_t hidden, const float* x_dev, const float* y_dev,
+                             const uint8_t** gu, const uint8_t** dn) {
+    if (!x_dev || !y_dev || !shared_gate_dev) return fail(LQ4_E_INVALID, "null device pointer");
+    if (shared_inter == 0 || shared_inter % kBlockWeights)
+        return fail(LQ4_E_INVALID, "shared expert intermediate size must be a non-zero multiple of 32, got %u", shared_inter);
+    if (shared_inter > UINT32_MAX / 2) return fail(LQ4_E_INVALID, "shared expert intermediate size too large");
+    if (reinterpret_cast<uintptr_t>(x_dev) % 16) return fail(LQ4_E_INVALID, "x must be 16-byte aligned");
+    int rc = resolve_weight(gate_up, 0, 2 * shared_inter, hidden, gu);
+    if (rc) return rc;
+    return resolve_weight(down, 0, hidden, shared_inter, dn);
+}
+
+}  // namespace
+
+int lq4_moe_shared_expert(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_weight* down,
+                          const float* shared_gate_dev, uint32_t shared_inter, uint32_t hidden, const float* x_dev,
+                          uint32_t tokens, float* y_dev, void* stream) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    if (tokens == 0 || hidden == 0) return LQ4_OK;
+    const uint8_t *gu, *dn;
+    int rc = check_shared_expert_args(gate_up, down, shared_gate_dev, shared_inter, hidden, x_dev, y_dev, &gu, &dn);
+    if (rc) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    DeviceGuard g(ctx->device);
+    const SharedScratch l = shared_scratch_layout(tokens, shared_inter, hidden, 0);
+    rc = grow_scratch(ctx, &ctx->shared_scratch, &ctx->shared_scratch_bytes, l.total, s, false);
+    if (rc) return rc;
+    rc = shared_expert_ffn(ctx, gate_up, down, gu, dn, shared_inter, hidden, x_dev, tokens, ctx->shared_scratch, l, s);
+    if (rc) return rc;
+    launch_moe_shared_gate_add(x_dev, shared_gate_dev, reinterpret_cast<const float*>(ctx->shared_scratch + l.o), hidden,
+                               tokens, y_dev, s);
+    ctx->counters.elementwise++;
+    LQ4_HIP(hipGetLastError());
+    return LQ4_OK;
+}
+
+int lq4_moe_ffn(lq4_ctx* ctx, const float* router_logits_dev, const lq4_weight* gate_up, const lq4_weight* down,
+                uint32_t num_experts, uint32_t top_k, uint32_t inter, const lq4_weight* shared_gate_up,
+                const lq4_weight* shared_down, const float* shared_gate_dev, uint32_t shared_inter, uint32_t hidden,
+                const float* x_dev, uint32_t tokens, float* y_dev, void* stream) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    if (tokens == 0 || hidden == 0) return LQ4_OK;
+    if (!router_logits_dev) return fail(LQ4_E_INVALID, "router logits pointer is null");
+    if (top_k == 0 || top_k > 16 || top_k > num_experts)
+        return fail(LQ4_E_INVALID, "top_k must be in 1..min(16, num_experts), got %u", top_k);
+    if (static_cast<uint64_t>(tokens) * top_k > 4096) return fail(LQ4_E_INVALID, "tokens*top_k must be in 1..4096");
+    const uint8_t *gu, *dn;
+    int rc = check_shared_expert_args(shared_gate_up, shared_down, shared_gate_dev, shared_inter, hidden, x_dev, y_dev, &gu, &dn);
+    if (rc) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    DeviceGuard g(ctx->device);
+    const SharedScratch l = shared_scratch_layout(tokens, shared_inter, hidden, top_k);
+    rc = grow_scratch(ctx, &ctx->shared_scratch, &ctx->shared_scratch_bytes, l.total, s, false);
+    if (rc) return rc;
+    uint8_t* base = ctx->shared_scratch;
+    int32_t* ids = reinterpret_cast<int32_t*>(base + l.ids);
+    float* wts = reinterpret_cast<float*>(base + l.wts);
+    // One stream: running the shared expert beside the routed experts on a second stream (forked and
+    // joined with events) was measured slower, eagerly and in a captured graph alike (1 token 38.3 ->
+    // 47.8 us, 16 tokens 68.0 -> 66.9 eager / 72.3 captured): each of these launches fills the GPU by
+    // itself, and the cross-stream waits cost more than the overlap of their ramps returns.
+    rc = lq4_moe_route(ctx, router_logits_dev, tokens, num_experts, top_k, ids, wts, stream);
+    if (rc) return rc;
+    rc = lq4_moe_grouped_gemv(ctx, gate_up, down, num_experts, inter, hidden, x_dev, tokens, ids, wts, top_k, y_dev, stream);
+    if (rc) return rc;
+    rc = shared_expert_ffn(ctx, shared_gate_up, shared_down, gu, dn, shared_inter, hidden, x_dev, tokens, base, l, s);
+    if (rc) return rc;
+    launch_moe_shared_gate_add(x_dev, shared_gate_dev, reinterpret_cast<const float*>(base + l.o), hidden, tokens, y_dev, s);
     ctx->counters.elementwise++;
     LQ4_HIP(hipGetLastError());
     return LQ4_OK;

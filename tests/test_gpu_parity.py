@@ -473,6 +473,58 @@ def test_moe_layer_routed_plus_shared_expert(be):
     assert e_stage <= 2 * REL_TOL and e_whole <= 2 * REL_TOL
 
 
+@pytest.mark.parametrize("tokens", [1, 6, 16, 40])
+def test_moe_ffn_one_call_equals_the_three_calls(be, tokens):
+    """lq4_moe_ffn against route + routed experts + shared expert called one after the other: the same
+    kernels, so the same bits; eagerly and as a captured graph replayed with other work in between."""
+    import torch
+    e_, inter, sh_inter, hidden, top_k = 8, 64, 128, 256, 2
+    gu = be.upload_q4_blocks(synth.q4_weight(e_ * 2 * inter, hidden, seed=3, tag="moe_gu"))
+    dn = be.upload_q4_blocks(synth.q4_weight(e_ * hidden, inter, seed=3, tag="moe_dn"))
+    sgu = be.upload_q4_blocks(synth.q4_weight(2 * sh_inter, hidden, seed=3, tag="sh_gu"))
+    sdn = be.upload_q4_blocks(synth.q4_weight(hidden, sh_inter, seed=3, tag="sh_dn"))
+    sg = dev((np.random.default_rng(3).normal(size=hidden) * 0.1).astype(np.float32))
+    print(f"moe ffn tokens={tokens}", flush=True)
+
+    def inputs(seed):
+        return dev(synth.activations(tokens, hidden, seed=seed, tag="moe_x")), dev(synth.router_logits(tokens, e_, seed=seed))
+
+    def three_calls(x, lg):
+        ids, wts = be.moe_route(lg, top_k)
+        y = torch.full((tokens, hidden), float("nan"), dtype=torch.float32, device="cuda")
+        be.moe_experts(gu, dn, e_, inter, hidden, x, ids, wts, y)
+        be.moe_shared_expert(sgu, sdn, sg, sh_inter, hidden, x, y)
+        return host(y)
+
+    x, lg = inputs(3)
+    want = three_calls(x, lg)
+    assert np.isfinite(want).all()
+    y = torch.full((tokens, hidden), float("nan"), dtype=torch.float32, device="cuda")
+    for _ in range(3):  # back-to-back calls share the scratch
+        y.fill_(float("nan"))
+        be.moe_ffn(lg, gu, dn, e_, top_k, inter, sgu, sdn, sg, sh_inter, hidden, x, y)
+        assert np.array_equal(host(y).view(np.uint32), want.view(np.uint32))
+
+    # captured: replays see new inputs through the same buffers
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        be.moe_ffn(lg, gu, dn, e_, top_k, inter, sgu, sdn, sg, sh_inter, hidden, x, y)  # scratch sized before the capture
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            be.moe_ffn(lg, gu, dn, e_, top_k, inter, sgu, sdn, sg, sh_inter, hidden, x, y)
+    for seed in (4, 5, 6):
+        x2, lg2 = inputs(seed)
+        want2 = three_calls(x2, lg2)  # eager work between the replays
+        x.copy_(x2)
+        lg.copy_(lg2)
+        y.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(host(y).view(np.uint32), want2.view(np.uint32)), seed
+
+
 def test_moe_shared_expert_argument_checks(be):
     import torch
     gu, dn = be.upload_q4_blocks(synth.q4_weight(128, 64)), be.upload_q4_blocks(synth.q4_weight(64, 64))

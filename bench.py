@@ -573,6 +573,19 @@ def main():
         for i in range(3):
             one_call(i)
         ms_one = tm(torch, one_call, 40)
+        # decode: the same layer for one token (8 routed experts + the shared one, 28.3 MB)
+        lg1, x1, y1 = lg[:1].contiguous(), xm[:1].contiguous(), torch.empty((1, H), device="cuda")
+        def decode_layer(i):
+            sh = shared[i % len(shared)]
+            be.moe_ffn(lg1, sets[i % len(sets)][0], sets[i % len(sets)][1], E, TK, I, sh[0], sh[1], sgate, I, H, x1, y1)
+        for i in range(3):
+            decode_layer(i)
+        ms_decode = tm(torch, decode_layer, 40)
+        decode_bytes = (TK + 1) * (2 * I * (H // 32) * 20 + H * (I // 32) * 20)
+        out["moe_layer_one_token"] = {"algorithmic_bytes": decode_bytes, "ms_per_step": round(ms_decode, 4),
+                                      "GB/s": round(decode_bytes / ms_decode / 1e6, 1),
+                                      "pct_of_hbm_peak": round(100 * decode_bytes / ms_decode / 1e6 / HBM_PEAK_GBPS, 2),
+                                      "launches": 3}
         out["moe_grouped_gemv"] = {"distinct_experts": distinct, "algorithmic_bytes": moe_bytes,
                                    "ms_per_step": round(ms, 4), "GB/s": round(moe_bytes / ms / 1e6, 1),
                                    "pct_of_hbm_peak": round(100 * moe_bytes / ms / 1e6 / HBM_PEAK_GBPS, 2),

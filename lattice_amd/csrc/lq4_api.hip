@@ -61,6 +61,7 @@ struct lq4_lora {
 namespace {
 
 constexpr size_t kFusedPrologueBytes = 64u << 10;  // lq4_gemv_fused_batch: see there
+constexpr uint32_t kMoeB1MaxTokens = 8;  // per-pair expert kernels up to here (measured: 1 / 2 / 4 / 8 / 16 tokens 27.5 / 30.5 / 43.2 / 45.1 / 48.6 us grouped, 13.7 / 18.3 / 25.9 / 39.1 / 65.0 per pair)
 constexpr uint32_t kLoraTRows = 4096;  // most rows one LoRA-fused call may carry
 
 thread_local char g_err[512] = "";
@@ -563,6 +564,22 @@ int lq4_moe_grouped_gemv(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_weig
     if (rc) return rc;
 
     DeviceGuard g(ctx->device);
+    // A few tokens (decode): per-pair one-token GEMVs.  Pairs rarely share an expert then, and what is
+    // read twice costs less than the grouped kernels' fixed parts.
+    static const uint32_t b1_tokens = [] {
+        const char* env = getenv("LQ4_MOE_B1_TOKENS");
+        return env ? static_cast<uint32_t>(strtoul(env, nullptr, 10)) : kMoeB1MaxTokens;
+    }();
+    if (tokens <= b1_tokens && moe_b1_serves(inter, hidden, top_k)) {
+        rc = ensure_scratch(ctx, moe_b1_scratch_bytes(tokens, top_k, inter), static_cast<hipStream_t>(stream));
+        if (rc) return rc;
+        launch_moe_b1(gu, dn, num_experts, inter, hidden, x_dev, tokens, ids_dev, weights_dev, top_k, y_dev,
+                      reinterpret_cast<float*>(ctx->moe_scratch), nullptr, nullptr, nullptr, static_cast<hipStream_t>(stream));
+        ctx->counters.moe_gate_up++;
+        ctx->counters.moe_down++;
+        LQ4_HIP(hipGetLastError());
+        return LQ4_OK;
+    }
     const size_t pairs = static_cast<size_t>(tokens) * top_k;
     auto up256 = [](size_t v) { return (v + 255) / 256 * 256; };
     const size_t off_counts = 0;
@@ -717,6 +734,31 @@ int lq4_moe_ffn(lq4_ctx* ctx, const float* router_logits_dev, const lq4_weight* 
     uint8_t* base = ctx->shared_scratch;
     int32_t* ids = reinterpret_cast<int32_t*>(base + l.ids);
     float* wts = reinterpret_cast<float*>(base + l.wts);
+    // A few tokens, shared expert as wide as the routed ones: it rides along as one more slot of the
+    // per-pair kernels (route, gate||up, down: three launches for the whole layer).
+    const uint8_t *rgu, *rdn;
+    static const uint32_t b1_tokens = [] {
+        const char* env = getenv("LQ4_MOE_B1_TOKENS");
+        return env ? static_cast<uint32_t>(strtoul(env, nullptr, 10)) : kMoeB1MaxTokens;
+    }();
+    if (tokens <= b1_tokens && shared_inter == inter && inter % kBlockWeights == 0 && moe_b1_serves(inter, hidden, top_k + 1) &&
+        num_experts <= 1024 && static_cast<uint64_t>(num_experts) * 2 * inter <= UINT32_MAX &&
+        static_cast<uint64_t>(num_experts) * hidden <= UINT32_MAX) {
+        rc = resolve_weight(gate_up, 0, num_experts * 2 * inter, hidden, &rgu);
+        if (rc) return rc;
+        rc = resolve_weight(down, 0, num_experts * hidden, inter, &rdn);
+        if (rc) return rc;
+        rc = lq4_moe_route(ctx, router_logits_dev, tokens, num_experts, top_k, ids, wts, stream);
+        if (rc) return rc;
+        rc = ensure_scratch(ctx, moe_b1_scratch_bytes(tokens, top_k + 1, inter), s);
+        if (rc) return rc;
+        launch_moe_b1(rgu, rdn, num_experts, inter, hidden, x_dev, tokens, ids, wts, top_k, y_dev,
+                      reinterpret_cast<float*>(ctx->moe_scratch), gu, dn, shared_gate_dev, s);
+        ctx->counters.moe_gate_up++;
+        ctx->counters.moe_down++;
+        LQ4_HIP(hipGetLastError());
+        return LQ4_OK;
+    }
     // One stream: running the shared expert beside the routed experts on a second stream (forked and
     // joined with events) was measured slower, eagerly and in a captured graph alike (1 token 38.3 ->
     // 47.8 us, 16 tokens 68.0 -> 66.9 eager / 72.3 captured): each of these launches fills the GPU by

@@ -473,6 +473,44 @@ def test_moe_layer_routed_plus_shared_expert(be):
     assert e_stage <= 2 * REL_TOL and e_whole <= 2 * REL_TOL
 
 
+@pytest.mark.parametrize("cfg", [dict(e=64, inter=512, hidden=2048, tokens=1, top_k=8),   # config 4's layer, decode
+                                 dict(e=64, inter=512, hidden=2048, tokens=4, top_k=8),
+                                 dict(e=6, inter=96, hidden=160, tokens=3, top_k=3),        # partial slabs
+                                 dict(e=5, inter=160, hidden=1056, tokens=2, top_k=2),
+                                 dict(e=9, inter=2048, hidden=4096, tokens=1, top_k=4),     # four slabs in the down pass
+                                 dict(e=16, inter=32, hidden=64, tokens=4, top_k=8),
+                                 dict(e=4, inter=1056, hidden=256, tokens=2, top_k=8)])     # top_k * inter > 8192: grouped kernels
+def test_moe_experts_for_a_few_tokens(be, cfg):
+    """Decode-sized steps take the per-pair kernels (one-token GEMV arithmetic, the weighted sum over the
+    slots inside the down pass); unfilled slots (-1) and ids past the expert count are skipped."""
+    import torch
+    e_, inter, hidden, tokens, top_k = cfg["e"], cfg["inter"], cfg["hidden"], cfg["tokens"], cfg["top_k"]
+    print(f"moe few tokens {cfg}", flush=True)
+    gu = synth.q4_weight(e_ * 2 * inter, hidden, seed=5, tag="moe_gu")
+    dn = synth.q4_weight(e_ * hidden, inter, seed=5, tag="moe_dn")
+    x = synth.activations(tokens, hidden, seed=5, tag="moe_x")
+    lg = synth.router_logits(tokens, e_, seed=5)
+    ids, wts, _ = oracle.moe_route(lg, min(top_k, e_))
+    if ids.shape[1] < top_k:  # more slots than experts: the rest unfilled
+        pad = top_k - ids.shape[1]
+        ids = np.concatenate([ids, np.full((tokens, pad), -1, np.int32)], axis=1)
+        wts = np.concatenate([wts, np.full((tokens, pad), 0.25, np.float32)], axis=1)
+    elif top_k >= 2:
+        ids[0, top_k - 1] = -1          # unfilled slot (moe.rs:147-149)
+        if tokens > 1:
+            ids[1, 0] = e_ + 3          # id past the expert count: skipped as well
+    qgu, qdn = be.upload_q4_blocks(gu), be.upload_q4_blocks(dn)
+    y = torch.full((tokens, hidden), float("nan"), dtype=torch.float32, device="cuda")
+    be.moe_experts(qgu, qdn, e_, inter, hidden, dev(x), dev(ids), dev(wts), y)
+    ref32 = oracle.moe_ffn(gu, dn, e_, inter, hidden, x, ids, wts)
+    ref64 = oracle.moe_ffn(gu, dn, e_, inter, hidden, x, ids, wts, f64=True)
+    e32, e64 = rel_err(host(y), ref32), rel_err(host(y), ref64)
+    print(f"  rel err vs f32 {e32:.2e}, vs f64 {e64:.2e}", flush=True)
+    assert e32 <= REL_TOL and e64 <= REL_TOL
+    if top_k * inter <= 8192:
+        assert e64 <= 2e-5  # f32-faithful: hi/lo f16 activations in both passes
+
+
 @pytest.mark.parametrize("tokens", [1, 6, 16, 40])
 def test_moe_ffn_one_call_equals_the_three_calls(be, tokens):
     """lq4_moe_ffn against route + routed experts + shared expert called one after the other: the same
@@ -523,6 +561,48 @@ def test_moe_ffn_one_call_equals_the_three_calls(be, tokens):
         graph.replay()
         torch.cuda.synchronize()
         assert np.array_equal(host(y).view(np.uint32), want2.view(np.uint32)), seed
+
+
+@pytest.mark.parametrize("cfg", [dict(e=64, inter=512, hidden=2048, tokens=1, top_k=8),   # config 4's layer, decode
+                                 dict(e=64, inter=512, hidden=2048, tokens=8, top_k=8),
+                                 dict(e=6, inter=96, hidden=160, tokens=3, top_k=3),
+                                 dict(e=8, inter=1024, hidden=512, tokens=2, top_k=7),      # 8 slots x 1024: four slabs
+                                 dict(e=8, inter=1024, hidden=512, tokens=2, top_k=8)])     # 9 x 1024 > 8192: three calls inside
+def test_moe_ffn_with_the_shared_expert_as_a_slot(be, cfg):
+    """A shared expert as wide as the routed ones rides along in the per-pair kernels for up to 8 tokens:
+    the whole layer against the oracle (routed f64 + shared f64) and against the three separate calls."""
+    import torch
+    e_, inter, hidden, tokens, top_k = cfg["e"], cfg["inter"], cfg["hidden"], cfg["tokens"], cfg["top_k"]
+    print(f"moe ffn, shared expert as a slot {cfg}", flush=True)
+    gu = synth.q4_weight(e_ * 2 * inter, hidden, seed=6, tag="moe_gu")
+    dn = synth.q4_weight(e_ * hidden, inter, seed=6, tag="moe_dn")
+    sgu = synth.q4_weight(2 * inter, hidden, seed=6, tag="sh_gu")
+    sdn = synth.q4_weight(hidden, inter, seed=6, tag="sh_dn")
+    x = synth.activations(tokens, hidden, seed=6, tag="moe_x")
+    lg = synth.router_logits(tokens, e_, seed=6)
+    sg = (np.random.default_rng(6).normal(size=hidden) * (2.0 / np.sqrt(hidden))).astype(np.float32)
+    ids, wts, _ = oracle.moe_route(lg, top_k)
+    routed64 = oracle.moe_ffn(gu, dn, e_, inter, hidden, x, ids, wts, f64=True)
+    want = oracle.moe_shared_expert(sgu, sdn, sg, inter, hidden, x, routed64, f64=True)
+    qgu, qdn, qsgu, qsdn = (be.upload_q4_blocks(b) for b in (gu, dn, sgu, sdn))
+    y = torch.full((tokens, hidden), float("nan"), dtype=torch.float32, device="cuda")
+    before = be.path_counters()
+    be.moe_ffn(dev(lg), qgu, qdn, e_, top_k, inter, qsgu, qsdn, dev(sg), inter, hidden, dev(x), y)
+    after = be.path_counters()
+    err = rel_err(host(y), want)
+    # the shared part alone, so that an error in it (or in its gate) cannot hide behind the routed sum
+    d_err = rel_err(host(y) - routed64, want - routed64)
+    print(f"  rel err {err:.2e}, shared part alone {d_err:.2e}", flush=True)
+    as_slot = (top_k + 1) * inter <= 8192
+    assert err <= (5e-5 if as_slot else REL_TOL) and d_err <= (2e-4 if as_slot else 2 * REL_TOL)
+    # route, gate||up, down: no separate shared-expert launches when it rode along
+    assert (after["gemv"] + after["gemm"] + after["gemv_fused"] + after["elementwise"] ==
+            before["gemv"] + before["gemm"] + before["gemv_fused"] + before["elementwise"]) == as_slot
+    y3 = torch.full((tokens, hidden), float("nan"), dtype=torch.float32, device="cuda")
+    d_ids, d_wts = be.moe_route(dev(lg), top_k)
+    be.moe_experts(qgu, qdn, e_, inter, hidden, dev(x), d_ids, d_wts, y3)
+    be.moe_shared_expert(qsgu, qsdn, dev(sg), inter, hidden, dev(x), y3)
+    assert rel_err(host(y), host(y3)) <= REL_TOL
 
 
 def test_moe_shared_expert_argument_checks(be):

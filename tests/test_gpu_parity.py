@@ -511,6 +511,34 @@ def test_moe_experts_for_a_few_tokens(be, cfg):
         assert e64 <= 2e-5  # f32-faithful: hi/lo f16 activations in both passes
 
 
+@pytest.mark.parametrize("cfg", [dict(e=64, inter=512, hidden=2048, tokens=16, top_k=8),   # config 4
+                                 dict(e=3, inter=512, hidden=512, tokens=21, top_k=2),     # every expert in several passes
+                                 dict(e=5, inter=1024, hidden=1024, tokens=9, top_k=3),    # 32 blocks per row both ways
+                                 dict(e=4, inter=2048, hidden=4096, tokens=10, top_k=2),   # one slab down, two up
+                                 dict(e=6, inter=544, hidden=2112, tokens=12, top_k=4),    # partial slabs
+                                 dict(e=40, inter=512, hidden=2048, tokens=120, top_k=8)]) # 960 pairs
+def test_moe_grouped_experts_with_several_passes_per_expert(be, cfg):
+    """Steps above 8 tokens: pairs grouped by expert, up to four per pass over the expert's blocks, experts
+    chosen by many tokens in several passes; unfilled slots skipped."""
+    import torch
+    e_, inter, hidden, tokens, top_k = cfg["e"], cfg["inter"], cfg["hidden"], cfg["tokens"], cfg["top_k"]
+    print(f"moe grouped, several passes {cfg}", flush=True)
+    gu = synth.q4_weight(e_ * 2 * inter, hidden, seed=8, tag="moe_gu")
+    dn = synth.q4_weight(e_ * hidden, inter, seed=8, tag="moe_dn")
+    x = synth.activations(tokens, hidden, seed=8, tag="moe_x")
+    lg = synth.router_logits(tokens, e_, seed=8)
+    ids, wts, _ = oracle.moe_route(lg, top_k)
+    ids[0, top_k - 1] = -1
+    ids[tokens - 1, 0] = e_ + 1
+    qgu, qdn = be.upload_q4_blocks(gu), be.upload_q4_blocks(dn)
+    y = torch.full((tokens, hidden), float("nan"), dtype=torch.float32, device="cuda")
+    be.moe_experts(qgu, qdn, e_, inter, hidden, dev(x), dev(ids), dev(wts), y)
+    ref64 = oracle.moe_ffn(gu, dn, e_, inter, hidden, x, ids, wts, f64=True)
+    err = rel_err(host(y), ref64)
+    print(f"  rel err vs f64 {err:.2e}", flush=True)
+    assert err <= 5e-5
+
+
 @pytest.mark.parametrize("tokens", [1, 6, 16, 40])
 def test_moe_ffn_one_call_equals_the_three_calls(be, tokens):
     """lq4_moe_ffn against route + routed experts + shared expert called one after the other: the same

@@ -219,7 +219,7 @@ template <bool DOWN>
 void launch_one(const MoeB1Args& a, uint32_t tokens, hipStream_t stream) {
     const uint32_t nb = a.k / kBlockWeights;
     const uint32_t slabs = (nb + 63) / 64;
-    const uint32_t rw = slabs == 1 ? 4 : slabs == 2 ? 2 : 1;
+    const uint32_t rw = slabs == 1 ? 4 : slabs <= 3 ? 2 : 1;
     const size_t lds = static_cast<size_t>(nb) * kXPitch * 4;
     // all waves of the step resident at once where the rows allow: 4096 waves over the tokens
     const uint32_t wave_rows = (a.n + rw - 1) / rw;
@@ -239,7 +239,7 @@ void launch_one(const MoeB1Args& a, uint32_t tokens, hipStream_t stream) {
     } while (0)
     if (slabs == 1) LQ4_MOE_B1(4, 1);
     else if (slabs == 2) LQ4_MOE_B1(2, 2);
-    else if (slabs == 3) LQ4_MOE_B1(1, 3);
+    else if (slabs == 3) LQ4_MOE_B1(2, 3);
     else LQ4_MOE_B1(1, 4);
 #undef LQ4_MOE_B1
 }

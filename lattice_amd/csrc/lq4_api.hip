@@ -574,7 +574,8 @@ int lq4_moe_grouped_gemv(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_weig
         rc = ensure_scratch(ctx, moe_b1_scratch_bytes(tokens, top_k, inter), static_cast<hipStream_t>(stream));
         if (rc) return rc;
         launch_moe_b1(gu, dn, num_experts, inter, hidden, x_dev, tokens, ids_dev, weights_dev, top_k, y_dev,
-                      reinterpret_cast<float*>(ctx->moe_scratch), nullptr, nullptr, nullptr, static_cast<hipStream_t>(stream));
+                      reinterpret_cast<float*>(ctx->moe_scratch), nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
+                      static_cast<hipStream_t>(stream));
         ctx->counters.moe_gate_up++;
         ctx->counters.moe_down++;
         LQ4_HIP(hipGetLastError());
@@ -748,12 +749,17 @@ int lq4_moe_ffn(lq4_ctx* ctx, const float* router_logits_dev, const lq4_weight* 
         if (rc) return rc;
         rc = resolve_weight(down, 0, num_experts * hidden, inter, &rdn);
         if (rc) return rc;
-        rc = lq4_moe_route(ctx, router_logits_dev, tokens, num_experts, top_k, ids, wts, stream);
-        if (rc) return rc;
+        // up to 256 experts the gate||up launch routes as well: two launches for the layer
+        const bool route_inside = num_experts <= 256;
+        if (!route_inside) {
+            rc = lq4_moe_route(ctx, router_logits_dev, tokens, num_experts, top_k, ids, wts, stream);
+            if (rc) return rc;
+        }
         rc = ensure_scratch(ctx, moe_b1_scratch_bytes(tokens, top_k + 1, inter), s);
         if (rc) return rc;
         launch_moe_b1(rgu, rdn, num_experts, inter, hidden, x_dev, tokens, ids, wts, top_k, y_dev,
-                      reinterpret_cast<float*>(ctx->moe_scratch), gu, dn, shared_gate_dev, s);
+                      reinterpret_cast<float*>(ctx->moe_scratch), gu, dn, shared_gate_dev,
+                      route_inside ? router_logits_dev : nullptr, ids, wts, s);
         ctx->counters.moe_gate_up++;
         ctx->counters.moe_down++;
         LQ4_HIP(hipGetLastError());

@@ -14,8 +14,12 @@
 // Slots with an id outside [0, E) are skipped as the reference skips them (moe.rs:147-149): they read
 // expert 0 (any valid address) and enter the sum with weight 0.
 // The shared expert (moe.rs:194-250) can ride along as one more slot with the weight
-// sigmoid(x . shared_gate): its 3 MB then cost two slightly longer launches instead of three more.
+// sigmoid(x . shared_gate): its 2 MB then cost two slightly longer launches instead of three more.
+// The router (moe.rs:39-125) can run inside the gate||up launch as well: one wave of every workgroup
+// repeats it for the workgroup's token (64 logits, eight wave-wide maxima), which costs each workgroup
+// about a microsecond before its first weight request and saves a launch of four.
 #include "lq4_b1_dev.hpp"
+#include "lq4_moe_route_dev.hpp"
 
 namespace lq4 {
 
@@ -39,6 +43,12 @@ struct MoeB1Args {
     const float* shared_gate;
     float* shared_wt;
     uint32_t slots;
+    // gate||up launch only: route inside the launch.  Wave 0 of every workgroup runs the router of its token
+    // from route_logits [tokens, E] (E <= 256) and the workgroup takes the ids from LDS; workgroup 0 of each
+    // token also stores ids and weights to ids_out / wts_out, where the down launch reads them.
+    const float* route_logits;
+    int32_t* ids_out;
+    float* wts_out;
 };
 
 __device__ __forceinline__ float silu_mul(float gate, float u) {
@@ -51,7 +61,9 @@ __device__ __forceinline__ float silu_mul(float gate, float u) {
 // chunks of RW rows, chunk c holding rows (c * RW + j) * n_waves + wid; the next chunk's blocks are in
 // flight while the current one is consumed.  SLABS = ceil(K / 2048): a lane owns block slab * 64 + lane
 // of a row.  Dynamic LDS: (K / 32) * kXPitch dwords.
-template <bool DOWN, int RW, int SLABS>
+// ROUTE (gate||up only): the router runs inside the launch (a separate instantiation, so that the plain one
+// carries none of it).
+template <bool DOWN, int RW, int SLABS, bool ROUTE>
 __global__ __launch_bounds__(256) void moe_b1_kernel(MoeB1Args a) {
     extern __shared__ __attribute__((aligned(16))) uint32_t xs[];
     lds_u32* const xsl = (lds_u32*)xs;
@@ -61,8 +73,9 @@ __global__ __launch_bounds__(256) void moe_b1_kernel(MoeB1Args a) {
     const uint32_t nbe = a.inter / kBlockWeights;  // blocks of one expert's down row
     const int32_t* ids = a.ids + static_cast<size_t>(token) * a.top_k;
     const float* wts = a.wts + static_cast<size_t>(token) * a.top_k;
+    __shared__ int32_t s_ids[ROUTE ? 16 : 1];
     auto expert_of = [&](uint32_t slot) {  // the shared expert's tensor holds one expert
-        const int32_t e = slot < a.top_k ? ids[slot] : 0;
+        const int32_t e = slot < a.top_k ? (ROUTE ? s_ids[slot] : ids[slot]) : 0;
         return (e >= 0 && static_cast<uint32_t>(e) < a.num_experts) ? static_cast<uint32_t>(e) : 0u;
     };
     // Read here, under a condition that is the same for the whole launch: inside weight_of the load would
@@ -100,6 +113,26 @@ __global__ __launch_bounds__(256) void moe_b1_kernel(MoeB1Args a) {
             ua[i] = reinterpret_cast<const float4*>(hp + a.inter)[0];
             ub[i] = reinterpret_cast<const float4*>(hp + a.inter)[1];
             wt[i] = weight_of(slot);
+        }
+    }
+
+    if constexpr (ROUTE) {
+        {
+            __shared__ float s_ev[256];
+            if (tid < 64) {
+                int32_t id;
+                float w;
+                route_one_token<4>(a.route_logits + static_cast<size_t>(token) * a.num_experts, a.num_experts, a.top_k, lane,
+                                   s_ev, id, w);
+                if (lane < a.top_k) {
+                    s_ids[lane] = id;
+                    if (blockIdx.x == 0) {
+                        a.ids_out[static_cast<size_t>(token) * a.top_k + lane] = id;
+                        a.wts_out[static_cast<size_t>(token) * a.top_k + lane] = w;
+                    }
+                }
+            }
+            __syncthreads();
         }
     }
 
@@ -215,7 +248,7 @@ __global__ __launch_bounds__(256) void moe_b1_kernel(MoeB1Args a) {
     if (c < chunks) consume(buf_a, c);
 }
 
-template <bool DOWN>
+template <bool DOWN, bool ROUTE = false>
 void launch_one(const MoeB1Args& a, uint32_t tokens, hipStream_t stream) {
     const uint32_t nb = a.k / kBlockWeights;
     const uint32_t slabs = (nb + 63) / 64;
@@ -231,11 +264,11 @@ void launch_one(const MoeB1Args& a, uint32_t tokens, hipStream_t stream) {
     do {                                                                                                       \
         static bool attr_set = false;                                                                          \
         if (!attr_set) {                                                                                       \
-            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(moe_b1_kernel<DOWN, RW_, SL_>),            \
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(moe_b1_kernel<DOWN, RW_, SL_, ROUTE>),     \
                                       hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);                  \
             attr_set = true;                                                                                   \
         }                                                                                                      \
-        hipLaunchKernelGGL((moe_b1_kernel<DOWN, RW_, SL_>), grid, block, lds, stream, a);                      \
+        hipLaunchKernelGGL((moe_b1_kernel<DOWN, RW_, SL_, ROUTE>), grid, block, lds, stream, a);               \
     } while (0)
     if (slabs == 1) LQ4_MOE_B1(4, 1);
     else if (slabs == 2) LQ4_MOE_B1(2, 2);
@@ -259,15 +292,20 @@ size_t moe_b1_scratch_bytes(uint32_t tokens, uint32_t slots, uint32_t inter) {
 void launch_moe_b1(const uint8_t* gate_up, const uint8_t* down, uint32_t num_experts, uint32_t inter, uint32_t hidden,
                    const float* x, uint32_t tokens, const int32_t* ids, const float* weights, uint32_t top_k, float* y,
                    float* scratch, const uint8_t* shared_gate_up, const uint8_t* shared_down, const float* shared_gate,
-                   hipStream_t stream) {
+                   const float* route_logits, int32_t* ids_out, float* wts_out, hipStream_t stream) {
     const uint32_t slots = shared_gate_up ? top_k + 1 : top_k;
     float* h = scratch;
     float* shared_wt = shared_gate_up ? scratch + static_cast<size_t>(tokens) * slots * 2 * inter : nullptr;
+    if (route_logits) {  // the gate||up launch routes; the down launch reads what it stored
+        ids = ids_out;
+        weights = wts_out;
+    }
     MoeB1Args g{gate_up, x, h, ids, weights, num_experts, top_k, inter, hidden, slots * 2 * inter, hidden,
-                shared_gate_up, shared_gate, shared_wt, slots};
-    launch_one<false>(g, tokens, stream);
+                shared_gate_up, shared_gate, shared_wt, slots, route_logits, ids_out, wts_out};
+    if (route_logits) launch_one<false, true>(g, tokens, stream);
+    else launch_one<false>(g, tokens, stream);
     MoeB1Args d{down, h, y, ids, weights, num_experts, top_k, inter, hidden, hidden, slots * inter,
-                shared_down, shared_gate, shared_wt, slots};
+                shared_down, shared_gate, shared_wt, slots, nullptr, nullptr, nullptr};
     launch_one<true>(d, tokens, stream);
 }
 

@@ -174,10 +174,6 @@ __device__ __forceinline__ void topk_select_tail(const float* __restrict__ logit
                                                  float* __restrict__ out_logits, uint32_t* __restrict__ out_ids) {
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63;
-#ifdef LQ4_TAIL_PROBE
-    uint64_t tp[6];
-    tp[0] = wall_clock64();
-#endif
     if (tid == 0) {
         ts.count = 0;
         ts.nsel = 0;
@@ -199,10 +195,6 @@ __device__ __forceinline__ void topk_select_tail(const float* __restrict__ logit
                                   : 0ull;
     const uint32_t most = topk_most_blocks(k);
     uint64_t tau = 0;
-#ifdef LQ4_TAIL_PROBE
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    tp[1] = wall_clock64();
-#endif
     for (int bit = 63, par = 0; bit >= 0; --bit, par ^= 1) {
         const uint64_t cand = tau | (1ull << bit);
         uint32_t c = 0;
@@ -217,9 +209,6 @@ __device__ __forceinline__ void topk_select_tail(const float* __restrict__ logit
         }
     }
 
-#ifdef LQ4_TAIL_PROBE
-    tp[2] = wall_clock64();
-#endif
     // (the block that holds the vector's last logit: its odd end is read separately below)
     const uint32_t last_blk = bl.runs == 1 ? (n - 1) / bl.run : ((n - 1) % bl.stride) / bl.run;
     // the blocks that can hold an element at or before tau: at most `most` (more only if tau is
@@ -240,9 +229,6 @@ __device__ __forceinline__ void topk_select_tail(const float* __restrict__ logit
     const uint32_t tau_u = static_cast<uint32_t>(tau >> 32);
     const float tau_f = tau_u < 0x007FFFFFu ? -INFINITY
                                             : __uint_as_float((tau_u >> 31) ? tau_u ^ 0x80000000u : ~tau_u);
-#ifdef LQ4_TAIL_PROBE
-    tp[3] = wall_clock64();
-#endif
     // All loads of a batch are issued before the first is looked at: one workgroup has to cover the
     // latency of the selected blocks by itself.  It also runs this code once per launch, straight from
     // memory: the batch is as small as the number of units allows (G loads per thread in flight), a unit
@@ -314,9 +300,6 @@ __device__ __forceinline__ void topk_select_tail(const float* __restrict__ logit
         }
     }
     __syncthreads();
-#ifdef LQ4_TAIL_PROBE
-    tp[4] = wall_clock64();
-#endif
     uint32_t total = ts.count;
     for (uint32_t e = tid; e < (total < kRankSlots ? total : kRankSlots); e += 256)
         ts.keys[e] = key_of(Cand{ts.vals[e], ts.ids[e]});
@@ -363,15 +346,6 @@ __device__ __forceinline__ void topk_select_tail(const float* __restrict__ logit
             out_ids[rank] = ~static_cast<uint32_t>(ck);
         }
     }
-#ifdef LQ4_TAIL_PROBE
-    __syncthreads();
-    tp[5] = wall_clock64();
-    if (tid == 0 && k <= 50) {
-        for (int i = 1; i < 6; ++i) out_logits[56 + i] = static_cast<float>(tp[i] - tp[i - 1]) * 10.0f;  // ns
-        out_logits[56] = static_cast<float>(total);
-        out_logits[62] = static_cast<float>(nsel);
-    }
-#endif
 }
 
 }  // namespace lq4

@@ -61,6 +61,7 @@ struct lq4_lora {
 namespace {
 
 constexpr size_t kFusedPrologueBytes = 64u << 10;  // lq4_gemv_fused_batch: see there
+constexpr uint32_t kSharedB1MaxTokens = 8;  // shared expert alone through the per-pair kernels up to here (route + routed + shared as three calls: 8 tokens 56.0 -> 51.7 us, 16 tokens 68.5 -> 66.6, 32 tokens 89.3 -> 94.3)
 constexpr uint32_t kMoeB1MaxTokens = 8;  // per-pair expert kernels up to here (measured: 1 / 2 / 4 / 8 / 16 tokens 27.5 / 30.5 / 43.2 / 45.1 / 48.6 us grouped, 13.7 / 18.3 / 25.9 / 39.1 / 65.0 per pair)
 constexpr uint32_t kLoraTRows = 4096;  // most rows one LoRA-fused call may carry
 
@@ -574,7 +575,7 @@ int lq4_moe_grouped_gemv(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_weig
         rc = ensure_scratch(ctx, moe_b1_scratch_bytes(tokens, top_k, inter), static_cast<hipStream_t>(stream));
         if (rc) return rc;
         launch_moe_b1(gu, dn, num_experts, inter, hidden, x_dev, tokens, ids_dev, weights_dev, top_k, y_dev,
-                      reinterpret_cast<float*>(ctx->moe_scratch), nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
+                      reinterpret_cast<float*>(ctx->moe_scratch), nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, false,
                       static_cast<hipStream_t>(stream));
         ctx->counters.moe_gate_up++;
         ctx->counters.moe_down++;
@@ -645,13 +646,31 @@ void small_batch_gemv(lq4_ctx* ctx, const uint8_t* wp, uint32_t n, uint32_t k, c
 }
 
 // The shared expert's FFN into scratch `o` (everything but the gate and the add).
+// Returns LQ4_OK with the result in `o`, 1 when the per-pair kernels did everything (gate and add onto y_accum
+// included: pass y_accum and shared_gate_dev to allow that), or an error.
 int shared_expert_ffn(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_weight* down, const uint8_t* gu,
                       const uint8_t* dn, uint32_t shared_inter, uint32_t hidden, const float* x_dev, uint32_t tokens,
-                      uint8_t* base, const SharedScratch& l, hipStream_t s) {
+                      uint8_t* base, const SharedScratch& l, hipStream_t s, const float* shared_gate_dev = nullptr,
+                      float* y_accum = nullptr) {
     float* gu_out = reinterpret_cast<float*>(base + l.gu);
     float* act = reinterpret_cast<float*>(base + l.act);
     float* o = reinterpret_cast<float*>(base + l.o);
     const LoraEpilogue none{};
+    static const uint32_t alone_tokens = [] {
+        const char* env = getenv("LQ4_MOE_SHARED_B1_TOKENS");
+        return env ? static_cast<uint32_t>(strtoul(env, nullptr, 10)) : kSharedB1MaxTokens;
+    }();
+    if (y_accum && tokens <= alone_tokens && moe_b1_serves(shared_inter, hidden, 1)) {
+        // a few tokens: the per-pair kernels with the shared expert as their only slot (its 2 MB are read
+        // once from memory and then out of the caches), gate and add inside: two launches
+        int rc = ensure_scratch(ctx, moe_b1_scratch_bytes(tokens, 1, shared_inter), s);
+        if (rc) return rc;
+        launch_moe_b1(gu, dn, 1, shared_inter, hidden, x_dev, tokens, nullptr, nullptr, 0, y_accum,
+                      reinterpret_cast<float*>(ctx->moe_scratch), gu, dn, shared_gate_dev, nullptr, nullptr, nullptr, true, s);
+        ctx->counters.moe_gate_up++;
+        ctx->counters.moe_down++;
+        return 1;  // done, including the gate and the add
+    }
     if (tokens == 1 && gemv_b1_lds_bytes(shared_inter) <= 128 * 1024) {
         // gate||up, then the down projection with silu(gate) * up computed as it stages its activations
         launch_gemv(gu, 2 * shared_inter, hidden, x_dev, hidden, 1, gu_out, 2 * shared_inter, none, s);
@@ -705,7 +724,12 @@ int lq4_moe_shared_expert(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_wei
     const SharedScratch l = shared_scratch_layout(tokens, shared_inter, hidden, 0);
     rc = grow_scratch(ctx, &ctx->shared_scratch, &ctx->shared_scratch_bytes, l.total, s, false);
     if (rc) return rc;
-    rc = shared_expert_ffn(ctx, gate_up, down, gu, dn, shared_inter, hidden, x_dev, tokens, ctx->shared_scratch, l, s);
+    rc = shared_expert_ffn(ctx, gate_up, down, gu, dn, shared_inter, hidden, x_dev, tokens, ctx->shared_scratch, l, s,
+                           shared_gate_dev, y_dev);
+    if (rc == 1) {
+        LQ4_HIP(hipGetLastError());
+        return LQ4_OK;
+    }
     if (rc) return rc;
     launch_moe_shared_gate_add(x_dev, shared_gate_dev, reinterpret_cast<const float*>(ctx->shared_scratch + l.o), hidden,
                                tokens, y_dev, s);
@@ -759,7 +783,7 @@ int lq4_moe_ffn(lq4_ctx* ctx, const float* router_logits_dev, const lq4_weight* 
         if (rc) return rc;
         launch_moe_b1(rgu, rdn, num_experts, inter, hidden, x_dev, tokens, ids, wts, top_k, y_dev,
                       reinterpret_cast<float*>(ctx->moe_scratch), gu, dn, shared_gate_dev,
-                      route_inside ? router_logits_dev : nullptr, ids, wts, s);
+                      route_inside ? router_logits_dev : nullptr, ids, wts, false, s);
         ctx->counters.moe_gate_up++;
         ctx->counters.moe_down++;
         LQ4_HIP(hipGetLastError());
@@ -773,7 +797,12 @@ int lq4_moe_ffn(lq4_ctx* ctx, const float* router_logits_dev, const lq4_weight* 
     if (rc) return rc;
     rc = lq4_moe_grouped_gemv(ctx, gate_up, down, num_experts, inter, hidden, x_dev, tokens, ids, wts, top_k, y_dev, stream);
     if (rc) return rc;
-    rc = shared_expert_ffn(ctx, shared_gate_up, shared_down, gu, dn, shared_inter, hidden, x_dev, tokens, base, l, s);
+    rc = shared_expert_ffn(ctx, shared_gate_up, shared_down, gu, dn, shared_inter, hidden, x_dev, tokens, base, l, s,
+                           shared_gate_dev, y_dev);
+    if (rc == 1) {
+        LQ4_HIP(hipGetLastError());
+        return LQ4_OK;
+    }
     if (rc) return rc;
     launch_moe_shared_gate_add(x_dev, shared_gate_dev, reinterpret_cast<const float*>(base + l.o), hidden, tokens, y_dev, s);
     ctx->counters.elementwise++;

@@ -142,13 +142,14 @@ void launch_add_and_copy(const float* src, float* residual, float* dst, size_t c
 // `slots` = top_k, or top_k + 1 with the shared expert riding along (its tensors and gate vector given,
 // its intermediate size equal to `inter`).  Serves hidden <= 8192 and slots * inter <= 8192.  With
 // `route_logits` [tokens, E] (E <= 256) the gate||up launch routes itself and stores ids and weights to
-// ids_out / wts_out (`ids` / `weights` are then ignored).
+// ids_out / wts_out (`ids` / `weights` are then ignored).  top_k == 0 with the shared tensors is the shared
+// expert alone; `accumulate` then adds it onto y (the routed experts' sum) instead of overwriting y.
 bool moe_b1_serves(uint32_t inter, uint32_t hidden, uint32_t slots);
 size_t moe_b1_scratch_bytes(uint32_t tokens, uint32_t slots, uint32_t inter);
 void launch_moe_b1(const uint8_t* gate_up, const uint8_t* down, uint32_t num_experts, uint32_t inter, uint32_t hidden,
                    const float* x, uint32_t tokens, const int32_t* ids, const float* weights, uint32_t top_k, float* y,
                    float* scratch, const uint8_t* shared_gate_up, const uint8_t* shared_down, const float* shared_gate,
-                   const float* route_logits, int32_t* ids_out, float* wts_out, hipStream_t stream);
+                   const float* route_logits, int32_t* ids_out, float* wts_out, bool accumulate, hipStream_t stream);
 // y[t, :] = fma(sigmoid(x[t] . gate), shared_out[t, :], y[t, :]) for every token
 void launch_moe_shared_gate_add(const float* x, const float* gate, const float* shared_out, uint32_t hidden,
                                 uint32_t tokens, float* y, hipStream_t stream);

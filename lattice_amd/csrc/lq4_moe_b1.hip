@@ -49,6 +49,7 @@ struct MoeB1Args {
     const float* route_logits;
     int32_t* ids_out;
     float* wts_out;
+    uint32_t accumulate;  // down launch: y += the result instead of y = (the shared expert alone, onto the routed sum)
 };
 
 __device__ __forceinline__ float silu_mul(float gate, float u) {
@@ -235,7 +236,10 @@ __global__ __launch_bounds__(256) void moe_b1_kernel(MoeB1Args a) {
             for (int t = 0; t < SLABS; ++t) acc = block_fma(cur[j][t], xb_[t], live[t], acc);
             acc = segment_sum<64>(acc);
             const uint32_t row = (c * RW + j) * n_waves + wid;
-            if (lane == 63 && row < a.n) a.y[static_cast<size_t>(token) * a.n + row] = acc;
+            if (lane == 63 && row < a.n) {
+                float* dst = a.y + static_cast<size_t>(token) * a.n + row;
+                *dst = (DOWN && a.accumulate) ? *dst + acc : acc;
+            }
         }
     };
     uint32_t c = 0;
@@ -292,7 +296,7 @@ size_t moe_b1_scratch_bytes(uint32_t tokens, uint32_t slots, uint32_t inter) {
 void launch_moe_b1(const uint8_t* gate_up, const uint8_t* down, uint32_t num_experts, uint32_t inter, uint32_t hidden,
                    const float* x, uint32_t tokens, const int32_t* ids, const float* weights, uint32_t top_k, float* y,
                    float* scratch, const uint8_t* shared_gate_up, const uint8_t* shared_down, const float* shared_gate,
-                   const float* route_logits, int32_t* ids_out, float* wts_out, hipStream_t stream) {
+                   const float* route_logits, int32_t* ids_out, float* wts_out, bool accumulate, hipStream_t stream) {
     const uint32_t slots = shared_gate_up ? top_k + 1 : top_k;
     float* h = scratch;
     float* shared_wt = shared_gate_up ? scratch + static_cast<size_t>(tokens) * slots * 2 * inter : nullptr;
@@ -301,11 +305,11 @@ void launch_moe_b1(const uint8_t* gate_up, const uint8_t* down, uint32_t num_exp
         weights = wts_out;
     }
     MoeB1Args g{gate_up, x, h, ids, weights, num_experts, top_k, inter, hidden, slots * 2 * inter, hidden,
-                shared_gate_up, shared_gate, shared_wt, slots, route_logits, ids_out, wts_out};
+                shared_gate_up, shared_gate, shared_wt, slots, route_logits, ids_out, wts_out, 0u};
     if (route_logits) launch_one<false, true>(g, tokens, stream);
     else launch_one<false>(g, tokens, stream);
     MoeB1Args d{down, h, y, ids, weights, num_experts, top_k, inter, hidden, hidden, slots * inter,
-                shared_down, shared_gate, shared_wt, slots, nullptr, nullptr, nullptr};
+                shared_down, shared_gate, shared_wt, slots, nullptr, nullptr, nullptr, accumulate ? 1u : 0u};
     launch_one<true>(d, tokens, stream);
 }
 

@@ -275,6 +275,40 @@ def test_fused_decode_mlp_for_several_rows(be, hidden, inter, batch):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("batch", [3, 8, 12])
+def test_fused_rows_with_a_lora_adapter_run_step_by_step(be, batch):
+    """lq4_gemv_fused_batch with an adapter on the projection: the prologue, the GEMV with its LoRA delta
+    (A.x of the normalised rows) and the residual add run one after the other; same result as the oracle."""
+    import torch
+    from lattice_amd import backend
+    n, k, rank = 96, 1024, 8
+    g = np.random.default_rng(31)
+    wq = synth.q4_weight(n, k, seed=31)
+    qw = be.upload_q4_blocks(wq)
+    base = g.normal(size=(batch, k)).astype(np.float32)
+    gamma = (g.normal(size=k) * 0.1).astype(np.float32)
+    res0 = g.normal(size=(batch, n)).astype(np.float32)
+    a, b = synth.lora_pair(rank, k, n, seed=31)
+    be.load_lora_adapter([backend.LoraLayerData(0, {"o_proj": (a, b)})], scale=1.5)
+    try:
+        before = be.path_counters()
+        y = torch.full((batch, n), float("nan"), device="cuda")
+        residual = dev(res0)
+        be.dispatch_matmul_fused(None, qw, y, n, k, norm=(dev(base), None, dev(gamma), 1e-6, None),
+                                 add_residual=(residual, None), layer_idx=0, module="o_proj", batch=batch)
+        after = be.path_counters()
+        assert after["gemv_fused"] == before["gemv_fused"] and after["elementwise"] == before["elementwise"] + 2
+        assert after["lora_a"] == before["lora_a"] + 1
+        xn = oracle.shifted_rms_norm(base, gamma, 1e-6)
+        want = oracle.lora_apply(a, b, 1.5, xn, oracle.gemm_f32(xn, wq, n, k))
+        for r in range(batch):
+            assert rel_err(host(y)[r], want[r]) <= REL_TOL, r
+        assert np.array_equal(host(residual), res0 + host(y))
+    finally:
+        be.unload_lora_adapter()
+
+
+@pytest.mark.gpu
 def test_fused_gemv_options_and_fallbacks(be):
     import torch
     from lattice_amd import backend

@@ -153,7 +153,9 @@ int lq4_moe_route(lq4_ctx* ctx, const float* logits_dev, uint32_t tokens, uint32
  * gate_up: [E, 2*inter, hidden] (gate rows then up rows per expert); down:
  * [E, hidden, inter]; both expert-major native blocks.  Tokens routed to the same
  * expert share one pass over that expert's weights.  x_dev f32 [tokens, hidden];
- * y_dev f32 [tokens, hidden] (overwritten).  tokens*top_k <= 4096. */
+ * y_dev f32 [tokens, hidden] (overwritten).  tokens*top_k <= 4096.  Up to 8 tokens (hidden <= 8192,
+ * top_k * inter <= 8192) every pair is served as a one-token GEMV and the weighted sum over a
+ * token's slots is formed inside the down pass; larger steps group the pairs by expert. */
 int lq4_moe_grouped_gemv(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_weight* down,
                          uint32_t num_experts, uint32_t inter, uint32_t hidden,
                          const float* x_dev, uint32_t tokens, const int32_t* ids_dev,
@@ -179,8 +181,12 @@ int lq4_moe_shared_expert(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_wei
  * lq4_moe_route, lq4_moe_grouped_gemv and lq4_moe_shared_expert behind one call, with the routing
  * tables in library scratch.  y_dev f32 [tokens, hidden] is overwritten.  Everything runs on
  * `stream` in order (the shared expert beside the routed experts on a second stream was measured
- * slower on MI355X).  Argument meaning and limits as in the three calls it replaces; same results
- * bit for bit. */
+ * slower on MI355X).  Argument meaning and limits as in the three calls it replaces, and the same
+ * results bit for bit, except for decode-sized steps: up to 8 tokens, with shared_inter == inter,
+ * hidden <= 8192 and (top_k + 1) * inter <= 8192, the layer runs as two launches (every
+ * (token, slot) pair as a one-token GEMV, the shared expert as one more slot, the router and the
+ * shared expert's gate inside the first launch when num_experts <= 256), whose sums are formed in a
+ * different order: equal to the three calls to f32 rounding (1e-5 relative). */
 int lq4_moe_ffn(lq4_ctx* ctx, const float* router_logits_dev, const lq4_weight* gate_up, const lq4_weight* down,
                 uint32_t num_experts, uint32_t top_k, uint32_t inter, const lq4_weight* shared_gate_up,
                 const lq4_weight* shared_down, const float* shared_gate_dev, uint32_t shared_inter,

@@ -149,6 +149,8 @@ __global__ __launch_bounds__(kThreads) void moe_expert_mfma(MoeGemvArgs p) {
     }
     constexpr int G = 4;
     const uint32_t total = static_cast<uint32_t>(nt) * items;
+    // (short rows: all of a pass's items fit one per thread; the round's other three slots are skipped)
+    const int live_slots = total <= kThreads ? 1 : G;
     struct Round {
         float4 va[G], vb[G];
         uint32_t wb[G], wi[G];
@@ -156,6 +158,7 @@ __global__ __launch_bounds__(kThreads) void moe_expert_mfma(MoeGemvArgs p) {
     auto load_round = [&](Round& r, uint32_t w0) {
 #pragma unroll
         for (int i = 0; i < G; ++i) {
+            if (i >= live_slots) break;  // uniform
             const uint32_t w = w0 + i * kThreads;
             const uint32_t wc = w < total ? w : 0;
             r.wb[i] = wc / items;
@@ -169,6 +172,7 @@ __global__ __launch_bounds__(kThreads) void moe_expert_mfma(MoeGemvArgs p) {
     auto store_round = [&](const Round& r, uint32_t w0) {
 #pragma unroll
         for (int i = 0; i < G; ++i) {
+            if (i >= live_slots) break;  // uniform
             const uint32_t blk = r.wi[i] >> 2, dw = r.wi[i] & 3, bb = r.wb[i];
             const float v[8] = {r.va[i].x, r.va[i].y, r.va[i].z, r.va[i].w, r.vb[i].x, r.vb[i].y, r.vb[i].z, r.vb[i].w};
             _Float16 h[8], l[8];
@@ -241,12 +245,12 @@ __global__ __launch_bounds__(kThreads) void moe_expert_mfma(MoeGemvArgs p) {
                 a_op[set][4 * i + 2] = v.z; a_op[set][4 * i + 3] = v.w;
             }
         }
-        float sum_x[kCols];
+        // sum of a pair's activations over the block (the bias term; it rides on the hi column only)
+        const float4 sums = *reinterpret_cast<const float4*>(xb + kCols * 4);
+        float sum_x[kTok] = {sums.x, sums.y, sums.z, sums.w};
 #pragma unroll
-        for (int c = 0; c < kCols; ++c) {
-            const bool has = (c % 2 == 0) && c / 2 < nt && live;
-            sum_x[c] = has ? reinterpret_cast<const float*>(xb + kCols * 4)[c / 2] : 0.0f;
-        }
+        for (int b = 0; b < kTok; ++b)
+            if (b >= nt || !live) sum_x[b] = 0.0f;
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             float4v prod[2] = {float4v{0.0f, 0.0f, 0.0f, 0.0f}, float4v{0.0f, 0.0f, 0.0f, 0.0f}};
@@ -270,23 +274,30 @@ __global__ __launch_bounds__(kThreads) void moe_expert_mfma(MoeGemvArgs p) {
             const float bias = f16_bits_to_f32(cur[t].sb >> 16);
             if (!live) d = 0.0f;
 #pragma unroll
-            for (int c = 0; c < kCols; ++c)
-                acc[t][c] = fmaf(d, prod[c / 4][c % 4], fmaf(bias, sum_x[c], acc[t][c]));
+            for (int c = 0; c < kCols; ++c) {
+                const float with_bias = (c & 1) ? acc[t][c] : fmaf(bias, sum_x[c / 2], acc[t][c]);
+                acc[t][c] = fmaf(d, prod[c / 4][c % 4], with_bias);
+            }
         }
     };
 
-    // tile pair finished for this wave: sum over the 16 blocks of a step (lanes with equal j)
+    // tile pair finished for this wave: sum over the 16 blocks of a step (lanes with equal j).  A pair's hi
+    // and lo column are joined first and only the pairs of this pass are reduced: with short rows (one
+    // step per tile pair) the cross-lane sums are a third of the kernel's vector instructions otherwise.
     auto finish = [&](uint32_t t_idx) {
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int c = 0; c < kCols; ++c) {
-                float v = acc[t][c];
-                acc[t][c] = 0.0f;
-                v = dpp_add<0x124>(v);  // row_ror:4
-                v = dpp_add<0x128>(v);  // row_ror:8
-                v = sum_over_rows(v);
-                if (lane < 4) red[(((wave * tp + t_idx) * 2 + t) * kCols + c) * 4 + lane] = v;
+            for (int b = 0; b < kTok; ++b) {
+                float v = fmaf(acc[t][2 * b + 1], 1.0f / kLoScale, acc[t][2 * b]);
+                acc[t][2 * b] = 0.0f;
+                acc[t][2 * b + 1] = 0.0f;
+                if (b < nt) {  // the same for the whole workgroup
+                    v = dpp_add<0x124>(v);  // row_ror:4
+                    v = dpp_add<0x128>(v);  // row_ror:8
+                    v = sum_over_rows(v);
+                    if (lane < 4) red[(((wave * tp + t_idx) * 2 + t) * kTok + b) * 4 + lane] = v;
+                }
             }
     };
 
@@ -318,14 +329,12 @@ __global__ __launch_bounds__(kThreads) void moe_expert_mfma(MoeGemvArgs p) {
         float v[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            float hi = 0.0f, lo = 0.0f;
+            float sum = 0.0f;
             for (int s = 0; s < KS; ++s) {
                 const uint32_t wv = rs_o * KS + s;
-                const float* r = red + (((wv * tp + t_idx) * 2 + t) * kCols) * 4;
-                hi += r[(2 * b) * 4 + jj];
-                lo += r[(2 * b + 1) * 4 + jj];
+                sum += red[((((wv * tp + t_idx) * 2 + t) * kTok) + b) * 4 + jj];
             }
-            v[t] = fmaf(lo, 1.0f / kLoScale, hi);
+            v[t] = sum;
         }
         const int32_t pair = s_pair[b];
         p.out[static_cast<size_t>(pair) * p.out_rows + row] = GATE_UP ? silu(v[0]) * v[1] : v[half];

@@ -149,8 +149,8 @@ __global__ __launch_bounds__(kThreads) void moe_expert_mfma(MoeGemvArgs p) {
     }
     constexpr int G = 4;
     const uint32_t total = static_cast<uint32_t>(nt) * items;
-    // (short rows: all of a pass's items fit one per thread; the round's other three slots are skipped)
-    const int live_slots = total <= kThreads ? 1 : G;
+    // (a pass with few items leaves slots of the round empty: they are skipped, not converted and dropped)
+    const int live_slots = total >= G * kThreads ? G : static_cast<int>((total + kThreads - 1) / kThreads);
     struct Round {
         float4 va[G], vb[G];
         uint32_t wb[G], wi[G];

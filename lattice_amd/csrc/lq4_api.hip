@@ -63,6 +63,7 @@ namespace {
 constexpr size_t kFusedPrologueBytes = 64u << 10;  // lq4_gemv_fused_batch: see there
 constexpr uint32_t kSharedB1MaxTokens = 8;  // shared expert alone through the per-pair kernels up to here (route + routed + shared as three calls: 8 tokens 56.0 -> 51.7 us, 16 tokens 68.5 -> 66.6, 32 tokens 89.3 -> 94.3)
 constexpr uint32_t kMoeB1MaxTokens = 8;  // per-pair expert kernels up to here (measured: 1 / 2 / 4 / 8 / 16 tokens 27.5 / 30.5 / 43.2 / 45.1 / 48.6 us grouped, 13.7 / 18.3 / 25.9 / 39.1 / 65.0 per pair)
+constexpr uint32_t kMoeSharedGroupedMaxTokens = 56;  // lq4_moe_ffn: shared expert as one more expert of the grouped kernels up to here
 constexpr uint32_t kLoraTRows = 4096;  // most rows one LoRA-fused call may carry
 
 thread_local char g_err[512] = "";
@@ -542,6 +543,26 @@ int lq4_moe_route(lq4_ctx* ctx, const float* logits_dev, uint32_t tokens, uint32
     return LQ4_OK;
 }
 
+// Scratch of the grouped expert kernels for `pairs` (token, slot) pairs over `experts` experts.
+static int grouped_scratch(lq4_ctx* ctx, uint32_t experts, size_t pairs, uint32_t inter, uint32_t hidden,
+                           hipStream_t stream, MoeScratch* s) {
+    auto up256 = [](size_t v) { return (v + 255) / 256 * 256; };
+    const size_t off_counts = 0;
+    const size_t off_offsets = off_counts + up256(sizeof(int32_t) * experts);
+    const size_t off_order = off_offsets + up256(sizeof(int32_t) * (experts + 1));
+    const size_t off_h = off_order + up256(sizeof(int32_t) * pairs);
+    const size_t off_o = off_h + up256(sizeof(float) * pairs * inter);
+    const size_t total = off_o + up256(sizeof(float) * pairs * hidden);
+    const int rc = ensure_scratch(ctx, total, stream);
+    if (rc) return rc;
+    s->counts = reinterpret_cast<int32_t*>(ctx->moe_scratch + off_counts);
+    s->offsets = reinterpret_cast<int32_t*>(ctx->moe_scratch + off_offsets);
+    s->order = reinterpret_cast<int32_t*>(ctx->moe_scratch + off_order);
+    s->h = reinterpret_cast<float*>(ctx->moe_scratch + off_h);
+    s->o = reinterpret_cast<float*>(ctx->moe_scratch + off_o);
+    return LQ4_OK;
+}
+
 int lq4_moe_grouped_gemv(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_weight* down,
                          uint32_t num_experts, uint32_t inter, uint32_t hidden, const float* x_dev,
                          uint32_t tokens, const int32_t* ids_dev, const float* weights_dev,
@@ -582,24 +603,10 @@ int lq4_moe_grouped_gemv(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_weig
         LQ4_HIP(hipGetLastError());
         return LQ4_OK;
     }
-    const size_t pairs = static_cast<size_t>(tokens) * top_k;
-    auto up256 = [](size_t v) { return (v + 255) / 256 * 256; };
-    const size_t off_counts = 0;
-    const size_t off_offsets = off_counts + up256(sizeof(int32_t) * num_experts);
-    const size_t off_order = off_offsets + up256(sizeof(int32_t) * (num_experts + 1));
-    const size_t off_h = off_order + up256(sizeof(int32_t) * pairs);
-    const size_t off_o = off_h + up256(sizeof(float) * pairs * inter);
-    const size_t total = off_o + up256(sizeof(float) * pairs * hidden);
-    {
-        const int src = ensure_scratch(ctx, total, static_cast<hipStream_t>(stream));
-        if (src) return src;
-    }
     MoeScratch s;
-    s.counts = reinterpret_cast<int32_t*>(ctx->moe_scratch + off_counts);
-    s.offsets = reinterpret_cast<int32_t*>(ctx->moe_scratch + off_offsets);
-    s.order = reinterpret_cast<int32_t*>(ctx->moe_scratch + off_order);
-    s.h = reinterpret_cast<float*>(ctx->moe_scratch + off_h);
-    s.o = reinterpret_cast<float*>(ctx->moe_scratch + off_o);
+    rc = grouped_scratch(ctx, num_experts, static_cast<size_t>(tokens) * top_k, inter, hidden,
+                         static_cast<hipStream_t>(stream), &s);
+    if (rc) return rc;
     launch_moe_grouped(gu, dn, num_experts, inter, hidden, x_dev, tokens, ids_dev, weights_dev, top_k, y_dev, s,
                        static_cast<hipStream_t>(stream));
     ctx->counters.moe_gate_up++;
@@ -625,8 +632,8 @@ SharedScratch shared_scratch_layout(uint32_t tokens, uint32_t shared_inter, uint
     l.pack = l.o + up256(sizeof(float) * tokens * hidden);
     const uint32_t kmax = hidden > shared_inter ? hidden : shared_inter;
     l.ids = l.pack + up256(tokens <= kMaxGemvBatch ? gemm_skinny_scratch_bytes(kmax, tokens) : 0);
-    l.wts = l.ids + up256(sizeof(int32_t) * tokens * top_k);
-    l.total = l.wts + up256(sizeof(float) * tokens * top_k);
+    l.wts = l.ids + up256(sizeof(int32_t) * tokens * (top_k + 1));  // (one more slot: the shared expert's)
+    l.total = l.wts + up256(sizeof(float) * tokens * (top_k + 1));
     return l;
 }
 
@@ -784,6 +791,34 @@ int lq4_moe_ffn(lq4_ctx* ctx, const float* router_logits_dev, const lq4_weight* 
         launch_moe_b1(rgu, rdn, num_experts, inter, hidden, x_dev, tokens, ids, wts, top_k, y_dev,
                       reinterpret_cast<float*>(ctx->moe_scratch), gu, dn, shared_gate_dev,
                       route_inside ? router_logits_dev : nullptr, ids, wts, false, s);
+        ctx->counters.moe_gate_up++;
+        ctx->counters.moe_down++;
+        LQ4_HIP(hipGetLastError());
+        return LQ4_OK;
+    }
+    // More tokens, shared expert as wide as the routed ones: it rides along in the grouped kernels as expert
+    // `num_experts`, chosen by every token in slot `top_k` with the sigmoid gate as its weight (the router
+    // launch computes it): route, gate||up, down, combine, and none of the shared expert's own launches.
+    // Whole layer, config 4's shapes, 12 / 16 / 32 / 48 tokens: 65.5 / 65.7 / 83.8 / 102.6 -> 49.9 / 50.0 / 71.4 / 88.8 us.
+    // From 64 tokens on the shared expert's own GEMMs (weights read once, 16x16x32 tiles) are level or ahead
+    // (64 / 128 / 512 tokens: 121.8 / 205.6 / 690 against 126.6 / 210.4 / 728).
+    static const uint32_t grouped_tokens = [] {
+        const char* env = getenv("LQ4_MOE_SHARED_GROUPED_TOKENS");
+        return env ? static_cast<uint32_t>(strtoul(env, nullptr, 10)) : kMoeSharedGroupedMaxTokens;
+    }();
+    if (tokens > b1_tokens && tokens <= grouped_tokens && shared_inter == inter && num_experts < 1024 && moe_mfma_serves(hidden) && moe_mfma_serves(inter) &&
+        static_cast<uint64_t>(num_experts) * 2 * inter <= UINT32_MAX &&
+        static_cast<uint64_t>(num_experts) * hidden <= UINT32_MAX) {
+        rc = resolve_weight(gate_up, 0, num_experts * 2 * inter, hidden, &rgu);
+        if (rc) return rc;
+        rc = resolve_weight(down, 0, num_experts * hidden, inter, &rdn);
+        if (rc) return rc;
+        MoeScratch ms;
+        rc = grouped_scratch(ctx, num_experts + 1, static_cast<size_t>(tokens) * (top_k + 1), inter, hidden, s, &ms);
+        if (rc) return rc;
+        launch_moe_route(router_logits_dev, tokens, num_experts, top_k, ids, wts, s, x_dev, shared_gate_dev, hidden);
+        ctx->counters.moe_route++;
+        launch_moe_grouped(rgu, rdn, num_experts, inter, hidden, x_dev, tokens, ids, wts, top_k, y_dev, ms, s, gu, dn);
         ctx->counters.moe_gate_up++;
         ctx->counters.moe_down++;
         LQ4_HIP(hipGetLastError());

@@ -229,8 +229,11 @@ bool launch_probe_read(const void* p, size_t nbytes, uint32_t grid, uint32_t in_
 void launch_probe_copy(const void* src, void* dst, size_t nbytes, hipStream_t stream);
 void launch_dequant(const uint8_t* w, uint32_t n, uint32_t k, float* out, hipStream_t stream);
 
+// With `shared_gate` the table has top_k + 1 slots per token and slot top_k carries expert id `num_experts`
+// with weight sigmoid(x[t] . shared_gate) (x: [tokens, hidden]).
 void launch_moe_route(const float* logits, uint32_t tokens, uint32_t num_experts, uint32_t top_k,
-                      int32_t* ids, float* weights, hipStream_t stream);
+                      int32_t* ids, float* weights, hipStream_t stream, const float* x = nullptr,
+                      const float* shared_gate = nullptr, uint32_t hidden = 0);
 
 // Scratch layout for the grouped MoE path, all sized by the caller:
 //   counts  i32 [E]        pairs routed to each expert
@@ -248,7 +251,12 @@ struct MoeScratch {
 void launch_moe_grouped(const uint8_t* gate_up, const uint8_t* down, uint32_t num_experts,
                         uint32_t inter, uint32_t hidden, const float* x, uint32_t tokens,
                         const int32_t* ids, const float* weights, uint32_t top_k, float* y,
-                        const MoeScratch& s, hipStream_t stream);
+                        const MoeScratch& s, hipStream_t stream, const uint8_t* shared_gate_up = nullptr,
+                        const uint8_t* shared_down = nullptr);
+// With shared tensors (an expert as wide as the routed ones; needs moe_mfma_serves(hidden) and
+// moe_mfma_serves(inter)) ids / weights are [tokens, top_k + 1] as launch_moe_route writes them with a shared
+// gate, and the scratch is sized for tokens * (top_k + 1) pairs and num_experts + 1 experts.
+bool moe_mfma_serves(uint32_t k);
 
 // Matrix-core forms of the two expert passes (activations of a pass staged in LDS:
 // moe_mfma_lds_bytes(k) bytes for a reduction length k).
@@ -257,10 +265,13 @@ size_t moe_mfma_lds_bytes(uint32_t k);
 // order are then unused); null: they read the grouping tables.
 void launch_moe_gate_up_mfma(const uint8_t* gate_up, uint32_t num_experts, uint32_t inter, uint32_t hidden,
                              const float* x, uint32_t tokens, uint32_t top_k, const int32_t* offsets,
-                             const int32_t* order, const int32_t* ids, float* h, hipStream_t stream);
+                             const int32_t* order, const int32_t* ids, float* h, hipStream_t stream,
+                             const uint8_t* last_expert = nullptr);
 void launch_moe_down_mfma(const uint8_t* down, uint32_t num_experts, uint32_t inter, uint32_t hidden,
                           const float* h, uint32_t tokens, uint32_t top_k, const int32_t* offsets,
-                          const int32_t* order, const int32_t* ids, float* o, hipStream_t stream);
+                          const int32_t* order, const int32_t* ids, float* o, hipStream_t stream,
+                          const uint8_t* last_expert = nullptr);
+// (`last_expert`: the tensor of expert num_experts - 1 when it does not follow the others in `gate_up` / `down`)
 
 // Exact top-k over n logits (k <= 256): out_logits / out_ids receive the k best in rank order.
 // `scratch` must hold topk_scratch_bytes(n, k) bytes; `ticket` is one device word that is zero

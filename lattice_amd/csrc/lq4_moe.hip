@@ -15,20 +15,63 @@ namespace {
 constexpr int kMaxExperts = 1024;
 constexpr uint32_t kSmallPairs = 512;  // pair count up to which the grouping kernel ranks by scanning
 
-// Router of one token per wave: see route_one_token.
+// Router of one token per wave: see route_one_token.  The routing table has `out_stride` slots per token.
+// With a shared expert (`shared_gate` not null) the wave also fills slot `top_k`: expert id `num_experts` (the
+// grouped kernels read that expert from the shared expert's own tensors) with weight sigmoid(x . shared_gate).
 template <int kPerLane>
 __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ logits, uint32_t tokens,
                                                        uint32_t num_experts, uint32_t top_k,
-                                                       int32_t* __restrict__ ids, float* __restrict__ weights) {
+                                                       int32_t* __restrict__ ids, float* __restrict__ weights,
+                                                       uint32_t out_stride, const float* __restrict__ x,
+                                                       const float* __restrict__ shared_gate, uint32_t hidden) {
     __shared__ float s_ev[64 * kPerLane];
     const uint32_t t = blockIdx.x;
     const uint32_t lane = threadIdx.x;
+    float dot = 0.0f;
+    if (shared_gate != nullptr) {
+        const float* xr = x + static_cast<size_t>(t) * hidden;
+        if (hidden % 4 == 0 && reinterpret_cast<uintptr_t>(xr) % 16 == 0 && reinterpret_cast<uintptr_t>(shared_gate) % 16 == 0) {
+            // 16-byte loads, four rounds in flight together (a dependent chain of single loads made this the
+            // longest launch of the layer)
+            const float4* x4 = reinterpret_cast<const float4*>(xr);
+            const float4* g4 = reinterpret_cast<const float4*>(shared_gate);
+            const uint32_t n4 = hidden / 4;
+            float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            for (uint32_t i0 = lane; i0 < n4; i0 += 4 * 64) {
+                float4 xv[4], gv[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const uint32_t i = i0 + r * 64 < n4 ? i0 + r * 64 : lane;
+                    xv[r] = x4[i];
+                    gv[r] = g4[i];
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if (i0 + r * 64 >= n4) continue;
+                    part[r] = fmaf(xv[r].x, gv[r].x, part[r]);
+                    part[r] = fmaf(xv[r].y, gv[r].y, part[r]);
+                    part[r] = fmaf(xv[r].z, gv[r].z, part[r]);
+                    part[r] = fmaf(xv[r].w, gv[r].w, part[r]);
+                }
+            }
+            dot = (part[0] + part[1]) + (part[2] + part[3]);
+        } else {
+            for (uint32_t i = lane; i < hidden; i += 64) dot = fmaf(xr[i], shared_gate[i], dot);
+        }
+    }
     int32_t id;
     float w;
     route_one_token<kPerLane>(logits + static_cast<size_t>(t) * num_experts, num_experts, top_k, lane, s_ev, id, w);
     if (lane < top_k) {
-        ids[t * top_k + lane] = id;
-        weights[t * top_k + lane] = w;
+        ids[t * out_stride + lane] = id;
+        weights[t * out_stride + lane] = w;
+    }
+    if (shared_gate != nullptr) {
+        dot = wave_sum(dot);
+        if (lane == 0) {
+            ids[t * out_stride + top_k] = static_cast<int32_t>(num_experts);
+            weights[t * out_stride + top_k] = 1.0f / (1.0f + expf(-dot));
+        }
     }
 }
 
@@ -228,6 +271,9 @@ __global__ __launch_bounds__(kMoeWaves * 64) void moe_down_kernel(
 }
 
 // y[t, c] = sum over slots, in slot order, of weights[t, s] * o[t*top_k + s, c].
+// R slots at a time: their routing entries, then their rows, are loaded together (the launcher picks R so that
+// the usual slot counts are one round without padding: a padded slot is a row load for nothing).
+template <int R>
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ o,
                                                           const int32_t* __restrict__ ids,
                                                           const float* __restrict__ weights,
@@ -237,11 +283,10 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
     const uint32_t c = blockIdx.x * 256 + threadIdx.x;
     if (c >= hidden) return;
     float acc = 0.0f;
-    // eight slots at a time: their routing entries, then their rows, are loaded together
-    for (uint32_t s0 = 0; s0 < top_k; s0 += 8) {
-        float wv[8], ov[8];
+    for (uint32_t s0 = 0; s0 < top_k; s0 += R) {
+        float wv[R], ov[R];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < R; ++i) {
             const uint32_t s = s0 + i < top_k ? s0 + i : top_k - 1;
             const int32_t e = ids[t * top_k + s];
             const bool ok = s0 + i < top_k && e >= 0 && e < static_cast<int32_t>(num_experts);
@@ -250,54 +295,82 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
             if (!ok) ov[i] = 0.0f;  // rows of invalid slots are never written
         }
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc += wv[i] * ov[i];
+        for (int i = 0; i < R; ++i) acc += wv[i] * ov[i];
     }
     y[static_cast<size_t>(t) * hidden + c] = acc;
+}
+
+template <int R>
+void launch_combine_r(const float* o, const int32_t* ids, const float* weights, uint32_t experts, uint32_t slots,
+                      uint32_t hidden, uint32_t tokens, float* y, hipStream_t stream) {
+    hipLaunchKernelGGL(moe_combine_kernel<R>, dim3((hidden + 255) / 256, tokens), dim3(256), 0, stream, o, ids, weights,
+                       experts, slots, hidden, y);
+}
+
+void launch_combine(const float* o, const int32_t* ids, const float* weights, uint32_t experts, uint32_t slots,
+                    uint32_t hidden, uint32_t tokens, float* y, hipStream_t stream) {
+    // (adding a padded product of zeros changes no bit of the sum, so R is free to choose)
+    if (slots <= 2) launch_combine_r<2>(o, ids, weights, experts, slots, hidden, tokens, y, stream);
+    else if (slots <= 4) launch_combine_r<4>(o, ids, weights, experts, slots, hidden, tokens, y, stream);
+    else if (slots == 9) launch_combine_r<9>(o, ids, weights, experts, slots, hidden, tokens, y, stream);
+    else if (slots > 8 && slots <= 12) launch_combine_r<12>(o, ids, weights, experts, slots, hidden, tokens, y, stream);
+    else if (slots == 17) launch_combine_r<17>(o, ids, weights, experts, slots, hidden, tokens, y, stream);
+    else launch_combine_r<8>(o, ids, weights, experts, slots, hidden, tokens, y, stream);
 }
 
 }  // namespace
 
 void launch_moe_route(const float* logits, uint32_t tokens, uint32_t num_experts, uint32_t top_k,
-                      int32_t* ids, float* weights, hipStream_t stream) {
+                      int32_t* ids, float* weights, hipStream_t stream, const float* x, const float* shared_gate,
+                      uint32_t hidden) {
+    const uint32_t out_stride = shared_gate ? top_k + 1 : top_k;
     if (num_experts <= 256)
         hipLaunchKernelGGL(moe_route_kernel<4>, dim3(tokens), dim3(64), 0, stream, logits, tokens, num_experts, top_k,
-                           ids, weights);
+                           ids, weights, out_stride, x, shared_gate, hidden);
     else
         hipLaunchKernelGGL(moe_route_kernel<kMaxExperts / 64>, dim3(tokens), dim3(64), 0, stream, logits, tokens,
-                           num_experts, top_k, ids, weights);
+                           num_experts, top_k, ids, weights, out_stride, x, shared_gate, hidden);
 }
 
 void launch_moe_grouped(const uint8_t* gate_up, const uint8_t* down, uint32_t num_experts,
                         uint32_t inter, uint32_t hidden, const float* x, uint32_t tokens,
                         const int32_t* ids, const float* weights, uint32_t top_k, float* y,
-                        const MoeScratch& s, hipStream_t stream) {
-    const uint32_t pairs = tokens * top_k;
+                        const MoeScratch& s, hipStream_t stream, const uint8_t* shared_gate_up,
+                        const uint8_t* shared_down) {
+    // A shared expert rides along as expert `num_experts` in slot `top_k` of every token (the routing table then
+    // has top_k + 1 slots per token): every kernel below simply sees one more expert and one more slot.
+    const bool shared = shared_gate_up != nullptr;
+    const uint32_t experts = num_experts + (shared ? 1 : 0), slots = top_k + (shared ? 1 : 0);
+    const uint32_t pairs = tokens * slots;
     // matrix-core kernels whenever one pass's activations fit in LDS; the plain kernels otherwise
-    const size_t lds_cap = 150 * 1024;
-    const bool mfma_up = moe_mfma_lds_bytes(hidden) <= lds_cap, mfma_down = moe_mfma_lds_bytes(inter) <= lds_cap;
+    const bool mfma_up = moe_mfma_serves(hidden), mfma_down = moe_mfma_serves(inter);
     // With few pairs every expert workgroup finds its own pairs in the routing table (one load and a
     // ballot): no grouping launch and no offsets -> order -> row chain of dependent loads.
-    const bool scan = mfma_up && mfma_down && pairs <= 1024;
+    // (every workgroup pays the scan: from about 300 pairs on the grouping launch is cheaper; whole layer at 48 /
+    // 64 / 96 / 128 tokens of top-8 with the limit at 1024 pairs 109.7 / 132.8 / 195.7 / 273.9 us, at 320 pairs
+    // 102.6 / 121.8 / 167.8 / 205.6)
+    const bool scan = mfma_up && mfma_down && pairs <= 320;
     const int32_t* scan_ids = scan ? ids : nullptr;
     if (!scan)
-        hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(256), 0, stream, ids, pairs, num_experts, s.counts,
+        hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(256), 0, stream, ids, pairs, experts, s.counts,
                            s.offsets, s.order);
     if (mfma_up)
-        launch_moe_gate_up_mfma(gate_up, num_experts, inter, hidden, x, tokens, top_k, s.offsets, s.order, scan_ids,
-                                s.h, stream);
+        launch_moe_gate_up_mfma(gate_up, experts, inter, hidden, x, tokens, slots, s.offsets, s.order, scan_ids,
+                                s.h, stream, shared_gate_up);
     else
         hipLaunchKernelGGL(moe_gate_up_kernel, dim3((inter + kMoeWaves - 1) / kMoeWaves, num_experts),
                            dim3(kMoeWaves * 64), 0, stream, gate_up, inter, hidden, x, top_k, s.offsets,
                            s.order, s.h);
     if (mfma_down)
-        launch_moe_down_mfma(down, num_experts, inter, hidden, s.h, tokens, top_k, s.offsets, s.order, scan_ids, s.o,
-                             stream);
+        launch_moe_down_mfma(down, experts, inter, hidden, s.h, tokens, slots, s.offsets, s.order, scan_ids, s.o,
+                             stream, shared_down);
     else
         hipLaunchKernelGGL(moe_down_kernel, dim3((hidden + 2 * kMoeWaves - 1) / (2 * kMoeWaves), num_experts),
                            dim3(kMoeWaves * 64), 0, stream, down, inter, hidden, s.h, s.offsets, s.order,
                            s.o);
-    hipLaunchKernelGGL(moe_combine_kernel, dim3((hidden + 255) / 256, tokens), dim3(256), 0, stream,
-                       s.o, ids, weights, num_experts, top_k, hidden, y);
+    launch_combine(s.o, ids, weights, experts, slots, hidden, tokens, y, stream);
 }
+
+bool moe_mfma_serves(uint32_t k) { return moe_mfma_lds_bytes(k) <= 150 * 1024; }
 
 }  // namespace lq4

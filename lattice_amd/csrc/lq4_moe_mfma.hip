@@ -65,6 +65,7 @@ struct MoeGemvArgs {
     uint32_t x_stride;         // floats between activation rows
     uint32_t x_div;            // activation row of a pair = pair / x_div (top_k for x, 1 for h)
     uint32_t tp_per_wave;      // tile pairs (2 x 4 weight rows) per wave
+    const uint8_t* w_last;     // not null: the last expert of the grid lives here, not behind the others in w
 };
 
 // KS: slices of K per workgroup (waves splitting the 16-block steps of a row).
@@ -72,7 +73,20 @@ template <bool GATE_UP, int KS>
 __global__ __launch_bounds__(kThreads) void moe_expert_mfma(MoeGemvArgs p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     constexpr int RS = 4 / KS;
-    const uint32_t e = blockIdx.y;
+    // (expert, pass) of this workgroup.  An expert with tensors of its own (w_last) is one that every token
+    // chose: all its passes are full-length work, so they are dispatched first instead of forming the tail
+    // of the launch (the grid is walked x, then y, then z).
+    uint32_t e = blockIdx.y, pass = blockIdx.z;
+    if (p.w_last != nullptr) {
+        const uint32_t lin = blockIdx.z * gridDim.y + blockIdx.y;
+        if (lin < gridDim.z) {
+            e = gridDim.y - 1;
+            pass = lin;
+        } else {
+            pass = (lin - gridDim.z) / (gridDim.y - 1);
+            e = (lin - gridDim.z) - pass * (gridDim.y - 1);
+        }
+    }
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -81,7 +95,7 @@ __global__ __launch_bounds__(kThreads) void moe_expert_mfma(MoeGemvArgs p) {
     int nt;  // pairs in this pass
     if (p.ids) {
         // Every workgroup scans the routing table itself: rank of a matching pair = matches before it.
-        const int first = static_cast<int>(blockIdx.z) * kTok;
+        const int first = static_cast<int>(pass) * kTok;
         int base = 0;
         for (uint32_t c0 = 0; c0 < p.n_pairs; c0 += kThreads) {
             const uint32_t pi = c0 + tid;
@@ -99,7 +113,7 @@ __global__ __launch_bounds__(kThreads) void moe_expert_mfma(MoeGemvArgs p) {
         if (base <= first) return;
         nt = base - first < kTok ? base - first : kTok;
     } else {
-        const int32_t beg = p.offsets[e] + static_cast<int32_t>(blockIdx.z) * kTok;
+        const int32_t beg = p.offsets[e] + static_cast<int32_t>(pass) * kTok;
         const int32_t end = p.offsets[e + 1];
         if (beg >= end) return;
         nt = end - beg < kTok ? end - beg : kTok;
@@ -122,8 +136,10 @@ __global__ __launch_bounds__(kThreads) void moe_expert_mfma(MoeGemvArgs p) {
     uint4* const zero_region = xs16 + nb * kPitch16;  // 64 B of zeros
     float* const red = reinterpret_cast<float*>(zero_region + 4);  // [4 waves][tp][2][kCols][4]
 
-    const uint32_t* wbase = reinterpret_cast<const uint32_t*>(p.w) +
-                            static_cast<size_t>(e) * p.rows_per_expert * (nb * 5);
+    const uint32_t* wbase = (p.w_last != nullptr && e == gridDim.y - 1)
+                                ? reinterpret_cast<const uint32_t*>(p.w_last)
+                                : reinterpret_cast<const uint32_t*>(p.w) +
+                                      static_cast<size_t>(e) * p.rows_per_expert * (nb * 5);
 
     auto load_unit = [&](Q4BlockRaw (&buf)[2], uint32_t u) {
         const uint32_t t = n_local ? u / n_local : 0, q = u - t * n_local;
@@ -385,15 +401,18 @@ size_t moe_mfma_lds_bytes(uint32_t k) {
 
 void launch_moe_gate_up_mfma(const uint8_t* gate_up, uint32_t num_experts, uint32_t inter, uint32_t hidden,
                              const float* x, uint32_t tokens, uint32_t top_k, const int32_t* offsets,
-                             const int32_t* order, const int32_t* ids, float* h, hipStream_t stream) {
-    MoeGemvArgs a{gate_up, x, h, offsets, order, ids, tokens * top_k, 2 * inter, inter, hidden, hidden, top_k, 0};
+                             const int32_t* order, const int32_t* ids, float* h, hipStream_t stream,
+                             const uint8_t* last_expert) {
+    MoeGemvArgs a{gate_up, x, h, offsets, order, ids, tokens * top_k, 2 * inter, inter, hidden, hidden, top_k, 0,
+                  last_expert};
     launch_phase<true>(a, num_experts, tokens, stream);
 }
 
 void launch_moe_down_mfma(const uint8_t* down, uint32_t num_experts, uint32_t inter, uint32_t hidden,
                           const float* h, uint32_t tokens, uint32_t top_k, const int32_t* offsets,
-                          const int32_t* order, const int32_t* ids, float* o, hipStream_t stream) {
-    MoeGemvArgs a{down, h, o, offsets, order, ids, tokens * top_k, hidden, hidden, inter, inter, 1, 0};
+                          const int32_t* order, const int32_t* ids, float* o, hipStream_t stream,
+                          const uint8_t* last_expert) {
+    MoeGemvArgs a{down, h, o, offsets, order, ids, tokens * top_k, hidden, hidden, inter, inter, 1, 0, last_expert};
     launch_phase<false>(a, num_experts, tokens, stream);
 }
 

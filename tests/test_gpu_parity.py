@@ -595,10 +595,14 @@ def test_moe_ffn_one_call_equals_the_three_calls(be, tokens):
                                  dict(e=64, inter=512, hidden=2048, tokens=8, top_k=8),
                                  dict(e=6, inter=96, hidden=160, tokens=3, top_k=3),
                                  dict(e=8, inter=1024, hidden=512, tokens=2, top_k=7),      # 8 slots x 1024: four slabs
-                                 dict(e=8, inter=1024, hidden=512, tokens=2, top_k=8)])     # 9 x 1024 > 8192: three calls inside
+                                 dict(e=8, inter=1024, hidden=512, tokens=2, top_k=8),      # 9 x 1024 > 8192: three calls inside
+                                 dict(e=64, inter=512, hidden=2048, tokens=16, top_k=8),    # config 4: the grouped kernels
+                                 dict(e=6, inter=96, hidden=160, tokens=13, top_k=3),       # ragged last pass of every expert
+                                 dict(e=12, inter=64, hidden=96, tokens=48, top_k=7)])      # 384 pairs: grouping launch
 def test_moe_ffn_with_the_shared_expert_as_a_slot(be, cfg):
-    """A shared expert as wide as the routed ones rides along in the per-pair kernels for up to 8 tokens:
-    the whole layer against the oracle (routed f64 + shared f64) and against the three separate calls."""
+    """A shared expert as wide as the routed ones rides along: as one more slot of the per-pair kernels for up to
+    8 tokens, as one more expert of the grouped kernels above that.  The whole layer against the oracle (routed
+    f64 + shared f64) and against the three separate calls."""
     import torch
     e_, inter, hidden, tokens, top_k = cfg["e"], cfg["inter"], cfg["hidden"], cfg["tokens"], cfg["top_k"]
     print(f"moe ffn, shared expert as a slot {cfg}", flush=True)
@@ -621,7 +625,7 @@ def test_moe_ffn_with_the_shared_expert_as_a_slot(be, cfg):
     # the shared part alone, so that an error in it (or in its gate) cannot hide behind the routed sum
     d_err = rel_err(host(y) - routed64, want - routed64)
     print(f"  rel err {err:.2e}, shared part alone {d_err:.2e}", flush=True)
-    as_slot = (top_k + 1) * inter <= 8192
+    as_slot = 8 < tokens <= 56 or (top_k + 1) * inter <= 8192  # (above 56 tokens: the shared expert's own GEMMs)
     assert err <= (5e-5 if as_slot else REL_TOL) and d_err <= (2e-4 if as_slot else 2 * REL_TOL)
     # gate||up and down once for the layer when the shared expert rode along; otherwise once for the routed
     # experts and once more for the shared expert alone (the same kernels with it as their only slot); no dense
@@ -634,6 +638,26 @@ def test_moe_ffn_with_the_shared_expert_as_a_slot(be, cfg):
     be.moe_experts(qgu, qdn, e_, inter, hidden, dev(x), d_ids, d_wts, y3)
     be.moe_shared_expert(qsgu, qsdn, dev(sg), inter, hidden, dev(x), y3)
     assert rel_err(host(y), host(y3)) <= REL_TOL
+    # a captured call replayed on new inputs (routing tables and the shared expert's weight live in library
+    # scratch) gives the bits of an eager call on them
+    dx, dlg, dsg = dev(x), dev(lg), dev(sg)
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            be.moe_ffn(dlg, qgu, qdn, e_, top_k, inter, qsgu, qsdn, dsg, inter, hidden, dx, y)
+    for seed in (7, 8):
+        x2 = dev(synth.activations(tokens, hidden, seed=seed, tag="moe_x"))
+        lg2 = dev(synth.router_logits(tokens, e_, seed=seed))
+        be.moe_ffn(lg2, qgu, qdn, e_, top_k, inter, qsgu, qsdn, dsg, inter, hidden, x2, y3)  # eager work between replays
+        dx.copy_(x2)
+        dlg.copy_(lg2)
+        y.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(host(y).view(np.uint32), host(y3).view(np.uint32)), seed
 
 
 def test_moe_shared_expert_argument_checks(be):

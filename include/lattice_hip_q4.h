@@ -116,10 +116,11 @@ int lq4_lora_apply(lq4_ctx* ctx, const lq4_lora* lora, float lora_scale, const v
  * dispatch_gemm_at, dispatch.rs:935-980).
  * At batch 1 with a LoRA adapter the launch computes A . x itself and keeps a few words of
  * hand-over state in the context: such calls must not overlap on two streams of one context.
- * Activation range: at batch 1 any finite f32 value (activations are staged as f16 pairs scaled by a
- * power of two per 32-element block, so the result tracks an f32 GEMV as the reference's
- * gemv_q4_decode does, shaders/qwen35.metal:794-866); at batch 2..16 activations are split into
- * unscaled f16 pairs and |x| >= 65504 becomes infinity. */
+ * Activation range: at batch 1 any finite f32 value (activations are staged as 23-bit fixed point
+ * scaled by a power of two per 32-element block and multiplied exactly, so the result tracks an f32
+ * GEMV as the reference's gemv_q4_decode does, shaders/qwen35.metal:794-866; an infinite or NaN
+ * activation makes every output NaN); at batch 2..16 activations are split into unscaled f16 pairs
+ * and |x| >= 65504 becomes infinity. */
 int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
              const float* x_dev, uint32_t batch, float* y_dev, const lq4_lora* lora,
              float lora_scale, void* stream);

@@ -1,20 +1,22 @@
-// Device helpers shared by the batch-1 GEMV kernel and the decode-chain kernel: how a lane reads a
-// 20-byte block, how activations are staged in LDS, and the per-block dot product.
+// Device helpers shared by the batch-1 GEMV kernel, the decode-chain kernel and the per-pair MoE kernels: how a
+// lane reads a 20-byte block, how activations are staged in LDS, and the per-block dot product.
 //
-// Arithmetic.  A naive unpack (shift, mask, int->float, fma per nibble) would make vector issue,
-// not HBM, the limit on this chip.  Instead a masked dword IS a pair of f16 subnormals:
-// q & 0x000F000F = (n_lo, n_hi) * 2^-24 and q & 0x00F000F0 = (n_lo, n_hi) * 2^-20 (gfx950's
-// v_dot2_f32_f16 honours f16 subnormals), so one v_and per two weights unpacks them exactly, and
-// v_dot2_f32_f16 does two MACs per op with f32 accumulation.  The activations paired with the
-// 2^-20 form are pre-scaled by 2^-4.
+// Arithmetic.  A naive unpack (shift, mask, int->float, fma per nibble) would make vector issue, not HBM, the
+// limit on this chip, and so does any form that touches the nibbles one or two at a time.  Here a packed dword
+// is never unpacked: v_dot8_u32_u4 multiplies the eight nibbles of a weight dword with eight 4-bit digits of
+// the activations and adds the products, exactly, in one full-rate instruction.
 //
-// Activations keep f32 accuracy and f32 range: the 32 activations of a block are divided by
-// 2^e, the power of two of the block's largest magnitude, and each quotient is split x = hi + lo/2048
-// with hi, lo both f16.  Every product is exact, the result tracks an f32 GEMV (not an f16 one), and
-// any finite f32 activation is representable (the reference's one-token kernel reads f32 x,
-// shaders/qwen35.metal:800-847).  Per block
-//   y += 2^e * (d * 2^24) * sum_k (n_k 2^-24) (x_k / 2^e)  +  b * sum_k x_k,
-// the bias-factored form of the reference kernel (shaders/qwen35.metal:838-847).
+// Activations keep f32 accuracy and f32 range: the 32 activations of a block are scaled by the power of two
+// above the block's largest magnitude and rounded to 23-bit fixed point, t = rint(x * 2^22 / S), |t| <= 2^22
+// (an absolute error of 2^-23 S per activation: the accuracy of an f32 at the block's largest magnitude), and
+// x' = t + 2^22 >= 0 is cut into six 4-bit digits.  With A_p = sum_k n_k digit_p(x'_k) (four dot8 per digit)
+// and Q = sum_k n_k (four more),
+//   sum_k n_k t_k = sum_p 16^p A_p - 2^22 Q,
+// an integer below 2^31 computed without rounding, then converted once.  Per block
+//   y += d * (S 2^-22) * sum_k n_k t_k  +  b * sum_k x_k,
+// the bias-factored form of the reference kernel (shaders/qwen35.metal:838-847), whose one-token kernel reads
+// f32 activations (shaders/qwen35.metal:800-847).  28 dot instructions per block and lane, against 20 masks and
+// 32 two-wide dot products for the f16 hi/lo form this replaces.
 #pragma once
 
 #include "lq4_internal.hpp"
@@ -43,18 +45,20 @@ __device__ __forceinline__ LQ4_GLOBAL T* as_global(T* p) {
     return (LQ4_GLOBAL T*)p;
 }
 
-constexpr int kXPitch = 36;  // dwords of LDS per block of x: 16 hi pairs, 16 lo pairs, sum, 2^e, 2 pad
-                             // (36 keeps 16-byte lane reads at stride 144 B conflict-free)
-constexpr float kLoScale = 2048.0f;
-constexpr float kTwo24 = 16777216.0f;
+constexpr int kXPitch = 36;  // dwords of LDS per block of x: 24 digit dwords (dword-column j of digit p at 6j + p),
+                             // 8 unused, sum, S * 2^-22, 2 pad (36 keeps 16-byte lane reads at stride 144 B
+                             // conflict-free)
+constexpr int kDigits = 6;
+constexpr float kRoundMagic = 12582912.0f;        // 1.5 * 2^23: x + magic has rint(x) + 2^22 in its low bits
+constexpr uint32_t kRoundMagicBits = 0x4B000000u;  // bits of 2^23
 
 struct __attribute__((packed, aligned(4))) Q4BlockRaw {
     uint32_t sb;    // f16 scale | f16 bias << 16
     uint32_t q[4];  // 32 nibbles, nibble i of dword j = weight 8j + i
 };
 
-__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
-    return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, a), __builtin_bit_cast(half2v, b), c, false);
+__device__ __forceinline__ uint32_t udot8(uint32_t a, uint32_t b, uint32_t c) {
+    return __builtin_amdgcn_udot8(a, b, c, false);
 }
 
 template <int CTRL, int ROW_MASK>
@@ -90,27 +94,31 @@ __device__ __forceinline__ float segment_sum(float v) {
     return v;
 }
 
-__device__ __forceinline__ uint32_t pack_h2(_Float16 a, _Float16 b) {
-    const half2v h = {a, b};
-    return __builtin_bit_cast(uint32_t, h);
+// Bytes b of four fixed-point values, one per byte: pair() interleaves the low two bytes of two values
+// ([a.B0, b.B0, a.B1, b.B1]) or takes their third byte ([a.B2, b.B2, 0, 0]); quad() joins two such pairs.
+__device__ __forceinline__ uint32_t perm(uint32_t high, uint32_t low, uint32_t sel) {
+    return __builtin_amdgcn_perm(high, low, sel);
 }
 
-// Converts 8 consecutive activations (the partners of one packed dword), already divided by the
-// block's power of two, into the pair order the unpack produces — (0,4) (1,5) (2,6) (3,7) — as f16 hi
-// parts and scaled f16 residuals.  Odd elements pair with the 2^-20 nibble form and are split
-// after scaling by 2^-4.
-__device__ __forceinline__ void convert_x8(const float (&v)[8], uint4& ph, uint4& pl) {
-    _Float16 hi[8], lo[8];
+// Cuts 8 consecutive fixed-point activations x'[i] (24 bits each, the partners of one packed dword: nibble i of
+// the dword is weight i) into the six digit dwords: nibble i of out[p] = digit p of x'[i].
+__device__ __forceinline__ void digits_x8(const uint32_t (&xf)[8], uint32_t (&out)[kDigits]) {
+    uint32_t byte_plane[2][3];  // [even / odd elements][byte]: the bytes of elements (0,2,4,6) or (1,3,5,7)
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const float s = (i & 1) ? v[i] * 0.0625f : v[i];
-        hi[i] = static_cast<_Float16>(s);
-        lo[i] = static_cast<_Float16>((s - static_cast<float>(hi[i])) * kLoScale);
+    for (int o = 0; o < 2; ++o) {
+        const uint32_t u0 = perm(xf[2 + o], xf[0 + o], 0x05010400u), u1 = perm(xf[6 + o], xf[4 + o], 0x05010400u);
+        const uint32_t v0 = perm(xf[2 + o], xf[0 + o], 0x0c0c0602u), v1 = perm(xf[6 + o], xf[4 + o], 0x0c0c0602u);
+        byte_plane[o][0] = perm(u1, u0, 0x05040100u);
+        byte_plane[o][1] = perm(u1, u0, 0x07060302u);
+        byte_plane[o][2] = perm(v1, v0, 0x05040100u);
     }
-    ph.x = pack_h2(hi[0], hi[4]); ph.y = pack_h2(hi[1], hi[5]);
-    ph.z = pack_h2(hi[2], hi[6]); ph.w = pack_h2(hi[3], hi[7]);
-    pl.x = pack_h2(lo[0], lo[4]); pl.y = pack_h2(lo[1], lo[5]);
-    pl.z = pack_h2(lo[2], lo[6]); pl.w = pack_h2(lo[3], lo[7]);
+    constexpr uint32_t kLow = 0x0F0F0F0Fu;
+#pragma unroll
+    for (int b = 0; b < 3; ++b) {
+        const uint32_t ev = byte_plane[0][b], od = byte_plane[1][b];
+        out[2 * b] = (ev & kLow) | ((od << 4) & ~kLow);
+        out[2 * b + 1] = ((ev >> 4) & kLow) | (od & ~kLow);
+    }
 }
 
 // Stages unit g = (block g >> 2, dword g & 3) of the activation vector: 8 activations in a, b.  The
@@ -118,7 +126,7 @@ __device__ __forceinline__ void convert_x8(const float (&v)[8], uint4& ph, uint4
 // (`store` = false for the clamped duplicates past the end of the vector).
 __device__ __forceinline__ void stage_x8(lds_u32* xs, uint32_t g, const float4 a, const float4 b, bool store) {
     const uint32_t blk = g >> 2, j = g & 3;
-    float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
     float sx = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
     float m = fmaxf(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))),
                     fmaxf(fmaxf(fabsf(v[4]), fabsf(v[5])), fmaxf(fabsf(v[6]), fabsf(v[7]))));
@@ -127,70 +135,71 @@ __device__ __forceinline__ void stage_x8(lds_u32* xs, uint32_t g, const float4 a
     sx = dpp_add<0x4E, 0xF>(sx);
     m = dpp_max_quad<0xB1>(m);
     m = dpp_max_quad<0x4E>(m);
-    // 2^e = the power of two at or below the block's largest magnitude (1 for an all-zero or
-    // subnormal block); its reciprocal is exact
+    // S = 2^(e - 126), the power of two above the block's largest magnitude (e its biased exponent; blocks below
+    // 2^-103 share that scale, so S * 2^-22 stays a normal number).  to_fixed = 2^22 / S and S * 2^-22 are exact.
     uint32_t e = __builtin_bit_cast(uint32_t, m) >> 23;
-    e = e == 0 ? 127u : e > 253u ? 253u : e;
-    const float scale = __builtin_bit_cast(float, e << 23);
-    const float inv = __builtin_bit_cast(float, (254u - e) << 23);
+    e = e < 23u ? 23u : e > 254u ? 254u : e;
+    const float to_fixed = __builtin_bit_cast(float, (275u - e) << 23);
+    float scale = __builtin_bit_cast(float, (e - 21u) << 23);
+    // an infinite or NaN activation (or a sum that overflows) reaches every row, as it does in f32 arithmetic
+    if (!(fabsf(sx) <= 3.402823466e38f)) scale = __builtin_nanf("");
+    uint32_t xf[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] *= inv;
-    uint4 ph, pl;
-    convert_x8(v, ph, pl);
+    for (int i = 0; i < 8; ++i)  // rint(v * to_fixed) + 2^22, rounded to nearest even by the addition itself
+        xf[i] = __builtin_bit_cast(uint32_t, fmaf(v[i], to_fixed, kRoundMagic)) - kRoundMagicBits;
+    uint32_t dg[kDigits];
+    digits_x8(xf, dg);
     if (store) {
-        *reinterpret_cast<LQ4_LDS u32x4*>(&xs[blk * kXPitch + 4 * j]) = u32x4{ph.x, ph.y, ph.z, ph.w};
-        *reinterpret_cast<LQ4_LDS u32x4*>(&xs[blk * kXPitch + 16 + 4 * j]) = u32x4{pl.x, pl.y, pl.z, pl.w};
+        typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+        LQ4_LDS u32x2* dst = reinterpret_cast<LQ4_LDS u32x2*>(&xs[blk * kXPitch + kDigits * j]);
+        dst[0] = u32x2{dg[0], dg[1]};
+        dst[1] = u32x2{dg[2], dg[3]};
+        dst[2] = u32x2{dg[4], dg[5]};
         if (j == 0) *reinterpret_cast<LQ4_LDS f32x2*>(&xs[blk * kXPitch + 32]) = f32x2{sx, scale};
     }
 }
 
 // The staged activations of one block, in a lane's registers.
 struct XBlock {
-    uint32_t h[16], l[16];
-    float sum, scale;
+    uint32_t n[4 * kDigits];  // digit p of dword-column j at kDigits * j + p
+    float sum, scale;         // sum of the block's activations; S * 2^-22
 };
 
 __device__ __forceinline__ void load_xblock(const lds_u32* xs, uint32_t blk, XBlock& x) {
     const LQ4_LDS u32x4* xsrc = reinterpret_cast<const LQ4_LDS u32x4*>(&xs[blk * kXPitch]);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const u32x4 h = xsrc[i], l = xsrc[4 + i];
-        x.h[4 * i + 0] = h.x; x.h[4 * i + 1] = h.y; x.h[4 * i + 2] = h.z; x.h[4 * i + 3] = h.w;
-        x.l[4 * i + 0] = l.x; x.l[4 * i + 1] = l.y; x.l[4 * i + 2] = l.z; x.l[4 * i + 3] = l.w;
+    for (int i = 0; i < kDigits; ++i) {
+        const u32x4 d = xsrc[i];
+        x.n[4 * i + 0] = d.x; x.n[4 * i + 1] = d.y; x.n[4 * i + 2] = d.z; x.n[4 * i + 3] = d.w;
     }
     const f32x2 ss = *reinterpret_cast<const LQ4_LDS f32x2*>(&xs[blk * kXPitch + 32]);
     x.sum = ss.x;
     x.scale = ss.y;
 }
 
-// 2^-24 * sum_k n_k * x_k over one block (x as staged: divided by the block's power of two).
-__device__ __forceinline__ float block_dot(const uint32_t (&q)[4], const uint32_t (&xh)[16],
-                                           const uint32_t (&xl)[16]) {
-    float ph = 0.0f, pl = 0.0f;
+// sum_k n_k * t_k over one block, t the block's fixed-point activations (exact).
+__device__ __forceinline__ float block_dot(const uint32_t (&q)[4], const uint32_t (&xn)[4 * kDigits]) {
+    uint32_t part[kDigits], nib = 0;
+#pragma unroll
+    for (int p = 0; p < kDigits; ++p) part[p] = 0;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const uint32_t w0 = q[j] & 0x000F000Fu;
-        const uint32_t w1 = q[j] & 0x00F000F0u;
-        const uint32_t q8 = q[j] >> 8;
-        const uint32_t w2 = q8 & 0x000F000Fu;
-        const uint32_t w3 = q8 & 0x00F000F0u;
-        ph = dot2(w0, xh[4 * j + 0], ph);
-        pl = dot2(w0, xl[4 * j + 0], pl);
-        ph = dot2(w1, xh[4 * j + 1], ph);
-        pl = dot2(w1, xl[4 * j + 1], pl);
-        ph = dot2(w2, xh[4 * j + 2], ph);
-        pl = dot2(w2, xl[4 * j + 2], pl);
-        ph = dot2(w3, xh[4 * j + 3], ph);
-        pl = dot2(w3, xl[4 * j + 3], pl);
+#pragma unroll
+        for (int p = 0; p < kDigits; ++p) part[p] = udot8(q[j], xn[kDigits * j + p], part[p]);
+        nib = udot8(q[j], 0x11111111u, nib);
     }
-    return fmaf(pl, 1.0f / kLoScale, ph);
+    // sum_p 16^p part[p] <= 480 * 2^23 < 2^32; minus 2^22 * nib it is below 2^31 in magnitude
+    const uint32_t lo = part[0] + (part[1] << 4) + (part[2] << 8);
+    const uint32_t hi = part[3] + (part[4] << 4) + (part[5] << 8);
+    const uint32_t total = lo + (hi << 12) - (nib << 22);
+    return static_cast<float>(static_cast<int32_t>(total));
 }
 
 // acc + (one block of one weight row) . (the staged block x); `live` = false drops the block
 // (a lane past the end of the row that re-read a valid block).
 __device__ __forceinline__ float block_fma(const Q4BlockRaw& w, const XBlock& x, bool live, float acc) {
-    const float p = block_dot(w.q, x.h, x.l);
-    float d = f16_bits_to_f32(w.sb & 0xffffu) * kTwo24;
+    const float p = block_dot(w.q, x.n);
+    float d = f16_bits_to_f32(w.sb & 0xffffu);
     const float b = f16_bits_to_f32(w.sb >> 16);
     if (!live) d = 0.0f;
     return fmaf(d * p, x.scale, fmaf(b, live ? x.sum : 0.0f, acc));

@@ -9,8 +9,9 @@
 // Waves are persistent: each walks a strided list of row groups and keeps the next
 // group's blocks in flight while it works on the current one.
 //
-// The unpack-free arithmetic (masked nibbles as f16 subnormals, activations as per-block scaled
-// hi/lo f16 pairs) and the LDS staging are in lq4_b1_dev.hpp, shared with the decode-chain kernel.
+// The unpack-free arithmetic (eight-wide 4-bit dot products of a packed dword with the digits of per-block
+// scaled fixed-point activations) and the LDS staging are in lq4_b1_dev.hpp, shared with the decode-chain
+// kernel and the per-pair MoE kernels.
 #include "lq4_b1_dev.hpp"
 #include "lq4_topk_dev.hpp"
 

@@ -1,6 +1,6 @@
 // Routed experts for a few tokens (decode): every (token, slot) pair is served as a one-token GEMV in
-// the arithmetic of the batch-1 kernel (lq4_b1_dev.hpp: dot2 on masked nibbles, f16 hi/lo activations
-// scaled per block), two launches for the whole step:
+// the arithmetic of the batch-1 kernel (lq4_b1_dev.hpp: 4-bit dot products on packed dwords, fixed-point
+// activations scaled per block), two launches for the whole step:
 //   1. gate||up: for token t the selected experts' [2I, H] matrices are one virtual matrix of
 //      top_k * 2I rows over x[t]; row v belongs to slot v / 2I and reads expert ids[t, slot]'s row.
 //   2. down: y[t] = sum_s w_s * W_down[e_s] . (silu(g_s) * u_s) is ONE GEMV over a K of top_k * I:

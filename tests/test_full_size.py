@@ -184,7 +184,7 @@ def test_moe_scalar_kernels_for_reductions_beyond_lds(be, cfg):
 @pytest.mark.parametrize("magnitude", [1e5, 3e38 / 2048, 1e-7, 1e-30])
 def test_gemv_batch1_takes_any_finite_f32_activation(be, magnitude):
     # the reference's one-token kernel reads f32 activations (shaders/qwen35.metal:800-847); here they
-    # are staged as f16 pairs scaled by a power of two per block, so their range is f32's
+    # are staged as fixed point scaled by a power of two per block, so their range is f32's
     import torch
     n, k = 96, 2048
     rng = np.random.default_rng(11)

@@ -29,8 +29,8 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense f16
 
 # rocprofv3 counters on this workload (profiles/gemv_q4_b1_decode_layer_traffic.md): per layer step
-# FETCH_SIZE 15110.0 KiB x 2.000 (copy-kernel scale) + WRITE_SIZE 144 KiB x 1.000, over 4 launches
-MEASURED_TRAFFIC_PER_LAUNCH = (15110.0 * 2.0 + 144.0) * 1024 / 4
+# FETCH_SIZE 15122.0 KiB x 2.000 (copy-kernel scale) + WRITE_SIZE 144 KiB x 1.000, over 4 launches
+MEASURED_TRAFFIC_PER_LAUNCH = (15122.0 * 2.0 + 144.0) * 1024 / 4
 
 LAYER = [("qkv", 3072, 2048), ("o", 2048, 2048), ("gate_up", 12288, 2048), ("down", 2048, 6144)]
 

@@ -202,3 +202,18 @@ def test_gemv_batch1_takes_any_finite_f32_activation(be, magnitude):
     e = rel_err(got, ref)
     print(f"  |x| ~ {magnitude:g}: rel err vs f64 {e:.2e}", flush=True)
     assert e <= 2e-5
+
+
+@pytest.mark.parametrize("bad", [float("nan"), float("inf"), -float("inf")])
+def test_gemv_batch1_non_finite_activation_reaches_every_row(be, bad):
+    # every row has a weight against every activation, so in f32 arithmetic a NaN or infinite activation
+    # leaves no finite output; the fixed-point staging must not turn it into a finite garbage value
+    import torch
+    n, k = 70, 2048
+    wq = synth.q4_weight(n, k, seed=12, symmetric_bias=False)
+    x = np.random.default_rng(12).normal(size=(1, k)).astype(np.float32)
+    x[0, 777] = bad
+    qw = be.upload_q4_blocks(wq)
+    y = torch.zeros((1, n), dtype=torch.float32, device="cuda")
+    be.gemv_batch(dev(x), qw, y, 1, n, k)
+    assert not np.any(np.isfinite(host(y)))

@@ -5,14 +5,16 @@
 //
 // Same work layout as the Q4 kernel: lane l owns block 64 s + l of every row its wave
 // processes, so a wave reads 2176 contiguous bytes per row and slab (blocks are only 2-byte
-// aligned; the vector memory path takes unaligned 16-byte loads).  The activations stay f32:
-// they are staged once per workgroup in LDS (36 dwords per block: 32 values, their sum, pad)
-// and a lane's 32 values serve all rows of a chunk.  Bytes are converted with the unsigned
-// byte-to-float instruction after flipping the sign bits (q ^ 0x80 = q + 128), and the offset
-// is taken out per block with the staged sum:  sum q x = sum (q + 128) x - 128 sum x.
+// aligned; the vector memory path takes unaligned 16-byte loads).
+// Arithmetic: the weight bytes are never converted.  The 32 activations of a block are staged once per
+// workgroup as 23-bit fixed point, t = rint(x * 2^22 / S) with S the power of two above the block's largest
+// magnitude (the accuracy of an f32 at that magnitude, the range of f32), cut into three signed bytes
+// t = b0 + 256 b1 + 65536 b2, and v_dot4_i32_i8 multiplies four weight bytes with four activation bytes and
+// adds the products exactly: 24 dot instructions per block and row instead of 32 conversions and 32 FMAs.
+// The three integer sums (each below 2^19) are joined in f32.
 // Waves are persistent over chunks of RW rows; the next unit's blocks are in flight while the
 // current one is consumed.
-#include "lq4_internal.hpp"
+#include "lq4_b1_dev.hpp"
 
 #include <type_traits>
 
@@ -21,7 +23,9 @@ namespace lq4 {
 namespace {
 
 constexpr int kWaves = 4;
-constexpr int kXPitch = 36;  // dwords of LDS per block of x (16-byte lane reads at stride 144 B are conflict-free)
+constexpr int kXPitch = 36;  // dwords of LDS per block of x: byte plane p of weight dword w at 3 w + p (24 dwords),
+                             // S * 2^-22 at 33 (16-byte lane reads at stride 144 B are conflict-free)
+constexpr int kPlanes = 3;
 constexpr int kQ8BlockBytes = 34;
 
 struct __attribute__((packed, aligned(2))) Q8BlockRaw {
@@ -46,18 +50,15 @@ __device__ __forceinline__ float wave_total(float v) {
     return v;
 }
 
-// sum_i (q_i + 128) * x_i over one block
-__device__ __forceinline__ float block_dot(const uint32_t (&q)[8], const float (&xv)[32]) {
-    float s0 = 0.0f, s1 = 0.0f;
+// sum_i q_i * t_i over one block, t the block's fixed-point activations
+__device__ __forceinline__ float block_dot(const uint32_t (&q)[8], const uint32_t (&xn)[8 * kPlanes]) {
+    int32_t part[kPlanes] = {0, 0, 0};
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const uint32_t u = q[j] ^ 0x80808080u;
-        s0 = fmaf(static_cast<float>(u & 0xffu), xv[4 * j + 0], s0);
-        s1 = fmaf(static_cast<float>((u >> 8) & 0xffu), xv[4 * j + 1], s1);
-        s0 = fmaf(static_cast<float>((u >> 16) & 0xffu), xv[4 * j + 2], s0);
-        s1 = fmaf(static_cast<float>(u >> 24), xv[4 * j + 3], s1);
-    }
-    return s0 + s1;
+    for (int w = 0; w < 8; ++w)
+#pragma unroll
+        for (int p = 0; p < kPlanes; ++p)
+            part[p] = __builtin_amdgcn_sdot4(static_cast<int32_t>(q[w]), static_cast<int32_t>(xn[kPlanes * w + p]), part[p], false);
+    return fmaf(static_cast<float>(part[2]), 65536.0f, fmaf(static_cast<float>(part[1]), 256.0f, static_cast<float>(part[0])));
 }
 
 // Chunk c of wave `wid` holds rows (c * RW + j) * n_waves + wid, j < RW; a unit is one
@@ -66,7 +67,7 @@ __device__ __forceinline__ float block_dot(const uint32_t (&q)[8], const float (
 template <int RW, int HX>
 __global__ __launch_bounds__(kWaves * 64) void gemv_q8_b1(const uint8_t* __restrict__ w, uint32_t n, uint32_t k,
                                                           const float* __restrict__ x, float* __restrict__ y) {
-    extern __shared__ __attribute__((aligned(16))) float xs[];
+    extern __shared__ __attribute__((aligned(16))) uint32_t xs[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const uint32_t nb = k / kBlockWeights;
@@ -93,14 +94,50 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q8_b1(const uint8_t* __restr
     // ---- stage x: thread g handles 8 activations of block g / 4 -----------------------------
     auto stage = [&](uint32_t g, const float4 a, const float4 b, bool store) {
         const uint32_t blk = g >> 2, j = g & 3;
-        float sx = ((a.x + a.y) + (a.z + a.w)) + ((b.x + b.y) + (b.z + b.w));
-        sx = dpp_add<0xB1>(sx);  // the 4 threads of a block are 4 adjacent lanes: quad butterfly
+        const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        float sx = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+        float m = fmaxf(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))),
+                        fmaxf(fmaxf(fabsf(v[4]), fabsf(v[5])), fmaxf(fabsf(v[6]), fabsf(v[7]))));
+        sx = dpp_add<0xB1>(sx);  // the 4 threads of a block are 4 adjacent lanes: quad butterflies
         sx = dpp_add<0x4E>(sx);
+        m = b1::dpp_max_quad<0xB1>(m);
+        m = b1::dpp_max_quad<0x4E>(m);
+        // S = 2^(e - 126), the power of two above the block's largest magnitude (blocks below 2^-103 share that
+        // scale, so S * 2^-22 stays a normal number); 2^22 / S and S * 2^-22 are exact
+        uint32_t e = __builtin_bit_cast(uint32_t, m) >> 23;
+        e = e < 23u ? 23u : e > 254u ? 254u : e;
+        const float to_fixed = __builtin_bit_cast(float, (275u - e) << 23);
+        float scale = __builtin_bit_cast(float, (e - 21u) << 23);
+        // an infinite or NaN activation (or a sum that overflows) reaches every row, as it does in f32 arithmetic
+        if (!(fabsf(sx) <= 3.402823466e38f)) scale = __builtin_nanf("");
+        // t = rint(v * to_fixed), rounded to nearest even by the addition of 1.5 * 2^23 itself; its balanced
+        // signed bytes are the low bytes of t, (t + 128) >> 8 and ((t + 128) >> 8) + 128 >> 8
+        uint32_t digit[kPlanes][8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int32_t t0 = static_cast<int32_t>(__builtin_bit_cast(uint32_t, fmaf(v[i], to_fixed, 12582912.0f)) - 0x4B400000u);
+            const int32_t t1 = (t0 + 128) >> 8;
+            const int32_t t2 = (t1 + 128) >> 8;
+            digit[0][i] = static_cast<uint32_t>(t0);
+            digit[1][i] = static_cast<uint32_t>(t1);
+            digit[2][i] = static_cast<uint32_t>(t2);
+        }
+        uint32_t out[2 * kPlanes];  // [weight dword 2j, 2j + 1][plane]
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int p = 0; p < kPlanes; ++p) {
+                const uint32_t lo = b1::perm(digit[p][4 * h + 1], digit[p][4 * h + 0], 0x0c0c0400u);
+                const uint32_t hi = b1::perm(digit[p][4 * h + 3], digit[p][4 * h + 2], 0x0c0c0400u);
+                out[kPlanes * h + p] = b1::perm(hi, lo, 0x05040100u);
+            }
         if (store) {
-            float4* dst = reinterpret_cast<float4*>(&xs[blk * kXPitch + 8 * j]);
-            dst[0] = a;
-            dst[1] = b;
-            if (j == 0) xs[blk * kXPitch + 32] = sx;
+            typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+            u32x2* dst = reinterpret_cast<u32x2*>(&xs[blk * kXPitch + 2 * kPlanes * j]);
+            dst[0] = u32x2{out[0], out[1]};
+            dst[1] = u32x2{out[2], out[3]};
+            dst[2] = u32x2{out[4], out[5]};
+            if (j == 0) xs[blk * kXPitch + 33] = __builtin_bit_cast(uint32_t, scale);
         }
     };
 
@@ -142,19 +179,19 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q8_b1(const uint8_t* __restr
         const uint32_t blk_raw = slab * 64 + lane;
         const bool live = blk_raw < nb;
         const uint32_t blk = live ? blk_raw : nb - 1;
-        float xv[32];
-        const float4* xsrc = reinterpret_cast<const float4*>(&xs[blk * kXPitch]);
+        uint32_t xn[8 * kPlanes];
+        const uint4* xsrc = reinterpret_cast<const uint4*>(&xs[blk * kXPitch]);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const float4 v = xsrc[i];
-            xv[4 * i + 0] = v.x; xv[4 * i + 1] = v.y; xv[4 * i + 2] = v.z; xv[4 * i + 3] = v.w;
+        for (int i = 0; i < 2 * kPlanes; ++i) {
+            const uint4 v = xsrc[i];
+            xn[4 * i + 0] = v.x; xn[4 * i + 1] = v.y; xn[4 * i + 2] = v.z; xn[4 * i + 3] = v.w;
         }
-        const float sum_x = xs[blk * kXPitch + 32];
+        const float scale_x = __builtin_bit_cast(float, xs[blk * kXPitch + 33]);
 #pragma unroll
         for (int j = 0; j < RW; ++j) {
-            const float p = block_dot(cur[j].q, xv) - 128.0f * sum_x;
+            const float p = block_dot(cur[j].q, xn);
             const float d = live ? f16_bits_to_f32(cur[j].d) : 0.0f;
-            acc[j] = fmaf(d, p, acc[j]);
+            acc[j] = fmaf(d * p, scale_x, acc[j]);
         }
         if (slab + 1 == slabs) {  // chunk complete
 #pragma unroll

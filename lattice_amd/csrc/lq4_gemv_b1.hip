@@ -27,7 +27,8 @@ constexpr int kWaves = 4;  // waves per workgroup unless a launch asks for more
 
 // A wave-row is 64/SEG weight rows side by side (SEG lanes each).  Wave `wid` of `n_waves`
 // works through chunks of RW wave-rows — chunk c holds wave-rows (c*RW + j)*n_waves + wid,
-// j < RW — and, inside a chunk, through groups of SG slabs.  One (chunk, slab group) is a
+// j < RW (with several chunks per wave: (c*n_waves + wid)*RW + j) — and, inside a chunk, through
+// groups of SG slabs.  One (chunk, slab group) is a
 // unit: RW*SG blocks per lane, loaded with one burst; the next unit's burst is in flight
 // while the current one is consumed.  Dynamic LDS: (K/32) * kXPitch dwords.
 //
@@ -128,13 +129,14 @@ struct FusionArg<3> {
 // it (release), the weight workgroups behind them pick t up (acquire) when their first rows are
 // complete, long after it was published.  The wait is bounded: a wave that runs out of polls
 // computes t itself, so every wave finishes whatever the dispatch order was.
+// 4 plain, with the row order of a persistent grid (see ADJ below).
 // 3 the lm_head pass with the exact top-k selection in the same launch (shaders/qwen35.metal:1935-1985
 // computes block candidates inside the GEMV kernel too): the logits go to `y` with device-scope stores,
 // every wave keeps the best key among the rows it produced, the workgroup publishes the best of its
 // waves and draws a ticket, and the workgroup that draws the last one (every logit and every maximum
 // is then in memory) runs the selection tail over those maxima.  A workgroup's rows are its selection
 // block; in this mode they are consecutive (every wave takes a run of wave-rows).
-constexpr int kPlainMode = 0, kFusedMode = 1, kLoraAMode = 2, kTopkMode = 3;
+constexpr int kPlainMode = 0, kFusedMode = 1, kLoraAMode = 2, kTopkMode = 3, kPlainAdjMode = 4;
 
 template <int RW, int SG, int SEG, int MODE, int WAVES = kWaves>
 __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restrict__ w, uint32_t n,
@@ -190,6 +192,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
     // chunks whose first wave-row exists for this wave (later waves may have one chunk fewer)
     const uint32_t first = wid < n_wrows ? n_wrows - wid : 0;  // wave-rows from this wave's first one on
     uint32_t chunks = (first + n_waves * RW - 1) / (n_waves * RW);
+    // kPlainAdjMode, for a persistent grid (waves that walk several chunks): the RW wave-rows of a chunk lie next
+    // to each other in memory, chunk c of wave wid = wave-rows (c * n_waves + wid) * RW + j, so the wave's requests
+    // of one unit fall into one run of RW rows (lm_head 63.4 -> 60.6 us in the same run on one device).  With one
+    // chunk per wave the interleaved order is the faster one (12288 x 2048 5.25 against 5.46 us, 2048 x 6144 3.8
+    // against 4.1), and the choice as a run-time flag cost those launches 6-11 %: hence a mode of its own.
+    constexpr bool ADJ = MODE == kPlainAdjMode;
+    if constexpr (ADJ) chunks = wid * RW < n_wrows ? (n_wrows - wid * RW + n_waves * RW - 1) / (n_waves * RW) : 0;
     // kTopkMode: a wave takes `per_wave` consecutive wave-rows instead, so that the logits of one
     // workgroup are one run in memory (the workgroup that selects reads the best workgroups' logits:
     // scattered over the vector they are a cache line each)
@@ -200,7 +209,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
         chunks = (mine + RW - 1) / RW;
     }
     // wave-row of round r = chunk * RW + j, and whether this wave owns it
-    auto wrow_of = [&](uint32_t r) { return MODE == kTopkMode ? wid * per_wave + r : r * n_waves + wid; };
+    auto wrow_of = [&](uint32_t r) {
+        if (MODE == kTopkMode) return wid * per_wave + r;
+        return ADJ ? (r / RW) * (n_waves * RW) + wid * RW + r % RW : r * n_waves + wid;
+    };
     auto wrow_mine = [&](uint32_t r) { return wrow_of(r) < n_wrows && (MODE != kTopkMode || r < per_wave); };
     const uint32_t units = chunks * slab_groups;
 
@@ -289,7 +301,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
         if constexpr (!INA) lora_t0 = lora.t[seg_lane];
 #pragma unroll
         for (int j = 0; j < RW; ++j) {
-            const uint32_t wrow = j * n_waves + wid;
+            const uint32_t wrow = wrow_of(j);
             uint32_t row = wrow * RPW + sub;
             row = (wrow < n_wrows && row < n) ? row : n - 1;
             const size_t bi = static_cast<size_t>(row) * lora.rank + seg_lane;
@@ -311,7 +323,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
     if constexpr (FUSED) {
 #pragma unroll
         for (int j = 0; j < RW; ++j) {
-            const uint32_t wrow = j * n_waves + wid;
+            const uint32_t wrow = wrow_of(j);
             const uint32_t row = wrow * RPW + sub;
             res_first[j] = (fz.epilogue == GemvFusion::kAddResidual && wrow < n_wrows && row < n) ? fz.residual[row] : 0.0f;
         }
@@ -587,8 +599,8 @@ void launch_cfg_topk(const uint8_t* w, uint32_t n, uint32_t k, const float* x, f
 
 template <int RW, int SG, int SEG, int WAVES = kWaves>
 void launch_cfg(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, const LoraEpilogue& lora,
-                const GemvFusion* fusion, size_t lds, uint32_t waves, hipStream_t stream) {
-    static bool attr_set[3] = {false, false, false};  // raise the dynamic-LDS cap once per instantiation
+                const GemvFusion* fusion, size_t lds, uint32_t waves, bool persistent, hipStream_t stream) {
+    static bool attr_set[4] = {false, false, false, false};  // raise the dynamic-LDS cap once per instantiation
     const dim3 grid((waves + WAVES - 1) / WAVES), block(WAVES * 64);
     if (fusion) {
         if (!attr_set[1]) {
@@ -610,6 +622,18 @@ void launch_cfg(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float*
         hipLaunchKernelGGL((gemv_q4_b1<RW, SG, SEG, kLoraAMode, WAVES>), grid_a, block, lds, stream, w, n, k, x, y,
                            lora, NoFusion{});
         return;
+    }
+    if constexpr (RW > 1) {  // (one row per chunk: both row orders are the same)
+        if (persistent) {
+            if (!attr_set[3]) {
+                (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, kPlainAdjMode, WAVES>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                attr_set[3] = true;
+            }
+            hipLaunchKernelGGL((gemv_q4_b1<RW, SG, SEG, kPlainAdjMode, WAVES>), grid, block, lds, stream, w, n, k, x, y,
+                               lora, NoFusion{});
+            return;
+        }
     }
     if (!attr_set[0]) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, kPlainMode, WAVES>),
@@ -643,6 +667,7 @@ namespace {
 struct B1Plan {
     size_t lds;
     uint32_t seg, wg_waves, waves, rw, sg;
+    bool persistent;  // waves walk several chunks
 };
 
 // `producers`: workgroups in front of the weight workgroups.  `four_waves`: never the eight-wave
@@ -669,6 +694,7 @@ B1Plan plan_b1(uint32_t n, uint32_t k, uint32_t producers, bool four_waves, size
     const uint32_t max_waves = (256 * wg_per_cu - producers) * wg_waves;
     uint32_t rw = (n_wrows + max_waves - 1) / max_waves;
     uint32_t waves;
+    p.persistent = rw > 4;
     if (rw <= 4) {
         // every wave resident, one chunk each
         waves = (n_wrows + rw - 1) / rw;
@@ -702,8 +728,8 @@ void launch_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* 
     const size_t lds = pl.lds;
     const uint32_t seg = pl.seg, wg_waves = pl.wg_waves, waves = pl.waves, rw = pl.rw, sg = pl.sg;
 
-#define LQ4_B1(RW_, SG_, SEG_) launch_cfg<RW_, SG_, SEG_>(w, n, k, x, y, lora, fusion, lds, waves, stream)
-#define LQ4_B1W(RW_, SG_) launch_cfg<RW_, SG_, 64, 8>(w, n, k, x, y, lora, fusion, lds, waves, stream)
+#define LQ4_B1(RW_, SG_, SEG_) launch_cfg<RW_, SG_, SEG_>(w, n, k, x, y, lora, fusion, lds, waves, pl.persistent, stream)
+#define LQ4_B1W(RW_, SG_) launch_cfg<RW_, SG_, 64, 8>(w, n, k, x, y, lora, fusion, lds, waves, pl.persistent, stream)
     if (seg == 32) {
         if (rw == 1) LQ4_B1(1, 1, 32); else if (rw == 2) LQ4_B1(2, 1, 32); else if (rw == 3) LQ4_B1(3, 1, 32); else LQ4_B1(4, 1, 32);
     } else if (seg == 16) {

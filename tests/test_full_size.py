@@ -217,3 +217,23 @@ def test_gemv_batch1_non_finite_activation_reaches_every_row(be, bad):
     y = torch.zeros((1, n), dtype=torch.float32, device="cuda")
     be.gemv_batch(dev(x), qw, y, 1, n, k)
     assert not np.any(np.isfinite(host(y)))
+
+
+@pytest.mark.parametrize("n,k", [(70001, 2048), (33333, 1024), (40000, 512), (25000, 6144)])
+def test_gemv_batch1_tall_matrix_with_waves_over_several_chunks(be, n, k):
+    # more rows than one chunk per resident wave covers: the grid is persistent, every wave walks several chunks
+    # whose rows lie next to each other in memory, and the last chunk is ragged; rows of 64, 32 and 16 blocks
+    # (one, two and four rows side by side in a wave) and of three slabs
+    import torch
+    print(f"tall gemv n={n} k={k}", flush=True)
+    wq = synth.q4_weight(n, k, seed=13, tag="tall")
+    x = synth.activations(1, k, seed=13, tag="tall")
+    qw = be.upload_q4_blocks(wq)
+    y = torch.full((1, n), float("nan"), dtype=torch.float32, device="cuda")
+    be.gemv_batch(dev(x), qw, y, 1, n, k)
+    ref = oracle.gemm_f64(x, wq, n, k)
+    e = rel_err(host(y), ref)
+    print(f"  rel err vs f64 {e:.2e}", flush=True)
+    assert e <= 2e-5
+    # every row against its own reference (a row written to another row's place would still be "small" above)
+    assert np.max(np.abs(host(y) - ref)) <= 1e-4 * np.max(np.abs(ref))

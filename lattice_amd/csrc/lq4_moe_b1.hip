@@ -2,10 +2,11 @@
 // the arithmetic of the batch-1 kernel (lq4_b1_dev.hpp: 4-bit dot products on packed dwords, fixed-point
 // activations scaled per block), two launches for the whole step:
 //   1. gate||up: for token t the selected experts' [2I, H] matrices are one virtual matrix of
-//      top_k * 2I rows over x[t]; row v belongs to slot v / 2I and reads expert ids[t, slot]'s row.
-//   2. down: y[t] = sum_s w_s * W_down[e_s] . (silu(g_s) * u_s) is ONE GEMV over a K of top_k * I:
-//      block b of a row belongs to slot b / (I/32) and is read from that expert's matrix; the
-//      activations silu(g) * u * w_s are formed while they are staged.  The weighted sum over the
+//      top_k * 2I rows over x[t], walked in (gate row, up row) pairs: pair q belongs to slot q / I and
+//      reads rows q % I and I + q % I of expert ids[t, slot].  A wave meets the two rows of a pair one
+//      after the other and writes act[t, q] = silu(g) * u * w_slot, so neither g nor u reaches memory.
+//   2. down: y[t] = sum_s W_down[e_s] . act[t, s] is ONE GEMV over a K of top_k * I: block b of a row
+//      belongs to slot b / (I/32) and is read from that expert's matrix.  The weighted sum over the
 //      slots happens inside the dot product, so there is no combine launch.
 // accumulate_routed_experts (crates/inference/src/model/qwen35/moe.rs:127-190) visits a token's
 // selected experts one after the other; with one token no two pairs share an expert, so nothing is
@@ -29,8 +30,8 @@ using namespace b1;
 
 struct MoeB1Args {
     const uint8_t* w;     // gate||up [E, 2I, H] or down [E, H, I], native blocks
-    const float* x;       // gate||up: x [tokens, H];  down: h [tokens, slots, 2I] (gate | up per pair)
-    float* y;             // gate||up: h;  down: y [tokens, H]
+    const float* x;       // gate||up: x [tokens, H];  down: act [tokens, slots * I]
+    float* y;             // gate||up: act;  down: y [tokens, H]
     const int32_t* ids;   // [tokens, top_k]
     const float* wts;     // [tokens, top_k]
     uint32_t num_experts, top_k, inter, hidden;
@@ -38,7 +39,8 @@ struct MoeB1Args {
     // The always-active shared expert (apply_shared_expert, moe.rs:194-250) as one more slot behind the
     // routed ones, when its intermediate size equals the routed experts': its own tensors (`w_shared`,
     // the gate||up or the down one), and as its weight sigmoid(x . shared_gate), which workgroup 0 of the
-    // gate||up launch computes into shared_wt[token] for the down launch.  slots = top_k (+ 1).
+    // gate||up launch computes into shared_wt[token] for the down launch (which applies it while it stages:
+    // the gate||up launch writes that slot's act without a weight).  slots = top_k (+ 1).
     const uint8_t* w_shared;
     const float* shared_gate;
     float* shared_wt;
@@ -59,8 +61,9 @@ __device__ __forceinline__ float silu_mul(float gate, float u) {
 }
 
 // grid (workgroups per token, tokens), block 256.  Wave `wid` of a token's `n_waves` works through
-// chunks of RW rows, chunk c holding rows (c * RW + j) * n_waves + wid; the next chunk's blocks are in
-// flight while the current one is consumed.  SLABS = ceil(K / 2048): a lane owns block slab * 64 + lane
+// chunks of RW rows; the next chunk's blocks are in flight while the current one is consumed.  Down: row
+// i * n_waves + wid is the wave's i-th.  Gate||up: its i-th row is the gate (i even) or up (i odd) row of
+// pair (i / 2) * n_waves + wid.  SLABS = ceil(K / 2048): a lane owns block slab * 64 + lane
 // of a row.  Dynamic LDS: (K / 32) * kXPitch dwords.
 // ROUTE (gate||up only): the router runs inside the launch (a separate instantiation, so that the plain one
 // carries none of it).
@@ -75,6 +78,7 @@ __global__ __launch_bounds__(256) void moe_b1_kernel(MoeB1Args a) {
     const int32_t* ids = a.ids + static_cast<size_t>(token) * a.top_k;
     const float* wts = a.wts + static_cast<size_t>(token) * a.top_k;
     __shared__ int32_t s_ids[ROUTE ? 16 : 1];
+    __shared__ float s_wts[ROUTE ? 16 : 1];
     auto expert_of = [&](uint32_t slot) {  // the shared expert's tensor holds one expert
         const int32_t e = slot < a.top_k ? (ROUTE ? s_ids[slot] : ids[slot]) : 0;
         return (e >= 0 && static_cast<uint32_t>(e) < a.num_experts) ? static_cast<uint32_t>(e) : 0u;
@@ -85,17 +89,20 @@ __global__ __launch_bounds__(256) void moe_b1_kernel(MoeB1Args a) {
     // shared expert.
     float shared_w = 0.0f;
     if (DOWN && a.shared_wt != nullptr) shared_w = a.shared_wt[token];
+    // Routing weight of a slot (`slot` is the same for the whole wave wherever this is called); a slot with an
+    // id outside [0, E) counts 0.  The shared expert's slot: 1 in the gate||up launch, its weight in the down one.
     auto weight_of = [&](uint32_t slot) {
-        if (slot >= a.top_k) return shared_w;
-        const int32_t e = ids[slot];
-        return (e >= 0 && static_cast<uint32_t>(e) < a.num_experts) ? wts[slot] : 0.0f;
+        if (slot >= a.top_k) return DOWN ? shared_w : 1.0f;
+        const int32_t e = ROUTE ? s_ids[slot] : ids[slot];
+        const float w = ROUTE ? s_wts[slot] : wts[slot];
+        return (e >= 0 && static_cast<uint32_t>(e) < a.num_experts) ? w : 0.0f;
     };
     auto tensor_of = [&](uint32_t slot) { return slot < a.top_k ? a.w : a.w_shared; };
 
     // ---- activations first: their loads are waited for alone, ahead of the weights ----
     constexpr int kUnitsPerThread = 4;  // K <= 8192: 1024 units of 8 activations
     const uint32_t n_units = nb * 4;
-    float4 va[kUnitsPerThread], vb[kUnitsPerThread], ua[kUnitsPerThread], ub[kUnitsPerThread];
+    float4 va[kUnitsPerThread], vb[kUnitsPerThread];
     float wt[kUnitsPerThread];
 #pragma unroll
     for (int i = 0; i < kUnitsPerThread; ++i) {
@@ -107,13 +114,10 @@ __global__ __launch_bounds__(256) void moe_b1_kernel(MoeB1Args a) {
             vb[i] = xp[1];
             wt[i] = 1.0f;
         } else {
-            const uint32_t slot = blk / nbe, kb = blk - slot * nbe;
-            const float* hp = a.x + (static_cast<size_t>(token) * a.slots + slot) * 2 * a.inter + kb * kBlockWeights + dw * 8;
+            const float* hp = a.x + static_cast<size_t>(token) * a.k + blk * kBlockWeights + dw * 8;
             va[i] = reinterpret_cast<const float4*>(hp)[0];
             vb[i] = reinterpret_cast<const float4*>(hp)[1];
-            ua[i] = reinterpret_cast<const float4*>(hp + a.inter)[0];
-            ub[i] = reinterpret_cast<const float4*>(hp + a.inter)[1];
-            wt[i] = weight_of(slot);
+            wt[i] = blk / nbe >= a.top_k ? shared_w : 1.0f;  // the routed slots carry their weight already
         }
     }
 
@@ -127,6 +131,7 @@ __global__ __launch_bounds__(256) void moe_b1_kernel(MoeB1Args a) {
                                    s_ev, id, w);
                 if (lane < a.top_k) {
                     s_ids[lane] = id;
+                    s_wts[lane] = w;
                     if (blockIdx.x == 0) {
                         a.ids_out[static_cast<size_t>(token) * a.top_k + lane] = id;
                         a.wts_out[static_cast<size_t>(token) * a.top_k + lane] = w;
@@ -140,8 +145,9 @@ __global__ __launch_bounds__(256) void moe_b1_kernel(MoeB1Args a) {
     // ---- rows of this wave ----
     const uint32_t n_waves = gridDim.x * 4;
     const uint32_t wid = __builtin_amdgcn_readfirstlane(blockIdx.x * 4 + (tid >> 6));
-    const uint32_t first = wid < a.n ? a.n - wid : 0;
-    const uint32_t chunks = (first + n_waves * RW - 1) / (n_waves * RW);
+    const uint32_t items = DOWN ? a.n : a.n / 2;  // rows, or (gate, up) pairs
+    const uint32_t mine = wid < items ? (items - wid + n_waves - 1) / n_waves : 0;
+    const uint32_t chunks = ((DOWN ? mine : 2 * mine) + RW - 1) / RW;
     // where this lane's block of each slab lives, apart from the row
     uintptr_t lane_base[SLABS];  // DOWN: the slot's tensor and expert and the block; else only the block's offset
     bool live[SLABS];
@@ -161,13 +167,16 @@ __global__ __launch_bounds__(256) void moe_b1_kernel(MoeB1Args a) {
     auto load_chunk = [&](Q4BlockRaw (&buf)[RW][SLABS], uint32_t c) {
 #pragma unroll
         for (int j = 0; j < RW; ++j) {
-            uint32_t row = (c * RW + j) * n_waves + wid;  // scalar
-            if (row >= a.n) row = a.n - 1;
+            const uint32_t i = c * RW + j;  // scalar, like everything derived from it
             uintptr_t row_off;  // the row's part of the address (with the tensor, for gate||up)
             if constexpr (DOWN) {
+                uint32_t row = i * n_waves + wid;
+                if (row >= a.n) row = a.n - 1;
                 row_off = static_cast<size_t>(row) * nbe * kBlockBytes;
             } else {
-                const uint32_t slot = row / (2 * a.inter), r = row - slot * 2 * a.inter;
+                uint32_t q = (i >> 1) * n_waves + wid;
+                if (q >= items) q = items - 1;
+                const uint32_t slot = q / a.inter, r = (i & 1) * a.inter + (q - slot * a.inter);
                 row_off = reinterpret_cast<uintptr_t>(tensor_of(slot)) +
                           (static_cast<size_t>(expert_of(slot)) * 2 * a.inter + r) * nb * kBlockBytes;
             }
@@ -191,10 +200,8 @@ __global__ __launch_bounds__(256) void moe_b1_kernel(MoeB1Args a) {
         const uint32_t g = tid + i * 256;
         float4 p = va[i], q = vb[i];
         if constexpr (DOWN) {
-            p.x = silu_mul(va[i].x, ua[i].x) * wt[i]; p.y = silu_mul(va[i].y, ua[i].y) * wt[i];
-            p.z = silu_mul(va[i].z, ua[i].z) * wt[i]; p.w = silu_mul(va[i].w, ua[i].w) * wt[i];
-            q.x = silu_mul(vb[i].x, ub[i].x) * wt[i]; q.y = silu_mul(vb[i].y, ub[i].y) * wt[i];
-            q.z = silu_mul(vb[i].z, ub[i].z) * wt[i]; q.w = silu_mul(vb[i].w, ub[i].w) * wt[i];
+            p.x *= wt[i]; p.y *= wt[i]; p.z *= wt[i]; p.w *= wt[i];
+            q.x *= wt[i]; q.y *= wt[i]; q.z *= wt[i]; q.w *= wt[i];
         }
         // whole quads call together: a quad's four units are one block, all inside or all outside
         if (i * 256 < n_units) stage_x8(xsl, g < n_units ? g : 0, p, q, g < n_units);
@@ -228,6 +235,7 @@ __global__ __launch_bounds__(256) void moe_b1_kernel(MoeB1Args a) {
 #pragma unroll
     for (int t = 0; t < SLABS; ++t) load_xblock(xsl, live[t] ? t * 64 + lane : nb - 1, xb_[t]);
 
+    float gate_kept = 0.0f;  // gate||up: the gate row's sum until the pair's up row is done
     auto consume = [&](Q4BlockRaw (&cur)[RW][SLABS], uint32_t c) {
 #pragma unroll
         for (int j = 0; j < RW; ++j) {
@@ -235,10 +243,21 @@ __global__ __launch_bounds__(256) void moe_b1_kernel(MoeB1Args a) {
 #pragma unroll
             for (int t = 0; t < SLABS; ++t) acc = block_fma(cur[j][t], xb_[t], live[t], acc);
             acc = segment_sum<64>(acc);
-            const uint32_t row = (c * RW + j) * n_waves + wid;
-            if (lane == 63 && row < a.n) {
-                float* dst = a.y + static_cast<size_t>(token) * a.n + row;
-                *dst = (DOWN && a.accumulate) ? *dst + acc : acc;
+            const uint32_t i = c * RW + j;
+            if constexpr (DOWN) {
+                const uint32_t row = i * n_waves + wid;
+                if (lane == 63 && row < a.n) {
+                    float* dst = a.y + static_cast<size_t>(token) * a.n + row;
+                    *dst = a.accumulate ? *dst + acc : acc;
+                }
+            } else if ((i & 1) == 0) {
+                gate_kept = acc;
+            } else {
+                const uint32_t q = (i >> 1) * n_waves + wid;
+                if (q < items) {  // (the same for the whole wave)
+                    const float w = weight_of(q / a.inter);
+                    if (lane == 63) a.y[static_cast<size_t>(token) * items + q] = silu_mul(gate_kept, acc) * w;
+                }
             }
         }
     };
@@ -259,7 +278,8 @@ void launch_one(const MoeB1Args& a, uint32_t tokens, hipStream_t stream) {
     const uint32_t rw = slabs == 1 ? 4 : slabs <= 3 ? 2 : 1;
     const size_t lds = static_cast<size_t>(nb) * kXPitch * 4;
     // all waves of the step resident at once where the rows allow: 4096 waves over the tokens
-    const uint32_t wave_rows = (a.n + rw - 1) / rw;
+    // (gate||up with one row per chunk: a wave needs two chunks for a pair, so a wave per pair is the most)
+    const uint32_t wave_rows = (!DOWN && rw == 1) ? a.n / 2 : (a.n + rw - 1) / rw;
     uint32_t budget = 4096 / tokens;
     if (budget < 64) budget = 64;
     const uint32_t waves = wave_rows < budget ? wave_rows : budget;
@@ -289,8 +309,8 @@ bool moe_b1_serves(uint32_t inter, uint32_t hidden, uint32_t slots) {
 }
 
 size_t moe_b1_scratch_bytes(uint32_t tokens, uint32_t slots, uint32_t inter) {
-    // h [tokens, slots, 2I], then the shared expert's weight per token
-    return static_cast<size_t>(tokens) * slots * 2 * inter * sizeof(float) + static_cast<size_t>(tokens) * sizeof(float);
+    // act [tokens, slots * I], then the shared expert's weight per token
+    return static_cast<size_t>(tokens) * slots * inter * sizeof(float) + static_cast<size_t>(tokens) * sizeof(float);
 }
 
 void launch_moe_b1(const uint8_t* gate_up, const uint8_t* down, uint32_t num_experts, uint32_t inter, uint32_t hidden,
@@ -299,7 +319,7 @@ void launch_moe_b1(const uint8_t* gate_up, const uint8_t* down, uint32_t num_exp
                    const float* route_logits, int32_t* ids_out, float* wts_out, bool accumulate, hipStream_t stream) {
     const uint32_t slots = shared_gate_up ? top_k + 1 : top_k;
     float* h = scratch;
-    float* shared_wt = shared_gate_up ? scratch + static_cast<size_t>(tokens) * slots * 2 * inter : nullptr;
+    float* shared_wt = shared_gate_up ? scratch + static_cast<size_t>(tokens) * slots * inter : nullptr;
     if (route_logits) {  // the gate||up launch routes; the down launch reads what it stored
         ids = ids_out;
         weights = wts_out;

@@ -479,6 +479,8 @@ def test_moe_layer_routed_plus_shared_expert(be):
                                  dict(e=5, inter=160, hidden=1056, tokens=2, top_k=2),
                                  dict(e=9, inter=2048, hidden=4096, tokens=1, top_k=4),     # four slabs in the down pass
                                  dict(e=16, inter=32, hidden=64, tokens=4, top_k=8),
+                                 dict(e=3, inter=96, hidden=6400, tokens=2, top_k=2),       # four slabs in the gate||up pass: a pair's rows in two chunks
+                                 dict(e=3, inter=256, hidden=8192, tokens=8, top_k=3),      # ... with waves that walk several pairs
                                  dict(e=4, inter=1056, hidden=256, tokens=2, top_k=8)])     # top_k * inter > 8192: grouped kernels
 def test_moe_experts_for_a_few_tokens(be, cfg):
     """Decode-sized steps take the per-pair kernels (one-token GEMV arithmetic, the weighted sum over the
@@ -508,7 +510,7 @@ def test_moe_experts_for_a_few_tokens(be, cfg):
     print(f"  rel err vs f32 {e32:.2e}, vs f64 {e64:.2e}", flush=True)
     assert e32 <= REL_TOL and e64 <= REL_TOL
     if top_k * inter <= 8192:
-        assert e64 <= 2e-5  # f32-faithful: hi/lo f16 activations in both passes
+        assert e64 <= 2e-5  # f32-faithful: fixed-point activations, exact products in both passes
 
 
 @pytest.mark.parametrize("cfg", [dict(e=64, inter=512, hidden=2048, tokens=16, top_k=8),   # config 4

@@ -445,8 +445,16 @@ def main():
                                              norm=(base_v, delta_v, gamma_v, 1e-6, res_v), batch=rows)
                     be.dispatch_matmul_fused(gu_v, bufs["down"], None, hid, inter, silu_mul=True,
                                              add_residual=(res_v, hid_v), batch=rows)
+
+                def mlp_fused_pairs(i):  # one row: silu(gate) * up formed by the first launch
+                    bufs = layers[i % len(layers)]
+                    be.dispatch_matmul_fused(None, bufs["gate_up"], act_v, 2 * inter, hid,
+                                             norm=(base_v, delta_v, gamma_v, 1e-6, res_v), silu_mul_pairs=True)
+                    be.dispatch_matmul_fused(act_v, bufs["down"], None, hid, inter, add_residual=(res_v, hid_v))
                 mlp = {}
-                for nm, f in (("five_launches", mlp_unfused), ("two_fused_launches", mlp_fused)):
+                forms = [("five_launches", mlp_unfused), ("two_fused_launches_silu_in_second", mlp_fused)]
+                forms.append(("two_fused_launches", mlp_fused_pairs) if rows == 1 else ("two_fused_launches", mlp_fused))
+                for nm, f in forms:
                     for i in range(len(layers)):
                         f(i)
                     mlp[nm + "_us"] = round(tm(torch, f, max(72, args.steps // 2)) * 1e3, 3)

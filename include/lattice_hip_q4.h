@@ -273,6 +273,10 @@ int lq4_add_and_copy(lq4_ctx* ctx, const float* src_dev, float* residual_dev, fl
 #define LQ4_EPI_NONE 0        /* y_dev[N] = W . activations (+ LoRA) */
 #define LQ4_EPI_ADD_RESIDUAL 1 /* also residual[N] += that; copy_dst[N] = residual (if not NULL);
                                   y_dev may then be NULL */
+/* LQ4_EPI_SILU_MUL_PAIRS (2, defined with the chain below): W = [N/2 gate rows | N/2 up rows] and
+ * y_dev[N/2] receives silu(W_i . activations) * (W_(N/2+i) . activations), the dispatch_silu_mul_fused
+ * that follows the gate||up GEMV (inner/dispatch.rs:916-930): a wave takes the two rows of a pair, so
+ * the [gate | up] vector never reaches memory.  One row only (lq4_gemv_fused, lq4_gemv_chain). */
 typedef struct lq4_gemv_fusion {
     int prologue;
     const float* base;   /* ADD_RMSNORM: [K] */
@@ -289,7 +293,8 @@ typedef struct lq4_gemv_fusion {
  * and while the result is stored.  Equals the unfused sequence lq4_residual_add_rmsnorm /
  * lq4_silu_mul -> lq4_gemv -> lq4_add_and_copy to f32 rounding (the sum of squares is formed in a
  * different order).  Shapes or options the fused kernel does not take (K too long for LDS, a LoRA
- * adapter together with a prologue) run as exactly that sequence through library scratch. */
+ * adapter together with a prologue, LQ4_EPI_SILU_MUL_PAIRS with K of 512 or 1024 or with an
+ * adapter) run as exactly that sequence through library scratch. */
 int lq4_gemv_fused(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
                    const float* x_dev, float* y_dev, const lq4_gemv_fusion* fusion, const lq4_lora* lora,
                    float lora_scale, void* stream);

@@ -424,13 +424,15 @@ class HipQ4Backend:
                                          self._stream()))
 
     def dispatch_matmul_fused(self, x, qw: Q4WeightBuf, y, n: int, k: int, *, norm=None, silu_mul=False,
-                              add_residual=None, qw_extra_offset: int = 0, layer_idx=None, module=None,
-                              batch: int = 1):
+                              add_residual=None, silu_mul_pairs=False, qw_extra_offset: int = 0, layer_idx=None,
+                              module=None, batch: int = 1):
         """``dispatch_matmul`` for 1..16 activation rows with the neighbouring elementwise dispatches
         folded in.  ``norm=(base, delta, gamma, eps, residual_out)`` replaces a preceding
         ``dispatch_fused_residual_add_norm`` / ``_batch`` (``x`` is then unused); ``silu_mul=True``
         replaces a preceding ``dispatch_silu_mul_fused`` (``x`` holds gate | up, 2k floats per row);
-        ``add_residual=(residual, dst)`` replaces a following ``dispatch_add_and_copy``.  With
+        ``add_residual=(residual, dst)`` replaces a following ``dispatch_add_and_copy``;
+        ``silu_mul_pairs=True`` (one row): the weight is gate rows then up rows and ``y`` receives the
+        ``n / 2`` values ``silu(gate) * up``, i.e. the following ``dispatch_silu_mul_fused`` as well.  With
         ``batch`` rows every per-row tensor is ``[batch, ...]`` and dense."""
         if n == 0:
             return
@@ -448,6 +450,9 @@ class HipQ4Backend:
         if add_residual is not None:
             residual, dst = add_residual
             f.epilogue, f.residual, f.copy_dst = LQ4_EPI_ADD_RESIDUAL, residual.data_ptr(), self._ptr(dst)
+        if silu_mul_pairs:
+            assert add_residual is None, "one epilogue at a time"
+            f.epilogue = LQ4_EPI_SILU_MUL_PAIRS
         lora = self._lora_for(layer_idx, module, n, k)
         _check(self.lib.lq4_gemv_fused_batch(self.ctx, qw.handle, qw_extra_offset, n, k, self._ptr(x), batch,
                                              self._ptr(y), C.byref(f), lora, self._lora_scale, self._stream()))

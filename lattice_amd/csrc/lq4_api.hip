@@ -1057,6 +1057,9 @@ int lq4_gemv_fused(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, u
             return fail(LQ4_E_INVALID, "fusion.residual and copy_dst must be 4-byte aligned");
     } else if (f.epilogue == LQ4_EPI_NONE) {
         if (!y_dev) return fail(LQ4_E_INVALID, "y device pointer is null");
+    } else if (f.epilogue == LQ4_EPI_SILU_MUL_PAIRS) {
+        if (!y_dev) return fail(LQ4_E_INVALID, "y device pointer is null");
+        if (n % 2) return fail(LQ4_E_INVALID, "LQ4_EPI_SILU_MUL_PAIRS needs an even number of rows, got %u", n);
     } else {
         return fail(LQ4_E_INVALID, "unknown fusion.epilogue %d", f.epilogue);
     }
@@ -1067,7 +1070,9 @@ int lq4_gemv_fused(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, u
     hipStream_t s = static_cast<hipStream_t>(stream);
     DeviceGuard g(ctx->device);
 
-    const bool fused_ok = gemv_b1_lds_bytes(k) <= 128 * 1024 && !(ep.rank && f.prologue != LQ4_PRO_NONE);
+    const bool pairs = f.epilogue == LQ4_EPI_SILU_MUL_PAIRS;
+    const bool fused_ok = gemv_b1_lds_bytes(k) <= 128 * 1024 && !(ep.rank && f.prologue != LQ4_PRO_NONE) &&
+                          !(pairs && (ep.rank || !gemv_b1_pairs_served(n, k)));
     if (fused_ok) {
         if (ep.rank) {
             launch_lora_a(lora->a, lora->is_f16, lora->rank, k, x_dev, 0, k, 1, ctx->lora_t, s);
@@ -1093,6 +1098,30 @@ int lq4_gemv_fused(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, u
     const size_t x_off = 0, y_off = (kbytes + 255) / 256 * 256;
     rc = ensure_scratch(ctx, y_off + static_cast<size_t>(n) * sizeof(float), static_cast<hipStream_t>(stream));
     if (rc) return rc;
+    if (pairs) {  // the product [gate | up] in scratch, then silu(gate) * up into y
+        const float* act_p = x_dev;
+        float* xs_p = reinterpret_cast<float*>(ctx->moe_scratch + x_off);
+        if (f.prologue == LQ4_PRO_ADD_RMSNORM) {
+            launch_residual_add_norm(f.base, f.delta, f.gamma, k, 1, f.eps, f.residual_out, xs_p, s);
+            act_p = xs_p;
+            ctx->counters.elementwise++;
+        } else if (f.prologue == LQ4_PRO_SILU_MUL) {
+            launch_silu_mul(x_dev, k, 1, xs_p, k, s);
+            act_p = xs_p;
+            ctx->counters.elementwise++;
+        }
+        if (ep.rank) {
+            launch_lora_a(lora->a, lora->is_f16, lora->rank, k, act_p, 0, k, 1, ctx->lora_t, s);
+            ctx->counters.lora_a++;
+        }
+        float* gu = reinterpret_cast<float*>(ctx->moe_scratch + y_off);
+        launch_gemv(wp, n, k, act_p, k, 1, gu, n, ep, s);
+        ctx->counters.gemv++;
+        launch_silu_mul(gu, n / 2, 1, y_dev, n / 2, s);
+        ctx->counters.elementwise++;
+        LQ4_HIP(hipGetLastError());
+        return LQ4_OK;
+    }
     const float* act = x_dev;
     float* xs = reinterpret_cast<float*>(ctx->moe_scratch + x_off);
     if (f.prologue == LQ4_PRO_ADD_RMSNORM) {
@@ -1468,6 +1497,12 @@ int lq4_gemv_chain(lq4_ctx* ctx, const lq4_chain_step* steps, uint32_t n_steps, 
             f.copy_dst = st.y_dev;
             rc = lq4_gemv_fused(ctx, st.w, st.w_extra_offset, st.n, st.k, x, nullptr, &f, nullptr, 0.0f, stream);
             result = st.residual;
+        } else if (st.epilogue == LQ4_EPI_SILU_MUL_PAIRS && gemv_b1_pairs_served(st.n, st.k) &&
+                   gemv_b1_lds_bytes(st.k) <= 128 * 1024) {
+            // the launch writes silu(gate) * up itself: no [gate | up] vector, no step after it
+            f.epilogue = LQ4_EPI_SILU_MUL_PAIRS;
+            result = st.y_dev ? st.y_dev : spare;
+            rc = lq4_gemv_fused(ctx, st.w, st.w_extra_offset, st.n, st.k, x, result, &f, nullptr, 0.0f, stream);
         } else if (st.epilogue == LQ4_EPI_SILU_MUL_PAIRS) {
             f.epilogue = LQ4_EPI_NONE;
             rc = lq4_gemv_fused(ctx, st.w, st.w_extra_offset, st.n, st.k, x, spare, &f, nullptr, 0.0f, stream);

@@ -120,6 +120,10 @@ template <>
 struct FusionArg<3> {
     typedef TopkEpilogue type;
 };
+template <>
+struct FusionArg<5> {
+    typedef GemvFusion type;
+};
 
 // WAVES: waves per workgroup.  Every workgroup stages the whole activation vector, so on long rows
 // (K of 4096..8192) eight waves share one staging where four would each pay half of it again.
@@ -136,7 +140,7 @@ struct FusionArg<3> {
 // waves and draws a ticket, and the workgroup that draws the last one (every logit and every maximum
 // is then in memory) runs the selection tail over those maxima.  A workgroup's rows are its selection
 // block; in this mode they are consecutive (every wave takes a run of wave-rows).
-constexpr int kPlainMode = 0, kFusedMode = 1, kLoraAMode = 2, kTopkMode = 3, kPlainAdjMode = 4;
+constexpr int kPlainMode = 0, kFusedMode = 1, kLoraAMode = 2, kTopkMode = 3, kPlainAdjMode = 4, kFusedPairsMode = 5;
 
 template <int RW, int SG, int SEG, int MODE, int WAVES = kWaves>
 __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restrict__ w, uint32_t n,
@@ -145,7 +149,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
                                                           typename FusionArg<MODE>::type fz) {
     extern __shared__ __attribute__((aligned(16))) uint32_t xs[];
     lds_u32* const xsl = (lds_u32*)xs;
-    constexpr bool FUSED = MODE == kFusedMode;
+    constexpr bool FUSED = MODE == kFusedMode || MODE == kFusedPairsMode;
+    constexpr bool PAIRS = MODE == kFusedPairsMode;  // fused, with the kSiluMulPairs epilogue (a mode of its own:
+                                                     // as a run-time flag it doubled the time of every fused launch)
     constexpr bool INA = MODE == kLoraAMode;
     constexpr int RPW = 64 / SEG;  // weight rows per wave-row
     const int tid = threadIdx.x;
@@ -208,12 +214,28 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
         const uint32_t mine = begin < n_wrows ? (n_wrows - begin < per_wave ? n_wrows - begin : per_wave) : 0;
         chunks = (mine + RW - 1) / RW;
     }
+    // Fused epilogue kSiluMulPairs (W = [gate rows | up rows], n / 2 of each; rows of 64 lanes, RW even): the
+    // wave's rounds come in pairs, rounds 2i and 2i + 1 are the gate and the up row of pair i * n_waves + wid, so
+    // that the wave itself forms silu(g) * u when the second row of a pair completes.
+    static_assert(!PAIRS || (RW % 2 == 0 && SEG == 64), "pairs: chunks of whole pairs, rows of 64 lanes");
+    const uint32_t n_pairs = n / 2;
+    if constexpr (PAIRS) {
+        const uint32_t mine = wid < n_pairs ? (n_pairs - wid + n_waves - 1) / n_waves : 0;
+        chunks = (2 * mine + RW - 1) / RW;
+    }
     // wave-row of round r = chunk * RW + j, and whether this wave owns it
     auto wrow_of = [&](uint32_t r) {
         if (MODE == kTopkMode) return wid * per_wave + r;
+        if (PAIRS) {
+            const uint32_t pair = (r >> 1) * n_waves + wid;
+            return (r & 1) ? n_pairs + pair : pair;  // (a pair past the end: past n, or an up row; clamped or dropped)
+        }
         return ADJ ? (r / RW) * (n_waves * RW) + wid * RW + r % RW : r * n_waves + wid;
     };
-    auto wrow_mine = [&](uint32_t r) { return wrow_of(r) < n_wrows && (MODE != kTopkMode || r < per_wave); };
+    auto wrow_mine = [&](uint32_t r) {
+        if (PAIRS) return (r >> 1) * n_waves + wid < n_pairs;
+        return wrow_of(r) < n_wrows && (MODE != kTopkMode || r < per_wave);
+    };
     const uint32_t units = chunks * slab_groups;
 
     // ---- the first activations are requested before any weight so they can be waited on alone ----
@@ -446,6 +468,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
 #pragma unroll
     for (int j = 0; j < RW; ++j) acc[j] = 0.0f;
     uint64_t best_key = key_of(sentinel());  // kTopkMode: best of the rows this lane stored
+    float gate_kept = 0.0f;                  // kSiluMulPairs: the gate row's sum until the pair's up row is done
     float t_reg = 0.0f;   // kLoraAMode: t[lane], fetched when the wave's first rows are complete
     bool t_have = false;
 
@@ -515,6 +538,17 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
                     }
                 }
                 v = segment_sum<SEG>(v);
+                if constexpr (PAIRS) {
+                    if (j % 2 == 0) {
+                        gate_kept = v;
+                    } else if (seg_lane == SEG - 1 && row_ok) {
+                        // silu through the hardware exp2 and reciprocal, the form the staging of a
+                        // [gate | up] vector uses
+                        const float e = __builtin_amdgcn_exp2f(gate_kept * -1.44269504088896340736f);
+                        y[row - n_pairs] = gate_kept * __builtin_amdgcn_rcpf(1.0f + e) * v;
+                    }
+                    continue;
+                }
                 if (seg_lane == SEG - 1 && row_ok) {
                     if constexpr (FUSED) {
                         if (y) y[row] = v;
@@ -602,6 +636,19 @@ void launch_cfg(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float*
                 const GemvFusion* fusion, size_t lds, uint32_t waves, bool persistent, hipStream_t stream) {
     static bool attr_set[4] = {false, false, false, false};  // raise the dynamic-LDS cap once per instantiation
     const dim3 grid((waves + WAVES - 1) / WAVES), block(WAVES * 64);
+    if constexpr (RW % 2 == 0 && SEG == 64) {
+        if (fusion && fusion->epilogue == GemvFusion::kSiluMulPairs) {
+            static bool attr_pairs = false;
+            if (!attr_pairs) {
+                (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, kFusedPairsMode, WAVES>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 159 * 1024);
+                attr_pairs = true;
+            }
+            hipLaunchKernelGGL((gemv_q4_b1<RW, SG, SEG, kFusedPairsMode, WAVES>), grid, block, lds, stream, w, n, k, x, y,
+                               lora, *fusion);
+            return;
+        }
+    }
     if (fusion) {
         if (!attr_set[1]) {
             (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, kFusedMode, WAVES>),
@@ -651,6 +698,12 @@ void launch_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* 
 
 size_t gemv_b1_lds_bytes(uint32_t k) { return static_cast<size_t>(k / kBlockWeights) * kXPitch * 4; }
 
+// The kSiluMulPairs epilogue needs rows of 64 lanes (any block count but 16 and 32, which put rows side by side).
+bool gemv_b1_pairs_served(uint32_t n, uint32_t k) {
+    const uint32_t nb = k / kBlockWeights;
+    return n >= 2 && n % 2 == 0 && nb != 16 && nb != 32;
+}
+
 void launch_gemv_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y,
                     const LoraEpilogue& lora, hipStream_t stream) {
     launch_b1(w, n, k, x, y, lora, nullptr, stream);
@@ -671,8 +724,9 @@ struct B1Plan {
 };
 
 // `producers`: workgroups in front of the weight workgroups.  `four_waves`: never the eight-wave
-// workgroups.  `lds_min`: dynamic LDS the launch needs beyond the staged x.
-B1Plan plan_b1(uint32_t n, uint32_t k, uint32_t producers, bool four_waves, size_t lds_min) {
+// workgroups.  `lds_min`: dynamic LDS the launch needs beyond the staged x.  `even_rw`: chunks of two or four
+// wave-rows only (the kSiluMulPairs epilogue).
+B1Plan plan_b1(uint32_t n, uint32_t k, uint32_t producers, bool four_waves, size_t lds_min, bool even_rw = false) {
     B1Plan p;
     p.lds = gemv_b1_lds_bytes(k);
     if (p.lds < lds_min) p.lds = lds_min;
@@ -693,6 +747,7 @@ B1Plan plan_b1(uint32_t n, uint32_t k, uint32_t producers, bool four_waves, size
     // starts after the producers have advanced the epoch.
     const uint32_t max_waves = (256 * wg_per_cu - producers) * wg_waves;
     uint32_t rw = (n_wrows + max_waves - 1) / max_waves;
+    if (even_rw && rw <= 4 && (rw & 1)) ++rw;
     uint32_t waves;
     p.persistent = rw > 4;
     if (rw <= 4) {
@@ -703,8 +758,8 @@ B1Plan plan_b1(uint32_t n, uint32_t k, uint32_t producers, bool four_waves, size
         // walk several chunks.  Waves differ by at most one chunk, so the chunk height is the
         // largest (most loads in flight) that keeps that imbalance under 8 %.
         waves = max_waves;
-        rw = 1;
-        for (uint32_t cand = 4; cand > 1; --cand) {
+        rw = even_rw ? 2 : 1;
+        for (uint32_t cand = 4; cand > 1; cand -= even_rw ? 2 : 1) {
             const uint32_t most = (n_wrows + max_waves * cand - 1) / (max_waves * cand) * cand;  // rows of the busiest wave
             if (static_cast<uint64_t>(most) * max_waves * 100 <= static_cast<uint64_t>(n_wrows) * 108) {
                 rw = cand;
@@ -724,7 +779,8 @@ B1Plan plan_b1(uint32_t n, uint32_t k, uint32_t producers, bool four_waves, size
 
 void launch_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, const LoraEpilogue& lora,
                const GemvFusion* fusion, hipStream_t stream) {
-    const B1Plan pl = plan_b1(n, k, (lora.rank && lora.a && !fusion) ? lora.rank : 0, false, 0);
+    const bool pairs = fusion && fusion->epilogue == GemvFusion::kSiluMulPairs;
+    const B1Plan pl = plan_b1(n, k, (lora.rank && lora.a && !fusion) ? lora.rank : 0, false, 0, pairs);
     const size_t lds = pl.lds;
     const uint32_t seg = pl.seg, wg_waves = pl.wg_waves, waves = pl.waves, rw = pl.rw, sg = pl.sg;
 

@@ -48,7 +48,9 @@ struct LoraEpilogue {
 //     stored only if its pointer is not null.
 struct GemvFusion {
     enum Prologue : int { kPlain = 0, kAddNorm = 1, kSiluMul = 2 };
-    enum Epilogue : int { kStore = 0, kAddResidual = 1 };
+    // kSiluMulPairs: W = [n / 2 gate rows | n / 2 up rows], y[i] = silu(W_i . x) * (W_(n/2 + i) . x), i < n / 2
+    // (the batch-1 kernel at rows of 2048 weights and more, without LoRA; see gemv_b1_pairs_served)
+    enum Epilogue : int { kStore = 0, kAddResidual = 1, kSiluMulPairs = 2 };
     int prologue;
     const float* base;
     const float* delta;
@@ -68,6 +70,7 @@ void launch_gemv(const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint3
 
 // Batch-1 fast path (x staged in LDS as f16 hi/lo pairs); needs gemv_b1_lds_bytes(k) of LDS.
 size_t gemv_b1_lds_bytes(uint32_t k);
+bool gemv_b1_pairs_served(uint32_t n, uint32_t k);
 void launch_gemv_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y,
                     const LoraEpilogue& lora, hipStream_t stream);
 // Same with fused elementwise steps (separate kernel instantiations; the plain ones are untouched).

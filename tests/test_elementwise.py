@@ -200,6 +200,54 @@ def test_fused_decode_mlp_matches_oracle_and_unfused(be, hidden, inter):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("hidden,inter", [(2048, 6144),   # three rows per wave rounded up to four
+                                          (2048, 20000),  # a persistent grid: waves walk several pairs
+                                          (160, 352), (96, 32), (4096, 64), (8192, 96),
+                                          (1024, 512), (512, 96)])  # rows side by side in a wave: the steps one by one
+def test_fused_decode_mlp_with_silu_in_the_first_launch(be, hidden, inter):
+    """norm + gate||up GEMV + silu(gate) * up in one launch (a wave takes the gate and the up row of a pair), then
+    down GEMV + residual add: against the oracle's five steps and against the form that leaves silu * up to
+    the second launch's prologue."""
+    import torch
+    gate_up, down, base, delta, gamma = _mlp_inputs(hidden, inter, 12)
+    eps = 1e-6
+    res_ref, normed_ref = oracle.residual_add_norm(base[None], delta[None], gamma, eps)
+    gu_ref = oracle.gemm_f32(normed_ref, gate_up, 2 * inter, hidden)
+    h_ref = oracle.silu_mul(gu_ref)
+    qgu = be.upload_q4_blocks(gate_up)
+    d_base, d_delta, d_gamma = dev(base), dev(delta), dev(gamma)
+    residual = torch.full((hidden,), float("nan"), device="cuda")
+    act = torch.full((inter + 1,), float("nan"), device="cuda")
+    before = be.path_counters()
+    be.dispatch_matmul_fused(None, qgu, act, 2 * inter, hidden, norm=(d_base, d_delta, d_gamma, eps, residual),
+                             silu_mul_pairs=True)
+    after = be.path_counters()
+    assert np.array_equal(host(residual), res_ref[0])
+    got = host(act)
+    assert np.isnan(got[-1]), "wrote past inter values"
+    e = rel_err(got[:-1], h_ref[0])
+    print(f"fused silu pairs hidden={hidden} inter={inter}: rel err {e:.2e}", flush=True)
+    assert e <= REL_TOL
+    one_launch = hidden // 32 not in (16, 32)
+    assert after["gemv_fused"] - before["gemv_fused"] == (1 if one_launch else 0)
+    assert after["elementwise"] - before["elementwise"] == (0 if one_launch else 2)
+    # the two-step form: [gate | up] out of the first launch, silu * up where the second one stages it
+    gu = torch.empty(2 * inter, device="cuda")
+    be.dispatch_matmul_fused(None, qgu, gu, 2 * inter, hidden, norm=(d_base, d_delta, d_gamma, eps, residual))
+    be.dispatch_silu_mul_fused(gu, inter)
+    assert rel_err(got[:-1], host(gu)[:inter]) <= 2e-6  # same sums; silu through exp2/rcp against expf and a divide
+    if inter % 32 == 0:  # the whole MLP: the second launch is then a plain GEMV with the residual add
+        ffn = torch.full((hidden,), float("nan"), device="cuda")
+        hidden_out = torch.full((hidden,), float("nan"), device="cuda")
+        qd = be.upload_q4_blocks(down)
+        be.dispatch_matmul_fused(act, qd, ffn, hidden, inter, add_residual=(residual, hidden_out))
+        ffn_ref = oracle.gemm_f32(h_ref, down, hidden, inter)
+        final_ref, _ = oracle.add_and_copy(ffn_ref[0], res_ref[0])
+        assert rel_err(host(ffn), ffn_ref[0]) <= REL_TOL
+        assert rel_err(host(hidden_out), final_ref) <= REL_TOL
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("hidden,inter,batch", [(2048, 6144, 8), (2048, 6144, 2), (1024, 512, 5), (160, 352, 3),
                                                 (512, 96, 16), (2048, 1024, 11), (5120, 544, 4),
                                                 (29184, 32, 3)])  # rows too long for LDS: the unfused sequence

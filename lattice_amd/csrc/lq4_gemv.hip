@@ -198,7 +198,7 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
 void launch_gemv(const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint32_t x_stride,
                  uint32_t batch, float* y, uint32_t y_stride, const LoraEpilogue& lora,
                  hipStream_t stream) {
-    // batch 1: the dot2 kernel (one wave streams whole 1280-byte row slabs); batch 2..16: the
+    // batch 1: the 4-bit dot-product kernel (one wave streams whole 1280-byte row slabs); batch 2..16: the
     // matrix-core kernel, 8 activation rows per pass.  Either needs the activations to fit in
     // LDS; the plain row kernel below covers K too large for that.
     if (batch == 1 && gemv_b1_lds_bytes(k) <= 128 * 1024) {

@@ -68,7 +68,7 @@ void launch_gemv(const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint3
                  uint32_t batch, float* y, uint32_t y_stride, const LoraEpilogue& lora,
                  hipStream_t stream);
 
-// Batch-1 fast path (x staged in LDS as f16 hi/lo pairs); needs gemv_b1_lds_bytes(k) of LDS.
+// Batch-1 fast path (x staged in LDS as per-block fixed point, lq4_b1_dev.hpp); needs gemv_b1_lds_bytes(k) of LDS.
 size_t gemv_b1_lds_bytes(uint32_t k);
 bool gemv_b1_pairs_served(uint32_t n, uint32_t k);
 void launch_gemv_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y,

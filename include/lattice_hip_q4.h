@@ -55,6 +55,11 @@ const char* lq4_last_error(void);
 const char* lq4_version(void);
 
 /* ---- context ------------------------------------------------------------------ */
+/* A context owns scratch buffers, the LoRA t = A.x buffer and a few hand-over words that its calls
+ * share.  A call that uses them on another stream than the previous such call first waits for the
+ * device, so calls alternating between streams are serialised instead of racing; this cannot be done
+ * for a stream that is being captured, for graph replays or for calls from several host threads at
+ * once: those need a context each. */
 int lq4_ctx_create(int device_ordinal, lq4_ctx** out);
 int lq4_ctx_destroy(lq4_ctx* ctx);
 /* hipStreamSynchronize(stream); the counterpart of commit()+wait_until_completed()

@@ -39,6 +39,11 @@ struct lq4_ctx {
     uint32_t cu_count;
     uint32_t chain_spin_limit;
     bool chain_unchecked;  // a chain launch was queued since the failure word was last read
+    // The stream of the last call that used the context's shared state (scratch buffers, hand-over words):
+    // a call on another stream first waits for the device, so that calls alternating between streams are
+    // serialised instead of racing on that state.
+    hipStream_t state_stream;
+    bool state_stream_known;
     lq4_path_counters counters;
 };
 
@@ -387,6 +392,7 @@ int lq4_lora_free(lq4_lora* l) {
 }
 
 static int ensure_scratch(lq4_ctx* ctx, size_t bytes, hipStream_t stream);
+static int enter_shared_state(lq4_ctx* ctx, hipStream_t stream);
 
 int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
              const float* x_dev, uint32_t batch, float* y_dev, const lq4_lora* lora, float lora_scale,
@@ -403,6 +409,10 @@ int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
     LoraEpilogue ep;
     rc = resolve_lora(ctx, lora, lora_scale, n, k, batch, &ep);
     if (rc) return rc;
+    if (ep.rank) {  // the A.x buffer (and, for one token, the hand-over words) belong to the context
+        rc = enter_shared_state(ctx, static_cast<hipStream_t>(stream));
+        if (rc) return rc;
+    }
     hipStream_t s = static_cast<hipStream_t>(stream);
     DeviceGuard g(ctx->device);
     if (ep.rank && batch == 1 && ctx->lora_in_kernel && gemv_b1_lds_bytes(k) <= 128 * 1024) {
@@ -445,6 +455,10 @@ int lq4_lora_apply(lq4_ctx* ctx, const lq4_lora* lora, float lora_scale, const v
     if (rows > kLoraTRows) return fail(LQ4_E_UNSUPPORTED, "LoRA call limited to %u rows, got %u", kLoraTRows, rows);
     hipStream_t s = static_cast<hipStream_t>(stream);
     DeviceGuard g(ctx->device);
+    {
+        const int rc = enter_shared_state(ctx, s);
+        if (rc) return rc;
+    }
     launch_lora_a(lora->a, lora->is_f16, lora->rank, lora->d_in, x_dev, x_dtype == LQ4_F16, lora->d_in, rows,
                   ctx->lora_t, s);
     launch_lora_b_accum(lora->b, lora->is_f16, lora->rank, lora->d_out, ctx->lora_t, lora_scale, rows, y_dev,
@@ -454,11 +468,28 @@ int lq4_lora_apply(lq4_ctx* ctx, const lq4_lora* lora, float lora_scale, const v
     return LQ4_OK;
 }
 
+// Called by every entry point that touches the context's shared state, before it launches anything.
+// A stream that is being captured cannot wait for the device: such calls stay the caller's to order.
+static int enter_shared_state(lq4_ctx* ctx, hipStream_t stream) {
+    if (ctx->state_stream_known && ctx->state_stream != stream) {
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &cap) != hipSuccess) (void)hipGetLastError();
+        if (cap == hipStreamCaptureStatusNone) LQ4_HIP(hipDeviceSynchronize());
+    }
+    ctx->state_stream = stream;
+    ctx->state_stream_known = true;
+    return LQ4_OK;
+}
+
 // Grows one of the context's scratch buffers to `bytes`.  The outgrown buffer is kept until the
 // context is destroyed: launches already queued, and launches captured into a graph, carry its
 // address.  Nothing may be allocated while the stream is capturing: the call then fails and names
 // lq4_ctx_reserve_scratch.  Steady-state calls reuse the buffer.
 static int grow_scratch(lq4_ctx* ctx, uint8_t** buf, size_t* have, size_t bytes, hipStream_t stream, bool zero) {
+    {
+        const int rc = enter_shared_state(ctx, stream);
+        if (rc) return rc;
+    }
     if (bytes <= *have) return LQ4_OK;
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &cap) != hipSuccess) (void)hipGetLastError();
@@ -489,7 +520,13 @@ static int ensure_scratch(lq4_ctx* ctx, size_t bytes, hipStream_t stream) {
 int lq4_ctx_reserve_scratch(lq4_ctx* ctx, size_t bytes) {
     if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
     DeviceGuard g(ctx->device);
-    return ensure_scratch(ctx, bytes, nullptr);
+    const hipStream_t was = ctx->state_stream;  // (no launch: the stream of the last one stays)
+    const bool known = ctx->state_stream_known;
+    ctx->state_stream_known = false;
+    const int rc = ensure_scratch(ctx, bytes, nullptr);
+    ctx->state_stream = was;
+    ctx->state_stream_known = known;
+    return rc;
 }
 
 int lq4_gemm(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
@@ -509,6 +546,10 @@ int lq4_gemm(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
     LoraEpilogue ep;
     rc = resolve_lora(ctx, lora, lora_scale, n, k, m, &ep);
     if (rc) return rc;
+    if (ep.rank) {  // the A.x buffer (and, for one token, the hand-over words) belong to the context
+        rc = enter_shared_state(ctx, static_cast<hipStream_t>(stream));
+        if (rc) return rc;
+    }
     hipStream_t s = static_cast<hipStream_t>(stream);
     DeviceGuard g(ctx->device);
     if (ep.rank) {
@@ -1067,6 +1108,10 @@ int lq4_gemv_fused(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, u
     LoraEpilogue ep;
     rc = resolve_lora(ctx, lora, lora_scale, n, k, 1, &ep);
     if (rc) return rc;
+    if (ep.rank) {  // the A.x buffer (and, for one token, the hand-over words) belong to the context
+        rc = enter_shared_state(ctx, static_cast<hipStream_t>(stream));
+        if (rc) return rc;
+    }
     hipStream_t s = static_cast<hipStream_t>(stream);
     DeviceGuard g(ctx->device);
 
@@ -1194,6 +1239,10 @@ int lq4_gemv_fused_batch(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_off
     LoraEpilogue ep;
     rc = resolve_lora(ctx, lora, lora_scale, n, k, batch, &ep);
     if (rc) return rc;
+    if (ep.rank) {  // the A.x buffer (and, for one token, the hand-over words) belong to the context
+        rc = enter_shared_state(ctx, static_cast<hipStream_t>(stream));
+        if (rc) return rc;
+    }
     hipStream_t s = static_cast<hipStream_t>(stream);
     DeviceGuard g(ctx->device);
 

@@ -678,6 +678,37 @@ def test_moe_shared_expert_argument_checks(be):
     assert np.all(host(y) == 5.0)
 
 
+def test_calls_alternating_between_two_streams_do_not_race_on_the_context(be):
+    """Routing tables, hidden rows and top-k candidates live in scratch the context owns: a call on another
+    stream than the last one first waits for the device, so two streams that take turns get the results of
+    calls made one after the other."""
+    import torch
+    e_, inter, hidden, top_k, tokens = 16, 128, 512, 4, 12
+    gu = be.upload_q4_blocks(synth.q4_weight(e_ * 2 * inter, hidden, seed=21, tag="moe_gu"))
+    dn = be.upload_q4_blocks(synth.q4_weight(e_ * hidden, inter, seed=21, tag="moe_dn"))
+    sgu = be.upload_q4_blocks(synth.q4_weight(2 * inter, hidden, seed=21, tag="sh_gu"))
+    sdn = be.upload_q4_blocks(synth.q4_weight(hidden, inter, seed=21, tag="sh_dn"))
+    sg = dev((np.random.default_rng(21).normal(size=hidden) * 0.1).astype(np.float32))
+    xs = [dev(synth.activations(tokens, hidden, seed=30 + i, tag="moe_x")) for i in range(2)]
+    lgs = [dev(synth.router_logits(tokens, e_, seed=30 + i)) for i in range(2)]
+    want = []
+    for i in range(2):
+        y = torch.empty((tokens, hidden), dtype=torch.float32, device="cuda")
+        be.moe_ffn(lgs[i], gu, dn, e_, top_k, inter, sgu, sdn, sg, inter, hidden, xs[i], y)
+        want.append(host(y))
+    assert not np.array_equal(want[0], want[1])
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    ys = [torch.full((tokens, hidden), float("nan"), dtype=torch.float32, device="cuda") for _ in range(2)]
+    torch.cuda.synchronize()
+    for _ in range(6):
+        for i in range(2):
+            with torch.cuda.stream(streams[i]):
+                be.moe_ffn(lgs[i], gu, dn, e_, top_k, inter, sgu, sdn, sg, inter, hidden, xs[i], ys[i])
+    torch.cuda.synchronize()
+    for i in range(2):
+        assert np.array_equal(host(ys[i]).view(np.uint32), want[i].view(np.uint32)), i
+
+
 # ---------------------------------------------------------------- error behaviour
 def test_dispatch_contract_errors_and_noops(be):
     import ctypes as C

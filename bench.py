@@ -389,8 +389,7 @@ def main():
                                           "pct_of_hbm_peak": round(100 * b8 / ms8 / 1e6 / HBM_PEAK_GBPS, 2)}
 
         # The same four matrices as the real dependent chain of a token (o -> +residual, RMSNorm -> gate||up
-        # -> silu*up -> down -> +residual, RMSNorm -> qkv) through lq4_gemv_chain: step by step (the
-        # default: one fused launch per step) and as the one persistent launch.
+        # -> silu*up -> down -> +residual, RMSNorm -> qkv) through lq4_gemv_chain (one fused launch per step).
         if B == 1:
             cres, cres1, cres2 = (torch.randn(2048, device="cuda", generator=gen) for _ in range(3))
             cg1, cg2 = (0.1 * torch.randn(2048, device="cuda", generator=gen) for _ in range(2))
@@ -403,19 +402,13 @@ def main():
                 be.chain_step(b["qkv"], 3072, 2048, from_previous=True, norm=(cres1, None, cg2, 1e-6, cres2), y=cqkv)]
                 for b in layers]
             cf = lambda i: be.dispatch_chain(chains[i % len(chains)])
-            ch = {}
-            for mode, nm in ((backend.CHAIN_STEPWISE, "stepwise"), (backend.CHAIN_ONE_LAUNCH, "one_launch")):
-                be.set_chain_mode(mode)
-                try:
-                    for i in range(len(layers)):
-                        cf(i)
-                    be.synchronize()
-                    ms_c = tm(torch, cf, max(72, args.steps // 2))
-                    be.synchronize()
-                finally:
-                    be.set_chain_mode(backend.CHAIN_STEPWISE)
-                ch[nm] = {"us_per_step": round(ms_c * 1e3, 3), "GB/s": round(step_bytes / ms_c / 1e6, 1),
-                          "pct_of_hbm_peak": round(100 * step_bytes / ms_c / 1e6 / HBM_PEAK_GBPS, 2)}
+            for i in range(len(layers)):
+                cf(i)
+            be.synchronize()
+            ms_c = tm(torch, cf, max(72, args.steps // 2))
+            be.synchronize()
+            ch = {"us_per_step": round(ms_c * 1e3, 3), "GB/s": round(step_bytes / ms_c / 1e6, 1),
+                  "pct_of_hbm_peak": round(100 * step_bytes / ms_c / 1e6 / HBM_PEAK_GBPS, 2)}
             ch["note"] = ("dependent chain incl. residual adds, RMSNorms and silu*up; the headline's four GEMVs "
                           "alone are independent launches over the same weights")
             out["decode_layer_chain"] = ch

@@ -320,20 +320,16 @@ int lq4_gemv_fused_batch(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_off
                          const float* x_dev, uint32_t batch, float* y_dev, const lq4_gemv_fusion* fusion,
                          const lq4_lora* lora, float lora_scale, void* stream);
 
-/* ---- a chain of one-token GEMVs in one launch -------------------------------------------------
+/* ---- a chain of one-token GEMVs behind one call ------------------------------------------------
  * The reference encodes a whole token into one command buffer (forward_step,
  * forward/metal_qwen35.rs:6943, committed once at :6447): o -> residual add + RMSNorm -> gate||up ->
  * silu * up -> down -> residual add + next layer's RMSNorm -> qkv follow each other without the host
  * in between (encode_mlp_block, inner/layers/mod.rs; the elementwise dispatches at
  * inner/dispatch.rs:916-930, 1171-1290).  lq4_gemv_chain is that unit here: up to
  * LQ4_CHAIN_MAX_STEPS batch-1 GEMVs, each fed by an external vector or by an earlier step's result,
- * behind one call.  By default every step is one fused launch (lq4_gemv_fused, plus the stand-alone
- * silu * up where a step ends in it).  With lq4_set_chain_mode(LQ4_CHAIN_ONE_LAUNCH) an eligible
- * chain (every K <= 8192) runs as ONE persistent launch whose waves request the weights of later
- * steps while earlier results are still on their way and hand results over through tagged words in
- * library scratch; on MI355X that hand-over costs more than the launches it saves (36 us against
- * 16 us for the four GEMVs of a 2B decode layer), so it is not the default.  Both forms give the same
- * results to f32 rounding.
+ * behind one call.  Every step is one fused launch (lq4_gemv_fused: the elementwise work rides in the
+ * GEMV's prologue and epilogue; only a step that ends in silu * up on rows too short for the fused form
+ * runs the stand-alone silu * up kernel).  Results that no step's y_dev asks for live in library scratch.
  *
  * Step j computes r_j = epilogue(W_j . prologue(...)):
  *   prologue   LQ4_PRO_NONE         activations = x_dev [K], or r_(j-1) when from_previous != 0
@@ -351,10 +347,8 @@ int lq4_gemv_fused_batch(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_off
  *   y_dev      receives r_j when not NULL (the last step needs y_dev or a residual).
  * With from_previous the step's K must equal the length of r_(j-1).  Any input vector (x_dev, base,
  * delta) may also be the y_dev or residual_out of an earlier step of the same chain.  Vectors of
- * different steps must be identical or disjoint.  The launch keeps hand-over state in the context:
- * chains must not overlap on two streams of one context.  A hand-over that never completes (the
- * grid not resident at once because another kernel holds the GPU) ends the launch after a bounded
- * wait and lq4_sync returns LQ4_E_HIP; the chain's results are then invalid. */
+ * different steps must be identical or disjoint.  The call keeps intermediate results in the context:
+ * chains must not overlap on two streams of one context. */
 #define LQ4_CHAIN_MAX_STEPS 16
 #define LQ4_EPI_SILU_MUL_PAIRS 2
 typedef struct lq4_chain_step {
@@ -374,10 +368,6 @@ typedef struct lq4_chain_step {
     float* y_dev;
 } lq4_chain_step;
 int lq4_gemv_chain(lq4_ctx* ctx, const lq4_chain_step* steps, uint32_t n_steps, void* stream);
-/* Process-wide: how lq4_gemv_chain runs a chain.  No counterpart in the reference. */
-#define LQ4_CHAIN_STEPWISE 0   /* one launch per step (default) */
-#define LQ4_CHAIN_ONE_LAUNCH 1 /* one persistent launch where the chain is eligible */
-int lq4_set_chain_mode(int mode);
 
 /* Grows the context's scratch (partial tiles of K-sliced GEMMs, packed few-token operands, MoE
  * intermediates, lm_head logits) to at least `bytes` ahead of time.  The library grows it on demand
@@ -446,7 +436,7 @@ int lq4_probe_copy(lq4_ctx* ctx, const void* src_dev, void* dst_dev, size_t nbyt
  * PathProofCounters, metal_qwen35.rs:2144-2190): proves which path served a call. */
 typedef struct lq4_path_counters {
     uint64_t gemv, gemm, lora_a, moe_route, moe_gate_up, moe_down, dequant, topk, gemv_fused, elementwise;
-    uint64_t gemv_chain;       /* lq4_gemv_chain calls served by the single persistent launch */
+    uint64_t gemv_chain;       /* lq4_gemv_chain calls (each of their steps also counts under gemv_fused) */
     uint64_t lora_t_fallback;  /* waves of one-token LoRA launches that computed A.x themselves because
                                   the producers' hand-over did not arrive in time (read from the device:
                                   this call waits for the GPU) */

@@ -47,8 +47,6 @@ pub const LQ4_EPI_NONE: c_int = 0;
 pub const LQ4_EPI_ADD_RESIDUAL: c_int = 1;
 pub const LQ4_EPI_SILU_MUL_PAIRS: c_int = 2;
 pub const LQ4_CHAIN_MAX_STEPS: usize = 16;
-pub const LQ4_CHAIN_STEPWISE: c_int = 0;
-pub const LQ4_CHAIN_ONE_LAUNCH: c_int = 1;
 pub const LQ4_MAX_TOP_K: u32 = 256;
 pub const LQ4_STATIC_SCRATCH_BYTES: usize = 2 << 20;
 
@@ -221,7 +219,6 @@ extern "C" {
         stream: *mut c_void,
     ) -> c_int;
     pub fn lq4_gemv_chain(ctx: *mut Lq4Ctx, steps: *const Lq4ChainStep, n_steps: u32, stream: *mut c_void) -> c_int;
-    pub fn lq4_set_chain_mode(mode: c_int) -> c_int;
     pub fn lq4_set_lm_head_mode(mode: c_int) -> c_int;
 
     // ---- MoE

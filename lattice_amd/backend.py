@@ -53,7 +53,7 @@ EXPORTS = [
     "lq4_set_gemm_kernel",
     "lq4_residual_add_rmsnorm", "lq4_silu_mul", "lq4_add_and_copy", "lq4_gemv_fused", "lq4_gemv_fused_batch",
     "lq4_lm_head_topk_static",
-    "lq4_gemv_chain", "lq4_set_chain_mode", "lq4_set_lm_head_mode", "lq4_ctx_reserve_scratch",
+    "lq4_gemv_chain", "lq4_set_lm_head_mode", "lq4_ctx_reserve_scratch",
     "lq4_gemv_q8", "lq4_gemm_q8", "lq4_gemv_q3", "lq4_gemm_q3",
     "lq4_get_path_counters", "lq4_malloc", "lq4_free", "lq4_memcpy_h2d", "lq4_memcpy_d2h",
 ]
@@ -81,7 +81,6 @@ class PathCounters(C.Structure):
 LQ4_PRO_NONE, LQ4_PRO_ADD_RMSNORM, LQ4_PRO_SILU_MUL = 0, 1, 2
 LQ4_EPI_NONE, LQ4_EPI_ADD_RESIDUAL, LQ4_EPI_SILU_MUL_PAIRS = 0, 1, 2
 CHAIN_MAX_STEPS = 16
-CHAIN_STEPWISE, CHAIN_ONE_LAUNCH = 0, 1  # lq4_set_chain_mode
 LM_HEAD_ONE_LAUNCH, LM_HEAD_TWO_LAUNCHES = 0, 1  # lq4_set_lm_head_mode
 
 
@@ -155,7 +154,6 @@ def load_library() -> C.CDLL:
         "lq4_gemv_fused_batch": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, C.c_uint32, vp,
                                            C.POINTER(GemvFusion), vp, C.c_float, vp]),
         "lq4_gemv_chain": (C.c_int, [vp, C.POINTER(ChainStep), C.c_uint32, vp]),
-        "lq4_set_chain_mode": (C.c_int, [C.c_int]),
         "lq4_set_lm_head_mode": (C.c_int, [C.c_int]),
         "lq4_ctx_reserve_scratch": (C.c_int, [vp, C.c_size_t]),
         "lq4_get_path_counters": (C.c_int, [vp, C.POINTER(PathCounters)]),
@@ -492,11 +490,6 @@ class HipQ4Backend:
         (``forward_step`` encodes them into one command buffer, metal_qwen35.rs:6943), as one library call."""
         arr = (ChainStep * len(steps))(*steps)
         _check(self.lib.lq4_gemv_chain(self.ctx, arr, len(steps), self._stream()))
-
-    def set_chain_mode(self, mode: int):
-        """``CHAIN_STEPWISE`` (default): one launch per step; ``CHAIN_ONE_LAUNCH``: one persistent launch
-        where the chain is eligible."""
-        _check(self.lib.lq4_set_chain_mode(int(mode)))
 
     def dispatch_gemm(self, x, x_offset: int, qw: Q4WeightBuf, y, y_offset: int, m: int, n: int,
                       k: int, *, layer_idx=None, module=None):

@@ -31,14 +31,10 @@ struct lq4_ctx {
     // Buffers the growable scratch outgrew: launches already queued (or captured into a graph) may
     // still use them, so they are only released with the context.
     std::vector<void*> retired;
-    // lq4_gemv_chain: launch epoch (word 0) and failure word (word 64) in one allocation, the tagged
-    // result vectors of the steps, the CU count that sizes the resident grid
-    uint32_t* chain_sync;
+    // lq4_gemv_chain: the result vectors of steps whose result nobody asked for
     uint8_t* chain_scratch;
     size_t chain_scratch_bytes;
     uint32_t cu_count;
-    uint32_t chain_spin_limit;
-    bool chain_unchecked;  // a chain launch was queued since the failure word was last read
     // The stream of the last call that used the context's shared state (scratch buffers, hand-over words):
     // a call on another stream first waits for the device, so that calls alternating between streams are
     // serialised instead of racing on that state.
@@ -218,21 +214,13 @@ int lq4_ctx_create(int device_ordinal, lq4_ctx** out) {
     c->lora_sync = c->topk_ticket + 64;
     hipDeviceProp_t prop;
     e = hipGetDeviceProperties(&prop, device_ordinal);
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&c->chain_sync), 512 + 16384);
-    if (e == hipSuccess) e = hipMemset(c->chain_sync, 0, 512 + 16384);
-    if (e == hipSuccess) e = hipMemcpy(c->chain_sync, &first_epoch, 4, hipMemcpyHostToDevice);
     if (e != hipSuccess) {
-        if (c->chain_sync) (void)hipFree(c->chain_sync);
         (void)hipFree(c->topk_ticket);
         (void)hipFree(c->lora_t);
         delete c;
-        return fail(LQ4_E_HIP, "context set-up (chain words): %s", hipGetErrorString(e));
+        return fail(LQ4_E_HIP, "hipGetDeviceProperties: %s", hipGetErrorString(e));
     }
     c->cu_count = static_cast<uint32_t>(prop.multiProcessorCount);
-    // LQ4_CHAIN_SPIN_LIMIT: polls a wave of the chain kernel spends on one hand-over (0: none, the
-    // launch reports failure at its first dependent step; every kernel still exits)
-    c->chain_spin_limit = 1u << 20;
-    if (const char* env = getenv("LQ4_CHAIN_SPIN_LIMIT")) c->chain_spin_limit = static_cast<uint32_t>(strtoul(env, nullptr, 10));
     // LQ4_LORA_SPIN_LIMIT: 0 makes every weight wave compute A.x itself (the path a wave takes when
     // the producers are late), "off" restores the separate A.x launch
     c->lora_spin_limit = 512;
@@ -253,7 +241,6 @@ int lq4_ctx_destroy(lq4_ctx* ctx) {
     if (ctx->moe_scratch) (void)hipFree(ctx->moe_scratch);
     if (ctx->shared_scratch) (void)hipFree(ctx->shared_scratch);
     if (ctx->chain_scratch) (void)hipFree(ctx->chain_scratch);
-    (void)hipFree(ctx->chain_sync);
     for (void* p : ctx->retired) (void)hipFree(p);
     delete ctx;
     return LQ4_OK;
@@ -262,19 +249,6 @@ int lq4_ctx_destroy(lq4_ctx* ctx) {
 int lq4_sync(lq4_ctx* ctx, void* stream) {
     if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
     LQ4_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
-    if (ctx->chain_unchecked) {
-        DeviceGuard g(ctx->device);
-        uint32_t failed_step = 0;
-        LQ4_HIP(hipMemcpy(&failed_step, ctx->chain_sync + 64, sizeof failed_step, hipMemcpyDeviceToHost));
-        ctx->chain_unchecked = false;
-        if (failed_step) {
-            LQ4_HIP(hipMemset(ctx->chain_sync + 64, 0, sizeof failed_step));
-            return fail(LQ4_E_HIP,
-                        "lq4_gemv_chain: the activations of step %u never arrived (workgroups not resident together, "
-                        "or the wait was cut short); the chain's results are invalid, run it per step",
-                        failed_step);
-        }
-    }
     return LQ4_OK;
 }
 
@@ -1318,8 +1292,6 @@ int lq4_gemv_fused_batch(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_off
 // ---- a chain of batch-1 GEMVs --------------------------------------------------------------------
 namespace {
 
-int g_chain_mode = LQ4_CHAIN_STEPWISE;
-
 inline size_t up256(size_t v) { return (v + 255) / 256 * 256; }
 
 inline uint32_t chain_result_len(const lq4_chain_step& st) {
@@ -1388,104 +1360,21 @@ int chain_validate(const lq4_chain_step* steps, uint32_t n_steps) {
     return LQ4_OK;
 }
 
-// Byte offsets, in the chain scratch, of every step's result vector and of the residual stream its
-// prologue forms (8 bytes per value), and the total.
+// Byte offsets, in the chain scratch, of every step's result vector, and the total.
 struct ChainLayout {
-    size_t result[kMaxChainSteps], resid[kMaxChainSteps], total;
+    size_t result[LQ4_CHAIN_MAX_STEPS], total;
 };
 ChainLayout chain_scratch_layout(const lq4_chain_step* steps, uint32_t n_steps) {
     ChainLayout l;
     l.total = 0;
     for (uint32_t j = 0; j < n_steps; ++j) {
         l.result[j] = l.total;
-        l.total += up256(static_cast<size_t>(steps[j].n) * 8);  // n, not n/2: the per-step path keeps W . x here too
-        l.resid[j] = l.total;
-        if (steps[j].prologue == LQ4_PRO_ADD_RMSNORM) l.total += up256(static_cast<size_t>(steps[j].k) * 8);
+        l.total += up256(static_cast<size_t>(steps[j].n) * 4);  // n, not n/2: a [gate | up] vector may be kept here
     }
     return l;
 }
 
-// Fills the device descriptors of the persistent launch; false = the chain is not eligible for it
-// (a K too long for LDS, or a vector that an earlier step of the same chain writes and that cannot be
-// taken from that step's tagged copy).
-bool chain_plan(lq4_ctx* ctx, const lq4_chain_step* steps, uint32_t n_steps, const ChainLayout& lay, ChainArgs* args,
-                uint32_t* k_max) {
-    *k_max = 0;
-    std::memset(args, 0, sizeof *args);
-    args->n_steps = n_steps;
-    args->spin_limit = ctx->chain_spin_limit;
-    args->epoch = ctx->chain_sync;
-    args->fail = ctx->chain_sync + 64;
-    args->idle = reinterpret_cast<const uint8_t*>(ctx->chain_sync + 128);  // 16 KB behind the 512 bytes of words
-    auto words = [&](size_t off) { return reinterpret_cast<unsigned long long*>(ctx->chain_scratch + off); };
-    for (uint32_t j = 0; j < n_steps; ++j) {
-        const lq4_chain_step& st = steps[j];
-        ChainStep& d = args->s[j];
-        if (st.k > gemv_chain_max_k()) return false;
-        *k_max = st.k > *k_max ? st.k : *k_max;
-        (void)resolve_weight(st.w, st.w_extra_offset, st.n, st.k, &d.w);
-        d.n = st.n;
-        d.k = st.k;
-        d.flags = static_cast<uint32_t>(st.prologue) | (static_cast<uint32_t>(st.epilogue) << 8);
-        d.gamma = st.gamma;
-        d.eps = st.eps;
-        d.y = st.y_dev;
-        // An input vector that an earlier step of this chain wrote for the caller is not coherent
-        // inside the launch; that step's tagged copy is.  Sets *tagged (and makes the writer keep the
-        // copy) or *plain; false if the writer has no usable copy.
-        auto source = [&](const float* p, const float** plain, const unsigned long long** tagged) -> bool {
-            *plain = nullptr;
-            *tagged = nullptr;
-            if (!p) return true;
-            for (int i = static_cast<int>(j) - 1; i >= 0; --i) {
-                if (chain_result_ptr(steps[i]) == p) {
-                    args->s[i].out_tagged = words(lay.result[i]);
-                    *tagged = args->s[i].out_tagged;
-                    return true;
-                }
-                if (steps[i].prologue == LQ4_PRO_ADD_RMSNORM && steps[i].residual_out == p) {
-                    args->s[i].resid_out_tagged = words(lay.resid[i]);
-                    *tagged = args->s[i].resid_out_tagged;
-                    return true;
-                }
-                if (steps[i].y_dev == p || steps[i].residual == p) return false;  // written, but not as a whole result
-            }
-            *plain = p;
-            return true;
-        };
-        if (st.from_previous) {
-            args->s[j - 1].out_tagged = words(lay.result[j - 1]);
-            d.x_tagged = args->s[j - 1].out_tagged;
-        } else {
-            const float* b_src = st.prologue == LQ4_PRO_ADD_RMSNORM ? st.delta : st.x_dev;
-            if (!source(b_src, &d.x, &d.x_tagged)) return false;
-            if (st.prologue == LQ4_PRO_SILU_MUL && d.x_tagged) return false;  // gate | up must be external
-        }
-        if (st.prologue == LQ4_PRO_ADD_RMSNORM) {
-            if (!source(st.base, &d.base, &d.base_tagged)) return false;
-            d.resid_out = st.residual_out;
-        }
-        if (st.epilogue == LQ4_EPI_ADD_RESIDUAL) {
-            const float* plain;
-            const unsigned long long* tagged;
-            // the ring requests a row's residual word far ahead of the row: it must come from outside the chain
-            if (!source(st.residual, &plain, &tagged) || tagged) return false;
-            d.res_plain = st.residual;
-            d.res_out = st.residual;
-        }
-        gemv_chain_plan_step(d);
-    }
-    return gemv_chain_lds_bytes(*k_max) <= 160 * 1024;
-}
-
 }  // namespace
-
-int lq4_set_chain_mode(int mode) {
-    if (mode != LQ4_CHAIN_STEPWISE && mode != LQ4_CHAIN_ONE_LAUNCH)
-        return fail(LQ4_E_INVALID, "chain mode must be LQ4_CHAIN_STEPWISE (0) or LQ4_CHAIN_ONE_LAUNCH (1)");
-    g_chain_mode = mode;
-    return LQ4_OK;
-}
 
 int lq4_gemv_chain(lq4_ctx* ctx, const lq4_chain_step* steps, uint32_t n_steps, void* stream) {
     if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
@@ -1497,18 +1386,10 @@ int lq4_gemv_chain(lq4_ctx* ctx, const lq4_chain_step* steps, uint32_t n_steps, 
     hipStream_t s = static_cast<hipStream_t>(stream);
     DeviceGuard g(ctx->device);
     const ChainLayout lay = chain_scratch_layout(steps, n_steps);
-    rc = grow_scratch(ctx, &ctx->chain_scratch, &ctx->chain_scratch_bytes, lay.total, s, true);
+    rc = grow_scratch(ctx, &ctx->chain_scratch, &ctx->chain_scratch_bytes, lay.total, s, false);
     if (rc) return rc;
 
-    ChainArgs args;
-    uint32_t k_max = 0;
-    if (g_chain_mode == LQ4_CHAIN_ONE_LAUNCH && chain_plan(ctx, steps, n_steps, lay, &args, &k_max)) {
-        const hipError_t e = launch_gemv_chain(args, ctx->cu_count, k_max, s);
-        if (e != hipSuccess) return fail(LQ4_E_HIP, "chain launch: %s", hipGetErrorString(e));
-        ctx->chain_unchecked = true;
-        ctx->counters.gemv_chain++;
-        return LQ4_OK;
-    }
+    ctx->counters.gemv_chain++;
 
     // Step by step: every step is lq4_gemv_fused; results nobody asked for live in the chain scratch as
     // plain floats.  A step that ends in silu(gate) * up runs plain and the NEXT step takes gate || up

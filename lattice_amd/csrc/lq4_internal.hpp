@@ -84,51 +84,6 @@ void launch_gemv_b1_topk(const uint8_t* w, uint32_t n, uint32_t k, const float* 
 void launch_gemv_b1_fused(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y,
                           const LoraEpilogue& lora, const GemvFusion& fusion, hipStream_t stream);
 
-// One launch for a chain of batch-1 GEMVs (lq4_gemv_chain.hip).  A step's result vector is W . x after
-// its epilogue: kStore W . x [n]; kAddResidual res_plain + W . x [n] (also written to res_out; the
-// residual comes from outside the chain); kSiluMulPairs silu(y[i]) * y[i + n/2] [n/2] for
-// W = [gate rows | up rows].  Later steps read it from `out_tagged` ({f32, launch epoch} words in
-// library scratch).  The activations are prologue(A + B): A = base or base_tagged (kAddNorm only), B =
-// x or x_tagged; a tagged source is an earlier result of the same launch, a plain one is external.
-// kPlain: x itself; kAddNorm: shifted RMSNorm of A + B with gamma, eps, the sum also written to
-// resid_out / resid_out_tagged by workgroup 0; kSiluMul: x holds gate | up (2k floats, external).
-constexpr int kMaxChainSteps = 16;
-struct ChainStep {
-    enum Prologue : int { kPlain = 0, kAddNorm = 1, kSiluMul = 2 };
-    enum Epilogue : int { kStore = 0, kAddResidual = 1, kSiluMulPairs = 2 };
-    const uint8_t* w;
-    const float* x;
-    const unsigned long long* x_tagged;
-    const float* base;
-    const unsigned long long* base_tagged;
-    const float* gamma;
-    float* resid_out;
-    unsigned long long* resid_out_tagged;
-    const float* res_plain;
-    float* res_out;
-    float* y;                        // plain copy of the result, or null
-    unsigned long long* out_tagged;  // null when no later step reads the result
-    uint32_t n, k;
-    float eps;
-    uint32_t flags;   // prologue | epilogue << 8 | rows per group << 16 (the last by gemv_chain_plan_step)
-    uint32_t slabs, groups;  // work split, filled by gemv_chain_plan_step
-    uint32_t pad_[2];
-};
-static_assert(sizeof(ChainStep) == 128, "ChainStep is copied to LDS as 32 dwords");
-struct ChainArgs {
-    uint32_t n_steps;
-    uint32_t spin_limit;   // polls a wave spends on one hand-over before it gives up (0: give up at once)
-    uint32_t xs_dwords;    // LDS dwords per activation buffer, filled by the launcher
-    uint32_t* epoch;       // launch epoch word
-    uint32_t* fail;        // set to the step index whose activations never arrived
-    const uint8_t* idle;   // 16 KB of readable bytes: what waves without work in a step load instead of weights
-    ChainStep s[kMaxChainSteps];
-};
-size_t gemv_chain_lds_bytes(uint32_t k_max);
-uint32_t gemv_chain_max_k();
-void gemv_chain_plan_step(ChainStep& st);
-hipError_t launch_gemv_chain(ChainArgs& args, uint32_t workgroups, uint32_t k_max, hipStream_t stream);
-
 // Stand-alone forms of the same steps for any number of rows.
 //   residual_add_norm: v = base + delta (delta may be null); residual_out = v if set;
 //     normed_out = shifted RMSNorm of v.  Rows are `hidden` floats apart.

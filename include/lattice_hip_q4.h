@@ -56,10 +56,12 @@ const char* lq4_version(void);
 
 /* ---- context ------------------------------------------------------------------ */
 /* A context owns scratch buffers, the LoRA t = A.x buffer and a few hand-over words that its calls
- * share.  A call that uses them on another stream than the previous such call first waits for the
- * device, so calls alternating between streams are serialised instead of racing; this cannot be done
- * for a stream that is being captured, for graph replays or for calls from several host threads at
- * once: those need a context each. */
+ * share.  A call that uses them on another stream than the previous such call makes its stream wait
+ * (hipStreamWaitEvent) for everything queued on that previous stream so far, so calls alternating
+ * between streams are ordered instead of racing, without a host stall; when one of the two streams is
+ * being captured the dependency becomes part of the capture, like any other cross-stream edge.  What
+ * this cannot order: replays of graphs captured on different streams, and calls from several host
+ * threads at once.  Those need a context each. */
 int lq4_ctx_create(int device_ordinal, lq4_ctx** out);
 int lq4_ctx_destroy(lq4_ctx* ctx);
 /* hipStreamSynchronize(stream); the counterpart of commit()+wait_until_completed()
@@ -228,9 +230,9 @@ int lq4_topk(lq4_ctx* ctx, const float* logits_dev, uint32_t n, uint32_t top_k, 
  * 2048, top 50: 82.9 us against 76.7): making the logits visible to the selecting workgroup inside
  * the launch (write-through stores, their acknowledgement, the maximum's exchange and the ticket, one
  * after the other at the end of every workgroup) costs more than the second launch's pass over 1 MB
- * of logits.  The setting is process-wide. */
+ * of logits.  The setting belongs to the context. */
 enum { LQ4_LM_HEAD_ONE_LAUNCH = 0, LQ4_LM_HEAD_TWO_LAUNCHES = 1 };
-int lq4_set_lm_head_mode(int mode);
+int lq4_set_lm_head_mode(lq4_ctx* ctx, int mode);
 int lq4_lm_head_topk(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t vocab, uint32_t k,
                      const float* x_dev, uint32_t top_k, float* out_logits_dev, uint32_t* out_ids_dev,
                      void* stream);
@@ -242,7 +244,8 @@ int lq4_lm_head_topk(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset,
  * scratch, so the call makes no hipMalloc / hipFree and calls no allocating routine.  Shapes whose
  * scratch (vocab * 4 bytes, rounded up to 256, plus the selection's candidate buffers) does not fit
  * return LQ4_E_UNSUPPORTED: vocabularies up to 262 144 with top_k <= 256 fit.  Every context on one
- * GPU shares that GPU's array: calls that overlap on one GPU (two streams, two contexts) race. */
+ * GPU shares that GPU's array: calls of one context on alternating streams are ordered like its other
+ * calls (see lq4_ctx_create), calls of two contexts that overlap on one GPU race. */
 #define LQ4_STATIC_SCRATCH_BYTES (2u << 20)
 int lq4_lm_head_topk_static(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t vocab, uint32_t k,
                             const float* x_dev, uint32_t top_k, float* out_logits_dev, uint32_t* out_ids_dev,
@@ -369,8 +372,9 @@ typedef struct lq4_chain_step {
 } lq4_chain_step;
 int lq4_gemv_chain(lq4_ctx* ctx, const lq4_chain_step* steps, uint32_t n_steps, void* stream);
 
-/* Grows the context's scratch (partial tiles of K-sliced GEMMs, packed few-token operands, MoE
- * intermediates, lm_head logits) to at least `bytes` ahead of time.  The library grows it on demand
+/* Grows every scratch buffer of the context (partial tiles of K-sliced GEMMs, packed few-token operands,
+ * MoE and shared-expert intermediates, lm_head logits, the results a chain keeps between its steps) to at
+ * least `bytes` ahead of time.  The library grows them on demand
  * otherwise, which allocates: a call that would have to grow it while its stream is being captured
  * into a HIP graph returns LQ4_E_UNSUPPORTED instead.  Outgrown buffers stay allocated until
  * lq4_ctx_destroy, so launches already queued or captured keep valid addresses.  No counterpart in
@@ -420,12 +424,13 @@ int lq4_probe_read(lq4_ctx* ctx, const void* p_dev, size_t nbytes, void* stream)
 int lq4_probe_read_config(lq4_ctx* ctx, const void* p_dev, size_t nbytes, uint32_t workgroups, uint32_t bytes_in_flight,
                           int strided, int nontemporal, void* stream);
 
-/* Tuning/test hook, process-wide: 0 = lq4_gemm picks its kernel by shape (default), 1 = always
+/* Tuning/test hook, per context (a new context starts from the environment variable LQ4_GEMM_KERNEL,
+ * else 0): 0 = lq4_gemm picks its kernel by shape (default), 1 = always
  * the LDS-staged tile kernel, 2 = always the weights-in-registers kernel, 3 = always the
  * few-token kernel, 4 = always the weights-in-registers kernel at two workgroups per CU (Q4 without
  * LoRA; packs the activations into scratch first).  Results are identical in contract either way.
  * No counterpart in the reference. */
-int lq4_set_gemm_kernel(int which);
+int lq4_set_gemm_kernel(lq4_ctx* ctx, int which);
 
 /* Calibration: plain device copy of `nbytes` (both buffers 16-byte aligned, nbytes a multiple
  * of 16).  It reads and writes exactly nbytes, which scales the memory-traffic counters of a

@@ -219,7 +219,7 @@ extern "C" {
         stream: *mut c_void,
     ) -> c_int;
     pub fn lq4_gemv_chain(ctx: *mut Lq4Ctx, steps: *const Lq4ChainStep, n_steps: u32, stream: *mut c_void) -> c_int;
-    pub fn lq4_set_lm_head_mode(mode: c_int) -> c_int;
+    pub fn lq4_set_lm_head_mode(ctx: *mut Lq4Ctx, mode: c_int) -> c_int;
 
     // ---- MoE
     pub fn lq4_moe_route(
@@ -416,7 +416,7 @@ extern "C" {
         stream: *mut c_void,
     ) -> c_int;
     pub fn lq4_probe_copy(ctx: *mut Lq4Ctx, src: *const c_void, dst: *mut c_void, nbytes: usize, stream: *mut c_void) -> c_int;
-    pub fn lq4_set_gemm_kernel(which: c_int) -> c_int;
+    pub fn lq4_set_gemm_kernel(ctx: *mut Lq4Ctx, which: c_int) -> c_int;
     pub fn lq4_get_path_counters(ctx: *const Lq4Ctx, out: *mut Lq4PathCounters) -> c_int;
 
     // ---- device memory for callers without a HIP binding of their own

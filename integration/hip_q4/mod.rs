@@ -99,10 +99,11 @@ struct HipLoraAdapter {
     scale: f32,
 }
 
-/// One GPU's Q4 backend: context, stream, optional adapter.
+/// One GPU's Q4 backend: context, stream, the model's configuration, optional adapter.
 pub struct HipQ4Backend {
     ctx: *mut Lq4Ctx,
     stream: *mut c_void, // hipStream_t; null = the default stream
+    config: crate::model::qwen35_config::Qwen35Config,
     lora: Option<HipLoraAdapter>,
 }
 
@@ -115,11 +116,30 @@ impl Drop for HipQ4Backend {
 }
 
 impl HipQ4Backend {
-    pub fn new(device_ordinal: i32) -> Result<Self, String> {
+    /// `config`: the engine's model configuration, as the Metal state reads it from `self.engine.config`
+    /// (layer count, hidden size and projection shapes for the adapter checks below).
+    pub fn new(device_ordinal: i32, config: crate::model::qwen35_config::Qwen35Config) -> Result<Self, String> {
         let mut ctx = ptr::null_mut();
         // SAFETY: out pointer is valid for the call.
         check(unsafe { lq4_ctx_create(device_ordinal, &mut ctx) })?;
-        Ok(Self { ctx, stream: ptr::null_mut(), lora: None })
+        Ok(Self { ctx, stream: ptr::null_mut(), config, lora: None })
+    }
+
+    /// `expected_lora_shape` (metal_qwen35.rs:3746-3768) without the Metal-only capability filter: the GDN
+    /// gate projections are consumed inside a fused recurrence kernel there and rejected; this path has no such
+    /// kernel, but the forward loop that would apply them is the host crate's, so the same modules are refused.
+    fn expected_lora_shape(&self, layer_idx: usize, module: &str) -> Result<(usize, usize), String> {
+        if matches!(module, "in_proj_b" | "in_proj_a") {
+            if self.config.is_full_attention(layer_idx) {
+                return Err(format!("unknown LoRA module '{module}'"));
+            }
+            return Err(format!(
+                "module '{module}' is not yet supported in the HIP forward (consumed inside the GDN recurrence); \
+                 target other GDN modules instead"
+            ));
+        }
+        let shape = crate::lora_hook::qwen35_projection_shape(&self.config, layer_idx, module)?;
+        Ok((shape.d_in, shape.d_out))
     }
 
     /// `mmap_q4_weight` (metal_qwen35.rs:660-702): header + shape check as today
@@ -267,14 +287,13 @@ impl HipQ4Backend {
         check(rc).expect("lq4_lora_apply");
     }
 
-    /// `load_lora_adapter` (metal_qwen35.rs:3806-3986): same argument checks and error strings;
-    /// the QuaRot pre-rotation of `A` stays on the host (`rotate_adapter_for_quarot`) before upload.
+    /// `load_lora_adapter` (metal_qwen35.rs:3806-3986): same signature, same checks in the same order, same
+    /// error strings; the QuaRot pre-rotation of `A` stays on the host (`rotate_adapter_for_quarot`) before upload.
     pub fn load_lora_adapter(
         &mut self,
         mut layers: Vec<LoraLayerData>,
         scale: f32,
         quarot_seed: Option<u64>,
-        hidden_dim: usize,
     ) -> Result<(), String> {
         if self.lora.is_some() {
             return Err("LoRA adapter already loaded; call unload_lora_adapter first".into());
@@ -285,11 +304,12 @@ impl HipQ4Backend {
         if !scale.is_finite() {
             return Err(format!("load_lora_adapter: scale must be finite, got {scale}"));
         }
+        let hidden_dim = self.config.hidden_size;
         if let Some(seed) = quarot_seed {
             rotate_layers_for_quarot(&mut layers, seed, hidden_dim)?;
         }
-        let n_layers = layers.iter().map(|l| l.layer_idx).max().unwrap_or(0) + 1;
-        let mut projections: Vec<HashMap<String, HipLoraProjection>> = (0..n_layers).map(|_| HashMap::new()).collect();
+        let num_layers = self.config.num_hidden_layers;
+        let mut projections: Vec<HashMap<String, HipLoraProjection>> = (0..num_layers).map(|_| HashMap::new()).collect();
         for l in &layers {
             if l.rank == 0 {
                 return Err(format!("load_lora_adapter: layer {} module '{}' has rank=0", l.layer_idx, l.module));
@@ -300,10 +320,41 @@ impl HipQ4Backend {
                     l.layer_idx, l.module, l.d_in, l.d_out
                 ));
             }
-            if l.a.len() != l.rank * l.d_in || l.b.len() != l.d_out * l.rank {
+            if l.layer_idx >= num_layers {
+                return Err(format!("load_lora_adapter: layer_idx {} >= num_hidden_layers {}", l.layer_idx, num_layers));
+            }
+            let (exp_d_in, exp_d_out) = self.expected_lora_shape(l.layer_idx, &l.module)?;
+            if l.d_in != exp_d_in || l.d_out != exp_d_out {
                 return Err(format!(
-                    "load_lora_adapter: layer {} module {}: A/B sizes do not match rank {} d_in {} d_out {}",
-                    l.layer_idx, l.module, l.rank, l.d_in, l.d_out
+                    "load_lora_adapter: layer {} module '{}' has (d_in={}, d_out={}) but model expects (d_in={}, d_out={})",
+                    l.layer_idx, l.module, l.d_in, l.d_out, exp_d_in, exp_d_out
+                ));
+            }
+            let expected_a = l.rank.checked_mul(l.d_in).ok_or_else(|| {
+                format!("load_lora_adapter: layer {} module '{}' rank*d_in overflow", l.layer_idx, l.module)
+            })?;
+            let expected_b = l.d_out.checked_mul(l.rank).ok_or_else(|| {
+                format!("load_lora_adapter: layer {} module '{}' d_out*rank overflow", l.layer_idx, l.module)
+            })?;
+            if l.a.len() != expected_a {
+                return Err(format!(
+                    "load_lora_adapter: layer {} module '{}' A length {} != rank*d_in {}",
+                    l.layer_idx, l.module, l.a.len(), expected_a
+                ));
+            }
+            if l.b.len() != expected_b {
+                return Err(format!(
+                    "load_lora_adapter: layer {} module '{}' B length {} != d_out*rank {}",
+                    l.layer_idx, l.module, l.b.len(), expected_b
+                ));
+            }
+            let rank = u32::try_from(l.rank).map_err(|_| format!("load_lora_adapter: rank {} exceeds u32", l.rank))?;
+            let d_in = u32::try_from(l.d_in).map_err(|_| format!("load_lora_adapter: d_in {} exceeds u32", l.d_in))?;
+            let d_out = u32::try_from(l.d_out).map_err(|_| format!("load_lora_adapter: d_out {} exceeds u32", l.d_out))?;
+            if projections[l.layer_idx].contains_key(&l.module) {
+                return Err(format!(
+                    "load_lora_adapter: duplicate projection for layer {} module '{}'",
+                    l.layer_idx, l.module
                 ));
             }
             let mut raw = ptr::null_mut();
@@ -314,9 +365,9 @@ impl HipQ4Backend {
                     l.a.as_ptr() as *const c_void,
                     l.b.as_ptr() as *const c_void,
                     LQ4_F32,
-                    l.rank as u32,
-                    l.d_in as u32,
-                    l.d_out as u32,
+                    rank,
+                    d_in,
+                    d_out,
                     &mut raw,
                 )
             })?;

@@ -27,7 +27,7 @@ from __future__ import annotations
 import ctypes as C
 import os
 from dataclasses import dataclass
-from typing import Dict, List, Optional, Sequence, Tuple
+from typing import Callable, Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
 
@@ -141,7 +141,7 @@ def load_library() -> C.CDLL:
         "lq4_probe_read": (C.c_int, [vp, vp, C.c_size_t, vp]),
         "lq4_probe_read_config": (C.c_int, [vp, vp, C.c_size_t, C.c_uint32, C.c_uint32, C.c_int, C.c_int, vp]),
         "lq4_probe_copy": (C.c_int, [vp, vp, vp, C.c_size_t, vp]),
-        "lq4_set_gemm_kernel": (C.c_int, [C.c_int]),
+        "lq4_set_gemm_kernel": (C.c_int, [vp, C.c_int]),
         "lq4_residual_add_rmsnorm": (C.c_int, [vp, vp, vp, vp, C.c_uint32, C.c_uint32, C.c_float, vp, vp, vp]),
         "lq4_silu_mul": (C.c_int, [vp, vp, C.c_uint32, C.c_uint32, vp, C.c_uint32, vp]),
         "lq4_add_and_copy": (C.c_int, [vp, vp, vp, vp, C.c_size_t, vp]),
@@ -154,7 +154,7 @@ def load_library() -> C.CDLL:
         "lq4_gemv_fused_batch": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, C.c_uint32, vp,
                                            C.POINTER(GemvFusion), vp, C.c_float, vp]),
         "lq4_gemv_chain": (C.c_int, [vp, C.POINTER(ChainStep), C.c_uint32, vp]),
-        "lq4_set_lm_head_mode": (C.c_int, [C.c_int]),
+        "lq4_set_lm_head_mode": (C.c_int, [vp, C.c_int]),
         "lq4_ctx_reserve_scratch": (C.c_int, [vp, C.c_size_t]),
         "lq4_get_path_counters": (C.c_int, [vp, C.POINTER(PathCounters)]),
         "lq4_malloc": (C.c_int, [vp, C.c_size_t, C.POINTER(vp)]),
@@ -213,6 +213,20 @@ class LoraLayerData:
     modules: Dict[str, Tuple[np.ndarray, np.ndarray]]
 
 
+@dataclass
+class ModelShapes:
+    """What ``load_lora_adapter`` reads from the engine's model configuration in the reference
+    (``self.engine.config``, metal_qwen35.rs:3832, 3852, 3746-3768): the layer count, the hidden size and
+    the projection shape of a ``(layer_idx, module)`` pair.  ``projection_shape`` returns ``(d_in, d_out)``
+    or raises ``ValueError`` with the reference's message ("unknown LoRA module ...").  ``quarot_rotate``
+    is the host crate's ``rotate_adapter_for_quarot`` (quant/quarot/lora.rs): it rotates the layers' factors in
+    place for a QuaRot-converted base, ``quarot_rotate(layers, seed, hidden_size)``."""
+    num_hidden_layers: int
+    hidden_size: int
+    projection_shape: Callable[[int, str], Tuple[int, int]]
+    quarot_rotate: Optional[Callable] = None
+
+
 class _LoraProjection:
     def __init__(self, handle, rank, d_in, d_out):
         self.handle, self.rank, self.d_in, self.d_out = handle, rank, d_in, d_out
@@ -230,7 +244,9 @@ def _dtype_code(t) -> int:
 class HipQ4Backend:
     """One GPU's Q4 matmul backend: owns a ``lq4_ctx`` and the loaded LoRA adapter."""
 
-    def __init__(self, device: int = 0):
+    def __init__(self, device: int = 0, model: Optional["ModelShapes"] = None):
+        """``model``: the engine's model configuration as far as this path reads it (adapter checks); without
+        it ``load_lora_adapter`` checks everything that does not need the model."""
         import torch
         if not torch.cuda.is_available():
             raise RuntimeError("HipQ4Backend needs a HIP device; there is no CPU fallback")
@@ -240,6 +256,7 @@ class HipQ4Backend:
         ctx = C.c_void_p()
         _check(self.lib.lq4_ctx_create(device, C.byref(ctx)))
         self.ctx = ctx
+        self.model = model
         self._lora: Dict[Tuple[int, str], _LoraProjection] = {}
         self._lora_scale = 0.0
 
@@ -280,7 +297,7 @@ class HipQ4Backend:
     def set_gemm_kernel(self, which: int):
         """0 = pick the prefill kernel by shape, 1 = LDS-staged tile, 2 = weights in registers,
         3 = few-token kernel, 4 = weights in registers at two workgroups per CU."""
-        _check(self.lib.lq4_set_gemm_kernel(int(which)))
+        _check(self.lib.lq4_set_gemm_kernel(self.ctx, int(which)))
 
     def probe_copy(self, src, dst):
         """One plain copy launch src -> dst (equal-sized tensors): traffic-counter calibration."""
@@ -560,31 +577,64 @@ class HipQ4Backend:
     def set_lm_head_mode(self, mode: int):
         """``LM_HEAD_TWO_LAUNCHES`` (default): GEMV, then the selection kernel; ``LM_HEAD_ONE_LAUNCH``:
         the lm_head GEMV selects the top-k in its own launch where the shape allows."""
-        _check(self.lib.lq4_set_lm_head_mode(int(mode)))
+        _check(self.lib.lq4_set_lm_head_mode(self.ctx, int(mode)))
 
     # -------------------------------------------------------------------- LoRA
     def load_lora_adapter(self, layers: List[LoraLayerData], scale: float,
                           quarot_seed: Optional[int] = None):
-        """``load_lora_adapter(layers, scale, quarot_seed)`` (metal_qwen35.rs:3806-3986): uploads
-        every projection's A/B, replacing any adapter already loaded; ``scale`` (= alpha/rank,
-        crates/fann/src/lora.rs:110-117) is applied verbatim.  Rotating A/B for a QuaRot
-        checkpoint is the offline converter's job and is not part of this path."""
+        """``load_lora_adapter(layers, scale, quarot_seed)`` (metal_qwen35.rs:3806-3986): the reference's
+        checks in the reference's order with its messages, then every projection's A/B to the device;
+        ``scale`` (= alpha/rank, crates/fann/src/lora.rs:110-117) is applied verbatim.  With
+        ``quarot_seed`` the factors are first rotated on the host by the model's ``quarot_rotate`` (the
+        reference calls ``rotate_adapter_for_quarot`` at the same point, :3834-3849)."""
+        if self._lora:
+            raise Q4Error(-1, "LoRA adapter already loaded; call unload_lora_adapter first")
+        if not layers:
+            raise Q4Error(-1, "load_lora_adapter: layers must not be empty")
+        if not np.isfinite(scale):
+            raise Q4Error(-1, f"load_lora_adapter: scale must be finite, got {scale}")
         if quarot_seed is not None:
-            raise Q4Error(-5, "QuaRot rotation of LoRA factors is not supported by this backend")
+            if self.model is None or self.model.quarot_rotate is None:
+                raise Q4Error(-5, "load_lora_adapter: quarot_seed needs the host crate's rotate_adapter_for_quarot "
+                                  "(ModelShapes.quarot_rotate) and the model's hidden size")
+            self.model.quarot_rotate(layers, int(quarot_seed), self.model.hidden_size)
         staged: Dict[Tuple[int, str], _LoraProjection] = {}
         try:
             for layer in layers:
                 for module, (a, b) in layer.modules.items():
                     a = np.ascontiguousarray(a)
                     b = np.ascontiguousarray(b)
-                    if a.ndim != 2 or b.ndim != 2 or b.shape[1] != a.shape[0]:
-                        raise Q4Error(-1, f"layer {layer.layer_idx} {module}: A {a.shape} / B {b.shape} "
-                                          "are not [rank, d_in] / [d_out, rank]")
-                    if a.dtype != b.dtype or a.dtype not in (np.float32, np.float16):
-                        raise Q4Error(-1, f"layer {layer.layer_idx} {module}: A and B must both be "
-                                          "float32 or float16")
+                    if a.ndim != 2 or b.ndim != 2:
+                        raise Q4Error(-1, f"load_lora_adapter: layer {layer.layer_idx} module '{module}': A {a.shape} / "
+                                          f"B {b.shape} are not [rank, d_in] / [d_out, rank]")
                     rank, d_in = a.shape
                     d_out = b.shape[0]
+                    if rank == 0:
+                        raise Q4Error(-1, f"load_lora_adapter: layer {layer.layer_idx} module '{module}' has rank=0")
+                    if d_in == 0 or d_out == 0:
+                        raise Q4Error(-1, f"load_lora_adapter: layer {layer.layer_idx} module '{module}' has zero "
+                                          f"dimension (d_in={d_in}, d_out={d_out})")
+                    if self.model is not None:
+                        if not 0 <= layer.layer_idx < self.model.num_hidden_layers:
+                            raise Q4Error(-1, f"load_lora_adapter: layer_idx {layer.layer_idx} >= num_hidden_layers "
+                                              f"{self.model.num_hidden_layers}")
+                        try:
+                            exp_in, exp_out = self.model.projection_shape(layer.layer_idx, module)
+                        except ValueError as e:
+                            raise Q4Error(-1, str(e)) from None
+                        if (d_in, d_out) != (exp_in, exp_out):
+                            raise Q4Error(-1, f"load_lora_adapter: layer {layer.layer_idx} module '{module}' has "
+                                              f"(d_in={d_in}, d_out={d_out}) but model expects "
+                                              f"(d_in={exp_in}, d_out={exp_out})")
+                    if b.shape[1] != rank:
+                        raise Q4Error(-1, f"load_lora_adapter: layer {layer.layer_idx} module '{module}' B length "
+                                          f"{b.size} != d_out*rank {d_out * rank}")
+                    if a.dtype != b.dtype or a.dtype not in (np.float32, np.float16):
+                        raise Q4Error(-1, f"load_lora_adapter: layer {layer.layer_idx} module '{module}': A and B "
+                                          "must both be float32 or float16")
+                    if (layer.layer_idx, module) in staged:
+                        raise Q4Error(-1, f"load_lora_adapter: duplicate projection for layer {layer.layer_idx} "
+                                          f"module '{module}'")
                     h = C.c_void_p()
                     _check(self.lib.lq4_lora_upload(self.ctx, a.ctypes.data, b.ctypes.data,
                                                     LQ4_F16 if a.dtype == np.float16 else LQ4_F32,
@@ -594,7 +644,6 @@ class HipQ4Backend:
             for p in staged.values():
                 self.lib.lq4_lora_free(p.handle)
             raise
-        self.unload_lora_adapter()
         self._lora, self._lora_scale = staged, float(scale)
 
     def unload_lora_adapter(self):

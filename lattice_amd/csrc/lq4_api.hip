@@ -36,10 +36,13 @@ struct lq4_ctx {
     size_t chain_scratch_bytes;
     uint32_t cu_count;
     // The stream of the last call that used the context's shared state (scratch buffers, hand-over words):
-    // a call on another stream first waits for the device, so that calls alternating between streams are
-    // serialised instead of racing on that state.
+    // a call on another stream makes its stream wait for everything queued on that one so far, so that calls
+    // alternating between streams are ordered instead of racing on that state.
     hipStream_t state_stream;
     bool state_stream_known;
+    hipEvent_t state_event;  // recorded on the previous stream when a call arrives on another one
+    int lm_head_mode;        // lq4_set_lm_head_mode
+    int gemm_kernel;         // lq4_set_gemm_kernel
     lq4_path_counters counters;
 };
 
@@ -221,6 +224,15 @@ int lq4_ctx_create(int device_ordinal, lq4_ctx** out) {
         return fail(LQ4_E_HIP, "hipGetDeviceProperties: %s", hipGetErrorString(e));
     }
     c->cu_count = static_cast<uint32_t>(prop.multiProcessorCount);
+    e = hipEventCreateWithFlags(&c->state_event, hipEventDisableTiming);
+    if (e != hipSuccess) {
+        (void)hipFree(c->topk_ticket);
+        (void)hipFree(c->lora_t);
+        delete c;
+        return fail(LQ4_E_HIP, "hipEventCreate: %s", hipGetErrorString(e));
+    }
+    c->lm_head_mode = LQ4_LM_HEAD_TWO_LAUNCHES;  // measured faster: see lq4_set_lm_head_mode in the header
+    c->gemm_kernel = gemm_kernel_choice_default();
     // LQ4_LORA_SPIN_LIMIT: 0 makes every weight wave compute A.x itself (the path a wave takes when
     // the producers are late), "off" restores the separate A.x launch
     c->lora_spin_limit = 512;
@@ -242,6 +254,7 @@ int lq4_ctx_destroy(lq4_ctx* ctx) {
     if (ctx->shared_scratch) (void)hipFree(ctx->shared_scratch);
     if (ctx->chain_scratch) (void)hipFree(ctx->chain_scratch);
     for (void* p : ctx->retired) (void)hipFree(p);
+    (void)hipEventDestroy(ctx->state_event);
     delete ctx;
     return LQ4_OK;
 }
@@ -383,12 +396,12 @@ int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
     LoraEpilogue ep;
     rc = resolve_lora(ctx, lora, lora_scale, n, k, batch, &ep);
     if (rc) return rc;
-    if (ep.rank) {  // the A.x buffer (and, for one token, the hand-over words) belong to the context
-        rc = enter_shared_state(ctx, static_cast<hipStream_t>(stream));
-        if (rc) return rc;
-    }
     hipStream_t s = static_cast<hipStream_t>(stream);
     DeviceGuard g(ctx->device);
+    if (ep.rank) {  // the A.x buffer (and, for one token, the hand-over words) belong to the context
+        rc = enter_shared_state(ctx, s);
+        if (rc) return rc;
+    }
     if (ep.rank && batch == 1 && ctx->lora_in_kernel && gemv_b1_lds_bytes(k) <= 128 * 1024) {
         // one token: the GEMV launch computes A.x in its first `rank` workgroups
         ep.a = lora->a;
@@ -442,13 +455,23 @@ int lq4_lora_apply(lq4_ctx* ctx, const lq4_lora* lora, float lora_scale, const v
     return LQ4_OK;
 }
 
-// Called by every entry point that touches the context's shared state, before it launches anything.
-// A stream that is being captured cannot wait for the device: such calls stay the caller's to order.
+// Called by every entry point that touches the context's shared state, before it launches anything (the
+// context's device is current).  A call on another stream than the last one: that stream waits for an event
+// recorded on the last one now, i.e. for everything queued there so far.  No host stall, and legal while either
+// stream is being captured (the dependency then becomes part of the capture, as any cross-stream one does).
 static int enter_shared_state(lq4_ctx* ctx, hipStream_t stream) {
     if (ctx->state_stream_known && ctx->state_stream != stream) {
-        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing(stream, &cap) != hipSuccess) (void)hipGetLastError();
-        if (cap == hipStreamCaptureStatusNone) LQ4_HIP(hipDeviceSynchronize());
+        hipError_t e = hipEventRecord(ctx->state_event, ctx->state_stream);
+        if (e == hipSuccess) e = hipStreamWaitEvent(stream, ctx->state_event, 0);
+        if (e != hipSuccess) {
+            // (the previous stream may have been destroyed since: then the device is the only thing left to wait for)
+            (void)hipGetLastError();
+            hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+            if (hipStreamIsCapturing(stream, &cap) != hipSuccess) (void)hipGetLastError();
+            if (cap != hipStreamCaptureStatusNone)
+                return fail(LQ4_E_HIP, "cannot order this call behind the context's previous stream: %s", hipGetErrorString(e));
+            LQ4_HIP(hipDeviceSynchronize());
+        }
     }
     ctx->state_stream = stream;
     ctx->state_stream_known = true;
@@ -497,7 +520,10 @@ int lq4_ctx_reserve_scratch(lq4_ctx* ctx, size_t bytes) {
     const hipStream_t was = ctx->state_stream;  // (no launch: the stream of the last one stays)
     const bool known = ctx->state_stream_known;
     ctx->state_stream_known = false;
-    const int rc = ensure_scratch(ctx, bytes, nullptr);
+    // every growable buffer: which one an entry point uses is the library's business, not the caller's
+    int rc = ensure_scratch(ctx, bytes, nullptr);
+    if (!rc) rc = grow_scratch(ctx, &ctx->shared_scratch, &ctx->shared_scratch_bytes, bytes, nullptr, false);
+    if (!rc) rc = grow_scratch(ctx, &ctx->chain_scratch, &ctx->chain_scratch_bytes, bytes, nullptr, false);
     ctx->state_stream = was;
     ctx->state_stream_known = known;
     return rc;
@@ -520,24 +546,24 @@ int lq4_gemm(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
     LoraEpilogue ep;
     rc = resolve_lora(ctx, lora, lora_scale, n, k, m, &ep);
     if (rc) return rc;
-    if (ep.rank) {  // the A.x buffer (and, for one token, the hand-over words) belong to the context
-        rc = enter_shared_state(ctx, static_cast<hipStream_t>(stream));
-        if (rc) return rc;
-    }
     hipStream_t s = static_cast<hipStream_t>(stream);
     DeviceGuard g(ctx->device);
+    if (ep.rank) {  // the A.x buffer (and, for one token, the hand-over words) belong to the context
+        rc = enter_shared_state(ctx, s);
+        if (rc) return rc;
+    }
     if (ep.rank) {
         launch_lora_a(lora->a, lora->is_f16, lora->rank, k, x_dev, x_dtype == LQ4_F16, k, m, ctx->lora_t, s);
         ctx->counters.lora_a++;
     }
     // shapes with too few tiles run as K slices into scratch partials, summed by a second kernel
-    const size_t scratch_bytes = gemm_scratch_floats(n, k, m, x_dtype == LQ4_F16, ep.rank != 0) * sizeof(float);
+    const size_t scratch_bytes = gemm_scratch_floats(n, k, m, x_dtype == LQ4_F16, ep.rank != 0, ctx->gemm_kernel) * sizeof(float);
     if (scratch_bytes) {
         rc = ensure_scratch(ctx, scratch_bytes, static_cast<hipStream_t>(stream));
         if (rc) return rc;
     }
     launch_gemm(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, ep,
-                scratch_bytes ? reinterpret_cast<float*>(ctx->moe_scratch) : nullptr, s);
+                scratch_bytes ? reinterpret_cast<float*>(ctx->moe_scratch) : nullptr, ctx->gemm_kernel, s);
     ctx->counters.gemm++;
     LQ4_HIP(hipGetLastError());
     return LQ4_OK;
@@ -912,12 +938,11 @@ int lq4_topk(lq4_ctx* ctx, const float* logits_dev, uint32_t n, uint32_t top_k, 
 
 namespace {
 
-int g_lm_head_mode = LQ4_LM_HEAD_TWO_LAUNCHES;  // measured faster: see lq4_set_lm_head_mode in the header
 
 // Scratch of one lm_head + top-k call: [vocab logits | maxima, candidates], in the layout of whichever
 // path serves the shape.
-size_t lm_head_scratch_need(uint32_t vocab, uint32_t k, uint32_t top_k, bool* one_launch) {
-    const size_t fused = g_lm_head_mode == LQ4_LM_HEAD_ONE_LAUNCH ? gemv_b1_topk_scratch_bytes(vocab, k, top_k) : 0;
+size_t lm_head_scratch_need(int mode, uint32_t vocab, uint32_t k, uint32_t top_k, bool* one_launch) {
+    const size_t fused = mode == LQ4_LM_HEAD_ONE_LAUNCH ? gemv_b1_topk_scratch_bytes(vocab, k, top_k) : 0;
     *one_launch = fused != 0;
     if (fused) return fused;
     const size_t logits_bytes = (static_cast<size_t>(vocab) * sizeof(float) + 255) / 256 * 256;
@@ -937,7 +962,7 @@ int lm_head_topk_common(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offs
     if (!x_dev || !out_logits_dev || !out_ids_dev) return fail(LQ4_E_INVALID, "null device pointer");
     if (reinterpret_cast<uintptr_t>(x_dev) % 16) return fail(LQ4_E_INVALID, "x must be 16-byte aligned");
     bool one_launch;
-    const size_t need = lm_head_scratch_need(vocab, k, top_k, &one_launch);
+    const size_t need = lm_head_scratch_need(ctx->lm_head_mode, vocab, k, top_k, &one_launch);
     hipStream_t s = static_cast<hipStream_t>(stream);
     DeviceGuard g(ctx->device);
     uint8_t* base;
@@ -947,6 +972,8 @@ int lm_head_topk_common(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offs
                         "lq4_lm_head_topk_static: vocab %u with top_k %u needs %zu bytes of scratch, the static buffer holds %zu; "
                         "use lq4_lm_head_topk", vocab, top_k, need, kStaticScratchBytes);
         base = ctx->static_scratch;
+        rc = enter_shared_state(ctx, s);  // the static array and the ticket word are shared like the scratch
+        if (rc) return rc;
     } else {
         rc = ensure_scratch(ctx, need, s);
         if (rc) return rc;
@@ -970,10 +997,11 @@ int lm_head_topk_common(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offs
 
 }  // namespace
 
-int lq4_set_lm_head_mode(int mode) {
+int lq4_set_lm_head_mode(lq4_ctx* ctx, int mode) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
     if (mode != LQ4_LM_HEAD_ONE_LAUNCH && mode != LQ4_LM_HEAD_TWO_LAUNCHES)
         return fail(LQ4_E_INVALID, "unknown lm_head mode %d", mode);
-    g_lm_head_mode = mode;
+    ctx->lm_head_mode = mode;
     return LQ4_OK;
 }
 
@@ -1082,12 +1110,12 @@ int lq4_gemv_fused(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, u
     LoraEpilogue ep;
     rc = resolve_lora(ctx, lora, lora_scale, n, k, 1, &ep);
     if (rc) return rc;
-    if (ep.rank) {  // the A.x buffer (and, for one token, the hand-over words) belong to the context
-        rc = enter_shared_state(ctx, static_cast<hipStream_t>(stream));
-        if (rc) return rc;
-    }
     hipStream_t s = static_cast<hipStream_t>(stream);
     DeviceGuard g(ctx->device);
+    if (ep.rank) {  // the A.x buffer (and, for one token, the hand-over words) belong to the context
+        rc = enter_shared_state(ctx, s);
+        if (rc) return rc;
+    }
 
     const bool pairs = f.epilogue == LQ4_EPI_SILU_MUL_PAIRS;
     const bool fused_ok = gemv_b1_lds_bytes(k) <= 128 * 1024 && !(ep.rank && f.prologue != LQ4_PRO_NONE) &&
@@ -1213,12 +1241,12 @@ int lq4_gemv_fused_batch(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_off
     LoraEpilogue ep;
     rc = resolve_lora(ctx, lora, lora_scale, n, k, batch, &ep);
     if (rc) return rc;
-    if (ep.rank) {  // the A.x buffer (and, for one token, the hand-over words) belong to the context
-        rc = enter_shared_state(ctx, static_cast<hipStream_t>(stream));
-        if (rc) return rc;
-    }
     hipStream_t s = static_cast<hipStream_t>(stream);
     DeviceGuard g(ctx->device);
+    if (ep.rank) {  // the A.x buffer (and, for one token, the hand-over words) belong to the context
+        rc = enter_shared_state(ctx, s);
+        if (rc) return rc;
+    }
 
     // Inside the launch every workgroup produces all rows' activations for itself: that pays while the
     // rows are small (one token always; more rows up to this many bytes of prologue input per workgroup:
@@ -1485,9 +1513,9 @@ int lq4_gemm_q8(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
         launch_gemm_skinny(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, none, ctx->moe_scratch, s, 1);
         ctx->counters.gemm++;
     } else {
-        const int src = ensure_scratch(ctx, gemm_sibling_scratch_floats(1, n, k, m) * sizeof(float), static_cast<hipStream_t>(stream));
+        const int src = ensure_scratch(ctx, gemm_sibling_scratch_floats(1, n, k, m, ctx->gemm_kernel) * sizeof(float), static_cast<hipStream_t>(stream));
         if (src) return src;
-        launch_gemm_q8(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, reinterpret_cast<float*>(ctx->moe_scratch), s);
+        launch_gemm_q8(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, reinterpret_cast<float*>(ctx->moe_scratch), ctx->gemm_kernel, s);
         ctx->counters.gemm++;
     }
     LQ4_HIP(hipGetLastError());
@@ -1526,9 +1554,9 @@ int lq4_gemm_q3(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
         launch_gemm_skinny(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, none, ctx->moe_scratch, s, 2);
         ctx->counters.gemm++;
     } else {
-        const int src = ensure_scratch(ctx, gemm_sibling_scratch_floats(2, n, k, m) * sizeof(float), static_cast<hipStream_t>(stream));
+        const int src = ensure_scratch(ctx, gemm_sibling_scratch_floats(2, n, k, m, ctx->gemm_kernel) * sizeof(float), static_cast<hipStream_t>(stream));
         if (src) return src;
-        launch_gemm_q3(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, reinterpret_cast<float*>(ctx->moe_scratch), s);
+        launch_gemm_q3(wp, n, k, x_dev, x_dtype == LQ4_F16, m, y_dev, reinterpret_cast<float*>(ctx->moe_scratch), ctx->gemm_kernel, s);
         ctx->counters.gemm++;
     }
     LQ4_HIP(hipGetLastError());
@@ -1542,9 +1570,10 @@ int lq4_gemv_q3(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
     return lq4_gemm_q3(ctx, w, w_extra_offset, n, k, x_dev, LQ4_F32, batch, y_dev, stream);
 }
 
-int lq4_set_gemm_kernel(int which) {
+int lq4_set_gemm_kernel(lq4_ctx* ctx, int which) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
     if (which < 0 || which > 4) return fail(LQ4_E_INVALID, "gemm kernel choice must be 0..4");
-    set_gemm_kernel_choice(which);
+    ctx->gemm_kernel = which;
     return LQ4_OK;
 }
 

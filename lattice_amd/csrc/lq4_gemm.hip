@@ -506,15 +506,14 @@ void launch_tile(const uint8_t* w, uint32_t n, uint32_t k, const void* x, uint32
 
 
 
-// kernel choice override: starts from the environment variable LQ4_GEMM_KERNEL (0, 1 or 2)
-std::atomic<int> g_gemm_choice{[] {
-    const char* e = getenv("LQ4_GEMM_KERNEL");
-    return e ? atoi(e) : 0;
-}()};
-
 }  // namespace
 
-void set_gemm_kernel_choice(int which) { g_gemm_choice.store(which, std::memory_order_relaxed); }
+// What a context's kernel choice starts from: the environment variable LQ4_GEMM_KERNEL (0..4).
+int gemm_kernel_choice_default() {
+    const char* e = getenv("LQ4_GEMM_KERNEL");
+    const int v = e ? atoi(e) : 0;
+    return v >= 0 && v <= 4 ? v : 0;
+}
 
 namespace {
 
@@ -525,8 +524,7 @@ struct GemmPlan {
     bool w2;  // the weights-in-registers tile at two workgroups per CU (activations packed first)
 };
 
-GemmPlan plan_gemm(uint32_t n, uint32_t k, uint32_t m, int x_is_f16, bool with_lora) {
-    const int forced = g_gemm_choice.load(std::memory_order_relaxed);
+GemmPlan plan_gemm(uint32_t n, uint32_t k, uint32_t m, int x_is_f16, bool with_lora, int forced) {
     if (forced == 3 || (forced == 0 && gemm_skinny_wants(n, k, m))) return {false, true, false};
     if (forced == 1 || !gemm_wreg_supports(n, k, m, x_is_f16)) return {false, false, false};
     if (!with_lora && (forced == 4 || (forced == 0 && gemm_w2_wants(n, k, m)))) return {false, false, true};
@@ -537,16 +535,16 @@ GemmPlan plan_gemm(uint32_t n, uint32_t k, uint32_t m, int x_is_f16, bool with_l
 
 }  // namespace
 
-size_t gemm_scratch_floats(uint32_t n, uint32_t k, uint32_t m, int x_is_f16, bool with_lora) {
-    const GemmPlan p = plan_gemm(n, k, m, x_is_f16, with_lora);
+size_t gemm_scratch_floats(uint32_t n, uint32_t k, uint32_t m, int x_is_f16, bool with_lora, int forced) {
+    const GemmPlan p = plan_gemm(n, k, m, x_is_f16, with_lora, forced);
     if (p.skinny) return (gemm_skinny_scratch_bytes(k, m) + sizeof(float) - 1) / sizeof(float);
     if (p.w2) return (gemm_w2_scratch_bytes(n, k, m) + sizeof(float) - 1) / sizeof(float);
     return p.wreg ? gemm_wreg_scratch_floats(n, k, m) : 0;
 }
 
 void launch_gemm(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
-                 float* y, const LoraEpilogue& lora, float* scratch, hipStream_t stream) {
-    const GemmPlan p = plan_gemm(n, k, m, x_is_f16, lora.rank != 0);
+                 float* y, const LoraEpilogue& lora, float* scratch, int forced, hipStream_t stream) {
+    const GemmPlan p = plan_gemm(n, k, m, x_is_f16, lora.rank != 0, forced);
     if (p.skinny) return launch_gemm_skinny(w, n, k, x, x_is_f16, m, y, lora, scratch, stream);
     if (p.w2) return launch_gemm_w2(w, n, k, x, x_is_f16, m, y, reinterpret_cast<uint8_t*>(scratch), stream);
     if (p.wreg) return launch_gemm_wreg(w, n, k, x, x_is_f16, m, y, lora, scratch, stream);
@@ -563,8 +561,7 @@ void launch_gemm(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_
 // kernel is forced (choice 1).  Q8_0 blocks are 1.7 x the bytes and 2-byte aligned, which costs the
 // register kernel more than the tile kernel (measured): it is taken on long, wide matrices only.
 namespace {
-bool sibling_wants_wreg(int fmt, uint32_t n, uint32_t k) {
-    const int forced = g_gemm_choice.load(std::memory_order_relaxed);
+bool sibling_wants_wreg(int fmt, uint32_t n, uint32_t k, int forced) {
     if (forced == 1) return false;
     if (forced == 2) return true;
     return fmt != 1 || (k >= 4096 && n >= 4096);
@@ -572,29 +569,29 @@ bool sibling_wants_wreg(int fmt, uint32_t n, uint32_t k) {
 
 template <int FMT>
 void launch_sibling(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
-                    float* scratch, hipStream_t stream) {
+                    float* scratch, int forced, hipStream_t stream) {
     const LoraEpilogue none{nullptr, nullptr, 0, 0, 0.0f};
-    if (sibling_wants_wreg(FMT, n, k)) return launch_gemm_wreg(w, n, k, x, x_is_f16, m, y, none, scratch, stream, FMT);
+    if (sibling_wants_wreg(FMT, n, k, forced)) return launch_gemm_wreg(w, n, k, x, x_is_f16, m, y, none, scratch, stream, FMT);
     if (x_is_f16) launch_tile<true, 128, false, FMT>(w, n, k, x, m, y, none, stream, scratch);
     else launch_tile<false, 128, false, FMT>(w, n, k, x, m, y, none, stream, scratch);
 }
 }  // namespace
 
-size_t gemm_sibling_scratch_floats(int fmt, uint32_t n, uint32_t k, uint32_t m) {
-    if (sibling_wants_wreg(fmt, n, k)) return gemm_wreg_scratch_floats(n, k, m);
+size_t gemm_sibling_scratch_floats(int fmt, uint32_t n, uint32_t k, uint32_t m, int forced) {
+    if (sibling_wants_wreg(fmt, n, k, forced)) return gemm_wreg_scratch_floats(n, k, m);
     const TileSlices ts = plan_tile_slices<128>(n, k, m);
     if (ts.count < 2) return 0;
     return static_cast<size_t>((n + 127) / 128) * ((m + BM - 1) / BM) * ts.count * (BM * 128);
 }
 
 void launch_gemm_q8(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
-                    float* scratch, hipStream_t stream) {
-    launch_sibling<1>(w, n, k, x, x_is_f16, m, y, scratch, stream);
+                    float* scratch, int forced, hipStream_t stream) {
+    launch_sibling<1>(w, n, k, x, x_is_f16, m, y, scratch, forced, stream);
 }
 
 void launch_gemm_q3(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
-                    float* scratch, hipStream_t stream) {
-    launch_sibling<2>(w, n, k, x, x_is_f16, m, y, scratch, stream);
+                    float* scratch, int forced, hipStream_t stream) {
+    launch_sibling<2>(w, n, k, x, x_is_f16, m, y, scratch, forced, stream);
 }
 
 }  // namespace lq4

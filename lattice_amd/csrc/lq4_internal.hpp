@@ -134,18 +134,18 @@ void launch_lora_b_accum(const void* b, int b_is_f16, uint32_t rank, uint32_t d_
 
 // Y[M,N] = X[M,K] . W^T (+ LoRA); X f32 or f16, Y f32.
 // gemm_scratch_floats = floats of scratch launch_gemm needs for the shape (0 = none).
-size_t gemm_scratch_floats(uint32_t n, uint32_t k, uint32_t m, int x_is_f16, bool with_lora);
+// `forced`: 0 = choose by shape, 1 = LDS-staged kernel, 2 = weights-in-registers kernel where supported,
+// 3 = few-token kernel, 4 = the weights-in-registers tile at two workgroups per CU (a context's setting).
+size_t gemm_scratch_floats(uint32_t n, uint32_t k, uint32_t m, int x_is_f16, bool with_lora, int forced);
 void launch_gemm(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
-                 float* y, const LoraEpilogue& lora, float* scratch, hipStream_t stream);
+                 float* y, const LoraEpilogue& lora, float* scratch, int forced, hipStream_t stream);
+int gemm_kernel_choice_default();  // from the environment variable LQ4_GEMM_KERNEL
 
 // Large-shape variant: weights dequantised in registers, only activations staged in LDS.
 // Tile 128 tokens x 256 weight rows; gemm_wreg_tiles = workgroups it would launch;
 // gemm_wreg_supports = the kernel can run the shape at all.
 uint32_t gemm_wreg_tiles(uint32_t n, uint32_t m);
 bool gemm_wreg_supports(uint32_t n, uint32_t k, uint32_t m, int x_is_f16);
-// 0 = choose by shape, 1 = LDS-staged kernel, 2 = weights-in-registers kernel where supported,
-// 3 = few-token kernel.
-void set_gemm_kernel_choice(int which);
 // A last, partly filled round of tiles is cut into K slices that meet in `partial`
 // (gemm_wreg_scratch_floats floats; null = no slicing) and are summed by a second kernel.
 size_t gemm_wreg_scratch_floats(uint32_t n, uint32_t k, uint32_t m);
@@ -163,16 +163,16 @@ void launch_gemm_wreg(const uint8_t* w, uint32_t n, uint32_t k, const void* x, i
 size_t gemv_q8_lds_bytes(uint32_t k);
 void launch_gemv_q8_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, hipStream_t stream);
 void launch_gemm_q8(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
-                    float* scratch, hipStream_t stream);
+                    float* scratch, int forced, hipStream_t stream);
 // Floats of scratch the sibling tile GEMMs use to cut K on shapes with few tiles (0 = none; a null
 // scratch pointer keeps K whole).
-size_t gemm_sibling_scratch_floats(int fmt, uint32_t n, uint32_t k, uint32_t m);  // fmt: 1 = Q8_0, 2 = Q3
+size_t gemm_sibling_scratch_floats(int fmt, uint32_t n, uint32_t k, uint32_t m, int forced);  // fmt: 1 = Q8_0, 2 = Q3
 
 // Q3 sibling format (16-byte blocks: f16 scale, f16 bias, 2-bit and 1-bit planes): same pair of paths.
 size_t gemv_q3_lds_bytes(uint32_t k);
 void launch_gemv_q3_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, hipStream_t stream);
 void launch_gemm_q3(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
-                    float* scratch, hipStream_t stream);
+                    float* scratch, int forced, hipStream_t stream);
 
 // Few-token variant (up to 128 tokens): activations packed once into matrix-core operand order
 // (gemm_skinny_scratch_bytes bytes at `packed_x`), then a kernel without LDS staging.

@@ -83,12 +83,9 @@ def test_decode_layer_chain_matches_oracle_sequence(hidden, inter, qkv_rows):
     # in fact f32-faithful
     assert rel_err(got_r, want_r2) <= 2e-5 and rel_err(got_qkv, want_qkv) <= 2e-5
 
-    # the same steps as separate calls of the fused GEMV (what the chain issues): identical bits
-    import torch
-    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
-    fused_before = be.path_counters()["gemv_fused"]
+    # a second run of the same chain: the same bits (every sum has a fixed order)
     got_r_again, got_qkv_again, _, _ = _run_layer_chain(be, qw, x_attn, r0, g1, g2, hidden, inter, qkv_rows, want_h=True)
-    assert be.path_counters()["gemv_fused"] >= fused_before + 4  # one fused launch per step at least
+    assert be.path_counters()["gemv_chain"] == before + 2
     assert np.array_equal(got_r, got_r_again) and np.array_equal(got_qkv, got_qkv_again)
     be.close()
 

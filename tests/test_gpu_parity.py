@@ -341,6 +341,94 @@ def test_lora_f32_factors_and_gemm_route(be):
         be.unload_lora_adapter()
 
 
+def test_load_lora_adapter_checks_like_the_reference():
+    """forward/metal_qwen35.rs:3795-3830 and :3852-3960: the reference's refusals, in its order and words."""
+    f = np.float32
+    shapes = {"q_proj": (64, 128), "v_proj": (64, 32)}
+
+    def projection_shape(layer_idx, module):
+        if module not in shapes:
+            raise ValueError(f"unknown LoRA module '{module}'")
+        return shapes[module]
+
+    rotated = []
+
+    def rotate(layers, seed, hidden):
+        rotated.append((len(layers), seed, hidden))
+
+    b = backend.HipQ4Backend(0, model=backend.ModelShapes(2, 64, projection_shape, quarot_rotate=rotate))
+    plain = backend.HipQ4Backend(0)
+    try:
+        ok_a, ok_b = np.zeros((4, 64), f), np.zeros((128, 4), f)
+        good = backend.LoraLayerData(0, {"q_proj": (ok_a, ok_b)})
+        with pytest.raises(backend.Q4Error, match="layers must not be empty"):
+            b.load_lora_adapter([], 1.0)
+        with pytest.raises(backend.Q4Error, match="scale must be finite"):
+            b.load_lora_adapter([good], float("nan"))
+        with pytest.raises(backend.Q4Error, match="has rank=0"):
+            b.load_lora_adapter([backend.LoraLayerData(0, {"q_proj": (np.zeros((0, 64), f), np.zeros((128, 0), f))})], 1.0)
+        with pytest.raises(backend.Q4Error, match=r"layer_idx 2 >= num_hidden_layers 2"):
+            b.load_lora_adapter([backend.LoraLayerData(2, {"q_proj": (ok_a, ok_b)})], 1.0)
+        with pytest.raises(backend.Q4Error, match="unknown LoRA module 'w_proj'"):
+            b.load_lora_adapter([backend.LoraLayerData(0, {"w_proj": (ok_a, ok_b)})], 1.0)
+        with pytest.raises(backend.Q4Error, match=r"has \(d_in=64, d_out=100\) but model expects \(d_in=64, d_out=128\)"):
+            b.load_lora_adapter([backend.LoraLayerData(0, {"q_proj": (ok_a, np.zeros((100, 4), f))})], 1.0)
+        with pytest.raises(backend.Q4Error, match="B length"):
+            b.load_lora_adapter([backend.LoraLayerData(0, {"q_proj": (ok_a, np.zeros((128, 5), f))})], 1.0)
+        with pytest.raises(backend.Q4Error, match="duplicate projection for layer 0 module 'q_proj'"):
+            b.load_lora_adapter([good, backend.LoraLayerData(0, {"q_proj": (ok_a, ok_b)})], 1.0)
+        assert not b._lora, "a refused adapter leaves nothing loaded"
+        # a QuaRot seed goes to the host's rotation, at the reference's point: before the per-layer checks
+        b.load_lora_adapter([good], 2.0, quarot_seed=7)
+        assert rotated == [(1, 7, 64)]
+        with pytest.raises(backend.Q4Error, match="already loaded; call unload_lora_adapter first"):
+            b.load_lora_adapter([good], 2.0)
+        b.unload_lora_adapter()
+        b.load_lora_adapter([good], 2.0)  # and again once unloaded
+        b.unload_lora_adapter()
+        # without a model the same wrapper still refuses what needs no model, and a seed it cannot serve
+        with pytest.raises(backend.Q4Error, match="quarot_seed needs"):
+            plain.load_lora_adapter([good], 1.0, quarot_seed=7)
+        with pytest.raises(backend.Q4Error, match="duplicate projection"):
+            plain.load_lora_adapter([good, good], 1.0)
+    finally:
+        b.close()
+        plain.close()
+
+
+def test_activations_beyond_f16_range_above_one_row(be):
+    """One row takes any finite f32 activation; kernels that stage several rows as f16 (as the reference's tiled
+    GEMM does, shaders/gemm_q4_tiled.metal:45-48) turn |x| >= 65504 into infinity in the row that holds it.
+    Pinned here: that row is either right or non-finite as a whole, and every other row is unaffected."""
+    import torch
+    n, k = 96, 256
+    wq = synth.q4_weight(n, k, seed=21)
+    qw = be.upload_q4_blocks(wq)
+    for rows, entry in ((1, "gemv"), (2, "gemv"), (4, "gemv"), (12, "gemv"), (40, "gemm")):
+        x = synth.activations(rows, k, seed=21)
+        big_row = rows - 1
+        x[big_row, 5] = 1.0e5
+        y = torch.empty((rows, n), dtype=torch.float32, device="cuda")
+        if entry == "gemv":
+            be.gemv_batch(dev(x), qw, y, rows, n, k)
+        else:
+            be.dispatch_gemm(dev(x), 0, qw, y, 0, rows, n, k)
+        got = host(y)
+        ref = oracle.gemm_f32(x, wq, n, k)
+        if rows == 1:
+            assert np.isfinite(got).all() and rel_err(got, ref) <= REL_TOL
+            continue
+        # the row that holds the value: either served faithfully (kernels that keep f32 activations) or
+        # non-finite as a whole, never a finite wrong number
+        if np.isfinite(got[big_row]).all():
+            assert rel_err(got[big_row], ref[big_row]) <= REL_TOL, (rows, entry)
+        else:
+            assert not np.isfinite(got[big_row]).any(), (rows, entry)
+            assert entry == "gemm" or rows >= 3, "one and two rows keep f32 range"
+        others = [r for r in range(rows) if r != big_row]
+        assert np.isfinite(got[others]).all() and rel_err(got[others], ref[others]) <= REL_TOL, (rows, entry)
+
+
 # --------------------------------------------------------------------------- MoE
 def test_moe_route_matches_oracle(be):
     lg = synth.router_logits(16, 64, seed=0)

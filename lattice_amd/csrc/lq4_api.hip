@@ -43,6 +43,7 @@ struct lq4_ctx {
     hipEvent_t state_event;  // recorded on the previous stream when a call arrives on another one
     int lm_head_mode;        // lq4_set_lm_head_mode
     int gemm_kernel;         // lq4_set_gemm_kernel
+    bool gemv_dma;           // one-token GEMVs without LoRA take the LDS-ring kernel (LQ4_GEMV_DMA)
     lq4_path_counters counters;
 };
 
@@ -233,6 +234,7 @@ int lq4_ctx_create(int device_ordinal, lq4_ctx** out) {
     }
     c->lm_head_mode = LQ4_LM_HEAD_TWO_LAUNCHES;  // measured faster: see lq4_set_lm_head_mode in the header
     c->gemm_kernel = gemm_kernel_choice_default();
+    c->gemv_dma = getenv("LQ4_GEMV_DMA") && atoi(getenv("LQ4_GEMV_DMA")) != 0;
     // LQ4_LORA_SPIN_LIMIT: 0 makes every weight wave compute A.x itself (the path a wave takes when
     // the producers are late), "off" restores the separate A.x launch
     c->lora_spin_limit = 512;
@@ -425,6 +427,9 @@ int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
         if (rc) return rc;
         launch_gemm_skinny(wp, n, k, x_dev, 0, batch, y_dev, ep, ctx->moe_scratch, s);
         ctx->counters.gemm++;
+    } else if (batch == 1 && !ep.rank && ctx->gemv_dma && gemv_dma_serves(n, k, ctx->cu_count)) {
+        launch_gemv_dma(wp, n, k, x_dev, y_dev, ctx->cu_count, s);
+        ctx->counters.gemv++;
     } else {
         launch_gemv(wp, n, k, x_dev, k, batch, y_dev, n, ep, s);
         ctx->counters.gemv++;

@@ -424,6 +424,19 @@ int lq4_probe_read(lq4_ctx* ctx, const void* p_dev, size_t nbytes, void* stream)
 int lq4_probe_read_config(lq4_ctx* ctx, const void* p_dev, size_t nbytes, uint32_t workgroups, uint32_t bytes_in_flight,
                           int strided, int nontemporal, void* stream);
 
+/* Which kernel serves y = W . x for one token without LoRA (lq4_gemv at batch 1, the GEMV of
+ * lq4_lm_head_topk in two launches, a one-row step of lq4_gemv_chain without LoRA).  Per context; a new
+ * context starts from the environment variable LQ4_GEMV_KERNEL, else AUTO.
+ *   AUTO        by shape: the LDS-ring kernel where it is measured faster (rows of at least 2048 weights and
+ *               64 MB of weights, or rows of at least 10240 weights and 32 MB), else the lane-owns-block kernel
+ *   LANE_BLOCKS always the kernel in which each lane loads its own blocks into registers
+ *   LDS_RING    the kernel that streams whole 1280-byte slabs into a per-wave ring of LDS slots wherever the
+ *               shape fits it (K <= 24576), else the other one
+ * Both accumulate a row's blocks in the same order inside a slab; results agree to the contract's tolerance
+ * and are bit-identical for rows of one slab (K <= 2048).  No counterpart in the reference. */
+enum { LQ4_GEMV_KERNEL_AUTO = 0, LQ4_GEMV_KERNEL_LANE_BLOCKS = 1, LQ4_GEMV_KERNEL_LDS_RING = 2 };
+int lq4_set_gemv_kernel(lq4_ctx* ctx, int which);
+
 /* Tuning/test hook, per context (a new context starts from the environment variable LQ4_GEMM_KERNEL,
  * else 0): 0 = lq4_gemm picks its kernel by shape (default), 1 = always
  * the LDS-staged tile kernel, 2 = always the weights-in-registers kernel, 3 = always the

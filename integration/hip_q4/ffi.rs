@@ -416,6 +416,8 @@ extern "C" {
         stream: *mut c_void,
     ) -> c_int;
     pub fn lq4_probe_copy(ctx: *mut Lq4Ctx, src: *const c_void, dst: *mut c_void, nbytes: usize, stream: *mut c_void) -> c_int;
+    /// 0 = by shape, 1 = lane-owns-block kernel, 2 = LDS-ring kernel wherever the shape fits.
+    pub fn lq4_set_gemv_kernel(ctx: *mut Lq4Ctx, which: c_int) -> c_int;
     pub fn lq4_set_gemm_kernel(ctx: *mut Lq4Ctx, which: c_int) -> c_int;
     pub fn lq4_get_path_counters(ctx: *const Lq4Ctx, out: *mut Lq4PathCounters) -> c_int;
 

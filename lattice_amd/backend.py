@@ -50,6 +50,7 @@ EXPORTS = [
     "lq4_probe_read",
     "lq4_probe_read_config",
     "lq4_probe_copy",
+    "lq4_set_gemv_kernel",
     "lq4_set_gemm_kernel",
     "lq4_residual_add_rmsnorm", "lq4_silu_mul", "lq4_add_and_copy", "lq4_gemv_fused", "lq4_gemv_fused_batch",
     "lq4_lm_head_topk_static",
@@ -82,6 +83,7 @@ LQ4_PRO_NONE, LQ4_PRO_ADD_RMSNORM, LQ4_PRO_SILU_MUL = 0, 1, 2
 LQ4_EPI_NONE, LQ4_EPI_ADD_RESIDUAL, LQ4_EPI_SILU_MUL_PAIRS = 0, 1, 2
 CHAIN_MAX_STEPS = 16
 LM_HEAD_ONE_LAUNCH, LM_HEAD_TWO_LAUNCHES = 0, 1  # lq4_set_lm_head_mode
+GEMV_KERNEL_AUTO, GEMV_KERNEL_LANE_BLOCKS, GEMV_KERNEL_LDS_RING = 0, 1, 2  # lq4_set_gemv_kernel
 
 
 class GemvFusion(C.Structure):
@@ -141,6 +143,7 @@ def load_library() -> C.CDLL:
         "lq4_probe_read": (C.c_int, [vp, vp, C.c_size_t, vp]),
         "lq4_probe_read_config": (C.c_int, [vp, vp, C.c_size_t, C.c_uint32, C.c_uint32, C.c_int, C.c_int, vp]),
         "lq4_probe_copy": (C.c_int, [vp, vp, vp, C.c_size_t, vp]),
+        "lq4_set_gemv_kernel": (C.c_int, [vp, C.c_int]),
         "lq4_set_gemm_kernel": (C.c_int, [vp, C.c_int]),
         "lq4_residual_add_rmsnorm": (C.c_int, [vp, vp, vp, vp, C.c_uint32, C.c_uint32, C.c_float, vp, vp, vp]),
         "lq4_silu_mul": (C.c_int, [vp, vp, C.c_uint32, C.c_uint32, vp, C.c_uint32, vp]),
@@ -293,6 +296,11 @@ class HipQ4Backend:
         """Grows the context's scratch ahead of time (growing it allocates, which a call under HIP
         graph capture refuses to do)."""
         _check(self.lib.lq4_ctx_reserve_scratch(self.ctx, int(nbytes)))
+
+    def set_gemv_kernel(self, which: int):
+        """Which kernel serves a one-token GEMV without LoRA: 0 = by shape, 1 = each lane loads its own
+        blocks, 2 = weights streamed into a per-wave ring of LDS slots wherever the shape fits."""
+        _check(self.lib.lq4_set_gemv_kernel(self.ctx, int(which)))
 
     def set_gemm_kernel(self, which: int):
         """0 = pick the prefill kernel by shape, 1 = LDS-staged tile, 2 = weights in registers,

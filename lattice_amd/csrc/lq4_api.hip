@@ -43,7 +43,7 @@ struct lq4_ctx {
     hipEvent_t state_event;  // recorded on the previous stream when a call arrives on another one
     int lm_head_mode;        // lq4_set_lm_head_mode
     int gemm_kernel;         // lq4_set_gemm_kernel
-    bool gemv_dma;           // one-token GEMVs without LoRA take the LDS-ring kernel (LQ4_GEMV_DMA)
+    int gemv_kernel;         // lq4_set_gemv_kernel: which kernel serves a plain one-token GEMV
     lq4_path_counters counters;
 };
 
@@ -234,7 +234,8 @@ int lq4_ctx_create(int device_ordinal, lq4_ctx** out) {
     }
     c->lm_head_mode = LQ4_LM_HEAD_TWO_LAUNCHES;  // measured faster: see lq4_set_lm_head_mode in the header
     c->gemm_kernel = gemm_kernel_choice_default();
-    c->gemv_dma = getenv("LQ4_GEMV_DMA") && atoi(getenv("LQ4_GEMV_DMA")) != 0;
+    c->gemv_kernel = getenv("LQ4_GEMV_KERNEL") ? atoi(getenv("LQ4_GEMV_KERNEL")) : 0;
+    if (c->gemv_kernel < 0 || c->gemv_kernel > 2) c->gemv_kernel = 0;
     // LQ4_LORA_SPIN_LIMIT: 0 makes every weight wave compute A.x itself (the path a wave takes when
     // the producers are late), "off" restores the separate A.x launch
     c->lora_spin_limit = 512;
@@ -383,6 +384,22 @@ int lq4_lora_free(lq4_lora* l) {
 static int ensure_scratch(lq4_ctx* ctx, size_t bytes, hipStream_t stream);
 static int enter_shared_state(lq4_ctx* ctx, hipStream_t stream);
 
+// y = W . x for one token without LoRA: the LDS-ring kernel where it is the faster one (or where the context asks
+// for it and the shape fits), else the lane-owns-block kernel.  Both give the same contract.
+static void plain_gemv_one_token(lq4_ctx* ctx, const uint8_t* wp, uint32_t n, uint32_t k, const float* x, float* y,
+                                 hipStream_t s) {
+    const bool ring = ctx->gemv_kernel == LQ4_GEMV_KERNEL_LDS_RING
+                          ? gemv_dma_serves(n, k, ctx->cu_count)
+                          : ctx->gemv_kernel == LQ4_GEMV_KERNEL_AUTO && gemv_dma_pays(n, k, ctx->cu_count);
+    if (ring) {
+        launch_gemv_dma(wp, n, k, x, y, ctx->cu_count, s);
+    } else {
+        const LoraEpilogue none{};
+        launch_gemv(wp, n, k, x, k, 1, y, n, none, s);
+    }
+    ctx->counters.gemv++;
+}
+
 int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
              const float* x_dev, uint32_t batch, float* y_dev, const lq4_lora* lora, float lora_scale,
              void* stream) {
@@ -427,9 +444,8 @@ int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
         if (rc) return rc;
         launch_gemm_skinny(wp, n, k, x_dev, 0, batch, y_dev, ep, ctx->moe_scratch, s);
         ctx->counters.gemm++;
-    } else if (batch == 1 && !ep.rank && ctx->gemv_dma && gemv_dma_serves(n, k, ctx->cu_count)) {
-        launch_gemv_dma(wp, n, k, x_dev, y_dev, ctx->cu_count, s);
-        ctx->counters.gemv++;
+    } else if (batch == 1 && !ep.rank) {
+        plain_gemv_one_token(ctx, wp, n, k, x_dev, y_dev, s);
     } else {
         launch_gemv(wp, n, k, x_dev, k, batch, y_dev, n, ep, s);
         ctx->counters.gemv++;
@@ -692,6 +708,8 @@ void small_batch_gemv(lq4_ctx* ctx, const uint8_t* wp, uint32_t n, uint32_t k, c
     if (rows >= 9 || (rows >= 5 && n < 8192 && !narrow && weights >= 6000000)) {
         launch_gemm_skinny(wp, n, k, x, 0, rows, y, none, pack, s);
         ctx->counters.gemm++;
+    } else if (rows == 1) {
+        plain_gemv_one_token(ctx, wp, n, k, x, y, s);
     } else {
         launch_gemv(wp, n, k, x, k, rows, y, n, none, s);
         ctx->counters.gemv++;
@@ -990,10 +1008,8 @@ int lm_head_topk_common(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offs
     } else {
         const size_t logits_bytes = (static_cast<size_t>(vocab) * sizeof(float) + 255) / 256 * 256;
         float* logits = reinterpret_cast<float*>(base);
-        const LoraEpilogue none{};
-        launch_gemv(wp, vocab, k, x_dev, k, 1, logits, vocab, none, s);
+        plain_gemv_one_token(ctx, wp, vocab, k, x_dev, logits, s);
         launch_topk(logits, vocab, top_k, base + logits_bytes, ctx->topk_ticket, out_logits_dev, out_ids_dev, s);
-        ctx->counters.gemv++;
         ctx->counters.topk++;
     }
     LQ4_HIP(hipGetLastError());
@@ -1573,6 +1589,14 @@ int lq4_gemv_q3(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint
     if (batch > kMaxGemvBatch)
         return fail(LQ4_E_INVALID, "lq4_gemv_q3 batch %u above %d; use lq4_gemm_q3", batch, kMaxGemvBatch);
     return lq4_gemm_q3(ctx, w, w_extra_offset, n, k, x_dev, LQ4_F32, batch, y_dev, stream);
+}
+
+int lq4_set_gemv_kernel(lq4_ctx* ctx, int which) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    if (which < LQ4_GEMV_KERNEL_AUTO || which > LQ4_GEMV_KERNEL_LDS_RING)
+        return fail(LQ4_E_INVALID, "gemv kernel choice must be 0..2");
+    ctx->gemv_kernel = which;
+    return LQ4_OK;
 }
 
 int lq4_set_gemm_kernel(lq4_ctx* ctx, int which) {

@@ -14,19 +14,40 @@
 // The compiler's wait-count pass knows nothing of these loads, so the waits are written by hand: a wave's loads
 // return in the order they were issued, `s_waitcnt vmcnt(N)` with N = the number of load instructions issued
 // after the slot at the head of the ring (two per slot) is exactly "the head has landed".  The y stores raise the
-// same counter and may complete early, which can only make a wait longer than needed.  The activations are loaded
-// by inline assembly too (ahead of the first weight request, so they are waited for alone) and staged in LDS as
-// in the lane-owns-block kernel (lq4_b1_dev.hpp: per-block scaled fixed point, eight-wide 4-bit dot products).
+// same counter and may complete early, which can only make a wait longer than needed.  The activations take the
+// same road (requested ahead of the first weights, so they are waited for alone): each wave brings its 512-element
+// piece of x into the staging area as raw floats, reads it back, and after a barrier the pieces are staged over it
+// as in the lane-owns-block kernel (lq4_b1_dev.hpp: per-block scaled fixed point, eight-wide 4-bit dot products).
+// No load of this kernel has a register as its destination.  That is deliberate: a register which inline assembly
+// fills "later" is not safe against the register allocator (a copy it inserts between the load and the wait reads
+// the old contents, and it may hand the original register to another value that the arriving data then destroys;
+// both happened here, the second as a memory fault through a clobbered address offset).
 //
-// Every wave takes one run of consecutive rows, so its slots are one run of memory and the address of the next
-// request is a running pointer.  The ring has a compile-time depth D and the loop is unrolled D times: the slot a
+// Work split.  A workgroup (one per CU) owns a run of consecutive rows, i.e. a run of slots that is also one run of
+// memory, and its sixteen waves cut that run into sixteen equal pieces to within one slot, wherever the row
+// boundaries fall: 5120 rows of nine slots are twenty rows a CU, which dealt out as whole rows would leave four
+// waves with eighteen slots and twelve with nine.  A wave's slots are again one run of memory, so the address of
+// the next request is a running pointer.  A row that starts in one wave and ends in a later one is finished by the
+// wave it starts in: every wave leaves the sum of the row that was already under way at its first slot (at most
+// one such row) in LDS, and after a barrier the starting wave adds those to its own part in wave order.  The ring has a compile-time depth D and the loop is unrolled D times: the slot a
 // wave has just emptied is the one its next request fills, so every LDS offset is a constant, the wait in the
 // steady state is the constant vmcnt(2 (D - 1)), and what is left per slot is a dozen scalar instructions.  (A
 // first version with run-time ring positions and a wait chosen by a switch spent ~80 scalar instructions and a
 // dozen branches per slot and was 10-15 % slower than the lane-owns-block kernel: a CU issues one scalar
-// instruction per cycle for all its waves.)  Shapes whose rows are 1, 2 or 3 whole slabs keep the lane's blocks of
-// x in registers for the whole launch; other shapes (a short last slab, longer rows) re-read them from LDS.
+// instruction per cycle for all its waves.)  The block of slot s + 1 is read out of LDS before the arithmetic of
+// slot s, so that read's latency hides behind ~50 vector instructions, and the refill of slot s is requested after
+// them, when its words have long been in registers.  Rows of up to three slabs keep the lane's blocks of x in
+// registers for the whole launch (104 bytes a lane and slab: read from LDS for every slot they cost six times the
+// LDS traffic of the weights themselves); the slab at an unrolled position then has to be a constant, so the loop
+// exists once per slab a wave's piece can start at.  Longer rows re-read their blocks from LDS slot by slot.
+//
+// One workgroup of sixteen waves per CU: the activations are staged once per CU, by as many waves as the vector
+// has 512-element pieces (the others skip the staging code altogether, which on short rows is most of what a
+// wave of the lane-owns-block kernel executes).
+#include <atomic>
 #include "lq4_b1_dev.hpp"
+
+#include <type_traits>
 
 namespace lq4 {
 
@@ -47,22 +68,16 @@ __device__ __forceinline__ float as_f32(uint32_t bits) { return __builtin_bit_ca
 __device__ __forceinline__ void dma16(uint32_t lds, const LQ4_GLOBAL void* base, uint32_t off) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds), "v"(off), "s"(base) : "memory");
 }
+// The same for data every workgroup reads (the activations): left to the caches.
+__device__ __forceinline__ void dma16_shared(uint32_t lds, const LQ4_GLOBAL void* base, uint32_t off) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(off), "s"(base) : "memory");
+}
 __device__ __forceinline__ void dma4(uint32_t lds, const LQ4_GLOBAL void* base, uint32_t off) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2 nt" ::"s"(lds), "v"(off), "s"(base) : "memory");
-}
-// 32 bytes (eight floats) as two loads into registers
-__device__ __forceinline__ void ld_32b(u32x4& lo, u32x4& hi, const LQ4_GLOBAL void* base, uint32_t off) {
-    asm volatile("global_load_dwordx4 %0, %2, %3\n\tglobal_load_dwordx4 %1, %2, %3 offset:16"
-                 : "=&v"(lo), "=&v"(hi)
-                 : "v"(off), "s"(base));
 }
 template <int N>
 __device__ __forceinline__ void wait_vm() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-template <typename T>
-__device__ __forceinline__ void tie(T& v) {
-    asm volatile("" : "+v"(v));
 }
 // The same loads for a subset of the lanes (`mask`, one bit a lane, not empty): a row's short last slab.
 __device__ __forceinline__ void dma16_masked(uint32_t lds, const LQ4_GLOBAL void* base, uint32_t off, uint64_t mask) {
@@ -80,17 +95,19 @@ __device__ __forceinline__ void dma4_masked(uint32_t lds, const LQ4_GLOBAL void*
                  : "memory");
 }
 
-// WAVES: waves per workgroup (every workgroup stages the whole activation vector: more waves share one staging on
-// longer rows).  XR: 8-activation units a thread stages (K <= 8 * 64 * WAVES * XR).  D: slots in a wave's ring.
-// SLABS: 1..3 = rows of exactly that many whole slabs, the lane's blocks of x stay in registers (D is a multiple
-// of SLABS, so the slab at an unrolled position is known at compile time); 0 = any row length, x from LDS.
-template <int WAVES, int XR, int D, int SLABS>
-__global__ __launch_bounds__(WAVES * 64) void gemv_q4_dma(const uint8_t* __restrict__ w_, uint32_t n, uint32_t k,
-                                                           const float* __restrict__ x_, float* __restrict__ y) {
+// XR: 8-activation units a thread stages (K <= 8 * 1024 * XR).  D: slots in a wave's ring.
+// SLABS: 1..3 = rows of that many slabs (the last may be short), the lane's blocks of x stay in registers (D is a
+// multiple of SLABS); 0 = any row length, x from LDS.
+constexpr int kWaves = 16;
+template <int XR, int D, int SLABS>
+__global__ __launch_bounds__(kWaves * 64) void gemv_q4_dma(const uint8_t* __restrict__ w_, uint32_t n, uint32_t k,
+                                                            const float* __restrict__ x_, float* __restrict__ y) {
+    static_assert(D >= 3, "one slot in registers, one landed, at least one on its way");
     static_assert(SLABS == 0 || D % SLABS == 0, "the slab at an unrolled position must not depend on the round");
+    constexpr bool ONE_SLAB = SLABS == 1;
     extern __shared__ __attribute__((aligned(16))) uint32_t lds_raw[];
     lds_u32* const xs = (lds_u32*)lds_raw;
-    constexpr int T = WAVES * 64;
+    constexpr int T = kWaves * 64;
     const int tid = threadIdx.x, lane = tid & 63;
     const uint32_t nb = k / kBlockWeights;
     const uint32_t row_bytes = nb * kBlockBytes;
@@ -98,29 +115,47 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_dma(const uint8_t* __restr
     const uint32_t last_blocks = nb - (slabs - 1) * 64;  // blocks of a row's last slab
     const uint32_t last_bytes = last_blocks * kBlockBytes;
     const uint32_t wave = uniform(tid >> 6);
-    const uint32_t n_waves = gridDim.x * WAVES;
-    const uint32_t wid = uniform(blockIdx.x * WAVES + wave);
     const LQ4_GLOBAL uint8_t* const w = as_global(w_);
     const LQ4_GLOBAL float* const x = as_global(x_);
-    // the wave's ring: behind the staged activations
+    // LDS: the staged activations | one partial sum a wave | the waves' rings
     const uint32_t xs_dwords = nb * kXPitch;
-    lds_u32* const ring_ptr = xs + xs_dwords + wave * D * (kSlotBytes / 4);
+    LQ4_LDS float* const part = reinterpret_cast<LQ4_LDS float*>(xs + xs_dwords);
+    lds_u32* const ring_ptr = xs + xs_dwords + kWaves + wave * D * (kSlotBytes / 4);
     const uint32_t ring_addr = uniform(static_cast<uint32_t>(reinterpret_cast<size_t>(ring_ptr)));
 
     // ---- the activations first: requested before any weight so they can be waited for alone ----
+    // Each wave moves the 512-element pieces it will stage (2 KB of raw floats a piece) into the staging area,
+    // at the bytes they have in x.  A piece that reaches past the end of x is cut at 16 bytes (K is a multiple of 32).
     const uint32_t n_units = nb * 4;
-    u32x4 xlo[XR], xhi[XR];
+    const uint32_t xs_addr = uniform(static_cast<uint32_t>(reinterpret_cast<size_t>(xs)));
+    const uint32_t x_bytes = k * 4;
 #pragma unroll
     for (int i = 0; i < XR; ++i) {
-        const uint32_t u = tid + i * T < n_units ? tid + i * T : 0;
-        ld_32b(xlo[i], xhi[i], x, u * 32u);
+        const uint32_t piece = (i * T + wave * 64) * 32u;  // first byte
+        if (piece < x_bytes) {                           // uniform
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const uint32_t first = piece + h * 1024u;
+                if (first + 1024u <= x_bytes) {
+                    dma16_shared(xs_addr + first, x + first / 4, lane * 16u);
+                } else if (first < x_bytes) {
+                    const uint64_t m = __builtin_amdgcn_ballot_w64(first + lane * 16u < x_bytes);
+                    dma16_masked(xs_addr + first, x + first / 4, lane * 16u, m);
+                }
+            }
+        }
     }
 
-    // ---- this wave's rows: one run, the first n % n_waves waves take one row more ----
-    const uint32_t share = n / n_waves, extra = n - share * n_waves;
-    const uint32_t my_rows = share + (wid < extra ? 1u : 0u);
-    const uint32_t first_row = wid * share + (wid < extra ? wid : extra);
-    const uint32_t total = my_rows * slabs;  // slots
+    // ---- this wave's slots ----
+    // the workgroup's rows: one run, the first n % workgroups of them take one row more
+    const uint32_t share = n / gridDim.x, extra = n - share * gridDim.x;
+    const uint32_t wg_rows = share + (blockIdx.x < extra ? 1u : 0u);
+    const uint32_t wg_first = blockIdx.x * share + (blockIdx.x < extra ? blockIdx.x : extra);
+    const uint32_t wg_slots = wg_rows * slabs;
+    auto piece_start = [&](uint32_t j) { return static_cast<uint32_t>(static_cast<uint64_t>(j) * wg_slots / kWaves); };
+    const uint32_t s0 = uniform(piece_start(wave)), s1 = uniform(piece_start(wave + 1));
+    const uint32_t total = s1 - s0;
+    const uint32_t row0 = uniform(s0 / slabs), slab0 = s0 - row0 * slabs;  // where the first slot lies
     // a short last slab: 20 * blocks bytes as whole 16-byte pieces, then the dwords behind them (fewer than four,
     // or what is left past 1024 bytes); lane 0 always takes part in the second load so that it is a load
     // instruction on every path (the waits count them)
@@ -128,13 +163,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_dma(const uint8_t* __restr
     const uint32_t rest = (last_bytes - n16 * 16) / 4;
     const uint64_t mask16 = __builtin_amdgcn_ballot_w64(static_cast<uint32_t>(lane) < n16);
     const uint64_t mask4 = __builtin_amdgcn_ballot_w64(static_cast<uint32_t>(lane) < (rest ? rest : 1u));
-    const bool short_last = SLABS == 0 && last_blocks != 64;
+    const bool short_last = last_blocks != 64;
 
-    const LQ4_GLOBAL uint8_t* rq_ptr = w + static_cast<uint64_t>(first_row) * row_bytes;  // the next slot to request
-    uint32_t rq_slab = 0;                                                                   // its slab (SLABS == 0)
+    // the next slot to request: its address and its slab
+    const LQ4_GLOBAL uint8_t* rq_ptr = w + static_cast<uint64_t>(wg_first + row0) * row_bytes + slab0 * static_cast<uint32_t>(kSlotBytes);
+    uint32_t rq_slab = slab0;
     const uint32_t off16 = lane * 16u, off4 = lane * 4u;
-    auto request_into = [&](uint32_t at) {  // `at`: LDS byte address of the slot
-        if (short_last && rq_slab + 1 == slabs) {
+    auto request_next = [&](int pos) {  // `pos`: ring position
+        const uint32_t at = ring_addr + pos * kSlotBytes;
+        const bool last = ONE_SLAB || rq_slab + 1 == slabs;
+        if (short_last && last) {
             dma16_masked(at, rq_ptr, off16, mask16);
             dma4_masked(at + n16 * 16, rq_ptr + (rest ? n16 * 16 : 0u), off4, mask4);
             rq_ptr += last_bytes;
@@ -143,127 +181,192 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_dma(const uint8_t* __restr
             dma4(at + 1024, rq_ptr + 1024, off4);
             rq_ptr += kSlotBytes;
         }
-        if (SLABS == 0) rq_slab = rq_slab + 1 == slabs ? 0 : rq_slab + 1;
+        if (!ONE_SLAB) rq_slab = last ? 0 : rq_slab + 1;
     };
+    // Two slots a wave now, the rest of the ring once the activations are staged: a CU accepts requests only as fast
+    // as earlier ones are answered once a few dozen KB are on their way, and a wave stuck issuing its whole ring
+    // would reach the staging barriers only when most of that data has arrived.
+    constexpr int E = 2;
     uint32_t to_request = total;
 #pragma unroll
-    for (int i = 0; i < D; ++i) {
+    for (int i = 0; i < E; ++i) {
         if (to_request) {  // uniform
-            request_into(ring_addr + i * kSlotBytes);
+            request_next(i);
             --to_request;
         }
     }
 
     // ---- stage x: the activation loads are older than every weight request ----
-    if (total >= static_cast<uint32_t>(D)) wait_vm<2 * D>();
+    if (total >= static_cast<uint32_t>(E)) wait_vm<2 * E>();
     else wait_vm<0>();
+    float4 xa[XR], xc[XR];
 #pragma unroll
     for (int i = 0; i < XR; ++i) {
-        tie(xlo[i]);
-        tie(xhi[i]);
-        const bool act = tid + i * T < n_units;
-        if (XR == 1 || static_cast<uint32_t>(i * T) < n_units) {
-            const u32x4 lo = xlo[i], hi = xhi[i];
-            stage_x8(xs, act ? tid + i * T : 0, make_float4(as_f32(lo.x), as_f32(lo.y), as_f32(lo.z), as_f32(lo.w)),
-                     make_float4(as_f32(hi.x), as_f32(hi.y), as_f32(hi.z), as_f32(hi.w)), act);
+        xa[i] = xc[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if ((i * T + wave * 64) * 32u < x_bytes) {  // uniform: this wave's own piece, which it has just waited for
+            const uint32_t u = tid + i * T < n_units ? tid + i * T : 0;
+            typedef float f32x4 __attribute__((ext_vector_type(4)));
+            const LQ4_LDS f32x4* const raw = reinterpret_cast<const LQ4_LDS f32x4*>(xs + u * 8);
+            const f32x4 lo = raw[0], hi = raw[1];
+            xa[i] = make_float4(lo.x, lo.y, lo.z, lo.w);
+            xc[i] = make_float4(hi.x, hi.y, hi.z, hi.w);
+        }
+    }
+    barrier_lds();  // every piece has been read: the staged form may overwrite the raw one
+#pragma unroll
+    for (int i = 0; i < XR; ++i) {
+        if ((i * T + wave * 64) * 32u < x_bytes) {  // uniform
+            const bool act = tid + i * T < n_units;
+            stage_x8(xs, act ? tid + i * T : 0, xa[i], xc[i], act);
         }
     }
     barrier_lds();
+#pragma unroll
+    for (int i = E; i < D; ++i) {
+        if (to_request) {  // uniform
+            request_next(i);
+            --to_request;
+        }
+    }
 
     // ---- the arithmetic: round after round over the ring ----
     constexpr int NX = SLABS ? SLABS : 1;
     XBlock xb[NX];
+    if (SLABS) {
 #pragma unroll
-    for (int sl = 0; sl < NX; ++sl) {
-        const uint32_t blk = sl * 64 + lane;
-        load_xblock(xs, blk < nb ? blk : nb - 1, xb[sl]);
-    }
-    float acc = 0.0f;
-    uint32_t left = total, cs_slab = 0, row = first_row;
-    const lds_u32* const my_block = ring_ptr + 5 * lane;  // the lane's block in slot 0: byte 20 l
-    while (left) {
-#pragma unroll
-        for (int i = 0; i < D; ++i) {
-            if (left == 0) break;  // uniform
-            if (to_request) wait_vm<2 * (D - 1)>();  // the ring is full behind the head
-            else wait_vm<0>();
-            const lds_u32* const slot = my_block + i * (kSlotBytes / 4);
-            Q4BlockRaw wb;
-            wb.sb = slot[0];
-            wb.q[0] = slot[1]; wb.q[1] = slot[2]; wb.q[2] = slot[3]; wb.q[3] = slot[4];
-            bool live = true;
-            if (SLABS == 0) {
-                const uint32_t blk_raw = cs_slab * 64 + lane;
-                live = blk_raw < nb;
-                if (slabs > 1) load_xblock(xs, live ? blk_raw : nb - 1, xb[0]);
-                // a lane past the end of the row has read what the slot held before: scale and bias of zero,
-                // whatever bits they were (a stale bias may be an infinity, and zero times that is not zero)
-                wb.sb = live ? wb.sb : 0u;
-            }
-            // The slot is free again once its words are in registers: the empty statement makes the compiler wait
-            // for those reads here, ahead of the request that refills the slot.
-            asm volatile("" : "+v"(wb.sb), "+v"(wb.q[0]), "+v"(wb.q[1]), "+v"(wb.q[2]), "+v"(wb.q[3]));
-            if (to_request) {
-                request_into(ring_addr + i * kSlotBytes);
-                --to_request;
-            }
-            acc = block_fma(wb, xb[SLABS ? i % NX : 0], live, acc);
-            bool row_done;
-            if (SLABS) {
-                row_done = i % NX == NX - 1;
-            } else {
-                row_done = cs_slab + 1 == slabs;
-                cs_slab = row_done ? 0 : cs_slab + 1;
-            }
-            if (row_done) {
-                const float v = segment_sum<64>(acc);
-                acc = 0.0f;
-                if (lane == 63) y[row] = v;
-                ++row;
-            }
-            --left;
+        for (int sl = 0; sl < NX; ++sl) {
+            const uint32_t blk = sl * 64 + lane;
+            load_xblock(xs, blk < nb ? blk : nb - 1, xb[sl]);
         }
     }
+    const lds_u32* const my_block = ring_ptr + 5 * lane;  // the lane's block in position 0: byte 20 l
+    auto read_block = [&](int pos, Q4BlockRaw& wb) {
+        const lds_u32* const slot = my_block + pos * (kSlotBytes / 4);
+        wb.sb = slot[0];
+        wb.q[0] = slot[1]; wb.q[1] = slot[2]; wb.q[2] = slot[3]; wb.q[3] = slot[4];
+    };
+    float acc = 0.0f;
+    uint32_t left = total, cs_slab = slab0, row = wg_first + row0;
+    bool in_head = slab0 != 0;  // the row under way at the first slot started in an earlier wave
+    // S0: the slab of the piece's first slot when rows have SLABS slabs (a constant inside each copy of the loop)
+    auto run = [&](auto s0_const) {
+        constexpr int S0 = decltype(s0_const)::value;
+        Q4BlockRaw cur, nxt;
+        if (left) {
+            if (total >= static_cast<uint32_t>(D)) wait_vm<2 * (D - 1)>();
+            else wait_vm<0>();
+            read_block(0, cur);
+        }
+        while (left) {
+#pragma unroll
+            for (int i = 0; i < D; ++i) {
+                if (left == 0) break;  // uniform
+                // the slot behind this one out of LDS now: its read hides behind this slot's arithmetic
+                if (left > 1) {
+                    if (to_request) wait_vm<2 * (D - 2)>();  // the ring is full behind this slot
+                    else wait_vm<0>();
+                    read_block((i + 1) % D, nxt);
+                }
+                const int slab_c = SLABS ? (S0 + i) % NX : 0;  // a constant once the loop is unrolled
+                bool live = true;
+                bool last_slab;
+                if constexpr (SLABS != 0) {
+                    last_slab = slab_c == SLABS - 1;
+                    if (last_slab) live = static_cast<uint32_t>(lane) < last_blocks;
+                } else {
+                    last_slab = cs_slab + 1 == slabs;
+                    const uint32_t blk_raw = cs_slab * 64 + lane;
+                    live = blk_raw < nb;
+                    load_xblock(xs, live ? blk_raw : nb - 1, xb[0]);
+                    cs_slab = last_slab ? 0 : cs_slab + 1;
+                }
+                // a lane past the end of the row has read what the slot held before: scale and bias of zero,
+                // whatever bits they were (a stale bias may be an infinity, and zero times that is not zero)
+                if (short_last && last_slab) cur.sb = live ? cur.sb : 0u;
+                acc = block_fma(cur, xb[slab_c], live, acc);
+                // the slot's words went into registers a slot ago: its place in the ring can be filled again
+                if (to_request) {
+                    request_next(i);
+                    --to_request;
+                }
+                if (last_slab) {
+                    const float v = segment_sum<64>(acc);
+                    acc = 0.0f;
+                    if (in_head) {  // uniform: the tail of a row that an earlier wave finishes
+                        if (lane == 63) part[wave] = v;
+                        in_head = false;
+                    } else if (lane == 63) {
+                        y[row] = v;
+                    }
+                    ++row;
+                }
+                cur = nxt;
+                --left;
+            }
+        }
+        if (SLABS) cs_slab = (slab0 + total) % NX;  // the slab the next slot would have had
+    };
+    if (SLABS <= 1 || slab0 == 0) run(std::integral_constant<int, 0>{});
+    else if (slab0 == 1) run(std::integral_constant<int, 1>{});
+    else run(std::integral_constant<int, SLABS == 3 ? 2 : 0>{});
     wait_vm<0>();  // nothing of this wave is on its way when it ends
+    if (ONE_SLAB) return;
+    // ---- rows that straddle waves ----
+    const bool open_row = total != 0 && cs_slab != 0;  // the last slot did not end its row
+    float own = 0.0f;
+    if (open_row) {
+        own = segment_sum<64>(acc);
+        if (in_head && lane == 63) part[wave] = own;  // the whole piece lies inside a row begun earlier
+    }
+    barrier_lds();
+    if (open_row && !in_head) {
+        // this wave began the row: the pieces behind it, in wave order, until the one that ends the row
+        const uint32_t row_end = (row - wg_first + 1) * slabs;  // first slot of the next row
+        for (uint32_t j = wave + 1; j < static_cast<uint32_t>(kWaves); ++j) {
+            const uint32_t b = piece_start(j), e = piece_start(j + 1);
+            if (b >= row_end) break;
+            if (e > b) own += part[j];
+        }
+        if (lane == 63) y[row] = own;
+    }
 }
 
 struct DmaPlan {
-    uint32_t waves, depth, slabs, grid;
+    uint32_t xr, depth, slabs, grid;
     size_t lds;
 };
 
-// One entry per instantiation: waves per workgroup, workgroups per CU, ring depth.
+// Which instantiation serves a row length: ring depth by what LDS leaves beside the staged activations.
 bool plan_dma(uint32_t n, uint32_t k, uint32_t cu_count, DmaPlan* out) {
     const uint32_t nb = k / kBlockWeights;
-    const size_t xs_bytes = static_cast<size_t>(nb) * kXPitch * 4;
+    const size_t fixed = static_cast<size_t>(nb) * kXPitch * 4 + kWaves * 4;
     DmaPlan p;
-    if (nb == 64) { p.waves = 4; p.depth = 6; p.slabs = 1; }
-    else if (nb == 128) { p.waves = 8; p.depth = 4; p.slabs = 2; }
-    else if (nb == 192) { p.waves = 16; p.depth = 6; p.slabs = 3; }
-    else if (k <= 2048) { p.waves = 4; p.depth = 4; p.slabs = 0; }
-    else if (k <= 8192) { p.waves = 8; p.depth = 4; p.slabs = 0; }
-    else if (k <= 24576) { p.waves = 16; p.depth = 3; p.slabs = 0; }
-    else return false;
-    const uint32_t wg_per_cu = 16 / p.waves;
-    p.lds = xs_bytes + static_cast<size_t>(p.waves) * p.depth * kSlotBytes;
-    if (p.lds * wg_per_cu > 160 * 1024) return false;
-    // every wave resident, rows dealt evenly; fewer workgroups when there are fewer rows than waves
-    const uint32_t wgs_resident = cu_count * wg_per_cu;
-    const uint32_t wgs_needed = (n + p.waves - 1) / p.waves;
-    p.grid = wgs_needed < wgs_resident ? wgs_needed : wgs_resident;
+    p.slabs = nb <= 192 ? (nb + 63) / 64 : 0;
+    p.xr = k <= 8192 ? 1 : 3;
+    p.depth = 6;
+    if (fixed + static_cast<size_t>(kWaves) * 6 * kSlotBytes > 160 * 1024) p.depth = 3;
+    p.lds = fixed + static_cast<size_t>(kWaves) * p.depth * kSlotBytes;
+    if (k > 24576 || p.lds > 160 * 1024) return false;
+    // one workgroup per CU, rows dealt evenly; fewer workgroups when there are fewer rows than CUs
+    p.grid = n < cu_count ? n : cu_count;
     *out = p;
     return true;
 }
 
-template <int WAVES, int XR, int D, int SLABS>
+template <int XR, int D, int SLABS>
 void launch_one(const DmaPlan& p, const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, hipStream_t stream) {
-    static bool attr_set = false;
-    if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_dma<WAVES, XR, D, SLABS>),
+    static std::atomic<uint64_t> attr_set{0};  // one bit a device: the attribute belongs to the device's copy of the code
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    const uint64_t bit = 1ull << (dev & 63);
+    if (!(attr_set.load(std::memory_order_relaxed) & bit)) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_dma<XR, D, SLABS>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        attr_set = true;
+        attr_set.fetch_or(bit, std::memory_order_relaxed);
     }
-    hipLaunchKernelGGL((gemv_q4_dma<WAVES, XR, D, SLABS>), dim3(p.grid), dim3(WAVES * 64), p.lds, stream, w, n, k, x, y);
+    // at least half a CU's LDS, so that the workgroups spread one to a CU
+    const size_t lds = p.lds < 96 * 1024 ? 96 * 1024 : p.lds;
+    hipLaunchKernelGGL((gemv_q4_dma<XR, D, SLABS>), dim3(p.grid), dim3(kWaves * 64), lds, stream, w, n, k, x, y);
 }
 
 }  // namespace
@@ -273,15 +376,27 @@ bool gemv_dma_serves(uint32_t n, uint32_t k, uint32_t cu_count) {
     return n != 0 && plan_dma(n, k, cu_count, &p);
 }
 
+// Measured against the lane-owns-block kernel on 256 CUs (us, that kernel -> this one): 32768 x 2048 (42 MB) 10.7 ->
+// 10.8; 65536 x 2048 (84 MB) 19.2 -> 17.4; 248320 x 2048 62.1 -> 54.3; 32768 x 4096 18.1 -> 16.7; 17408 x 5120 (56 MB)
+// 13.3 -> 13.5; 151936 x 5120 94.4 -> 82.7; 16384 x 8192 19.1 -> 18.0; 8192 x 12288 (63 MB) 15.5 -> 13.2; 4096 x 14336
+// (37 MB) 11.2 -> 9.6; 5120 x 17408 16.8 -> 13.5; 2048 x 17408 (22 MB) 8.9 -> 9.1.  Behind for every row shorter than
+// one slab (131072 x 1024 18.9 -> 21.9: the other kernel puts two rows side by side in a wave) and for the decode
+// layer's matrices (2..16 MB, 1.0 us behind: its start costs two workgroup barriers of sixteen waves).
+bool gemv_dma_pays(uint32_t n, uint32_t k, uint32_t cu_count) {
+    if (!gemv_dma_serves(n, k, cu_count) || k < 2048) return false;
+    const uint64_t bytes = static_cast<uint64_t>(n) * (k / kBlockWeights) * kBlockBytes;
+    return bytes >= (64ull << 20) || (k >= 10240 && bytes >= (32ull << 20));
+}
+
 void launch_gemv_dma(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, uint32_t cu_count, hipStream_t stream) {
     DmaPlan p;
     if (!plan_dma(n, k, cu_count, &p)) return;  // the caller asked gemv_dma_serves first
-    if (p.slabs == 1) launch_one<4, 1, 6, 1>(p, w, n, k, x, y, stream);
-    else if (p.slabs == 2) launch_one<8, 2, 4, 2>(p, w, n, k, x, y, stream);
-    else if (p.slabs == 3) launch_one<16, 1, 6, 3>(p, w, n, k, x, y, stream);
-    else if (p.waves == 4) launch_one<4, 1, 4, 0>(p, w, n, k, x, y, stream);
-    else if (p.waves == 8) launch_one<8, 2, 4, 0>(p, w, n, k, x, y, stream);
-    else launch_one<16, 3, 3, 0>(p, w, n, k, x, y, stream);
+    if (p.slabs == 1) launch_one<1, 6, 1>(p, w, n, k, x, y, stream);
+    else if (p.slabs == 2) launch_one<1, 6, 2>(p, w, n, k, x, y, stream);
+    else if (p.slabs == 3) launch_one<1, 6, 3>(p, w, n, k, x, y, stream);
+    else if (p.xr == 1 && p.depth == 6) launch_one<1, 6, 0>(p, w, n, k, x, y, stream);
+    else if (p.xr == 1) launch_one<1, 3, 0>(p, w, n, k, x, y, stream);
+    else launch_one<3, 3, 0>(p, w, n, k, x, y, stream);
 }
 
 }  // namespace lq4

@@ -76,6 +76,8 @@ void launch_gemv_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, fl
 // Batch-1 kernel whose weights go from memory straight into a per-wave ring of LDS slots (lq4_gemv_dma.hip): plain
 // y = W . x only.  gemv_dma_serves: the shape fits (K <= 24576 and LDS for the activations plus two slots a wave).
 bool gemv_dma_serves(uint32_t n, uint32_t k, uint32_t cu_count);
+// ... and it is measured faster than the lane-owns-block kernel there (full slabs, enough bytes to hide its start).
+bool gemv_dma_pays(uint32_t n, uint32_t k, uint32_t cu_count);
 void launch_gemv_dma(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, uint32_t cu_count, hipStream_t stream);
 // Same with fused elementwise steps (separate kernel instantiations; the plain ones are untouched).
 // The lm_head pass with the exact top-k selected in the same launch: logits (kept in `scratch`), block

@@ -493,6 +493,28 @@ def main():
                                              "with_lora_us": round(res[True] * 1e3, 3),
                                              "GB/s_with_lora": round(lb / res[True] / 1e6, 1),
                                              "lora_overhead_pct": round(100 * (res[True] / res[False] - 1), 1)}
+                if bsz <= 16:
+                    # the same two projections through lq4_gemv_multi: one call for both (one launch at batch 1,
+                    # every adapter's A . x in one more)
+                    def mstep(i, use_lora, bsz=bsz, xl=xl, yl=yl):
+                        bufs = pool[i % len(pool)]
+                        be.gemv_multi(xl, [(bufs[nm], n, yl[nm], nm) for nm, n, _ in projs], bsz, 2048,
+                                      layer_idx=0 if use_lora else None)
+                    mres = {}
+                    for use_lora in (False, True):
+                        if use_lora:
+                            be.load_lora_adapter([backend.LoraLayerData(0, mods)], scale=32 / r)
+                        f = lambda i, u=use_lora: mstep(i, u)
+                        for i in range(len(pool)):
+                            f(i)
+                        mres[use_lora] = tm(torch, f, 192)
+                        if use_lora:
+                            be.unload_lora_adapter()
+                    lora_out["batch%d" % bsz].update({
+                        "one_call_base_us": round(mres[False] * 1e3, 3),
+                        "one_call_with_lora_us": round(mres[True] * 1e3, 3),
+                        "one_call_GB/s_with_lora": round(lb / mres[True] / 1e6, 1),
+                        "one_call_lora_overhead_pct": round(100 * (mres[True] / mres[False] - 1), 1)})
             out["lora_q_v_rank16"] = lora_out
             del pool
 

@@ -132,6 +132,34 @@ int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
              const float* x_dev, uint32_t batch, float* y_dev, const lq4_lora* lora,
              float lora_scale, void* stream);
 
+/* Several projections of the same activations in one call: y_i[b, 0..n_i) = W_i . x[b, 0..K) for i < count, each
+ * with its own optional LoRA epilogue as in lq4_gemv.  Replaces the runs of dispatch_matmul calls on one input
+ * buffer -- q, k and v of an attention layer (inner/layers/gqa.rs:72-98 with their LoRA deltas behind them,
+ * gqa.rs:100-127), qkv and z of a GDN layer, for which the reference had to write a merged weight file to save a
+ * dispatch (inner/layers/gdn.rs:68-73, weights/q4_weights.rs:1553-1643) -- without asking the caller to store the
+ * matrices together: the views may lie anywhere.
+ * At batch 1 the projections are ONE launch: the GEMV kernel walks the rows of the matrices stacked one under the
+ * other (launch, staging of x and start of the stream paid once), and the A . x of every adapter among them is
+ * computed by a few workgroups of that same launch, as lq4_gemv does for one adapter (ranks summing to more than 64:
+ * one more launch in front instead).  Needs K * 4.5 bytes <= 128 KB of LDS (K <= 29120) and, for K of 512 or 1024 (rows
+ * side by side in a wave), every n_i a multiple of 4 or 2; other shapes and batch 2..LQ4_MAX_GEMV_BATCH go projection
+ * by projection through lq4_gemv's own routing (still one A . x launch for all adapters).
+ * A projection with n == 0 is skipped.  Results are those of `count` lq4_gemv calls to the contract's tolerance
+ * (bit-identical without LoRA at batch 1: same kernel, same order of summation).  The A . x values live in the
+ * context: calls with adapters must not overlap on two streams of one context.  Every projection is checked
+ * before anything is launched. */
+#define LQ4_MAX_PROJECTIONS 8
+typedef struct lq4_projection {
+    const lq4_weight* w;
+    uint64_t w_extra_offset;
+    uint32_t n;
+    float* y_dev;            /* f32 [batch, n] */
+    const lq4_lora* lora;    /* NULL = none */
+    float lora_scale;
+} lq4_projection;
+int lq4_gemv_multi(lq4_ctx* ctx, const lq4_projection* proj, uint32_t count, uint32_t k, const float* x_dev,
+                   uint32_t batch, void* stream);
+
 /* ---- prefill GEMM --------------------------------------------------------------
  * Replaces dispatch_gemm / dispatch_gemm_at -> dispatch_gemm_q4[_at]
  * (dispatch.rs:170-229, 507-525, 935-1097): Y[M,N] = X[M,K] . W^T, X f32 or f16
@@ -459,6 +487,7 @@ typedef struct lq4_path_counters {
                                   the producers' hand-over did not arrive in time (read from the device:
                                   this call waits for the GPU) */
     uint64_t lm_head_one_launch; /* lq4_lm_head_topk calls whose GEMV selected the top-k in its own launch */
+    uint64_t gemv_multi;       /* lq4_gemv_multi calls served by one stacked launch */
 } lq4_path_counters;
 int lq4_get_path_counters(const lq4_ctx* ctx, lq4_path_counters* out);
 

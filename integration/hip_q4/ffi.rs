@@ -104,7 +104,20 @@ pub struct Lq4PathCounters {
     pub gemv_chain: u64,
     pub lora_t_fallback: u64,
     pub lm_head_one_launch: u64,
+    pub gemv_multi: u64,
 }
+
+/// One weight view of `lq4_gemv_multi` with its output and optional adapter.
+#[repr(C)]
+pub struct Lq4Projection {
+    pub w: *const Lq4Weight,
+    pub w_extra_offset: u64,
+    pub n: u32,
+    pub y_dev: *mut f32,
+    pub lora: *const Lq4Lora,
+    pub lora_scale: f32,
+}
+pub const LQ4_MAX_PROJECTIONS: usize = 8;
 
 #[link(name = "lattice_hip_q4")]
 extern "C" {
@@ -175,6 +188,16 @@ extern "C" {
         y: *mut f32,
         lora: *const Lq4Lora,
         lora_scale: f32,
+        stream: *mut c_void,
+    ) -> c_int;
+    /// Several projections of one x: one launch at batch 1 (q, k, v of gqa.rs:72-127 without a merged file).
+    pub fn lq4_gemv_multi(
+        ctx: *mut Lq4Ctx,
+        proj: *const Lq4Projection,
+        count: u32,
+        k: u32,
+        x: *const f32,
+        batch: u32,
         stream: *mut c_void,
     ) -> c_int;
     pub fn lq4_gemm(

@@ -50,6 +50,7 @@ EXPORTS = [
     "lq4_probe_read",
     "lq4_probe_read_config",
     "lq4_probe_copy",
+    "lq4_gemv_multi",
     "lq4_set_gemv_kernel",
     "lq4_set_gemm_kernel",
     "lq4_residual_add_rmsnorm", "lq4_silu_mul", "lq4_add_and_copy", "lq4_gemv_fused", "lq4_gemv_fused_batch",
@@ -76,7 +77,16 @@ class Q4Error(RuntimeError):
 class PathCounters(C.Structure):
     _fields_ = [(n, C.c_uint64) for n in ("gemv", "gemm", "lora_a", "moe_route", "moe_gate_up",
                                          "moe_down", "dequant", "topk", "gemv_fused", "elementwise",
-                                         "gemv_chain", "lora_t_fallback", "lm_head_one_launch")]
+                                         "gemv_chain", "lora_t_fallback", "lm_head_one_launch", "gemv_multi")]
+
+
+MAX_PROJECTIONS = 8
+
+
+class Projection(C.Structure):
+    """lq4_projection: one weight view of lq4_gemv_multi with its output and optional adapter."""
+    _fields_ = [("w", C.c_void_p), ("w_extra_offset", C.c_uint64), ("n", C.c_uint32), ("y_dev", C.c_void_p),
+                ("lora", C.c_void_p), ("lora_scale", C.c_float)]
 
 
 LQ4_PRO_NONE, LQ4_PRO_ADD_RMSNORM, LQ4_PRO_SILU_MUL = 0, 1, 2
@@ -143,6 +153,7 @@ def load_library() -> C.CDLL:
         "lq4_probe_read": (C.c_int, [vp, vp, C.c_size_t, vp]),
         "lq4_probe_read_config": (C.c_int, [vp, vp, C.c_size_t, C.c_uint32, C.c_uint32, C.c_int, C.c_int, vp]),
         "lq4_probe_copy": (C.c_int, [vp, vp, vp, C.c_size_t, vp]),
+        "lq4_gemv_multi": (C.c_int, [vp, C.POINTER(Projection), C.c_uint32, C.c_uint32, vp, C.c_uint32, vp]),
         "lq4_set_gemv_kernel": (C.c_int, [vp, C.c_int]),
         "lq4_set_gemm_kernel": (C.c_int, [vp, C.c_int]),
         "lq4_residual_add_rmsnorm": (C.c_int, [vp, vp, vp, vp, C.c_uint32, C.c_uint32, C.c_float, vp, vp, vp]),
@@ -544,6 +555,29 @@ class HipQ4Backend:
         lora = self._lora_for(layer_idx, module, n, k)
         _check(self.lib.lq4_gemv(self.ctx, qw.handle, qw_extra_offset, n, k, x.data_ptr(), batch,
                                  y.data_ptr(), lora, self._lora_scale, self._stream()))
+
+    def gemv_multi(self, x, projections, batch: int, k: int, *, layer_idx=None):
+        """Several projections of the same activations in one call (one launch at batch 1): ``projections`` is a
+        list of ``(qw, n, y)`` or ``(qw, n, y, module)`` or ``(qw, n, y, module, qw_extra_offset)``; with
+        ``layer_idx`` and a module name the loaded adapter's delta for that projection is fused in, as
+        ``gemv_batch`` does.  The q/k/v run of dispatch_matmul calls on one input (inner/layers/gqa.rs:72-127)."""
+        if batch == 0 or not projections:
+            return
+        self._assert_k(k, "dispatch_matmul_q4")
+        if len(projections) > MAX_PROJECTIONS:
+            raise ValueError(f"{len(projections)} projections, at most {MAX_PROJECTIONS} a call")
+        arr = (Projection * len(projections))()
+        for i, p in enumerate(projections):
+            qw, n, y = p[0], p[1], p[2]
+            module = p[3] if len(p) > 3 else None
+            lora = self._lora_for(layer_idx, module, n, k) if module is not None else None
+            arr[i].w = qw.handle
+            arr[i].w_extra_offset = p[4] if len(p) > 4 else 0
+            arr[i].n = n
+            arr[i].y_dev = y.data_ptr()
+            arr[i].lora = lora
+            arr[i].lora_scale = self._lora_scale
+        _check(self.lib.lq4_gemv_multi(self.ctx, arr, len(projections), k, x.data_ptr(), batch, self._stream()))
 
     def dequantize(self, qw: Q4WeightBuf, n: int, k: int, qw_extra_offset: int = 0):
         """f32 [n, k] tensor of ``f32(nibble)*scale + bias`` (bit-exactness probe)."""

@@ -22,7 +22,7 @@ struct lq4_ctx {
     uint8_t* static_scratch;  // this device's copy of `scratch` below (lq4_lm_head_topk_static)
     uint8_t* moe_scratch; // grown on demand
     uint32_t* topk_ticket; // finished-workgroup count of the top-k kernel, zero between launches
-    uint32_t* lora_sync;   // epoch, producer count and slots of the batch-1 GEMV that computes A.x itself (same allocation)
+    uint32_t* lora_sync;   // fall-back count (word 2) and, from word 64 on, the slots of the batch-1 GEMV that computes A.x itself (same allocation)
     bool lora_in_kernel;
     uint32_t lora_spin_limit;  // polls a weight wave spends on those counters before it computes A.x alone
     size_t moe_scratch_bytes;
@@ -197,11 +197,10 @@ int lq4_ctx_create(int device_ordinal, lq4_ctx** out) {
         delete c;
         return fail(LQ4_E_HIP, "hipMalloc(lora scratch): %s", hipGetErrorString(e));
     }
-    // 256 B of top-k ticket, 256 B for the LoRA epoch and producer count, 512 B of LoRA slots
+    // 256 B of top-k ticket, 256 B for the LoRA fall-back count, 512 B of LoRA slots (a zeroed slot matches no
+    // launch: every tag has its top bit set)
     e = hipMalloc(reinterpret_cast<void**>(&c->topk_ticket), 1024);
     if (e == hipSuccess) e = hipMemset(c->topk_ticket, 0, 1024);
-    const uint32_t first_epoch = 1;  // the zeroed slots carry epoch 0
-    if (e == hipSuccess) e = hipMemcpy(c->topk_ticket + 64, &first_epoch, 4, hipMemcpyHostToDevice);
     if (e != hipSuccess) {
         (void)hipFree(c->topk_ticket);
         (void)hipFree(c->lora_t);
@@ -400,6 +399,32 @@ static void plain_gemv_one_token(lq4_ctx* ctx, const uint8_t* wp, uint32_t n, ui
     ctx->counters.gemv++;
 }
 
+// The routing of lq4_gemv once the LoRA factor t (if any) is in ep: which kernel serves (batch, n, k).
+static int gemv_dispatch(lq4_ctx* ctx, const uint8_t* wp, uint32_t n, uint32_t k, const float* x_dev, uint32_t batch,
+                         float* y_dev, const LoraEpilogue& ep, hipStream_t s) {
+    int rc;
+    // Above four activation rows the few-token matrix-core kernel (operands packed once, eight K
+    // slices per workgroup) overtakes the 4x4x4 GEMV kernel: always from nine rows; from five for
+    // mid-sized matrices only (measured: behind for 512 x 2048, where its two launches dominate,
+    // and for 12288 x 2048, where the GEMV kernel's grid already fills the chip).
+    const uint64_t weights = static_cast<uint64_t>(n) * k;
+    // (not for up to 2048 rows while the GEMV kernel can stage the activations: its eight-wave
+    // workgroups then win, 2048 x 6144 at 5..8 rows 9.5 -> 7.2..8.2 us)
+    const bool narrow = n <= 2048 && gemv_mfma_lds_bytes(k, batch < 8 ? batch : 8) <= 150 * 1024;
+    if (batch >= 9 || (batch >= 5 && n < 8192 && !narrow && weights >= 6000000)) {
+        rc = ensure_scratch(ctx, gemm_skinny_scratch_bytes(k, batch), s);
+        if (rc) return rc;
+        launch_gemm_skinny(wp, n, k, x_dev, 0, batch, y_dev, ep, ctx->moe_scratch, s);
+        ctx->counters.gemm++;
+    } else if (batch == 1 && !ep.rank) {
+        plain_gemv_one_token(ctx, wp, n, k, x_dev, y_dev, s);
+    } else {
+        launch_gemv(wp, n, k, x_dev, k, batch, y_dev, n, ep, s);
+        ctx->counters.gemv++;
+    }
+    return LQ4_OK;
+}
+
 int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
              const float* x_dev, uint32_t batch, float* y_dev, const lq4_lora* lora, float lora_scale,
              void* stream) {
@@ -431,24 +456,91 @@ int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
         launch_lora_a(lora->a, lora->is_f16, lora->rank, k, x_dev, 0, k, batch, ctx->lora_t, s);
         ctx->counters.lora_a++;
     }
-    // Above four activation rows the few-token matrix-core kernel (operands packed once, eight K
-    // slices per workgroup) overtakes the 4x4x4 GEMV kernel: always from nine rows; from five for
-    // mid-sized matrices only (measured: behind for 512 x 2048, where its two launches dominate,
-    // and for 12288 x 2048, where the GEMV kernel's grid already fills the chip).
-    const uint64_t weights = static_cast<uint64_t>(n) * k;
-    // (not for up to 2048 rows while the GEMV kernel can stage the activations: its eight-wave
-    // workgroups then win, 2048 x 6144 at 5..8 rows 9.5 -> 7.2..8.2 us)
-    const bool narrow = n <= 2048 && gemv_mfma_lds_bytes(k, batch < 8 ? batch : 8) <= 150 * 1024;
-    if (batch >= 9 || (batch >= 5 && n < 8192 && !narrow && weights >= 6000000)) {
-        rc = ensure_scratch(ctx, gemm_skinny_scratch_bytes(k, batch), static_cast<hipStream_t>(stream));
+    rc = gemv_dispatch(ctx, wp, n, k, x_dev, batch, y_dev, ep, s);
+    if (rc) return rc;
+    LQ4_HIP(hipGetLastError());
+    return LQ4_OK;
+}
+
+int lq4_gemv_multi(lq4_ctx* ctx, const lq4_projection* proj, uint32_t count, uint32_t k, const float* x_dev,
+                   uint32_t batch, void* stream) {
+    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
+    if (count == 0 || batch == 0) return LQ4_OK;
+    if (!proj) return fail(LQ4_E_INVALID, "proj is null");
+    if (count > LQ4_MAX_PROJECTIONS) return fail(LQ4_E_INVALID, "%u projections, at most %d a call", count, LQ4_MAX_PROJECTIONS);
+    if (batch > kMaxGemvBatch) return fail(LQ4_E_INVALID, "lq4_gemv_multi batch %u above %d; use lq4_gemm", batch, kMaxGemvBatch);
+    if (!x_dev) return fail(LQ4_E_INVALID, "x device pointer is null");
+    if (reinterpret_cast<uintptr_t>(x_dev) % 16) return fail(LQ4_E_INVALID, "x must be 16-byte aligned");
+    // every projection is checked before anything is launched: a call fails whole or not at all
+    const uint8_t* wp[LQ4_MAX_PROJECTIONS];
+    LoraEpilogue ep[LQ4_MAX_PROJECTIONS];
+    MultiViews mv{};
+    LoraAViews av{};
+    uint32_t with_lora = 0, total_rank = 0;
+    for (uint32_t i = 0; i < count; ++i) {
+        const lq4_projection& p = proj[i];
+        if (p.n == 0) continue;
+        int rc = resolve_weight(p.w, p.w_extra_offset, p.n, k, &wp[i]);
         if (rc) return rc;
-        launch_gemm_skinny(wp, n, k, x_dev, 0, batch, y_dev, ep, ctx->moe_scratch, s);
-        ctx->counters.gemm++;
-    } else if (batch == 1 && !ep.rank) {
-        plain_gemv_one_token(ctx, wp, n, k, x_dev, y_dev, s);
+        if (!p.y_dev) return fail(LQ4_E_INVALID, "projection %u: y device pointer is null", i);
+        if (reinterpret_cast<uintptr_t>(p.y_dev) % 4) return fail(LQ4_E_INVALID, "projection %u: y must be 4-byte aligned", i);
+        rc = resolve_lora(ctx, p.lora, p.lora_scale, p.n, k, batch, &ep[i]);
+        if (rc) return rc;
+        const uint32_t v = mv.count++;
+        if (static_cast<uint64_t>(mv.begin[v]) + p.n > 0xFFFFFFFFull) return fail(LQ4_E_INVALID, "more than 2^32 - 1 rows in all");
+        mv.begin[v + 1] = mv.begin[v] + p.n;
+        mv.w[v] = wp[i];
+        mv.y[v] = p.y_dev;
+        // view v keeps its A . x in its own part of the context's buffer: [batch, rank] from row v * batch on
+        float* t = ctx->lora_t + static_cast<size_t>(v) * batch * kMaxLoraRank;
+        ep[i].t = t;
+        mv.b[v] = ep[i].b;
+        mv.t[v] = t;
+        mv.rank[v] = ep[i].rank;
+        mv.b_is_f16[v] = ep[i].b_is_f16;
+        mv.scale[v] = ep[i].scale;
+        av.a[v] = ep[i].rank ? p.lora->a : nullptr;
+        av.t[v] = t;
+        av.rank[v] = ep[i].rank;
+        av.a_is_f16[v] = ep[i].b_is_f16;
+        mv.a[v] = av.a[v];
+        mv.t_off[v] = total_rank;
+        total_rank += ep[i].rank;
+        with_lora += ep[i].rank != 0;
+    }
+    av.count = mv.count;
+    if (mv.count == 0) return LQ4_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    DeviceGuard g(ctx->device);
+    const bool stacked = batch == 1 && (mv.count > 1 || with_lora) && gemv_multi_serves(mv, k);
+    // one token: the stacked launch computes every A_v . x in producer workgroups of its own (lane l of a weight
+    // wave holds the factor of stacked row l, hence at most 64 rows of A in all)
+    const bool in_launch = stacked && with_lora && ctx->lora_in_kernel && total_rank <= 64;
+    if (with_lora) {  // the A . x buffer and the hand-over words belong to the context
+        int rc = enter_shared_state(ctx, s);
+        if (rc) return rc;
+        if (!in_launch) {
+            launch_lora_a_views(av, k, x_dev, k, batch, s);  // every adapter's A . x in one launch
+            ctx->counters.lora_a++;
+        }
+    }
+    if (stacked) {
+        LoraEpilogue hand{};
+        if (in_launch) {
+            hand.rank = total_rank;
+            hand.slots = reinterpret_cast<unsigned long long*>(ctx->lora_sync + 64);
+            hand.sync = ctx->lora_sync;
+            hand.spin_limit = ctx->lora_spin_limit;
+        }
+        launch_gemv_multi(mv, k, x_dev, in_launch ? &hand : nullptr, s);
+        ctx->counters.gemv_multi++;
     } else {
-        launch_gemv(wp, n, k, x_dev, k, batch, y_dev, n, ep, s);
-        ctx->counters.gemv++;
+        // several rows (or a shape the stacked launch does not take): each projection through lq4_gemv's routing
+        for (uint32_t i = 0; i < count; ++i) {
+            if (proj[i].n == 0) continue;
+            int rc = gemv_dispatch(ctx, wp[i], proj[i].n, k, x_dev, batch, proj[i].y_dev, ep[i], s);
+            if (rc) return rc;
+        }
     }
     LQ4_HIP(hipGetLastError());
     return LQ4_OK;

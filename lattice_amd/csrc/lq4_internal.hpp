@@ -25,19 +25,51 @@ struct LoraEpilogue {
     float scale;
     // Batch-1 GEMV only.  With `a` set the launch carries `rank` extra workgroups that compute
     // t = A.x themselves while the others stream weights, so no separate launch precedes it.
-    // sync[0] is the launch epoch: every workgroup reads it when it starts.  Producer j stores
-    // slots[j] = {bits of t[j], epoch} as one 64-bit word; a weight wave polls the slots until
-    // all carry its epoch (at most `spin_limit` polls, then it computes t on its own).  The
-    // producers count themselves in sync[1]; the last one zeroes that count and advances the
-    // epoch, which happens only after every producer has read it.  A weight workgroup that starts
-    // after that reads the next epoch, never sees it in the slots and takes the slow path; one
-    // that started before sees exactly this launch's values.  No counter is touched by the weight
-    // workgroups, and nothing has to be reset between launches.
+    // Producer j stores slots[j] = {bits of t[j], tag of the launch} as one 64-bit word; the tag is the place of
+    // the launch's dispatch packet in its queue, which every workgroup of the launch reads from its own input
+    // registers, so nothing has to be agreed on through memory and nothing has to be reset between launches.  A
+    // weight wave polls the slots until all carry its tag (at most `spin_limit` polls, then it computes t on its
+    // own and counts itself in sync[2]).
     const void* a;     // [rank, d_in] row-major, f32 or f16 (b_is_f16 applies to both factors)
     unsigned long long* slots;  // [kMaxLoraRank]
     uint32_t* sync;
     uint32_t spin_limit;
 };
+
+// Several matrices with rows of the same K against one activation vector in one batch-1 launch: the rows of the
+// views stacked one under the other, view v = rows [begin[v], begin[v + 1]).  Each view has its own output and its
+// own LoRA epilogue (rank 0 = none; t = A . x is in memory when the launch starts).
+constexpr int kMaxViews = 8;
+struct MultiViews {
+    uint32_t count;
+    uint32_t begin[kMaxViews + 1];
+    const uint8_t* w[kMaxViews];
+    float* y[kMaxViews];
+    const void* b[kMaxViews];   // [n_v, rank] row-major, f32 or f16
+    const float* t[kMaxViews];  // [rank] f32
+    uint32_t rank[kMaxViews];
+    int b_is_f16[kMaxViews];
+    float scale[kMaxViews];
+    // when the launch computes the factors itself (the LoraEpilogue beside it then carries the hand-over words and
+    // rank = the ranks' sum, at most 64): the A matrices, and where each view's factors start in the stacked t
+    const void* a[kMaxViews];   // [rank, k] row-major, dtype as b
+    uint32_t t_off[kMaxViews];
+};
+
+// The A factors of the views' adapters for one launch that computes every t_v = A_v . x (rank 0 = no adapter).
+struct LoraAViews {
+    uint32_t count;
+    const void* a[kMaxViews];  // [rank, d_in] row-major, f32 or f16
+    float* t[kMaxViews];       // [rows, rank] f32
+    uint32_t rank[kMaxViews];
+    int a_is_f16[kMaxViews];
+};
+bool gemv_multi_serves(const MultiViews& mv, uint32_t k);
+// `in_launch`: null = every t_v is in memory; else the hand-over words (slots, sync, spin_limit, rank = the ranks' sum)
+// of a launch that computes the factors in producer workgroups of its own.
+void launch_gemv_multi(const MultiViews& mv, uint32_t k, const float* x, const LoraEpilogue* in_launch, hipStream_t stream);
+void launch_lora_a_views(const LoraAViews& av, uint32_t d_in, const float* x, uint32_t x_stride, uint32_t rows,
+                         hipStream_t stream);
 
 // Elementwise steps fused into the batch-1 GEMV.
 //   prologue kAddNorm: v = base + delta (delta may be null), the activation is the shifted RMSNorm

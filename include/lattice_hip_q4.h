@@ -127,7 +127,12 @@ int lq4_lora_apply(lq4_ctx* ctx, const lq4_lora* lora, float lora_scale, const v
  * scaled by a power of two per 32-element block and multiplied exactly, so the result tracks an f32
  * GEMV as the reference's gemv_q4_decode does, shaders/qwen35.metal:794-866; an infinite or NaN
  * activation makes every output NaN); at batch 2..16 activations are split into unscaled f16 pairs
- * and |x| >= 65504 becomes infinity. */
+ * (two rows) or rounded to f16 (more), and |x| >= 65504 becomes infinity -- except where the integer
+ * matrix-core kernel serves the call (3..8 rows of a matrix of at most 4096 x 2048 unless the context
+ * was created under LQ4_GEMV_I8=0): it keeps 24 bits (up to four rows: an f32 GEMV, as the
+ * reference's gemm_q4 is) or 16 bits (five to eight) of every activation below its 32-element block's
+ * largest magnitude and takes any finite f32 value; a row that holds an infinity or a NaN comes back
+ * NaN.  The guaranteed contract is the weaker one. */
 int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t n, uint32_t k,
              const float* x_dev, uint32_t batch, float* y_dev, const lq4_lora* lora,
              float lora_scale, void* stream);

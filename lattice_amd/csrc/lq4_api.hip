@@ -44,6 +44,8 @@ struct lq4_ctx {
     int lm_head_mode;        // lq4_set_lm_head_mode
     int gemm_kernel;         // lq4_set_gemm_kernel
     int gemv_kernel;         // lq4_set_gemv_kernel: which kernel serves a plain one-token GEMV
+    int gemv_i8;             // LQ4_GEMV_I8: 1 = 3..8 rows of small matrices take the integer matrix-core kernel (default),
+                             // 0 = never, 2 = 2..8 rows of every matrix it can serve (tests)
     lq4_path_counters counters;
 };
 
@@ -235,6 +237,8 @@ int lq4_ctx_create(int device_ordinal, lq4_ctx** out) {
     c->gemm_kernel = gemm_kernel_choice_default();
     c->gemv_kernel = getenv("LQ4_GEMV_KERNEL") ? atoi(getenv("LQ4_GEMV_KERNEL")) : 0;
     if (c->gemv_kernel < 0 || c->gemv_kernel > 2) c->gemv_kernel = 0;
+    c->gemv_i8 = getenv("LQ4_GEMV_I8") ? atoi(getenv("LQ4_GEMV_I8")) : 1;
+    if (c->gemv_i8 < 0 || c->gemv_i8 > 2) c->gemv_i8 = 1;
     // LQ4_LORA_SPIN_LIMIT: 0 makes every weight wave compute A.x itself (the path a wave takes when
     // the producers are late), "off" restores the separate A.x launch
     c->lora_spin_limit = 512;
@@ -418,6 +422,17 @@ static int gemv_dispatch(lq4_ctx* ctx, const uint8_t* wp, uint32_t n, uint32_t k
         ctx->counters.gemm++;
     } else if (batch == 1 && !ep.rank) {
         plain_gemv_one_token(ctx, wp, n, k, x_dev, y_dev, s);
+    } else if (batch >= 2 && batch <= 8 && ctx->gemv_i8 &&
+               (ctx->gemv_i8 == 2 || (batch >= 3 && k <= 2048 && n <= 4096)) &&
+               gemv_i8_serves(n, k, batch, ctx->cu_count)) {
+        // Three to eight rows of a matrix of up to 4096 x 2048: the integer matrix-core kernel, which is as fast as
+        // or faster than the 4x4x4 kernel there (512 x 2048: 4.33 -> 4.09 us at four rows, 4.71 -> 4.53 at eight;
+        // 2048 x 2048: 4.67 -> 4.54, 5.09 -> 4.98; 3072 x 2048 at four rows 5.58 -> 4.82) and keeps 24 (up to four rows)
+        // or 16 bits of every activation below its block's maximum instead of rounding it to f16.  Behind on long rows
+        // and many rows (2048 x 6144 at eight rows 8.7 -> 10.4 us, 12288 x 2048 at four 7.8 -> 8.8), which stay where
+        // they were.
+        launch_gemv_i8(wp, n, k, x_dev, k, batch, y_dev, n, ep, ctx->cu_count, s);
+        ctx->counters.gemv++;
     } else {
         launch_gemv(wp, n, k, x_dev, k, batch, y_dev, n, ep, s);
         ctx->counters.gemv++;

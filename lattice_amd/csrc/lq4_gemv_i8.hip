@@ -1,0 +1,436 @@
+// Decode GEMV for up to eight activation rows on the integer matrix cores:
+//   y[b, n] = sum_k W[n, k] * x[b, k],  b < batch <= 8.
+//
+// Instruction.  v_mfma_i32_16x16x32_i8 multiplies a 16 x 32 by a 32 x 16 matrix of signed bytes into 16 x 16 32-bit
+// sums.  K = 32 is exactly one Q4 block, so one instruction forms the integer dot products of one block of 16 weight
+// rows with 16 activation columns, and the block's scale and bias are applied to its result in f32 afterwards.
+//   B operand (32 x 16): the weights.  Lane l supplies column n = l % 16 (a weight row), k = 8 * (l / 16) .. + 7:
+//     the eight nibbles of payload dword l / 16 of that row's block, spread into bytes by two masks.
+//   A operand (16 x 32): the activations, staged as fixed point scaled per block (x = xs * q, xs = the block's largest
+//     magnitude / the largest q) and cut into signed byte digits.  Five to eight activation rows: two digits each
+//     (q = 256 hi + lo, 16 bits), operand row m = 2 b + digit, so eight rows fill the operand and nothing of the
+//     instruction is idle.  Up to four rows ("wide"): three digits each (24 bits), m = 4 b + digit.
+//   D (16 x 16): lane l receives column n = l % 16, rows m = 4 (l / 16) .. + 3, i.e. for ITS weight row both digits
+//     of activation rows 2 (l / 16) and 2 (l / 16) + 1 (wide: the three digits of row l / 16).  256 hi + lo is one
+//     integer multiply-add, and
+//       y[b, n] += (scale_n * xs_b) * (256 hi + lo) + bias_n * (xs_b * sum of the block's fixed-point x)
+//     needs the block header of the lane's own row only: no value crosses lanes after the instruction, and every
+//     lane owns two outputs of its row from the first block to the last.
+// Per instruction (16 rows x 32 weights = 320 bytes of weights): 3 operations to spread the nibbles, 2 to convert the
+// header, 10 for the two outputs.  Four SIMDs at that rate consume weights several times faster than memory
+// delivers them, which the 4x4x4 f16 kernel (eight instructions and their operand shuffles per block of four rows)
+// does not.
+//
+// Memory.  A unit is 16 rows x 8 blocks (2.5 KB).  Lane l loads block l % 8 of rows l / 8 and l / 8 + 8 as whole
+// 20-byte blocks (dwordx4 + dword, 160 contiguous bytes per row), keeps four units in flight in registers, and
+// passes the blocks through a wave-private LDS tile to reach the operand layout (row pitch 44 dwords: the 16 rows
+// x 4 dwords a read touches fall into 64 different banks).  Nothing is fetched twice; no barrier: a wave's LDS
+// accesses are carried out in order.
+//
+// Work split.  A workgroup takes tiles of 16 rows (tile = blockIdx, then += gridDim); its waves split K in chunks
+// of 8 blocks and add their partial sums through LDS in wave order.  Each wave stages the activations of its own
+// chunks only, once for all tiles of the workgroup, behind its first weight loads.
+//
+// Precision.  The weights enter exactly, the integer sums are exact.  An activation is rounded to a multiple of its
+// block's largest magnitude / 32639 (two digits: step 3e-5 of the block maximum, against 5e-4 of the element for the
+// f16 rounding of the 4x4x4 kernel and of the reference's tiled kernel, shaders/gemm_q4_tiled.metal:45-48) or
+// / 8355711 (wide: 1.2e-7, the resolution of the f32 activation itself, so up to four rows track an f32 GEMV as the
+// reference's gemm_q4 does).  Any finite f32 activation is in range (the scale is per block); a block whose largest
+// magnitude is below 2^-100 counts as zero; an infinite or NaN activation makes the outputs of its row NaN.
+#include "lq4_internal.hpp"
+
+#include <atomic>
+#include <type_traits>
+
+namespace lq4 {
+
+namespace {
+
+typedef int int4v __attribute__((ext_vector_type(4)));
+
+constexpr int kBpw = 8;            // blocks per wave chunk
+constexpr int kTilePitch = 44;     // dwords per row of the LDS tile (40 used; 44 r mod 64 differs for every r < 16)
+constexpr int kTileDwords = 16 * kTilePitch;
+constexpr int kXqBytes = 512;      // per block: [4 k groups][16 operand rows] x 8 bytes
+constexpr int kXfBytes = 64;       // per block: [4 lane groups][xs of rows 2g, 2g + 1, then their sums] f32
+
+struct __attribute__((packed, aligned(4))) Q4BlockRaw {
+    uint32_t sb;    // f16 scale | f16 bias << 16
+    uint32_t q[4];  // 32 nibbles, nibble i of dword j = weight 8j + i
+};
+
+__device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+__device__ __forceinline__ float half_lo(uint32_t sb) {
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(sb & 0xFFFFu)));
+}
+__device__ __forceinline__ float half_hi(uint32_t sb) {
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(sb >> 16)));
+}
+
+// WIDE: up to four activation rows at three digits; else up to eight at two.
+// CW x TW waves: CW waves split the chunks of one tile, TW tiles are worked on side by side.
+template <int CW, int TW, bool WIDE>
+__global__ __launch_bounds__(64 * CW * TW) void gemv_q4_i8(const uint8_t* __restrict__ w, uint32_t n, uint32_t k,
+                                                           const float* __restrict__ x, uint32_t x_stride,
+                                                           uint32_t batch, float* __restrict__ y, uint32_t y_stride,
+                                                           LoraEpilogue lora) {
+    constexpr int WAVES = CW * TW;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t tw = wave / CW, cw = wave % CW;
+    const uint32_t nb = k / kBlockWeights;
+    const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
+    // LDS: [nb] activation digits | [nb] activation scales and sums | [WAVES] tiles | [WAVES][64][2] partial sums
+    uint8_t* const xq = smem;
+    uint8_t* const xf = xq + static_cast<size_t>(nb) * kXqBytes;
+    uint32_t* const tile = reinterpret_cast<uint32_t*>(xf + static_cast<size_t>(nb) * kXfBytes) + wave * kTileDwords;
+    float* const part = reinterpret_cast<float*>(xf + static_cast<size_t>(nb) * kXfBytes) + WAVES * kTileDwords;
+
+    const uint32_t n_tiles = (n + 15) / 16;
+    const uint32_t chunks = (nb + kBpw - 1) / kBpw;
+    const uint32_t my_chunks = cw < chunks ? (chunks - cw + CW - 1) / CW : 0;  // chunk c * CW + cw
+    // tiles of the workgroup: blockIdx + j * gridDim; of this wave: j = tw, tw + TW, ...; a round = TW tiles
+    const uint32_t wg_tiles = blockIdx.x < n_tiles ? (n_tiles - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
+    const uint32_t rounds = (wg_tiles + TW - 1) / TW;
+    const uint32_t my_tiles = tw < wg_tiles ? (wg_tiles - tw + TW - 1) / TW : 0;
+    const uint32_t units = my_tiles * my_chunks;  // unit u = (my tile u / my_chunks, my chunk u % my_chunks)
+    auto first_row = [&](uint32_t t) { return (blockIdx.x + (t * TW + tw) * gridDim.x) * 16; };
+
+    // load mapping: lane = (block jl, row rq), rows rq + kRowStep * i
+    constexpr int kRowStep = 64 / kBpw, kLoads = 16 / kRowStep;
+    const uint32_t jl = lane % kBpw, rq = lane / kBpw;
+    auto load_unit = [&](Q4BlockRaw (&buf)[kLoads], uint32_t u) {
+        const uint32_t t = u / my_chunks, c = u - t * my_chunks;
+        const uint32_t row0 = first_row(t);
+        uint32_t blk = (c * CW + cw) * kBpw + jl;
+        if (blk >= nb) blk = nb - 1;
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) {
+            uint32_t row = row0 + rq + kRowStep * i;
+            if (row >= n) row = n - 1;
+            const uint8_t* bp = w + row * row_bytes + blk * static_cast<uint32_t>(kBlockBytes);
+            // (plain loads: a unit's 160-byte pieces share their cache lines with the neighbouring waves' pieces)
+            buf[i].sb = *reinterpret_cast<const uint32_t*>(bp);
+            typedef uint32_t u32x4u __attribute__((ext_vector_type(4), aligned(4)));
+            const u32x4u q = *reinterpret_cast<const u32x4u*>(bp + 4);
+            buf[i].q[0] = q.x; buf[i].q[1] = q.y; buf[i].q[2] = q.z; buf[i].q[3] = q.w;
+        }
+    };
+
+    // ---- stage the activations, all waves together: task = (block, activation row, k group), 8 values each ----
+    // The values of a thread's first tasks are requested before any weight (loads are answered in the order a CU
+    // issued them: behind the weight prefetch the staging would wait for the weights), all at once.
+    constexpr uint32_t kRows = WIDE ? 4 : 8;      // activation rows the operand holds
+    constexpr int kHoist = WAVES >= 16 ? 2 : 4;   // tasks a thread requests ahead (K = 2048 at eight rows: all of them)
+    // q = rint(x / xs) with xs = block maximum / kQScale: |q| stays below kQScale + 2 whatever the rounding of the
+    // reciprocal, every digit within -128..127; wide: 22 bits and sign, what the float trick below can hold
+    constexpr float kQScale = WIDE ? 4194000.0f : 32639.0f;
+    const uint32_t n_tasks = nb * 4 * kRows;
+    auto task_ptr = [&](uint32_t idx) {
+        const uint32_t kg = idx & 3, b = (idx >> 2) & (kRows - 1), blk = idx / (4 * kRows);
+        // rows and blocks that do not exist re-read an existing one; their digits are zeroed below
+        const uint32_t bb = b < batch ? b : 0, bl = blk < nb ? blk : nb - 1;
+        return reinterpret_cast<const float4*>(x + static_cast<size_t>(bb) * x_stride + bl * kBlockWeights + kg * 8);
+    };
+    auto quad_max = [](uint32_t v) {
+        v = max(v, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0xB1, 0xF, 0xF, false)));
+        return max(v, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x4E, 0xF, 0xF, false)));
+    };
+    auto quad_sum = [](int v) {
+        v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, false);
+        return v + __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, false);
+    };
+    auto stage_task = [&](uint32_t idx, const float4 xa, const float4 xb) {
+        const uint32_t kg = idx & 3, b = (idx >> 2) & (kRows - 1), blk = idx / (4 * kRows);
+        const bool live = blk < nb && b < batch;  // (the four lanes of a (block, row) agree)
+        const float v[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+        // largest magnitude as a bit pattern: infinities and NaNs come out on top of every finite value
+        uint32_t abits = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) abits = max(abits, as_u32(v[i]) & 0x7FFFFFFFu);
+        abits = quad_max(live ? abits : 0u);
+        const bool finite = abits < 0x7F800000u;
+        float inv = 0.0f, xs = 0.0f;
+        if (finite && abits >= 0x0D800000u) {  // 2^-100 and up
+            xs = as_f32(abits) * (1.0f / kQScale);
+            inv = __builtin_amdgcn_rcpf(xs);
+        } else if (!finite) {
+            xs = as_f32(0x7FC00000u);  // infinite or NaN activation: the row's outputs become NaN
+        }
+        // 1.5 * 2^23 + q as a float has q in its low 23 bits in two's complement: bits = 0x4B400000 + q
+        uint32_t qb[8], sum_bits = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            qb[i] = as_u32(fmaf(v[i], inv, 12582912.0f));  // (a row that does not exist: inv = 0, digits 0)
+            sum_bits += qb[i];
+        }
+        const int sum = quad_sum(static_cast<int>(sum_bits - 8u * 0x4B400000u));
+        // Digits -128..127 from the lowest up: byte 0 of q, byte 1 of q + 0x80, byte 2 of q + 0x8080 (minus the
+        // 0x40 the float's own bits hold there).  Byte p of an operand word pair = element {0, 2, 4, 6, 1, 3, 5,
+        // 7}[p] of the k group: the order in which the two masks lay out a payload dword's nibbles.
+        constexpr int kDigits = WIDE ? 3 : 2;
+        uint32_t dg[kDigits][2];
+#pragma unroll
+        for (int t = 0; t < kDigits; ++t) {
+            const uint32_t add = t == 0 ? 0u : t == 1 ? 0x80u : 0xFFC08080u;
+            // byte t of (qb + add) of four elements into one dword: 0x0c selects a zero byte
+            const uint32_t sel_lo = 0x0c0c0400u + 0x0101u * t, sel_hi = 0x04000c0cu + 0x01010000u * t;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {  // h = 0: elements 0, 2, 4, 6;  h = 1: elements 1, 3, 5, 7
+                const uint32_t e0 = qb[h] + add, e1 = qb[2 + h] + add, e2 = qb[4 + h] + add, e3 = qb[6 + h] + add;
+                dg[t][h] = __builtin_amdgcn_perm(e1, e0, sel_lo) | __builtin_amdgcn_perm(e3, e2, sel_hi);
+            }
+        }
+        if (blk < nb) {
+            // operand row of (b, digit): the highest digit first
+            uint2* dst = reinterpret_cast<uint2*>(xq + static_cast<size_t>(blk) * kXqBytes + kg * 128 + ((WIDE ? 4 : 2) * b) * 8);
+#pragma unroll
+            for (int t = 0; t < kDigits; ++t) dst[t] = make_uint2(dg[kDigits - 1 - t][0], dg[kDigits - 1 - t][1]);
+            if (WIDE) dst[3] = make_uint2(0u, 0u);
+            if (kg == 0) {
+                // per lane group g of the product: {xs, xs} then {sum, sum} of rows 2g, 2g + 1; wide: {xs, sum} of row g
+                float* f = reinterpret_cast<float*>(xf + static_cast<size_t>(blk) * kXfBytes);
+                const float sx = xs * static_cast<float>(sum);
+                if (WIDE) {
+                    f[4 * b] = xs;
+                    f[4 * b + 1] = sx;
+                } else {
+                    f[4 * (b >> 1) + (b & 1)] = xs;
+                    f[4 * (b >> 1) + 2 + (b & 1)] = sx;
+                }
+            }
+        }
+    };
+
+    float4 xv[kHoist][2];
+#pragma unroll
+    for (int it = 0; it < kHoist; ++it) {
+        const float4* xp = task_ptr(tid + it * 64 * WAVES);
+        xv[it][0] = xp[0];
+        xv[it][1] = xp[1];
+    }
+    // kDepth units in flight per wave, in a ring of register buffers that the unrolled loop below walks with
+    // compile-time indices.  Requests are skipped past the wave's last unit (a wave cannot end before its last load
+    // has come back); the compiler then waits in front of a buffer's use as if the skipped request had not been
+    // made, one unit earlier than needed, so three units are in flight where it matters.
+    constexpr int kDepth = 4;
+    Q4BlockRaw ring[kDepth][kLoads];
+#pragma unroll
+    for (int i = 0; i < kDepth; ++i) {
+        if (static_cast<uint32_t>(i) < units) load_unit(ring[i], i);
+    }
+    __builtin_amdgcn_sched_barrier(0);  // nothing below is scheduled above these loads
+#pragma unroll
+    for (int it = 0; it < kHoist; ++it) {
+        const uint32_t idx = tid + it * 64 * WAVES;
+        if (idx < n_tasks) stage_task(idx, xv[it][0], xv[it][1]);  // (whole quads: n_tasks is a multiple of 4)
+    }
+    for (uint32_t idx = tid + kHoist * 64 * WAVES; idx < n_tasks; idx += 64 * WAVES) {
+        const float4* xp = task_ptr(idx);
+        stage_task(idx, xp[0], xp[1]);
+    }
+    __syncthreads();
+
+    // ---- the product ----
+    const uint32_t r = lane & 15, g = lane >> 4;  // operand mapping: weight row r of the tile, k group / row pair g
+    float acc0 = 0.0f, acc1 = 0.0f;
+    auto process = [&](Q4BlockRaw (&cur)[kLoads], uint32_t u) {
+        if (u >= units) return;  // uniform
+        // through the tile: tile[row][5 * block + d]; the buffer is then free for the unit kDepth ahead
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) {
+            uint32_t* tp = tile + (rq + kRowStep * i) * kTilePitch + 5 * jl;
+            tp[0] = cur[i].sb;
+            tp[1] = cur[i].q[0]; tp[2] = cur[i].q[1]; tp[3] = cur[i].q[2]; tp[4] = cur[i].q[3];
+        }
+        if (u + kDepth < units) load_unit(cur, u + kDepth);  // uniform
+        const uint32_t t = u / my_chunks, c = u - t * my_chunks;
+        const uint32_t blk0 = (c * CW + cw) * kBpw;
+        const uint32_t* tr = tile + r * kTilePitch;
+        // four blocks at a time, straight-line: their LDS reads, then their four matrix instructions back to back,
+        // then their results (a block past the end of the row re-reads the row's last one and counts for nothing)
+#pragma unroll
+        for (int j0 = 0; j0 < kBpw; j0 += 4) {
+            uint32_t sb[4], qd[4];
+            long aop[4];
+            float4 f[4];
+            bool live[4];
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj) {
+                const uint32_t blk_raw = blk0 + j0 + jj;
+                live[jj] = blk_raw < nb;  // uniform
+                const uint32_t blk = live[jj] ? blk_raw : nb - 1;
+                sb[jj] = tr[5 * (j0 + jj)];
+                qd[jj] = tr[5 * (j0 + jj) + 1 + g];
+                aop[jj] = *reinterpret_cast<const long*>(xq + static_cast<size_t>(blk) * kXqBytes + lane * 8);
+                f[jj] = *reinterpret_cast<const float4*>(xf + static_cast<size_t>(blk) * kXfBytes + g * 16);
+            }
+            int4v d[4];
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj) {
+                const uint32_t even = qd[jj] & 0x0F0F0F0Fu, odd = (qd[jj] >> 4) & 0x0F0F0F0Fu;
+                const long bop = static_cast<long>((static_cast<uint64_t>(odd) << 32) | even);
+                const int4v zero = {0, 0, 0, 0};
+                d[jj] = __builtin_amdgcn_mfma_i32_16x16x32_i8(aop[jj], bop, zero, 0, 0, 0);
+            }
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj) {
+                const float scale = live[jj] ? half_lo(sb[jj]) : 0.0f, bias = live[jj] ? half_hi(sb[jj]) : 0.0f;
+                if constexpr (WIDE) {
+                    // the top digit's sum times 2^16 is exact in f32, so is 256 mid + low: one rounding in the add
+                    const float d0 = fmaf(static_cast<float>(d[jj].x), 65536.0f, static_cast<float>(d[jj].y * 256 + d[jj].z));
+                    acc0 = fmaf(scale * f[jj].x, d0, acc0);
+                    acc0 = fmaf(bias, f[jj].y, acc0);
+                } else {
+                    const float d0 = static_cast<float>(d[jj].x * 256 + d[jj].y), d1 = static_cast<float>(d[jj].z * 256 + d[jj].w);
+                    acc0 = fmaf(scale * f[jj].x, d0, acc0);
+                    acc1 = fmaf(scale * f[jj].y, d1, acc1);
+                    acc0 = fmaf(bias, f[jj].z, acc0);
+                    acc1 = fmaf(bias, f[jj].w, acc1);
+                }
+            }
+        }
+        if (c + 1 == my_chunks) {  // the wave's part of the tile is complete: meet the tile's other waves in LDS
+            const uint32_t row = first_row(t) + r;
+            if constexpr (WAVES > 1) {
+                __syncthreads();  // (every wave passes here once a round; waves without work bring zeros)
+                part[(wave * 64 + lane) * 2] = acc0;
+                part[(wave * 64 + lane) * 2 + 1] = acc1;
+                __syncthreads();
+                acc0 = 0.0f;
+                acc1 = 0.0f;
+                if (cw == 0) {
+#pragma unroll
+                    for (int v = 0; v < CW; ++v) {
+                        acc0 += part[((tw * CW + v) * 64 + lane) * 2];
+                        acc1 += part[((tw * CW + v) * 64 + lane) * 2 + 1];
+                    }
+                }
+            }
+            if (cw == 0 && row < n) {
+                const uint32_t b0 = WIDE ? g : 2 * g, b1 = WIDE ? batch : 2 * g + 1;  // (wide: one row a lane)
+                if (lora.rank) {
+                    // (every load of this loop is used inside it and unconditional: a load left pending on one path
+                    // would make the compiler wait for the whole weight ring wherever its register is reused)
+                    const uint32_t t0 = (b0 < batch ? b0 : 0) * lora.rank, t1 = (b1 < batch ? b1 : 0) * lora.rank;
+                    float l0 = 0.0f, l1 = 0.0f;
+                    for (uint32_t i = 0; i < lora.rank; ++i) {
+                        const size_t bi = static_cast<size_t>(row) * lora.rank + i;
+                        const float bv = lora.b_is_f16 ? static_cast<float>(static_cast<const _Float16*>(lora.b)[bi])
+                                                       : static_cast<const float*>(lora.b)[bi];
+                        l0 = fmaf(bv, lora.t[t0 + i], l0);
+                        l1 = fmaf(bv, lora.t[t1 + i], l1);
+                    }
+                    acc0 = fmaf(lora.scale, l0, acc0);
+                    acc1 = fmaf(lora.scale, l1, acc1);
+                }
+                if (b0 < batch) y[static_cast<size_t>(b0) * y_stride + row] = acc0;
+                if (b1 < batch) y[static_cast<size_t>(b1) * y_stride + row] = acc1;
+            }
+            acc0 = 0.0f;
+            acc1 = 0.0f;
+        }
+    };
+
+    for (uint32_t u = 0; u < units; u += kDepth) {
+#pragma unroll
+        for (int i = 0; i < kDepth; ++i) process(ring[i], u + i);
+    }
+    // a wave meets the others once a round: those with fewer tiles than rounds (or no chunk at all) make up for it
+    if constexpr (WAVES > 1) {
+        const uint32_t met = my_chunks ? my_tiles : 0;
+        for (uint32_t t = met; t < rounds; ++t) {
+            __syncthreads();
+            part[(wave * 64 + lane) * 2] = 0.0f;
+            part[(wave * 64 + lane) * 2 + 1] = 0.0f;
+            __syncthreads();
+        }
+    }
+}
+
+struct I8Plan {
+    uint32_t cw, tw, grid;
+    size_t lds;
+};
+
+bool plan_i8(uint32_t n, uint32_t k, uint32_t batch, uint32_t cu_count, I8Plan* out) {
+    if (k == 0 || k % kBlockWeights || n == 0 || batch == 0 || batch > 8) return false;
+    const uint32_t nb = k / kBlockWeights;
+    const uint32_t chunks = (nb + kBpw - 1) / kBpw;
+    const uint32_t n_tiles = (n + 15) / 16;
+    I8Plan p;
+    // waves that split one tile's chunks: a power of two up to sixteen; tiles side by side: as many as fill a
+    // sixteen-wave workgroup, but no more than leaves every CU a workgroup (one workgroup a CU stages the
+    // activations once for all the tiles that CU works on)
+    p.cw = chunks >= 16 ? 16 : chunks >= 8 ? 8 : chunks >= 4 ? 4 : chunks >= 2 ? 2 : 1;
+    p.tw = 16 / p.cw;
+    while (p.tw > 1 && (n_tiles + p.tw - 1) / p.tw < cu_count) p.tw /= 2;
+    for (;;) {
+        const uint32_t waves = p.cw * p.tw;
+        p.lds = static_cast<size_t>(nb) * (kXqBytes + kXfBytes) + static_cast<size_t>(waves) * kTileDwords * 4 +
+                static_cast<size_t>(waves) * 64 * 2 * 4;
+        if (p.lds <= 160 * 1024) break;
+        if (p.tw > 1) p.tw /= 2;
+        else if (p.cw > 1) p.cw /= 2;
+        else return false;
+    }
+    const uint32_t groups = (n_tiles + p.tw - 1) / p.tw;  // rounds of tiles in all
+    if (groups <= cu_count) {
+        p.grid = groups;
+    } else {
+        const uint32_t per = (groups + cu_count - 1) / cu_count;
+        p.grid = (groups + per - 1) / per;  // the same number of rounds for every workgroup, to within one
+    }
+    *out = p;
+    return true;
+}
+
+template <int CW, int TW, bool WIDE>
+void launch_i8(const I8Plan& p, const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint32_t x_stride,
+               uint32_t batch, float* y, uint32_t y_stride, const LoraEpilogue& lora, hipStream_t stream) {
+    static std::atomic<uint64_t> attr_set{0};  // one bit a device: the attribute belongs to the device's copy of the code
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    const uint64_t bit = 1ull << (dev & 63);
+    if (!(attr_set.load(std::memory_order_relaxed) & bit)) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_i8<CW, TW, WIDE>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        attr_set.fetch_or(bit, std::memory_order_relaxed);
+    }
+    hipLaunchKernelGGL((gemv_q4_i8<CW, TW, WIDE>), dim3(p.grid), dim3(64 * CW * TW), p.lds, stream, w, n, k, x, x_stride,
+                       batch, y, y_stride, lora);
+}
+
+template <bool WIDE>
+void launch_i8_shape(const I8Plan& p, const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint32_t x_stride,
+                     uint32_t batch, float* y, uint32_t y_stride, const LoraEpilogue& lora, hipStream_t stream) {
+#define LQ4_I8(CW_, TW_) \
+    if (p.cw == CW_ && p.tw == TW_) return launch_i8<CW_, TW_, WIDE>(p, w, n, k, x, x_stride, batch, y, y_stride, lora, stream)
+    LQ4_I8(16, 1);
+    LQ4_I8(8, 2); LQ4_I8(8, 1);
+    LQ4_I8(4, 4); LQ4_I8(4, 2); LQ4_I8(4, 1);
+    LQ4_I8(2, 8); LQ4_I8(2, 4); LQ4_I8(2, 2); LQ4_I8(2, 1);
+    LQ4_I8(1, 16); LQ4_I8(1, 8); LQ4_I8(1, 4); LQ4_I8(1, 2); LQ4_I8(1, 1);
+#undef LQ4_I8
+}
+
+}  // namespace
+
+bool gemv_i8_serves(uint32_t n, uint32_t k, uint32_t batch, uint32_t cu_count) {
+    I8Plan p;
+    return plan_i8(n, k, batch, cu_count, &p);
+}
+
+void launch_gemv_i8(const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint32_t x_stride, uint32_t batch,
+                    float* y, uint32_t y_stride, const LoraEpilogue& lora, uint32_t cu_count, hipStream_t stream) {
+    I8Plan p;
+    if (!plan_i8(n, k, batch, cu_count, &p)) return;  // the caller asked gemv_i8_serves first
+    if (batch <= 4) launch_i8_shape<true>(p, w, n, k, x, x_stride, batch, y, y_stride, lora, stream);
+    else launch_i8_shape<false>(p, w, n, k, x, x_stride, batch, y, y_stride, lora, stream);
+}
+
+}  // namespace lq4

@@ -105,6 +105,12 @@ size_t gemv_b1_lds_bytes(uint32_t k);
 bool gemv_b1_pairs_served(uint32_t n, uint32_t k);
 void launch_gemv_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y,
                     const LoraEpilogue& lora, hipStream_t stream);
+// 2..8 activation rows on the integer matrix cores (lq4_gemv_i8.hip): y = W . x, optional LoRA epilogue with t in
+// memory.  gemv_i8_serves: the staged activations fit the LDS (K up to about 7000).
+bool gemv_i8_serves(uint32_t n, uint32_t k, uint32_t batch, uint32_t cu_count);
+void launch_gemv_i8(const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint32_t x_stride, uint32_t batch,
+                    float* y, uint32_t y_stride, const LoraEpilogue& lora, uint32_t cu_count, hipStream_t stream);
+
 // Batch-1 kernel whose weights go from memory straight into a per-wave ring of LDS slots (lq4_gemv_dma.hip): plain
 // y = W . x only.  gemv_dma_serves: the shape fits (K <= 24576 and LDS for the activations plus two slots a wave).
 bool gemv_dma_serves(uint32_t n, uint32_t k, uint32_t cu_count);

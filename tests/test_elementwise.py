@@ -311,7 +311,9 @@ def test_fused_decode_mlp_for_several_rows(be, hidden, inter, batch):
     be.dispatch_fused_residual_add_norm(d_base, d_delta, res2, normed, d_gamma, hidden, eps, num_rows=batch)
     gu2 = torch.empty((batch, 2 * inter), device="cuda")
     be.gemv_batch(normed, qgu, gu2, batch, 2 * inter, hidden)
-    same_kernel = 2e-5
+    # (three to eight rows of a small matrix: the plain call takes the integer matrix-core kernel, which keeps 16 or
+    # 24 bits of an activation, while the fused call rounds it to f16 - each is within the contract of the oracle)
+    same_kernel = 2e-5 if batch <= 2 else REL_TOL
     assert rel_err(got_gu, host(gu2)) <= same_kernel
     # (the second stage from the fused first stage's own output, so that only this stage is compared)
     gu2 = dev(got_gu)

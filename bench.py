@@ -31,6 +31,11 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense f16
 # rocprofv3 counters on this workload (profiles/gemv_q4_b1_decode_layer_traffic.md): per layer step
 # FETCH_SIZE 15122.0 KiB x 2.000 (copy-kernel scale) + WRITE_SIZE 144 KiB x 1.000, over 4 launches
 MEASURED_TRAFFIC_PER_LAUNCH = (15122.0 * 2.0 + 144.0) * 1024 / 4
+# The same counters on the prefill GEMM of config 2 at M = 2048, N = 17408, K = 5120 (same file): gemm_q4_w2 and its
+# pack pass fetch 797.1 + 21.0 MB and write 242.5 + 21.0 MB per call, against 76.7 + 21.0 MB read and 142.6 MB written
+# algorithmically (the packed activations are re-read per XCD and group of weight-tile columns, out of the
+# Infinity Cache; K-sliced tail tiles write partial sums)
+MEASURED_GEMM_TRAFFIC_PER_LAUNCH = (797.1 + 21.0 + 242.5 + 21.0) * 1e6
 
 LAYER = [("qkv", 3072, 2048), ("o", 2048, 2048), ("gate_up", 12288, 2048), ("down", 2048, 6144)]
 
@@ -530,7 +535,7 @@ def main():
             "achieved": big["TFLOP/s"], "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": round(big["TFLOP/s"] / MFMA_F16_PEAK_TFLOPS, 4),
             "flops_per_launch": 2.0 * 2048 * 17408 * 5120, "avg_launch_us": round(big["ms"] * 1e3, 2),
-            "traffic": None,
+            "traffic": MEASURED_GEMM_TRAFFIC_PER_LAUNCH,
             "other_shapes_frac": {k_: round(v_["TFLOP/s"] / MFMA_F16_PEAK_TFLOPS, 4) for k_, v_ in gemm.items()},
         }
 

@@ -430,7 +430,8 @@ static int gemv_dispatch(lq4_ctx* ctx, const uint8_t* wp, uint32_t n, uint32_t k
         // 2048 x 2048: 4.67 -> 4.54, 5.09 -> 4.98; 3072 x 2048 at four rows 5.58 -> 4.82) and keeps 24 (up to four rows)
         // or 16 bits of every activation below its block's maximum instead of rounding it to f16.  Behind on long rows
         // and many rows (2048 x 6144 at eight rows 8.7 -> 10.4 us, 12288 x 2048 at four 7.8 -> 8.8), which stay where
-        // they were.
+        // they were.  With a LoRA epilogue alike (q+v of the 2B model at eight rows 17.6 -> 16.2 us), so that a
+        // projection is served by the same arithmetic with and without its adapter.
         launch_gemv_i8(wp, n, k, x_dev, k, batch, y_dev, n, ep, ctx->cu_count, s);
         ctx->counters.gemv++;
     } else {
@@ -539,7 +540,14 @@ int lq4_gemv_multi(lq4_ctx* ctx, const lq4_projection* proj, uint32_t count, uin
             ctx->counters.lora_a++;
         }
     }
-    if (stacked) {
+    // two to eight rows: the integer matrix-core kernel over the stacked rows, where it is the faster one
+    const bool stacked_rows = !stacked && batch >= 2 && batch <= 8 && mv.count > 1 && ctx->gemv_i8 &&
+                              (ctx->gemv_i8 == 2 || (k <= 2048 && mv.begin[mv.count] <= 4096)) &&
+                              gemv_i8_multi_serves(mv, k, batch, ctx->cu_count);
+    if (stacked_rows) {
+        launch_gemv_i8_multi(mv, k, x_dev, k, batch, ctx->cu_count, s);
+        ctx->counters.gemv_multi++;
+    } else if (stacked) {
         LoraEpilogue hand{};
         if (in_launch) {
             hand.rank = total_rank;

@@ -71,11 +71,14 @@ __device__ __forceinline__ float half_hi(uint32_t sb) {
 
 // WIDE: up to four activation rows at three digits; else up to eight at two.
 // CW x TW waves: CW waves split the chunks of one tile, TW tiles are worked on side by side.
-template <int CW, int TW, bool WIDE>
+// MULTI: the rows are those of several matrices stacked one under the other (MultiViews: view v = rows [begin[v],
+// begin[v + 1]), every view a whole number of 16-row tiles), each with its own output [batch, rows of the view] and its
+// own LoRA factors; w, y, y_stride and lora are then unused.
+template <int CW, int TW, bool WIDE, bool MULTI>
 __global__ __launch_bounds__(64 * CW * TW) void gemv_q4_i8(const uint8_t* __restrict__ w, uint32_t n, uint32_t k,
                                                            const float* __restrict__ x, uint32_t x_stride,
                                                            uint32_t batch, float* __restrict__ y, uint32_t y_stride,
-                                                           LoraEpilogue lora) {
+                                                           LoraEpilogue lora, MultiViews mv) {
     constexpr int WAVES = CW * TW;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int tid = threadIdx.x;
@@ -99,6 +102,15 @@ __global__ __launch_bounds__(64 * CW * TW) void gemv_q4_i8(const uint8_t* __rest
     const uint32_t my_tiles = tw < wg_tiles ? (wg_tiles - tw + TW - 1) / TW : 0;
     const uint32_t units = my_tiles * my_chunks;  // unit u = (my tile u / my_chunks, my chunk u % my_chunks)
     auto first_row = [&](uint32_t t) { return (blockIdx.x + (t * TW + tw) * gridDim.x) * 16; };
+    // MULTI: the view that holds stacked row `row` (uniform: called with a tile's first row)
+    auto view_of = [&](uint32_t row) {
+        uint32_t v = 0;
+        if constexpr (MULTI) {
+#pragma unroll
+            for (int i = 1; i < kMaxViews; ++i) v += (static_cast<uint32_t>(i) < mv.count && row >= mv.begin[i]) ? 1u : 0u;
+        }
+        return v;
+    };
 
     // load mapping: lane = (block jl, row rq), rows rq + kRowStep * i
     constexpr int kRowStep = 64 / kBpw, kLoads = 16 / kRowStep;
@@ -108,11 +120,20 @@ __global__ __launch_bounds__(64 * CW * TW) void gemv_q4_i8(const uint8_t* __rest
         const uint32_t row0 = first_row(t);
         uint32_t blk = (c * CW + cw) * kBpw + jl;
         if (blk >= nb) blk = nb - 1;
+        const uint8_t* wv = w;
+        uint32_t row_base = 0, row_end = n;
+        if constexpr (MULTI) {
+            const uint32_t v = view_of(row0);
+            wv = mv.w[v];
+            row_base = mv.begin[v];
+            row_end = mv.begin[v + 1];
+        }
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) {
             uint32_t row = row0 + rq + kRowStep * i;
-            if (row >= n) row = n - 1;
-            const uint8_t* bp = w + row * row_bytes + blk * static_cast<uint32_t>(kBlockBytes);
+            if (row >= row_end) row = row_end - 1;
+            row -= row_base;
+            const uint8_t* bp = wv + row * row_bytes + blk * static_cast<uint32_t>(kBlockBytes);
             // (plain loads: a unit's 160-byte pieces share their cache lines with the neighbouring waves' pieces)
             buf[i].sb = *reinterpret_cast<const uint32_t*>(bp);
             typedef uint32_t u32x4u __attribute__((ext_vector_type(4), aligned(4)));
@@ -313,23 +334,58 @@ __global__ __launch_bounds__(64 * CW * TW) void gemv_q4_i8(const uint8_t* __rest
             }
             if (cw == 0 && row < n) {
                 const uint32_t b0 = WIDE ? g : 2 * g, b1 = WIDE ? batch : 2 * g + 1;  // (wide: one row a lane)
-                if (lora.rank) {
-                    // (every load of this loop is used inside it and unconditional: a load left pending on one path
-                    // would make the compiler wait for the whole weight ring wherever its register is reused)
-                    const uint32_t t0 = (b0 < batch ? b0 : 0) * lora.rank, t1 = (b1 < batch ? b1 : 0) * lora.rank;
-                    float l0 = 0.0f, l1 = 0.0f;
-                    for (uint32_t i = 0; i < lora.rank; ++i) {
-                        const size_t bi = static_cast<size_t>(row) * lora.rank + i;
-                        const float bv = lora.b_is_f16 ? static_cast<float>(static_cast<const _Float16*>(lora.b)[bi])
-                                                       : static_cast<const float*>(lora.b)[bi];
-                        l0 = fmaf(bv, lora.t[t0 + i], l0);
-                        l1 = fmaf(bv, lora.t[t1 + i], l1);
-                    }
-                    acc0 = fmaf(lora.scale, l0, acc0);
-                    acc1 = fmaf(lora.scale, l1, acc1);
+                // this row's adapter and output: the launch's, or (several views) those of the tile's view
+                LoraEpilogue lo = lora;
+                float* yv = y;
+                uint32_t ys = y_stride, lrow = row;
+                if constexpr (MULTI) {
+                    const uint32_t v = view_of(first_row(t));
+                    lo.b = mv.b[v];
+                    lo.t = mv.t[v];
+                    lo.rank = mv.rank[v];
+                    lo.b_is_f16 = mv.b_is_f16[v];
+                    lo.scale = mv.scale[v];
+                    yv = mv.y[v];
+                    ys = mv.begin[v + 1] - mv.begin[v];
+                    lrow = row - mv.begin[v];
                 }
-                if (b0 < batch) y[static_cast<size_t>(b0) * y_stride + row] = acc0;
-                if (b1 < batch) y[static_cast<size_t>(b1) * y_stride + row] = acc1;
+                if (lo.rank) {
+                    // (every load below is unconditional and used where it is made: a load left pending on one path
+                    // would make the compiler wait for the whole weight ring wherever its register is reused)
+                    const float* t0 = lo.t + (b0 < batch ? b0 : 0) * lo.rank;
+                    const float* t1 = lo.t + (b1 < batch ? b1 : 0) * lo.rank;
+                    float l0 = 0.0f, l1 = 0.0f;
+                    if (lo.b_is_f16 && lo.rank % 8 == 0) {
+                        // eight factors a step: one 16-byte load of B[row, i..i+7] and four of t
+                        const _Float16* brow = static_cast<const _Float16*>(lo.b) + static_cast<size_t>(lrow) * lo.rank;
+                        for (uint32_t i = 0; i < lo.rank; i += 8) {
+                            struct alignas(16) H8 { _Float16 v[8]; };
+                            const H8 bq = *reinterpret_cast<const H8*>(brow + i);
+                            const float4 ta = *reinterpret_cast<const float4*>(t0 + i), tb = *reinterpret_cast<const float4*>(t0 + i + 4);
+                            const float4 ua = *reinterpret_cast<const float4*>(t1 + i), ub = *reinterpret_cast<const float4*>(t1 + i + 4);
+                            const float tv[8] = {ta.x, ta.y, ta.z, ta.w, tb.x, tb.y, tb.z, tb.w};
+                            const float uv[8] = {ua.x, ua.y, ua.z, ua.w, ub.x, ub.y, ub.z, ub.w};
+#pragma unroll
+                            for (int jj = 0; jj < 8; ++jj) {
+                                const float bv = static_cast<float>(bq.v[jj]);
+                                l0 = fmaf(bv, tv[jj], l0);
+                                l1 = fmaf(bv, uv[jj], l1);
+                            }
+                        }
+                    } else {
+                        for (uint32_t i = 0; i < lo.rank; ++i) {
+                            const size_t bi = static_cast<size_t>(lrow) * lo.rank + i;
+                            const float bv = lo.b_is_f16 ? static_cast<float>(static_cast<const _Float16*>(lo.b)[bi])
+                                                         : static_cast<const float*>(lo.b)[bi];
+                            l0 = fmaf(bv, t0[i], l0);
+                            l1 = fmaf(bv, t1[i], l1);
+                        }
+                    }
+                    acc0 = fmaf(lo.scale, l0, acc0);
+                    acc1 = fmaf(lo.scale, l1, acc1);
+                }
+                if (b0 < batch) yv[static_cast<size_t>(b0) * ys + lrow] = acc0;
+                if (b1 < batch) yv[static_cast<size_t>(b1) * ys + lrow] = acc1;
             }
             acc0 = 0.0f;
             acc1 = 0.0f;
@@ -389,27 +445,30 @@ bool plan_i8(uint32_t n, uint32_t k, uint32_t batch, uint32_t cu_count, I8Plan* 
     return true;
 }
 
-template <int CW, int TW, bool WIDE>
+template <int CW, int TW, bool WIDE, bool MULTI>
 void launch_i8(const I8Plan& p, const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint32_t x_stride,
-               uint32_t batch, float* y, uint32_t y_stride, const LoraEpilogue& lora, hipStream_t stream) {
+               uint32_t batch, float* y, uint32_t y_stride, const LoraEpilogue& lora, const MultiViews& mv,
+               hipStream_t stream) {
     static std::atomic<uint64_t> attr_set{0};  // one bit a device: the attribute belongs to the device's copy of the code
     int dev = 0;
     (void)hipGetDevice(&dev);
     const uint64_t bit = 1ull << (dev & 63);
     if (!(attr_set.load(std::memory_order_relaxed) & bit)) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_i8<CW, TW, WIDE>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_i8<CW, TW, WIDE, MULTI>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         attr_set.fetch_or(bit, std::memory_order_relaxed);
     }
-    hipLaunchKernelGGL((gemv_q4_i8<CW, TW, WIDE>), dim3(p.grid), dim3(64 * CW * TW), p.lds, stream, w, n, k, x, x_stride,
-                       batch, y, y_stride, lora);
+    hipLaunchKernelGGL((gemv_q4_i8<CW, TW, WIDE, MULTI>), dim3(p.grid), dim3(64 * CW * TW), p.lds, stream, w, n, k, x,
+                       x_stride, batch, y, y_stride, lora, mv);
 }
 
-template <bool WIDE>
+template <bool WIDE, bool MULTI>
 void launch_i8_shape(const I8Plan& p, const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint32_t x_stride,
-                     uint32_t batch, float* y, uint32_t y_stride, const LoraEpilogue& lora, hipStream_t stream) {
-#define LQ4_I8(CW_, TW_) \
-    if (p.cw == CW_ && p.tw == TW_) return launch_i8<CW_, TW_, WIDE>(p, w, n, k, x, x_stride, batch, y, y_stride, lora, stream)
+                     uint32_t batch, float* y, uint32_t y_stride, const LoraEpilogue& lora, const MultiViews& mv,
+                     hipStream_t stream) {
+#define LQ4_I8(CW_, TW_)                \
+    if (p.cw == CW_ && p.tw == TW_)     \
+    return launch_i8<CW_, TW_, WIDE, MULTI>(p, w, n, k, x, x_stride, batch, y, y_stride, lora, mv, stream)
     LQ4_I8(16, 1);
     LQ4_I8(8, 2); LQ4_I8(8, 1);
     LQ4_I8(4, 4); LQ4_I8(4, 2); LQ4_I8(4, 1);
@@ -429,8 +488,28 @@ void launch_gemv_i8(const uint8_t* w, uint32_t n, uint32_t k, const float* x, ui
                     float* y, uint32_t y_stride, const LoraEpilogue& lora, uint32_t cu_count, hipStream_t stream) {
     I8Plan p;
     if (!plan_i8(n, k, batch, cu_count, &p)) return;  // the caller asked gemv_i8_serves first
-    if (batch <= 4) launch_i8_shape<true>(p, w, n, k, x, x_stride, batch, y, y_stride, lora, stream);
-    else launch_i8_shape<false>(p, w, n, k, x, x_stride, batch, y, y_stride, lora, stream);
+    const MultiViews none{};
+    if (batch <= 4) launch_i8_shape<true, false>(p, w, n, k, x, x_stride, batch, y, y_stride, lora, none, stream);
+    else launch_i8_shape<false, false>(p, w, n, k, x, x_stride, batch, y, y_stride, lora, none, stream);
+}
+
+// The stacked launch serves views that are whole numbers of 16-row tiles.
+bool gemv_i8_multi_serves(const MultiViews& mv, uint32_t k, uint32_t batch, uint32_t cu_count) {
+    if (mv.count == 0 || mv.count > static_cast<uint32_t>(kMaxViews)) return false;
+    for (uint32_t v = 0; v < mv.count; ++v)
+        if ((mv.begin[v + 1] - mv.begin[v]) % 16) return false;
+    I8Plan p;
+    return plan_i8(mv.begin[mv.count], k, batch, cu_count, &p);
+}
+
+void launch_gemv_i8_multi(const MultiViews& mv, uint32_t k, const float* x, uint32_t x_stride, uint32_t batch,
+                          uint32_t cu_count, hipStream_t stream) {
+    const uint32_t n = mv.begin[mv.count];
+    I8Plan p;
+    if (!plan_i8(n, k, batch, cu_count, &p)) return;  // the caller asked gemv_i8_multi_serves first
+    const LoraEpilogue none{};
+    if (batch <= 4) launch_i8_shape<true, true>(p, nullptr, n, k, x, x_stride, batch, nullptr, 0, none, mv, stream);
+    else launch_i8_shape<false, true>(p, nullptr, n, k, x, x_stride, batch, nullptr, 0, none, mv, stream);
 }
 
 }  // namespace lq4

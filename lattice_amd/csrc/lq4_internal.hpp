@@ -65,6 +65,10 @@ struct LoraAViews {
     int a_is_f16[kMaxViews];
 };
 bool gemv_multi_serves(const MultiViews& mv, uint32_t k);
+// The same for 2..8 activation rows on the integer matrix-core kernel (views of whole 16-row tiles; t in memory).
+bool gemv_i8_multi_serves(const MultiViews& mv, uint32_t k, uint32_t batch, uint32_t cu_count);
+void launch_gemv_i8_multi(const MultiViews& mv, uint32_t k, const float* x, uint32_t x_stride, uint32_t batch,
+                          uint32_t cu_count, hipStream_t stream);
 // `in_launch`: null = every t_v is in memory; else the hand-over words (slots, sync, spin_limit, rank = the ranks' sum)
 // of a launch that computes the factors in producer workgroups of its own.
 void launch_gemv_multi(const MultiViews& mv, uint32_t k, const float* x, const LoraEpilogue* in_launch, hipStream_t stream);

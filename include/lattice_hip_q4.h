@@ -255,19 +255,11 @@ int lq4_topk(lq4_ctx* ctx, const float* logits_dev, uint32_t n, uint32_t top_k, 
  * GEMV, f32-faithful) are kept in library scratch and never handed to the caller; the top_k
  * best (logit, token id) pairs come back in rank order.  Both stages are exact, so the result
  * equals lq4_gemv followed by lq4_topk.
- * By default the GEMV and the selection are two launches.  lq4_set_lm_head_mode(LQ4_LM_HEAD_ONE_LAUNCH)
- * makes the selection part of the GEMV's own launch, as lm_head_block_topk_q4 computes its block
- * candidates inside the GEMV kernel: every workgroup publishes the best of the logits it produced
- * (written with device-scope stores) and the workgroup that finishes last selects.  Served for
- * top_k <= 64 and rows the one-token kernel takes 64 blocks at a time (K >= 2048 other than the 512-
- * and 1024-wide forms), between top_k and 1024 workgroups; other shapes keep two launches.  The
- * results are the same bits either way.  On MI355X the one-launch form is the slower one (248 320 x
- * 2048, top 50: 82.9 us against 76.7): making the logits visible to the selecting workgroup inside
- * the launch (write-through stores, their acknowledgement, the maximum's exchange and the ticket, one
- * after the other at the end of every workgroup) costs more than the second launch's pass over 1 MB
- * of logits.  The setting belongs to the context. */
-enum { LQ4_LM_HEAD_ONE_LAUNCH = 0, LQ4_LM_HEAD_TWO_LAUNCHES = 1 };
-int lq4_set_lm_head_mode(lq4_ctx* ctx, int mode);
+ * The GEMV and the selection are two launches.  (A form that selected inside the GEMV's own launch, as
+ * lm_head_block_topk_q4 computes its block candidates inside the GEMV kernel, existed and was removed: making the
+ * logits visible to the selecting workgroup inside the launch - write-through stores, their acknowledgement, the
+ * maximum's exchange and a ticket, one after the other at the end of every workgroup - cost more than the second
+ * launch's pass over 1 MB of logits: 248 320 x 2048, top 50: 82.9 us against 76.7.) */
 int lq4_lm_head_topk(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t vocab, uint32_t k,
                      const float* x_dev, uint32_t top_k, float* out_logits_dev, uint32_t* out_ids_dev,
                      void* stream);
@@ -493,7 +485,6 @@ typedef struct lq4_path_counters {
     uint64_t lora_t_fallback;  /* waves of one-token LoRA launches that computed A.x themselves because
                                   the producers' hand-over did not arrive in time (read from the device:
                                   this call waits for the GPU) */
-    uint64_t lm_head_one_launch; /* lq4_lm_head_topk calls whose GEMV selected the top-k in its own launch */
     uint64_t gemv_multi;       /* lq4_gemv_multi calls served by one stacked launch */
 } lq4_path_counters;
 int lq4_get_path_counters(const lq4_ctx* ctx, lq4_path_counters* out);

@@ -103,7 +103,6 @@ pub struct Lq4PathCounters {
     pub elementwise: u64,
     pub gemv_chain: u64,
     pub lora_t_fallback: u64,
-    pub lm_head_one_launch: u64,
     pub gemv_multi: u64,
 }
 
@@ -241,8 +240,6 @@ extern "C" {
         lora_scale: f32,
         stream: *mut c_void,
     ) -> c_int;
-    pub fn lq4_gemv_chain(ctx: *mut Lq4Ctx, steps: *const Lq4ChainStep, n_steps: u32, stream: *mut c_void) -> c_int;
-    pub fn lq4_set_lm_head_mode(ctx: *mut Lq4Ctx, mode: c_int) -> c_int;
 
     // ---- MoE
     pub fn lq4_moe_route(

@@ -55,7 +55,7 @@ EXPORTS = [
     "lq4_set_gemm_kernel",
     "lq4_residual_add_rmsnorm", "lq4_silu_mul", "lq4_add_and_copy", "lq4_gemv_fused", "lq4_gemv_fused_batch",
     "lq4_lm_head_topk_static",
-    "lq4_gemv_chain", "lq4_set_lm_head_mode", "lq4_ctx_reserve_scratch",
+    "lq4_gemv_chain", "lq4_ctx_reserve_scratch",
     "lq4_gemv_q8", "lq4_gemm_q8", "lq4_gemv_q3", "lq4_gemm_q3",
     "lq4_get_path_counters", "lq4_malloc", "lq4_free", "lq4_memcpy_h2d", "lq4_memcpy_d2h",
 ]
@@ -77,7 +77,7 @@ class Q4Error(RuntimeError):
 class PathCounters(C.Structure):
     _fields_ = [(n, C.c_uint64) for n in ("gemv", "gemm", "lora_a", "moe_route", "moe_gate_up",
                                          "moe_down", "dequant", "topk", "gemv_fused", "elementwise",
-                                         "gemv_chain", "lora_t_fallback", "lm_head_one_launch", "gemv_multi")]
+                                         "gemv_chain", "lora_t_fallback", "gemv_multi")]
 
 
 MAX_PROJECTIONS = 8
@@ -92,7 +92,6 @@ class Projection(C.Structure):
 LQ4_PRO_NONE, LQ4_PRO_ADD_RMSNORM, LQ4_PRO_SILU_MUL = 0, 1, 2
 LQ4_EPI_NONE, LQ4_EPI_ADD_RESIDUAL, LQ4_EPI_SILU_MUL_PAIRS = 0, 1, 2
 CHAIN_MAX_STEPS = 16
-LM_HEAD_ONE_LAUNCH, LM_HEAD_TWO_LAUNCHES = 0, 1  # lq4_set_lm_head_mode
 GEMV_KERNEL_AUTO, GEMV_KERNEL_LANE_BLOCKS, GEMV_KERNEL_LDS_RING = 0, 1, 2  # lq4_set_gemv_kernel
 
 
@@ -168,7 +167,6 @@ def load_library() -> C.CDLL:
         "lq4_gemv_fused_batch": (C.c_int, [vp, vp, C.c_uint64, C.c_uint32, C.c_uint32, vp, C.c_uint32, vp,
                                            C.POINTER(GemvFusion), vp, C.c_float, vp]),
         "lq4_gemv_chain": (C.c_int, [vp, C.POINTER(ChainStep), C.c_uint32, vp]),
-        "lq4_set_lm_head_mode": (C.c_int, [vp, C.c_int]),
         "lq4_ctx_reserve_scratch": (C.c_int, [vp, C.c_size_t]),
         "lq4_get_path_counters": (C.c_int, [vp, C.POINTER(PathCounters)]),
         "lq4_malloc": (C.c_int, [vp, C.c_size_t, C.POINTER(vp)]),
@@ -615,11 +613,6 @@ class HipQ4Backend:
         _check(fn(self.ctx, qw.handle, qw_extra_offset, vocab, k, x.data_ptr(), top_k,
                   out_l.data_ptr(), out_i.data_ptr(), self._stream()))
         return out_l, out_i
-
-    def set_lm_head_mode(self, mode: int):
-        """``LM_HEAD_TWO_LAUNCHES`` (default): GEMV, then the selection kernel; ``LM_HEAD_ONE_LAUNCH``:
-        the lm_head GEMV selects the top-k in its own launch where the shape allows."""
-        _check(self.lib.lq4_set_lm_head_mode(self.ctx, int(mode)))
 
     # -------------------------------------------------------------------- LoRA
     def load_lora_adapter(self, layers: List[LoraLayerData], scale: float,

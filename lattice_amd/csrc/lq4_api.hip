@@ -41,7 +41,6 @@ struct lq4_ctx {
     hipStream_t state_stream;
     bool state_stream_known;
     hipEvent_t state_event;  // recorded on the previous stream when a call arrives on another one
-    int lm_head_mode;        // lq4_set_lm_head_mode
     int gemm_kernel;         // lq4_set_gemm_kernel
     int gemv_kernel;         // lq4_set_gemv_kernel: which kernel serves a plain one-token GEMV
     int gemv_i8;             // LQ4_GEMV_I8: 1 = 3..8 rows of small matrices take the integer matrix-core kernel (default),
@@ -233,7 +232,6 @@ int lq4_ctx_create(int device_ordinal, lq4_ctx** out) {
         delete c;
         return fail(LQ4_E_HIP, "hipEventCreate: %s", hipGetErrorString(e));
     }
-    c->lm_head_mode = LQ4_LM_HEAD_TWO_LAUNCHES;  // measured faster: see lq4_set_lm_head_mode in the header
     c->gemm_kernel = gemm_kernel_choice_default();
     c->gemv_kernel = getenv("LQ4_GEMV_KERNEL") ? atoi(getenv("LQ4_GEMV_KERNEL")) : 0;
     if (c->gemv_kernel < 0 || c->gemv_kernel > 2) c->gemv_kernel = 0;
@@ -1077,12 +1075,8 @@ int lq4_topk(lq4_ctx* ctx, const float* logits_dev, uint32_t n, uint32_t top_k, 
 namespace {
 
 
-// Scratch of one lm_head + top-k call: [vocab logits | maxima, candidates], in the layout of whichever
-// path serves the shape.
-size_t lm_head_scratch_need(int mode, uint32_t vocab, uint32_t k, uint32_t top_k, bool* one_launch) {
-    const size_t fused = mode == LQ4_LM_HEAD_ONE_LAUNCH ? gemv_b1_topk_scratch_bytes(vocab, k, top_k) : 0;
-    *one_launch = fused != 0;
-    if (fused) return fused;
+// Scratch of one lm_head + top-k call: [vocab logits | maxima, candidates].
+size_t lm_head_scratch_need(uint32_t vocab, uint32_t top_k) {
     const size_t logits_bytes = (static_cast<size_t>(vocab) * sizeof(float) + 255) / 256 * 256;
     return logits_bytes + topk_scratch_bytes(vocab, top_k);
 }
@@ -1099,8 +1093,7 @@ int lm_head_topk_common(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offs
     if (rc) return rc;
     if (!x_dev || !out_logits_dev || !out_ids_dev) return fail(LQ4_E_INVALID, "null device pointer");
     if (reinterpret_cast<uintptr_t>(x_dev) % 16) return fail(LQ4_E_INVALID, "x must be 16-byte aligned");
-    bool one_launch;
-    const size_t need = lm_head_scratch_need(ctx->lm_head_mode, vocab, k, top_k, &one_launch);
+    const size_t need = lm_head_scratch_need(vocab, top_k);
     hipStream_t s = static_cast<hipStream_t>(stream);
     DeviceGuard g(ctx->device);
     uint8_t* base;
@@ -1117,29 +1110,16 @@ int lm_head_topk_common(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offs
         if (rc) return rc;
         base = ctx->moe_scratch;
     }
-    if (one_launch) {
-        launch_gemv_b1_topk(wp, vocab, k, x_dev, base, ctx->topk_ticket, top_k, out_logits_dev, out_ids_dev, s);
-        ctx->counters.lm_head_one_launch++;
-    } else {
-        const size_t logits_bytes = (static_cast<size_t>(vocab) * sizeof(float) + 255) / 256 * 256;
-        float* logits = reinterpret_cast<float*>(base);
-        plain_gemv_one_token(ctx, wp, vocab, k, x_dev, logits, s);
-        launch_topk(logits, vocab, top_k, base + logits_bytes, ctx->topk_ticket, out_logits_dev, out_ids_dev, s);
-        ctx->counters.topk++;
-    }
+    const size_t logits_bytes = (static_cast<size_t>(vocab) * sizeof(float) + 255) / 256 * 256;
+    float* logits = reinterpret_cast<float*>(base);
+    plain_gemv_one_token(ctx, wp, vocab, k, x_dev, logits, s);
+    launch_topk(logits, vocab, top_k, base + logits_bytes, ctx->topk_ticket, out_logits_dev, out_ids_dev, s);
+    ctx->counters.topk++;
     LQ4_HIP(hipGetLastError());
     return LQ4_OK;
 }
 
 }  // namespace
-
-int lq4_set_lm_head_mode(lq4_ctx* ctx, int mode) {
-    if (!ctx) return fail(LQ4_E_INVALID, "ctx is null");
-    if (mode != LQ4_LM_HEAD_ONE_LAUNCH && mode != LQ4_LM_HEAD_TWO_LAUNCHES)
-        return fail(LQ4_E_INVALID, "unknown lm_head mode %d", mode);
-    ctx->lm_head_mode = mode;
-    return LQ4_OK;
-}
 
 int lq4_lm_head_topk(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_t vocab, uint32_t k,
                      const float* x_dev, uint32_t top_k, float* out_logits_dev, uint32_t* out_ids_dev,

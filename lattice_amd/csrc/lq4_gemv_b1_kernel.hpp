@@ -14,7 +14,6 @@
 // scaled fixed-point activations) and the LDS staging are in lq4_b1_dev.hpp, shared with the decode-chain
 // kernel and the per-pair MoE kernels.
 #include "lq4_b1_dev.hpp"
-#include "lq4_topk_dev.hpp"
 
 #include <type_traits>
 
@@ -118,15 +117,6 @@ __device__ __forceinline__ float lora_t_acquire(const LoraEpilogue& lora, uint32
 }
 
 struct NoFusion {};
-// What the top-k mode needs beside the GEMV's own arguments: y is then the logits buffer.
-struct TopkEpilogue {
-    uint64_t* maxima;   // [workgroups] best key of each workgroup's rows
-    Cand* surv;         // topk_most_blocks(k) * (rows of one workgroup, rounded up to whole runs) candidates
-    uint32_t* ticket;   // zero between launches
-    uint32_t k;
-    float* out_logits;
-    uint32_t* out_ids;
-};
 template <int MODE>
 struct FusionArg {
     typedef NoFusion type;
@@ -134,10 +124,6 @@ struct FusionArg {
 template <>
 struct FusionArg<1> {
     typedef GemvFusion type;
-};
-template <>
-struct FusionArg<3> {
-    typedef TopkEpilogue type;
 };
 template <>
 struct FusionArg<5> {
@@ -161,12 +147,6 @@ struct FusionArg<7> {
 // complete, as a rule long after it was published.  The wait is bounded: a wave that runs out of polls
 // computes t itself, so every wave finishes whatever the dispatch order was.
 // 4 plain, with the row order of a persistent grid (see ADJ below).
-// 3 the lm_head pass with the exact top-k selection in the same launch (shaders/qwen35.metal:1935-1985
-// computes block candidates inside the GEMV kernel too): the logits go to `y` with device-scope stores,
-// every wave keeps the best key among the rows it produced, the workgroup publishes the best of its
-// waves and draws a ticket, and the workgroup that draws the last one (every logit and every maximum
-// is then in memory) runs the selection tail over those maxima.  A workgroup's rows are its selection
-// block; in this mode they are consecutive (every wave takes a run of wave-rows).
 // 6 several matrices with rows of the same K against one x (MultiViews): the launch walks the rows of the matrices
 // stacked one under the other, view v holding rows [begin[v], begin[v + 1]); a wave-row never straddles two views
 // (the launcher sees to it), so the view of a wave-row is uniform across the wave.  Each view has its own output
@@ -174,7 +154,7 @@ struct FusionArg<7> {
 // 7 the same with the adapters' factors computed inside the launch as in mode 2: the A matrices of the views
 // stacked (at most 64 rows in all), one producer workgroup a row in front of the weight workgroups; lane l of a
 // weight wave picks up t of stacked row l, view v's factors start at lane t_off[v].
-constexpr int kPlainMode = 0, kFusedMode = 1, kLoraAMode = 2, kTopkMode = 3, kPlainAdjMode = 4, kFusedPairsMode = 5,
+constexpr int kPlainMode = 0, kFusedMode = 1, kLoraAMode = 2, kPlainAdjMode = 4, kFusedPairsMode = 5,
               kMultiMode = 6, kMultiLoraAMode = 7;
 
 template <int RW, int SG, int SEG, int MODE, int WAVES = kWaves>
@@ -246,15 +226,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
     // against 4.1), and the choice as a run-time flag cost those launches 6-11 %: hence a mode of its own.
     constexpr bool ADJ = MODE == kPlainAdjMode;
     if constexpr (ADJ) chunks = wid * RW < n_wrows ? (n_wrows - wid * RW + n_waves * RW - 1) / (n_waves * RW) : 0;
-    // kTopkMode: a wave takes `per_wave` consecutive wave-rows instead, so that the logits of one
-    // workgroup are one run in memory (the workgroup that selects reads the best workgroups' logits:
-    // scattered over the vector they are a cache line each)
-    const uint32_t per_wave = (n_wrows + n_waves - 1) / n_waves;
-    if constexpr (MODE == kTopkMode) {
-        const uint32_t begin = wid * per_wave;
-        const uint32_t mine = begin < n_wrows ? (n_wrows - begin < per_wave ? n_wrows - begin : per_wave) : 0;
-        chunks = (mine + RW - 1) / RW;
-    }
     // Fused epilogue kSiluMulPairs (W = [gate rows | up rows], n / 2 of each; rows of 64 lanes, RW even): the
     // wave's rounds come in pairs, rounds 2i and 2i + 1 are the gate and the up row of pair i * n_waves + wid, so
     // that the wave itself forms silu(g) * u when the second row of a pair completes.
@@ -266,7 +237,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
     }
     // wave-row of round r = chunk * RW + j, and whether this wave owns it
     auto wrow_of = [&](uint32_t r) {
-        if (MODE == kTopkMode) return wid * per_wave + r;
         if (PAIRS) {
             const uint32_t pair = (r >> 1) * n_waves + wid;
             return (r & 1) ? n_pairs + pair : pair;  // (a pair past the end: past n, or an up row; clamped or dropped)
@@ -275,7 +245,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
     };
     auto wrow_mine = [&](uint32_t r) {
         if (PAIRS) return (r >> 1) * n_waves + wid < n_pairs;
-        return wrow_of(r) < n_wrows && (MODE != kTopkMode || r < per_wave);
+        return wrow_of(r) < n_wrows;
     };
     const uint32_t units = chunks * slab_groups;
     // kMultiMode: the view that holds stacked row `row` (uniform: called with the first row of a wave-row)
@@ -537,7 +507,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
     float acc[RW];
 #pragma unroll
     for (int j = 0; j < RW; ++j) acc[j] = 0.0f;
-    uint64_t best_key = key_of(sentinel());  // kTopkMode: best of the rows this lane stored
     float gate_kept = 0.0f;                  // kSiluMulPairs: the gate row's sum until the pair's up row is done
     float t_reg = 0.0f;   // kLoraAMode: t[lane], fetched when the wave's first rows are complete
     bool t_have = false;
@@ -659,11 +628,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
                             fz.residual[row] = r;
                             if (fz.copy_dst) fz.copy_dst[row] = r;
                         }
-                    } else if constexpr (MODE == kTopkMode) {
-                        // device scope: written through to where the workgroup that selects reads it
-                        __hip_atomic_store(y + row, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        const uint64_t key = key_of(v == v ? Cand{v, row} : sentinel());
-                        best_key = key > best_key ? key : best_key;
                     } else if constexpr (MULTI) {
                         const uint32_t vw = view_of(wrow * RPW);  // (row_ok: the wave-row exists)
                         fz.y[vw][row - fz.begin[vw]] = v;
@@ -691,36 +655,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4_b1(const uint8_t* __restri
         process(kLast, buf_a, buf_b, u);
     }
 
-    if constexpr (MODE == kTopkMode) {
-        static_assert(WAVES == 4, "the selection tail is written for 256 threads");
-        // this wave's logit stores have been carried out (a store counts as outstanding until then)
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        best_key = wave_max_key(best_key);
-        __syncthreads();  // every wave is past the staged activations: the LDS is free
-        TopkTailShared& ts = *reinterpret_cast<TopkTailShared*>(xs);
-        uint64_t* part = reinterpret_cast<uint64_t*>(reinterpret_cast<uint8_t*>(xs) + sizeof(TopkTailShared));  // [WAVES], then the flag
-        uint32_t* last_flag = reinterpret_cast<uint32_t*>(part + WAVES);
-        if (lane == 0) part[tid >> 6] = best_key;
-        __syncthreads();
-        if (tid == 0) {
-            uint64_t best = part[0];
-#pragma unroll
-            for (int v = 1; v < WAVES; ++v) best = part[v] > best ? part[v] : best;
-            // An exchange at device scope is carried out where every part of the chip sees it, and once
-            // its old value has come back it is done; only then is the ticket drawn.
-            const uint64_t old = __hip_atomic_exchange(fz.maxima + w_group, best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            asm volatile("s_waitcnt vmcnt(0)" ::"v"(static_cast<uint32_t>(old)) : "memory");
-            const uint32_t t = atomicAdd(fz.ticket, 1u);
-            const bool last = t == w_groups - 1;
-            if (last) __hip_atomic_store(fz.ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
-            *last_flag = last;
-        }
-        __syncthreads();
-        if (!*last_flag) return;
-        __syncthreads();  // the flag has been read by all before the tail reuses the LDS
-        const TopkBlocks blocks{WAVES * per_wave * RPW, 0, 1};  // a workgroup's logits: one run
-        topk_select_tail<true>(y, n, blocks, w_groups, fz.k, fz.maxima, fz.surv, ts, fz.out_logits, fz.out_ids);
-    }
 }
 
 // Grid shape of one launch: waves in all, wave-rows per chunk, slabs per unit.

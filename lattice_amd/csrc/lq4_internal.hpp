@@ -122,13 +122,6 @@ bool gemv_dma_serves(uint32_t n, uint32_t k, uint32_t cu_count);
 bool gemv_dma_pays(uint32_t n, uint32_t k, uint32_t cu_count);
 void launch_gemv_dma(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, uint32_t cu_count, hipStream_t stream);
 // Same with fused elementwise steps (separate kernel instantiations; the plain ones are untouched).
-// The lm_head pass with the exact top-k selected in the same launch: logits (kept in `scratch`), block
-// maxima and survivors live in `scratch` of gemv_b1_topk_scratch_bytes(n, k, topk) bytes; 0 bytes means
-// the shape is not served (the caller then runs GEMV and top-k as two launches).  `ticket`: a counter
-// that is zero between launches.
-size_t gemv_b1_topk_scratch_bytes(uint32_t n, uint32_t k, uint32_t topk);
-void launch_gemv_b1_topk(const uint8_t* w, uint32_t n, uint32_t k, const float* x, void* scratch, uint32_t* ticket,
-                         uint32_t topk, float* out_logits, uint32_t* out_ids, hipStream_t stream);
 void launch_gemv_b1_fused(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y,
                           const LoraEpilogue& lora, const GemvFusion& fusion, hipStream_t stream);
 

@@ -144,48 +144,36 @@ def _lm_head_cases():
 
 
 @pytest.mark.gpu
-def test_gpu_lm_head_selection_inside_the_gemv_launch_matches_two_launches():
+def test_gpu_lm_head_topk_is_the_exact_topk_of_the_gemv_logits():
     import torch
     from lattice_amd import backend
     be = backend.HipQ4Backend(0)
     try:
-        served = 0
         for name, vocab, k, top_k, wq, x in _lm_head_cases():
-            print(f"lm_head one launch vs two: {name}", flush=True)
+            print(f"lm_head top-k: {name}", flush=True)
             qw = be.upload_q4_blocks(wq)
             xd = torch.from_numpy(x).cuda()
-            be.set_lm_head_mode(backend.LM_HEAD_TWO_LAUNCHES)
-            two_l, two_i = be.lm_head_topk(xd, qw, vocab, k, top_k)
-            two_l, two_i = two_l.cpu().numpy().view(np.uint32), two_i.cpu().numpy().view(np.uint32)
-            be.set_lm_head_mode(backend.LM_HEAD_ONE_LAUNCH)
-            before = be.path_counters()["lm_head_one_launch"]
-            for rep in range(3):  # the ticket and the maxima are shared by back-to-back calls
-                one_l, one_i = be.lm_head_topk(xd, qw, vocab, k, top_k)
-                assert np.array_equal(one_i.cpu().numpy().view(np.uint32), two_i), (name, rep)
-                assert np.array_equal(one_l.cpu().numpy().view(np.uint32), two_l), (name, rep)
-            served += be.path_counters()["lm_head_one_launch"] - before
-            # and both are the exact top-k of the GEMV's logits
             y = torch.empty((1, vocab), dtype=torch.float32, device="cuda")
             be.dispatch_matmul(xd, qw, y, 1, vocab, k)
             ref_l, ref_i = oracle.topk(y.cpu().numpy().reshape(-1), top_k)
-            assert np.array_equal(two_i, ref_i), name
-            assert np.array_equal(two_l, ref_l.view(np.uint32)), name
+            for rep in range(3):  # the ticket and the maxima are shared by back-to-back calls
+                two_l, two_i = be.lm_head_topk(xd, qw, vocab, k, top_k)
+                two_l, two_i = two_l.cpu().numpy().view(np.uint32), two_i.cpu().numpy().view(np.uint32)
+                assert np.array_equal(two_i, ref_i), (name, rep)
+                assert np.array_equal(two_l, ref_l.view(np.uint32)), (name, rep)
             if name == "exact_ties":
                 # the best row's copies, lower token ids first
                 assert np.array_equal(two_i, two_i[0] + 37 * np.arange(top_k, dtype=np.uint32)) and two_i[0] < 37
             if name == "all_nan_logits":
                 assert np.all(two_i == 0xFFFFFFFF) and np.isnan(y.cpu().numpy()).all()
-        # every case but the tiny vocabulary, the 1024-wide rows and top_k 65 went through the one-launch form
-        assert served == 3 * (len(_lm_head_cases()) - 3), served
     finally:
-        be.set_lm_head_mode(backend.LM_HEAD_TWO_LAUNCHES)
         be.close()
 
 
 @pytest.mark.gpu
-def test_gpu_lm_head_one_launch_alternating_inputs():
+def test_gpu_lm_head_topk_alternating_inputs():
     """Calls that alternate between two vocabularies and activations share the logits buffer, the
-    maxima and the ticket: each call must select from its own launch's values."""
+    maxima and the ticket: each call must select from its own launches' values."""
     import torch
     from lattice_amd import backend
     be = backend.HipQ4Backend(0)
@@ -198,16 +186,13 @@ def test_gpu_lm_head_one_launch_alternating_inputs():
         y = torch.empty((1, vocab), dtype=torch.float32, device="cuda")
         be.dispatch_matmul(xd, qw, y, 1, vocab, k)
         sets.append((vocab, qw, xd, oracle.topk(y.cpu().numpy().reshape(-1), 50)))
-    be.set_lm_head_mode(backend.LM_HEAD_ONE_LAUNCH)
     try:
         for it in range(40):
             vocab, qw, xd, (ref_l, ref_i) = sets[it % 2]
             out_l, out_i = be.lm_head_topk(xd, qw, vocab, k, 50)
             assert np.array_equal(out_i.cpu().numpy().view(np.uint32), ref_i), it
             assert np.array_equal(out_l.cpu().numpy().view(np.uint32), ref_l.view(np.uint32)), it
-        assert be.path_counters()["lm_head_one_launch"] == 40
     finally:
-        be.set_lm_head_mode(backend.LM_HEAD_TWO_LAUNCHES)
         be.close()
 
 

@@ -33,18 +33,12 @@ def test_static_scratch_lm_head_topk_matches_the_allocating_entry_point():
 
     # the larger input first, then a smaller one that finds the first call's logits and candidates
     # still in the array; a third, larger again
-    # (the 2048-wide ones are served by the one-launch form when that mode is on: run in both modes)
-    try:
-        for mode in (backend.LM_HEAD_TWO_LAUNCHES, backend.LM_HEAD_ONE_LAUNCH):
-            be.set_lm_head_mode(mode)
-            for vocab, k, top_k, seed in [(40000, 1024, 50, 5), (9000, 512, 8, 6), (65536 + 3, 256, 200, 7),
-                                          (50000, 2048, 50, 8), (7000, 2048, 8, 9)]:
-                (got_l, got_i), (want_l, want_i) = both(vocab, k, top_k, seed)
-                assert np.array_equal(got_i, want_i), (mode, vocab, k, top_k)
-                assert np.array_equal(got_l, want_l), (mode, vocab, k, top_k)
-                assert got_i.max() < vocab
-    finally:
-        be.set_lm_head_mode(backend.LM_HEAD_TWO_LAUNCHES)
+    for vocab, k, top_k, seed in [(40000, 1024, 50, 5), (9000, 512, 8, 6), (65536 + 3, 256, 200, 7),
+                                  (50000, 2048, 50, 8), (7000, 2048, 8, 9)]:
+        (got_l, got_i), (want_l, want_i) = both(vocab, k, top_k, seed)
+        assert np.array_equal(got_i, want_i), (vocab, k, top_k)
+        assert np.array_equal(got_l, want_l), (vocab, k, top_k)
+        assert got_i.max() < vocab
 
     # beyond the static array: refused with a clear error, nothing launched
     big_vocab, k = 600000, 32

@@ -491,12 +491,8 @@ void launch_tile(const uint8_t* w, uint32_t n, uint32_t k, const void* x, uint32
     if (!partial || (LORA && lora.rank)) ts = TileSlices{1, (k / kBlockWeights + 1) / 2};
     const KSlices slices{ts.count, ts.steps, partial};
     const size_t lds = 2 * (BM + BN_) * kPitch * sizeof(_Float16);
-    static bool attr_set = false;
-    if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4_mfma<X_F16, BN_, LORA, FMT>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        attr_set = true;
-    }
+    static LdsCapOnce lds_cap;
+    lds_cap.raise(reinterpret_cast<const void*>(gemm_q4_mfma<X_F16, BN_, LORA, FMT>), 160 * 1024);
     hipLaunchKernelGGL((gemm_q4_mfma<X_F16, BN_, LORA, FMT>), dim3(tiles * ts.count), dim3(2 * BN_), lds, stream, w, n,
                        k, x, m, y, lora, slices);
     if (ts.count > 1)

@@ -927,12 +927,8 @@ namespace {
 template <bool X_F16, bool LORA, int FMT>
 void launch_wreg_t(const uint8_t* w, uint32_t n, uint32_t k, const void* x, uint32_t m, float* y,
                    const LoraEpilogue& lora, const HostPlan& hp, float* partial, hipStream_t stream) {
-    static bool attr_set = false;
-    if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4_wreg<X_F16, LORA, FMT>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        attr_set = true;
-    }
+    static LdsCapOnce lds_cap;
+    lds_cap.raise(reinterpret_cast<const void*>(gemm_q4_wreg<X_F16, LORA, FMT>), 160 * 1024);
     const size_t lds = 2 * kBuf16 * sizeof(uint4);
     const WregPlan plan{hp.full, hp.slices, partial};
     const uint32_t wgs = hp.full + (hp.tiles - hp.full) * hp.slices;
@@ -993,11 +989,8 @@ void launch_gemm_w2(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int
     const uint64_t units = w2_packed_bytes(k, m) / 16;
     hipLaunchKernelGGL(pack_x_tiles_kernel, dim3(static_cast<uint32_t>((units + 255) / 256)), dim3(256), 0, stream, x,
                        x_is_f16, m, k, kc_pad, packed, units);
-    static bool attr_set = false;
-    if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4_w2), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
-        attr_set = true;
-    }
+    static LdsCapOnce lds_cap;
+    lds_cap.raise(reinterpret_cast<const void*>(gemm_q4_w2), 64 * 1024);
     const size_t lds = 2 * kStepUnits * sizeof(uint4);
     const WregPlan plan{hp.full, hp.slices, partial};
     const uint32_t wgs = hp.full + (hp.tiles - hp.full) * hp.slices;

@@ -8,37 +8,25 @@ namespace {
 template <int RW, int SG, int SEG, int WAVES = kWaves>
 void launch_cfg(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, const LoraEpilogue& lora,
                 const GemvFusion* fusion, size_t lds, uint32_t waves, bool persistent, hipStream_t stream) {
-    static bool attr_set[4] = {false, false, false, false};  // raise the dynamic-LDS cap once per instantiation
+    static LdsCapOnce cap[4];  // one per kernel mode of this instantiation
     const dim3 grid((waves + WAVES - 1) / WAVES), block(WAVES * 64);
     if constexpr (RW % 2 == 0 && SEG == 64) {
         if (fusion && fusion->epilogue == GemvFusion::kSiluMulPairs) {
-            static bool attr_pairs = false;
-            if (!attr_pairs) {
-                (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, kFusedPairsMode, WAVES>),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, 159 * 1024);
-                attr_pairs = true;
-            }
+            static LdsCapOnce cap_pairs;
+            cap_pairs.raise(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, kFusedPairsMode, WAVES>), 159 * 1024);
             hipLaunchKernelGGL((gemv_q4_b1<RW, SG, SEG, kFusedPairsMode, WAVES>), grid, block, lds, stream, w, n, k, x, y,
                                lora, *fusion);
             return;
         }
     }
     if (fusion) {
-        if (!attr_set[1]) {
-            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, kFusedMode, WAVES>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, 159 * 1024);
-            attr_set[1] = true;
-        }
+        cap[1].raise(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, kFusedMode, WAVES>), 159 * 1024);
         hipLaunchKernelGGL((gemv_q4_b1<RW, SG, SEG, kFusedMode, WAVES>), grid, block, lds, stream, w, n, k, x, y, lora,
                            *fusion);
         return;
     }
     if (lora.rank && lora.a) {
-        if (!attr_set[2]) {
-            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, kLoraAMode, WAVES>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-            attr_set[2] = true;
-        }
+        cap[2].raise(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, kLoraAMode, WAVES>), 160 * 1024);
         const dim3 grid_a(grid.x + lora.rank);  // the rank producer workgroups come first
         hipLaunchKernelGGL((gemv_q4_b1<RW, SG, SEG, kLoraAMode, WAVES>), grid_a, block, lds, stream, w, n, k, x, y,
                            lora, NoFusion{});
@@ -46,21 +34,13 @@ void launch_cfg(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float*
     }
     if constexpr (RW > 1) {  // (one row per chunk: both row orders are the same)
         if (persistent) {
-            if (!attr_set[3]) {
-                (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, kPlainAdjMode, WAVES>),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-                attr_set[3] = true;
-            }
+            cap[3].raise(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, kPlainAdjMode, WAVES>), 160 * 1024);
             hipLaunchKernelGGL((gemv_q4_b1<RW, SG, SEG, kPlainAdjMode, WAVES>), grid, block, lds, stream, w, n, k, x, y,
                                lora, NoFusion{});
             return;
         }
     }
-    if (!attr_set[0]) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, kPlainMode, WAVES>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        attr_set[0] = true;
-    }
+    cap[0].raise(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, kPlainMode, WAVES>), 160 * 1024);
     hipLaunchKernelGGL((gemv_q4_b1<RW, SG, SEG, kPlainMode, WAVES>), grid, block, lds, stream, w, n, k, x, y, lora,
                        NoFusion{});
 }

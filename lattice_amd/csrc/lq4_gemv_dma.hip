@@ -44,7 +44,6 @@
 // One workgroup of sixteen waves per CU: the activations are staged once per CU, by as many waves as the vector
 // has 512-element pieces (the others skip the staging code altogether, which on short rows is most of what a
 // wave of the lane-owns-block kernel executes).
-#include <atomic>
 #include "lq4_b1_dev.hpp"
 
 #include <type_traits>
@@ -355,15 +354,8 @@ bool plan_dma(uint32_t n, uint32_t k, uint32_t cu_count, DmaPlan* out) {
 
 template <int XR, int D, int SLABS>
 void launch_one(const DmaPlan& p, const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, hipStream_t stream) {
-    static std::atomic<uint64_t> attr_set{0};  // one bit a device: the attribute belongs to the device's copy of the code
-    int dev = 0;
-    (void)hipGetDevice(&dev);
-    const uint64_t bit = 1ull << (dev & 63);
-    if (!(attr_set.load(std::memory_order_relaxed) & bit)) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_dma<XR, D, SLABS>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        attr_set.fetch_or(bit, std::memory_order_relaxed);
-    }
+    static LdsCapOnce lds_cap;
+    lds_cap.raise(reinterpret_cast<const void*>(gemv_q4_dma<XR, D, SLABS>), 160 * 1024);
     // at least half a CU's LDS, so that the workgroups spread one to a CU
     const size_t lds = p.lds < 96 * 1024 ? 96 * 1024 : p.lds;
     hipLaunchKernelGGL((gemv_q4_dma<XR, D, SLABS>), dim3(p.grid), dim3(kWaves * 64), lds, stream, w, n, k, x, y);

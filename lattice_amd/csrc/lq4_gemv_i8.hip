@@ -39,7 +39,6 @@
 // magnitude is below 2^-100 counts as zero; an infinite or NaN activation makes the outputs of its row NaN.
 #include "lq4_internal.hpp"
 
-#include <atomic>
 #include <type_traits>
 
 namespace lq4 {
@@ -449,15 +448,8 @@ template <int CW, int TW, bool WIDE, bool MULTI>
 void launch_i8(const I8Plan& p, const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint32_t x_stride,
                uint32_t batch, float* y, uint32_t y_stride, const LoraEpilogue& lora, const MultiViews& mv,
                hipStream_t stream) {
-    static std::atomic<uint64_t> attr_set{0};  // one bit a device: the attribute belongs to the device's copy of the code
-    int dev = 0;
-    (void)hipGetDevice(&dev);
-    const uint64_t bit = 1ull << (dev & 63);
-    if (!(attr_set.load(std::memory_order_relaxed) & bit)) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_i8<CW, TW, WIDE, MULTI>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        attr_set.fetch_or(bit, std::memory_order_relaxed);
-    }
+    static LdsCapOnce lds_cap;
+    lds_cap.raise(reinterpret_cast<const void*>(gemv_q4_i8<CW, TW, WIDE, MULTI>), 160 * 1024);
     hipLaunchKernelGGL((gemv_q4_i8<CW, TW, WIDE, MULTI>), dim3(p.grid), dim3(64 * CW * TW), p.lds, stream, w, n, k, x,
                        x_stride, batch, y, y_stride, lora, mv);
 }

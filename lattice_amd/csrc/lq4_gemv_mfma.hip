@@ -516,12 +516,8 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_mfma(GemvArgs p) {
 
 template <int NSETS, bool HILO, int T, int KS, bool LONG, int WAVES>
 void launch_long(const GemvArgs& a, size_t lds, uint32_t wgs, hipStream_t stream) {
-    static bool attr_set = false;  // raise the dynamic-LDS cap once per instantiation
-    if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_mfma<NSETS, HILO, T, KS, LONG, WAVES>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        attr_set = true;
-    }
+    static LdsCapOnce lds_cap;
+    lds_cap.raise(reinterpret_cast<const void*>(gemv_q4_mfma<NSETS, HILO, T, KS, LONG, WAVES>), 160 * 1024);
     hipLaunchKernelGGL((gemv_q4_mfma<NSETS, HILO, T, KS, LONG, WAVES>), dim3(wgs), dim3(64 * WAVES), lds, stream, a);
 }
 

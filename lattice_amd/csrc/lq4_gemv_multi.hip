@@ -4,8 +4,6 @@
 // an adapter come from one launch as well.
 #include "lq4_gemv_b1_kernel.hpp"
 
-#include <atomic>
-
 namespace lq4 {
 
 namespace {
@@ -49,15 +47,8 @@ __global__ __launch_bounds__(256) void lora_a_views_kernel(LoraAViews av, uint32
 template <int RW, int SG, int SEG, int MODE>
 void launch_multi_cfg(const MultiViews& mv, uint32_t n, uint32_t k, const float* x, const LoraEpilogue& lora, size_t lds,
                       uint32_t waves, hipStream_t stream) {
-    static std::atomic<uint64_t> attr_set{0};  // one bit a device: the attribute belongs to the device's copy of the code
-    int dev = 0;
-    (void)hipGetDevice(&dev);
-    const uint64_t bit = 1ull << (dev & 63);
-    if (!(attr_set.load(std::memory_order_relaxed) & bit)) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, MODE, 4>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        attr_set.fetch_or(bit, std::memory_order_relaxed);
-    }
+    static LdsCapOnce lds_cap;
+    lds_cap.raise(reinterpret_cast<const void*>(gemv_q4_b1<RW, SG, SEG, MODE, 4>), 160 * 1024);
     // (producer workgroups, if any, come first)
     hipLaunchKernelGGL((gemv_q4_b1<RW, SG, SEG, MODE, 4>), dim3((waves + 3) / 4 + lora.rank), dim3(256), lds, stream,
                        static_cast<const uint8_t*>(nullptr), n, k, x, static_cast<float*>(nullptr), lora, mv);

@@ -6,7 +6,24 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace lq4 {
+
+// A kernel's dynamic-LDS cap (hipFuncAttributeMaxDynamicSharedMemorySize) belongs to one device's copy of the code,
+// so a launcher raises it once on every device it launches on: one bit a device, one object (static, in the
+// launcher) per kernel instantiation.  Two threads that race both set the attribute, which is harmless.
+struct LdsCapOnce {
+    std::atomic<uint64_t> done{0};
+    void raise(const void* kernel, int bytes) {
+        int dev = 0;
+        (void)hipGetDevice(&dev);
+        const uint64_t bit = 1ull << (dev & 63);
+        if (done.load(std::memory_order_relaxed) & bit) return;
+        (void)hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        done.fetch_or(bit, std::memory_order_relaxed);
+    }
+};
 
 constexpr int kBlockBytes = 20;    // one Q4 block: u16 scale, u16 bias, 16 packed bytes
 constexpr int kBlockWeights = 32;  // weights per block

@@ -286,12 +286,8 @@ void launch_one(const MoeB1Args& a, uint32_t tokens, hipStream_t stream) {
     const dim3 grid((waves + 3) / 4, tokens), block(256);
 #define LQ4_MOE_B1(RW_, SL_)                                                                                   \
     do {                                                                                                       \
-        static bool attr_set = false;                                                                          \
-        if (!attr_set) {                                                                                       \
-            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(moe_b1_kernel<DOWN, RW_, SL_, ROUTE>),     \
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);                  \
-            attr_set = true;                                                                                   \
-        }                                                                                                      \
+        static LdsCapOnce lds_cap;                                                                             \
+        lds_cap.raise(reinterpret_cast<const void*>(moe_b1_kernel<DOWN, RW_, SL_, ROUTE>), 64 * 1024);         \
         hipLaunchKernelGGL((moe_b1_kernel<DOWN, RW_, SL_, ROUTE>), grid, block, lds, stream, a);               \
     } while (0)
     if (slabs == 1) LQ4_MOE_B1(4, 1);

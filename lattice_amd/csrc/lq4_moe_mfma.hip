@@ -363,12 +363,8 @@ void launch_ks(const MoeGemvArgs& a, uint32_t num_experts, uint32_t max_pairs_pe
     const uint32_t rows_per_wg = (4 / KS) * a.tp_per_wave * rows_per_tp;
     const uint32_t nb = a.k / kBlockWeights;
     const size_t lds = static_cast<size_t>(nb) * kPitch16 * 16 + 64 + 4 * a.tp_per_wave * 2 * kCols * 4 * sizeof(float);
-    static bool attr_set = false;
-    if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(moe_expert_mfma<GATE_UP, KS>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 159 * 1024);  // the rest is static
-        attr_set = true;
-    }
+    static LdsCapOnce lds_cap;
+    lds_cap.raise(reinterpret_cast<const void*>(moe_expert_mfma<GATE_UP, KS>), 159 * 1024);  // the rest is static
     const dim3 grid((a.out_rows + rows_per_wg - 1) / rows_per_wg, num_experts, (max_pairs_per_expert + kTok - 1) / kTok);
     hipLaunchKernelGGL((moe_expert_mfma<GATE_UP, KS>), grid, dim3(kThreads), lds, stream, a);
 }

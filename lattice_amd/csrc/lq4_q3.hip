@@ -249,12 +249,8 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q3_b1(const uint8_t* __restr
 template <int RW, int HX>
 void launch_hx(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, size_t lds, uint32_t waves,
                hipStream_t stream) {
-    static bool attr_set = false;
-    if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_q3_b1<RW, HX>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        attr_set = true;
-    }
+    static LdsCapOnce lds_cap;
+    lds_cap.raise(reinterpret_cast<const void*>(gemv_q3_b1<RW, HX>), 160 * 1024);
     hipLaunchKernelGGL((gemv_q3_b1<RW, HX>), dim3((waves + kWaves - 1) / kWaves), dim3(kWaves * 64), lds, stream, w, n, k,
                        x, y);
 }

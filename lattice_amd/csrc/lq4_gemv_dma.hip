@@ -23,7 +23,8 @@
 // the old contents, and it may hand the original register to another value that the arriving data then destroys;
 // both happened here, the second as a memory fault through a clobbered address offset).
 //
-// Work split.  A workgroup (one per CU) owns a run of consecutive rows, i.e. a run of slots that is also one run of
+// Work split, rows of more than one slab (gemv_q4_dma).  A workgroup (one per CU) owns a run of consecutive rows,
+// i.e. a run of slots that is also one run of
 // memory, and its sixteen waves cut that run into sixteen equal pieces to within one slot, wherever the row
 // boundaries fall: 5120 rows of nine slots are twenty rows a CU, which dealt out as whole rows would leave four
 // waves with eighteen slots and twelve with nine.  A wave's slots are again one run of memory, so the address of
@@ -44,6 +45,17 @@
 // One workgroup of sixteen waves per CU: the activations are staged once per CU, by as many waves as the vector
 // has 512-element pieces (the others skip the staging code altogether, which on short rows is most of what a
 // wave of the lane-owns-block kernel executes).
+//
+// Rows of at most one slab (gemv_q4_dma_rows: K <= 2048, the lm_head) are slots by themselves, so there the waves
+// of a workgroup take rows as they come free instead of owning equal pieces: time stamps of the equal-pieces form
+// on 248320 x 2048 showed a workgroup's first wave done after 38 us and its last after 48.6, the last fifth of
+// the rows streaming from ever fewer waves.  Taking rows from a counter in LDS brings the waves' ends within one
+// slot of each other (45.4 / 46.8 us) and the launch from 52.6 to 51.0 us.  The same was tried for longer rows (a
+// slot = one slab of one row, the slots' sums added per row afterwards) and is not kept: the slab a wave meets is
+// then known only at run time, so the blocks of x come from LDS for every slot and every slot ends in its own
+// cross-lane sum, which cost more than the even ends returned (151936 x 5120 79.5 -> 88.2 us, 32768 x 4096
+// 16.6 -> 17.2, 5120 x 17408 13.4 -> 12.9).  What remains uneven is between workgroups (ends 41..52 us in one
+// launch, 44..49 in the next, whole XCDs ahead or behind).
 #include "lq4_b1_dev.hpp"
 
 #include <type_traits>
@@ -94,38 +106,14 @@ __device__ __forceinline__ void dma4_masked(uint32_t lds, const LQ4_GLOBAL void*
                  : "memory");
 }
 
-// XR: 8-activation units a thread stages (K <= 8 * 1024 * XR).  D: slots in a wave's ring.
-// SLABS: 1..3 = rows of that many slabs (the last may be short), the lane's blocks of x stay in registers (D is a
-// multiple of SLABS); 0 = any row length, x from LDS.
 constexpr int kWaves = 16;
-template <int XR, int D, int SLABS>
-__global__ __launch_bounds__(kWaves * 64) void gemv_q4_dma(const uint8_t* __restrict__ w_, uint32_t n, uint32_t k,
-                                                            const float* __restrict__ x_, float* __restrict__ y) {
-    static_assert(D >= 3, "one slot in registers, one landed, at least one on its way");
-    static_assert(SLABS == 0 || D % SLABS == 0, "the slab at an unrolled position must not depend on the round");
-    constexpr bool ONE_SLAB = SLABS == 1;
-    extern __shared__ __attribute__((aligned(16))) uint32_t lds_raw[];
-    lds_u32* const xs = (lds_u32*)lds_raw;
-    constexpr int T = kWaves * 64;
-    const int tid = threadIdx.x, lane = tid & 63;
-    const uint32_t nb = k / kBlockWeights;
-    const uint32_t row_bytes = nb * kBlockBytes;
-    const uint32_t slabs = SLABS ? SLABS : (nb + 63) / 64;
-    const uint32_t last_blocks = nb - (slabs - 1) * 64;  // blocks of a row's last slab
-    const uint32_t last_bytes = last_blocks * kBlockBytes;
-    const uint32_t wave = uniform(tid >> 6);
-    const LQ4_GLOBAL uint8_t* const w = as_global(w_);
-    const LQ4_GLOBAL float* const x = as_global(x_);
-    // LDS: the staged activations | one partial sum a wave | the waves' rings
-    const uint32_t xs_dwords = nb * kXPitch;
-    LQ4_LDS float* const part = reinterpret_cast<LQ4_LDS float*>(xs + xs_dwords);
-    lds_u32* const ring_ptr = xs + xs_dwords + kWaves + wave * D * (kSlotBytes / 4);
-    const uint32_t ring_addr = uniform(static_cast<uint32_t>(reinterpret_cast<size_t>(ring_ptr)));
 
-    // ---- the activations first: requested before any weight so they can be waited for alone ----
-    // Each wave moves the 512-element pieces it will stage (2 KB of raw floats a piece) into the staging area,
-    // at the bytes they have in x.  A piece that reaches past the end of x is cut at 16 bytes (K is a multiple of 32).
-    const uint32_t n_units = nb * 4;
+// The activations' way into LDS, first half: each wave moves the 512-element pieces it will stage (2 KB of raw floats a
+// piece) into the staging area, at the bytes they have in x.  A piece that reaches past the end of x is cut at 16
+// bytes (K is a multiple of 32).  Requested before any weight, so that they can be waited for alone.
+template <int XR>
+__device__ __forceinline__ void request_x(lds_u32* xs, const LQ4_GLOBAL float* x, uint32_t k, uint32_t wave, int lane) {
+    constexpr int T = kWaves * 64;
     const uint32_t xs_addr = uniform(static_cast<uint32_t>(reinterpret_cast<size_t>(xs)));
     const uint32_t x_bytes = k * 4;
 #pragma unroll
@@ -144,6 +132,65 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_dma(const uint8_t* __rest
             }
         }
     }
+}
+
+// Second half, once the wave's own pieces have landed (the caller has waited for them): the raw floats out of the
+// staging area, a barrier, the staged form (lq4_b1_dev.hpp) over them, a barrier.
+template <int XR>
+__device__ __forceinline__ void stage_x(lds_u32* xs, uint32_t k, uint32_t wave, int tid) {
+    constexpr int T = kWaves * 64;
+    const uint32_t n_units = k / 8, x_bytes = k * 4;
+    float4 xa[XR], xc[XR];
+#pragma unroll
+    for (int i = 0; i < XR; ++i) {
+        xa[i] = xc[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if ((i * T + wave * 64) * 32u < x_bytes) {  // uniform: this wave's own piece
+            const uint32_t u = tid + i * T < n_units ? tid + i * T : 0;
+            typedef float f32x4 __attribute__((ext_vector_type(4)));
+            const LQ4_LDS f32x4* const raw = reinterpret_cast<const LQ4_LDS f32x4*>(xs + u * 8);
+            const f32x4 lo = raw[0], hi = raw[1];
+            xa[i] = make_float4(lo.x, lo.y, lo.z, lo.w);
+            xc[i] = make_float4(hi.x, hi.y, hi.z, hi.w);
+        }
+    }
+    barrier_lds();  // every piece has been read: the staged form may overwrite the raw one
+#pragma unroll
+    for (int i = 0; i < XR; ++i) {
+        if ((i * T + wave * 64) * 32u < x_bytes) {  // uniform
+            const bool act = tid + i * T < n_units;
+            stage_x8(xs, act ? tid + i * T : 0, xa[i], xc[i], act);
+        }
+    }
+    barrier_lds();
+}
+
+// XR: 8-activation units a thread stages (K <= 8 * 1024 * XR).  D: slots in a wave's ring.
+// SLABS: 2 or 3 = rows of that many slabs (the last may be short), the lane's blocks of x stay in registers (D is a
+// multiple of SLABS); 0 = any longer row, x from LDS.  Rows of one slab have a kernel of their own below.
+template <int XR, int D, int SLABS>
+__global__ __launch_bounds__(kWaves * 64) void gemv_q4_dma(const uint8_t* __restrict__ w_, uint32_t n, uint32_t k,
+                                                            const float* __restrict__ x_, float* __restrict__ y) {
+    static_assert(D >= 3, "one slot in registers, one landed, at least one on its way");
+    static_assert(SLABS != 1 && (SLABS == 0 || D % SLABS == 0), "the slab at an unrolled position must not depend on the round");
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds_raw[];
+    lds_u32* const xs = (lds_u32*)lds_raw;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const uint32_t nb = k / kBlockWeights;
+    const uint32_t row_bytes = nb * kBlockBytes;
+    const uint32_t slabs = SLABS ? SLABS : (nb + 63) / 64;
+    const uint32_t last_blocks = nb - (slabs - 1) * 64;  // blocks of a row's last slab
+    const uint32_t last_bytes = last_blocks * kBlockBytes;
+    const uint32_t wave = uniform(tid >> 6);
+    const LQ4_GLOBAL uint8_t* const w = as_global(w_);
+    const LQ4_GLOBAL float* const x = as_global(x_);
+    // LDS: the staged activations | one partial sum a wave | the waves' rings
+    const uint32_t xs_dwords = nb * kXPitch;
+    LQ4_LDS float* const part = reinterpret_cast<LQ4_LDS float*>(xs + xs_dwords);
+    lds_u32* const ring_ptr = xs + xs_dwords + kWaves + wave * D * (kSlotBytes / 4);
+    const uint32_t ring_addr = uniform(static_cast<uint32_t>(reinterpret_cast<size_t>(ring_ptr)));
+
+    // ---- the activations first: requested before any weight so they can be waited for alone ----
+    request_x<XR>(xs, x, k, wave, lane);
 
     // ---- this wave's slots ----
     // the workgroup's rows: one run, the first n % workgroups of them take one row more
@@ -170,7 +217,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_dma(const uint8_t* __rest
     const uint32_t off16 = lane * 16u, off4 = lane * 4u;
     auto request_next = [&](int pos) {  // `pos`: ring position
         const uint32_t at = ring_addr + pos * kSlotBytes;
-        const bool last = ONE_SLAB || rq_slab + 1 == slabs;
+        const bool last = rq_slab + 1 == slabs;
         if (short_last && last) {
             dma16_masked(at, rq_ptr, off16, mask16);
             dma4_masked(at + n16 * 16, rq_ptr + (rest ? n16 * 16 : 0u), off4, mask4);
@@ -180,7 +227,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_dma(const uint8_t* __rest
             dma4(at + 1024, rq_ptr + 1024, off4);
             rq_ptr += kSlotBytes;
         }
-        if (!ONE_SLAB) rq_slab = last ? 0 : rq_slab + 1;
+        rq_slab = last ? 0 : rq_slab + 1;
     };
     // Two slots a wave now, the rest of the ring once the activations are staged: a CU accepts requests only as fast
     // as earlier ones are answered once a few dozen KB are on their way, and a wave stuck issuing its whole ring
@@ -198,28 +245,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_dma(const uint8_t* __rest
     // ---- stage x: the activation loads are older than every weight request ----
     if (total >= static_cast<uint32_t>(E)) wait_vm<2 * E>();
     else wait_vm<0>();
-    float4 xa[XR], xc[XR];
-#pragma unroll
-    for (int i = 0; i < XR; ++i) {
-        xa[i] = xc[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        if ((i * T + wave * 64) * 32u < x_bytes) {  // uniform: this wave's own piece, which it has just waited for
-            const uint32_t u = tid + i * T < n_units ? tid + i * T : 0;
-            typedef float f32x4 __attribute__((ext_vector_type(4)));
-            const LQ4_LDS f32x4* const raw = reinterpret_cast<const LQ4_LDS f32x4*>(xs + u * 8);
-            const f32x4 lo = raw[0], hi = raw[1];
-            xa[i] = make_float4(lo.x, lo.y, lo.z, lo.w);
-            xc[i] = make_float4(hi.x, hi.y, hi.z, hi.w);
-        }
-    }
-    barrier_lds();  // every piece has been read: the staged form may overwrite the raw one
-#pragma unroll
-    for (int i = 0; i < XR; ++i) {
-        if ((i * T + wave * 64) * 32u < x_bytes) {  // uniform
-            const bool act = tid + i * T < n_units;
-            stage_x8(xs, act ? tid + i * T : 0, xa[i], xc[i], act);
-        }
-    }
-    barrier_lds();
+    stage_x<XR>(xs, k, wave, tid);
 #pragma unroll
     for (int i = E; i < D; ++i) {
         if (to_request) {  // uniform
@@ -305,11 +331,10 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_dma(const uint8_t* __rest
         }
         if (SLABS) cs_slab = (slab0 + total) % NX;  // the slab the next slot would have had
     };
-    if (SLABS <= 1 || slab0 == 0) run(std::integral_constant<int, 0>{});
+    if (SLABS == 0 || slab0 == 0) run(std::integral_constant<int, 0>{});
     else if (slab0 == 1) run(std::integral_constant<int, 1>{});
     else run(std::integral_constant<int, SLABS == 3 ? 2 : 0>{});
     wait_vm<0>();  // nothing of this wave is on its way when it ends
-    if (ONE_SLAB) return;
     // ---- rows that straddle waves ----
     const bool open_row = total != 0 && cs_slab != 0;  // the last slot did not end its row
     float own = 0.0f;
@@ -330,6 +355,138 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_dma(const uint8_t* __rest
     }
 }
 
+// Rows of at most one slab (K <= 2048): a slot is a row, the lane's block of x stays in registers, and a slot's sum
+// is its row's result.  The waves of a workgroup do not advance at one pace (with equal shares the first is done
+// when the last has a fifth of its rows to go, and what is left then streams from fewer waves), so only a wave's
+// first D slots are fixed: slot 16 i + wave goes into position i, the sixteen waves' requests forming one run of
+// memory, and every later request takes the next row nobody has asked for yet, from a counter in LDS.
+template <int D>
+__global__ __launch_bounds__(kWaves * 64) void gemv_q4_dma_rows(const uint8_t* __restrict__ w_, uint32_t n, uint32_t k,
+                                                                 const float* __restrict__ x_, float* __restrict__ y) {
+    static_assert(D >= 3, "one slot in registers, one landed, at least one on its way");
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds_raw[];
+    lds_u32* const xs = (lds_u32*)lds_raw;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const uint32_t nb = k / kBlockWeights;  // at most 64
+    const uint32_t row_bytes = nb * kBlockBytes;
+    const uint32_t wave = uniform(tid >> 6);
+    const LQ4_GLOBAL uint8_t* const w = as_global(w_);
+    // LDS: the staged activations | the row counter | the waves' rings
+    const uint32_t xs_dwords = nb * kXPitch;
+    lds_u32* const counter = xs + xs_dwords;
+    lds_u32* const ring_ptr = counter + kWaves + wave * D * (kSlotBytes / 4);
+    const uint32_t ring_addr = uniform(static_cast<uint32_t>(reinterpret_cast<size_t>(ring_ptr)));
+
+    request_x<1>(xs, as_global(x_), k, wave, lane);
+
+    // the workgroup's rows: one run, the first n % workgroups of them take one row more
+    const uint32_t share = n / gridDim.x, extra = n - share * gridDim.x;
+    const uint32_t wg_rows = share + (blockIdx.x < extra ? 1u : 0u);
+    const uint32_t wg_first = blockIdx.x * share + (blockIdx.x < extra ? blockIdx.x : extra);
+    // a short row: 20 * blocks bytes as whole 16-byte pieces, then the dwords behind them (fewer than four); lane 0
+    // always takes part in the second load so that it is a load instruction on every path (the waits count them)
+    const uint32_t n16 = row_bytes / 16 < 64 ? row_bytes / 16 : 64;
+    const uint32_t rest = (row_bytes - n16 * 16) / 4;
+    const uint64_t mask16 = __builtin_amdgcn_ballot_w64(static_cast<uint32_t>(lane) < n16);
+    const uint64_t mask4 = __builtin_amdgcn_ballot_w64(static_cast<uint32_t>(lane) < (rest ? rest : 1u));
+    const bool short_row = nb != 64;
+    const LQ4_GLOBAL uint8_t* const w_wg = w + static_cast<uint64_t>(wg_first) * row_bytes;
+    const uint32_t off16 = lane * 16u, off4 = lane * 4u;
+    uint32_t slot_row[D];  // the row in each ring position (scalar registers: the positions are constants)
+    auto request = [&](int pos, uint32_t row) {  // row `row` of the workgroup into ring position `pos`
+        const LQ4_GLOBAL uint8_t* const src = w_wg + static_cast<uint64_t>(row) * row_bytes;
+        const uint32_t at = ring_addr + pos * kSlotBytes;
+        if (short_row) {
+            dma16_masked(at, src, off16, mask16);
+            dma4_masked(at + n16 * 16, src + (rest ? n16 * 16 : 0u), off4, mask4);
+        } else {
+            dma16(at, src, off16);
+            dma4(at + 1024, src + 1024, off4);
+        }
+        slot_row[pos] = row;
+    };
+    // two slots a wave now, the rest of the ring once the activations are staged (as in the kernel above)
+    constexpr int E = 2;
+    uint32_t have = 0;  // occupied ring positions: always consecutive ones
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+        const uint32_t row = i * kWaves + wave;
+        if (row < wg_rows) {  // uniform
+            request(i, row);
+            ++have;
+        }
+    }
+    if (tid == 0) *counter = D * kWaves;  // the first row that is nobody's yet
+
+    // ---- stage x: the activation loads are older than every weight request ----
+    if (have == static_cast<uint32_t>(E)) wait_vm<2 * E>();
+    else wait_vm<0>();
+    stage_x<1>(xs, k, wave, tid);  // (its barriers publish the counter as well)
+#pragma unroll
+    for (int i = E; i < D; ++i) {
+        const uint32_t row = i * kWaves + wave;
+        if (row < wg_rows) {  // uniform
+            request(i, row);
+            ++have;
+        }
+    }
+    // a wave that found fewer than D rows finds none behind them either; from the first request the counter turns
+    // down on, a wave asks no more: its occupied positions stay consecutive and the ring drains
+    bool more = have == static_cast<uint32_t>(D);
+
+    // ---- the arithmetic: round after round over the ring ----
+    XBlock xb;
+    load_xblock(xs, static_cast<uint32_t>(lane) < nb ? lane : nb - 1, xb);
+    const bool live = static_cast<uint32_t>(lane) < nb;
+    const lds_u32* const my_block = ring_ptr + 5 * lane;  // the lane's block in position 0: byte 20 l
+    auto read_block = [&](int pos, Q4BlockRaw& wb) {
+        const lds_u32* const slot = my_block + pos * (kSlotBytes / 4);
+        wb.sb = slot[0];
+        wb.q[0] = slot[1]; wb.q[1] = slot[2]; wb.q[2] = slot[3]; wb.q[3] = slot[4];
+    };
+    Q4BlockRaw cur, nxt;
+    if (have) {
+        if (more) wait_vm<2 * (D - 1)>();
+        else wait_vm<0>();
+        read_block(0, cur);
+    }
+    while (have) {
+#pragma unroll
+        for (int i = 0; i < D; ++i) {
+            if (have == 0) break;  // uniform
+            // the row that will take this position: asked for now, needed after the arithmetic.  (A plain LDS atomic
+            // of one lane; the wave-wide ds_append was tried for it and did not count as its description says.)
+            uint32_t claim = 0;
+            if (more && lane == 0) claim = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            // the slot behind this one out of LDS now: its read hides behind this slot's arithmetic
+            if (have > 1) {
+                if (more) wait_vm<2 * (D - 2)>();  // the ring is full behind this slot
+                else wait_vm<0>();
+                read_block((i + 1) % D, nxt);
+            }
+            // a lane past the end of the row has read what the slot held before: scale and bias of zero,
+            // whatever bits they were (a stale bias may be an infinity, and zero times that is not zero)
+            if (short_row) cur.sb = live ? cur.sb : 0u;
+            const float v = segment_sum<64>(block_fma(cur, xb, live, 0.0f));
+            if (lane == 63) y[wg_first + slot_row[i]] = v;
+            // the slot's words went into registers a slot ago: its place in the ring can be filled again
+            if (more) {
+                const uint32_t row = uniform(claim);
+                if (row < wg_rows) {
+                    request(i, row);
+                } else {
+                    more = false;
+                    --have;
+                }
+            } else {
+                --have;
+            }
+            cur = nxt;
+        }
+    }
+    wait_vm<0>();  // nothing of this wave is on its way when it ends
+}
+
 struct DmaPlan {
     uint32_t xr, depth, slabs, grid;
     size_t lds;
@@ -338,6 +495,7 @@ struct DmaPlan {
 // Which instantiation serves a row length: ring depth by what LDS leaves beside the staged activations.
 bool plan_dma(uint32_t n, uint32_t k, uint32_t cu_count, DmaPlan* out) {
     const uint32_t nb = k / kBlockWeights;
+    // (sixteen dwords between the activations and the rings: the waves' partial sums, or the row counter)
     const size_t fixed = static_cast<size_t>(nb) * kXPitch * 4 + kWaves * 4;
     DmaPlan p;
     p.slabs = nb <= 192 ? (nb + 63) / 64 : 0;
@@ -350,6 +508,14 @@ bool plan_dma(uint32_t n, uint32_t k, uint32_t cu_count, DmaPlan* out) {
     p.grid = n < cu_count ? n : cu_count;
     *out = p;
     return true;
+}
+
+template <int D>
+void launch_rows(const DmaPlan& p, const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, hipStream_t stream) {
+    static LdsCapOnce lds_cap;
+    lds_cap.raise(reinterpret_cast<const void*>(gemv_q4_dma_rows<D>), 160 * 1024);
+    const size_t lds = p.lds < 96 * 1024 ? 96 * 1024 : p.lds;  // one workgroup to a CU
+    hipLaunchKernelGGL((gemv_q4_dma_rows<D>), dim3(p.grid), dim3(kWaves * 64), lds, stream, w, n, k, x, y);
 }
 
 template <int XR, int D, int SLABS>
@@ -368,11 +534,11 @@ bool gemv_dma_serves(uint32_t n, uint32_t k, uint32_t cu_count) {
     return n != 0 && plan_dma(n, k, cu_count, &p);
 }
 
-// Measured against the lane-owns-block kernel on 256 CUs (us, that kernel -> this one): 32768 x 2048 (42 MB) 10.7 ->
-// 10.8; 65536 x 2048 (84 MB) 19.2 -> 17.4; 248320 x 2048 62.1 -> 54.3; 32768 x 4096 18.1 -> 16.7; 17408 x 5120 (56 MB)
-// 13.3 -> 13.5; 151936 x 5120 94.4 -> 82.7; 16384 x 8192 19.1 -> 18.0; 8192 x 12288 (63 MB) 15.5 -> 13.2; 4096 x 14336
-// (37 MB) 11.2 -> 9.6; 5120 x 17408 16.8 -> 13.5; 2048 x 17408 (22 MB) 8.9 -> 9.1.  Behind for every row shorter than
-// one slab (131072 x 1024 18.9 -> 21.9: the other kernel puts two rows side by side in a wave) and for the decode
+// Measured against the lane-owns-block kernel on 256 CUs (us, that kernel -> this one): 32768 x 2048 (42 MB) 10.2 ->
+// 10.35; 65536 x 2048 (84 MB) 17.4 -> 16.3; 248320 x 2048 62.1 -> 51.4; 32768 x 4096 16.7 -> 16.7; 17408 x 5120 (56 MB)
+// 12.6..13.3 -> 13.6; 151936 x 5120 87.8 -> 79.5; 16384 x 8192 17.8 -> 18.0; 8192 x 12288 (63 MB) 14.9 -> 13.0; 4096 x
+// 14336 (37 MB) 10.8 -> 9.4; 5120 x 17408 16.8 -> 13.5; 2048 x 17408 (22 MB) 8.6 -> 9.0.  Behind for every row shorter
+// than one slab (131072 x 1024 18.9 -> 21.7: the other kernel puts two rows side by side in a wave) and for the decode
 // layer's matrices (2..16 MB, 1.0 us behind: its start costs two workgroup barriers of sixteen waves).
 bool gemv_dma_pays(uint32_t n, uint32_t k, uint32_t cu_count) {
     if (!gemv_dma_serves(n, k, cu_count) || k < 2048) return false;
@@ -383,7 +549,7 @@ bool gemv_dma_pays(uint32_t n, uint32_t k, uint32_t cu_count) {
 void launch_gemv_dma(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, uint32_t cu_count, hipStream_t stream) {
     DmaPlan p;
     if (!plan_dma(n, k, cu_count, &p)) return;  // the caller asked gemv_dma_serves first
-    if (p.slabs == 1) launch_one<1, 6, 1>(p, w, n, k, x, y, stream);
+    if (p.slabs == 1) launch_rows<6>(p, w, n, k, x, y, stream);
     else if (p.slabs == 2) launch_one<1, 6, 2>(p, w, n, k, x, y, stream);
     else if (p.slabs == 3) launch_one<1, 6, 3>(p, w, n, k, x, y, stream);
     else if (p.xr == 1 && p.depth == 6) launch_one<1, 6, 0>(p, w, n, k, x, y, stream);

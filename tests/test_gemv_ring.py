@@ -7,8 +7,9 @@ bit-identical to the lane-owns-block kernel, which adds a row's blocks in the sa
 
 Shapes cover what the kernel branches on: rows shorter than a slab, a short last slab, two and three slabs with the
 activations in registers, more slabs with the activations read from LDS, K above 8192 (three activation pieces a
-wave) up to the kernel's limit 24576, fewer rows than CUs, rows that straddle waves and workgroups, and a vocabulary-
-sized matrix.
+wave) up to the kernel's limit 24576, fewer rows than CUs, rows that straddle waves and workgroups, a vocabulary-
+sized matrix, and one-slab rows with more than 96 rows a workgroup (full and short rows), where the waves take
+rows from the workgroup's counter once their first six are under way.
 """
 import numpy as np
 import pytest
@@ -54,7 +55,7 @@ def run(be, w, x, n, k):
 
 RING_SHAPES = [(1, 32), (64, 64), (5, 96), (33, 32), (300, 2048), (2048, 2048), (1000, 1024), (12288, 2048),
                (2048, 6144), (700, 8160), (300, 17408), (4099, 5120), (70000, 256), (9, 24576), (255, 4096),
-               (257, 4128), (513, 10240)]
+               (257, 4128), (513, 10240), (30001, 2048), (25000, 1056)]
 
 
 @pytest.mark.parametrize("n,k", RING_SHAPES)

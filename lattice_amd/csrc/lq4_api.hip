@@ -62,6 +62,7 @@ struct lq4_lora {
     void* b;  // [d_out, rank]
     int is_f16;
     uint32_t rank, d_in, d_out;
+    void* a_packed;  // A as the few-token GEMM's operand (ranks it accepts; else null): that kernel's in-launch A . X
 };
 
 namespace {
@@ -356,14 +357,29 @@ int lq4_lora_upload(lq4_ctx* ctx, const void* a_host, const void* b_host, int dt
     if (rank > kMaxLoraRank) return fail(LQ4_E_UNSUPPORTED, "LoRA rank %u above the supported maximum %d", rank, kMaxLoraRank);
     const size_t es = dtype == LQ4_F16 ? 2 : 4;
     DeviceGuard g(ctx->device);
-    lq4_lora* l = new (std::nothrow) lq4_lora{ctx, nullptr, nullptr, dtype == LQ4_F16, rank, d_in, d_out};
+    lq4_lora* l = new (std::nothrow) lq4_lora{ctx, nullptr, nullptr, dtype == LQ4_F16, rank, d_in, d_out, nullptr};
     if (!l) return fail(LQ4_E_NOMEM, "out of host memory");
     const size_t a_bytes = es * rank * d_in, b_bytes = es * d_out * rank;
     hipError_t e = hipMalloc(&l->a, a_bytes);
     if (e == hipSuccess) e = hipMalloc(&l->b, b_bytes);
     if (e == hipSuccess) e = hipMemcpy(l->a, a_host, a_bytes, hipMemcpyHostToDevice);
     if (e == hipSuccess) e = hipMemcpy(l->b, b_host, b_bytes, hipMemcpyHostToDevice);
+    if (e == hipSuccess && gemm_skinny_packs_lora_a(rank)) {  // A once more, as the few-token GEMM's own operand
+        const size_t bytes = gemm_skinny_packed_lora_a_bytes(d_in);
+        void* host = malloc(bytes);
+        if (!host) {
+            (void)hipFree(l->a);
+            (void)hipFree(l->b);
+            delete l;
+            return fail(LQ4_E_NOMEM, "out of host memory");
+        }
+        gemm_skinny_pack_lora_a(a_host, dtype == LQ4_F16, rank, d_in, host);
+        e = hipMalloc(&l->a_packed, bytes);
+        if (e == hipSuccess) e = hipMemcpy(l->a_packed, host, bytes, hipMemcpyHostToDevice);
+        free(host);
+    }
     if (e != hipSuccess) {
+        if (l->a_packed) (void)hipFree(l->a_packed);
         if (l->a) (void)hipFree(l->a);
         if (l->b) (void)hipFree(l->b);
         delete l;
@@ -376,6 +392,7 @@ int lq4_lora_upload(lq4_ctx* ctx, const void* a_host, const void* b_host, int dt
 int lq4_lora_free(lq4_lora* l) {
     if (!l) return LQ4_OK;
     DeviceGuard g(l->ctx->device);
+    (void)hipFree(l->a_packed);
     (void)hipFree(l->a);
     (void)hipFree(l->b);
     delete l;
@@ -401,22 +418,30 @@ static void plain_gemv_one_token(lq4_ctx* ctx, const uint8_t* wp, uint32_t n, ui
     ctx->counters.gemv++;
 }
 
-// The routing of lq4_gemv once the LoRA factor t (if any) is in ep: which kernel serves (batch, n, k).
-static int gemv_dispatch(lq4_ctx* ctx, const uint8_t* wp, uint32_t n, uint32_t k, const float* x_dev, uint32_t batch,
-                         float* y_dev, const LoraEpilogue& ep, hipStream_t s) {
-    int rc;
-    // Above four activation rows the few-token matrix-core kernel (operands packed once, eight K
-    // slices per workgroup) overtakes the 4x4x4 GEMV kernel: always from nine rows; from five for
-    // mid-sized matrices only (measured: behind for 512 x 2048, where its two launches dominate,
-    // and for 12288 x 2048, where the GEMV kernel's grid already fills the chip).
+// Above four activation rows the few-token matrix-core kernel (operands packed once, eight K
+// slices per workgroup) overtakes the 4x4x4 GEMV kernel: always from nine rows; from five for
+// mid-sized matrices only (measured: behind for 512 x 2048, where its two launches dominate,
+// and for 12288 x 2048, where the GEMV kernel's grid already fills the chip).
+static bool gemv_takes_few_token_gemm(uint32_t n, uint32_t k, uint32_t batch) {
     const uint64_t weights = static_cast<uint64_t>(n) * k;
     // (not for up to 2048 rows while the GEMV kernel can stage the activations: its eight-wave
     // workgroups then win, 2048 x 6144 at 5..8 rows 9.5 -> 7.2..8.2 us)
     const bool narrow = n <= 2048 && gemv_mfma_lds_bytes(k, batch < 8 ? batch : 8) <= 150 * 1024;
-    if (batch >= 9 || (batch >= 5 && n < 8192 && !narrow && weights >= 6000000)) {
+    return batch >= 9 || (batch >= 5 && n < 8192 && !narrow && weights >= 6000000);
+}
+
+// The routing of lq4_gemv once the LoRA factor t (if any) is in ep, or ep.a says that the few-token GEMM computes
+// it: which kernel serves (batch, n, k).
+// `x_packed` (may be null): calls in a row on the same x, K and batch share the few-token GEMM's packed activations;
+// true once a call has packed them into the context's scratch.
+static int gemv_dispatch(lq4_ctx* ctx, const uint8_t* wp, uint32_t n, uint32_t k, const float* x_dev, uint32_t batch,
+                         float* y_dev, const LoraEpilogue& ep, hipStream_t s, bool* x_packed = nullptr) {
+    int rc;
+    if (gemv_takes_few_token_gemm(n, k, batch)) {
         rc = ensure_scratch(ctx, gemm_skinny_scratch_bytes(k, batch), s);
         if (rc) return rc;
-        launch_gemm_skinny(wp, n, k, x_dev, 0, batch, y_dev, ep, ctx->moe_scratch, s);
+        launch_gemm_skinny(wp, n, k, x_dev, 0, batch, y_dev, ep, ctx->moe_scratch, s, 0, !(x_packed && *x_packed));
+        if (x_packed) *x_packed = true;
         ctx->counters.gemm++;
     } else if (batch == 1 && !ep.rank) {
         plain_gemv_one_token(ctx, wp, n, k, x_dev, y_dev, s);
@@ -466,6 +491,8 @@ int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
         ep.slots = reinterpret_cast<unsigned long long*>(ctx->lora_sync + 64);
         ep.sync = ctx->lora_sync;
         ep.spin_limit = ctx->lora_spin_limit;
+    } else if (ep.rank && batch > 1 && gemv_takes_few_token_gemm(n, k, batch) && gemm_skinny_computes_t(ep.rank, batch)) {
+        ep.a = lora->a_packed;  // the few-token GEMM computes A.x for its token tile itself
     } else if (ep.rank) {
         launch_lora_a(lora->a, lora->is_f16, lora->rank, k, x_dev, 0, k, batch, ctx->lora_t, s);
         ctx->counters.lora_a++;
@@ -530,6 +557,22 @@ int lq4_gemv_multi(lq4_ctx* ctx, const lq4_projection* proj, uint32_t count, uin
     // one token: the stacked launch computes every A_v . x in producer workgroups of its own (lane l of a weight
     // wave holds the factor of stacked row l, hence at most 64 rows of A in all)
     const bool in_launch = stacked && with_lora && ctx->lora_in_kernel && total_rank <= 64;
+    // two to eight rows: the integer matrix-core kernel over the stacked rows, where it is the faster one
+    const bool stacked_rows = !stacked && batch >= 2 && batch <= 8 && mv.count > 1 && ctx->gemv_i8 &&
+                              (ctx->gemv_i8 == 2 || (k <= 2048 && mv.begin[mv.count] <= 4096)) &&
+                              gemv_i8_multi_serves(mv, k, batch, ctx->cu_count);
+    if (with_lora && !stacked && !stacked_rows) {
+        // projection by projection: those that go to the few-token GEMM get their A . x there
+        for (uint32_t i = 0, v = 0; i < count; ++i) {
+            if (proj[i].n == 0) continue;
+            if (ep[i].rank && gemv_takes_few_token_gemm(proj[i].n, k, batch) && gemm_skinny_computes_t(ep[i].rank, batch)) {
+                ep[i].a = proj[i].lora->a_packed;
+                av.rank[v] = 0;
+                --with_lora;
+            }
+            ++v;
+        }
+    }
     if (with_lora) {  // the A . x buffer and the hand-over words belong to the context
         int rc = enter_shared_state(ctx, s);
         if (rc) return rc;
@@ -538,10 +581,6 @@ int lq4_gemv_multi(lq4_ctx* ctx, const lq4_projection* proj, uint32_t count, uin
             ctx->counters.lora_a++;
         }
     }
-    // two to eight rows: the integer matrix-core kernel over the stacked rows, where it is the faster one
-    const bool stacked_rows = !stacked && batch >= 2 && batch <= 8 && mv.count > 1 && ctx->gemv_i8 &&
-                              (ctx->gemv_i8 == 2 || (k <= 2048 && mv.begin[mv.count] <= 4096)) &&
-                              gemv_i8_multi_serves(mv, k, batch, ctx->cu_count);
     if (stacked_rows) {
         launch_gemv_i8_multi(mv, k, x_dev, k, batch, ctx->cu_count, s);
         ctx->counters.gemv_multi++;
@@ -557,9 +596,10 @@ int lq4_gemv_multi(lq4_ctx* ctx, const lq4_projection* proj, uint32_t count, uin
         ctx->counters.gemv_multi++;
     } else {
         // several rows (or a shape the stacked launch does not take): each projection through lq4_gemv's routing
+        bool x_packed = false;  // the few-token GEMM's packed activations serve every projection that takes it
         for (uint32_t i = 0; i < count; ++i) {
             if (proj[i].n == 0) continue;
-            int rc = gemv_dispatch(ctx, wp[i], proj[i].n, k, x_dev, batch, proj[i].y_dev, ep[i], s);
+            int rc = gemv_dispatch(ctx, wp[i], proj[i].n, k, x_dev, batch, proj[i].y_dev, ep[i], s, &x_packed);
             if (rc) return rc;
         }
     }
@@ -686,7 +726,9 @@ int lq4_gemm(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
         rc = enter_shared_state(ctx, s);
         if (rc) return rc;
     }
-    if (ep.rank) {
+    if (ep.rank && gemm_takes_few_token_kernel(n, k, m, x_dtype == LQ4_F16, ctx->gemm_kernel) && gemm_skinny_computes_t(ep.rank, m)) {
+        ep.a = lora->a_packed;  // the few-token GEMM computes A.X for its token tile itself
+    } else if (ep.rank) {
         launch_lora_a(lora->a, lora->is_f16, lora->rank, k, x_dev, x_dtype == LQ4_F16, k, m, ctx->lora_t, s);
         ctx->counters.lora_a++;
     }

@@ -531,6 +531,10 @@ GemmPlan plan_gemm(uint32_t n, uint32_t k, uint32_t m, int x_is_f16, bool with_l
 
 }  // namespace
 
+bool gemm_takes_few_token_kernel(uint32_t n, uint32_t k, uint32_t m, int x_is_f16, int forced) {
+    return plan_gemm(n, k, m, x_is_f16, true, forced).skinny;
+}
+
 size_t gemm_scratch_floats(uint32_t n, uint32_t k, uint32_t m, int x_is_f16, bool with_lora, int forced) {
     const GemmPlan p = plan_gemm(n, k, m, x_is_f16, with_lora, forced);
     if (p.skinny) return (gemm_skinny_scratch_bytes(k, m) + sizeof(float) - 1) / sizeof(float);

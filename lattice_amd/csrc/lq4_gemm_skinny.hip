@@ -21,6 +21,10 @@
 //    run-time condition would make the compiler wait for loads it cannot count).
 //    Each wave adds its share of the LoRA delta (ranks w, w + 8, ...) to its partial result in
 //    f32; the eight partial results then meet in LDS in a fixed order and y is stored once.
+//    LA = true (Q4, rank <= 16): the factor t = A . X of the workgroup's token tile is computed here as well, A
+//    riding through the K loop as one more 16-row tile against the same packed operands (f16 inputs, f32
+//    accumulation, like the product itself), so that no launch for t precedes this one.  Every workgroup repeats
+//    it for its token tile: 64 KB of A from L2 beside the 256 KB of packed X it reads anyway.
 //
 // Dequantised value: half(q*d + b) with one rounding (shaders/gemm_q4_tiled.metal:57-66), f32
 // accumulation.
@@ -179,14 +183,20 @@ __global__ __launch_bounds__(256) void pack_x_kernel(const void* __restrict__ xv
 // RT: 16-row weight tiles per wave (rows per workgroup = 16 RT).  grid (ceil(N / 16 RT), token tiles).
 // FMT: 0 = Q4, 1 = Q8_0, 2 = Q3 blocks.
 // NTG: 16-token groups a workgroup computes (1, 2 or 4); a token tile with fewer groups re-reads its
-// last group and drops the results.  Fixed per instantiation, like the prefetches of the K loop below:
+// last group and drops the results.  tile_groups (<= NTG): token groups from one workgroup's tile to the next
+// (grid.y tiles: four groups a tile, or two where NTG is held at two for a larger batch).  Fixed per instantiation, like the prefetches of the K loop below:
 // a load behind a run-time condition makes the compiler wait for loads it cannot count, and the
 // pipeline collapses to one unit in flight.
-template <int RT, int FMT, int NTG>
+// LA: lora.a is the adapter's A packed by gemm_skinny_pack_lora_a and t = A . X is computed here (rank <= 16, Q4
+// only); lora.t is then not read.
+template <int RT, int FMT, int NTG, bool LA = false>
 __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __restrict__ w, uint32_t n, uint32_t k,
                                                                 const uint4* __restrict__ xp, uint32_t m,
-                                                                float* __restrict__ y, LoraEpilogue lora) {
-    extern __shared__ float4v red[];  // 4 slots of RT * 4 * 64 accumulators
+                                                                float* __restrict__ y, LoraEpilogue lora,
+                                                                uint32_t tile_groups) {
+    static_assert(!LA || FMT == 0, "the adapter's A is packed in the Q4 decoder's order");
+    static_assert(!LA || NTG <= 2, "with A in the K loop four token groups do not fit the registers");
+    extern __shared__ float4v red[];  // 4 slots of RT * NTG * 64 accumulators; LA: then 8 * NTG * 64 partial t, then t
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -195,8 +205,8 @@ __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __
 
     const uint32_t n0 = blockIdx.x * (16 * RT);
     const uint32_t groups = (m + 15) / 16;             // token groups in X (and in the packed image)
-    const uint32_t tg0 = blockIdx.y * (kTokens / 16);  // first token group of this workgroup
-    const uint32_t ntg = groups - tg0 < 4 ? groups - tg0 : 4;
+    const uint32_t tg0 = blockIdx.y * tile_groups;  // first token group of this workgroup
+    const uint32_t ntg = groups - tg0 < tile_groups ? groups - tg0 : tile_groups;
     const uint32_t nb = k / kBlockWeights;
     const uint32_t steps_total = (nb + 3) / 4;
     const uint32_t cnt = steps_total > static_cast<uint32_t>(wave) ? (steps_total - wave + kWavesK - 1) / kWavesK : 0;
@@ -211,9 +221,35 @@ __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __
         w_row[u] = w + static_cast<size_t>(row) * (nb * kBytes);
     }
 
+    // LA: A packed like the activations (lq4_pack_lora_a): the operands of step s, instruction j at [(4 s + j) * 64 + lane]
+    const uint4* const a_lane = static_cast<const uint4*>(lora.a) + lane;
+    // The LoRA factor B of this wave's first two ranks (w and w + 8) is requested now, as raw bits, and converted in
+    // the epilogue: requested there, the loads' whole latency stood between the K loop and the reduction (two token
+    // groups of K steps a wave on a 2048-long row: the launch is latency from end to end).
+    // (one row tile only: with two, the sixteen registers this holds through the K loop spill)
+    constexpr bool kEarlyB = RT == 1;
+    uint32_t b_raw[2][RT][4];
+    if (kEarlyB && lora.rank) {
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            const uint32_t jj = wave + p * kWavesK;
+            const uint32_t jc = jj < lora.rank ? jj : 0;
+#pragma unroll
+            for (int r = 0; r < RT; ++r)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    uint32_t row = n0 + 16 * r + 4 * g + v;
+                    row = row < n ? row : n - 1;
+                    const size_t idx = static_cast<size_t>(row) * lora.rank + jc;
+                    b_raw[p][r][v] = lora.b_is_f16 ? static_cast<uint32_t>(static_cast<const uint16_t*>(lora.b)[idx])
+                                                   : static_cast<const uint32_t*>(lora.b)[idx];
+                }
+        }
+    }
     struct Unit {
         WBlock wb[RT];
         uint4 x[NTG][4];  // [token group][instruction]
+        uint4 a[LA ? 4 : 1];  // LA: the lane's operand of A for instruction j
     };
     uint32_t xg[NTG];  // packed-image group of token group t (clamped to the last one)
 #pragma unroll
@@ -225,6 +261,11 @@ __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __
         blk = blk < nb ? blk : nb - 1;
 #pragma unroll
         for (int r = 0; r < RT; ++r) u.wb[r] = *reinterpret_cast<const WBlock*>(w_row[r] + blk * kBytes);
+        if constexpr (LA) {
+            const uint32_t sc = s < steps_total ? s : steps_total - 1;  // (a wave's clamped re-read of its last step)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) u.a[j] = a_lane[(static_cast<size_t>(sc) * 4 + j) * 64];
+        }
         const uint4* xs = xp + static_cast<size_t>(s) * groups * 256 + lane;
 #pragma unroll
         for (int t = 0; t < NTG; ++t)
@@ -237,6 +278,9 @@ __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __
     for (int r = 0; r < RT; ++r)
 #pragma unroll
         for (int t = 0; t < NTG; ++t) acc[r][t] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+    float4v acc_a[NTG];  // LA: element v of lane (lr, g) = t[token 16 (tg0 + t) + lr][rank 4 g + v], this wave's K slice
+#pragma unroll
+    for (int t = 0; t < NTG; ++t) acc_a[t] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
 
     auto compute = [&](const Unit& u, uint32_t i) {
         const bool live = (wave + i * kWavesK) * 4 + g < nb;  // K tail: a block past the end of the row counts as zero
@@ -258,6 +302,14 @@ __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __
                     acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
                         __builtin_bit_cast(half8, a), __builtin_bit_cast(half8, u.x[t][j]), acc[r][t], 0, 0, 0);
             }
+        }
+        if constexpr (LA) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int t = 0; t < NTG; ++t)
+                    acc_a[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                        __builtin_bit_cast(half8, u.a[j]), __builtin_bit_cast(half8, u.x[t][j]), acc_a[t], 0, 0, 0);
         }
     };
 
@@ -305,9 +357,59 @@ __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __
 
     // ---- LoRA: wave w adds the ranks w, w + 8, ... of scale * B[row, :] . t[token, :] to its own
     //      partial result in f32, so the delta is spread over all waves and joins the same reduction
+    constexpr int kSlot = RT * NTG * 64;
+    float* const t_full = reinterpret_cast<float*>(red + 4 * kSlot + kWavesK * NTG * 64);  // [token of the tile][16]
+    if constexpr (LA) {
+        // the eight K slices of t meet in LDS; every (token, rank) is summed in wave order by one thread
+        float4v* const t_part = red + 4 * kSlot;
+#pragma unroll
+        for (int t = 0; t < NTG; ++t) t_part[(wave * NTG + t) * 64 + lane] = acc_a[t];
+        __syncthreads();
+        for (uint32_t e = threadIdx.x; e < NTG * 64; e += 64 * kWavesK) {
+            float4v sum = t_part[e];
+#pragma unroll
+            for (int wv = 1; wv < kWavesK; ++wv) sum += t_part[wv * NTG * 64 + e];
+            const uint32_t tg = e >> 6, ln = e & 63;  // token 16 tg + ln % 16, ranks 4 (ln / 16) ..
+            *reinterpret_cast<float4v*>(t_full + (16 * tg + (ln & 15)) * 16 + 4 * (ln >> 4)) = sum;
+        }
+        __syncthreads();
+    }
     if (lora.rank) {
-        for (uint32_t jj = wave; jj < lora.rank; jj += kWavesK) {
-            float bv[RT][4], tv[NTG];
+        auto add_rank = [&](uint32_t jj, const float (&bv)[RT][4]) {
+            float tv[NTG];
+#pragma unroll
+            for (int t = 0; t < NTG; ++t) {
+                if constexpr (LA) {
+                    tv[t] = t_full[(16 * t + lr) * 16 + jj];
+                } else {
+                    uint32_t tok = 16 * (tg0 + t) + lr;
+                    tok = tok < m ? tok : m - 1;
+                    tv[t] = lora.t[static_cast<size_t>(tok) * lora.rank + jj];
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < RT; ++r)
+#pragma unroll
+                for (int t = 0; t < NTG; ++t)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) acc[r][t][v] = fmaf(bv[r][v], tv[t], acc[r][t][v]);
+        };
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {  // the two ranks whose B was requested at the start
+            const uint32_t jj = wave + p * kWavesK;
+            if (kEarlyB && jj < lora.rank) {
+                float bv[RT][4];
+#pragma unroll
+                for (int r = 0; r < RT; ++r)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        bv[r][v] = lora.scale * (lora.b_is_f16 ? f16_bits_to_f32(b_raw[p][r][v])
+                                                               : __builtin_bit_cast(float, b_raw[p][r][v]));
+                add_rank(jj, bv);
+            }
+        }
+        for (uint32_t jj = wave + (kEarlyB ? 2 * kWavesK : 0); jj < lora.rank; jj += kWavesK) {  // the other ranks
+            float bv[RT][4];
 #pragma unroll
             for (int r = 0; r < RT; ++r)
 #pragma unroll
@@ -316,24 +418,12 @@ __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __
                     row = row < n ? row : n - 1;
                     bv[r][v] = lora.scale * load_b(lora.b, lora.b_is_f16, static_cast<size_t>(row) * lora.rank + jj);
                 }
-#pragma unroll
-            for (int t = 0; t < NTG; ++t) {
-                uint32_t tok = 16 * (tg0 + t) + lr;
-                tok = tok < m ? tok : m - 1;
-                tv[t] = lora.t[static_cast<size_t>(tok) * lora.rank + jj];
-            }
-#pragma unroll
-            for (int r = 0; r < RT; ++r)
-#pragma unroll
-                for (int t = 0; t < NTG; ++t)
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) acc[r][t][v] = fmaf(bv[r][v], tv[t], acc[r][t][v]);
+            add_rank(jj, bv);
         }
     }
 
     // ---- the eight K slices meet in LDS in three rounds: (w, w + 4), then (w, w + 2), then (0, 1);
     //      the order is fixed, so the result does not depend on timing
-    constexpr int kSlot = RT * NTG * 64;
 #pragma unroll
     for (int half = kWavesK / 2; half >= 1; half >>= 1) {
         if (wave >= half && wave < 2 * half) {
@@ -379,9 +469,25 @@ __global__ __launch_bounds__(64 * kWavesK) void gemm_q4_skinny(const uint8_t* __
 template <int RT, int FMT, int NTG>
 void launch_ntg(const uint8_t* w, uint32_t n, uint32_t k, const uint4* xp, uint32_t m, float* y,
                 const LoraEpilogue& lora, hipStream_t stream) {
-    const dim3 grid((n + 16 * RT - 1) / (16 * RT), (m + kTokens - 1) / kTokens);
+    const uint32_t groups = (m + 15) / 16;
     const size_t lds = static_cast<size_t>(kWavesK / 2) * RT * NTG * 64 * sizeof(float4v);
-    hipLaunchKernelGGL((gemm_q4_skinny<RT, FMT, NTG>), grid, dim3(64 * kWavesK), lds, stream, w, n, k, xp, m, y, lora);
+    if constexpr (FMT == 0 && RT == 1 && NTG <= 2) {
+        if (lora.rank && lora.a) {  // t = A . X inside the launch: the waves' partial t and t itself behind the slots
+            const dim3 grid((n + 15) / 16, (groups + NTG - 1) / NTG);
+            const size_t lds_t = lds + static_cast<size_t>(kWavesK) * NTG * 64 * sizeof(float4v) + NTG * 16 * 16 * sizeof(float);
+            hipLaunchKernelGGL((gemm_q4_skinny<RT, FMT, NTG, true>), grid, dim3(64 * kWavesK), lds_t, stream, w, n, k, xp, m,
+                               y, lora, static_cast<uint32_t>(NTG));
+            return;
+        }
+    }
+    if (NTG == 2 && groups > 2) {  // tiles of two token groups (launch_rt decides when)
+        const dim3 grid2((n + 16 * RT - 1) / (16 * RT), (groups + 1) / 2);
+        hipLaunchKernelGGL((gemm_q4_skinny<RT, FMT, NTG>), grid2, dim3(64 * kWavesK), lds, stream, w, n, k, xp, m, y, lora, 2u);
+        return;
+    }
+    const dim3 grid((n + 16 * RT - 1) / (16 * RT), (m + kTokens - 1) / kTokens);
+    hipLaunchKernelGGL((gemm_q4_skinny<RT, FMT, NTG>), grid, dim3(64 * kWavesK), lds, stream, w, n, k, xp, m, y, lora,
+                       static_cast<uint32_t>(kTokens / 16));
 }
 
 // Widest row tile (of 1 or 2) whose two units in flight fit the 256 registers of a wave without spilling.
@@ -395,12 +501,62 @@ template <int RT, int FMT>
 void launch_rt(const uint8_t* w, uint32_t n, uint32_t k, const uint4* xp, uint32_t m, float* y, const LoraEpilogue& lora,
                hipStream_t stream) {
     const uint32_t groups = (m + 15) / 16;
+    if (lora.rank && lora.a) {
+        // with A as one more tile in the K loop neither a second row tile nor four token groups fit the registers:
+        // one row tile, and tiles of two token groups from 33 tokens on (more workgroups, each re-reading its rows)
+        if constexpr (RT > 1) return launch_rt<1, FMT>(w, n, k, xp, m, y, lora, stream);
+        if (groups > 2) return launch_ntg<1, FMT, 2>(w, n, k, xp, m, y, lora, stream);
+    }
+    if constexpr (RT == 1 && FMT == 0) {  // (measured for Q4 only)
+        // Token tiles of 32 instead of 64 where that fills the chip better: twice the workgroups, each 0.6-0.65 of the
+        // time (its rows are read once more, its fixed parts stay).  One workgroup runs per CU, so it pays when the
+        // workgroups of the 64-token form are at most half the CUs, or leave the second round of workgroups at most
+        // half full (measured at 64 tokens, us: 2048 x 2048 8.15 -> 6.91, 512 x 2048 7.63 -> 6.21, 2048 x 6144 14.9 ->
+        // 11.2, 2048 x 12288 30.7 -> 22.9, 5120 x 5120 26.6 -> 23.0, 6144 x 2048 12.8 -> 11.0; against 3072 x 2048 8.23 ->
+        // 8.72, 4096 x 2048 8.44 -> 8.80, 4096 x 4096 12.5 -> 13.6, which keep 64).
+        const uint32_t wgs = ((n + 15) / 16) * ((m + kTokens - 1) / kTokens);
+        if (groups > 2 && (wgs <= 128 || (wgs > 256 && wgs <= 384)))
+            return launch_ntg<1, FMT, 2>(w, n, k, xp, m, y, lora, stream);
+    }
     if (groups == 1) launch_ntg<(RT < max_rt(FMT, 1) ? RT : max_rt(FMT, 1)), FMT, 1>(w, n, k, xp, m, y, lora, stream);
     else if (groups == 2) launch_ntg<(RT < max_rt(FMT, 2) ? RT : max_rt(FMT, 2)), FMT, 2>(w, n, k, xp, m, y, lora, stream);
     else launch_ntg<(RT < max_rt(FMT, 4) ? RT : max_rt(FMT, 4)), FMT, 4>(w, n, k, xp, m, y, lora, stream);
 }
 
 }  // namespace
+
+// The few-token kernel computes t = A . X itself (LoraEpilogue::a set, no launch for t) for Q4, ranks up to 16 and
+// up to 64 tokens (q and v of the 2B model, rank 16, 64 tokens: 13.6 us with a launch for t -> 8.3 / 7.7, against
+// 8.0 / 7.6 without an adapter; at 128 tokens its tiles of 32 tokens are four to a row tile and it is behind).
+bool gemm_skinny_packs_lora_a(uint32_t rank) { return rank != 0 && rank <= 16; }
+bool gemm_skinny_computes_t(uint32_t rank, uint32_t m) { return gemm_skinny_packs_lora_a(rank) && m <= kTokens; }
+
+// A [rank <= 16, K] (f32 or f16, host memory) as the kernel's matrix-core operand, f16: for K step s (128 wide) and
+// instruction j the 64 lanes' 16-byte operands are contiguous; lane (r = lane % 16, g = lane / 16) holds row r,
+// K offsets 128 s + 32 g + 8 j .. + 7 in the order x0 x4 x1 x5 x2 x6 x3 x7 of the packed activations.  Rows past
+// the rank and K past the end are zero.  (Read row by row, sixteen rows K * 2 bytes apart, every workgroup's loads
+// of a step fell on a few memory channels at once and the launch took 4 us longer.)
+size_t gemm_skinny_packed_lora_a_bytes(uint32_t k) { return static_cast<size_t>((k + TK - 1) / TK) * 4 * 64 * 16; }
+void gemm_skinny_pack_lora_a(const void* a, int a_is_f16, uint32_t rank, uint32_t k, void* out) {
+    _Float16* dst = static_cast<_Float16*>(out);
+    const uint32_t steps = (k + TK - 1) / TK;
+    for (uint32_t s = 0; s < steps; ++s)
+        for (uint32_t j = 0; j < 4; ++j)
+            for (uint32_t lane = 0; lane < 64; ++lane) {
+                const uint32_t r = lane % 16, g = lane / 16;
+                const uint32_t k0 = s * TK + 32 * g + 8 * j;
+                _Float16* o = dst + ((static_cast<size_t>(s) * 4 + j) * 64 + lane) * 8;
+                for (uint32_t e = 0; e < 8; ++e) {
+                    const uint32_t src = (e >> 1) + 4 * (e & 1);  // x0 x4 x1 x5 x2 x6 x3 x7
+                    float v = 0.0f;
+                    if (r < rank && k0 + src < k) {
+                        const size_t idx = static_cast<size_t>(r) * k + k0 + src;
+                        v = a_is_f16 ? static_cast<float>(static_cast<const _Float16*>(a)[idx]) : static_cast<const float*>(a)[idx];
+                    }
+                    o[e] = static_cast<_Float16>(v);
+                }
+            }
+}
 
 bool gemm_skinny_wants(uint32_t n, uint32_t k, uint32_t m) {
     // Against the large-tile kernel, which wastes the empty part of its 128-token tile but shares the
@@ -425,11 +581,12 @@ namespace {
 
 template <int FMT>
 void launch_fmt(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
-                const LoraEpilogue& lora, void* packed_x, hipStream_t stream) {
+                const LoraEpilogue& lora, void* packed_x, hipStream_t stream, bool pack) {
     const uint32_t steps = (k / kBlockWeights + 3) / 4, groups = (m + 15) / 16;
     uint4* xp = static_cast<uint4*>(packed_x);
     constexpr bool kInterleave = FMT == 0;
-    if (x_is_f16)
+    if (!pack) {
+    } else if (x_is_f16)
         hipLaunchKernelGGL((pack_x_kernel<true, kInterleave>), dim3(steps, groups), dim3(256), 0, stream, x, m, k, xp);
     else
         hipLaunchKernelGGL((pack_x_kernel<false, kInterleave>), dim3(steps, groups), dim3(256), 0, stream, x, m, k, xp);
@@ -446,10 +603,10 @@ void launch_fmt(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_i
 }  // namespace
 
 void launch_gemm_skinny(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
-                        const LoraEpilogue& lora, void* packed_x, hipStream_t stream, int fmt) {
-    if (fmt == 1) launch_fmt<1>(w, n, k, x, x_is_f16, m, y, lora, packed_x, stream);
-    else if (fmt == 2) launch_fmt<2>(w, n, k, x, x_is_f16, m, y, lora, packed_x, stream);
-    else launch_fmt<0>(w, n, k, x, x_is_f16, m, y, lora, packed_x, stream);
+                        const LoraEpilogue& lora, void* packed_x, hipStream_t stream, int fmt, bool pack) {
+    if (fmt == 1) launch_fmt<1>(w, n, k, x, x_is_f16, m, y, lora, packed_x, stream, pack);
+    else if (fmt == 2) launch_fmt<2>(w, n, k, x, x_is_f16, m, y, lora, packed_x, stream, pack);
+    else launch_fmt<0>(w, n, k, x, x_is_f16, m, y, lora, packed_x, stream, pack);
 }
 
 }  // namespace lq4

@@ -47,7 +47,8 @@ struct LoraEpilogue {
     // registers, so nothing has to be agreed on through memory and nothing has to be reset between launches.  A
     // weight wave polls the slots until all carry its tag (at most `spin_limit` polls, then it computes t on its
     // own and counts itself in sync[2]).
-    const void* a;     // [rank, d_in] row-major, f32 or f16 (b_is_f16 applies to both factors)
+    const void* a;     // [rank, d_in] row-major, f32 or f16 (b_is_f16 applies to both factors); the few-token GEMM
+                       // takes its packed A here (see gemm_skinny_pack_lora_a)
     unsigned long long* slots;  // [kMaxLoraRank]
     uint32_t* sync;
     uint32_t spin_limit;
@@ -195,6 +196,8 @@ void launch_lora_b_accum(const void* b, int b_is_f16, uint32_t rank, uint32_t d_
 // `forced`: 0 = choose by shape, 1 = LDS-staged kernel, 2 = weights-in-registers kernel where supported,
 // 3 = few-token kernel, 4 = the weights-in-registers tile at two workgroups per CU (a context's setting).
 size_t gemm_scratch_floats(uint32_t n, uint32_t k, uint32_t m, int x_is_f16, bool with_lora, int forced);
+// true = launch_gemm serves the shape (with a LoRA epilogue) with the few-token kernel below
+bool gemm_takes_few_token_kernel(uint32_t n, uint32_t k, uint32_t m, int x_is_f16, int forced);
 void launch_gemm(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m,
                  float* y, const LoraEpilogue& lora, float* scratch, int forced, hipStream_t stream);
 int gemm_kernel_choice_default();  // from the environment variable LQ4_GEMM_KERNEL
@@ -236,9 +239,16 @@ void launch_gemm_q3(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int
 // (gemm_skinny_scratch_bytes bytes at `packed_x`), then a kernel without LDS staging.
 bool gemm_skinny_wants(uint32_t n, uint32_t k, uint32_t m);
 size_t gemm_skinny_scratch_bytes(uint32_t k, uint32_t m);
+// For Q4 and a LoRA rank this accepts, the kernel computes t = A . X itself when LoraEpilogue::a points to A as
+// packed (on the host, once) by gemm_skinny_pack_lora_a; t is then not read and no launch for it has to precede.
+bool gemm_skinny_computes_t(uint32_t rank, uint32_t m);
+bool gemm_skinny_packs_lora_a(uint32_t rank);  // an adapter of this rank gets a packed copy of A at upload
+size_t gemm_skinny_packed_lora_a_bytes(uint32_t k);
+void gemm_skinny_pack_lora_a(const void* a_host, int a_is_f16, uint32_t rank, uint32_t k, void* out_host);
 // fmt: 0 = Q4 blocks, 1 = Q8_0, 2 = Q3.
+// pack = false: `packed_x` already holds the packed image of this x (an earlier call with the same x, K, m and format).
 void launch_gemm_skinny(const uint8_t* w, uint32_t n, uint32_t k, const void* x, int x_is_f16, uint32_t m, float* y,
-                        const LoraEpilogue& lora, void* packed_x, hipStream_t stream, int fmt = 0);
+                        const LoraEpilogue& lora, void* packed_x, hipStream_t stream, int fmt = 0, bool pack = true);
 
 bool launch_probe_read(const void* p, size_t nbytes, uint32_t grid, uint32_t in_flight, bool strided, bool nontemporal,
                        uint32_t* sink, hipStream_t stream);

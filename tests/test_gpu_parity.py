@@ -929,14 +929,14 @@ def test_gemm_weights_in_registers_kernel_with_lora(be):
 
 SKINNY_CASES = [(17, 16, 32, "f32"), (64, 2048, 2048, "f32"), (64, 512, 2048, "f16"), (33, 50, 96, "f32"),
                 (100, 130, 416, "f16"), (128, 36, 1024, "f32"), (20, 7, 160, "f32"), (200, 65, 224, "f16"),
-                (48, 8200, 256, "f32"), (64, 16400, 128, "f16")]
+                (48, 8200, 256, "f32"), (64, 16400, 128, "f16"), (64, 2100, 256, "f16"), (40, 4200, 128, "f32")]
 
 
 @pytest.mark.parametrize("m,n,k,xdt", SKINNY_CASES)
 def test_gemm_few_token_kernel_matches_oracle(be, m, n, k, xdt):
     # the few-token kernel: ragged token groups, N tails (also N % 4 != 0), K tails inside a
-    # 128-wide step, fewer K steps than waves, both row-tile widths; forced, so M > 128 is
-    # covered too
+    # 128-wide step, fewer K steps than waves, both row-tile widths, token tiles of 64 (132 row tiles at 64
+    # tokens) and of 32 (up to 128 workgroups, or 257..384 of them); forced, so M > 128 is covered too
     import torch
     print(f"gemm few-token m={m} n={n} k={k} x={xdt}", flush=True)
     wq = synth.q4_weight(n, k, seed=8, symmetric_bias=(k != 96))

@@ -498,9 +498,9 @@ def main():
                                              "with_lora_us": round(res[True] * 1e3, 3),
                                              "GB/s_with_lora": round(lb / res[True] / 1e6, 1),
                                              "lora_overhead_pct": round(100 * (res[True] / res[False] - 1), 1)}
-                if bsz <= 16:
+                if bsz <= 128:
                     # the same two projections through lq4_gemv_multi: one call for both (one launch at batch 1,
-                    # every adapter's A . x in one more)
+                    # every adapter's A . x in one more up to 16 rows; above, one packed image of x for both)
                     def mstep(i, use_lora, bsz=bsz, xl=xl, yl=yl):
                         bufs = pool[i % len(pool)]
                         be.gemv_multi(xl, [(bufs[nm], n, yl[nm], nm) for nm, n, _ in projs], bsz, 2048,

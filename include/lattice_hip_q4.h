@@ -149,8 +149,11 @@ int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
  * one more launch in front instead).  Needs K * 4.5 bytes <= 128 KB of LDS (K <= 29120) and, for K of 512 or 1024 (rows
  * side by side in a wave), every n_i a multiple of 4 or 2.  At batch 2..8 projections whose n_i are multiples of 16,
  * with K <= 2048 and at most 4096 rows in all, are one launch of the integer matrix-core kernel over the stacked rows
- * (plus the one A . X launch for all adapters).  Other shapes and batches go projection by projection through
- * lq4_gemv's own routing (still one A . X launch for all adapters).
+ * (plus the one A . X launch for all adapters).  Other shapes and batches up to 16 go projection by projection
+ * through lq4_gemv's own routing (still one A . X launch for all adapters that need one).  At batch 17..128 every
+ * projection takes lq4_gemm's routing for f32 activations, and those the few-token kernel serves share one packed
+ * image of x (one pack launch for q, k and v instead of three; adapters of rank <= 16 up to 64 rows have their
+ * A . X computed inside that kernel, no launch for it).  Above 128 rows: LQ4_E_INVALID, use lq4_gemm.
  * A projection with n == 0 is skipped.  Results are those of `count` lq4_gemv calls to the contract's tolerance
  * (bit-identical without LoRA at batch 1: same kernel, same order of summation).  The A . x values live in the
  * context: calls with adapters must not overlap on two streams of one context.  Every projection is checked

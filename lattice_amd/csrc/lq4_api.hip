@@ -71,6 +71,7 @@ constexpr size_t kFusedPrologueBytes = 64u << 10;  // lq4_gemv_fused_batch: see 
 constexpr uint32_t kSharedB1MaxTokens = 8;  // shared expert alone through the per-pair kernels up to here (route + routed + shared as three calls: 8 tokens 56.0 -> 51.7 us, 16 tokens 68.5 -> 66.6, 32 tokens 89.3 -> 94.3)
 constexpr uint32_t kMoeB1MaxTokens = 8;  // per-pair expert kernels up to here (measured: 1 / 2 / 4 / 8 / 16 tokens 27.5 / 30.5 / 43.2 / 45.1 / 48.6 us grouped, 13.7 / 18.3 / 25.9 / 39.1 / 65.0 per pair)
 constexpr uint32_t kMoeSharedGroupedMaxTokens = 56;  // lq4_moe_ffn: shared expert as one more expert of the grouped kernels up to here
+constexpr uint32_t kMultiMaxRows = 128;  // lq4_gemv_multi: up to the few-token GEMM's range
 constexpr uint32_t kLoraTRows = 4096;  // most rows one LoRA-fused call may carry
 
 thread_local char g_err[512] = "";
@@ -509,7 +510,7 @@ int lq4_gemv_multi(lq4_ctx* ctx, const lq4_projection* proj, uint32_t count, uin
     if (count == 0 || batch == 0) return LQ4_OK;
     if (!proj) return fail(LQ4_E_INVALID, "proj is null");
     if (count > LQ4_MAX_PROJECTIONS) return fail(LQ4_E_INVALID, "%u projections, at most %d a call", count, LQ4_MAX_PROJECTIONS);
-    if (batch > kMaxGemvBatch) return fail(LQ4_E_INVALID, "lq4_gemv_multi batch %u above %d; use lq4_gemm", batch, kMaxGemvBatch);
+    if (batch > kMultiMaxRows) return fail(LQ4_E_INVALID, "lq4_gemv_multi batch %u above %u; use lq4_gemm", batch, kMultiMaxRows);
     if (!x_dev) return fail(LQ4_E_INVALID, "x device pointer is null");
     if (reinterpret_cast<uintptr_t>(x_dev) % 16) return fail(LQ4_E_INVALID, "x must be 16-byte aligned");
     // every projection is checked before anything is launched: a call fails whole or not at all
@@ -553,6 +554,44 @@ int lq4_gemv_multi(lq4_ctx* ctx, const lq4_projection* proj, uint32_t count, uin
     if (mv.count == 0) return LQ4_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
     DeviceGuard g(ctx->device);
+    if (batch > kMaxGemvBatch) {
+        // 17..128 rows: lq4_gemm's routing projection by projection.  Those the few-token GEMM serves share one packed
+        // image of x (packed by the first of them) and compute their A . X themselves where that kernel can.
+        if (with_lora) {
+            const int rc = enter_shared_state(ctx, s);
+            if (rc) return rc;
+        }
+        bool x_packed = false;
+        for (uint32_t i = 0; i < count; ++i) {
+            const lq4_projection& p = proj[i];
+            if (p.n == 0) continue;
+            const bool few = gemm_takes_few_token_kernel(p.n, k, batch, 0, ctx->gemm_kernel);
+            LoraEpilogue e = ep[i];
+            if (e.rank && few && gemm_skinny_computes_t(e.rank, batch)) {
+                e.a = p.lora->a_packed;
+            } else if (e.rank) {
+                e.t = ctx->lora_t;  // one after the other on this stream
+                launch_lora_a(p.lora->a, p.lora->is_f16, e.rank, k, x_dev, 0, k, batch, ctx->lora_t, s);
+                ctx->counters.lora_a++;
+            }
+            const size_t scratch_bytes = gemm_scratch_floats(p.n, k, batch, 0, e.rank != 0, ctx->gemm_kernel) * sizeof(float);
+            if (scratch_bytes) {
+                const int rc = ensure_scratch(ctx, scratch_bytes, s);
+                if (rc) return rc;
+            }
+            if (few) {
+                launch_gemm_skinny(wp[i], p.n, k, x_dev, 0, batch, p.y_dev, e, ctx->moe_scratch, s, 0, !x_packed);
+                x_packed = true;
+            } else {
+                launch_gemm(wp[i], p.n, k, x_dev, 0, batch, p.y_dev, e,
+                            scratch_bytes ? reinterpret_cast<float*>(ctx->moe_scratch) : nullptr, ctx->gemm_kernel, s);
+                x_packed = false;  // (that kernel's partial tiles share the scratch)
+            }
+            ctx->counters.gemm++;
+        }
+        LQ4_HIP(hipGetLastError());
+        return LQ4_OK;
+    }
     const bool stacked = batch == 1 && (mv.count > 1 || with_lora) && gemv_multi_serves(mv, k);
     // one token: the stacked launch computes every A_v . x in producer workgroups of its own (lane l of a weight
     // wave holds the factor of stacked row l, hence at most 64 rows of A in all)

@@ -194,6 +194,48 @@ def test_multi_rows_stacked_on_the_integer_kernel(be, batch):
             assert e <= ((5e-6 if batch <= 4 else 1e-4) if one else REL_TOL), (n, e)
 
 
+@pytest.mark.parametrize("batch", [40, 64, 128])
+def test_multi_above_sixteen_rows_goes_through_the_gemm_routing(be, batch):
+    # 17..128 rows: projection by projection as lq4_gemm would, the few-token GEMM's packed activations shared;
+    # adapters of rank <= 16 up to 64 rows get their A . X inside that kernel, others a launch of their own.  The
+    # wide projection in the middle (more than 2^26 weights) is served by the large-tile kernel, whose partial
+    # tiles overwrite the packed activations: the projection behind it packs them again.
+    import torch
+    print(f"multi rows={batch}", flush=True)
+    k = 2048
+    names, shapes = ("q_proj", "up_proj", "v_proj", "k_proj"), (2048, 33000, 512, 512)
+    ws, qs = _views(be, shapes, k, seed=50)
+    mods = {"q_proj": synth.lora_pair(16, k, 2048, seed=1, tag="q"),
+            "v_proj": synth.lora_pair(8, k, 512, seed=2, tag="v"),
+            "k_proj": synth.lora_pair(24, k, 512, seed=3, tag="k")}
+    x = synth.activations(batch, k, seed=9)
+    xd = dev(x)
+    be.load_lora_adapter([backend.LoraLayerData(1, mods)], scale=2.0)
+    try:
+        ys = [torch.full((batch, n), float("nan"), dtype=torch.float32, device="cuda") for n in shapes]
+        c0 = be.path_counters()
+        be.gemv_multi(xd, [(q, n, y, nm) for q, n, y, nm in zip(qs, shapes, ys, names)], batch, k, layer_idx=1)
+        be.synchronize()
+        c1 = be.path_counters()
+        assert c1["gemm"] == c0["gemm"] + 4 and c1["gemv_multi"] == c0["gemv_multi"]
+        # rank 24 always has its own A . X launch; ranks 16 and 8 only above 64 rows
+        assert c1["lora_a"] == c0["lora_a"] + (1 if batch <= 64 else 3)
+        for w, q, n, y, nm in zip(ws, qs, shapes, ys, names):
+            base = oracle.gemm_f32(x, w, n, k)
+            want = base
+            if nm in mods:
+                a, b = mods[nm]
+                want = oracle.lora_apply(a.astype(np.float32), b.astype(np.float32), 2.0, x, base)
+            e = rel_err(host(y), want)
+            print(f"  {nm}: rel err {e:.2e}", flush=True)
+            assert e <= REL_TOL
+            sep = torch.empty((batch, n), dtype=torch.float32, device="cuda")
+            be.dispatch_gemm(xd, 0, q, sep, 0, batch, n, k, layer_idx=1, module=nm)
+            assert np.array_equal(host(y), host(sep)), "the same kernels as a single lq4_gemm call"
+    finally:
+        be.unload_lora_adapter()
+
+
 def test_multi_fallbacks_keep_the_contract(be):
     # K 1024 with an odd-sized view (rows side by side would straddle two views), a single view, K beyond the LDS
     # staging: served projection by projection, same results
@@ -225,7 +267,7 @@ def test_multi_contract_errors_launch_nothing(be):
     with pytest.raises(backend.Q4Error):
         be.gemv_multi(x, [(qs[0], 64, y0), (qs[1], 65, small)], 1, k)
     with pytest.raises(backend.Q4Error):
-        be.gemv_multi(x, [(qs[0], 64, y0), (qs[1], 64, small)], 17, k)
+        be.gemv_multi(x, [(qs[0], 64, y0), (qs[1], 64, small)], 129, k)
     arr = (backend.Projection * 2)()
     arr[0].w, arr[0].n, arr[0].y_dev = qs[0].handle, 64, y0.data_ptr()
     arr[1].w, arr[1].n, arr[1].y_dev = qs[1].handle, 64, None

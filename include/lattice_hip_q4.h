@@ -122,7 +122,10 @@ int lq4_lora_apply(lq4_ctx* ctx, const lq4_lora* lora, float lora_scale, const v
  * payload_offset + w_extra_offset bytes into the weight buffer (qw_extra_offset of
  * dispatch_gemm_at, dispatch.rs:935-980).
  * At batch 1 with a LoRA adapter the launch computes A . x itself and keeps a few words of
- * hand-over state in the context: such calls must not overlap on two streams of one context.
+ * hand-over state in the context: such calls must not overlap on two streams of one context.  The
+ * same holds at 2..8 rows where the integer matrix-core kernel serves the call and its tiles leave
+ * `rank` CUs idle, and (without any state) from 9 rows on for ranks up to 16, where the few-token
+ * kernel computes A . X for its own token tile: no launch for A . x precedes any of these.
  * Activation range: at batch 1 any finite f32 value (activations are staged as 23-bit fixed point
  * scaled by a power of two per 32-element block and multiplied exactly, so the result tracks an f32
  * GEMV as the reference's gemv_q4_decode does, shaders/qwen35.metal:794-866; an infinite or NaN
@@ -149,7 +152,8 @@ int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
  * one more launch in front instead).  Needs K * 4.5 bytes <= 128 KB of LDS (K <= 29120) and, for K of 512 or 1024 (rows
  * side by side in a wave), every n_i a multiple of 4 or 2.  At batch 2..8 projections whose n_i are multiples of 16,
  * with K <= 2048 and at most 4096 rows in all, are one launch of the integer matrix-core kernel over the stacked rows
- * (plus the one A . X launch for all adapters).  Other shapes and batches up to 16 go projection by projection
+ * (the A . X of all adapters in producer workgroups of that launch where CUs are idle for them, else in one
+ * launch in front).  Other shapes and batches up to 16 go projection by projection
  * through lq4_gemv's own routing (still one A . X launch for all adapters that need one).  At batch 17..128 every
  * projection takes lq4_gemm's routing for f32 activations, and those the few-token kernel serves share one packed
  * image of x (one pack launch for q, k and v instead of three; adapters of rank <= 16 up to 64 rows have their

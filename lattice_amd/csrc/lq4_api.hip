@@ -23,6 +23,7 @@ struct lq4_ctx {
     uint8_t* moe_scratch; // grown on demand
     uint32_t* topk_ticket; // finished-workgroup count of the top-k kernel, zero between launches
     uint32_t* lora_sync;   // fall-back count (word 2) and, from word 64 on, the slots of the batch-1 GEMV that computes A.x itself (same allocation)
+    unsigned long long* lora_slots_rows;  // [kMaxLoraRank][8]: the slots of the 2..8-row GEMV that computes A.x itself (same allocation)
     bool lora_in_kernel;
     uint32_t lora_spin_limit;  // polls a weight wave spends on those counters before it computes A.x alone
     size_t moe_scratch_bytes;
@@ -200,10 +201,10 @@ int lq4_ctx_create(int device_ordinal, lq4_ctx** out) {
         delete c;
         return fail(LQ4_E_HIP, "hipMalloc(lora scratch): %s", hipGetErrorString(e));
     }
-    // 256 B of top-k ticket, 256 B for the LoRA fall-back count, 512 B of LoRA slots (a zeroed slot matches no
-    // launch: every tag has its top bit set)
-    e = hipMalloc(reinterpret_cast<void**>(&c->topk_ticket), 1024);
-    if (e == hipSuccess) e = hipMemset(c->topk_ticket, 0, 1024);
+    // 256 B of top-k ticket, 256 B for the LoRA fall-back count, 512 B of LoRA slots for one activation row, 4 KB
+    // of them for up to eight rows (a zeroed slot matches no launch: every tag has its top bit set)
+    e = hipMalloc(reinterpret_cast<void**>(&c->topk_ticket), 1024 + 8 * kMaxLoraRank * 8);
+    if (e == hipSuccess) e = hipMemset(c->topk_ticket, 0, 1024 + 8 * kMaxLoraRank * 8);
     if (e != hipSuccess) {
         (void)hipFree(c->topk_ticket);
         (void)hipFree(c->lora_t);
@@ -218,6 +219,7 @@ int lq4_ctx_create(int device_ordinal, lq4_ctx** out) {
         return fail(LQ4_E_HIP, "hipGetSymbolAddress(static scratch): %s", hipGetErrorString(e));
     }
     c->lora_sync = c->topk_ticket + 64;
+    c->lora_slots_rows = reinterpret_cast<unsigned long long*>(c->topk_ticket + 256);
     hipDeviceProp_t prop;
     e = hipGetDeviceProperties(&prop, device_ordinal);
     if (e != hipSuccess) {
@@ -431,8 +433,14 @@ static bool gemv_takes_few_token_gemm(uint32_t n, uint32_t k, uint32_t batch) {
     return batch >= 9 || (batch >= 5 && n < 8192 && !narrow && weights >= 6000000);
 }
 
-// The routing of lq4_gemv once the LoRA factor t (if any) is in ep, or ep.a says that the few-token GEMM computes
-// it: which kernel serves (batch, n, k).
+// 2..8 rows on the integer matrix-core kernel (after the few-token GEMM has had its pick).
+static bool gemv_takes_i8(const lq4_ctx* ctx, uint32_t n, uint32_t k, uint32_t batch) {
+    return !gemv_takes_few_token_gemm(n, k, batch) && batch >= 2 && batch <= 8 && ctx->gemv_i8 &&
+           (ctx->gemv_i8 == 2 || (batch >= 3 && k <= 2048 && n <= 4096)) && gemv_i8_serves(n, k, batch, ctx->cu_count);
+}
+
+// The routing of lq4_gemv once the LoRA factor t (if any) is in ep, or ep.a says that the kernel which serves the
+// shape computes it: which kernel serves (batch, n, k).
 // `x_packed` (may be null): calls in a row on the same x, K and batch share the few-token GEMM's packed activations;
 // true once a call has packed them into the context's scratch.
 static int gemv_dispatch(lq4_ctx* ctx, const uint8_t* wp, uint32_t n, uint32_t k, const float* x_dev, uint32_t batch,
@@ -446,9 +454,7 @@ static int gemv_dispatch(lq4_ctx* ctx, const uint8_t* wp, uint32_t n, uint32_t k
         ctx->counters.gemm++;
     } else if (batch == 1 && !ep.rank) {
         plain_gemv_one_token(ctx, wp, n, k, x_dev, y_dev, s);
-    } else if (batch >= 2 && batch <= 8 && ctx->gemv_i8 &&
-               (ctx->gemv_i8 == 2 || (batch >= 3 && k <= 2048 && n <= 4096)) &&
-               gemv_i8_serves(n, k, batch, ctx->cu_count)) {
+    } else if (gemv_takes_i8(ctx, n, k, batch)) {
         // Three to eight rows of a matrix of up to 4096 x 2048: the integer matrix-core kernel, which is as fast as
         // or faster than the 4x4x4 kernel there (512 x 2048: 4.33 -> 4.09 us at four rows, 4.71 -> 4.53 at eight;
         // 2048 x 2048: 4.67 -> 4.54, 5.09 -> 4.98; 3072 x 2048 at four rows 5.58 -> 4.82) and keeps 24 (up to four rows)
@@ -494,6 +500,13 @@ int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
         ep.spin_limit = ctx->lora_spin_limit;
     } else if (ep.rank && batch > 1 && gemv_takes_few_token_gemm(n, k, batch) && gemm_skinny_computes_t(ep.rank, batch)) {
         ep.a = lora->a_packed;  // the few-token GEMM computes A.x for its token tile itself
+    } else if (ep.rank && ctx->lora_in_kernel && gemv_takes_i8(ctx, n, k, batch) &&
+               gemv_i8_lora_in_launch(n, k, batch, ep.rank, ctx->cu_count)) {
+        // 2..8 rows: `rank` producer workgroups of the launch, on CUs the matrix leaves idle
+        ep.a = lora->a;
+        ep.slots = ctx->lora_slots_rows;
+        ep.sync = ctx->lora_sync;
+        ep.spin_limit = ctx->lora_spin_limit;
     } else if (ep.rank) {
         launch_lora_a(lora->a, lora->is_f16, lora->rank, k, x_dev, 0, k, batch, ctx->lora_t, s);
         ctx->counters.lora_a++;
@@ -612,16 +625,26 @@ int lq4_gemv_multi(lq4_ctx* ctx, const lq4_projection* proj, uint32_t count, uin
             ++v;
         }
     }
+    // ... and computes every A_v . x in producer workgroups of its own where CUs are left idle for them
+    const bool rows_in_launch = stacked_rows && with_lora && ctx->lora_in_kernel &&
+                                gemv_i8_lora_in_launch(mv.begin[mv.count], k, batch, total_rank, ctx->cu_count);
     if (with_lora) {  // the A . x buffer and the hand-over words belong to the context
         int rc = enter_shared_state(ctx, s);
         if (rc) return rc;
-        if (!in_launch) {
+        if (!in_launch && !rows_in_launch) {
             launch_lora_a_views(av, k, x_dev, k, batch, s);  // every adapter's A . x in one launch
             ctx->counters.lora_a++;
         }
     }
     if (stacked_rows) {
-        launch_gemv_i8_multi(mv, k, x_dev, k, batch, ctx->cu_count, s);
+        LoraEpilogue hand{};
+        if (rows_in_launch) {
+            hand.rank = total_rank;
+            hand.slots = ctx->lora_slots_rows;
+            hand.sync = ctx->lora_sync;
+            hand.spin_limit = ctx->lora_spin_limit;
+        }
+        launch_gemv_i8_multi(mv, k, x_dev, k, batch, ctx->cu_count, rows_in_launch ? &hand : nullptr, s);
         ctx->counters.gemv_multi++;
     } else if (stacked) {
         LoraEpilogue hand{};

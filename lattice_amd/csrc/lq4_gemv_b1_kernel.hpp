@@ -36,42 +36,6 @@ constexpr int kWaves = 4;  // waves per workgroup unless a launch asks for more
 // (residual add + shifted RMSNorm, or silu(gate) * up) and the result can be added into a
 // residual stream as it is stored.  Every workgroup stages the whole activation vector anyway,
 // so the norm costs one extra pass over K floats per workgroup and no launch.
-// Partial dot product of row `j` of A (f16 or f32, `k` long, k a multiple of 32) with x, for thread
-// `t` of `nt`: eight elements per step through 16-byte loads.
-__device__ __forceinline__ float lora_a_row_partial(const void* a, int a_is_f16, uint32_t j, uint32_t k,
-                                                    const float* __restrict__ x, uint32_t t, uint32_t nt) {
-    float p = 0.0f;
-    for (uint32_t kk = t * 8; kk < k; kk += nt * 8) {
-        const float4 x0 = *reinterpret_cast<const float4*>(x + kk), x1 = *reinterpret_cast<const float4*>(x + kk + 4);
-        float av[8];
-        if (a_is_f16) {
-            struct alignas(16) H8 { _Float16 v[8]; };
-            const H8 h = *reinterpret_cast<const H8*>(static_cast<const _Float16*>(a) + static_cast<size_t>(j) * k + kk);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) av[i] = static_cast<float>(h.v[i]);
-        } else {
-            const float4* ap = reinterpret_cast<const float4*>(static_cast<const float*>(a) + static_cast<size_t>(j) * k + kk);
-            const float4 a0 = ap[0], a1 = ap[1];
-            av[0] = a0.x; av[1] = a0.y; av[2] = a0.z; av[3] = a0.w;
-            av[4] = a1.x; av[5] = a1.y; av[6] = a1.z; av[7] = a1.w;
-        }
-        p = fmaf(av[0], x0.x, p); p = fmaf(av[1], x0.y, p); p = fmaf(av[2], x0.z, p); p = fmaf(av[3], x0.w, p);
-        p = fmaf(av[4], x1.x, p); p = fmaf(av[5], x1.y, p); p = fmaf(av[6], x1.z, p); p = fmaf(av[7], x1.w, p);
-    }
-    return p;
-}
-
-// The tag of a launch: where its dispatch packet lies in the queue's ring (a 64-byte slot of it; the address is an
-// input register of every wave).  Every workgroup of one launch sees the same packet, the next launch on the queue
-// the next slot, also when a captured graph is replayed (the packets are written again); other queues of the
-// process have their rings elsewhere.  31 bits of the slot number, the top bit set so that a zeroed word never
-// matches.  A launch could only take another launch's words for its own if that one lay a whole number of laps of
-// the ring earlier AND no launch in between had published to the same slots.
-__device__ __forceinline__ uint32_t launch_tag() {
-    const uintptr_t packet = reinterpret_cast<uintptr_t>(__builtin_amdgcn_dispatch_ptr());
-    return static_cast<uint32_t>(packet >> 6) | 0x80000000u;
-}
-
 // Whole-wave call.  Returns t[lane] (0 beyond the rank) once every slot carries this launch's tag; polls the
 // slots at most `spin_limit` times and otherwise computes t in this wave.  The slots are read with
 // agent-scope atomic loads (they do not hit in this XCD's caches), value and tag in one word.

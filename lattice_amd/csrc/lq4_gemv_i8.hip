@@ -31,6 +31,15 @@
 // of 8 blocks and add their partial sums through LDS in wave order.  Each wave stages the activations of its own
 // chunks only, once for all tiles of the workgroup, behind its first weight loads.
 //
+// LoRA.  The factor t = A . x of the adapter (of every view's adapter) is either in memory when the launch starts
+// (lora.t / mv.t), or computed by the launch itself (lora.slots set): the first lora.rank workgroups are producers,
+// one per row of A (the views' A stacked), each forming that row's dot products with the batch's activation rows
+// and publishing them as {value, tag of the launch} words; the other workgroups pick them up into LDS after their
+// staging barrier, by which time the producers, who have nothing else to do, are long done.  The launcher adds the
+// producers only where CUs are idle anyway (tiles + producers <= CUs): a matrix of 2560 rows occupies 160.  A value
+// that has not arrived after the poll limit is computed by the wave that misses it, in the producers' order of
+// summation (same bits), and counted in sync[2].
+//
 // Precision.  The weights enter exactly, the integer sums are exact.  An activation is rounded to a multiple of its
 // block's largest magnitude / 32639 (two digits: step 3e-5 of the block maximum, against 5e-4 of the element for the
 // f16 rounding of the 4x4x4 kernel and of the reference's tiled kernel, shaders/gemm_q4_tiled.metal:45-48) or
@@ -83,24 +92,55 @@ __global__ __launch_bounds__(64 * CW * TW) void gemv_q4_i8(const uint8_t* __rest
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // ---- producers of the LoRA factors (see the head of the file): workgroup p < prod owns stacked row p of A ----
+    const uint32_t prod = lora.slots ? lora.rank : 0;  // (several views: lora.rank is the ranks of all views together)
+    auto a_row_of = [&](uint32_t p, const void*& a, int& a_is_f16, uint32_t& j) {
+        a = lora.a;
+        a_is_f16 = lora.b_is_f16;
+        j = p;
+        if constexpr (MULTI) {
+            uint32_t v = 0;
+#pragma unroll
+            for (int i = 1; i < kMaxViews; ++i) v += (static_cast<uint32_t>(i) < mv.count && p >= mv.t_off[i]) ? 1u : 0u;
+            a = mv.a[v];
+            a_is_f16 = mv.b_is_f16[v];
+            j = p - mv.t_off[v];
+        }
+    };
+    if (blockIdx.x < prod) {
+        const void* a;
+        int a_is_f16;
+        uint32_t j;
+        a_row_of(blockIdx.x, a, a_is_f16, j);
+        // a wave per activation row: no barrier, nothing through LDS, one cross-lane sum before the word goes out
+        for (uint32_t b = wave; b < batch; b += WAVES) {
+            const float total = wave_sum(lora_a_row_partial(a, a_is_f16, j, k, x + static_cast<size_t>(b) * x_stride, lane, 64));
+            const unsigned long long word = (static_cast<unsigned long long>(launch_tag()) << 32) | as_u32(total);
+            if (lane == 0) __hip_atomic_store(&lora.slots[blockIdx.x * 8 + b], word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        return;
+    }
+    const uint32_t wg = blockIdx.x - prod, n_wg = gridDim.x - prod;  // this workgroup among those that stream weights
     const uint32_t tw = wave / CW, cw = wave % CW;
     const uint32_t nb = k / kBlockWeights;
     const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
-    // LDS: [nb] activation digits | [nb] activation scales and sums | [WAVES] tiles | [WAVES][64][2] partial sums
+    // LDS: [nb] activation digits | [nb] activation scales and sums | [WAVES] tiles | [WAVES][64][2] partial sums |
+    // [8][64] LoRA factors
     uint8_t* const xq = smem;
     uint8_t* const xf = xq + static_cast<size_t>(nb) * kXqBytes;
     uint32_t* const tile = reinterpret_cast<uint32_t*>(xf + static_cast<size_t>(nb) * kXfBytes) + wave * kTileDwords;
     float* const part = reinterpret_cast<float*>(xf + static_cast<size_t>(nb) * kXfBytes) + WAVES * kTileDwords;
+    float* const t_lds = part + WAVES * 64 * 2;  // [8 activation rows][kMaxLoraRank]: the factors picked up from the producers
 
     const uint32_t n_tiles = (n + 15) / 16;
     const uint32_t chunks = (nb + kBpw - 1) / kBpw;
     const uint32_t my_chunks = cw < chunks ? (chunks - cw + CW - 1) / CW : 0;  // chunk c * CW + cw
     // tiles of the workgroup: blockIdx + j * gridDim; of this wave: j = tw, tw + TW, ...; a round = TW tiles
-    const uint32_t wg_tiles = blockIdx.x < n_tiles ? (n_tiles - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
+    const uint32_t wg_tiles = wg < n_tiles ? (n_tiles - wg + n_wg - 1) / n_wg : 0;
     const uint32_t rounds = (wg_tiles + TW - 1) / TW;
     const uint32_t my_tiles = tw < wg_tiles ? (wg_tiles - tw + TW - 1) / TW : 0;
     const uint32_t units = my_tiles * my_chunks;  // unit u = (my tile u / my_chunks, my chunk u % my_chunks)
-    auto first_row = [&](uint32_t t) { return (blockIdx.x + (t * TW + tw) * gridDim.x) * 16; };
+    auto first_row = [&](uint32_t t) { return (wg + (t * TW + tw) * n_wg) * 16; };
     // MULTI: the view that holds stacked row `row` (uniform: called with a tile's first row)
     auto view_of = [&](uint32_t row) {
         uint32_t v = 0;
@@ -111,6 +151,7 @@ __global__ __launch_bounds__(64 * CW * TW) void gemv_q4_i8(const uint8_t* __rest
         return v;
     };
 
+    auto r_of = [](int l) { return static_cast<uint32_t>(l & 15); };  // the weight row of the tile a lane's outputs belong to
     // load mapping: lane = (block jl, row rq), rows rq + kRowStep * i
     constexpr int kRowStep = 64 / kBpw, kLoads = 16 / kRowStep;
     const uint32_t jl = lane % kBpw, rq = lane / kBpw;
@@ -226,6 +267,33 @@ __global__ __launch_bounds__(64 * CW * TW) void gemv_q4_i8(const uint8_t* __rest
         }
     };
 
+    // The LoRA factor B of the wave's first tile (its first sixteen ranks, f16 in eights) is requested before
+    // anything else and used in that tile's epilogue: requested there, its whole latency stood between the last
+    // matrix instruction and the store, and a workgroup of these launches has one tile or two.
+    struct alignas(16) H8 { _Float16 v[8]; };
+    H8 b_pre[2] = {};
+    bool use_pre = false;
+    if (cw == 0 && my_tiles) {  // uniform
+        const uint32_t row0 = first_row(0);
+        const void* bq = lora.b;
+        uint32_t rank = lora.rank, row_end = n, row_base = 0;
+        int b16 = lora.b_is_f16;
+        if constexpr (MULTI) {
+            const uint32_t v = view_of(row0);
+            bq = mv.b[v];
+            rank = mv.rank[v];
+            b16 = mv.b_is_f16[v];
+            row_end = mv.begin[v + 1];
+            row_base = mv.begin[v];
+        }
+        if (rank && b16 && rank % 8 == 0) {
+            use_pre = true;
+            const uint32_t row = (row0 + r_of(lane) < row_end ? row0 + r_of(lane) : row_end - 1) - row_base;
+            const _Float16* brow = static_cast<const _Float16*>(bq) + static_cast<size_t>(row) * rank;
+            b_pre[0] = *reinterpret_cast<const H8*>(brow);
+            b_pre[1] = *reinterpret_cast<const H8*>(brow + (rank >= 16 ? 8 : 0));
+        }
+    }
     float4 xv[kHoist][2];
 #pragma unroll
     for (int it = 0; it < kHoist; ++it) {
@@ -244,8 +312,17 @@ __global__ __launch_bounds__(64 * CW * TW) void gemv_q4_i8(const uint8_t* __rest
         if (static_cast<uint32_t>(i) < units) load_unit(ring[i], i);
     }
     __builtin_amdgcn_sched_barrier(0);  // nothing below is scheduled above these loads
+    // The LoRA factors of the producers: item i = (stacked row of A i / 8, activation row i % 8), thread i looks at
+    // item i while it still has staging to do (the producers need about 2 us, the activations arrive after 1.5),
+    // so that in the usual case the value is there when the staging is, and one barrier publishes both.
+    const uint32_t tag = launch_tag();
+    const unsigned long long none = static_cast<unsigned long long>(tag) << 32;  // lanes without an item: as if published
+    const bool early_mine = static_cast<uint32_t>(tid) < prod * 8 && (static_cast<uint32_t>(tid) & 7) < batch;
+    unsigned long long early = none;
 #pragma unroll
     for (int it = 0; it < kHoist; ++it) {
+        if (it == kHoist - 1 && early_mine && lora.spin_limit)
+            early = __hip_atomic_load(&lora.slots[tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         const uint32_t idx = tid + it * 64 * WAVES;
         if (idx < n_tasks) stage_task(idx, xv[it][0], xv[it][1]);  // (whole quads: n_tasks is a multiple of 4)
     }
@@ -253,7 +330,46 @@ __global__ __launch_bounds__(64 * CW * TW) void gemv_q4_i8(const uint8_t* __rest
         const float4* xp = task_ptr(idx);
         stage_task(idx, xp[0], xp[1]);
     }
+    if (prod && static_cast<uint32_t>(tid) < prod * 8)
+        t_lds[(tid & 7) * kMaxLoraRank + (tid >> 3)] = early_mine ? as_f32(static_cast<uint32_t>(early)) : 0.0f;
     __syncthreads();
+    // A wave some of whose values were not there yet (or that has more items than lanes) goes the patient way.  No
+    // barrier of its own: whoever reads t_lds does so in a tile's epilogue, behind the two barriers of the partial
+    // sums that every wave passes once a round (a workgroup of one wave reads its own writes).
+    const bool early_bad = early_mine && (!lora.spin_limit || static_cast<uint32_t>(early >> 32) != tag);
+    if (prod && (__any(early_bad) || prod * 8 > 64 * WAVES)) {  // uniform in the wave
+        for (uint32_t i0 = wave * 64; i0 < prod * 8; i0 += 64 * WAVES) {  // uniform
+            const uint32_t i = i0 + lane;
+            const bool mine = i < prod * 8 && (i & 7) < batch;
+            // first through the caches (the usual case: the producers are done, one fetch per XCD), then past them
+            unsigned long long v = none;
+            if (lora.spin_limit) {
+                if (mine) v = *static_cast<const volatile unsigned long long*>(&lora.slots[i]);
+                for (uint32_t spin = 0; spin < lora.spin_limit && !__all(static_cast<uint32_t>(v >> 32) == tag); ++spin) {
+                    __builtin_amdgcn_s_sleep(4);
+                    if (mine) v = __hip_atomic_load(&lora.slots[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            } else if (mine) {
+                v = 0;  // (no polling at all: every item is computed here)
+            }
+            float val = as_f32(static_cast<uint32_t>(v));
+            uint64_t missing = __ballot(static_cast<uint32_t>(v >> 32) != tag);
+            while (missing) {  // uniform: the wave computes the item itself, in the producers' order of summation
+                const uint32_t fl = static_cast<uint32_t>(__builtin_ctzll(missing));
+                missing &= missing - 1;
+                const uint32_t item = i0 + fl;
+                const void* a;
+                int a_is_f16;
+                uint32_t j;
+                a_row_of(item >> 3, a, a_is_f16, j);
+                const float* xr = x + static_cast<size_t>(item & 7) * x_stride;
+                const float total = wave_sum(lora_a_row_partial(a, a_is_f16, j, k, xr, lane, 64));
+                if (static_cast<uint32_t>(lane) == fl) val = total;
+                if (lane == 0) __hip_atomic_fetch_add(&lora.sync[2], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            if (i < prod * 8) t_lds[(i & 7) * kMaxLoraRank + (i >> 3)] = mine ? val : 0.0f;
+        }
+    }
 
     // ---- the product ----
     const uint32_t r = lane & 15, g = lane >> 4;  // operand mapping: weight row r of the tile, k group / row pair g
@@ -348,18 +464,16 @@ __global__ __launch_bounds__(64 * CW * TW) void gemv_q4_i8(const uint8_t* __rest
                     ys = mv.begin[v + 1] - mv.begin[v];
                     lrow = row - mv.begin[v];
                 }
-                if (lo.rank) {
+                // t of activation rows b0 and b1, `t0[i]` = factor i: from memory, or (producers) from LDS
+                auto delta = [&](auto* t0, auto* t1) {
                     // (every load below is unconditional and used where it is made: a load left pending on one path
                     // would make the compiler wait for the whole weight ring wherever its register is reused)
-                    const float* t0 = lo.t + (b0 < batch ? b0 : 0) * lo.rank;
-                    const float* t1 = lo.t + (b1 < batch ? b1 : 0) * lo.rank;
                     float l0 = 0.0f, l1 = 0.0f;
                     if (lo.b_is_f16 && lo.rank % 8 == 0) {
-                        // eight factors a step: one 16-byte load of B[row, i..i+7] and four of t
+                        // eight factors a step: one 16-byte load of B[row, i..i+7] (the first two steps of the wave's
+                        // first tile: requested at the start of the kernel) and four of t
                         const _Float16* brow = static_cast<const _Float16*>(lo.b) + static_cast<size_t>(lrow) * lo.rank;
-                        for (uint32_t i = 0; i < lo.rank; i += 8) {
-                            struct alignas(16) H8 { _Float16 v[8]; };
-                            const H8 bq = *reinterpret_cast<const H8*>(brow + i);
+                        auto eight = [&](const H8& bq, uint32_t i) {
                             const float4 ta = *reinterpret_cast<const float4*>(t0 + i), tb = *reinterpret_cast<const float4*>(t0 + i + 4);
                             const float4 ua = *reinterpret_cast<const float4*>(t1 + i), ub = *reinterpret_cast<const float4*>(t1 + i + 4);
                             const float tv[8] = {ta.x, ta.y, ta.z, ta.w, tb.x, tb.y, tb.z, tb.w};
@@ -370,7 +484,14 @@ __global__ __launch_bounds__(64 * CW * TW) void gemv_q4_i8(const uint8_t* __rest
                                 l0 = fmaf(bv, tv[jj], l0);
                                 l1 = fmaf(bv, uv[jj], l1);
                             }
+                        };
+                        uint32_t i = 0;
+                        if (use_pre && t == 0) {  // uniform
+                            eight(b_pre[0], 0);
+                            if (lo.rank >= 16) eight(b_pre[1], 8);
+                            i = lo.rank >= 16 ? 16 : 8;
                         }
+                        for (; i < lo.rank; i += 8) eight(*reinterpret_cast<const H8*>(brow + i), i);
                     } else {
                         for (uint32_t i = 0; i < lo.rank; ++i) {
                             const size_t bi = static_cast<size_t>(lrow) * lo.rank + i;
@@ -382,6 +503,16 @@ __global__ __launch_bounds__(64 * CW * TW) void gemv_q4_i8(const uint8_t* __rest
                     }
                     acc0 = fmaf(lo.scale, l0, acc0);
                     acc1 = fmaf(lo.scale, l1, acc1);
+                };
+                if (lo.rank) {
+                    const uint32_t c0 = b0 < batch ? b0 : 0, c1 = b1 < batch ? b1 : 0;
+                    if (prod) {
+                        uint32_t off = 0;
+                        if constexpr (MULTI) off = mv.t_off[view_of(first_row(t))];
+                        delta(t_lds + c0 * kMaxLoraRank + off, t_lds + c1 * kMaxLoraRank + off);
+                    } else {
+                        delta(lo.t + c0 * lo.rank, lo.t + c1 * lo.rank);
+                    }
                 }
                 if (b0 < batch) yv[static_cast<size_t>(b0) * ys + lrow] = acc0;
                 if (b1 < batch) yv[static_cast<size_t>(b1) * ys + lrow] = acc1;
@@ -427,7 +558,7 @@ bool plan_i8(uint32_t n, uint32_t k, uint32_t batch, uint32_t cu_count, I8Plan* 
     for (;;) {
         const uint32_t waves = p.cw * p.tw;
         p.lds = static_cast<size_t>(nb) * (kXqBytes + kXfBytes) + static_cast<size_t>(waves) * kTileDwords * 4 +
-                static_cast<size_t>(waves) * 64 * 2 * 4;
+                static_cast<size_t>(waves) * 64 * 2 * 4 + 8 * kMaxLoraRank * 4;
         if (p.lds <= 160 * 1024) break;
         if (p.tw > 1) p.tw /= 2;
         else if (p.cw > 1) p.cw /= 2;
@@ -450,8 +581,9 @@ void launch_i8(const I8Plan& p, const uint8_t* w, uint32_t n, uint32_t k, const 
                hipStream_t stream) {
     static LdsCapOnce lds_cap;
     lds_cap.raise(reinterpret_cast<const void*>(gemv_q4_i8<CW, TW, WIDE, MULTI>), 160 * 1024);
-    hipLaunchKernelGGL((gemv_q4_i8<CW, TW, WIDE, MULTI>), dim3(p.grid), dim3(64 * CW * TW), p.lds, stream, w, n, k, x,
-                       x_stride, batch, y, y_stride, lora, mv);
+    const uint32_t producers = lora.slots ? lora.rank : 0;
+    hipLaunchKernelGGL((gemv_q4_i8<CW, TW, WIDE, MULTI>), dim3(producers + p.grid), dim3(64 * CW * TW), p.lds, stream, w, n,
+                       k, x, x_stride, batch, y, y_stride, lora, mv);
 }
 
 template <bool WIDE, bool MULTI>
@@ -485,6 +617,15 @@ void launch_gemv_i8(const uint8_t* w, uint32_t n, uint32_t k, const float* x, ui
     else launch_i8_shape<false, false>(p, w, n, k, x, x_stride, batch, y, y_stride, lora, none, stream);
 }
 
+// The launch can carry `rank_total` producer workgroups for the LoRA factors when they find idle CUs beside the
+// workgroups that stream weights (one workgroup runs per CU), the slots (rank_total x 8) and the LDS hold them, and a
+// 16-byte row of A can be loaded (K a multiple of 8 elements is given: K is a multiple of 32).
+bool gemv_i8_lora_in_launch(uint32_t n, uint32_t k, uint32_t batch, uint32_t rank_total, uint32_t cu_count) {
+    I8Plan p;
+    return rank_total != 0 && rank_total <= static_cast<uint32_t>(kMaxLoraRank) && plan_i8(n, k, batch, cu_count, &p) &&
+           p.grid + rank_total <= cu_count;
+}
+
 // The stacked launch serves views that are whole numbers of 16-row tiles.
 bool gemv_i8_multi_serves(const MultiViews& mv, uint32_t k, uint32_t batch, uint32_t cu_count) {
     if (mv.count == 0 || mv.count > static_cast<uint32_t>(kMaxViews)) return false;
@@ -495,13 +636,13 @@ bool gemv_i8_multi_serves(const MultiViews& mv, uint32_t k, uint32_t batch, uint
 }
 
 void launch_gemv_i8_multi(const MultiViews& mv, uint32_t k, const float* x, uint32_t x_stride, uint32_t batch,
-                          uint32_t cu_count, hipStream_t stream) {
+                          uint32_t cu_count, const LoraEpilogue* in_launch, hipStream_t stream) {
     const uint32_t n = mv.begin[mv.count];
     I8Plan p;
     if (!plan_i8(n, k, batch, cu_count, &p)) return;  // the caller asked gemv_i8_multi_serves first
-    const LoraEpilogue none{};
-    if (batch <= 4) launch_i8_shape<true, true>(p, nullptr, n, k, x, x_stride, batch, nullptr, 0, none, mv, stream);
-    else launch_i8_shape<false, true>(p, nullptr, n, k, x, x_stride, batch, nullptr, 0, none, mv, stream);
+    const LoraEpilogue hand = in_launch ? *in_launch : LoraEpilogue{};  // rank = the views' ranks together, slots, sync
+    if (batch <= 4) launch_i8_shape<true, true>(p, nullptr, n, k, x, x_stride, batch, nullptr, 0, hand, mv, stream);
+    else launch_i8_shape<false, true>(p, nullptr, n, k, x, x_stride, batch, nullptr, 0, hand, mv, stream);
 }
 
 }  // namespace lq4

@@ -86,7 +86,7 @@ bool gemv_multi_serves(const MultiViews& mv, uint32_t k);
 // The same for 2..8 activation rows on the integer matrix-core kernel (views of whole 16-row tiles; t in memory).
 bool gemv_i8_multi_serves(const MultiViews& mv, uint32_t k, uint32_t batch, uint32_t cu_count);
 void launch_gemv_i8_multi(const MultiViews& mv, uint32_t k, const float* x, uint32_t x_stride, uint32_t batch,
-                          uint32_t cu_count, hipStream_t stream);
+                          uint32_t cu_count, const LoraEpilogue* in_launch, hipStream_t stream);
 // `in_launch`: null = every t_v is in memory; else the hand-over words (slots, sync, spin_limit, rank = the ranks' sum)
 // of a launch that computes the factors in producer workgroups of its own.
 void launch_gemv_multi(const MultiViews& mv, uint32_t k, const float* x, const LoraEpilogue* in_launch, hipStream_t stream);
@@ -128,8 +128,12 @@ bool gemv_b1_pairs_served(uint32_t n, uint32_t k);
 void launch_gemv_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y,
                     const LoraEpilogue& lora, hipStream_t stream);
 // 2..8 activation rows on the integer matrix cores (lq4_gemv_i8.hip): y = W . x, optional LoRA epilogue with t in
-// memory.  gemv_i8_serves: the staged activations fit the LDS (K up to about 7000).
+// memory or computed by producer workgroups of the launch (gemv_i8_lora_in_launch).  gemv_i8_serves: the staged activations fit the LDS (K up to about 7000).
 bool gemv_i8_serves(uint32_t n, uint32_t k, uint32_t batch, uint32_t cu_count);
+// true = the launch has room for `rank_total` producer workgroups that compute the LoRA factors t = A . x themselves
+// (LoraEpilogue::a and ::slots set, [rank_total][8] slots; for several views a, t_off of MultiViews and
+// in_launch->rank = rank_total): no launch for t has to precede.
+bool gemv_i8_lora_in_launch(uint32_t n, uint32_t k, uint32_t batch, uint32_t rank_total, uint32_t cu_count);
 void launch_gemv_i8(const uint8_t* w, uint32_t n, uint32_t k, const float* x, uint32_t x_stride, uint32_t batch,
                     float* y, uint32_t y_stride, const LoraEpilogue& lora, uint32_t cu_count, hipStream_t stream);
 
@@ -332,6 +336,42 @@ __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
     return v;
+}
+
+// Partial dot product of row `j` of A (f16 or f32, `k` long, k a multiple of 32) with x, for thread
+// `t` of `nt`: eight elements per step through 16-byte loads.
+__device__ __forceinline__ float lora_a_row_partial(const void* a, int a_is_f16, uint32_t j, uint32_t k,
+                                                    const float* __restrict__ x, uint32_t t, uint32_t nt) {
+    float p = 0.0f;
+    for (uint32_t kk = t * 8; kk < k; kk += nt * 8) {
+        const float4 x0 = *reinterpret_cast<const float4*>(x + kk), x1 = *reinterpret_cast<const float4*>(x + kk + 4);
+        float av[8];
+        if (a_is_f16) {
+            struct alignas(16) H8 { _Float16 v[8]; };
+            const H8 h = *reinterpret_cast<const H8*>(static_cast<const _Float16*>(a) + static_cast<size_t>(j) * k + kk);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) av[i] = static_cast<float>(h.v[i]);
+        } else {
+            const float4* ap = reinterpret_cast<const float4*>(static_cast<const float*>(a) + static_cast<size_t>(j) * k + kk);
+            const float4 a0 = ap[0], a1 = ap[1];
+            av[0] = a0.x; av[1] = a0.y; av[2] = a0.z; av[3] = a0.w;
+            av[4] = a1.x; av[5] = a1.y; av[6] = a1.z; av[7] = a1.w;
+        }
+        p = fmaf(av[0], x0.x, p); p = fmaf(av[1], x0.y, p); p = fmaf(av[2], x0.z, p); p = fmaf(av[3], x0.w, p);
+        p = fmaf(av[4], x1.x, p); p = fmaf(av[5], x1.y, p); p = fmaf(av[6], x1.z, p); p = fmaf(av[7], x1.w, p);
+    }
+    return p;
+}
+
+// The tag of a launch: where its dispatch packet lies in the queue's ring (a 64-byte slot of it; the address is an
+// input register of every wave).  Every workgroup of one launch sees the same packet, the next launch on the queue
+// the next slot, also when a captured graph is replayed (the packets are written again); other queues of the
+// process have their rings elsewhere.  31 bits of the slot number, the top bit set so that a zeroed word never
+// matches.  A launch could only take another launch's words for its own if that one lay a whole number of laps of
+// the ring earlier AND no launch in between had published to the same slots.
+__device__ __forceinline__ uint32_t launch_tag() {
+    const uintptr_t packet = reinterpret_cast<uintptr_t>(__builtin_amdgcn_dispatch_ptr());
+    return static_cast<uint32_t>(packet >> 6) | 0x80000000u;
 }
 
 // Shared inner loop of the GEMV-class kernels.  One wave accumulates R weight rows

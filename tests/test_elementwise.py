@@ -348,8 +348,9 @@ def test_fused_rows_with_a_lora_adapter_run_step_by_step(be, batch):
                                  add_residual=(residual, None), layer_idx=0, module="o_proj", batch=batch)
         after = be.path_counters()
         assert after["gemv_fused"] == before["gemv_fused"] and after["elementwise"] == before["elementwise"] + 2
-        # (from nine rows on the few-token GEMM serves the projection and computes A.x itself: no launch for it)
-        assert after["lora_a"] == before["lora_a"] + (1 if batch <= 8 else 0)
+        # (no launch for A.x: at three and eight rows the integer matrix-core kernel computes it in producer workgroups
+        # of its own launch, from nine rows on the few-token GEMM computes it for its token tile)
+        assert after["lora_a"] == before["lora_a"]
         xn = oracle.shifted_rms_norm(base, gamma, 1e-6)
         want = oracle.lora_apply(a, b, 1.5, xn, oracle.gemm_f32(xn, wq, n, k))
         for r in range(batch):

@@ -113,8 +113,9 @@ def test_multi_with_lora_on_q_and_v(be, batch, f16):
         if batch == 1:  # one launch in all: the A . x of both adapters inside the stacked launch
             assert c1["lora_a"] == c0["lora_a"] and c1["gemv_multi"] == c0["gemv_multi"] + 1
             assert c1["lora_t_fallback"] == c0["lora_t_fallback"], "the factors were handed over, not recomputed"
-        elif batch <= 8:  # every adapter's A . X in one launch, then one launch over the stacked rows
-            assert c1["lora_a"] == c0["lora_a"] + 1 and c1["gemv_multi"] == c0["gemv_multi"] + 1
+        elif batch <= 8:  # one launch over the stacked rows, every adapter's A . X in producer workgroups of it
+            assert c1["lora_a"] == c0["lora_a"] and c1["gemv_multi"] == c0["gemv_multi"] + 1
+            assert c1["lora_t_fallback"] <= c0["lora_t_fallback"] + 16
         else:             # projection by projection through the few-token GEMM, which computes A . X itself (ranks <= 16)
             assert c1["lora_a"] == c0["lora_a"] and c1["gemv_multi"] == c0["gemv_multi"]
         for w, q, n, y, nm in zip(ws, qs, shapes, ys, names):

@@ -1058,9 +1058,76 @@ def test_lora_one_token_a_inside_the_launch(mode):
         b2.close()
 
 
-def test_lora_one_token_graph_replays(be):
-    # the launch that computes A.x itself keeps two counters in device memory; a captured launch
-    # must leave them ready for its own replay, with the program's eager work in between
+@pytest.mark.parametrize("mode", ["wait", "0", "off"])
+def test_lora_two_to_eight_rows_a_inside_the_launch(mode):
+    """2..8 rows on the integer matrix-core kernel: `rank` producer workgroups of the launch compute A.x on CUs the
+    matrix leaves idle (tiles + rank <= CUs), the others pick the values up after their staging barrier.  Same three
+    modes as the one-token form; with "0" every value is computed by the wave that needs it, in the producers'
+    order of summation, so "wait" and "0" agree to the bit."""
+    import torch
+    old = os.environ.get("LQ4_LORA_SPIN_LIMIT")
+    os.environ["LQ4_LORA_SPIN_LIMIT"] = mode if mode != "wait" else "512"
+    try:
+        b2 = backend.HipQ4Backend(0)
+    finally:
+        if old is None:
+            os.environ.pop("LQ4_LORA_SPIN_LIMIT", None)
+        else:
+            os.environ["LQ4_LORA_SPIN_LIMIT"] = old
+    ref_be = backend.HipQ4Backend(0)  # (default mode: the bits "0" must reproduce)
+    try:
+        # n, k, rank, dtype, batch: f16 factors in eights (vector epilogue), f32 and odd ranks (scalar epilogue), wide
+        # digits (<= 4 rows) and two digits, tiles + rank just within 256 CUs, and one shape beyond (4000 rows = 250
+        # tiles + 16 > 256: the separate launch)
+        cases = [(2048, 2048, 16, np.float16, 8), (512, 2048, 16, np.float16, 3), (2048, 2048, 64, np.float32, 5),
+                 (304, 512, 3, np.float16, 4), (1040, 1024, 40, np.float16, 8), (3072, 2048, 64, np.float16, 4),
+                 (4000, 2048, 16, np.float16, 4)]
+        for n, k, rank, dt, batch in cases:
+            print(f"lora rows mode={mode} n={n} k={k} rank={rank} {np.dtype(dt).name} batch={batch}", flush=True)
+            wq = synth.q4_weight(n, k, seed=2, tag="lora_rows")
+            a, b = synth.lora_pair(rank, k, n, seed=2, tag="lora_rows", std=0.05, dtype=dt)
+            x = synth.activations(batch, k, seed=30)
+            ref = _lora_ref(x, wq, n, k, a, b, 2.0)
+            base = oracle.gemm_f32(x, wq, n, k)
+            got = {}
+            for which, bk in (("this", b2), ("default", ref_be)):
+                qw = bk.upload_q4_blocks(wq)
+                bk.load_lora_adapter([backend.LoraLayerData(0, {"p": (a, b)})], scale=2.0)
+                c0 = bk.path_counters()
+                try:
+                    y = torch.full((batch, n), float("nan"), dtype=torch.float32, device="cuda")
+                    for call in range(2):  # twice: the second launch must not take the first one's words for its own
+                        bk.gemv_batch(dev(x if call else x[::-1].copy()), qw, y, batch, n, k, layer_idx=0, module="p")
+                    bk.synchronize()
+                finally:
+                    c1 = bk.path_counters()
+                    bk.unload_lora_adapter()
+                got[which] = host(y)
+                if which == "this":
+                    in_launch = mode != "off" and (n + 15) // 16 + rank <= 256
+                    assert c1["lora_a"] - c0["lora_a"] == (0 if in_launch else 2), "which path computed A.x"
+                    fb = c1["lora_t_fallback"] - c0["lora_t_fallback"]
+                    print(f"  values computed by the waves that missed them: {fb}", flush=True)
+                    if mode == "wait":
+                        assert fb <= 64
+                    elif mode == "0" and in_launch:
+                        assert fb > 0
+            e = rel_err(got["this"], ref)
+            e_delta = rel_err(got["this"] - base, ref - base)
+            print(f"  rel err {e:.2e}, delta rel err {e_delta:.2e}", flush=True)
+            assert e <= REL_TOL and e_delta <= 2e-3
+            if mode != "off":
+                assert np.array_equal(got["this"], got["default"]), "same bits whichever way a value was obtained"
+    finally:
+        b2.close()
+        ref_be.close()
+
+
+@pytest.mark.parametrize("rows", [1, 8])
+def test_lora_one_token_graph_replays(be, rows):
+    # the launch that computes A.x itself (one row: the batch-1 kernel; eight: the integer matrix-core kernel) hands
+    # the values over through words that carry the launch's tag; a captured launch must find its own replay's words,
+    # with the program's eager work in between
     import torch
     n, k = synth.LORA_2B["q"]
     wq = synth.q4_weight(n, k, seed=2, tag="lora_graph")
@@ -1068,26 +1135,26 @@ def test_lora_one_token_graph_replays(be):
     qw = be.upload_q4_blocks(wq)
     be.load_lora_adapter([backend.LoraLayerData(0, {"p": (a, b)})], scale=2.0)
     try:
-        xd = torch.zeros((1, k), dtype=torch.float32, device="cuda")
-        y = torch.empty((1, n), dtype=torch.float32, device="cuda")
+        xd = torch.zeros((rows, k), dtype=torch.float32, device="cuda")
+        y = torch.empty((rows, n), dtype=torch.float32, device="cuda")
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
-            be.gemv_batch(xd, qw, y, 1, n, k, layer_idx=0, module="p")  # warm-up outside the capture
+            be.gemv_batch(xd, qw, y, rows, n, k, layer_idx=0, module="p")  # warm-up outside the capture
         torch.cuda.current_stream().wait_stream(side)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            be.gemv_batch(xd, qw, y, 1, n, k, layer_idx=0, module="p")
+            be.gemv_batch(xd, qw, y, rows, n, k, layer_idx=0, module="p")
         for replay in range(4):
             print(f"lora graph replay {replay}", flush=True)
-            x = synth.activations(1, k, seed=20 + replay)
+            x = synth.activations(rows, k, seed=20 + replay)
             xd.copy_(dev(x))
             graph.replay()
             torch.cuda.synchronize()
             got = host(y)
             # eager call between the replays, same operands
             y2 = torch.empty_like(y)
-            be.gemv_batch(xd, qw, y2, 1, n, k, layer_idx=0, module="p")
+            be.gemv_batch(xd, qw, y2, rows, n, k, layer_idx=0, module="p")
             assert np.array_equal(got, host(y2))
             assert rel_err(got, _lora_ref(x, wq, n, k, a, b, 2.0)) <= REL_TOL
     finally:

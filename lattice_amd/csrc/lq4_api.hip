@@ -421,22 +421,24 @@ static void plain_gemv_one_token(lq4_ctx* ctx, const uint8_t* wp, uint32_t n, ui
     ctx->counters.gemv++;
 }
 
+// 2..8 rows on the integer matrix-core kernel: three to eight rows of a matrix of up to 4096 x 2048 (or, for the
+// tests, whatever it can hold).
+static bool gemv_takes_i8(const lq4_ctx* ctx, uint32_t n, uint32_t k, uint32_t batch) {
+    return batch >= 2 && batch <= 8 && ctx->gemv_i8 && (ctx->gemv_i8 == 2 || (batch >= 3 && k <= 2048 && n <= 4096)) &&
+           gemv_i8_serves(n, k, batch, ctx->cu_count);
+}
+
 // Above four activation rows the few-token matrix-core kernel (operands packed once, eight K
 // slices per workgroup) overtakes the 4x4x4 GEMV kernel: always from nine rows; from five for
 // mid-sized matrices only (measured: behind for 512 x 2048, where its two launches dominate,
-// and for 12288 x 2048, where the GEMV kernel's grid already fills the chip).
-static bool gemv_takes_few_token_gemm(uint32_t n, uint32_t k, uint32_t batch) {
+// and for 12288 x 2048, where the GEMV kernel's grid already fills the chip), and not where the integer
+// matrix-core kernel serves (3072 x 2048 at 5..8 rows 5.8-5.9 us here, 5.4-5.5 there; 4096 x 2048 6.2 / 5.5).
+static bool gemv_takes_few_token_gemm(const lq4_ctx* ctx, uint32_t n, uint32_t k, uint32_t batch) {
     const uint64_t weights = static_cast<uint64_t>(n) * k;
     // (not for up to 2048 rows while the GEMV kernel can stage the activations: its eight-wave
     // workgroups then win, 2048 x 6144 at 5..8 rows 9.5 -> 7.2..8.2 us)
     const bool narrow = n <= 2048 && gemv_mfma_lds_bytes(k, batch < 8 ? batch : 8) <= 150 * 1024;
-    return batch >= 9 || (batch >= 5 && n < 8192 && !narrow && weights >= 6000000);
-}
-
-// 2..8 rows on the integer matrix-core kernel (after the few-token GEMM has had its pick).
-static bool gemv_takes_i8(const lq4_ctx* ctx, uint32_t n, uint32_t k, uint32_t batch) {
-    return !gemv_takes_few_token_gemm(n, k, batch) && batch >= 2 && batch <= 8 && ctx->gemv_i8 &&
-           (ctx->gemv_i8 == 2 || (batch >= 3 && k <= 2048 && n <= 4096)) && gemv_i8_serves(n, k, batch, ctx->cu_count);
+    return batch >= 9 || (batch >= 5 && n < 8192 && !narrow && weights >= 6000000 && !gemv_takes_i8(ctx, n, k, batch));
 }
 
 // The routing of lq4_gemv once the LoRA factor t (if any) is in ep, or ep.a says that the kernel which serves the
@@ -446,7 +448,7 @@ static bool gemv_takes_i8(const lq4_ctx* ctx, uint32_t n, uint32_t k, uint32_t b
 static int gemv_dispatch(lq4_ctx* ctx, const uint8_t* wp, uint32_t n, uint32_t k, const float* x_dev, uint32_t batch,
                          float* y_dev, const LoraEpilogue& ep, hipStream_t s, bool* x_packed = nullptr) {
     int rc;
-    if (gemv_takes_few_token_gemm(n, k, batch)) {
+    if (gemv_takes_few_token_gemm(ctx, n, k, batch)) {
         rc = ensure_scratch(ctx, gemm_skinny_scratch_bytes(k, batch), s);
         if (rc) return rc;
         launch_gemm_skinny(wp, n, k, x_dev, 0, batch, y_dev, ep, ctx->moe_scratch, s, 0, !(x_packed && *x_packed));
@@ -498,7 +500,7 @@ int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
         ep.slots = reinterpret_cast<unsigned long long*>(ctx->lora_sync + 64);
         ep.sync = ctx->lora_sync;
         ep.spin_limit = ctx->lora_spin_limit;
-    } else if (ep.rank && batch > 1 && gemv_takes_few_token_gemm(n, k, batch) && gemm_skinny_computes_t(ep.rank, batch)) {
+    } else if (ep.rank && batch > 1 && gemv_takes_few_token_gemm(ctx, n, k, batch) && gemm_skinny_computes_t(ep.rank, batch)) {
         ep.a = lora->a_packed;  // the few-token GEMM computes A.x for its token tile itself
     } else if (ep.rank && ctx->lora_in_kernel && gemv_takes_i8(ctx, n, k, batch) &&
                gemv_i8_lora_in_launch(n, k, batch, ep.rank, ctx->cu_count)) {
@@ -617,7 +619,7 @@ int lq4_gemv_multi(lq4_ctx* ctx, const lq4_projection* proj, uint32_t count, uin
         // projection by projection: those that go to the few-token GEMM get their A . x there
         for (uint32_t i = 0, v = 0; i < count; ++i) {
             if (proj[i].n == 0) continue;
-            if (ep[i].rank && gemv_takes_few_token_gemm(proj[i].n, k, batch) && gemm_skinny_computes_t(ep[i].rank, batch)) {
+            if (ep[i].rank && gemv_takes_few_token_gemm(ctx, proj[i].n, k, batch) && gemm_skinny_computes_t(ep[i].rank, batch)) {
                 ep[i].a = proj[i].lora->a_packed;
                 av.rank[v] = 0;
                 --with_lora;

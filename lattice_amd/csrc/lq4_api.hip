@@ -500,7 +500,7 @@ int lq4_gemv(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
         ep.slots = reinterpret_cast<unsigned long long*>(ctx->lora_sync + 64);
         ep.sync = ctx->lora_sync;
         ep.spin_limit = ctx->lora_spin_limit;
-    } else if (ep.rank && batch > 1 && gemv_takes_few_token_gemm(ctx, n, k, batch) && gemm_skinny_computes_t(ep.rank, batch)) {
+    } else if (ep.rank && batch > 1 && gemv_takes_few_token_gemm(ctx, n, k, batch) && gemm_skinny_computes_t(ep.rank, batch, n)) {
         ep.a = lora->a_packed;  // the few-token GEMM computes A.x for its token tile itself
     } else if (ep.rank && ctx->lora_in_kernel && gemv_takes_i8(ctx, n, k, batch) &&
                gemv_i8_lora_in_launch(n, k, batch, ep.rank, ctx->cu_count)) {
@@ -582,7 +582,7 @@ int lq4_gemv_multi(lq4_ctx* ctx, const lq4_projection* proj, uint32_t count, uin
             if (p.n == 0) continue;
             const bool few = gemm_takes_few_token_kernel(p.n, k, batch, 0, ctx->gemm_kernel);
             LoraEpilogue e = ep[i];
-            if (e.rank && few && gemm_skinny_computes_t(e.rank, batch)) {
+            if (e.rank && few && gemm_skinny_computes_t(e.rank, batch, p.n)) {
                 e.a = p.lora->a_packed;
             } else if (e.rank) {
                 e.t = ctx->lora_t;  // one after the other on this stream
@@ -619,7 +619,7 @@ int lq4_gemv_multi(lq4_ctx* ctx, const lq4_projection* proj, uint32_t count, uin
         // projection by projection: those that go to the few-token GEMM get their A . x there
         for (uint32_t i = 0, v = 0; i < count; ++i) {
             if (proj[i].n == 0) continue;
-            if (ep[i].rank && gemv_takes_few_token_gemm(ctx, proj[i].n, k, batch) && gemm_skinny_computes_t(ep[i].rank, batch)) {
+            if (ep[i].rank && gemv_takes_few_token_gemm(ctx, proj[i].n, k, batch) && gemm_skinny_computes_t(ep[i].rank, batch, proj[i].n)) {
                 ep[i].a = proj[i].lora->a_packed;
                 av.rank[v] = 0;
                 --with_lora;
@@ -790,7 +790,7 @@ int lq4_gemm(lq4_ctx* ctx, const lq4_weight* w, uint64_t w_extra_offset, uint32_
         rc = enter_shared_state(ctx, s);
         if (rc) return rc;
     }
-    if (ep.rank && gemm_takes_few_token_kernel(n, k, m, x_dtype == LQ4_F16, ctx->gemm_kernel) && gemm_skinny_computes_t(ep.rank, m)) {
+    if (ep.rank && gemm_takes_few_token_kernel(n, k, m, x_dtype == LQ4_F16, ctx->gemm_kernel) && gemm_skinny_computes_t(ep.rank, m, n)) {
         ep.a = lora->a_packed;  // the few-token GEMM computes A.X for its token tile itself
     } else if (ep.rank) {
         launch_lora_a(lora->a, lora->is_f16, lora->rank, k, x_dev, x_dtype == LQ4_F16, k, m, ctx->lora_t, s);

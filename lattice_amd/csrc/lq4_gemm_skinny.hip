@@ -527,9 +527,15 @@ void launch_rt(const uint8_t* w, uint32_t n, uint32_t k, const uint4* xp, uint32
 
 // The few-token kernel computes t = A . X itself (LoraEpilogue::a set, no launch for t) for Q4, ranks up to 16 and
 // up to 64 tokens (q and v of the 2B model, rank 16, 64 tokens: 13.6 us with a launch for t -> 8.3 / 7.7, against
-// 8.0 / 7.6 without an adapter; at 128 tokens its tiles of 32 tokens are four to a row tile and it is behind).
+// 8.0 / 7.6 without an adapter).  From 65 tokens on its tiles of 32 tokens are three or four to a row tile: taken
+// while those workgroups still find a CU each (512 x 2048 at 128 tokens 10.2 -> 8.0 us; 2048 x 2048, 512 workgroups,
+// 12.8 -> 13.0 and left with the launch for t).
 bool gemm_skinny_packs_lora_a(uint32_t rank) { return rank != 0 && rank <= 16; }
-bool gemm_skinny_computes_t(uint32_t rank, uint32_t m) { return gemm_skinny_packs_lora_a(rank) && m <= kTokens; }
+bool gemm_skinny_computes_t(uint32_t rank, uint32_t m, uint32_t n) {
+    if (!gemm_skinny_packs_lora_a(rank)) return false;
+    const uint32_t groups = (m + 15) / 16;
+    return m <= kTokens || ((n + 15) / 16) * ((groups + 1) / 2) <= 256;
+}
 
 // A [rank <= 16, K] (f32 or f16, host memory) as the kernel's matrix-core operand, f16: for K step s (128 wide) and
 // instruction j the 64 lanes' 16-byte operands are contiguous; lane (r = lane % 16, g = lane / 16) holds row r,

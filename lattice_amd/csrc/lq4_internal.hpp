@@ -245,7 +245,7 @@ bool gemm_skinny_wants(uint32_t n, uint32_t k, uint32_t m);
 size_t gemm_skinny_scratch_bytes(uint32_t k, uint32_t m);
 // For Q4 and a LoRA rank this accepts, the kernel computes t = A . X itself when LoraEpilogue::a points to A as
 // packed (on the host, once) by gemm_skinny_pack_lora_a; t is then not read and no launch for it has to precede.
-bool gemm_skinny_computes_t(uint32_t rank, uint32_t m);
+bool gemm_skinny_computes_t(uint32_t rank, uint32_t m, uint32_t n);
 bool gemm_skinny_packs_lora_a(uint32_t rank);  // an adapter of this rank gets a packed copy of A at upload
 size_t gemm_skinny_packed_lora_a_bytes(uint32_t k);
 void gemm_skinny_pack_lora_a(const void* a_host, int a_is_f16, uint32_t rank, uint32_t k, void* out_host);

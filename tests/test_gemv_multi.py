@@ -219,8 +219,9 @@ def test_multi_above_sixteen_rows_goes_through_the_gemm_routing(be, batch):
         be.synchronize()
         c1 = be.path_counters()
         assert c1["gemm"] == c0["gemm"] + 4 and c1["gemv_multi"] == c0["gemv_multi"]
-        # rank 24 always has its own A . X launch; ranks 16 and 8 only above 64 rows
-        assert c1["lora_a"] == c0["lora_a"] + (1 if batch <= 64 else 3)
+        # rank 24 always has its own A . X launch; above 64 rows also the 2048-row projection (its 32-token tiles
+        # would be 512 workgroups), while the 512-row one keeps computing A . X in the kernel
+        assert c1["lora_a"] == c0["lora_a"] + (1 if batch <= 64 else 2)
         for w, q, n, y, nm in zip(ws, qs, shapes, ys, names):
             base = oracle.gemm_f32(x, w, n, k)
             want = base

@@ -316,9 +316,10 @@ def main():
         # streaming rate.
         shapes = {}
         # "lm_head" is the reference's largest single GEMV per token (vocabulary 248,320 x hidden 2048,
-        # 318 MB of Q4 blocks): one launch big enough to show the kernel's streaming rate.
+        # 318 MB of Q4 blocks): one launch big enough to show the kernel's streaming rate; "27b_lm_head" the same
+        # projection at the 27B-shaped hidden size of config 2 (151,936 x 5120, 486 MB).
         extra_shapes = [("cfg0", 4096, 1024), ("27b_up", 17408, 5120), ("27b_down", 5120, 17408),
-                        ("lm_head", 248320, 2048)]
+                        ("lm_head", 248320, 2048), ("27b_lm_head", 151936, 5120)]
         for name, n, k in LAYER + extra_shapes:
             wbytes = n * (k // 32) * 20
             pool = [l[name] for l in layers] if name in dict((a, 1) for a, _, _ in LAYER) else \

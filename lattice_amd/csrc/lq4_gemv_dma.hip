@@ -23,10 +23,9 @@
 // the old contents, and it may hand the original register to another value that the arriving data then destroys;
 // both happened here, the second as a memory fault through a clobbered address offset).
 //
-// Work split, rows of more than one slab (gemv_q4_dma).  A workgroup (one per CU) owns a run of consecutive rows,
-// i.e. a run of slots that is also one run of
-// memory, and its sixteen waves cut that run into sixteen equal pieces to within one slot, wherever the row
-// boundaries fall: 5120 rows of nine slots are twenty rows a CU, which dealt out as whole rows would leave four
+// Work split, rows of more than three slabs (gemv_q4_dma).  A workgroup (one per CU) owns a run of consecutive
+// rows, i.e. a run of slots that is also one run of memory, and its sixteen waves cut that run into sixteen equal
+// pieces to within one slot, wherever the row boundaries fall: 5120 rows of nine slots are twenty rows a CU, which dealt out as whole rows would leave four
 // waves with eighteen slots and twelve with nine.  A wave's slots are again one run of memory, so the address of
 // the next request is a running pointer.  A row that starts in one wave and ends in a later one is finished by the
 // wave it starts in: every wave leaves the sum of the row that was already under way at its first slot (at most
@@ -37,28 +36,26 @@
 // dozen branches per slot and was 10-15 % slower than the lane-owns-block kernel: a CU issues one scalar
 // instruction per cycle for all its waves.)  The block of slot s + 1 is read out of LDS before the arithmetic of
 // slot s, so that read's latency hides behind ~50 vector instructions, and the refill of slot s is requested after
-// them, when its words have long been in registers.  Rows of up to three slabs keep the lane's blocks of x in
-// registers for the whole launch (104 bytes a lane and slab: read from LDS for every slot they cost six times the
-// LDS traffic of the weights themselves); the slab at an unrolled position then has to be a constant, so the loop
-// exists once per slab a wave's piece can start at.  Longer rows re-read their blocks from LDS slot by slot.
+// them, when its words have long been in registers.  The lane's block of x is read from LDS slot by slot (104 bytes
+// a lane: six times the LDS traffic of the weights themselves); rows of up to three slabs, which can keep those
+// blocks in registers for the whole launch, have the kernel described at the end.
 //
 // One workgroup of sixteen waves per CU: the activations are staged once per CU, by as many waves as the vector
 // has 512-element pieces (the others skip the staging code altogether, which on short rows is most of what a
 // wave of the lane-owns-block kernel executes).
 //
-// Rows of at most one slab (gemv_q4_dma_rows: K <= 2048, the lm_head) are slots by themselves, so there the waves
-// of a workgroup take rows as they come free instead of owning equal pieces: time stamps of the equal-pieces form
-// on 248320 x 2048 showed a workgroup's first wave done after 38 us and its last after 48.6, the last fifth of
-// the rows streaming from ever fewer waves.  Taking rows from a counter in LDS brings the waves' ends within one
-// slot of each other (45.4 / 46.8 us) and the launch from 52.6 to 51.0 us.  The same was tried for longer rows (a
-// slot = one slab of one row, the slots' sums added per row afterwards) and is not kept: the slab a wave meets is
-// then known only at run time, so the blocks of x come from LDS for every slot and every slot ends in its own
-// cross-lane sum, which cost more than the even ends returned (151936 x 5120 79.5 -> 88.2 us, 32768 x 4096
-// 16.6 -> 17.2, 5120 x 17408 13.4 -> 12.9).  What remains uneven is between workgroups (ends 41..52 us in one
-// launch, 44..49 in the next, whole XCDs ahead or behind).
+// Rows of one to three slabs (gemv_q4_dma_rows: K <= 6144, the lm_heads) are short enough to be handed out whole,
+// so there the waves of a workgroup take rows as they come free instead of owning equal pieces: time stamps of the
+// equal-pieces form on 248320 x 2048 showed a workgroup's first wave done after 38 us and its last after 48.6, the
+// last fifth of the rows streaming from ever fewer waves.  Taking rows from a counter in LDS brings the waves' ends
+// within one slot of each other (45.4 / 46.8 us): 248320 x 2048 52.6 -> 51.0 us, 151936 x 5120 80.0 -> 76.2,
+// 65536 x 3072 24.7 -> 22.6, 17408 x 5120 13.6 -> 12.3.  A row keeps its ring positions' order (position i holds slab
+// i % SLABS), so the blocks of x stay in registers and a row still ends in one cross-lane sum.  Handing out single
+// slots of longer rows was tried first and is not kept: the slab a wave meets is then known only at run time, so the
+// blocks of x come from LDS for every slot and every slot ends in its own cross-lane sum, which cost more than the
+// even ends returned (151936 x 5120 79.5 -> 88.2 us, 32768 x 4096 16.6 -> 17.2, 5120 x 17408 13.4 -> 12.9).  What
+// remains uneven is between workgroups (ends 41..52 us in one launch, 44..49 in the next, whole XCDs ahead or behind).
 #include "lq4_b1_dev.hpp"
-
-#include <type_traits>
 
 namespace lq4 {
 
@@ -164,20 +161,19 @@ __device__ __forceinline__ void stage_x(lds_u32* xs, uint32_t k, uint32_t wave, 
     barrier_lds();
 }
 
-// XR: 8-activation units a thread stages (K <= 8 * 1024 * XR).  D: slots in a wave's ring.
-// SLABS: 2 or 3 = rows of that many slabs (the last may be short), the lane's blocks of x stay in registers (D is a
-// multiple of SLABS); 0 = any longer row, x from LDS.  Rows of one slab have a kernel of their own below.
-template <int XR, int D, int SLABS>
+// Rows of any length (launched for more than three slabs; up to three have the kernel below): the lane's block of x
+// comes from LDS for every slot.  XR: 8-activation units a thread stages (K <= 8 * 1024 * XR).  D: slots in a wave's
+// ring.
+template <int XR, int D>
 __global__ __launch_bounds__(kWaves * 64) void gemv_q4_dma(const uint8_t* __restrict__ w_, uint32_t n, uint32_t k,
                                                             const float* __restrict__ x_, float* __restrict__ y) {
     static_assert(D >= 3, "one slot in registers, one landed, at least one on its way");
-    static_assert(SLABS != 1 && (SLABS == 0 || D % SLABS == 0), "the slab at an unrolled position must not depend on the round");
     extern __shared__ __attribute__((aligned(16))) uint32_t lds_raw[];
     lds_u32* const xs = (lds_u32*)lds_raw;
     const int tid = threadIdx.x, lane = tid & 63;
     const uint32_t nb = k / kBlockWeights;
     const uint32_t row_bytes = nb * kBlockBytes;
-    const uint32_t slabs = SLABS ? SLABS : (nb + 63) / 64;
+    const uint32_t slabs = (nb + 63) / 64;
     const uint32_t last_blocks = nb - (slabs - 1) * 64;  // blocks of a row's last slab
     const uint32_t last_bytes = last_blocks * kBlockBytes;
     const uint32_t wave = uniform(tid >> 6);
@@ -255,15 +251,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_dma(const uint8_t* __rest
     }
 
     // ---- the arithmetic: round after round over the ring ----
-    constexpr int NX = SLABS ? SLABS : 1;
-    XBlock xb[NX];
-    if (SLABS) {
-#pragma unroll
-        for (int sl = 0; sl < NX; ++sl) {
-            const uint32_t blk = sl * 64 + lane;
-            load_xblock(xs, blk < nb ? blk : nb - 1, xb[sl]);
-        }
-    }
+    XBlock xb;
     const lds_u32* const my_block = ring_ptr + 5 * lane;  // the lane's block in position 0: byte 20 l
     auto read_block = [&](int pos, Q4BlockRaw& wb) {
         const lds_u32* const slot = my_block + pos * (kSlotBytes / 4);
@@ -273,67 +261,51 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_dma(const uint8_t* __rest
     float acc = 0.0f;
     uint32_t left = total, cs_slab = slab0, row = wg_first + row0;
     bool in_head = slab0 != 0;  // the row under way at the first slot started in an earlier wave
-    // S0: the slab of the piece's first slot when rows have SLABS slabs (a constant inside each copy of the loop)
-    auto run = [&](auto s0_const) {
-        constexpr int S0 = decltype(s0_const)::value;
-        Q4BlockRaw cur, nxt;
-        if (left) {
-            if (total >= static_cast<uint32_t>(D)) wait_vm<2 * (D - 1)>();
-            else wait_vm<0>();
-            read_block(0, cur);
-        }
-        while (left) {
+    Q4BlockRaw cur, nxt;
+    if (left) {
+        if (total >= static_cast<uint32_t>(D)) wait_vm<2 * (D - 1)>();
+        else wait_vm<0>();
+        read_block(0, cur);
+    }
+    while (left) {
 #pragma unroll
-            for (int i = 0; i < D; ++i) {
-                if (left == 0) break;  // uniform
-                // the slot behind this one out of LDS now: its read hides behind this slot's arithmetic
-                if (left > 1) {
-                    if (to_request) wait_vm<2 * (D - 2)>();  // the ring is full behind this slot
-                    else wait_vm<0>();
-                    read_block((i + 1) % D, nxt);
-                }
-                const int slab_c = SLABS ? (S0 + i) % NX : 0;  // a constant once the loop is unrolled
-                bool live = true;
-                bool last_slab;
-                if constexpr (SLABS != 0) {
-                    last_slab = slab_c == SLABS - 1;
-                    if (last_slab) live = static_cast<uint32_t>(lane) < last_blocks;
-                } else {
-                    last_slab = cs_slab + 1 == slabs;
-                    const uint32_t blk_raw = cs_slab * 64 + lane;
-                    live = blk_raw < nb;
-                    load_xblock(xs, live ? blk_raw : nb - 1, xb[0]);
-                    cs_slab = last_slab ? 0 : cs_slab + 1;
-                }
-                // a lane past the end of the row has read what the slot held before: scale and bias of zero,
-                // whatever bits they were (a stale bias may be an infinity, and zero times that is not zero)
-                if (short_last && last_slab) cur.sb = live ? cur.sb : 0u;
-                acc = block_fma(cur, xb[slab_c], live, acc);
-                // the slot's words went into registers a slot ago: its place in the ring can be filled again
-                if (to_request) {
-                    request_next(i);
-                    --to_request;
-                }
-                if (last_slab) {
-                    const float v = segment_sum<64>(acc);
-                    acc = 0.0f;
-                    if (in_head) {  // uniform: the tail of a row that an earlier wave finishes
-                        if (lane == 63) part[wave] = v;
-                        in_head = false;
-                    } else if (lane == 63) {
-                        y[row] = v;
-                    }
-                    ++row;
-                }
-                cur = nxt;
-                --left;
+        for (int i = 0; i < D; ++i) {
+            if (left == 0) break;  // uniform
+            // the slot behind this one out of LDS now: its read hides behind this slot's arithmetic
+            if (left > 1) {
+                if (to_request) wait_vm<2 * (D - 2)>();  // the ring is full behind this slot
+                else wait_vm<0>();
+                read_block((i + 1) % D, nxt);
             }
+            const bool last_slab = cs_slab + 1 == slabs;
+            const uint32_t blk_raw = cs_slab * 64 + lane;
+            const bool live = blk_raw < nb;
+            load_xblock(xs, live ? blk_raw : nb - 1, xb);
+            cs_slab = last_slab ? 0 : cs_slab + 1;
+            // a lane past the end of the row has read what the slot held before: scale and bias of zero,
+            // whatever bits they were (a stale bias may be an infinity, and zero times that is not zero)
+            if (short_last && last_slab) cur.sb = live ? cur.sb : 0u;
+            acc = block_fma(cur, xb, live, acc);
+            // the slot's words went into registers a slot ago: its place in the ring can be filled again
+            if (to_request) {
+                request_next(i);
+                --to_request;
+            }
+            if (last_slab) {
+                const float v = segment_sum<64>(acc);
+                acc = 0.0f;
+                if (in_head) {  // uniform: the tail of a row that an earlier wave finishes
+                    if (lane == 63) part[wave] = v;
+                    in_head = false;
+                } else if (lane == 63) {
+                    y[row] = v;
+                }
+                ++row;
+            }
+            cur = nxt;
+            --left;
         }
-        if (SLABS) cs_slab = (slab0 + total) % NX;  // the slab the next slot would have had
-    };
-    if (SLABS == 0 || slab0 == 0) run(std::integral_constant<int, 0>{});
-    else if (slab0 == 1) run(std::integral_constant<int, 1>{});
-    else run(std::integral_constant<int, SLABS == 3 ? 2 : 0>{});
+    }
     wait_vm<0>();  // nothing of this wave is on its way when it ends
     // ---- rows that straddle waves ----
     const bool open_row = total != 0 && cs_slab != 0;  // the last slot did not end its row
@@ -355,20 +327,25 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_dma(const uint8_t* __rest
     }
 }
 
-// Rows of at most one slab (K <= 2048): a slot is a row, the lane's block of x stays in registers, and a slot's sum
-// is its row's result.  The waves of a workgroup do not advance at one pace (with equal shares the first is done
+// Rows of one to three slabs (K <= 6144): the lane's blocks of x stay in registers and a wave works on whole rows.
+// The waves of a workgroup do not advance at one pace (with equal shares the first is done
 // when the last has a fifth of its rows to go, and what is left then streams from fewer waves), so only a wave's
-// first D slots are fixed: slot 16 i + wave goes into position i, the sixteen waves' requests forming one run of
-// memory, and every later request takes the next row nobody has asked for yet, from a counter in LDS.
-template <int D>
+// first D / SLABS rows are fixed: row 16 j + wave goes into ring positions SLABS j .., the sixteen waves' requests
+// forming one run of memory, and every later row is the next one nobody has asked for yet, from a counter in LDS:
+// taken when the first slab of the row it replaces has been consumed, its slabs requested one by one as their
+// positions come free.  Position i of the ring always holds slab i % SLABS (D is a multiple of SLABS), so every
+// register index and LDS offset of the unrolled loop is a constant.
+template <int D, int SLABS>
 __global__ __launch_bounds__(kWaves * 64) void gemv_q4_dma_rows(const uint8_t* __restrict__ w_, uint32_t n, uint32_t k,
                                                                  const float* __restrict__ x_, float* __restrict__ y) {
-    static_assert(D >= 3, "one slot in registers, one landed, at least one on its way");
+    static_assert(D >= 3 && SLABS >= 1 && SLABS <= 3 && D % SLABS == 0, "whole rows in the ring");
     extern __shared__ __attribute__((aligned(16))) uint32_t lds_raw[];
     lds_u32* const xs = (lds_u32*)lds_raw;
     const int tid = threadIdx.x, lane = tid & 63;
-    const uint32_t nb = k / kBlockWeights;  // at most 64
+    const uint32_t nb = k / kBlockWeights;  // at most 64 SLABS, more than 64 (SLABS - 1)
     const uint32_t row_bytes = nb * kBlockBytes;
+    const uint32_t last_blocks = nb - (SLABS - 1) * 64;  // blocks of a row's last slab
+    const uint32_t last_bytes = last_blocks * kBlockBytes;
     const uint32_t wave = uniform(tid >> 6);
     const LQ4_GLOBAL uint8_t* const w = as_global(w_);
     // LDS: the staged activations | the row counter | the waves' rings
@@ -383,20 +360,22 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_dma_rows(const uint8_t* _
     const uint32_t share = n / gridDim.x, extra = n - share * gridDim.x;
     const uint32_t wg_rows = share + (blockIdx.x < extra ? 1u : 0u);
     const uint32_t wg_first = blockIdx.x * share + (blockIdx.x < extra ? blockIdx.x : extra);
-    // a short row: 20 * blocks bytes as whole 16-byte pieces, then the dwords behind them (fewer than four); lane 0
-    // always takes part in the second load so that it is a load instruction on every path (the waits count them)
-    const uint32_t n16 = row_bytes / 16 < 64 ? row_bytes / 16 : 64;
-    const uint32_t rest = (row_bytes - n16 * 16) / 4;
+    // a short last slab: 20 * blocks bytes as whole 16-byte pieces, then the dwords behind them (fewer than four, or
+    // what is left past 1024 bytes); lane 0 always takes part in the second load so that it is a load instruction on
+    // every path (the waits count them)
+    const uint32_t n16 = last_bytes / 16 < 64 ? last_bytes / 16 : 64;
+    const uint32_t rest = (last_bytes - n16 * 16) / 4;
     const uint64_t mask16 = __builtin_amdgcn_ballot_w64(static_cast<uint32_t>(lane) < n16);
     const uint64_t mask4 = __builtin_amdgcn_ballot_w64(static_cast<uint32_t>(lane) < (rest ? rest : 1u));
-    const bool short_row = nb != 64;
+    const bool short_last = last_blocks != 64;
     const LQ4_GLOBAL uint8_t* const w_wg = w + static_cast<uint64_t>(wg_first) * row_bytes;
     const uint32_t off16 = lane * 16u, off4 = lane * 4u;
     uint32_t slot_row[D];  // the row in each ring position (scalar registers: the positions are constants)
-    auto request = [&](int pos, uint32_t row) {  // row `row` of the workgroup into ring position `pos`
-        const LQ4_GLOBAL uint8_t* const src = w_wg + static_cast<uint64_t>(row) * row_bytes;
+    auto request = [&](int pos, uint32_t row) {  // slab pos % SLABS of row `row` of the workgroup into ring position `pos`
+        const int slab = pos % SLABS;
+        const LQ4_GLOBAL uint8_t* const src = w_wg + static_cast<uint64_t>(row) * row_bytes + slab * kSlotBytes;
         const uint32_t at = ring_addr + pos * kSlotBytes;
-        if (short_row) {
+        if (short_last && slab == SLABS - 1) {
             dma16_masked(at, src, off16, mask16);
             dma4_masked(at + n16 * 16, src + (rest ? n16 * 16 : 0u), off4, mask4);
         } else {
@@ -410,13 +389,13 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_dma_rows(const uint8_t* _
     uint32_t have = 0;  // occupied ring positions: always consecutive ones
 #pragma unroll
     for (int i = 0; i < E; ++i) {
-        const uint32_t row = i * kWaves + wave;
+        const uint32_t row = (i / SLABS) * kWaves + wave;
         if (row < wg_rows) {  // uniform
             request(i, row);
             ++have;
         }
     }
-    if (tid == 0) *counter = D * kWaves;  // the first row that is nobody's yet
+    if (tid == 0) *counter = (D / SLABS) * kWaves;  // the first row that is nobody's yet
 
     // ---- stage x: the activation loads are older than every weight request ----
     if (have == static_cast<uint32_t>(E)) wait_vm<2 * E>();
@@ -424,20 +403,24 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_dma_rows(const uint8_t* _
     stage_x<1>(xs, k, wave, tid);  // (its barriers publish the counter as well)
 #pragma unroll
     for (int i = E; i < D; ++i) {
-        const uint32_t row = i * kWaves + wave;
+        const uint32_t row = (i / SLABS) * kWaves + wave;
         if (row < wg_rows) {  // uniform
             request(i, row);
             ++have;
         }
     }
-    // a wave that found fewer than D rows finds none behind them either; from the first request the counter turns
-    // down on, a wave asks no more: its occupied positions stay consecutive and the ring drains
+    // a wave that found fewer than D / SLABS rows finds none behind them either; from the first request the counter
+    // turns down on, a wave asks no more: its occupied positions stay consecutive and the ring drains
     bool more = have == static_cast<uint32_t>(D);
 
     // ---- the arithmetic: round after round over the ring ----
-    XBlock xb;
-    load_xblock(xs, static_cast<uint32_t>(lane) < nb ? lane : nb - 1, xb);
-    const bool live = static_cast<uint32_t>(lane) < nb;
+    XBlock xb[SLABS];
+#pragma unroll
+    for (int sl = 0; sl < SLABS; ++sl) {
+        const uint32_t blk = sl * 64 + lane;
+        load_xblock(xs, blk < nb ? blk : nb - 1, xb[sl]);
+    }
+    const bool live_last = static_cast<uint32_t>(lane) < last_blocks;
     const lds_u32* const my_block = ring_ptr + 5 * lane;  // the lane's block in position 0: byte 20 l
     auto read_block = [&](int pos, Q4BlockRaw& wb) {
         const lds_u32* const slot = my_block + pos * (kSlotBytes / 4);
@@ -445,6 +428,8 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_dma_rows(const uint8_t* _
         wb.q[0] = slot[1]; wb.q[1] = slot[2]; wb.q[2] = slot[3]; wb.q[3] = slot[4];
     };
     Q4BlockRaw cur, nxt;
+    float acc = 0.0f;
+    uint32_t next_row = 0;  // the row whose slabs are replacing the row under way (while `more`)
     if (have) {
         if (more) wait_vm<2 * (D - 1)>();
         else wait_vm<0>();
@@ -454,10 +439,13 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_dma_rows(const uint8_t* _
 #pragma unroll
         for (int i = 0; i < D; ++i) {
             if (have == 0) break;  // uniform
-            // the row that will take this position: asked for now, needed after the arithmetic.  (A plain LDS atomic
-            // of one lane; the wave-wide ds_append was tried for it and did not count as its description says.)
+            const int slab = i % SLABS;  // a constant once the loop is unrolled
+            // at a row's first slab: the row that will take this row's positions, asked for now, needed after the
+            // arithmetic.  (A plain LDS atomic of one lane; the wave-wide ds_append was tried for it and did not
+            // count as its description says.)
             uint32_t claim = 0;
-            if (more && lane == 0) claim = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (slab == 0 && more && lane == 0)
+                claim = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             // the slot behind this one out of LDS now: its read hides behind this slot's arithmetic
             if (have > 1) {
                 if (more) wait_vm<2 * (D - 2)>();  // the ring is full behind this slot
@@ -466,21 +454,23 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4_dma_rows(const uint8_t* _
             }
             // a lane past the end of the row has read what the slot held before: scale and bias of zero,
             // whatever bits they were (a stale bias may be an infinity, and zero times that is not zero)
-            if (short_row) cur.sb = live ? cur.sb : 0u;
-            const float v = segment_sum<64>(block_fma(cur, xb, live, 0.0f));
-            if (lane == 63) y[wg_first + slot_row[i]] = v;
+            const bool live = slab == SLABS - 1 ? live_last : true;
+            if (short_last && slab == SLABS - 1) cur.sb = live ? cur.sb : 0u;
+            acc = block_fma(cur, xb[slab], live, acc);
+            if (slab == SLABS - 1) {
+                const float v = segment_sum<64>(acc);
+                acc = 0.0f;
+                if (lane == 63) y[wg_first + slot_row[i]] = v;
+            }
             // the slot's words went into registers a slot ago: its place in the ring can be filled again
             if (more) {
-                const uint32_t row = uniform(claim);
-                if (row < wg_rows) {
-                    request(i, row);
-                } else {
-                    more = false;
-                    --have;
+                if (slab == 0) {
+                    next_row = uniform(claim);
+                    if (next_row >= wg_rows) more = false;
                 }
-            } else {
-                --have;
             }
+            if (more) request(i, next_row);
+            else --have;
             cur = nxt;
         }
     }
@@ -510,21 +500,21 @@ bool plan_dma(uint32_t n, uint32_t k, uint32_t cu_count, DmaPlan* out) {
     return true;
 }
 
-template <int D>
+template <int D, int SLABS>
 void launch_rows(const DmaPlan& p, const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, hipStream_t stream) {
     static LdsCapOnce lds_cap;
-    lds_cap.raise(reinterpret_cast<const void*>(gemv_q4_dma_rows<D>), 160 * 1024);
+    lds_cap.raise(reinterpret_cast<const void*>(gemv_q4_dma_rows<D, SLABS>), 160 * 1024);
     const size_t lds = p.lds < 96 * 1024 ? 96 * 1024 : p.lds;  // one workgroup to a CU
-    hipLaunchKernelGGL((gemv_q4_dma_rows<D>), dim3(p.grid), dim3(kWaves * 64), lds, stream, w, n, k, x, y);
+    hipLaunchKernelGGL((gemv_q4_dma_rows<D, SLABS>), dim3(p.grid), dim3(kWaves * 64), lds, stream, w, n, k, x, y);
 }
 
-template <int XR, int D, int SLABS>
+template <int XR, int D>
 void launch_one(const DmaPlan& p, const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, hipStream_t stream) {
     static LdsCapOnce lds_cap;
-    lds_cap.raise(reinterpret_cast<const void*>(gemv_q4_dma<XR, D, SLABS>), 160 * 1024);
+    lds_cap.raise(reinterpret_cast<const void*>(gemv_q4_dma<XR, D>), 160 * 1024);
     // at least half a CU's LDS, so that the workgroups spread one to a CU
     const size_t lds = p.lds < 96 * 1024 ? 96 * 1024 : p.lds;
-    hipLaunchKernelGGL((gemv_q4_dma<XR, D, SLABS>), dim3(p.grid), dim3(kWaves * 64), lds, stream, w, n, k, x, y);
+    hipLaunchKernelGGL((gemv_q4_dma<XR, D>), dim3(p.grid), dim3(kWaves * 64), lds, stream, w, n, k, x, y);
 }
 
 }  // namespace
@@ -535,26 +525,27 @@ bool gemv_dma_serves(uint32_t n, uint32_t k, uint32_t cu_count) {
 }
 
 // Measured against the lane-owns-block kernel on 256 CUs (us, that kernel -> this one): 32768 x 2048 (42 MB) 10.2 ->
-// 10.35; 65536 x 2048 (84 MB) 17.4 -> 16.3; 248320 x 2048 62.1 -> 51.4; 32768 x 4096 16.7 -> 16.7; 17408 x 5120 (56 MB)
-// 12.6..13.3 -> 13.6; 151936 x 5120 87.8 -> 79.5; 16384 x 8192 17.8 -> 18.0; 8192 x 12288 (63 MB) 14.9 -> 13.0; 4096 x
-// 14336 (37 MB) 10.8 -> 9.4; 5120 x 17408 16.8 -> 13.5; 2048 x 17408 (22 MB) 8.6 -> 9.0.  Behind for every row shorter
-// than one slab (131072 x 1024 18.9 -> 21.7: the other kernel puts two rows side by side in a wave) and for the decode
-// layer's matrices (2..16 MB, 1.0 us behind: its start costs two workgroup barriers of sixteen waves).
+// 10.35; 65536 x 2048 (84 MB) 17.4 -> 16.3; 248320 x 2048 62.1 -> 51.3; 151936 x 5120 87.8 -> 76.2; 32768 x 3072 (63 MB)
+// 14.4 -> 13.4; 17408 x 5120 (56 MB) 12.6 -> 12.3; 24576 x 2560 (39 MB) 12.9 -> 10.6; 12288 x 5120 (39 MB) 10.3 -> 10.0;
+// 16384 x 4096 (42 MB) 9.7 -> 10.1; 8192 x 6144 (31 MB) 8.4 -> 8.5; 16384 x 8192 17.8 -> 18.0; 8192 x 12288 (63 MB) 14.9 ->
+// 13.0; 4096 x 14336 (37 MB) 10.8 -> 9.4; 5120 x 17408 16.8 -> 13.5; 2048 x 17408 (22 MB) 8.6 -> 9.0.  Behind for every
+// row shorter than one slab (131072 x 1024 18.9 -> 21.7: the other kernel puts two rows side by side in a wave) and
+// for the decode layer's matrices (2..16 MB, 1.0 us behind: its start costs two workgroup barriers of sixteen waves).
 bool gemv_dma_pays(uint32_t n, uint32_t k, uint32_t cu_count) {
     if (!gemv_dma_serves(n, k, cu_count) || k < 2048) return false;
     const uint64_t bytes = static_cast<uint64_t>(n) * (k / kBlockWeights) * kBlockBytes;
-    return bytes >= (64ull << 20) || (k >= 10240 && bytes >= (32ull << 20));
+    return bytes >= (64ull << 20) || (k >= 10240 && bytes >= (32ull << 20)) || (k <= 6144 && bytes >= (48ull << 20));
 }
 
 void launch_gemv_dma(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, uint32_t cu_count, hipStream_t stream) {
     DmaPlan p;
     if (!plan_dma(n, k, cu_count, &p)) return;  // the caller asked gemv_dma_serves first
-    if (p.slabs == 1) launch_rows<6>(p, w, n, k, x, y, stream);
-    else if (p.slabs == 2) launch_one<1, 6, 2>(p, w, n, k, x, y, stream);
-    else if (p.slabs == 3) launch_one<1, 6, 3>(p, w, n, k, x, y, stream);
-    else if (p.xr == 1 && p.depth == 6) launch_one<1, 6, 0>(p, w, n, k, x, y, stream);
-    else if (p.xr == 1) launch_one<1, 3, 0>(p, w, n, k, x, y, stream);
-    else launch_one<3, 3, 0>(p, w, n, k, x, y, stream);
+    if (p.slabs == 1) launch_rows<6, 1>(p, w, n, k, x, y, stream);
+    else if (p.slabs == 2) launch_rows<6, 2>(p, w, n, k, x, y, stream);
+    else if (p.slabs == 3) launch_rows<6, 3>(p, w, n, k, x, y, stream);
+    else if (p.xr == 1 && p.depth == 6) launch_one<1, 6>(p, w, n, k, x, y, stream);
+    else if (p.xr == 1) launch_one<1, 3>(p, w, n, k, x, y, stream);
+    else launch_one<3, 3>(p, w, n, k, x, y, stream);
 }
 
 }  // namespace lq4

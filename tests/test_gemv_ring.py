@@ -5,11 +5,11 @@ Bars: one-hot activations return dequantised columns bit-exactly; max|delta| / m
 f32-accumulated oracle (tests/util.py; achieved ~2e-6, printed); rows of at most one slab (K <= 2048) are
 bit-identical to the lane-owns-block kernel, which adds a row's blocks in the same order.
 
-Shapes cover what the kernel branches on: rows shorter than a slab, a short last slab, two and three slabs with the
+Shapes cover what the kernels branch on: rows shorter than a slab, a short last slab, two and three slabs with the
 activations in registers, more slabs with the activations read from LDS, K above 8192 (three activation pieces a
 wave) up to the kernel's limit 24576, fewer rows than CUs, rows that straddle waves and workgroups, a vocabulary-
-sized matrix, and one-slab rows with more than 96 rows a workgroup (full and short rows), where the waves take
-rows from the workgroup's counter once their first six are under way.
+sized matrix, and rows of one, two and three slabs with more rows a workgroup than the waves' first ring fillings
+hold (96, 48, 32; full and short last slabs), where the waves take rows from the workgroup's counter.
 """
 import numpy as np
 import pytest
@@ -55,7 +55,7 @@ def run(be, w, x, n, k):
 
 RING_SHAPES = [(1, 32), (64, 64), (5, 96), (33, 32), (300, 2048), (2048, 2048), (1000, 1024), (12288, 2048),
                (2048, 6144), (700, 8160), (300, 17408), (4099, 5120), (70000, 256), (9, 24576), (255, 4096),
-               (257, 4128), (513, 10240), (30001, 2048), (25000, 1056)]
+               (257, 4128), (513, 10240), (30001, 2048), (25000, 1056), (13001, 4096), (9000, 5152)]
 
 
 @pytest.mark.parametrize("n,k", RING_SHAPES)

@@ -14,7 +14,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "liblattice_hip_q4.so")
-SOURCES = ["lq4_api.hip", "lq4_gemv.hip", "lq4_gemv_b1.hip", "lq4_gemv_dma.hip", "lq4_gemv_multi.hip", "lq4_gemv_i8.hip", "lq4_gemv_mfma.hip", "lq4_gemm.hip", "lq4_gemm_wreg.hip", "lq4_gemm_skinny.hip", "lq4_moe.hip", "lq4_moe_mfma.hip", "lq4_moe_b1.hip", "lq4_topk.hip", "lq4_elementwise.hip", "lq4_q8.hip", "lq4_q3.hip"]
+SOURCES = ["lq4_api.hip", "lq4_gemv.hip", "lq4_gemv_b1.hip", "lq4_gemv_dma.hip", "lq4_gemv_multi.hip", "lq4_gemv_i8.hip", "lq4_gemv_mfma.hip", "lq4_gemm.hip", "lq4_gemm_wreg.hip", "lq4_gemm_skinny.hip", "lq4_moe.hip", "lq4_moe_i8.hip", "lq4_moe_b1.hip", "lq4_topk.hip", "lq4_elementwise.hip", "lq4_q8.hip", "lq4_q3.hip"]
 
 # -packed-fp32-ops: keep the compiler from forming v_pk_*_f32 out of scalar float code.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",

@@ -1089,7 +1089,7 @@ int lq4_moe_ffn(lq4_ctx* ctx, const float* router_logits_dev, const lq4_weight* 
         const char* env = getenv("LQ4_MOE_SHARED_GROUPED_TOKENS");
         return env ? static_cast<uint32_t>(strtoul(env, nullptr, 10)) : kMoeSharedGroupedMaxTokens;
     }();
-    if (tokens > b1_tokens && tokens <= grouped_tokens && shared_inter == inter && num_experts < 1024 && moe_mfma_serves(hidden) && moe_mfma_serves(inter) &&
+    if (tokens > b1_tokens && tokens <= grouped_tokens && shared_inter == inter && num_experts < 1024 && moe_i8_serves(hidden) && moe_i8_serves(inter) &&
         static_cast<uint64_t>(num_experts) * 2 * inter <= UINT32_MAX &&
         static_cast<uint64_t>(num_experts) * hidden <= UINT32_MAX) {
         rc = resolve_weight(gate_up, 0, num_experts * 2 * inter, hidden, &rgu);

@@ -283,24 +283,21 @@ void launch_moe_grouped(const uint8_t* gate_up, const uint8_t* down, uint32_t nu
                         const int32_t* ids, const float* weights, uint32_t top_k, float* y,
                         const MoeScratch& s, hipStream_t stream, const uint8_t* shared_gate_up = nullptr,
                         const uint8_t* shared_down = nullptr);
-// With shared tensors (an expert as wide as the routed ones; needs moe_mfma_serves(hidden) and
-// moe_mfma_serves(inter)) ids / weights are [tokens, top_k + 1] as launch_moe_route writes them with a shared
+// With shared tensors (an expert as wide as the routed ones; needs moe_i8_serves(hidden) and
+// moe_i8_serves(inter)) ids / weights are [tokens, top_k + 1] as launch_moe_route writes them with a shared
 // gate, and the scratch is sized for tokens * (top_k + 1) pairs and num_experts + 1 experts.
-bool moe_mfma_serves(uint32_t k);
 
-// Matrix-core forms of the two expert passes (activations of a pass staged in LDS:
-// moe_mfma_lds_bytes(k) bytes for a reduction length k).
-size_t moe_mfma_lds_bytes(uint32_t k);
-// `ids` not null: the kernels find every expert's pairs in the routing table themselves (offsets and
-// order are then unused); null: they read the grouping tables.
-void launch_moe_gate_up_mfma(const uint8_t* gate_up, uint32_t num_experts, uint32_t inter, uint32_t hidden,
-                             const float* x, uint32_t tokens, uint32_t top_k, const int32_t* offsets,
-                             const int32_t* order, const int32_t* ids, float* h, hipStream_t stream,
-                             const uint8_t* last_expert = nullptr);
-void launch_moe_down_mfma(const uint8_t* down, uint32_t num_experts, uint32_t inter, uint32_t hidden,
-                          const float* h, uint32_t tokens, uint32_t top_k, const int32_t* offsets,
-                          const int32_t* order, const int32_t* ids, float* o, hipStream_t stream,
-                          const uint8_t* last_expert = nullptr);
+// Matrix-core form of the two expert passes (lq4_moe_i8.hip; the activations of a pass are staged in LDS, which
+// bounds the reduction length it takes).
+bool moe_i8_serves(uint32_t k);
+// `ids` not null (up to 512 pairs): the kernels find every expert's pairs in the routing table themselves (offsets
+// and order are then unused); null: they read the grouping tables.
+void launch_moe_gate_up_i8(const uint8_t* gate_up, uint32_t num_experts, uint32_t inter, uint32_t hidden, const float* x,
+                           uint32_t tokens, uint32_t top_k, const int32_t* offsets, const int32_t* order,
+                           const int32_t* ids, float* h, hipStream_t stream, const uint8_t* last_expert = nullptr);
+void launch_moe_down_i8(const uint8_t* down, uint32_t num_experts, uint32_t inter, uint32_t hidden, const float* h,
+                        uint32_t tokens, uint32_t top_k, const int32_t* offsets, const int32_t* order,
+                        const int32_t* ids, float* o, hipStream_t stream, const uint8_t* last_expert = nullptr);
 // (`last_expert`: the tensor of expert num_experts - 1 when it does not follow the others in `gate_up` / `down`)
 
 // Exact top-k over n logits (k <= 256): out_logits / out_ids receive the k best in rank order.

@@ -343,26 +343,24 @@ void launch_moe_grouped(const uint8_t* gate_up, const uint8_t* down, uint32_t nu
     const uint32_t experts = num_experts + (shared ? 1 : 0), slots = top_k + (shared ? 1 : 0);
     const uint32_t pairs = tokens * slots;
     // matrix-core kernels whenever one pass's activations fit in LDS; the plain kernels otherwise
-    const bool mfma_up = moe_mfma_serves(hidden), mfma_down = moe_mfma_serves(inter);
-    // With few pairs every expert workgroup finds its own pairs in the routing table (one load and a
-    // ballot): no grouping launch and no offsets -> order -> row chain of dependent loads.
-    // (every workgroup pays the scan: from about 300 pairs on the grouping launch is cheaper; whole layer at 48 /
-    // 64 / 96 / 128 tokens of top-8 with the limit at 1024 pairs 109.7 / 132.8 / 195.7 / 273.9 us, at 320 pairs
-    // 102.6 / 121.8 / 167.8 / 205.6)
-    const bool scan = mfma_up && mfma_down && pairs <= 320;
+    const bool mfma_up = moe_i8_serves(hidden), mfma_down = moe_i8_serves(inter);
+    // Up to 512 pairs the expert kernels read the routing table themselves (a thread per pair): no grouping launch, no
+    // offsets -> order -> row chain of dependent loads, and they enumerate the (expert, pass) combinations that
+    // exist, so the grid has no workgroups for the others.
+    const bool scan = mfma_up && mfma_down && pairs <= 512;
     const int32_t* scan_ids = scan ? ids : nullptr;
     if (!scan)
         hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(256), 0, stream, ids, pairs, experts, s.counts,
                            s.offsets, s.order);
     if (mfma_up)
-        launch_moe_gate_up_mfma(gate_up, experts, inter, hidden, x, tokens, slots, s.offsets, s.order, scan_ids,
+        launch_moe_gate_up_i8(gate_up, experts, inter, hidden, x, tokens, slots, s.offsets, s.order, scan_ids,
                                 s.h, stream, shared_gate_up);
     else
         hipLaunchKernelGGL(moe_gate_up_kernel, dim3((inter + kMoeWaves - 1) / kMoeWaves, num_experts),
                            dim3(kMoeWaves * 64), 0, stream, gate_up, inter, hidden, x, top_k, s.offsets,
                            s.order, s.h);
     if (mfma_down)
-        launch_moe_down_mfma(down, experts, inter, hidden, s.h, tokens, slots, s.offsets, s.order, scan_ids, s.o,
+        launch_moe_down_i8(down, experts, inter, hidden, s.h, tokens, slots, s.offsets, s.order, scan_ids, s.o,
                              stream, shared_down);
     else
         hipLaunchKernelGGL(moe_down_kernel, dim3((hidden + 2 * kMoeWaves - 1) / (2 * kMoeWaves), num_experts),
@@ -370,7 +368,5 @@ void launch_moe_grouped(const uint8_t* gate_up, const uint8_t* down, uint32_t nu
                            s.o);
     launch_combine(s.o, ids, weights, experts, slots, hidden, tokens, y, stream);
 }
-
-bool moe_mfma_serves(uint32_t k) { return moe_mfma_lds_bytes(k) <= 150 * 1024; }
 
 }  // namespace lq4

@@ -11,7 +11,7 @@
 // accumulate_routed_experts (crates/inference/src/model/qwen35/moe.rs:127-190) visits a token's
 // selected experts one after the other; with one token no two pairs share an expert, so nothing is
 // read twice, and with a few tokens the little that is costs less than the grouped kernels' fixed
-// parts (lq4_moe_mfma.hip serves larger steps, where tokens do share experts).
+// parts (lq4_moe_i8.hip serves larger steps, where tokens do share experts).
 // Slots with an id outside [0, E) are skipped as the reference skips them (moe.rs:147-149): they read
 // expert 0 (any valid address) and enter the sum with weight 0.
 // The shared expert (moe.rs:194-250) can ride along as one more slot with the weight

@@ -606,7 +606,9 @@ def test_moe_experts_for_a_few_tokens(be, cfg):
                                  dict(e=5, inter=1024, hidden=1024, tokens=9, top_k=3),    # 32 blocks per row both ways
                                  dict(e=4, inter=2048, hidden=4096, tokens=10, top_k=2),   # one slab down, two up
                                  dict(e=6, inter=544, hidden=2112, tokens=12, top_k=4),    # partial slabs
-                                 dict(e=40, inter=512, hidden=2048, tokens=120, top_k=8)]) # 960 pairs
+                                 dict(e=40, inter=512, hidden=2048, tokens=120, top_k=8),  # 960 pairs: grouping launch
+                                 dict(e=16, inter=256, hidden=512, tokens=60, top_k=8),    # 480 pairs: table of 8 words an expert
+                                 dict(e=600, inter=64, hidden=128, tokens=10, top_k=4)])   # more experts than the table takes
 def test_moe_grouped_experts_with_several_passes_per_expert(be, cfg):
     """Steps above 8 tokens: pairs grouped by expert, up to four per pass over the expert's blocks, experts
     chosen by many tokens in several passes; unfilled slots skipped."""

@@ -71,7 +71,7 @@ namespace {
 constexpr size_t kFusedPrologueBytes = 64u << 10;  // lq4_gemv_fused_batch: see there
 constexpr uint32_t kSharedB1MaxTokens = 8;  // shared expert alone through the per-pair kernels up to here (route + routed + shared as three calls: 8 tokens 56.0 -> 51.7 us, 16 tokens 68.5 -> 66.6, 32 tokens 89.3 -> 94.3)
 constexpr uint32_t kMoeB1MaxTokens = 8;  // per-pair expert kernels up to here (measured: 1 / 2 / 4 / 8 / 16 tokens 27.5 / 30.5 / 43.2 / 45.1 / 48.6 us grouped, 13.7 / 18.3 / 25.9 / 39.1 / 65.0 per pair)
-constexpr uint32_t kMoeSharedGroupedMaxTokens = 56;  // lq4_moe_ffn: shared expert as one more expert of the grouped kernels up to here
+constexpr uint32_t kMoeSharedGroupedMaxTokens = 384;  // lq4_moe_ffn: shared expert as one more expert of the grouped kernels up to here (level at 512)
 constexpr uint32_t kMultiMaxRows = 128;  // lq4_gemv_multi: up to the few-token GEMM's range
 constexpr uint32_t kLoraTRows = 4096;  // most rows one LoRA-fused call may carry
 
@@ -1082,9 +1082,8 @@ int lq4_moe_ffn(lq4_ctx* ctx, const float* router_logits_dev, const lq4_weight* 
     // More tokens, shared expert as wide as the routed ones: it rides along in the grouped kernels as expert
     // `num_experts`, chosen by every token in slot `top_k` with the sigmoid gate as its weight (the router
     // launch computes it): route, gate||up, down, combine, and none of the shared expert's own launches.
-    // Whole layer, config 4's shapes, 12 / 16 / 32 / 48 tokens: 65.5 / 65.7 / 83.8 / 102.6 -> 49.9 / 50.0 / 71.4 / 88.8 us.
-    // From 64 tokens on the shared expert's own GEMMs (weights read once, 16x16x32 tiles) are level or ahead
-    // (64 / 128 / 512 tokens: 121.8 / 205.6 / 690 against 126.6 / 210.4 / 728).
+    // Whole layer, config 4's shapes, against the shared expert's own launches after the routed experts (16 / 64 /
+    // 128 / 256 / 512 tokens): 61.8 / 100.2 / 152.3 / 270.6 / 455.6 -> 43.6 / 95.1 / 147.1 / 251.4 / 457.1 us.
     static const uint32_t grouped_tokens = [] {
         const char* env = getenv("LQ4_MOE_SHARED_GROUPED_TOKENS");
         return env ? static_cast<uint32_t>(strtoul(env, nullptr, 10)) : kMoeSharedGroupedMaxTokens;

@@ -290,8 +290,9 @@ void launch_moe_grouped(const uint8_t* gate_up, const uint8_t* down, uint32_t nu
 // Matrix-core form of the two expert passes (lq4_moe_i8.hip; the activations of a pass are staged in LDS, which
 // bounds the reduction length it takes).
 bool moe_i8_serves(uint32_t k);
-// `ids` not null (up to 512 pairs): the kernels find every expert's pairs in the routing table themselves (offsets
-// and order are then unused); null: they read the grouping tables.
+// `ids` not null (up to kMoeIdsMaxPairs pairs and kMoeIdsMaxExperts experts): the kernels find every expert's pairs in
+// the routing table themselves (offsets and order are then unused); null: they read the grouping tables.
+constexpr uint32_t kMoeIdsMaxPairs = 512, kMoeIdsMaxExperts = 512;
 void launch_moe_gate_up_i8(const uint8_t* gate_up, uint32_t num_experts, uint32_t inter, uint32_t hidden, const float* x,
                            uint32_t tokens, uint32_t top_k, const int32_t* offsets, const int32_t* order,
                            const int32_t* ids, float* h, hipStream_t stream, const uint8_t* last_expert = nullptr);

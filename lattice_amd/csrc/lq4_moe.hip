@@ -13,7 +13,6 @@ namespace lq4 {
 namespace {
 
 constexpr int kMaxExperts = 1024;
-constexpr uint32_t kSmallPairs = 512;  // pair count up to which the grouping kernel ranks by scanning
 
 // Router of one token per wave: see route_one_token.  The routing table has `out_stride` slots per token.
 // With a shared expert (`shared_gate` not null) the wave also fills slot `top_k`: expert id `num_experts` (the
@@ -75,118 +74,97 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
     }
 }
 
-// Single workgroup: counts per expert, exclusive prefix, then a stable fill of `order` (the
-// pairs of one expert stay in ascending pair index).  Each of the four waves owns a contiguous
-// segment of the pairs: it counts its segment, receives a cursor per expert that starts where
-// the lower segments end, and then walks its segment 64 pairs at a time, ranking the lanes
-// that share an expert with a ballot.
-__global__ __launch_bounds__(256) void moe_group_kernel(const int32_t* __restrict__ ids,
-                                                        uint32_t pairs, uint32_t num_experts,
-                                                        int32_t* __restrict__ counts,
-                                                        int32_t* __restrict__ offsets,
-                                                        int32_t* __restrict__ order) {
-    __shared__ int32_t s_cnt[4 * kMaxExperts];  // [wave][expert]: counts, later cursors
-    __shared__ int32_t s_off[kMaxExperts + 1];
+// Stable grouping of the (token, slot) pairs by expert: counts, offsets (exclusive prefix) and `order`, in which the
+// pairs of one expert stay in ascending pair index.  One workgroup of sixteen waves:
+//   1. a histogram of the experts (LDS integer atomics: the totals do not depend on the order of arrival) and its
+//      exclusive scan, which also becomes every expert's cursor;
+//   2. rounds of 1024 pairs, a wave per 64 of them: the lanes of a wave that share an expert rank themselves with
+//      ballots (registers only, one turn per distinct expert of the wave) and the first of them notes how many they
+//      are in a [wave][expert] table; a thread per expert turns its column into an exclusive prefix over the waves and
+//      moves the expert's cursor on; every pair then knows its place: cursor + pairs of its expert in the waves
+//      before it + its rank in its wave.
+// (An earlier form of four waves that walked their segments with a cursor in LDS per ballot turn needed 34 us for 576
+// pairs and 54 us for 1152; this one about 5.)
+constexpr int kGroupThreads = 1024, kGroupWaves = kGroupThreads / 64;
+
+__global__ __launch_bounds__(kGroupThreads) void moe_group_kernel(const int32_t* __restrict__ ids, uint32_t pairs,
+                                                                  uint32_t num_experts, int32_t* __restrict__ counts,
+                                                                  int32_t* __restrict__ offsets,
+                                                                  int32_t* __restrict__ order) {
+    __shared__ int32_t s_cur[kMaxExperts + 2];   // counts, then the cursor of every expert
+    __shared__ int32_t s_base[kMaxExperts + 2];  // the cursor at the start of the round
+    __shared__ int32_t s_wsum[kGroupWaves];
+    __shared__ uint16_t s_tbl[kGroupWaves][kMaxExperts + 2];  // pairs of an expert in a wave, then in the waves before it
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    if (pairs <= kSmallPairs && num_experts <= 256) {
-        // decode-sized batches: ids live in LDS, every thread ranks its own pairs by scanning the
-        // ids before them (a broadcast read per step), one global round trip in and one out
-        int32_t* s_ids = s_cnt + kMaxExperts;
-        for (uint32_t p = tid; p < pairs; p += 256) s_ids[p] = ids[p];
-        if (tid < num_experts) s_cnt[tid] = 0;
-        __syncthreads();
-        for (uint32_t p = tid; p < pairs; p += 256) {
-            const int32_t e = s_ids[p];
-            if (e >= 0 && e < static_cast<int32_t>(num_experts)) atomicAdd(&s_cnt[e], 1);
-        }
-        __syncthreads();
-        if (wave == 0) {
-            int32_t carry = 0;
-            for (uint32_t base = 0; base < num_experts; base += 64) {
-                const uint32_t e = base + lane;
-                const int32_t c = e < num_experts ? s_cnt[e] : 0;
-                int32_t v = c;
-                for (int d = 1; d < 64; d <<= 1) {
-                    const int32_t up = __shfl_up(v, d, 64);
-                    if (static_cast<int>(lane) >= d) v += up;
-                }
-                if (e < num_experts) {
-                    counts[e] = c;
-                    offsets[e + 1] = v + carry;
-                    s_off[e] = v + carry - c;
-                }
-                carry += __shfl(v, 63, 64);
-            }
-            if (lane == 0) offsets[0] = 0;
-        }
-        __syncthreads();
-        for (uint32_t p = tid; p < pairs; p += 256) {
-            const int32_t e = s_ids[p];
-            if (e < 0 || e >= static_cast<int32_t>(num_experts)) continue;
-            int32_t rank = 0;
-            for (uint32_t q = 0; q < p; ++q) rank += (s_ids[q] == e);
-            order[s_off[e] + rank] = static_cast<int32_t>(p);
-        }
-        return;
-    }
-    for (uint32_t i = tid; i < 4 * kMaxExperts; i += 256) s_cnt[i] = 0;
+    auto valid_id = [&](int32_t e) { return e >= 0 && e < static_cast<int32_t>(num_experts); };
+    for (uint32_t e = tid; e < num_experts; e += kGroupThreads) s_cur[e] = 0;
     __syncthreads();
-    const uint32_t seg = (((pairs + 3) / 4 + 63) / 64) * 64;
-    const uint32_t p_beg = wave * seg < pairs ? wave * seg : pairs;
-    const uint32_t p_end = p_beg + seg < pairs ? p_beg + seg : pairs;
-    for (uint32_t p = p_beg + lane; p < p_end; p += 64) {
+    for (uint32_t p = tid; p < pairs; p += kGroupThreads) {
         const int32_t e = ids[p];
-        if (e >= 0 && e < static_cast<int32_t>(num_experts)) atomicAdd(&s_cnt[wave * kMaxExperts + e], 1);
+        if (valid_id(e)) atomicAdd(&s_cur[e], 1);
     }
     __syncthreads();
-    for (uint32_t e = tid; e < num_experts; e += 256) {
-        const int32_t c = s_cnt[e] + s_cnt[kMaxExperts + e] + s_cnt[2 * kMaxExperts + e] + s_cnt[3 * kMaxExperts + e];
-        counts[e] = c;
-        s_off[e + 1] = c;
-    }
-    __syncthreads();
-    if (wave == 0) {  // inclusive scan of the counts, 64 experts at a time
-        int32_t carry = 0;
-        for (uint32_t base = 0; base < num_experts; base += 64) {
-            const uint32_t e = base + lane;
-            int32_t v = e < num_experts ? s_off[e + 1] : 0;
-            for (int d = 1; d < 64; d <<= 1) {
-                const int32_t up = __shfl_up(v, d, 64);
-                if (static_cast<int>(lane) >= d) v += up;
-            }
-            if (e < num_experts) s_off[e + 1] = v + carry;
-            carry += __shfl(v, 63, 64);
+    int32_t carry = 0;
+    for (uint32_t base = 0; base < num_experts; base += kGroupThreads) {  // (uniform)
+        const uint32_t e = base + tid;
+        const int32_t c = e < num_experts ? s_cur[e] : 0;
+        int32_t incl = c;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int32_t up = __shfl_up(incl, d, 64);
+            if (static_cast<int>(lane) >= d) incl += up;
         }
-        if (lane == 0) s_off[0] = 0;
-    }
-    __syncthreads();
-    for (uint32_t e = tid; e <= num_experts; e += 256) offsets[e] = s_off[e];
-    for (uint32_t e = tid; e < num_experts; e += 256) {
-        int32_t run = s_off[e];
-        for (int w = 0; w < 4; ++w) {
-            const int32_t c = s_cnt[w * kMaxExperts + e];
-            s_cnt[w * kMaxExperts + e] = run;
-            run += c;
+        if (lane == 63) s_wsum[wave] = incl;
+        __syncthreads();
+        int32_t before = 0, total = 0;
+#pragma unroll
+        for (int w = 0; w < kGroupWaves; ++w) {
+            before += static_cast<uint32_t>(w) < wave ? s_wsum[w] : 0;
+            total += s_wsum[w];
         }
+        __syncthreads();  // (s_wsum is written again in the next turn)
+        if (e < num_experts) {
+            const int32_t excl = carry + before + incl - c;
+            counts[e] = c;
+            offsets[e] = excl;
+            s_cur[e] = excl;
+        }
+        carry += total;
     }
-    __syncthreads();
-    volatile int32_t* cur = s_cnt + wave * kMaxExperts;
-    for (uint32_t base = p_beg; base < p_end; base += 64) {
-        const uint32_t p = base + lane;
-        const int32_t e = p < p_end ? ids[p] : -1;
-        const bool valid = e >= 0 && e < static_cast<int32_t>(num_experts);
+    if (tid == 0) offsets[num_experts] = carry;
+    for (uint32_t p0 = 0; p0 < pairs; p0 += kGroupThreads) {  // (uniform)
+        for (int w = 0; w < kGroupWaves; ++w)
+            for (uint32_t e = tid; e < num_experts; e += kGroupThreads) s_tbl[w][e] = 0;
+        __syncthreads();  // (also: the cursors are in place)
+        const uint32_t p = p0 + tid;
+        const int32_t e = p < pairs ? ids[p] : -1;
+        const bool valid = valid_id(e);
+        int32_t rank = 0;
         unsigned long long active = __ballot(valid);
-        while (active) {
+        while (active) {  // (uniform in the wave)
             const int leader = __ffsll(static_cast<long long>(active)) - 1;
             const int32_t le = __shfl(e, leader, 64);
             const bool mine = valid && e == le;
             const unsigned long long m = __ballot(mine);
-            if (mine) order[cur[le] + __popcll(m & ((1ull << lane) - 1ull))] = static_cast<int32_t>(p);
-            __builtin_amdgcn_wave_barrier();
-            if (static_cast<int>(lane) == leader) cur[le] = cur[le] + __popcll(m);
-            __builtin_amdgcn_wave_barrier();
+            if (mine) rank = __popcll(m & ((1ull << lane) - 1ull));
+            if (static_cast<int>(lane) == leader) s_tbl[wave][le] = static_cast<uint16_t>(__popcll(m));
             active &= ~m;
         }
+        __syncthreads();
+        for (uint32_t e2 = tid; e2 < num_experts; e2 += kGroupThreads) {
+            const int32_t start = s_cur[e2];
+            int32_t run = 0;
+            for (int w = 0; w < kGroupWaves; ++w) {
+                const int32_t c = s_tbl[w][e2];
+                s_tbl[w][e2] = static_cast<uint16_t>(run);
+                run += c;
+            }
+            s_base[e2] = start;
+            s_cur[e2] = start + run;
+        }
+        __syncthreads();
+        if (valid) order[s_base[e] + s_tbl[wave][e] + rank] = static_cast<int32_t>(p);
+        __syncthreads();  // (the table is cleared again in the next round)
     }
 }
 
@@ -347,10 +325,10 @@ void launch_moe_grouped(const uint8_t* gate_up, const uint8_t* down, uint32_t nu
     // Up to 512 pairs the expert kernels read the routing table themselves (a thread per pair): no grouping launch, no
     // offsets -> order -> row chain of dependent loads, and they enumerate the (expert, pass) combinations that
     // exist, so the grid has no workgroups for the others.
-    const bool scan = mfma_up && mfma_down && pairs <= 512;
+    const bool scan = mfma_up && mfma_down && pairs <= kMoeIdsMaxPairs && experts <= kMoeIdsMaxExperts;
     const int32_t* scan_ids = scan ? ids : nullptr;
     if (!scan)
-        hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(256), 0, stream, ids, pairs, experts, s.counts,
+        hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(kGroupThreads), 0, stream, ids, pairs, experts, s.counts,
                            s.offsets, s.order);
     if (mfma_up)
         launch_moe_gate_up_i8(gate_up, experts, inter, hidden, x, tokens, slots, s.offsets, s.order, scan_ids,

@@ -21,10 +21,10 @@
 // CW waves split the 8-block chunks of a tile and add their partial sums through LDS in wave order; TW = 8 / CW tiles
 // are worked on side by side; a workgroup does `rounds` such rounds.
 //
-// Grid.  With the routing table at hand (up to 512 pairs, a thread per pair) the y index counts only the (expert,
-// pass) combinations that exist (moe_combo_pairs): a workgroup that finds nothing to do still holds a CU slot for a
-// microsecond, and a grid over every expert and every possible pass is mostly such workgroups.  Otherwise (grouping
-// tables from a launch before this one) the grid is (row chunks, experts, passes).
+// Grid.  The y index counts only the (expert, pass) combinations that exist, found from the routing table itself (up
+// to 512 pairs, a thread per pair: moe_combo_from_ids) or from the grouping tables of a launch before this one
+// (moe_combo_from_tables): a workgroup that finds nothing to do still holds a CU slot for a microsecond, and a grid
+// over every expert and every possible pass is mostly such workgroups.
 //
 // What the time stamps of a development build showed for 16 tokens of top 8 among 64 experts (73 MB gate/up, 37 MB
 // down), and what this file does about it: (1) with four waves and 32 output rows a workgroup, 912 workgroups had
@@ -32,7 +32,8 @@
 // 64 (gate/up) or 256 (down) rows make about 460, which all start at once; (2) a CU's share of the memory system is
 // about 18 KB/us and answers in the order of asking, so activations asked for behind a whole ring of every wave on the
 // CU arrived last and the matrix work that could have run beside the stream ran after it -- one unit a wave is
-// requested before the staging, the rest of the ring after its barrier; (3) per CU the vector instructions (about 140
+// requested before the staging, the rest of the ring after its barrier (none, two or four units before it, with or
+// without a barrier between the requests for activations and for weights, all measured level or behind); (3) per CU the vector instructions (about 140
 // a unit) and the LDS traffic (14 KB a unit) each still add up to about half the streaming time.
 //
 // Precision: weights and integer sums are exact; an activation is rounded to a multiple of its block's largest
@@ -52,85 +53,89 @@ struct MoeGemvArgs {
     float* out;              // h (GATE_UP) or o
     const int32_t* offsets;  // [E + 1]
     const int32_t* order;    // pair indices grouped by expert
-    const int32_t* ids;      // routed expert of every pair; not null = find the expert's pairs here
-    uint32_t n_pairs;        // instead of in offsets/order (few pairs: saves a launch and two dependent loads)
+    const int32_t* ids;      // routed expert of every pair; not null = find the expert's pairs here instead of in
+    uint32_t n_pairs;        // offsets/order (up to 512 pairs: saves a launch and two dependent loads)
     uint32_t rows_per_expert;  // weight rows of one expert (2I or H)
     uint32_t out_rows;         // output rows per pair (I or H)
     uint32_t k;                // reduction length (H or I)
     uint32_t x_stride;         // floats between activation rows
     uint32_t x_div;            // activation row of a pair = pair / x_div (top_k for x, 1 for h)
     uint32_t rounds;           // rounds of tiles per workgroup
-    const uint8_t* w_last;     // not null: the last expert of the grid lives here, not behind the others in w
-    uint32_t experts;          // experts in all (the grid's y extent unless the kernel enumerates (expert, pass) itself)
+    const uint8_t* w_last;     // not null: the last expert lives here, not behind the others in w
+    uint32_t experts;          // experts in all
 };
 
-// (expert, pass) of this workgroup.  An expert with tensors of its own (w_last) is one that every token chose: all
-// its passes are full-length work, so they are dispatched first instead of forming the tail of the launch (the
-// grid is walked x, then y, then z).
-__device__ __forceinline__ void moe_expert_and_pass(const MoeGemvArgs& p, uint32_t& e, uint32_t& pass) {
-    e = blockIdx.y;
-    pass = blockIdx.z;
-    if (p.w_last != nullptr) {
-        const uint32_t lin = blockIdx.z * gridDim.y + blockIdx.y;
-        if (lin < gridDim.z) {
-            e = gridDim.y - 1;
-            pass = lin;
-        } else {
-            pass = (lin - gridDim.z) / (gridDim.y - 1);
-            e = (lin - gridDim.z) - pass * (gridDim.y - 1);
-        }
-    }
-}
-
-// The pairs of (expert e, pass) into s_pair[0 .. n), ascending pair index (= the stable grouping order); returns n,
-// 0 when the expert has no pair left for this pass (the same value in every thread of the workgroup).  s_pair holds
-// kMoePassPairs entries, s_cnt one per wave; both are LDS.  Ends with a barrier when n > 0.  THREADS = the workgroup's size.
+// The grid's y index counts (expert, pass) combinations that exist, not every expert times every possible pass: a
+// workgroup with nothing to do still holds a CU slot for a microsecond, and a grid over all of them is mostly such
+// workgroups (16 tokens of top 8 among 64 experts make about 60 combinations, not 64 x 4).  The host bounds their
+// number (combo_bound); a workgroup whose y is beyond the real count exits.
+//
+// From the grouping tables of a launch before this one (offsets [experts + 1], order [pairs]): combination blockIdx.y
+// in expert order (see expert_at); its pairs into s_pair[0 .. n), in the tables' (stable) order.  Returns n (0: beyond the
+// combinations; the same value in every thread) and the expert.  s_cnt holds a word per wave, s_misc two.
 template <int THREADS>
-__device__ __forceinline__ int moe_pass_pairs(const MoeGemvArgs& p, uint32_t e, uint32_t pass, int32_t* s_pair,
-                                              int32_t* s_cnt) {
+__device__ __forceinline__ int moe_combo_from_tables(const MoeGemvArgs& p, int32_t* s_pair, int32_t* s_cnt,
+                                                     int32_t* s_misc, uint32_t& e) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int first = static_cast<int>(pass) * kMoePassPairs;
-    if (p.ids) {
-        // Every workgroup scans the routing table itself: rank of a matching pair = matches before it.
-        int base = 0;
-        for (uint32_t c0 = 0; c0 < p.n_pairs; c0 += THREADS) {
-            const uint32_t pi = c0 + tid;
-            const bool hit = pi < p.n_pairs && p.ids[pi] == static_cast<int32_t>(e);
-            const uint64_t mask = __ballot(hit);
-            if (lane == 0) s_cnt[wave] = __popcll(mask);
-            __syncthreads();
-            int before = base;
-            for (int w2 = 0; w2 < wave; ++w2) before += s_cnt[w2];
-            const int rank = before + __popcll(mask & ((1ull << lane) - 1ull));
-            if (hit && rank >= first && rank < first + kMoePassPairs) s_pair[rank - first] = static_cast<int32_t>(pi);
+    // Order: expert order, except that an expert with tensors of its own (w_last: one that every token chose, all
+    // its passes full-length work) comes first instead of forming the tail of the launch.
+    auto expert_at = [&](uint32_t i) { return p.w_last == nullptr ? i : i == 0 ? p.experts - 1 : i - 1; };
+    auto passes_at = [&](uint32_t i) {
+        if (i >= p.experts) return 0;
+        const uint32_t ee = expert_at(i);
+        return (p.offsets[ee + 1] - p.offsets[ee] + kMoePassPairs - 1) / kMoePassPairs;
+    };
+    // a thread takes `per` consecutive places of the order; combinations before its first = an exclusive scan
+    const uint32_t per = (p.experts + THREADS - 1) / THREADS, e0 = static_cast<uint32_t>(tid) * per;
+    int local = 0;
+    for (uint32_t r = 0; r < per; ++r) local += passes_at(e0 + r);
+    int incl = local;
 #pragma unroll
-            for (int w2 = 0; w2 < THREADS / 64; ++w2) base += s_cnt[w2];
-            __syncthreads();
-        }
-        if (base <= first) return 0;
-        return base - first < kMoePassPairs ? base - first : kMoePassPairs;
+    for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += up;
     }
-    const int32_t beg = p.offsets[e] + first;
-    const int32_t end = p.offsets[e + 1];
-    if (beg >= end) return 0;
+    if (lane == 63) s_cnt[wave] = incl;
+    __syncthreads();
+    int before = 0, n_combos = 0;
+#pragma unroll
+    for (int w2 = 0; w2 < THREADS / 64; ++w2) {
+        before += w2 < wave ? s_cnt[w2] : 0;
+        n_combos += s_cnt[w2];
+    }
+    const int y = static_cast<int>(blockIdx.y);
+    if (y >= n_combos) return 0;
+    int c = before + incl - local;
+    if (y >= c && y < c + local) {  // one thread: the combination is among its experts
+        for (uint32_t r = 0; r < per; ++r) {
+            const int n = passes_at(e0 + r);
+            if (y < c + n) {
+                s_misc[0] = static_cast<int32_t>(expert_at(e0 + r));
+                s_misc[1] = y - c;
+                break;
+            }
+            c += n;
+        }
+    }
+    __syncthreads();
+    e = static_cast<uint32_t>(s_misc[0]);
+    const int32_t beg = p.offsets[e] + s_misc[1] * kMoePassPairs, end = p.offsets[e + 1];
     const int nt = end - beg < kMoePassPairs ? end - beg : kMoePassPairs;
     if (tid < nt) s_pair[tid] = p.order[beg + tid];
     __syncthreads();
     return nt;
 }
 
-// The same for a grid whose y index counts only the (expert, pass) combinations that exist, in the order of their
-// first pair (grid y = blockIdx.y, z unused; a thread per pair: n_pairs <= THREADS; ids given).  A workgroup with nothing
-// to do costs a CU slot for a microsecond, and a grid over every expert and every possible pass is mostly such
-// workgroups: 16 tokens of top 8 among 64 experts make about 60 combinations, not 64 x 4.
+// From the routing table itself (ids; a thread per pair: n_pairs <= THREADS): combination blockIdx.y in the order of
+// the combinations' first pairs; no grouping launch, no offsets -> order -> row chain of dependent loads.
 //   `mask` is LDS for experts x THREADS / 64 64-bit words (bit t % 64 of word t / 64 of an expert = pair t chose it;
 //   set with atomic ORs, so the table does not depend on the order of arrival), free again on return; s_misc holds 4
 //   words, s_cnt one per wave.
 // Returns n (0: blockIdx.y is beyond the combinations) and the expert.  An id outside [0, experts) matches nothing.
 template <int THREADS>
-__device__ __forceinline__ int moe_combo_pairs(const MoeGemvArgs& p, unsigned long long* mask, int32_t* s_pair,
+__device__ __forceinline__ int moe_combo_from_ids(const MoeGemvArgs& p, unsigned long long* mask, int32_t* s_pair,
                                                int32_t* s_cnt, int32_t* s_misc, uint32_t& e) {
     constexpr int W = THREADS / 64;  // words of an expert's row in the table
     const int tid = threadIdx.x;
@@ -208,8 +213,9 @@ size_t lds_bytes(uint32_t nb, uint32_t waves) {
 }
 
 // p.rounds = rounds of the workgroup; the launcher gives every wave a chunk (chunks of a row >= CW).
-// COMBOS: grid (row chunks, existing (expert, pass) combinations at most); else (row chunks, experts, passes).
-template <bool GATE_UP, int CW, int TW, bool COMBOS>
+// Grid (row chunks, a bound on the (expert, pass) combinations).  FROM_IDS: these come from the routing table, else
+// from the grouping tables.
+template <bool GATE_UP, int CW, int TW, bool FROM_IDS>
 __global__ __launch_bounds__(64 * CW * TW) void moe_expert_i8(MoeGemvArgs p) {
     constexpr int kWaves = CW * TW, kThreads = 64 * kWaves;
     constexpr int PRE = 1;  // units a wave requests before the activations are staged (the rest of its ring right after)
@@ -221,14 +227,10 @@ __global__ __launch_bounds__(64 * CW * TW) void moe_expert_i8(MoeGemvArgs p) {
     __shared__ int32_t s_pair[kMoePassPairs];
     __shared__ int32_t s_cnt[kWaves];
     __shared__ int32_t s_misc[4];
-    uint32_t e, pass;
+    uint32_t e;
     int nt;
-    if constexpr (COMBOS) {
-        nt = moe_combo_pairs<kThreads>(p, reinterpret_cast<unsigned long long*>(smem), s_pair, s_cnt, s_misc, e);
-    } else {
-        moe_expert_and_pass(p, e, pass);
-        nt = moe_pass_pairs<kThreads>(p, e, pass, s_pair, s_cnt);
-    }
+    if constexpr (FROM_IDS) nt = moe_combo_from_ids<kThreads>(p, reinterpret_cast<unsigned long long*>(smem), s_pair, s_cnt, s_misc, e);
+    else nt = moe_combo_from_tables<kThreads>(p, s_pair, s_cnt, s_misc, e);
     if (nt == 0) return;
 
     const uint32_t tw = wave / CW, cw = wave % CW;
@@ -474,23 +476,23 @@ __global__ __launch_bounds__(64 * CW * TW) void moe_expert_i8(MoeGemvArgs p) {
     }
 }
 
-template <bool GATE_UP, int CW, int TW, bool COMBOS>
+template <bool GATE_UP, int CW, int TW, bool FROM_IDS>
 void launch_cw(const MoeGemvArgs& a, uint32_t rows_per_wg, uint32_t passes, size_t lds, hipStream_t stream) {
     static LdsCapOnce lds_cap;
-    lds_cap.raise(reinterpret_cast<const void*>(moe_expert_i8<GATE_UP, CW, TW, COMBOS>), 159 * 1024);  // the rest is static
+    lds_cap.raise(reinterpret_cast<const void*>(moe_expert_i8<GATE_UP, CW, TW, FROM_IDS>), 159 * 1024);  // the rest is static
     const uint32_t row_chunks = (a.out_rows + rows_per_wg - 1) / rows_per_wg;
     // combinations at most: all but the last of an expert hold four pairs (pairs / 4 + experts); every one has a
     // first pair of its own (pairs); experts x passes
-    uint32_t combos = a.n_pairs / kMoePassPairs + a.experts;
-    if (combos > a.n_pairs) combos = a.n_pairs;
-    if (combos > a.experts * passes) combos = a.experts * passes;
-    const dim3 grid = COMBOS ? dim3(row_chunks, combos) : dim3(row_chunks, a.experts, passes);
-    hipLaunchKernelGGL((moe_expert_i8<GATE_UP, CW, TW, COMBOS>), grid, dim3(64 * CW * TW), lds, stream, a);
+    uint32_t combo_bound = a.n_pairs / kMoePassPairs + a.experts;
+    if (combo_bound > a.n_pairs) combo_bound = a.n_pairs;
+    if (combo_bound > a.experts * passes) combo_bound = a.experts * passes;
+    hipLaunchKernelGGL((moe_expert_i8<GATE_UP, CW, TW, FROM_IDS>), dim3(row_chunks, combo_bound), dim3(64 * CW * TW), lds,
+                       stream, a);
 }
 
 template <bool GATE_UP, int CW, int TW>
-void launch_combos(bool combos, const MoeGemvArgs& a, uint32_t rows_per_wg, uint32_t passes, size_t lds, hipStream_t stream) {
-    if (combos) launch_cw<GATE_UP, CW, TW, true>(a, rows_per_wg, passes, lds, stream);
+void launch_from(bool from_ids, const MoeGemvArgs& a, uint32_t rows_per_wg, uint32_t passes, size_t lds, hipStream_t stream) {
+    if (from_ids) launch_cw<GATE_UP, CW, TW, true>(a, rows_per_wg, passes, lds, stream);
     else launch_cw<GATE_UP, CW, TW, false>(a, rows_per_wg, passes, lds, stream);
 }
 
@@ -508,9 +510,8 @@ void launch_moe_expert_i8(MoeGemvArgs a, uint32_t num_experts, uint32_t max_pair
     size_t lds = lds_bytes(nb, kWaves);
     if (!moe_i8_serves(a.k)) return;  // the caller asked first
     a.experts = num_experts;
-    // The kernel enumerates the combinations itself where a thread per pair and its table of experts allow.
-    const bool combos = a.ids != nullptr && a.n_pairs <= 64 * kWaves && num_experts <= 512;
-    if (combos && lds < static_cast<size_t>(num_experts) * kWaves * 8) lds = static_cast<size_t>(num_experts) * kWaves * 8;
+    const bool from_ids = a.ids != nullptr;  // (the caller: up to kMoeIdsMaxPairs pairs and kMoeIdsMaxExperts experts)
+    if (from_ids && lds < static_cast<size_t>(num_experts) * kWaves * 8) lds = static_cast<size_t>(num_experts) * kWaves * 8;
     // Waves split K only where every one of them finds a chunk or two.  Workgroups of eight waves over about 64
     // (gate/up) or 256 (down) output rows, 160 KB of blocks each: 16 tokens of top 8 among 64 experts then make
     // about 460 workgroups with work, which all start at once (two fit a CU).  Measured there against four waves
@@ -523,8 +524,8 @@ void launch_moe_expert_i8(MoeGemvArgs a, uint32_t num_experts, uint32_t max_pair
     if (rounds < 1) rounds = 1;
     a.rounds = rounds;
     const uint32_t rows_per_wg = rounds * tw * 16, passes = (max_pairs_per_expert + kMoePassPairs - 1) / kMoePassPairs;
-    if (cw == 2) launch_combos<GATE_UP, 2, 4>(combos, a, rows_per_wg, passes, lds, stream);
-    else launch_combos<GATE_UP, 1, 8>(combos, a, rows_per_wg, passes, lds, stream);
+    if (cw == 2) launch_from<GATE_UP, 2, 4>(from_ids, a, rows_per_wg, passes, lds, stream);
+    else launch_from<GATE_UP, 1, 8>(from_ids, a, rows_per_wg, passes, lds, stream);
 }
 
 }  // namespace

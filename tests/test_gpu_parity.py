@@ -608,7 +608,8 @@ def test_moe_experts_for_a_few_tokens(be, cfg):
                                  dict(e=6, inter=544, hidden=2112, tokens=12, top_k=4),    # partial slabs
                                  dict(e=40, inter=512, hidden=2048, tokens=120, top_k=8),  # 960 pairs: grouping launch
                                  dict(e=16, inter=256, hidden=512, tokens=60, top_k=8),    # 480 pairs: table of 8 words an expert
-                                 dict(e=600, inter=64, hidden=128, tokens=10, top_k=4)])   # more experts than the table takes
+                                 dict(e=600, inter=64, hidden=128, tokens=10, top_k=4),    # more experts than the table takes
+                                 dict(e=24, inter=64, hidden=128, tokens=150, top_k=8)])   # 1200 pairs: two rounds of the grouping
 def test_moe_grouped_experts_with_several_passes_per_expert(be, cfg):
     """Steps above 8 tokens: pairs grouped by expert, up to four per pass over the expert's blocks, experts
     chosen by many tokens in several passes; unfilled slots skipped."""
@@ -690,7 +691,8 @@ def test_moe_ffn_one_call_equals_the_three_calls(be, tokens):
                                  dict(e=8, inter=1024, hidden=512, tokens=2, top_k=8),      # 9 x 1024 > 8192: three calls inside
                                  dict(e=64, inter=512, hidden=2048, tokens=16, top_k=8),    # config 4: the grouped kernels
                                  dict(e=6, inter=96, hidden=160, tokens=13, top_k=3),       # ragged last pass of every expert
-                                 dict(e=12, inter=64, hidden=96, tokens=48, top_k=7)])      # 384 pairs: grouping launch
+                                 dict(e=12, inter=64, hidden=96, tokens=48, top_k=7),       # 384 pairs: pairs found from the routing table
+                                 dict(e=12, inter=64, hidden=96, tokens=80, top_k=7)])      # 640 pairs: grouping launch, shared expert's passes first
 def test_moe_ffn_with_the_shared_expert_as_a_slot(be, cfg):
     """A shared expert as wide as the routed ones rides along: as one more slot of the per-pair kernels for up to
     8 tokens, as one more expert of the grouped kernels above that.  The whole layer against the oracle (routed
@@ -717,7 +719,7 @@ def test_moe_ffn_with_the_shared_expert_as_a_slot(be, cfg):
     # the shared part alone, so that an error in it (or in its gate) cannot hide behind the routed sum
     d_err = rel_err(host(y) - routed64, want - routed64)
     print(f"  rel err {err:.2e}, shared part alone {d_err:.2e}", flush=True)
-    as_slot = 8 < tokens <= 56 or (top_k + 1) * inter <= 8192  # (above 56 tokens: the shared expert's own GEMMs)
+    as_slot = 8 < tokens <= 384 or (top_k + 1) * inter <= 8192  # (above 384 tokens: the shared expert's own GEMMs)
     assert err <= (5e-5 if as_slot else REL_TOL) and d_err <= (2e-4 if as_slot else 2 * REL_TOL)
     # gate||up and down once for the layer when the shared expert rode along; otherwise once for the routed
     # experts and once more for the shared expert alone (the same kernels with it as their only slot); no dense

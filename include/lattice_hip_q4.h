@@ -238,9 +238,10 @@ int lq4_moe_shared_expert(lq4_ctx* ctx, const lq4_weight* gate_up, const lq4_wei
  *   - up to 8 tokens with hidden <= 8192 and (top_k + 1) * inter <= 8192: two launches (every
  *     (token, slot) pair as a one-token GEMV, the shared expert as one more slot, the router and the
  *     shared expert's gate inside the first launch when num_experts <= 256);
- *   - from 9 to 56 tokens (num_experts < 1024): the shared expert is one more expert of the grouped
+ *   - from 9 to 384 tokens (num_experts < 1024): the shared expert is one more expert of the grouped
  *     kernels, chosen by every token with sigmoid(x . shared_gate) as its routing weight, which the
- *     router launch computes: four launches, none of the shared expert's own. */
+ *     router launch computes: four launches (five above 512 (token, slot) pairs, where a grouping
+ *     launch runs first), none of the shared expert's own. */
 int lq4_moe_ffn(lq4_ctx* ctx, const float* router_logits_dev, const lq4_weight* gate_up, const lq4_weight* down,
                 uint32_t num_experts, uint32_t top_k, uint32_t inter, const lq4_weight* shared_gate_up,
                 const lq4_weight* shared_down, const float* shared_gate_dev, uint32_t shared_inter,

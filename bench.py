@@ -174,6 +174,74 @@ def prefill_gemm(torch, be, gen, tm):
     return gemm
 
 
+def moe_section(torch, be, gen, tm, synth):
+    """BASELINE config 4 (grouped expert GEMV), the whole MoE layer in its call forms, and the one-token layer."""
+    out = {}
+    # MoE grouped expert GEMV, benchmark config 4
+    mo = synth.MOE_35B
+    E, I, H, T, TK = mo["experts"], mo["inter"], mo["hidden"], mo["tokens"], mo["top_k"]
+    sets = []
+    for _ in range(10):  # 10 x 125.8 MB of expert tensors
+        sets.append((be.wrap_device_blocks(device_q4_weight(torch, E * 2 * I, H, gen)),
+                     be.wrap_device_blocks(device_q4_weight(torch, E * H, I, gen))))
+    lg = torch.from_numpy(synth.router_logits(T, E, seed=0)).cuda()
+    ids, wts = be.moe_route(lg, TK)
+    xm = torch.randn((T, H), device="cuda", generator=gen)
+    ym = torch.empty((T, H), device="cuda")
+    distinct = int(torch.unique(ids).numel())
+    moe_bytes = distinct * (2 * I * (H // 32) * 20 + H * (I // 32) * 20) + 2 * T * H * 4
+    f = lambda i: be.moe_experts(sets[i % len(sets)][0], sets[i % len(sets)][1], E, I, H, xm, ids, wts, ym)
+    for i in range(len(sets)):
+        f(i)
+    ms = tm(torch, f, 40)
+    # the same step with the router in front of it (softmax, top-k, renormalise from the logits)
+    def routed(i):
+        ids_i, wts_i = be.moe_route(lg, TK)
+        be.moe_experts(sets[i % len(sets)][0], sets[i % len(sets)][1], E, I, H, xm, ids_i, wts_i, ym)
+    for i in range(3):
+        routed(i)
+    ms_routed = tm(torch, routed, 40)
+    # ... and with the always-active shared expert (same intermediate size) added onto the sum
+    shared = [(be.wrap_device_blocks(device_q4_weight(torch, 2 * I, H, gen)),
+               be.wrap_device_blocks(device_q4_weight(torch, H, I, gen))) for _ in range(len(sets))]
+    sgate = torch.randn((H,), device="cuda", generator=gen) * (1.0 / H ** 0.5)
+    def whole_layer(i):
+        routed(i)
+        sh = shared[i % len(shared)]
+        be.moe_shared_expert(sh[0], sh[1], sgate, I, H, xm, ym)
+    for i in range(3):
+        whole_layer(i)
+    ms_layer = tm(torch, whole_layer, 40)
+    # ... and as one call (lq4_moe_ffn)
+    def one_call(i):
+        sh = shared[i % len(shared)]
+        be.moe_ffn(lg, sets[i % len(sets)][0], sets[i % len(sets)][1], E, TK, I, sh[0], sh[1], sgate, I, H, xm, ym)
+    for i in range(3):
+        one_call(i)
+    ms_one = tm(torch, one_call, 40)
+    # decode: the same layer for one token (8 routed experts + the shared one, 28.3 MB)
+    lg1, x1, y1 = lg[:1].contiguous(), xm[:1].contiguous(), torch.empty((1, H), device="cuda")
+    def decode_layer(i):
+        sh = shared[i % len(shared)]
+        be.moe_ffn(lg1, sets[i % len(sets)][0], sets[i % len(sets)][1], E, TK, I, sh[0], sh[1], sgate, I, H, x1, y1)
+    for i in range(3):
+        decode_layer(i)
+    ms_decode = tm(torch, decode_layer, 40)
+    decode_bytes = (TK + 1) * (2 * I * (H // 32) * 20 + H * (I // 32) * 20)
+    out["moe_layer_one_token"] = {"algorithmic_bytes": decode_bytes, "ms_per_step": round(ms_decode, 4),
+                                  "GB/s": round(decode_bytes / ms_decode / 1e6, 1),
+                                  "pct_of_hbm_peak": round(100 * decode_bytes / ms_decode / 1e6 / HBM_PEAK_GBPS, 2),
+                                  "launches": 2}
+    out["moe_grouped_gemv"] = {"distinct_experts": distinct, "algorithmic_bytes": moe_bytes,
+                               "ms_per_step": round(ms, 4), "GB/s": round(moe_bytes / ms / 1e6, 1),
+                               "pct_of_hbm_peak": round(100 * moe_bytes / ms / 1e6 / HBM_PEAK_GBPS, 2),
+                               "ms_per_step_with_router": round(ms_routed, 4),
+                               "ms_per_step_with_router_and_shared_expert": round(ms_layer, 4),
+                               "ms_per_step_whole_layer_one_call": round(ms_one, 4)}
+    del sets, shared
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -187,6 +255,8 @@ def main():
                     help="run nothing but warmup and the timed headline region (for kernel-trace profiles)")
     ap.add_argument("--gemm-only", action="store_true",
                     help="run the four config-2 prefill GEMM shapes and nothing else (for counter runs)")
+    ap.add_argument("--moe-only", action="store_true",
+                    help="only the MoE lines (config 4, whole layer, one-token layer): for profiling")
     ap.add_argument("--read-sweep", action="store_true",
                     help="print the read-probe sweep (grid x bytes in flight x access pattern x size) and exit")
     ap.add_argument("--eager", action="store_true",
@@ -209,6 +279,9 @@ def main():
     B = args.batch
     if args.gemm_only:
         print(json.dumps({"prefill_gemm_f16": prefill_gemm(torch, be, gen, graph_timed)}))
+        return
+    if args.moe_only:
+        print(json.dumps(moe_section(torch, be, gen, graph_timed, synth)))
         return
 
     # ---- resident inputs ------------------------------------------------------------
@@ -560,68 +633,7 @@ def main():
             sib[fmt] = res
         out["sibling_gemm_f16"] = sib
 
-        # MoE grouped expert GEMV, benchmark config 4
-        mo = synth.MOE_35B
-        E, I, H, T, TK = mo["experts"], mo["inter"], mo["hidden"], mo["tokens"], mo["top_k"]
-        sets = []
-        for _ in range(10):  # 10 x 125.8 MB of expert tensors
-            sets.append((be.wrap_device_blocks(device_q4_weight(torch, E * 2 * I, H, gen)),
-                         be.wrap_device_blocks(device_q4_weight(torch, E * H, I, gen))))
-        lg = torch.from_numpy(synth.router_logits(T, E, seed=0)).cuda()
-        ids, wts = be.moe_route(lg, TK)
-        xm = torch.randn((T, H), device="cuda", generator=gen)
-        ym = torch.empty((T, H), device="cuda")
-        distinct = int(torch.unique(ids).numel())
-        moe_bytes = distinct * (2 * I * (H // 32) * 20 + H * (I // 32) * 20) + 2 * T * H * 4
-        f = lambda i: be.moe_experts(sets[i % len(sets)][0], sets[i % len(sets)][1], E, I, H, xm, ids, wts, ym)
-        for i in range(len(sets)):
-            f(i)
-        ms = tm(torch, f, 40)
-        # the same step with the router in front of it (softmax, top-k, renormalise from the logits)
-        def routed(i):
-            ids_i, wts_i = be.moe_route(lg, TK)
-            be.moe_experts(sets[i % len(sets)][0], sets[i % len(sets)][1], E, I, H, xm, ids_i, wts_i, ym)
-        for i in range(3):
-            routed(i)
-        ms_routed = tm(torch, routed, 40)
-        # ... and with the always-active shared expert (same intermediate size) added onto the sum
-        shared = [(be.wrap_device_blocks(device_q4_weight(torch, 2 * I, H, gen)),
-                   be.wrap_device_blocks(device_q4_weight(torch, H, I, gen))) for _ in range(len(sets))]
-        sgate = torch.randn((H,), device="cuda", generator=gen) * (1.0 / H ** 0.5)
-        def whole_layer(i):
-            routed(i)
-            sh = shared[i % len(shared)]
-            be.moe_shared_expert(sh[0], sh[1], sgate, I, H, xm, ym)
-        for i in range(3):
-            whole_layer(i)
-        ms_layer = tm(torch, whole_layer, 40)
-        # ... and as one call (lq4_moe_ffn)
-        def one_call(i):
-            sh = shared[i % len(shared)]
-            be.moe_ffn(lg, sets[i % len(sets)][0], sets[i % len(sets)][1], E, TK, I, sh[0], sh[1], sgate, I, H, xm, ym)
-        for i in range(3):
-            one_call(i)
-        ms_one = tm(torch, one_call, 40)
-        # decode: the same layer for one token (8 routed experts + the shared one, 28.3 MB)
-        lg1, x1, y1 = lg[:1].contiguous(), xm[:1].contiguous(), torch.empty((1, H), device="cuda")
-        def decode_layer(i):
-            sh = shared[i % len(shared)]
-            be.moe_ffn(lg1, sets[i % len(sets)][0], sets[i % len(sets)][1], E, TK, I, sh[0], sh[1], sgate, I, H, x1, y1)
-        for i in range(3):
-            decode_layer(i)
-        ms_decode = tm(torch, decode_layer, 40)
-        decode_bytes = (TK + 1) * (2 * I * (H // 32) * 20 + H * (I // 32) * 20)
-        out["moe_layer_one_token"] = {"algorithmic_bytes": decode_bytes, "ms_per_step": round(ms_decode, 4),
-                                      "GB/s": round(decode_bytes / ms_decode / 1e6, 1),
-                                      "pct_of_hbm_peak": round(100 * decode_bytes / ms_decode / 1e6 / HBM_PEAK_GBPS, 2),
-                                      "launches": 2}
-        out["moe_grouped_gemv"] = {"distinct_experts": distinct, "algorithmic_bytes": moe_bytes,
-                                   "ms_per_step": round(ms, 4), "GB/s": round(moe_bytes / ms / 1e6, 1),
-                                   "pct_of_hbm_peak": round(100 * moe_bytes / ms / 1e6 / HBM_PEAK_GBPS, 2),
-                                   "ms_per_step_with_router": round(ms_routed, 4),
-                                   "ms_per_step_with_router_and_shared_expert": round(ms_layer, 4),
-                                   "ms_per_step_whole_layer_one_call": round(ms_one, 4)}
-        del sets, shared
+        out.update(moe_section(torch, be, gen, tm, synth))
 
         # plain copies of known size: what a profiler's HBM traffic counters are scaled by
         csrc = torch.empty(64 << 20, dtype=torch.int32, device="cuda").random_(generator=gen)

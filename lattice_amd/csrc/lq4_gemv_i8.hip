@@ -301,11 +301,12 @@ __global__ __launch_bounds__(64 * CW * TW) void gemv_q4_i8(const uint8_t* __rest
         xv[it][0] = xp[0];
         xv[it][1] = xp[1];
     }
-    // kDepth units in flight per wave, in a ring of register buffers that the unrolled loop below walks with
-    // compile-time indices.  Requests are skipped past the wave's last unit (a wave cannot end before its last load
-    // has come back); the compiler then waits in front of a buffer's use as if the skipped request had not been
-    // made, one unit earlier than needed, so three units are in flight where it matters.
-    constexpr int kDepth = 4;
+    // kDepth units per wave in registers (beside the one in its LDS tile), in a ring of register buffers that the
+    // unrolled loop below walks with compile-time indices.  One: the next unit is on its way while the current one is
+    // multiplied.  A ring of four was measured slower on the large matrices (12288 x 2048 at 8 / 4 rows 10.0 / 9.2 ->
+    // 9.1 / 8.2 us, 2048 x 6144 11.3 -> 10.5) and level on the small ones, where a wave has one unit anyway: what a
+    // CU asks for beyond its share of the memory system queues in front of the activations the staging waits for.
+    constexpr int kDepth = 1;
     Q4BlockRaw ring[kDepth][kLoads];
 #pragma unroll
     for (int i = 0; i < kDepth; ++i) {
@@ -543,6 +544,20 @@ struct I8Plan {
     size_t lds;
 };
 
+size_t lds_eight_waves(uint32_t nb) {
+    return static_cast<size_t>(nb) * (kXqBytes + kXfBytes) + 8 * kTileDwords * 4 + 8 * 64 * 2 * 4 + 8 * kMaxLoraRank * 4;
+}
+
+}  // namespace
+
+// At least two 16-row tiles per CU and rows short enough that two eight-wave workgroups share a CU's LDS.
+bool gemv_i8_many_short_rows(uint32_t n, uint32_t k, uint32_t cu_count) {
+    const uint32_t nb = k / kBlockWeights;
+    return (n + 15) / 16 >= 2 * cu_count && nb >= 4 * kBpw && lds_eight_waves(nb) <= 78 * 1024;
+}
+
+namespace {
+
 bool plan_i8(uint32_t n, uint32_t k, uint32_t batch, uint32_t cu_count, I8Plan* out) {
     if (k == 0 || k % kBlockWeights || n == 0 || batch == 0 || batch > 8) return false;
     const uint32_t nb = k / kBlockWeights;
@@ -563,6 +578,17 @@ bool plan_i8(uint32_t n, uint32_t k, uint32_t batch, uint32_t cu_count, I8Plan* 
         if (p.tw > 1) p.tw /= 2;
         else if (p.cw > 1) p.cw /= 2;
         else return false;
+    }
+    // Many tiles of short rows (12288 x 2048: 768 tiles): workgroups of eight waves (two split K, four tiles side by
+    // side), two of which fit a CU, one round each, instead of sixteen-wave workgroups that walk two rounds
+    // (at 8 / 4 rows 9.1 / 8.1 -> 8.8 / 7.9 us).
+    if (gemv_i8_many_short_rows(n, k, cu_count)) {
+        p.cw = 2;
+        p.tw = 4;
+        p.lds = lds_eight_waves(nb);
+        p.grid = (n_tiles + 3) / 4;
+        *out = p;
+        return true;
     }
     const uint32_t groups = (n_tiles + p.tw - 1) / p.tw;  // rounds of tiles in all
     if (groups <= cu_count) {

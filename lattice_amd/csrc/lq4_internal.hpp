@@ -129,6 +129,9 @@ void launch_gemv_b1(const uint8_t* w, uint32_t n, uint32_t k, const float* x, fl
                     const LoraEpilogue& lora, hipStream_t stream);
 // 2..8 activation rows on the integer matrix cores (lq4_gemv_i8.hip): y = W . x, optional LoRA epilogue with t in
 // memory or computed by producer workgroups of the launch (gemv_i8_lora_in_launch).  gemv_i8_serves: the staged activations fit the LDS (K up to about 7000).
+// Tall matrices of short rows (at least two 16-row tiles per CU, K up to about 2900), which the kernel serves with
+// two eight-wave workgroups per CU.
+bool gemv_i8_many_short_rows(uint32_t n, uint32_t k, uint32_t cu_count);
 bool gemv_i8_serves(uint32_t n, uint32_t k, uint32_t batch, uint32_t cu_count);
 // true = the launch has room for `rank_total` producer workgroups that compute the LoRA factors t = A . x themselves
 // (LoraEpilogue::a and ::slots set, [rank_total][8] slots; for several views a, t_off of MultiViews and

@@ -17,7 +17,7 @@
 // projection ([E, H, I]), o[pair, row] = W . h[pair].
 //
 // Memory: a unit is 16 rows x 8 blocks (2.5 KB); lane l loads block l % 8 of rows l / 8 and l / 8 + 8 as whole 20-byte
-// blocks, four units in flight in registers, and passes them through a wave-private LDS tile into the operand layout.
+// blocks, and passes them through a wave-private LDS tile into the operand layout (the next unit on its way meanwhile).
 // CW waves split the 8-block chunks of a tile and add their partial sums through LDS in wave order; TW = 8 / CW tiles
 // are worked on side by side; a workgroup does `rounds` such rounds.
 //
@@ -30,11 +30,10 @@
 // down), and what this file does about it: (1) with four waves and 32 output rows a workgroup, 912 workgroups had
 // work and 768 fit the chip: the last 144 started when the first ended, 14 us into a 25 us launch -- eight waves over
 // 64 (gate/up) or 256 (down) rows make about 460, which all start at once; (2) a CU's share of the memory system is
-// about 18 KB/us and answers in the order of asking, so activations asked for behind a whole ring of every wave on the
-// CU arrived last and the matrix work that could have run beside the stream ran after it -- one unit a wave is
-// requested before the staging, the rest of the ring after its barrier (none, two or four units before it, with or
-// without a barrier between the requests for activations and for weights, all measured level or behind); (3) per CU the vector instructions (about 140
-// a unit) and the LDS traffic (14 KB a unit) each still add up to about half the streaming time.
+// about 18 KB/us and answers in the order of asking, so activations asked for behind a ring of four units of every
+// wave on the CU arrived last, and the matrix work that could have run beside the stream ran after it -- a wave
+// holds one unit (kDepth); (3) per CU the vector instructions (about 130 a unit) and the LDS traffic (14 KB a unit)
+// each still add up to about a third of the streaming time.
 //
 // Precision: weights and integer sums are exact; an activation is rounded to a multiple of its block's largest
 // magnitude / 4194000 (1.2e-7 of the block maximum, the resolution of the f32 activation itself).  A block whose
@@ -188,7 +187,13 @@ constexpr int kTilePitch = 44;     // dwords per row of the LDS tile (40 used; 4
 constexpr int kTileDwords = 16 * kTilePitch;
 constexpr int kXqBytes = 512;      // per block: [4 k groups][16 operand rows] x 8 bytes
 constexpr int kXfBytes = 64;       // per block: [4 pairs]{xs, xs * sum of the block's fixed-point x, -, -} f32
-constexpr int kDepth = 4;          // units in flight per wave
+// Units a wave holds in registers (beside the one in its LDS tile).  One: the next unit is requested when the current
+// one has been copied into the tile and arrives while that is multiplied.  Deeper rings were measured and are
+// slower (16 tokens of top 8 among 64 experts, both launches and the combine: 4 / 3 / 2 / 1 units 36.2 / 35.7 / 34.7 /
+// 34.2 us; 64 tokens 74.3 / 69.7 / 68.3 / 67.2): the 3600 waves of a launch with one unit each have about what the
+// memory system holds in flight anyway (9 MB), and whatever is asked for beyond that only queues in front of the
+// loads a workgroup's start waits for (the routing table, the activations).
+constexpr int kDepth = 1;
 constexpr float kQScale = 4194000.0f;
 
 struct __attribute__((packed, aligned(4))) Q4BlockRaw {
@@ -218,7 +223,6 @@ size_t lds_bytes(uint32_t nb, uint32_t waves) {
 template <bool GATE_UP, int CW, int TW, bool FROM_IDS>
 __global__ __launch_bounds__(64 * CW * TW) void moe_expert_i8(MoeGemvArgs p) {
     constexpr int kWaves = CW * TW, kThreads = 64 * kWaves;
-    constexpr int PRE = 1;  // units a wave requests before the activations are staged (the rest of its ring right after)
     constexpr uint32_t TPR = GATE_UP ? 2 : 1;  // tiles of a wave per round
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int tid = threadIdx.x;
@@ -368,7 +372,7 @@ __global__ __launch_bounds__(64 * CW * TW) void moe_expert_i8(MoeGemvArgs p) {
     }
     Q4BlockRaw ring[kDepth][2];
 #pragma unroll
-    for (int i = 0; i < PRE; ++i) {
+    for (int i = 0; i < kDepth; ++i) {
         if (static_cast<uint32_t>(i) < units) load_unit(ring[i], i);
     }
     __builtin_amdgcn_sched_barrier(0);  // nothing below is scheduled above these loads
@@ -385,13 +389,6 @@ __global__ __launch_bounds__(64 * CW * TW) void moe_expert_i8(MoeGemvArgs p) {
     // blocks past the end of a row (K not a whole number of chunks): scale and sum zero, so they count for nothing
     for (uint32_t i = nb * 16 + tid; i < nbp * 16; i += kThreads) reinterpret_cast<float*>(xf)[i] = 0.0f;
     __syncthreads();
-    // The rest of the ring only now: a CU's share of the memory system answers in the order of asking, and activations
-    // asked for behind a whole ring of every wave of every workgroup on the CU arrive last, the matrix instructions
-    // that could have run beside the stream then run after it.
-#pragma unroll
-    for (int i = PRE; i < kDepth; ++i) {
-        if (static_cast<uint32_t>(i) < units) load_unit(ring[i], i);
-    }
 
     // ---- the product ----
     const uint32_t r = lane & 15, g = lane >> 4;  // operand mapping: weight row r of the tile, k group / pair g

@@ -422,12 +422,12 @@ static void plain_gemv_one_token(lq4_ctx* ctx, const uint8_t* wp, uint32_t n, ui
 }
 
 // 2..8 rows on the integer matrix-core kernel: three to eight rows of a matrix of up to 4096 x 2048; five to eight
-// rows (any number from 16384 rows on) of a tall matrix of short rows (12288 x 2048 at 5..8 rows 9.5-9.8 -> 8.6-8.8 us,
-// 16384 x 2048 at 2..8 rows 9.1-12.4 -> 8.1-9.0, 9728 x 2560 at 5..8 rows 11.7-13.6 -> 10.0-10.1; at 2..4 rows of the
-// first level, 7.7-8.0 us both); or, for the tests, whatever it can hold.
+// rows of a tall matrix of short rows (12288 x 2048 9.6-10.0 -> 8.7-8.8 us, 16384 x 2048 11.0-11.6 -> 8.8-9.0,
+// 9728 x 2560 12.0-12.6 -> 10.0-10.1; at 2..4 rows the 4x4x4 kernel is ahead there, 6.3-7.3 us against 7.8); or, for
+// the tests, whatever it can hold.
 static bool gemv_takes_i8(const lq4_ctx* ctx, uint32_t n, uint32_t k, uint32_t batch) {
     const bool small = batch >= 3 && k <= 2048 && n <= 4096;
-    const bool tall = (batch >= 5 || n >= 16384) && gemv_i8_many_short_rows(n, k, ctx->cu_count);
+    const bool tall = batch >= 5 && gemv_i8_many_short_rows(n, k, ctx->cu_count);
     return batch >= 2 && batch <= 8 && ctx->gemv_i8 && (ctx->gemv_i8 == 2 || small || tall) &&
            gemv_i8_serves(n, k, batch, ctx->cu_count);
 }

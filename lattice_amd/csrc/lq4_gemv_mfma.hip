@@ -102,7 +102,7 @@ struct GemvArgs {
 // Workgroups are persistent: workgroup g handles row groups g, g + gridDim.x, ... (a row group
 // is 4*T*(WAVES/KS) rows) with the activations staged once.  For one wave the work is a list of
 // units (row group, step); unit u+1 is in flight while unit u is consumed.
-template <int NSETS, bool HILO, int T, int KS, bool LONG, int WAVES>
+template <int NSETS, bool HILO, int T, int KS, bool LONG, int WAVES, bool DEEP>
 __global__ __launch_bounds__(64 * WAVES) void gemv_q4_mfma(GemvArgs p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     constexpr int kThreads = 64 * WAVES;
@@ -174,11 +174,18 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_mfma(GemvArgs p) {
         }
     };
 
-    // ring of four unit buffers: three units are in flight while one is consumed
+    // Unit buffers in registers.  DEEP: a ring of four, three units in flight while one is consumed; else two, the
+    // next unit in flight while one is consumed.  The shallow form is the faster one except on very long rows
+    // (measured at 2 / 4 / 8 rows: 12288 x 2048 8.0 / 7.8 / - -> 6.3 / 7.4 / - us, 6144 x 2048 at 2 rows 6.8 -> 5.0,
+    // 2048 x 6144 5.8 / 6.6 / 8.4 -> 5.8 / 6.4 / 8.0, 17408 x 5120 18.1 / 20.4 / 24.2 -> 17.0 / 18.6 / 24.2, 8192 x 8192
+    // 13.9 / 15.2 / 19.2 -> 13.2 / 14.5 / 18.0; but 5120 x 17408 19.6 / 21.5 -> 21.4 / 23.1): what a CU asks for beyond
+    // its share of the memory system queues in front of the activations its workgroups' staging waits for.
     Q4BlockRaw buf_a[T], buf_b[T], buf_c[T], buf_d[T];
     load_unit(buf_a, 0);
-    load_unit(buf_b, units > 1 ? 1 : 0);
-    load_unit(buf_c, units > 2 ? 2 : 0);
+    if constexpr (DEEP) {
+        load_unit(buf_b, units > 1 ? 1 : 0);
+        load_unit(buf_c, units > 2 ? 2 : 0);
+    }
     __builtin_amdgcn_sched_barrier(0);  // nothing below is scheduled above these loads
 
     // ---- stage activations: one (block, dword) item = 8 values per activation row ------------
@@ -353,8 +360,9 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_mfma(GemvArgs p) {
         // LONG streams prefetch without a condition (past the end: the last unit again), so the wait
         // for the current unit counts exactly and three units stay in flight; short streams, whose
         // units are all in flight from the start, skip the redundant loads instead
-        if (LONG) load_unit(nxt, u + 3 < units ? u + 3 : units - 1);
-        else if (u + 3 < units) load_unit(nxt, u + 3);
+        constexpr uint32_t kAhead = DEEP ? 3 : 1;
+        if (LONG) load_unit(nxt, u + kAhead < units ? u + kAhead : units - 1);
+        else if (u + kAhead < units) load_unit(nxt, u + kAhead);
         const uint32_t it = u / n_local, q = u - it * n_local;
         const uint32_t blk_raw = (ks + q * KS) * 16 + g;
         const bool live = blk_raw < nb;
@@ -499,6 +507,16 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_mfma(GemvArgs p) {
     }
     // the buffers rotate roles every unit, so no block is ever copied between registers
     uint32_t q = 0, it = 0;
+    if constexpr (!DEEP) {
+        for (uint32_t u = 0; u < units; u += 2) {
+            process(buf_a, buf_b, u);
+            if (++q == n_local) { finish(it++); q = 0; }
+            if (u + 1 >= units) break;
+            process(buf_b, buf_a, u + 1);
+            if (++q == n_local) { finish(it++); q = 0; }
+        }
+        return;
+    }
     for (uint32_t u = 0; u < units; u += 4) {
         process(buf_a, buf_d, u);
         if (++q == n_local) { finish(it++); q = 0; }
@@ -514,11 +532,20 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_mfma(GemvArgs p) {
     }
 }
 
+template <int NSETS, bool HILO, int T, int KS, bool LONG, int WAVES, bool DEEP>
+void launch_deep(const GemvArgs& a, size_t lds, uint32_t wgs, hipStream_t stream) {
+    static LdsCapOnce lds_cap;
+    lds_cap.raise(reinterpret_cast<const void*>(gemv_q4_mfma<NSETS, HILO, T, KS, LONG, WAVES, DEEP>), 160 * 1024);
+    hipLaunchKernelGGL((gemv_q4_mfma<NSETS, HILO, T, KS, LONG, WAVES, DEEP>), dim3(wgs), dim3(64 * WAVES), lds, stream, a);
+}
+
+// the ring of four only for very long rows, which come with eight-wave workgroups (one staged copy per CU)
 template <int NSETS, bool HILO, int T, int KS, bool LONG, int WAVES>
 void launch_long(const GemvArgs& a, size_t lds, uint32_t wgs, hipStream_t stream) {
-    static LdsCapOnce lds_cap;
-    lds_cap.raise(reinterpret_cast<const void*>(gemv_q4_mfma<NSETS, HILO, T, KS, LONG, WAVES>), 160 * 1024);
-    hipLaunchKernelGGL((gemv_q4_mfma<NSETS, HILO, T, KS, LONG, WAVES>), dim3(wgs), dim3(64 * WAVES), lds, stream, a);
+    if constexpr (WAVES == 8 && LONG) {
+        if (a.k >= 12288) return launch_deep<NSETS, HILO, T, KS, LONG, WAVES, true>(a, lds, wgs, stream);
+    }
+    launch_deep<NSETS, HILO, T, KS, LONG, WAVES, false>(a, lds, wgs, stream);
 }
 
 template <int NSETS, bool HILO, int T, int KS, int WAVES>

@@ -482,7 +482,7 @@ struct DmaPlan {
     size_t lds;
 };
 
-// Which instantiation serves a row length: ring depth by what LDS leaves beside the staged activations.
+// Which instantiation serves a row length (ring depth: see launch_gemv_dma).
 bool plan_dma(uint32_t n, uint32_t k, uint32_t cu_count, DmaPlan* out) {
     const uint32_t nb = k / kBlockWeights;
     // (sixteen dwords between the activations and the rings: the waves' partial sums, or the row counter)
@@ -490,8 +490,7 @@ bool plan_dma(uint32_t n, uint32_t k, uint32_t cu_count, DmaPlan* out) {
     DmaPlan p;
     p.slabs = nb <= 192 ? (nb + 63) / 64 : 0;
     p.xr = k <= 8192 ? 1 : 3;
-    p.depth = 6;
-    if (fixed + static_cast<size_t>(kWaves) * 6 * kSlotBytes > 160 * 1024) p.depth = 3;
+    p.depth = p.slabs == 2 ? 4 : 3;
     p.lds = fixed + static_cast<size_t>(kWaves) * p.depth * kSlotBytes;
     if (k > 24576 || p.lds > 160 * 1024) return false;
     // one workgroup per CU, rows dealt evenly; fewer workgroups when there are fewer rows than CUs
@@ -524,26 +523,37 @@ bool gemv_dma_serves(uint32_t n, uint32_t k, uint32_t cu_count) {
     return n != 0 && plan_dma(n, k, cu_count, &p);
 }
 
-// Measured against the lane-owns-block kernel on 256 CUs (us, that kernel -> this one): 32768 x 2048 (42 MB) 10.2 ->
-// 10.35; 65536 x 2048 (84 MB) 17.4 -> 16.3; 248320 x 2048 62.1 -> 51.3; 151936 x 5120 87.8 -> 76.2; 32768 x 3072 (63 MB)
-// 14.4 -> 13.4; 17408 x 5120 (56 MB) 12.6 -> 12.3; 24576 x 2560 (39 MB) 12.9 -> 10.6; 12288 x 5120 (39 MB) 10.3 -> 10.0;
-// 16384 x 4096 (42 MB) 9.7 -> 10.1; 8192 x 6144 (31 MB) 8.4 -> 8.5; 16384 x 8192 17.8 -> 18.0; 8192 x 12288 (63 MB) 14.9 ->
-// 13.0; 4096 x 14336 (37 MB) 10.8 -> 9.4; 5120 x 17408 16.8 -> 13.5; 2048 x 17408 (22 MB) 8.6 -> 9.0.  Behind for every
-// row shorter than one slab (131072 x 1024 18.9 -> 21.7: the other kernel puts two rows side by side in a wave) and
-// for the decode layer's matrices (2..16 MB, 1.0 us behind: its start costs two workgroup barriers of sixteen waves).
+// Measured against the lane-owns-block kernel on 256 CUs (us, that kernel -> this one, ring depth three):
+//   large: 248320 x 2048 62.1 -> 49.6; 151936 x 5120 87.8 -> 75.1; 65536 x 2048 (84 MB) 17.4 -> 15.3; 17408 x 5120 (56 MB)
+//     12.6 -> 11.6; 32768 x 2048 (42 MB) 10.2 -> 9.1; 16384 x 4096 9.6 -> 9.2; 8192 x 8192 10.7 -> 9.7; 12288 x 5120 (39 MB)
+//     10.3 -> 9.4; 4096 x 14336 (37 MB) 10.8 -> 9.4; 8192 x 6144 (31 MB) 8.4 -> 7.9; 20480 x 2048 (26 MB) 7.2 -> 6.9;
+//     5120 x 17408 16.8 -> 13.5; 3072 x 12288 (24 MB) 9.3 -> 8.2; level at 16384 x 2048 (21 MB, 6.1) and 12288 x 2048 (16 MB,
+//     5.2); behind with few long rows (2048 x 17408, 22 MB: 8.6 -> 9.1);
+//   rows that are not whole 2048-weight slabs, where the other kernel's lanes idle through part of a step: 24576 x
+//     2560 12.9 -> 9.7; 12288 x 3072 8.9 -> 6.7; 9728 x 2560 (16 MB) 8.3 -> 5.9; 8192 x 3072 7.5 -> 5.5; 6144 x 3584 6.5 -> 4.9;
+//     6144 x 2560 (10 MB) 6.1 -> 4.6; 4096 x 3072 (8 MB) 6.0 -> 4.0; 6144 x 5120 7.5 -> 6.4;
+//   rows of two slabs: 6144 x 4096 (16 MB) 6.1 -> 5.0; 8192 x 4096 6.4 -> 6.1;
+//   level or behind below that: 4096 x 8192 6.8 -> 6.9, 4096 x 6144 5.5 -> 5.7, 2048 x 6144 (8 MB) 3.7 -> 4.7, every row
+//     shorter than one slab (131072 x 1024 18.9 -> 21.7: the other kernel puts two rows side by side in a wave) and the
+//     decode layer's matrices (its start costs two workgroup barriers of sixteen waves).
 bool gemv_dma_pays(uint32_t n, uint32_t k, uint32_t cu_count) {
     if (!gemv_dma_serves(n, k, cu_count) || k < 2048) return false;
     const uint64_t bytes = static_cast<uint64_t>(n) * (k / kBlockWeights) * kBlockBytes;
-    return bytes >= (64ull << 20) || (k >= 10240 && bytes >= (32ull << 20)) || (k <= 6144 && bytes >= (48ull << 20));
+    if (bytes >= (20ull << 20) && n >= 3072) return true;
+    if (k % 2048 != 0) return bytes >= (6ull << 20);
+    return k == 4096 && bytes >= (12ull << 20);
 }
 
 void launch_gemv_dma(const uint8_t* w, uint32_t n, uint32_t k, const float* x, float* y, uint32_t cu_count, hipStream_t stream) {
     DmaPlan p;
     if (!plan_dma(n, k, cu_count, &p)) return;  // the caller asked gemv_dma_serves first
-    if (p.slabs == 1) launch_rows<6, 1>(p, w, n, k, x, y, stream);
-    else if (p.slabs == 2) launch_rows<6, 2>(p, w, n, k, x, y, stream);
-    else if (p.slabs == 3) launch_rows<6, 3>(p, w, n, k, x, y, stream);
-    else if (p.xr == 1 && p.depth == 6) launch_one<1, 6>(p, w, n, k, x, y, stream);
+    // Ring depth: the least the kernels allow (three slots a wave; four where a row is two slabs).  Six were measured
+    // slower on every shape (248320 x 2048 51.4 -> 49.6 us, 17408 x 5120 12.3 -> 11.6, 151936 x 5120 76.3 -> 75.1,
+    // 65536 x 2048 16.4 -> 15.3, 32768 x 4096 16.0 -> 14.9, 16384 x 8192 18.0 -> 16.1, 32768 x 3072 13.5 -> 12.4): what a
+    // CU has asked for beyond its share of the memory system only queues.
+    if (p.slabs == 1) launch_rows<3, 1>(p, w, n, k, x, y, stream);
+    else if (p.slabs == 2) launch_rows<4, 2>(p, w, n, k, x, y, stream);
+    else if (p.slabs == 3) launch_rows<3, 3>(p, w, n, k, x, y, stream);
     else if (p.xr == 1) launch_one<1, 3>(p, w, n, k, x, y, stream);
     else launch_one<3, 3>(p, w, n, k, x, y, stream);
 }

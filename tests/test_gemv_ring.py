@@ -77,6 +77,25 @@ def test_ring_gemv_against_the_oracle_and_the_other_kernel(ring, lanes, n, k):
         assert same
 
 
+@pytest.fixture(scope="module")
+def routed():
+    b = backend.HipQ4Backend(0)  # the library's own choice between the two kernels
+    yield b
+    b.close()
+
+
+@pytest.mark.parametrize("n,k", [(4100, 2560), (6200, 4096), (10300, 3072), (3072, 8192), (20500, 2048), (2048, 17408)])
+def test_one_token_gemv_as_the_library_routes_it(routed, lanes, n, k):
+    """Matrices on either side of the rule that sends a one-token GEMV to the ring kernel (size, rows that are not
+    whole slabs, rows of two slabs): the call as routed agrees with the oracle and with the lane-owns-block kernel."""
+    print(f"routed one-token gemv n={n} k={k}", flush=True)
+    w = synth.q4_weight(n, k, seed=n ^ k)
+    x = synth.activations(1, k, seed=k)
+    got = run(routed, w, x, n, k)
+    assert rel_err(got, oracle.gemm_f32(x, w, n, k)[0]) <= REL_TOL
+    assert rel_err(got, run(lanes, w, x, n, k)) <= 1e-5
+
+
 def test_ring_gemv_one_hot_columns_are_bit_exact(ring):
     # 65 blocks a row: one full slab and a last slab of a single block; 257 rows straddle waves and workgroups
     import torch

@@ -463,8 +463,8 @@ int lq4_probe_read_config(lq4_ctx* ctx, const void* p_dev, size_t nbytes, uint32
  * lq4_lm_head_topk in two launches, a one-row step of lq4_gemv_chain without LoRA).  Per context; a new
  * context starts from the environment variable LQ4_GEMV_KERNEL, else AUTO.
  *   AUTO        by shape: the LDS-ring kernel where it is measured faster (rows of at least 2048 weights and
- *               64 MB of weights, 48 MB with rows of at most 6144 weights, or 32 MB with rows of at least 10240),
- *               else the lane-owns-block kernel
+ *               20 MB of weights in at least 3072 rows, 6 MB when K is not a multiple of 2048, 12 MB at
+ *               K = 4096), else the lane-owns-block kernel
  *   LANE_BLOCKS always the kernel in which each lane loads its own blocks into registers
  *   LDS_RING    the kernel that streams whole 1280-byte slabs into a per-wave ring of LDS slots wherever the
  *               shape fits it (K <= 24576), else the other one
